@@ -1,0 +1,1540 @@
+"""CPU oracle: a numpy interpreter for the StableHLO subset on the hot path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the product path may import this file; it
+is the checker that the HIP path is compared with (tests/, the smoke entry and
+the cpu_baseline leg of the benchmark).
+
+It restates, op by op, what the reference's handlers compute
+(`/root/reference/src/pjrt_plugin/ops/*.cc`); the arithmetic itself lives in the
+third-party MLX library (pinned commit a025496c8f6da9d599e2010019ea5ee328c2d119,
+not vendored in the reference), so every function here follows the StableHLO
+specification for the op and the edge-case rules spelled out at the reference's
+call sites (cited per function).  Contractions and float reductions accumulate in
+float64 by default so that the oracle is a tighter truth than any f32 ordering;
+`accum="f32"` switches them to float32 BLAS for the timed CPU baseline.
+
+Pins (tests/test_oracle_*.py): literal gather/scatter/control-flow cases of the
+reference's own tests, torch-CPU conv2d / conv_transpose2d and brute-force loops
+for convolution, numpy einsum for dot_general, closed forms for while/case,
+IEEE special cases for shifts/remainder/sign/round.  bf16 results are pinned only
+by the rounding rule (round-to-nearest-even of the f32 result) — the reference
+holds no bf16 expectation ("parity unpinned" by the reference for bf16).
+"""
+from __future__ import annotations
+
+import math
+import re
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+# ----------------------------------------------------------------------------
+# types
+# ----------------------------------------------------------------------------
+_NP = {
+    "f32": np.float32, "f64": np.float64, "f16": np.float16, "bf16": np.float32,
+    "i1": np.bool_, "i8": np.int8, "i16": np.int16, "i32": np.int32, "i64": np.int64,
+    "ui8": np.uint8, "ui16": np.uint16, "ui32": np.uint32, "ui64": np.uint64,
+}
+FLOATS = ("f32", "f64", "f16", "bf16")
+
+
+def round_bf16(a: np.ndarray) -> np.ndarray:
+    """float32 values rounded to the nearest bfloat16 (ties to even), kept as float32."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    u = a.view(np.uint32)
+    nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    r = (u + (np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1)))) & np.uint32(0xFFFF0000)
+    r = np.where(nan, u | np.uint32(0x00400000), r).astype(np.uint32)
+    return r.view(np.float32).reshape(a.shape)
+
+
+def bf16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
+    return (bits.astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
+    return (round_bf16(a).view(np.uint32) >> np.uint32(16)).astype(np.uint16)
+
+
+class TType:
+    __slots__ = ("shape", "dtype")
+
+    def __init__(self, shape, dtype):
+        self.shape = tuple(shape)
+        self.dtype = dtype
+
+    def __repr__(self):
+        return f"tensor<{'x'.join(map(str, self.shape + (self.dtype,)))}>"
+
+
+class Op:
+    __slots__ = ("name", "results", "operands", "attrs", "regions", "in_types", "out_types")
+
+    def __init__(self):
+        self.name = ""
+        self.results: List[str] = []
+        self.operands: List[str] = []
+        self.attrs: Dict[str, object] = {}
+        self.regions: List["Region"] = []
+        self.in_types: List[TType] = []
+        self.out_types: List[TType] = []
+
+
+class Region:
+    __slots__ = ("args", "arg_types", "ops")
+
+    def __init__(self):
+        self.args: List[str] = []
+        self.arg_types: List[TType] = []
+        self.ops: List[Op] = []
+
+
+class Func:
+    def __init__(self, name):
+        self.name = name
+        self.body = Region()
+        self.result_types: List[TType] = []
+
+
+# ----------------------------------------------------------------------------
+# parser (recursive descent over characters; independent of the C++ front end)
+# ----------------------------------------------------------------------------
+class _P:
+    def __init__(self, text: str):
+        self.s = text
+        self.i = 0
+        self.n = len(text)
+
+    def err(self, msg):
+        ln = self.s.count("\n", 0, self.i) + 1
+        raise SyntaxError(f"stablehlo text line {ln}: {msg}: ...{self.s[self.i:self.i + 60]!r}")
+
+    def ws(self):
+        s, n = self.s, self.n
+        while self.i < n:
+            c = s[self.i]
+            if c in " \t\r\n":
+                self.i += 1
+            elif c == "/" and s.startswith("//", self.i):
+                j = s.find("\n", self.i)
+                self.i = n if j < 0 else j
+            else:
+                break
+
+    def peek(self, lit: str) -> bool:
+        self.ws()
+        return self.s.startswith(lit, self.i)
+
+    def eat(self, lit: str) -> bool:
+        self.ws()
+        if self.s.startswith(lit, self.i):
+            self.i += len(lit)
+            return True
+        return False
+
+    def expect(self, lit: str):
+        if not self.eat(lit):
+            self.err(f"expected {lit!r}")
+
+    _ident = re.compile(r"[A-Za-z_][A-Za-z0-9_.$]*")
+    _ssa = re.compile(r"%[A-Za-z0-9_.$]+(#[0-9]+)?")
+    _num = re.compile(r"[-+]?(0x[0-9A-Fa-f]+|[0-9]+(\.[0-9]*)?([eE][-+]?[0-9]+)?|inf|nan)")
+
+    def ident(self) -> str:
+        self.ws()
+        m = self._ident.match(self.s, self.i)
+        if not m:
+            self.err("identifier expected")
+        self.i = m.end()
+        return m.group(0)
+
+    def try_ident(self) -> Optional[str]:
+        self.ws()
+        m = self._ident.match(self.s, self.i)
+        if not m:
+            return None
+        self.i = m.end()
+        return m.group(0)
+
+    def ssa(self) -> str:
+        self.ws()
+        m = self._ssa.match(self.s, self.i)
+        if not m:
+            self.err("SSA value expected")
+        self.i = m.end()
+        return m.group(0)
+
+    def string(self) -> str:
+        self.ws()
+        if self.s[self.i] != '"':
+            self.err("string expected")
+        j = self.i + 1
+        out = []
+        while self.s[j] != '"':
+            if self.s[j] == "\\":
+                out.append(self.s[j + 1])
+                j += 2
+            else:
+                out.append(self.s[j])
+                j += 1
+        self.i = j + 1
+        return "".join(out)
+
+    def integer(self) -> int:
+        self.ws()
+        m = re.compile(r"[-+]?[0-9]+").match(self.s, self.i)
+        if not m:
+            self.err("integer expected")
+        self.i = m.end()
+        return int(m.group(0))
+
+    def int_list(self, open_="[", close="]") -> List[int]:
+        self.expect(open_)
+        out = []
+        if self.eat(close):
+            return out
+        while True:
+            out.append(self.integer())
+            if self.eat(close):
+                return out
+            self.expect(",")
+
+    def type(self) -> TType:
+        self.ws()
+        if self.eat("tensor<"):
+            j = self.s.index(">", self.i)
+            body = self.s[self.i:j]
+            self.i = j + 1
+            parts = body.split("x")
+            dims = []
+            k = 0
+            while k < len(parts) - 1 and re.fullmatch(r"[0-9]+", parts[k]):
+                dims.append(int(parts[k]))
+                k += 1
+            dt = "x".join(parts[k:]).strip()
+            if "," in dt:
+                dt = dt.split(",")[0].strip()
+            return TType(dims, dt)
+        if self.eat("!stablehlo.token"):
+            return TType((), "token")
+        t = self.ident()  # bare scalar element type (i32, f32 ...) in attributes
+        return TType((), t)
+
+    def type_list_paren(self) -> List[TType]:
+        out = []
+        self.expect("(")
+        if self.eat(")"):
+            return out
+        while True:
+            out.append(self.type())
+            self.skip_attr_dict()
+            if self.eat(")"):
+                return out
+            self.expect(",")
+
+    def skip_attr_dict(self):
+        if self.peek("{"):
+            self.attr_dict()
+
+    # ---- attributes
+    def attr_value(self):
+        self.ws()
+        s = self.s
+        c = s[self.i]
+        if c == '"':
+            v = self.string()
+            if self.eat(":"):
+                self.type()
+            return v
+        if c == "[":
+            self.i += 1
+            out = []
+            if self.eat("]"):
+                return out
+            while True:
+                out.append(self.attr_value())
+                if self.eat("]"):
+                    return out
+                self.expect(",")
+        if c == "{":
+            return self.attr_dict()
+        if c == "#":
+            return self.hash_attr()
+        if c == "@":
+            self.i += 1
+            return "@" + self.ident()
+        if s.startswith("dense<", self.i):
+            return self.dense()
+        if s.startswith("array<", self.i):
+            self.i += 6
+            self.ident()
+            out = []
+            if self.eat(">"):
+                return out
+            self.expect(":")
+            while True:
+                out.append(self.integer() if not (self.peek("true") or self.peek("false")) else (self.ident() == "true"))
+                if self.eat(">"):
+                    return out
+                self.expect(",")
+        if s.startswith("true", self.i):
+            self.i += 4
+            return True
+        if s.startswith("false", self.i):
+            self.i += 5
+            return False
+        if s.startswith("unit", self.i):
+            self.i += 4
+            return True
+        m = self._num.match(s, self.i)
+        if m:
+            self.i = m.end()
+            tok = m.group(0)
+            isf = any(ch in tok for ch in ".eE") and not tok.lower().startswith(("0x", "-0x")) or tok in ("inf", "nan")
+            v = float(tok) if isf else int(tok, 0)
+            if self.eat(":"):
+                self.type()
+            return v
+        if s.startswith("tensor<", self.i):
+            return self.type()
+        idn = self.try_ident()
+        if idn is not None:
+            return idn
+        self.err("attribute value expected")
+
+    def hash_attr(self):
+        """#stablehlo.gather<...>, #stablehlo<precision DEFAULT>, #stablehlo.conv<...> ..."""
+        self.expect("#")
+        name = self.ident()
+        if not self.eat("<"):
+            return ("#" + name, None)
+        if name == "stablehlo":
+            kind = self.ident()
+            val = self.ident() if not self.peek(">") else None
+            self.expect(">")
+            return ("#" + kind, val)
+        d = {}
+        if name == "stablehlo.conv":
+            raw = self.raw_until_balanced(">")
+            return ("#stablehlo.conv", raw)
+        while not self.eat(">"):
+            k = self.ident()
+            self.expect("=")
+            d[k] = self.attr_value()
+            self.eat(",")
+        return ("#" + name, d)
+
+    def raw_until_balanced(self, close):
+        depth = 0
+        j = self.i
+        while True:
+            c = self.s[j]
+            if c in "<[({":
+                depth += 1
+            elif c in ">])}":
+                if depth == 0 and c == close:
+                    break
+                depth -= 1
+            j += 1
+        raw = self.s[self.i:j]
+        self.i = j + 1
+        return raw
+
+    def attr_dict(self) -> Dict[str, object]:
+        self.expect("{")
+        d = {}
+        if self.eat("}"):
+            return d
+        while True:
+            self.ws()
+            k = self.string() if self.s[self.i] == '"' else self.ident()
+            if self.eat("="):
+                d[k] = self.attr_value()
+            else:
+                d[k] = True
+            if self.eat("}"):
+                return d
+            self.expect(",")
+
+    def dense(self):
+        """dense<...> : tensor<...> -> numpy array (bf16 kept as rounded float32)."""
+        self.expect("dense<")
+        self.ws()
+        start = self.i
+        if self.s[self.i] == '"':
+            payload = ("hex", self.string())
+            self.expect(">")
+        else:
+            raw = self.raw_until_balanced(">")
+            payload = ("lit", raw)
+        self.expect(":")
+        t = self.type()
+        return _dense_to_numpy(payload, t)
+
+    # ---- module structure
+    def module(self) -> Dict[str, Func]:
+        funcs = {}
+        self.ws()
+        wrapped = False
+        if self.eat("module"):
+            wrapped = True
+            if self.eat("@"):
+                self.ident()
+            if self.eat("attributes"):
+                self.attr_dict()
+            self.expect("{")
+        while True:
+            self.ws()
+            if self.i >= self.n:
+                break
+            if wrapped and self.eat("}"):
+                break
+            f = self.func()
+            funcs[f.name] = f
+        return funcs
+
+    def func(self) -> Func:
+        self.expect("func.func")
+        self.ws()
+        if self.peek("public") or self.peek("private"):
+            self.ident()
+        self.expect("@")
+        f = Func(self.ident())
+        self.expect("(")
+        if not self.eat(")"):
+            while True:
+                f.body.args.append(self.ssa())
+                self.expect(":")
+                f.body.arg_types.append(self.type())
+                self.skip_attr_dict()
+                if self.eat(")"):
+                    break
+                self.expect(",")
+        if self.eat("->"):
+            if self.peek("("):
+                f.result_types = self.type_list_paren()
+            else:
+                f.result_types = [self.type()]
+                self.skip_attr_dict()
+        if self.eat("attributes"):
+            self.attr_dict()
+        self.expect("{")
+        self.block_ops(f.body)
+        self.expect("}")
+        return f
+
+    def block_ops(self, region: Region):
+        """Parse ops until the closing brace of the enclosing region (not consumed)."""
+        while True:
+            self.ws()
+            if self.peek("}"):
+                return
+            region.ops.append(self.op())
+
+    def region(self) -> Region:
+        """{ [^bb0(args):] ops }"""
+        r = Region()
+        self.expect("{")
+        self.ws()
+        if self.eat("^"):
+            self.ident()
+            if self.eat("("):
+                if not self.eat(")"):
+                    while True:
+                        r.args.append(self.ssa())
+                        self.expect(":")
+                        r.arg_types.append(self.type())
+                        if self.eat(")"):
+                            break
+                        self.expect(",")
+            self.expect(":")
+        self.block_ops(r)
+        self.expect("}")
+        return r
+
+    def op(self) -> Op:
+        op = Op()
+        self.ws()
+        nres = 1
+        if self.s[self.i] == "%":
+            m = re.compile(r"%[A-Za-z0-9_.$]+").match(self.s, self.i)
+            base = m.group(0)
+            self.i = m.end()
+            if self.eat(":"):
+                nres = self.integer()
+            self.expect("=")
+            op.results = [base] if nres == 1 else [f"{base}#{k}" for k in range(nres)]
+            has_res = True
+        else:
+            has_res = False
+        self.ws()
+        if self.s[self.i] == '"':
+            op.name = self.string()
+            self.generic_op(op)
+        else:
+            op.name = self.ident()
+            if op.name in ("return", "func.return", "stablehlo.return"):
+                op.name = "return"
+                if not self.peek("}"):
+                    self.ws()
+                    if self.s[self.i] == "%":
+                        op.operands = self.ssa_list()
+                        self.expect(":")
+                        op.in_types = self.types_bare()
+            elif op.name in ("call", "func.call"):
+                op.name = "call"
+                self.expect("@")
+                op.attrs["callee"] = self.ident()
+                self.expect("(")
+                op.operands = [] if self.peek(")") else self.ssa_list()
+                self.expect(")")
+                self.skip_attr_dict()
+                self.expect(":")
+                op.in_types = self.type_list_paren()
+                self.expect("->")
+                op.out_types = self.type_list_paren() if self.peek("(") else [self.type()]
+            else:
+                self.pretty_op(op)
+        if has_res and nres == 1 and len(op.out_types) > 1:
+            op.results = [f"{op.results[0]}#{k}" for k in range(len(op.out_types))]
+        return op
+
+    def ssa_list(self) -> List[str]:
+        out = [self.ssa()]
+        while True:
+            save = self.i
+            if not self.eat(","):
+                break
+            self.ws()
+            if self.i >= self.n or self.s[self.i] != "%":
+                self.i = save
+                break
+            out.append(self.ssa())
+        return out
+
+    def types_bare(self) -> List[TType]:
+        out = [self.type()]
+        while self.eat(","):
+            out.append(self.type())
+        return out
+
+    def fn_type(self, op: Op):
+        """(in types) -> out types   |   type (same for operands and result)"""
+        if self.peek("("):
+            op.in_types = self.type_list_paren()
+            self.expect("->")
+            op.out_types = self.type_list_paren() if self.peek("(") else [self.type()]
+        else:
+            t = self.type()
+            op.in_types = [t] * len(op.operands)
+            op.out_types = [t]
+
+    def generic_op(self, op: Op):
+        self.expect("(")
+        op.operands = [] if self.peek(")") else self.ssa_list()
+        self.expect(")")
+        if self.eat("<"):
+            op.attrs.update(self.attr_dict())
+            self.expect(">")
+        if self.peek("("):
+            self.expect("(")
+            while True:
+                op.regions.append(self.region())
+                if not self.eat(","):
+                    break
+            self.expect(")")
+        if self.peek("{"):
+            op.attrs.update(self.attr_dict())
+        self.expect(":")
+        op.in_types = self.type_list_paren()
+        self.expect("->")
+        op.out_types = self.type_list_paren() if self.peek("(") else [self.type()]
+
+    def pretty_op(self, op: Op):
+        n = op.name
+        short = n[len("stablehlo."):] if n.startswith("stablehlo.") else n
+        if short == "constant":
+            self.skip_attr_dict()
+            op.attrs["value"] = self.dense()
+            a = op.attrs["value"]
+            op.out_types = [a[1]]
+            op.attrs["value"] = a[0]
+            return
+        if short == "iota":
+            self.expect("dim")
+            self.expect("=")
+            op.attrs["iota_dimension"] = self.integer()
+            self.expect(":")
+            op.out_types = [self.type()]
+            return
+        if short == "compare":
+            op.attrs["comparison_direction"] = self.ident()
+            self.expect(",")
+            op.operands = [self.ssa()]
+            self.expect(",")
+            op.operands.append(self.ssa())
+            if self.eat(","):
+                op.attrs["compare_type"] = self.ident()
+            self.expect(":")
+            self.fn_type(op)
+            return
+        if short == "reduce":
+            return self.reduce_op(op)
+        if short == "while":
+            return self.while_op(op)
+        if short == "convolution":
+            return self.conv_op(op)
+        if short == "custom_call":
+            self.expect("@")
+            op.attrs["call_target_name"] = self.ident()
+            self.expect("(")
+            op.operands = [] if self.peek(")") else self.ssa_list()
+            self.expect(")")
+            if self.peek("{"):
+                op.attrs.update(self.attr_dict())
+            self.expect(":")
+            self.fn_type(op)
+            return
+        if short == "optimization_barrier":
+            op.operands = self.ssa_list() if self.peek("%") else []
+            self.expect(":")
+            ts = self.types_bare()
+            op.in_types = ts
+            op.out_types = ts
+            return
+        # generic pretty: operands, then keyword attrs, then type
+        self.ws()
+        if self.s[self.i] == "%":
+            op.operands = self.ssa_list()
+        if short == "slice":
+            self.expect("[")
+            st, li, sr = [], [], []
+            if not self.eat("]"):
+                while True:
+                    st.append(self.integer())
+                    self.expect(":")
+                    li.append(self.integer())
+                    sr.append(self.integer() if self.eat(":") else 1)
+                    if self.eat("]"):
+                        break
+                    self.expect(",")
+            op.attrs.update(start_indices=st, limit_indices=li, strides=sr)
+        while self.eat(","):
+            k = self.ident()
+            self.expect("=")
+            if k in ("batching_dims", "contracting_dims"):
+                a = self.int_list()
+                self.expect("x")
+                bb = self.int_list()
+                op.attrs[k] = (a, bb)
+            else:
+                op.attrs[k] = self.attr_value()
+        if self.peek("{"):
+            op.attrs.update(self.attr_dict())
+        self.expect(":")
+        if short == "select" and not self.peek("("):
+            tp = self.type()
+            self.expect(",")
+            tv = self.type()
+            op.in_types = [tp, tv, tv]
+            op.out_types = [tv]
+        else:
+            self.fn_type(op)
+
+    def reduce_op(self, op: Op):
+        # stablehlo.reduce(%x init: %c), (%y init: %d) [applies stablehlo.add] across dimensions = [..] : (..) -> ..
+        ins, inits = [], []
+        while True:
+            self.expect("(")
+            ins.append(self.ssa())
+            self.expect("init:")
+            inits.append(self.ssa())
+            self.expect(")")
+            if not self.eat(","):
+                break
+        op.operands = ins + inits
+        applies = None
+        if self.eat("applies"):
+            applies = self.ident()
+        self.expect("across")
+        self.expect("dimensions")
+        self.expect("=")
+        op.attrs["dimensions"] = self.int_list()
+        self.skip_attr_dict()
+        self.expect(":")
+        self.fn_type(op)
+        if applies is not None:
+            r = Region()
+            st = TType((), op.out_types[0].dtype)
+            r.args = ["%__a", "%__b"]
+            r.arg_types = [st, st]
+            o = Op()
+            o.name = applies
+            o.results = ["%__r"]
+            o.operands = ["%__a", "%__b"]
+            o.in_types = [st, st]
+            o.out_types = [st]
+            rt = Op()
+            rt.name = "return"
+            rt.operands = ["%__r"]
+            r.ops = [o, rt]
+            op.regions = [r]
+        else:
+            self.expect("reducer")
+            r = Region()
+            pairs = []
+            while self.eat("("):
+                a = self.ssa(); self.expect(":"); ta = self.type(); self.expect(",")
+                b_ = self.ssa(); self.expect(":"); tb = self.type(); self.expect(")")
+                pairs.append((a, ta, b_, tb))
+            r.args = [p[0] for p in pairs] + [p[2] for p in pairs]
+            r.arg_types = [p[1] for p in pairs] + [p[3] for p in pairs]
+            self.expect("{")
+            self.block_ops(r)
+            self.expect("}")
+            op.regions = [r]
+
+    def while_op(self, op: Op):
+        self.expect("(")
+        names = []
+        if not self.eat(")"):
+            while True:
+                names.append(self.ssa())
+                self.expect("=")
+                op.operands.append(self.ssa())
+                if self.eat(")"):
+                    break
+                self.expect(",")
+        if self.eat(":"):
+            ts = self.types_bare()
+        else:
+            ts = []
+        op.in_types = ts
+        op.out_types = ts
+        if self.eat("attributes"):
+            self.attr_dict()
+        self.expect("cond")
+        cond = Region()
+        cond.args, cond.arg_types = list(names), list(ts)
+        self.expect("{")
+        self.block_ops(cond)
+        self.expect("}")
+        self.expect("do")
+        body = Region()
+        body.args, body.arg_types = list(names), list(ts)
+        self.expect("{")
+        self.block_ops(body)
+        self.expect("}")
+        op.regions = [cond, body]
+
+    def conv_op(self, op: Op):
+        self.expect("(")
+        op.operands = self.ssa_list()
+        self.expect(")")
+        self.expect("dim_numbers")
+        self.expect("=")
+
+        def spec():
+            self.expect("[")
+            out = []
+            while True:
+                self.ws()
+                m = re.compile(r"[a-z0-9]+").match(self.s, self.i)
+                out.append(m.group(0))
+                self.i = m.end()
+                if self.eat("]"):
+                    return out
+                self.expect(",")
+        l = spec(); self.expect("x"); r = spec(); self.expect("->"); o = spec()
+        op.attrs["dim_numbers"] = (l, r, o)
+        self.expect(",")
+        self.expect("window")
+        self.expect("=")
+        self.expect("{")
+        win = {}
+        while not self.eat("}"):
+            k = self.ident()
+            self.expect("=")
+            win[k] = self.attr_value()
+            self.eat(",")
+        op.attrs["window"] = win
+        if self.peek("{"):
+            op.attrs.update(self.attr_dict())
+        self.expect(":")
+        self.fn_type(op)
+
+
+def _dense_to_numpy(payload, t: TType):
+    kind, raw = payload
+    dt = t.dtype
+    n = int(np.prod(t.shape)) if t.shape else 1
+    if kind == "hex":
+        b = bytes.fromhex(raw[2:])
+        if dt == "bf16":
+            a = bf16_bits_to_f32(np.frombuffer(b, dtype=np.uint16))
+        elif dt == "i1":
+            a = np.frombuffer(b, dtype=np.uint8).astype(np.bool_)
+        else:
+            a = np.frombuffer(b, dtype=_NP[dt])
+        if a.size == 1 and n != 1:
+            a = np.full(n, a[0])
+        return (a.reshape(t.shape).copy(), t)
+    toks = re.findall(r"[^\s,\[\]]+", raw)
+
+    def conv(tok):
+        if tok == "true":
+            return True
+        if tok == "false":
+            return False
+        if dt in FLOATS:
+            if tok.lower().startswith("0x"):
+                bits = int(tok, 16)
+                if dt == "f32":
+                    return np.array([bits], dtype=np.uint32).view(np.float32)[0]
+                if dt == "bf16":
+                    return bf16_bits_to_f32(np.array([bits], dtype=np.uint16))[0]
+                if dt == "f64":
+                    return np.array([bits], dtype=np.uint64).view(np.float64)[0]
+                if dt == "f16":
+                    return np.array([bits], dtype=np.uint16).view(np.float16)[0]
+            return float(tok)
+        return int(tok, 0)
+    vals = [conv(tk) for tk in toks]
+    if dt in FLOATS:
+        a = np.array(vals, dtype=np.float64).astype(_NP[dt])
+        if dt == "bf16":
+            a = round_bf16(a)
+    else:
+        a = np.array([int(v) for v in vals], dtype=object)
+        a = np.array([v & ((1 << 64) - 1) if dt == "ui64" else v for v in vals]).astype(_NP[dt])
+    if a.size == 1 and n != 1:
+        a = np.full(n, a.reshape(-1)[0], dtype=a.dtype)
+    return (a.reshape(t.shape), t)
+
+
+def parse(text: str) -> Dict[str, Func]:
+    return _P(text).module()
+
+
+# ----------------------------------------------------------------------------
+# interpreter
+# ----------------------------------------------------------------------------
+def _cast_result(a: np.ndarray, t: TType) -> np.ndarray:
+    a = np.asarray(a)
+    if t.dtype == "token":
+        return a
+    want = _NP[t.dtype]
+    if a.dtype != want:
+        a = a.astype(want)
+    if t.dtype == "bf16":
+        a = round_bf16(a)
+    if a.shape != t.shape:
+        a = a.reshape(t.shape)
+    return a
+
+
+class Oracle:
+    def __init__(self, text: str, accum: str = "f64"):
+        self.funcs = parse(text)
+        self.accum = np.float64 if accum == "f64" else np.float32
+        self.main = self.funcs["main"]
+
+    # -- public
+    def run(self, *args: np.ndarray) -> List[np.ndarray]:
+        f = self.main
+        assert len(args) == len(f.body.args), (len(args), len(f.body.args))
+        vals = [_cast_result(np.asarray(a), t) for a, t in zip(args, f.body.arg_types)]
+        return self._run_region(f.body, vals, {})
+
+    @property
+    def arg_types(self):
+        return [(t.shape, t.dtype) for t in self.main.body.arg_types]
+
+    @property
+    def result_types(self):
+        return [(t.shape, t.dtype) for t in self.main.result_types]
+
+    # -- engine
+    def _run_region(self, region: Region, args, outer_env) -> List[np.ndarray]:
+        env = dict(outer_env)
+        for n, v in zip(region.args, args):
+            env[n] = v
+        for op in region.ops:
+            if op.name == "return":
+                return [env[o] for o in op.operands]
+            ins = [env[o] for o in op.operands]
+            outs = self._eval(op, ins, env)
+            if not isinstance(outs, (list, tuple)):
+                outs = [outs]
+            for name, val, t in zip(op.results, outs, op.out_types):
+                env[name] = _cast_result(val, t)
+        return []
+
+    def _eval(self, op: Op, ins, env):
+        n = op.name
+        if n.startswith("stablehlo."):
+            n = n[10:]
+        elif n.startswith("chlo."):
+            n = "chlo_" + n[5:]
+        fn = getattr(self, "op_" + n, None)
+        if fn is None:
+            raise NotImplementedError(f"oracle: unsupported op {op.name}")
+        return fn(op, ins, env)
+
+    # ------------------------------------------------------------------
+    # elementwise (reference: ops/arithmetic.cc:535-607)
+    # ------------------------------------------------------------------
+    @staticmethod
+    def _f(op):
+        return op.out_types[0].dtype in FLOATS
+
+    def _un(self, op, ins, f):
+        x = ins[0]
+        dt = op.out_types[0].dtype
+        if dt in ("bf16", "f16"):
+            return f(x.astype(np.float32))
+        with np.errstate(all="ignore"):
+            return f(x)
+
+    def op_add(self, op, ins, env):
+        a, b = ins
+        if a.dtype == np.bool_:
+            return a | b
+        with np.errstate(all="ignore"):
+            return a + b
+
+    def op_subtract(self, op, ins, env):
+        with np.errstate(all="ignore"):
+            return ins[0] - ins[1]
+
+    def op_multiply(self, op, ins, env):
+        a, b = ins
+        if a.dtype == np.bool_:
+            return a & b
+        with np.errstate(all="ignore"):
+            return a * b
+
+    def op_divide(self, op, ins, env):
+        """Float: IEEE divide.  Integer: truncation toward zero (arithmetic.cc:496-513)."""
+        a, b = ins
+        with np.errstate(all="ignore"):
+            if a.dtype.kind == "f":
+                return a / b
+            bz = np.where(b == 0, 1, b)
+            if a.dtype.kind == "u":
+                q = a // bz
+                return np.where(b == 0, np.iinfo(a.dtype).max, q).astype(a.dtype)
+            q = np.abs(a.astype(np.int64)) // np.abs(bz.astype(np.int64))
+            q = np.where((a < 0) != (b < 0), -q, q)
+            return np.where(b == 0, -1, q).astype(a.dtype)
+
+    def op_remainder(self, op, ins, env):
+        """C-style remainder: sign follows the dividend (arithmetic.cc:46-83)."""
+        a, b = ins
+        with np.errstate(all="ignore"):
+            if a.dtype.kind == "f":
+                return np.fmod(a, b)
+            bz = np.where(b == 0, 1, b)
+            r = np.fmod(a, bz)
+            return np.where(b == 0, a, r).astype(a.dtype)
+
+    def op_maximum(self, op, ins, env):
+        a, b = ins
+        if a.dtype == np.bool_:
+            return a | b
+        return np.maximum(a, b)  # NaN-propagating, as in StableHLO
+
+    def op_minimum(self, op, ins, env):
+        a, b = ins
+        if a.dtype == np.bool_:
+            return a & b
+        return np.minimum(a, b)
+
+    def op_power(self, op, ins, env):
+        a, b = ins
+        with np.errstate(all="ignore"):
+            if a.dtype.kind == "f":
+                return np.power(a.astype(np.float64), b.astype(np.float64))
+            out = np.ones_like(a)
+            base, e = a.copy(), b.copy()
+            neg = e < 0 if e.dtype.kind == "i" else np.zeros(e.shape, bool)
+            e = np.where(neg, 0, e)
+            for _ in range(64):
+                out = np.where((e & 1) == 1, out * base, out)
+                base = base * base
+                e = e >> 1
+            special = np.where(a == 1, 1, np.where(a == -1, np.where((b & 1) == 1, -1, 1), 0)) if a.dtype.kind == "i" else np.where(a == 1, 1, 0)
+            return np.where(neg, special, out).astype(a.dtype)
+
+    def op_atan2(self, op, ins, env): return np.arctan2(ins[0].astype(np.float64), ins[1].astype(np.float64))
+    def op_and(self, op, ins, env): return ins[0] & ins[1]
+    def op_or(self, op, ins, env): return ins[0] | ins[1]
+    def op_xor(self, op, ins, env): return ins[0] ^ ins[1]
+
+    def op_not(self, op, ins, env):
+        x = ins[0]
+        return ~x
+
+    @staticmethod
+    def _bits(dt):
+        return np.dtype(dt).itemsize * 8
+
+    def op_shift_left(self, op, ins, env):
+        """Shift amounts >= bit width give 0 (mlx_executable.cc:293-301)."""
+        a, b = ins
+        w = self._bits(a.dtype)
+        ub = b.astype(np.uint64)
+        ok = ub < w
+        u = a.view(np.dtype(f"u{a.dtype.itemsize}"))
+        r = (u << np.where(ok, ub, 0).astype(u.dtype)).astype(u.dtype)
+        return np.where(ok, r, 0).astype(u.dtype).view(a.dtype)
+
+    def op_shift_right_logical(self, op, ins, env):
+        a, b = ins
+        w = self._bits(a.dtype)
+        ub = b.astype(np.uint64)
+        ok = ub < w
+        u = a.view(np.dtype(f"u{a.dtype.itemsize}"))
+        r = (u >> np.where(ok, ub, 0).astype(u.dtype)).astype(u.dtype)
+        return np.where(ok, r, 0).astype(u.dtype).view(a.dtype)
+
+    def op_shift_right_arithmetic(self, op, ins, env):
+        """Out-of-range shift fills with the sign bit (arithmetic.cc:119-143)."""
+        a, b = ins
+        w = self._bits(a.dtype)
+        ub = b.astype(np.uint64)
+        sh = np.minimum(ub, w - 1).astype(a.dtype)
+        return a >> sh
+
+    def op_popcnt(self, op, ins, env):
+        a = ins[0]
+        u = a.view(np.dtype(f"u{a.dtype.itemsize}")).astype(np.uint64)
+        c = np.zeros(a.shape, np.uint64)
+        for k in range(self._bits(a.dtype)):
+            c += (u >> np.uint64(k)) & np.uint64(1)
+        return c.astype(a.dtype)
+
+    def op_count_leading_zeros(self, op, ins, env):
+        a = ins[0]
+        w = self._bits(a.dtype)
+        u = a.view(np.dtype(f"u{a.dtype.itemsize}")).astype(np.uint64)
+        c = np.full(a.shape, w, np.int64)
+        for k in range(w):
+            c = np.where((u >> np.uint64(k)) != 0, w - 1 - k, c)
+        return c.astype(a.dtype)
+
+    def op_negate(self, op, ins, env):
+        with np.errstate(all="ignore"):
+            return -ins[0]
+
+    def op_abs(self, op, ins, env):
+        with np.errstate(all="ignore"):
+            return np.abs(ins[0])
+
+    def _f64un(self, op, ins, f):
+        x = ins[0].astype(np.float64)
+        with np.errstate(all="ignore"):
+            return f(x)
+
+    def op_exponential(self, op, ins, env): return self._f64un(op, ins, np.exp)
+    def op_exponential_minus_one(self, op, ins, env): return self._f64un(op, ins, np.expm1)
+    def op_log(self, op, ins, env): return self._f64un(op, ins, np.log)
+    def op_log_plus_one(self, op, ins, env): return self._f64un(op, ins, np.log1p)
+    def op_sqrt(self, op, ins, env): return self._un(op, ins, np.sqrt)
+    def op_cbrt(self, op, ins, env): return self._f64un(op, ins, np.cbrt)
+    def op_rsqrt(self, op, ins, env): return self._f64un(op, ins, lambda x: 1.0 / np.sqrt(x))
+    def op_tanh(self, op, ins, env): return self._f64un(op, ins, np.tanh)
+    def op_tan(self, op, ins, env): return self._f64un(op, ins, np.tan)
+    def op_sine(self, op, ins, env): return self._f64un(op, ins, np.sin)
+    def op_cosine(self, op, ins, env): return self._f64un(op, ins, np.cos)
+    def op_logistic(self, op, ins, env): return self._f64un(op, ins, lambda x: 1.0 / (1.0 + np.exp(-x)))
+    def op_floor(self, op, ins, env): return self._un(op, ins, np.floor)
+    def op_ceil(self, op, ins, env): return self._un(op, ins, np.ceil)
+    def op_round_nearest_even(self, op, ins, env): return self._un(op, ins, np.rint)
+
+    def op_round_nearest_afz(self, op, ins, env):
+        """Half away from zero (arithmetic.cc:316-327)."""
+        return self._un(op, ins, lambda x: np.where(np.isfinite(x), np.sign(x) * np.floor(np.abs(x) + 0.5), x))
+
+    def op_is_finite(self, op, ins, env): return np.isfinite(ins[0])
+
+    def op_sign(self, op, ins, env):
+        """NaN stays NaN, -0 stays -0 (arithmetic.cc:517-531)."""
+        x = ins[0]
+        if x.dtype.kind == "f":
+            with np.errstate(all="ignore"):
+                return np.where(np.isnan(x), x, np.where(x == 0, x, np.sign(x)))
+        return np.sign(x)
+
+    def op_erf(self, op, ins, env):
+        from scipy import special
+        return special.erf(ins[0].astype(np.float64))
+    op_chlo_erf = op_erf
+
+    def op_clamp(self, op, ins, env):
+        lo, x, hi = ins
+        return np.minimum(np.maximum(x, lo), hi)
+
+    def op_select(self, op, ins, env):
+        p, a, b = ins
+        return np.where(p, a, b)
+
+    def op_compare(self, op, ins, env):
+        """EQ/NE/LT/LE/GT/GE; TOTALORDER compares the sign-magnitude key (arithmetic.cc:239-313)."""
+        a, b = ins
+        d = op.attrs["comparison_direction"]
+        if op.attrs.get("compare_type") == "TOTALORDER" and a.dtype.kind == "f":
+            def key(x):
+                x = x.astype(np.float32) if x.dtype != np.float64 else x
+                w = 32 if x.dtype == np.float32 else 64
+                i = x.view(np.int32 if w == 32 else np.int64)
+                mask = np.iinfo(i.dtype).max
+                return np.where(i < 0, i ^ mask, i)
+            a, b = key(a), key(b)
+        with np.errstate(all="ignore"):
+            return {"EQ": np.equal, "NE": np.not_equal, "LT": np.less, "LE": np.less_equal,
+                    "GT": np.greater, "GE": np.greater_equal}[d](a, b)
+
+    def op_convert(self, op, ins, env):
+        """Value conversion; float->int truncates toward zero and saturates, NaN->0 (XLA rule)."""
+        x = ins[0]
+        dt = op.out_types[0].dtype
+        want = np.dtype(_NP[dt])
+        if want == np.bool_:
+            return x != 0
+        if x.dtype.kind == "f" and want.kind in "iu":
+            info = np.iinfo(want)
+            with np.errstate(all="ignore"):
+                t = np.trunc(x.astype(np.float64))
+                t = np.where(np.isnan(t), 0, t)
+                t = np.clip(t, float(info.min), float(info.max))
+                out = np.empty(x.shape, dtype=want)
+                hi = t >= float(info.max)
+                lo = t <= float(info.min)
+                mid = ~(hi | lo)
+                out[hi] = info.max
+                out[lo] = info.min
+                out[mid] = t[mid].astype(want)
+                return out
+        with np.errstate(all="ignore"):
+            return x.astype(want)
+
+    def op_bitcast_convert(self, op, ins, env):
+        x = ins[0]
+        it, ot = op.in_types[0].dtype, op.out_types[0].dtype
+        if it == "bf16":
+            x = f32_to_bf16_bits(x)
+        x = np.ascontiguousarray(x)
+        if ot == "bf16":
+            return bf16_bits_to_f32(x.view(np.uint16).reshape(op.out_types[0].shape))
+        return x.view(_NP[ot]).reshape(op.out_types[0].shape)
+
+    def op_reduce_precision(self, op, ins, env):
+        x = ins[0].astype(np.float32)
+        eb, mb = int(op.attrs["exponent_bits"]), int(op.attrs["mantissa_bits"])
+        u = x.view(np.uint32).copy()
+        if mb < 23:
+            sh = 23 - mb
+            lsb = (u >> np.uint32(sh)) & np.uint32(1)
+            rnd = np.uint32((1 << (sh - 1)) - 1) + lsb
+            nan = np.isnan(x)
+            u2 = (u + rnd) & np.uint32(~((1 << sh) - 1) & 0xFFFFFFFF)
+            u = np.where(nan, u, u2)
+        y = u.view(np.float32)
+        if eb < 8:
+            maxexp = (1 << (eb - 1)) - 1
+            minexp = 1 - maxexp
+            e = ((u >> np.uint32(23)) & np.uint32(0xFF)).astype(np.int32) - 127
+            sign = np.signbit(y)
+            big = (e > maxexp) & np.isfinite(x)
+            small = (e < minexp)
+            y = np.where(big, np.where(sign, -np.inf, np.inf), y)
+            y = np.where(small & ~np.isnan(x), np.where(sign, -0.0, 0.0), y)
+        return y.astype(np.float32)
+
+    # ------------------------------------------------------------------
+    # shape / data movement (reference: ops/shape.cc:260-270, ops/slice.cc:280-285)
+    # ------------------------------------------------------------------
+    def op_constant(self, op, ins, env): return op.attrs["value"]
+
+    def op_iota(self, op, ins, env):
+        t = op.out_types[0]
+        d = op.attrs["iota_dimension"]
+        shp = [1] * len(t.shape)
+        shp[d] = t.shape[d]
+        return np.broadcast_to(np.arange(t.shape[d]).reshape(shp), t.shape).astype(_NP[t.dtype])
+
+    def op_reshape(self, op, ins, env): return ins[0].reshape(op.out_types[0].shape)
+
+    def op_broadcast_in_dim(self, op, ins, env):
+        x = ins[0]
+        dims = op.attrs.get("dims", op.attrs.get("broadcast_dimensions"))
+        shape = op.out_types[0].shape
+        shp = [1] * len(shape)
+        for k, d in enumerate(dims):
+            shp[d] = x.shape[k]
+        return np.broadcast_to(x.reshape(shp), shape).copy()
+
+    def op_transpose(self, op, ins, env):
+        return np.ascontiguousarray(np.transpose(ins[0], op.attrs.get("dims", op.attrs.get("permutation"))))
+
+    def op_reverse(self, op, ins, env):
+        return np.flip(ins[0], axis=tuple(op.attrs.get("dims", op.attrs.get("dimensions")))).copy()
+
+    def op_concatenate(self, op, ins, env):
+        return np.concatenate(ins, axis=op.attrs.get("dim", op.attrs.get("dimension")))
+
+    def op_slice(self, op, ins, env):
+        sl = tuple(slice(s, l, st) for s, l, st in zip(op.attrs["start_indices"], op.attrs["limit_indices"], op.attrs["strides"]))
+        return ins[0][sl].copy()
+
+    @staticmethod
+    def _clamped_starts(starts, opshape, sizes):
+        """start = max(0, min(start, dim - size)) (slice.cc:90-107)."""
+        out = []
+        for s, d, z in zip(starts, opshape, sizes):
+            out.append(int(max(0, min(int(np.asarray(s).reshape(())), d - z))))
+        return out
+
+    def op_dynamic_slice(self, op, ins, env):
+        x = ins[0]
+        sizes = op.attrs.get("sizes", op.attrs.get("slice_sizes"))
+        st = self._clamped_starts(ins[1:], x.shape, sizes)
+        return x[tuple(slice(s, s + z) for s, z in zip(st, sizes))].copy()
+
+    def op_dynamic_update_slice(self, op, ins, env):
+        x, u = ins[0], ins[1]
+        st = self._clamped_starts(ins[2:], x.shape, u.shape)
+        out = x.copy()
+        out[tuple(slice(s, s + z) for s, z in zip(st, u.shape))] = u
+        return out
+
+    def op_pad(self, op, ins, env):
+        """Interior dilation first, then edge padding; negative edge padding crops (slice.cc:202-276)."""
+        x, pv = ins
+        lo, hi, it = op.attrs["low"], op.attrs["high"], op.attrs["interior"]
+        shp = [d + max(d - 1, 0) * i for d, i in zip(x.shape, it)]
+        y = np.full(shp, pv, dtype=x.dtype)
+        y[tuple(slice(0, None, i + 1) for i in it)] = x
+        out_shape = op.out_types[0].shape
+        out = np.full(out_shape, pv, dtype=x.dtype)
+        src, dst = [], []
+        for d in range(x.ndim):
+            s0 = max(0, -lo[d])
+            s1 = shp[d] - max(0, -hi[d])
+            d0 = max(0, lo[d])
+            src.append(slice(s0, max(s0, s1)))
+            dst.append(slice(d0, d0 + max(0, s1 - s0)))
+        out[tuple(dst)] = y[tuple(src)]
+        return out
+
+    # ------------------------------------------------------------------
+    # reductions (reference: ops/reduction.cc:83-162)
+    # ------------------------------------------------------------------
+    def op_reduce(self, op, ins, env):
+        k = len(ins) // 2
+        xs, inits = ins[:k], ins[k:]
+        dims = tuple(op.attrs["dimensions"])
+        body = op.regions[0]
+        if k == 1 and len(body.ops) == 2 and body.ops[0].name.startswith("stablehlo.") \
+                and set(body.ops[0].operands) == set(body.args) and len(dims) > 0:
+            kind = body.ops[0].name[10:]
+            x, init = xs[0], inits[0]
+            dt = op.out_types[0].dtype
+            red = None
+            with np.errstate(all="ignore"):
+                if kind == "add":
+                    if dt in FLOATS:
+                        red = np.sum(x.astype(self.accum), axis=dims) + init.astype(self.accum)
+                    elif dt == "i1":
+                        red = np.any(x, axis=dims) | init
+                    else:
+                        red = np.add.reduce(x, axis=dims, dtype=x.dtype) + init
+                elif kind == "multiply":
+                    red = (np.prod(x.astype(self.accum), axis=dims) * init) if dt in FLOATS else np.multiply.reduce(x, axis=dims, dtype=x.dtype) * init
+                elif kind == "maximum":
+                    red = np.maximum(np.max(x, axis=dims, initial=None) if x.size else np.full(op.out_types[0].shape, init), init)
+                elif kind == "minimum":
+                    red = np.minimum(np.min(x, axis=dims, initial=None) if x.size else np.full(op.out_types[0].shape, init), init)
+                elif kind == "and":
+                    red = np.bitwise_and.reduce(x, axis=dims) & init if x.size else np.full(op.out_types[0].shape, init)
+                elif kind == "or":
+                    red = np.bitwise_or.reduce(x, axis=dims) | init if x.size else np.full(op.out_types[0].shape, init)
+            if red is not None:
+                return [red]
+        # generic fold in row-major order of the reduced dims
+        keep = [d for d in range(xs[0].ndim) if d not in dims]
+        perm = list(dims) + keep
+        xt = [np.transpose(x, perm).reshape((-1,) + tuple(x.shape[d] for d in keep)) for x in xs]
+        acc = [np.broadcast_to(i, xt[0].shape[1:]).astype(i.dtype).copy() for i in inits]
+        for r in range(xt[0].shape[0]):
+            acc = self._run_region(body, acc + [x[r] for x in xt], env)
+        return acc
+
+    # ------------------------------------------------------------------
+    # contractions (reference: ops/linalg.cc:89-250, 253-550)
+    # ------------------------------------------------------------------
+    def op_dot_general(self, op, ins, env):
+        a, b = ins
+        if "dot_dimension_numbers" in op.attrs:
+            d = op.attrs["dot_dimension_numbers"][1]
+            ba, bb = d.get("lhs_batching_dimensions", []), d.get("rhs_batching_dimensions", [])
+            ca, cb = d.get("lhs_contracting_dimensions", []), d.get("rhs_contracting_dimensions", [])
+        else:
+            ba, bb = op.attrs.get("batching_dims", ([], []))
+            ca, cb = op.attrs.get("contracting_dims", ([], []))
+        fa = [i for i in range(a.ndim) if i not in ca and i not in ba]
+        fb = [i for i in range(b.ndim) if i not in cb and i not in bb]
+        isf = a.dtype.kind == "f"
+        acc = self.accum if isf else (np.int64 if a.dtype.kind in "iub" else a.dtype)
+        at = np.transpose(a, list(ba) + fa + list(ca)).astype(acc)
+        bt = np.transpose(b, list(bb) + list(cb) + fb).astype(acc)
+        B = int(np.prod([a.shape[i] for i in ba])) if ba else 1
+        M = int(np.prod([a.shape[i] for i in fa])) if fa else 1
+        K = int(np.prod([a.shape[i] for i in ca])) if ca else 1
+        N = int(np.prod([b.shape[i] for i in fb])) if fb else 1
+        r = np.matmul(at.reshape(B, M, K), bt.reshape(B, K, N))
+        if op.out_types[0].dtype == "i1":
+            r = r != 0
+        return r.reshape(op.out_types[0].shape)
+
+    def op_convolution(self, op, ins, env):
+        """StableHLO order of operations: dilate lhs, pad (may be negative), dilate rhs, slide."""
+        lhs, rhs = ins
+        if "dim_numbers" in op.attrs:
+            ls, rs, os_ = op.attrs["dim_numbers"]
+            win = op.attrs.get("window", {})
+            nsp = len(ls) - 2
+            strides = win.get("stride", [1] * nsp)
+            pad = win.get("pad", [[0, 0]] * nsp)
+            ldil = win.get("lhs_dilate", [1] * nsp)
+            rdil = win.get("rhs_dilate", [1] * nsp)
+            wrev = win.get("reverse", [False] * nsp)
+        else:
+            raise NotImplementedError("generic-form convolution attributes")
+        fg = int(op.attrs.get("feature_group_count", 1))
+        bg = int(op.attrs.get("batch_group_count", 1))
+        sp = [str(k) for k in range(nsp)]
+        l_perm = [ls.index("b")] + [ls.index(s) for s in sp] + [ls.index("f")]
+        r_perm = [rs.index(s) for s in sp] + [rs.index("i"), rs.index("o")]
+        x = np.transpose(lhs, l_perm).astype(self.accum)
+        w = np.transpose(rhs, r_perm).astype(self.accum)
+        for d in range(nsp):
+            if wrev[d] in (True, "true"):
+                w = np.flip(w, axis=d)
+        # lhs dilation
+        shp = list(x.shape)
+        for d in range(nsp):
+            shp[1 + d] = (x.shape[1 + d] - 1) * ldil[d] + 1 if x.shape[1 + d] > 0 else 0
+        xd = np.zeros(shp, dtype=x.dtype)
+        xd[(slice(None),) + tuple(slice(0, None, ldil[d]) for d in range(nsp)) + (slice(None),)] = x
+        # padding (negative crops)
+        shp2 = list(xd.shape)
+        src, dst = [slice(None)], [slice(None)]
+        for d in range(nsp):
+            lo, hi = pad[d]
+            shp2[1 + d] = max(0, xd.shape[1 + d] + lo + hi)
+            s0, s1 = max(0, -lo), xd.shape[1 + d] - max(0, -hi)
+            d0 = max(0, lo)
+            src.append(slice(s0, max(s0, s1)))
+            dst.append(slice(d0, d0 + max(0, s1 - s0)))
+        src.append(slice(None)); dst.append(slice(None))
+        xp = np.zeros(shp2, dtype=x.dtype)
+        xp[tuple(dst)] = xd[tuple(src)]
+        # rhs dilation
+        wshp = list(w.shape)
+        for d in range(nsp):
+            wshp[d] = (w.shape[d] - 1) * rdil[d] + 1 if w.shape[d] > 0 else 0
+        wd = np.zeros(wshp, dtype=w.dtype)
+        wd[tuple(slice(0, None, rdil[d]) for d in range(nsp)) + (slice(None), slice(None))] = w
+        out_shape = op.out_types[0].shape
+        osp = [out_shape[os_.index(s)] for s in sp]
+        N = x.shape[0]
+        Cin = x.shape[-1]
+        O = w.shape[-1]
+        G = fg * bg
+        res = np.zeros([N // bg] + osp + [O], dtype=self.accum)
+        # windows as strided view: [N, out..., k..., C]
+        for g in range(G):
+            if fg > 1:
+                cs = Cin // fg
+                xg = xp[..., g * cs:(g + 1) * cs]
+                wg = wd[..., g * (O // fg):(g + 1) * (O // fg)]
+                osl = slice(g * (O // fg), (g + 1) * (O // fg))
+            elif bg > 1:
+                nb = N // bg
+                xg = xp[g * nb:(g + 1) * nb]
+                wg = wd[..., g * (O // bg):(g + 1) * (O // bg)]
+                osl = slice(g * (O // bg), (g + 1) * (O // bg))
+            else:
+                xg, wg, osl = xp, wd, slice(None)
+            acc = np.zeros([xg.shape[0]] + osp + [wg.shape[-1]], dtype=self.accum)
+            # accumulate one kernel tap at a time: a GEMM per tap, no im2col blow-up
+            for tap in np.ndindex(*wd.shape[:nsp]):
+                wt = wg[tap]
+                if not np.any(wt):
+                    continue
+                sl = [slice(None)]
+                for d in range(nsp):
+                    sl.append(slice(tap[d], tap[d] + (osp[d] - 1) * strides[d] + 1, strides[d]))
+                sl.append(slice(None))
+                patch = xg[tuple(sl)]
+                acc += np.matmul(patch.reshape(-1, patch.shape[-1]), wt).reshape(acc.shape)
+            res[..., osl] = acc
+        # to output layout
+        cur = ["b"] + sp + ["f"]
+        return np.transpose(res, [cur.index(c) for c in os_])
+
+    # ------------------------------------------------------------------
+    # gather / scatter (reference: ops/gather_scatter.cc:200-294, 296-699)
+    # ------------------------------------------------------------------
+    @staticmethod
+    def _dn(op, key):
+        v = op.attrs[key]
+        return v[1] if isinstance(v, tuple) else v
+
+    def op_gather(self, op, ins, env):
+        operand, idx = ins
+        dn = self._dn(op, "dimension_numbers")
+        offset_dims = dn.get("offset_dims", [])
+        collapsed = dn.get("collapsed_slice_dims", [])
+        obatch = dn.get("operand_batching_dims", [])
+        ibatch = dn.get("start_indices_batching_dims", [])
+        sim = dn.get("start_index_map", [])
+        ivd = dn.get("index_vector_dim", idx.ndim)
+        sizes = op.attrs["slice_sizes"]
+        out_shape = op.out_types[0].shape
+        if ivd == idx.ndim:
+            idx = idx[..., None]
+        idxm = np.moveaxis(idx, ivd, -1).astype(np.int64)       # [batch..., K]
+        batch_dims_out = [d for d in range(len(out_shape)) if d not in offset_dims]
+        grids = np.indices(out_shape, sparse=True)
+        bidx = tuple(grids[d] for d in batch_dims_out)
+        # operand dims that carry an offset
+        off_operand_dims = [d for d in range(operand.ndim) if d not in collapsed and d not in obatch]
+        index = [0] * operand.ndim
+        for d in range(operand.ndim):
+            index[d] = np.zeros((), dtype=np.int64)
+        for k, d in enumerate(sim):
+            start = idxm[bidx + (k,)] if bidx else idxm[..., k].reshape(())
+            start = np.clip(start, 0, operand.shape[d] - sizes[d])   # clamp rule gather_scatter.cc:233-239
+            index[d] = index[d] + start
+        # batching dims: position in the batch index space (index_vector_dim removed)
+        idx_batch_axes = [a for a in range(idx.ndim) if a != ivd]
+        for od, ib in zip(obatch, ibatch):
+            pos = idx_batch_axes.index(ib)
+            index[od] = index[od] + grids[batch_dims_out[pos]]
+        for k, d in enumerate(off_operand_dims):
+            index[d] = index[d] + grids[offset_dims[k]]
+        index = np.broadcast_arrays(*index) if operand.ndim else []
+        return operand[tuple(index)].reshape(out_shape)
+
+    def op_scatter(self, op, ins, env):
+        """Updates are applied in row-major order of the update tensor, one after
+        the other (the order XLA's CPU backend uses), so duplicate indices
+        accumulate deterministically.  A window that does not fit entirely inside
+        the operand is dropped."""
+        k = len(ins) // 2 if len(ins) > 3 else 1
+        operand, idx, upd = ins[0], ins[-2] if len(ins) == 3 else ins[k], ins[-1]
+        assert len(ins) == 3, "variadic scatter not needed on this path"
+        dn = self._dn(op, "scatter_dimension_numbers")
+        uwd = dn.get("update_window_dims", [])
+        iwd = dn.get("inserted_window_dims", [])
+        ibd = dn.get("input_batching_dims", [])
+        sibd = dn.get("scatter_indices_batching_dims", [])
+        sdo = dn.get("scatter_dims_to_operand_dims", [])
+        ivd = dn.get("index_vector_dim", idx.ndim)
+        if ivd == idx.ndim:
+            idx = idx[..., None]
+        idxm = np.moveaxis(idx, ivd, -1).astype(np.int64)
+        scatter_dims_upd = [d for d in range(upd.ndim) if d not in uwd]
+        grids = np.indices(upd.shape, sparse=True)
+        bidx = tuple(grids[d] for d in scatter_dims_upd)
+        win_operand_dims = [d for d in range(operand.ndim) if d not in iwd and d not in ibd]
+        win_sizes = {d: upd.shape[uwd[k_]] for k_, d in enumerate(win_operand_dims)}
+        index = [np.zeros((), dtype=np.int64) for _ in range(operand.ndim)]
+        inb = np.ones((), dtype=bool)
+        for k_, d in enumerate(sdo):
+            start = idxm[bidx + (k_,)] if bidx else idxm[..., k_].reshape(())
+            ws = win_sizes.get(d, 1)
+            inb = inb & (start >= 0) & (start <= operand.shape[d] - ws)
+            index[d] = index[d] + start
+        idx_batch_axes = [a for a in range(idx.ndim) if a != ivd]
+        for od, ib in zip(ibd, sibd):
+            pos = idx_batch_axes.index(ib)
+            index[od] = index[od] + grids[scatter_dims_upd[pos]]
+        for k_, d in enumerate(win_operand_dims):
+            index[d] = index[d] + grids[uwd[k_]]
+        bc = np.broadcast_arrays(*(index + [inb, np.zeros(upd.shape, dtype=bool)]))
+        index, inb = bc[:-2], bc[-2]
+        flat = np.ravel_multi_index([i.reshape(-1) for i in index], operand.shape, mode="clip") if operand.ndim else np.zeros(upd.size, np.int64)
+        inb = inb.reshape(-1)
+        flat = flat[inb]
+        u = upd.reshape(-1)[inb]
+        out = operand.copy().reshape(-1)
+        body = op.regions[0]
+        kind = None
+        if len(body.ops) == 1 and body.ops[0].name == "return" and body.ops[0].operands == [body.args[1]]:
+            kind = "set"
+        elif len(body.ops) == 2 and set(body.ops[0].operands) == set(body.args):
+            kind = body.ops[0].name.replace("stablehlo.", "")
+            if kind == "subtract" and body.ops[0].operands != body.args:
+                kind = None
+        with np.errstate(all="ignore"):
+            if kind == "set":
+                out[flat] = u
+            elif kind == "add":
+                if out.dtype == np.bool_:
+                    np.logical_or.at(out, flat, u)
+                else:
+                    np.add.at(out, flat, u)
+            elif kind == "subtract":
+                np.subtract.at(out, flat, u)
+            elif kind == "multiply":
+                np.multiply.at(out, flat, u)
+            elif kind == "minimum":
+                np.minimum.at(out, flat, u)
+            elif kind == "maximum":
+                np.maximum.at(out, flat, u)
+            else:
+                t = op.out_types[0]
+                st = TType((), t.dtype)
+                for j in range(flat.size):
+                    r = self._run_region(body, [np.asarray(out[flat[j]]), np.asarray(u[j])], env)[0]
+                    out[flat[j]] = _cast_result(r, st)
+        return out.reshape(operand.shape)
+
+    # ------------------------------------------------------------------
+    # control flow (reference: ops/control_flow.cc:702-989, 992-1277)
+    # ------------------------------------------------------------------
+    def op_while(self, op, ins, env):
+        cond, body = op.regions
+        state = list(ins)
+        while bool(np.asarray(self._run_region(cond, state, env)[0]).reshape(())):
+            state = [_cast_result(v, t) for v, t in zip(self._run_region(body, state, env), op.out_types)]
+        return state
+
+    def op_case(self, op, ins, env):
+        """Out-of-range index selects the last branch (control_flow.cc:672-675)."""
+        i = int(np.asarray(ins[0]).reshape(()))
+        nb = len(op.regions)
+        if i < 0 or i >= nb:
+            i = nb - 1
+        return self._run_region(op.regions[i], [], env)
+
+    def op_call(self, op, ins, env):
+        f = self.funcs[op.attrs["callee"]]
+        return self._run_region(f.body, ins, {})
+
+    def op_optimization_barrier(self, op, ins, env): return list(ins)
+
+    def op_custom_call(self, op, ins, env):
+        tgt = op.attrs.get("call_target_name")
+        if tgt in ("Sharding", "SPMDFullToShardShape", "SPMDShardToFullShape"):
+            return ins[0]
+        raise NotImplementedError(f"oracle: custom_call {tgt}")
+
+
+def run_text(text: str, *args, accum="f64"):
+    return Oracle(text, accum=accum).run(*args)
