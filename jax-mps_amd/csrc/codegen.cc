@@ -1,0 +1,1308 @@
+// Generator of fused HIP kernels (loop fusion, dynamic_update_slice windows and
+// reductions).  Every generated kernel is built from the same hand-written
+// skeletons below: a streaming skeleton that moves 16 bytes per lane with
+// vector loads/stores, a row-reduction skeleton (lanes along the reduced,
+// contiguous axis; wavefront shuffles then one LDS step) and a column-reduction
+// skeleton (lanes along the kept, contiguous axis; LDS step across row groups;
+// optional second pass over partials).  Only the per-element expression inside
+// the skeleton is produced from the StableHLO ops.
+//
+// Op semantics follow the reference's handlers: ops/arithmetic.cc:535-607
+// (elementwise, compare, shifts, remainder, integer divide, sign, rounding),
+// ops/shape.cc:260-270, ops/slice.cc:90-276 (clamped dynamic starts, pad),
+// ops/gather_scatter.cc:200-294 (gather with clamped starts),
+// ops/reduction.cc:83-162 (reduce by body pattern).
+#include "codegen.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <numeric>
+#include <sstream>
+#include <unordered_map>
+
+namespace mi355 {
+
+namespace {
+
+const char* kPrelude = R"HIP(
+typedef unsigned short u16; typedef unsigned int u32; typedef unsigned long long u64; typedef long long i64;
+typedef signed char i8; typedef unsigned char u8; typedef short i16;
+template <typename T, int N> struct __attribute__((aligned(sizeof(T) * N))) Vec { T e[N]; };
+__device__ __forceinline__ float bf2f(u16 b) { return __uint_as_float(((u32)b) << 16); }
+__device__ __forceinline__ u16 f2bf(float f) {
+  u32 u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u16)((u >> 16) | 0x40);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (u16)(u >> 16);
+}
+__device__ __forceinline__ float bfr(float f) { return bf2f(f2bf(f)); }
+__device__ __forceinline__ float hfr(float f) { return (float)(_Float16)f; }
+template <typename T> __device__ __forceinline__ T mx(T a, T b) { return (a > b || a != a) ? a : b; }
+template <typename T> __device__ __forceinline__ T mn(T a, T b) { return (a < b || a != a) ? a : b; }
+template <typename I, typename F> __device__ __forceinline__ I f2i(F f) {
+  if (f != f) return (I)0;
+  const bool sg = (I)(-1) < (I)0;
+  const int bits = (int)sizeof(I) * 8;
+  const F hi = sg ? (F)(1ull << (bits - 1)) : (bits == 64 ? (F)18446744073709551615.0 : (F)(1ull << (bits & 63)));
+  if (f >= hi) return sg ? (I)((1ull << (bits - 1)) - 1ull) : (I)~(I)0;
+  if (sg) { if (f <= -hi) return (I)(1ull << (bits - 1)); }
+  else if (f <= (F)0) return (I)0;
+  return (I)f;
+}
+template <typename T> __device__ __forceinline__ T ipow(T a, T b) {
+  if (b < (T)0) return a == (T)1 ? (T)1 : (a == (T)-1 ? ((b & (T)1) ? (T)-1 : (T)1) : (T)0);
+  T r = (T)1;
+  while (b) { if (b & (T)1) r *= a; a *= a; b >>= 1; }
+  return r;
+}
+template <typename T> __device__ __forceinline__ T idiv(T a, T b) { return b == (T)0 ? (T)-1 : ((b == (T)-1) ? (T)(0 - a) : (T)(a / b)); }
+template <typename T> __device__ __forceinline__ T irem(T a, T b) { return b == (T)0 ? a : ((b == (T)-1) ? (T)0 : (T)(a % b)); }
+__device__ __forceinline__ float sgnf(float x) { return (x != x || x == 0.f) ? x : (x > 0.f ? 1.f : -1.f); }
+__device__ __forceinline__ double sgnd(double x) { return (x != x || x == 0.0) ? x : (x > 0.0 ? 1.0 : -1.0); }
+__device__ __forceinline__ int tokey(float f) { int i = __float_as_int(f); return i < 0 ? (i ^ 0x7FFFFFFF) : i; }
+__device__ __forceinline__ float redprec(float x, int eb, int mb) {
+  u32 u = __float_as_uint(x);
+  if (mb < 23 && x == x) { int sh = 23 - mb; u32 lsb = (u >> sh) & 1u; u = (u + ((1u << (sh - 1)) - 1u) + lsb) & ~((1u << sh) - 1u); }
+  float y = __uint_as_float(u);
+  if (eb < 8 && x == x) {
+    int maxe = (1 << (eb - 1)) - 1, mine = 1 - maxe;
+    int e = (int)((u >> 23) & 0xFF) - 127;
+    bool neg = (u >> 31) != 0;
+    if (e > maxe && e != 128) y = neg ? -__builtin_inff() : __builtin_inff();
+    if (e < mine) y = neg ? -0.f : 0.f;
+  }
+  return y;
+}
+)HIP";
+
+std::string storageT(DType d) {
+  switch (d) {
+    case DType::F32: return "float";
+    case DType::F64: return "double";
+    case DType::F16: return "_Float16";
+    case DType::BF16: return "u16";
+    case DType::S8: return "i8";
+    case DType::U8: return "u8";
+    case DType::Pred: return "u8";
+    case DType::S16: return "i16";
+    case DType::U16: return "u16";
+    case DType::S32: return "int";
+    case DType::U32: return "u32";
+    case DType::S64: return "i64";
+    case DType::U64: return "u64";
+    default: throw CompileError("codegen: unsupported element type");
+  }
+}
+std::string computeT(DType d) {
+  switch (d) {
+    case DType::F32: case DType::F16: case DType::BF16: return "float";
+    case DType::F64: return "double";
+    case DType::Pred: return "bool";
+    default: return storageT(d);
+  }
+}
+std::string loadExpr(DType d, const std::string& e) {
+  if (d == DType::BF16) return "bf2f(" + e + ")";
+  if (d == DType::F16) return "(float)(" + e + ")";
+  if (d == DType::Pred) return "((" + e + ") != 0)";
+  return e;
+}
+std::string storeExpr(DType d, const std::string& e) {
+  if (d == DType::BF16) return "f2bf(" + e + ")";
+  if (d == DType::F16) return "(_Float16)(" + e + ")";
+  if (d == DType::Pred) return "(u8)((" + e + ") ? 1 : 0)";
+  return e;
+}
+std::string roundTo(DType d, const std::string& e) {
+  if (d == DType::BF16) return "bfr(" + e + ")";
+  if (d == DType::F16) return "hfr(" + e + ")";
+  return e;
+}
+
+std::string literalFromBytes(DType d, const uint8_t* p) {
+  char buf[64];
+  switch (d) {
+    case DType::F32: { uint32_t u; memcpy(&u, p, 4); snprintf(buf, sizeof buf, "__uint_as_float(0x%08xu)", u); return buf; }
+    case DType::BF16: { uint16_t h; memcpy(&h, p, 2); snprintf(buf, sizeof buf, "__uint_as_float(0x%08xu)", ((uint32_t)h) << 16); return buf; }
+    case DType::F16: { _Float16 h; memcpy(&h, p, 2); float f = (float)h; uint32_t u; memcpy(&u, &f, 4); snprintf(buf, sizeof buf, "__uint_as_float(0x%08xu)", u); return buf; }
+    case DType::F64: { uint64_t u; memcpy(&u, p, 8); snprintf(buf, sizeof buf, "__longlong_as_double(0x%016llxll)", (unsigned long long)u); return buf; }
+    case DType::Pred: return *p ? "true" : "false";
+    case DType::S8: snprintf(buf, sizeof buf, "(i8)%d", (int)*(const int8_t*)p); return buf;
+    case DType::U8: snprintf(buf, sizeof buf, "(u8)%u", (unsigned)*p); return buf;
+    case DType::S16: { int16_t v; memcpy(&v, p, 2); snprintf(buf, sizeof buf, "(i16)%d", (int)v); return buf; }
+    case DType::U16: { uint16_t v; memcpy(&v, p, 2); snprintf(buf, sizeof buf, "(u16)%u", (unsigned)v); return buf; }
+    case DType::S32: { int32_t v; memcpy(&v, p, 4); if (v == INT32_MIN) return "(-2147483647 - 1)"; snprintf(buf, sizeof buf, "%d", v); return buf; }
+    case DType::U32: { uint32_t v; memcpy(&v, p, 4); snprintf(buf, sizeof buf, "%uu", v); return buf; }
+    case DType::S64: { int64_t v; memcpy(&v, p, 8); if (v == INT64_MIN) return "(-9223372036854775807ll - 1)"; snprintf(buf, sizeof buf, "%lldll", (long long)v); return buf; }
+    case DType::U64: { uint64_t v; memcpy(&v, p, 8); snprintf(buf, sizeof buf, "%lluull", (unsigned long long)v); return buf; }
+    default: throw CompileError("codegen: literal of unsupported type");
+  }
+}
+
+int64_t gcd64(int64_t a, int64_t b) {
+  a = a < 0 ? -a : a;
+  b = b < 0 ? -b : b;
+  while (b) { int64_t t = a % b; a = b; b = t; }
+  return a;
+}
+
+// One index component: value = base + coef * v, where v is the lane number inside the thread's vector.
+struct IdxDim {
+  std::string base = "0";
+  int64_t coef = 0;
+  bool inBody = false;   // base is a variable of the per-lane loop body
+  bool isConst = true;
+  int64_t cval = 0;
+  int64_t mult = 0;      // base is a known multiple of `mult` (0 = the constant zero, divisible by anything)
+  bool lane() const { return inBody || coef != 0; }
+};
+
+IdxDim constDim(int64_t c) {
+  IdxDim d;
+  d.base = std::to_string(c);
+  d.isConst = true;
+  d.cval = c;
+  d.mult = c;
+  return d;
+}
+
+struct Index {
+  bool linear = false;
+  IdxDim lin;
+  std::vector<int64_t> shape;   // shape the index addresses
+  std::vector<IdxDim> dims;     // valid when !linear
+  std::string sig;              // structural signature for memoisation
+  bool lane() const {
+    if (linear) return lin.lane();
+    for (auto& d : dims) if (d.lane()) return true;
+    return false;
+  }
+};
+
+class Emitter {
+ public:
+  Emitter(const LeafPredicate& isLeaf, int V, bool idx64) : isLeaf_(isLeaf), V_(V), idx64_(idx64) {
+    body_.emplace_back();
+    cache_.emplace_back();
+  }
+
+  int V_;
+  bool idx64_;
+  std::string pre_;
+  std::vector<std::string> body_;
+  std::vector<Value*> leaves_;
+
+  std::string idxT() const { return idx64_ ? "i64" : "int"; }
+  std::string fresh(const char* p) { return std::string(p) + std::to_string(tmp_++); }
+  void pre(const std::string& s) { pre_ += "  " + s + "\n"; }
+  void body(const std::string& s) { body_.back() += std::string(2 + 2 * body_.size(), ' ') + s + "\n"; }
+  void emit(bool inBody, const std::string& s) { (inBody || guard_ > 0) ? body(s) : pre(s); }
+
+  int leafId(Value* v) {
+    auto it = leafIndex_.find(v);
+    if (it != leafIndex_.end()) return it->second;
+    int id = (int)leaves_.size();
+    leaves_.push_back(v);
+    leafIndex_[v] = id;
+    return id;
+  }
+
+  std::string dimExpr(const IdxDim& d) const {
+    if (d.isConst) return d.base;
+    if (d.inBody || d.coef == 0) return d.base;
+    if (d.coef == 1) return "(" + d.base + " + v)";
+    return "(" + d.base + " + " + std::to_string(d.coef) + " * v)";
+  }
+
+  // new index variable holding `expr`
+  IdxDim var(const std::string& expr, bool inBody, int64_t coef = 0, int64_t mult = 1) {
+    IdxDim d;
+    d.isConst = false;
+    d.inBody = inBody || guard_ > 0;
+    d.base = fresh("ix");
+    d.coef = d.inBody ? 0 : coef;
+    d.mult = mult;
+    emit(d.inBody, "const " + idxT() + " " + d.base + " = " + expr + ";");
+    return d;
+  }
+
+  IdxDim toBody(const IdxDim& d) {
+    if (d.isConst || d.inBody) return d;
+    if (d.coef == 0 && guard_ == 0) return d;
+    IdxDim r;
+    r.isConst = false;
+    r.inBody = true;
+    r.base = fresh("ix");
+    body("const " + idxT() + " " + r.base + " = " + dimExpr(d) + ";");
+    return r;
+  }
+
+  // a*d + c
+  IdxDim affine(const IdxDim& d, int64_t a, int64_t c) {
+    if (d.isConst) return constDim(a * d.cval + c);
+    if (a == 1 && c == 0) return d;
+    if (d.inBody) return var("(" + d.base + " * " + std::to_string(a) + " + " + std::to_string(c) + ")", true);
+    std::string e = a == 1 ? d.base : "(" + d.base + " * " + std::to_string(a) + ")";
+    if (c != 0) e = "(" + e + " + " + std::to_string(c) + ")";
+    int64_t m = gcd64(d.mult * a, c);
+    return var(e, false, d.coef * a, m == 0 ? 1 : m);
+  }
+
+  IdxDim addDims(const IdxDim& a, const IdxDim& b) {
+    if (a.isConst) return affine(b, 1, a.cval);
+    if (b.isConst) return affine(a, 1, b.cval);
+    if (a.inBody || b.inBody) return var("(" + dimExpr(a) + " + " + dimExpr(b) + ")", true);
+    return var("(" + a.base + " + " + b.base + ")", false, a.coef + b.coef, std::max<int64_t>(1, gcd64(a.mult, b.mult)));
+  }
+
+  std::vector<IdxDim> delinearize(IdxDim lin, const std::vector<int64_t>& shape) {
+    int n = (int)shape.size();
+    std::vector<IdxDim> out(n);
+    if (n == 0) return out;
+    if (lin.isConst) {
+      int64_t r = lin.cval;
+      for (int d = n - 1; d >= 0; --d) {
+        int64_t D = std::max<int64_t>(shape[d], 1);
+        out[d] = constDim(d == 0 ? r : r % D);
+        r /= D;
+      }
+      return out;
+    }
+    int last = n - 1;
+    if (!lin.inBody && lin.coef != 0) {
+      int64_t D = shape[last];
+      bool ok = lin.coef == 1 && D % V_ == 0 && lin.mult % V_ == 0;
+      if (!ok) lin = toBody(lin);
+      else {
+        if (n == 1) { out[0] = lin; return out; }
+        out[last] = var("(" + lin.base + " % " + std::to_string(D) + ")", false, 1, V_);
+        IdxDim rest = var("(" + lin.base + " / " + std::to_string(D) + ")", false, 0, 1);
+        auto head = delinearize(rest, std::vector<int64_t>(shape.begin(), shape.begin() + last));
+        for (int d = 0; d < last; ++d) out[d] = head[d];
+        return out;
+      }
+    }
+    // lane-invariant or per-lane scalar: plain div/mod chain
+    bool inB = lin.inBody;
+    std::string rem = lin.base;
+    for (int d = n - 1; d >= 0; --d) {
+      int64_t D = shape[d];
+      if (D == 1) { out[d] = constDim(0); continue; }
+      bool anyLeft = false;
+      for (int q = 0; q < d; ++q) if (shape[q] != 1) anyLeft = true;
+      if (!anyLeft) { IdxDim r; r.isConst = false; r.inBody = inB; r.base = rem; r.mult = 1; out[d] = r; for (int q = 0; q < d; ++q) out[q] = constDim(0); break; }
+      out[d] = var("(" + rem + " % " + std::to_string(D) + ")", inB);
+      IdxDim q = var("(" + rem + " / " + std::to_string(D) + ")", inB);
+      rem = q.base;
+    }
+    return out;
+  }
+
+  IdxDim linearize(const std::vector<IdxDim>& dims, const std::vector<int64_t>& shape) {
+    int n = (int)shape.size();
+    std::vector<int64_t> stride(n, 1);
+    for (int d = n - 2; d >= 0; --d) stride[d] = stride[d + 1] * shape[d + 1];
+    bool anyBody = false, allConst = true;
+    int64_t cst = 0;
+    for (int d = 0; d < n; ++d) {
+      if (dims[d].isConst) cst += dims[d].cval * stride[d];
+      else { allConst = false; if (dims[d].inBody) anyBody = true; }
+    }
+    if (allConst) return constDim(cst);
+    std::string e;
+    int64_t coef = 0, mult = cst;
+    int terms = 0;
+    const IdxDim* single = nullptr;
+    for (int d = 0; d < n; ++d) {
+      if (dims[d].isConst) continue;
+      std::string t = anyBody ? dimExpr(dims[d]) : dims[d].base;
+      if (stride[d] != 1) t = t + " * " + std::to_string(stride[d]);
+      e += (e.empty() ? "" : " + ") + t;
+      coef += dims[d].coef * stride[d];
+      mult = gcd64(mult, dims[d].mult * stride[d]);
+      ++terms;
+      if (stride[d] == 1) single = &dims[d];
+    }
+    if (terms == 1 && cst == 0 && single) return *single;
+    if (cst != 0) e += " + " + std::to_string(cst);
+    if (anyBody) return var("(" + e + ")", true);
+    return var("(" + e + ")", false, coef, mult == 0 ? 1 : mult);
+  }
+
+  Index multi(const Index& idx) {
+    if (!idx.linear) return idx;
+    Index m;
+    m.linear = false;
+    m.shape = idx.shape;
+    m.dims = delinearize(idx.lin, idx.shape);
+    finishSig(m);
+    return m;
+  }
+
+  void finishSig(Index& idx) {
+    std::string s;
+    if (idx.linear) s = "L" + idx.lin.base + "#" + std::to_string(idx.lin.coef);
+    else for (auto& d : idx.dims) s += d.base + "#" + std::to_string(d.coef) + ",";
+    idx.sig = s;
+  }
+
+  Index linearIndex(const IdxDim& lin, const std::vector<int64_t>& shape) {
+    Index i;
+    i.linear = true;
+    i.lin = lin;
+    i.shape = shape;
+    finishSig(i);
+    return i;
+  }
+  Index multiIndex(std::vector<IdxDim> dims, const std::vector<int64_t>& shape) {
+    Index i;
+    i.linear = false;
+    i.dims = std::move(dims);
+    i.shape = shape;
+    finishSig(i);
+    return i;
+  }
+
+  // ----------------------------------------------------------------- loads
+  std::string load(Value* leaf, const Index& idx) {
+    int id = leafId(leaf);
+    DType dt = leaf->type.dt;
+    std::string ptr = "in" + std::to_string(id);
+    IdxDim off = idx.linear ? idx.lin : linearize(idx.dims, leaf->type.dims);
+    bool inB = off.inBody || guard_ > 0;
+    if (!inB && off.coef == 1 && V_ > 1 && !off.isConst && off.mult % V_ == 0 && leaf->type.numel() % V_ == 0) {
+      // one aligned vector load per thread, hoisted out of the lane loop
+      std::string key = ptr + "@" + off.base;
+      auto it = vecLoads_.find(key);
+      std::string name;
+      if (it == vecLoads_.end()) {
+        name = fresh("lv");
+        pre("const Vec<" + storageT(dt) + ", " + std::to_string(V_) + "> " + name + " = *(const Vec<" + storageT(dt) + ", " +
+            std::to_string(V_) + ">*)(" + ptr + " + " + off.base + ");");
+        vecLoads_[key] = name;
+      } else {
+        name = it->second;
+      }
+      return loadExpr(dt, name + ".e[v]");
+    }
+    std::string t = fresh("ld");
+    if (!inB && off.coef == 0) {
+      pre("const " + computeT(dt) + " " + t + " = " + loadExpr(dt, ptr + "[" + (off.isConst ? off.base : off.base) + "]") + ";");
+      return t;
+    }
+    body("const " + computeT(dt) + " " + t + " = " + loadExpr(dt, ptr + "[" + dimExpr(off) + "]") + ";");
+    return t;
+  }
+
+  // --------------------------------------------------------- value generation
+  std::string gen(Value* v, const Index& idx) {
+    std::string key = std::to_string(v->id) + "|" + idx.sig;
+    for (int s = (int)cache_.size() - 1; s >= 0; --s) {
+      auto it = cache_[s].find(key);
+      if (it != cache_[s].end()) return it->second;
+    }
+    std::string r = genUncached(v, idx);
+    // values emitted into the lane-invariant prologue are visible everywhere
+    bool laneInv = !idx.lane() && guard_ == 0;
+    (laneInv ? cache_.front() : cache_.back())[key] = r;
+    return r;
+  }
+
+ private:
+  const LeafPredicate& isLeaf_;
+  int tmp_ = 0;
+  int guard_ = 0;
+  std::unordered_map<Value*, int> leafIndex_;
+  std::unordered_map<std::string, std::string> vecLoads_;
+  std::vector<std::unordered_map<std::string, std::string>> cache_;
+
+  std::string def(const TensorType& t, const std::string& expr, bool inBody) {
+    std::string name = fresh("t");
+    emit(inBody, "const " + computeT(t.dt) + " " + name + " = " + roundTo(t.dt, expr) + ";");
+    return name;
+  }
+
+  // guarded evaluation: value = cond ? gen(inner) : other
+  template <typename F>
+  std::string guarded(const TensorType& t, const std::string& cond, F inner, const std::string& other) {
+    std::string name = fresh("t");
+    body(computeT(t.dt) + " " + name + " = " + other + ";");
+    body("if (" + cond + ") {");
+    body_.emplace_back();
+    cache_.emplace_back();
+    ++guard_;
+    std::string val = inner();
+    --guard_;
+    std::string inside = body_.back();
+    body_.pop_back();
+    cache_.pop_back();
+    body_.back() += inside;
+    body("  " + name + " = " + val + ";");
+    body("}");
+    return name;
+  }
+
+  std::string genUncached(Value* v, const Index& idx) {
+    if (isLeaf_(v)) return load(v, idx);
+    Op* op = v->def;
+    if (!op) throw CompileError("codegen: region argument " + v->name + " is not materialised");
+    const std::string& n = op->name;
+    const TensorType& rt = v->type;
+    bool inB = idx.lane();
+    auto in = [&](int k) { return gen(op->operands[k], idx); };
+    auto bin = [&](const std::string& e) { return def(rt, e, inB); };
+    DType odt = op->operands.empty() ? rt.dt : op->operands[0]->type.dt;
+    bool isF = isFloat(rt.dt), isD = rt.dt == DType::F64, isP = rt.dt == DType::Pred;
+    std::string sfx = isD ? "" : "f";
+
+    // ---- structural ops
+    if (n == "constant") {
+      auto& d = *op->attrs.at("value").dense;
+      if (d.splat || d.type.numel() == 1) return literalFromBytes(d.type.dt, d.bytes.data());
+      throw CompileError("codegen: dense constant must be materialised");
+    }
+    if (n == "iota") {
+      Index m = multi(idx);
+      return def(rt, "(" + computeT(rt.dt) + ")" + dimExpr(m.dims[op->integer("dim")]), inB);
+    }
+    if (n == "reshape") {
+      Value* x = op->operands[0];
+      if (idx.linear) return gen(x, linearIndex(idx.lin, x->type.dims));
+      // same dims up to unit dims: remap without div/mod
+      std::vector<IdxDim> od(x->type.rank());
+      size_t a = 0;
+      bool simple = true;
+      for (int d = 0; d < x->type.rank() && simple; ++d) {
+        if (x->type.dims[d] == 1) { od[d] = constDim(0); continue; }
+        while (a < rt.dims.size() && rt.dims[a] == 1) ++a;
+        if (a < rt.dims.size() && rt.dims[a] == x->type.dims[d]) od[d] = idx.dims[a++];
+        else simple = false;
+      }
+      if (simple) {
+        while (a < rt.dims.size() && rt.dims[a] == 1) ++a;
+        if (a == rt.dims.size()) return gen(x, multiIndex(od, x->type.dims));
+      }
+      IdxDim lin = linearize(idx.dims, rt.dims);
+      return gen(x, linearIndex(lin, x->type.dims));
+    }
+    if (n == "broadcast_in_dim") {
+      Value* x = op->operands[0];
+      auto& dims = op->ints("dims");
+      if (x->type.rank() == 0) return gen(x, multiIndex({}, {}));
+      Index m = multi(idx);
+      std::vector<IdxDim> od(x->type.rank());
+      for (int k = 0; k < x->type.rank(); ++k) od[k] = x->type.dims[k] == 1 ? constDim(0) : m.dims[dims[k]];
+      return gen(x, multiIndex(od, x->type.dims));
+    }
+    if (n == "transpose") {
+      Value* x = op->operands[0];
+      auto& perm = op->ints("dims");
+      Index m = multi(idx);
+      std::vector<IdxDim> od(x->type.rank());
+      for (int k = 0; k < x->type.rank(); ++k) od[perm[k]] = m.dims[k];
+      return gen(x, multiIndex(od, x->type.dims));
+    }
+    if (n == "reverse") {
+      Value* x = op->operands[0];
+      Index m = multi(idx);
+      for (auto d : op->ints("dims")) m.dims[d] = affine(m.dims[d], -1, x->type.dims[d] - 1);
+      finishSig(m);
+      return gen(x, m);
+    }
+    if (n == "slice") {
+      Value* x = op->operands[0];
+      Index m = multi(idx);
+      auto& st = op->ints("start");
+      auto& sr = op->ints("strides");
+      for (int d = 0; d < x->type.rank(); ++d) m.dims[d] = affine(m.dims[d], sr.empty() ? 1 : sr[d], st[d]);
+      m.shape = x->type.dims;
+      finishSig(m);
+      return gen(x, m);
+    }
+    if (n == "dynamic_slice") {
+      Value* x = op->operands[0];
+      Index m = multi(idx);
+      auto& sizes = op->ints("sizes");
+      for (int d = 0; d < x->type.rank(); ++d) {
+        int64_t hi = x->type.dims[d] - sizes[d];
+        if (hi == 0) continue;   // start is clamped to 0
+        std::string s = gen(op->operands[1 + d], multiIndex({}, {}));
+        IdxDim st = var("(" + idxT() + ")mn<i64>(mx<i64>((i64)" + s + ", 0), " + std::to_string(hi) + ")", false);
+        m.dims[d] = addDims(m.dims[d], st);
+      }
+      m.shape = x->type.dims;
+      finishSig(m);
+      return gen(x, m);
+    }
+    if (n == "pad") {
+      Value* x = op->operands[0];
+      auto& lo = op->ints("low");
+      auto& hi = op->ints("high");
+      auto& it = op->ints("interior");
+      bool trivial = true;
+      for (int d = 0; d < x->type.rank(); ++d) if (lo[d] != 0 || hi[d] != 0 || it[d] != 0) trivial = false;
+      if (trivial) return gen(x, idx);
+      Index m = multi(idx);
+      std::string pv = gen(op->operands[1], multiIndex({}, {}));
+      std::string cond;
+      std::vector<IdxDim> od(x->type.rank());
+      for (int d = 0; d < x->type.rank(); ++d) {
+        if (lo[d] == 0 && hi[d] == 0 && it[d] == 0) { od[d] = m.dims[d]; continue; }
+        IdxDim s = toBody(affine(m.dims[d], 1, -lo[d]));   // position in the dilated operand
+        std::string e = dimExpr(s);
+        std::string c = "(" + e + " >= 0)";
+        if (it[d] > 0) {
+          int64_t q = it[d] + 1;
+          c += " && (" + e + " % " + std::to_string(q) + " == 0) && (" + e + " / " + std::to_string(q) + " < " + std::to_string(x->type.dims[d]) + ")";
+          IdxDim r;
+          r.isConst = false; r.inBody = true; r.base = "(" + e + " / " + std::to_string(q) + ")";
+          od[d] = r;
+        } else {
+          c += " && (" + e + " < " + std::to_string(x->type.dims[d]) + ")";
+          od[d] = s;
+        }
+        cond += (cond.empty() ? "" : " && ") + c;
+      }
+      Index oi = multiIndex(od, x->type.dims);
+      return guarded(rt, cond, [&] { return gen(x, oi); }, pv);
+    }
+    if (n == "concatenate") {
+      int64_t dim = op->integer("dim");
+      Index m = multi(idx);
+      // lane-invariant along `dim` and not guarded: still emitted in the body for simplicity
+      IdxDim pos = toBody(m.dims[dim]);
+      std::string e = dimExpr(pos);
+      std::string name = fresh("t");
+      body(computeT(rt.dt) + " " + name + ";");
+      int64_t off = 0;
+      for (size_t k = 0; k < op->operands.size(); ++k) {
+        Value* x = op->operands[k];
+        int64_t sz = x->type.dims[dim];
+        if (sz == 0) continue;
+        bool lastPiece = true;
+        for (size_t q = k + 1; q < op->operands.size(); ++q) if (op->operands[q]->type.dims[dim] != 0) lastPiece = false;
+        body(std::string(off == 0 ? "if" : "else if") + " (" + (lastPiece ? "true" : e + " < " + std::to_string(off + sz)) + ") {");
+        body_.emplace_back();
+        cache_.emplace_back();
+        ++guard_;
+        Index oi = m;
+        IdxDim r;
+        r.isConst = false; r.inBody = true; r.base = "(" + e + " - " + std::to_string(off) + ")";
+        oi.dims[dim] = r;
+        oi.shape = x->type.dims;
+        finishSig(oi);
+        std::string val = gen(x, oi);
+        --guard_;
+        std::string inside = body_.back();
+        body_.pop_back();
+        cache_.pop_back();
+        body_.back() += inside;
+        body("  " + name + " = " + val + ";");
+        body("}");
+        off += sz;
+      }
+      return name;
+    }
+    if (n == "gather") return genGather(op, v, idx);
+    if (n == "optimization_barrier") return gen(op->operands[v->defIndex], idx);
+    if (n == "custom_call") return in(0);
+
+    // ---- conversions
+    if (n == "convert") {
+      std::string x = in(0);
+      std::string e;
+      if (isP) e = "(" + x + " != 0)";
+      else if (isFloat(odt) && !isF) e = "f2i<" + computeT(rt.dt) + ", " + computeT(odt) + ">(" + x + ")";
+      else e = "(" + computeT(rt.dt) + ")(" + x + ")";
+      return bin(e);
+    }
+    if (n == "bitcast_convert") {
+      std::string x = in(0);
+      size_t a = dtypeSize(odt), b = dtypeSize(rt.dt);
+      if (a != b) throw CompileError("bitcast_convert between element types of different width is not supported");
+      auto toBits = [&](DType d, const std::string& e) -> std::string {
+        if (d == DType::F32) return "__float_as_uint(" + e + ")";
+        if (d == DType::F64) return "(u64)__double_as_longlong(" + e + ")";
+        if (d == DType::BF16) return "f2bf(" + e + ")";
+        if (d == DType::F16) { return "__half_as_ushort(__float2half(" + e + "))"; }
+        return "(" + std::string(b == 1 ? "u8" : b == 2 ? "u16" : b == 4 ? "u32" : "u64") + ")(" + e + ")";
+      };
+      std::string bits = toBits(odt, x);
+      std::string e;
+      if (rt.dt == DType::F32) e = "__uint_as_float(" + bits + ")";
+      else if (rt.dt == DType::F64) e = "__longlong_as_double((i64)" + bits + ")";
+      else if (rt.dt == DType::BF16) e = "bf2f(" + bits + ")";
+      else if (rt.dt == DType::F16) e = "__half2float(__ushort_as_half(" + bits + "))";
+      else e = "(" + computeT(rt.dt) + ")(" + bits + ")";
+      return def(rt, e, inB);
+    }
+    if (n == "reduce_precision")
+      return bin("redprec(" + in(0) + ", " + std::to_string(op->integer("exponent_bits")) + ", " + std::to_string(op->integer("mantissa_bits")) + ")");
+
+    // ---- comparisons / selection
+    if (n == "compare") {
+      std::string a = in(0), b = in(1);
+      const std::string& dir = op->str("direction");
+      const char* c = dir == "EQ" ? "==" : dir == "NE" ? "!=" : dir == "LT" ? "<" : dir == "LE" ? "<=" : dir == "GT" ? ">" : ">=";
+      if (op->str("compare_type") == "TOTALORDER" && isFloat(odt) && odt != DType::F64) { a = "tokey(" + a + ")"; b = "tokey(" + b + ")"; }
+      return bin("(" + a + " " + c + " " + b + ")");
+    }
+    if (n == "select") {
+      Value* p = op->operands[0];
+      std::string ps = p->type.rank() == 0 && rt.rank() != 0 ? gen(p, multiIndex({}, {})) : gen(p, idx);
+      return bin("(" + ps + " ? " + in(1) + " : " + in(2) + ")");
+    }
+    if (n == "clamp") {
+      auto side = [&](int k) {
+        Value* s = op->operands[k];
+        return s->type.rank() == 0 && rt.rank() != 0 ? gen(s, multiIndex({}, {})) : gen(s, idx);
+      };
+      std::string T = computeT(rt.dt);
+      return bin("mn<" + T + ">(mx<" + T + ">(" + in(1) + ", " + side(0) + "), " + side(2) + ")");
+    }
+
+    // ---- binary arithmetic
+    std::string T = computeT(rt.dt);
+    if (n == "add") return bin(isP ? "(" + in(0) + " || " + in(1) + ")" : "(" + in(0) + " + " + in(1) + ")");
+    if (n == "subtract") return bin("(" + in(0) + " - " + in(1) + ")");
+    if (n == "multiply") return bin(isP ? "(" + in(0) + " && " + in(1) + ")" : "(" + in(0) + " * " + in(1) + ")");
+    if (n == "divide") return bin(isF ? "(" + in(0) + " / " + in(1) + ")" : "idiv<" + T + ">(" + in(0) + ", " + in(1) + ")");
+    if (n == "remainder") return bin(isF ? "fmod" + sfx + "(" + in(0) + ", " + in(1) + ")" : "irem<" + T + ">(" + in(0) + ", " + in(1) + ")");
+    if (n == "maximum") return bin(isP ? "(" + in(0) + " || " + in(1) + ")" : "mx<" + T + ">(" + in(0) + ", " + in(1) + ")");
+    if (n == "minimum") return bin(isP ? "(" + in(0) + " && " + in(1) + ")" : "mn<" + T + ">(" + in(0) + ", " + in(1) + ")");
+    if (n == "power") return bin(isF ? "pow" + sfx + "(" + in(0) + ", " + in(1) + ")" : "ipow<" + T + ">(" + in(0) + ", " + in(1) + ")");
+    if (n == "atan2") return bin("atan2" + sfx + "(" + in(0) + ", " + in(1) + ")");
+    if (n == "and") return bin(isP ? "(" + in(0) + " && " + in(1) + ")" : "(" + T + ")(" + in(0) + " & " + in(1) + ")");
+    if (n == "or") return bin(isP ? "(" + in(0) + " || " + in(1) + ")" : "(" + T + ")(" + in(0) + " | " + in(1) + ")");
+    if (n == "xor") return bin(isP ? "(" + in(0) + " != " + in(1) + ")" : "(" + T + ")(" + in(0) + " ^ " + in(1) + ")");
+    if (n == "shift_left" || n == "shift_right_logical" || n == "shift_right_arithmetic") {
+      int bits = (int)dtypeSize(rt.dt) * 8;
+      std::string U = bits == 8 ? "u8" : bits == 16 ? "u16" : bits == 32 ? "u32" : "u64";
+      std::string a = in(0), s = in(1);
+      std::string inr = "((u64)(" + s + ") < " + std::to_string(bits) + "ull)";
+      if (n == "shift_left") return bin("(" + inr + " ? (" + T + ")((" + U + ")" + a + " << (" + s + ")) : (" + T + ")0)");
+      if (n == "shift_right_logical") return bin("(" + inr + " ? (" + T + ")((" + U + ")" + a + " >> (" + s + ")) : (" + T + ")0)");
+      return bin("(" + T + ")(" + a + " >> (" + inr + " ? (int)(" + s + ") : " + std::to_string(bits - 1) + "))");
+    }
+
+    // ---- unary
+    if (n == "negate") return bin(isP ? in(0) : "(" + T + ")(-" + in(0) + ")");
+    if (n == "abs") return bin(isF ? "fabs" + sfx + "(" + in(0) + ")" : "(" + T + ")(" + in(0) + " < 0 ? -" + in(0) + " : " + in(0) + ")");
+    if (n == "not") return bin(isP ? "(!" + in(0) + ")" : "(" + T + ")(~" + in(0) + ")");
+    if (n == "sign") return bin(isF ? (isD ? "sgnd(" : "sgnf(") + in(0) + ")" : "(" + T + ")((" + in(0) + " > 0) - (" + in(0) + " < 0))");
+    if (n == "is_finite") return bin("isfinite(" + in(0) + ")");
+    if (n == "logistic") return bin(isD ? "(1.0 / (1.0 + exp(-" + in(0) + ")))" : "(1.f / (1.f + expf(-" + in(0) + ")))");
+    if (n == "rsqrt") return bin(isD ? "(1.0 / sqrt(" + in(0) + "))" : "(1.f / sqrtf(" + in(0) + "))");
+    if (n == "popcnt") return bin(dtypeSize(rt.dt) == 8 ? "(" + T + ")__popcll((u64)" + in(0) + ")" : "(" + T + ")__popc((u32)(" + std::string(dtypeSize(rt.dt) == 4 ? "u32" : dtypeSize(rt.dt) == 2 ? "u16" : "u8") + ")" + in(0) + ")");
+    if (n == "count_leading_zeros") {
+      int bits = (int)dtypeSize(rt.dt) * 8;
+      if (bits == 64) return bin("(" + T + ")__clzll((i64)" + in(0) + ")");
+      std::string U = bits == 8 ? "u8" : bits == 16 ? "u16" : "u32";
+      return bin("(" + T + ")(__clz((int)(u32)(" + U + ")" + in(0) + ") - " + std::to_string(32 - bits) + ")");
+    }
+    static const std::unordered_map<std::string, const char*> unary = {
+        {"exponential", "exp"}, {"exponential_minus_one", "expm1"}, {"log", "log"}, {"log_plus_one", "log1p"},
+        {"sqrt", "sqrt"}, {"cbrt", "cbrt"}, {"tanh", "tanh"}, {"tan", "tan"}, {"sine", "sin"}, {"cosine", "cos"},
+        {"floor", "floor"}, {"ceil", "ceil"}, {"round_nearest_even", "rint"}, {"round_nearest_afz", "round"}};
+    auto it = unary.find(n);
+    if (it != unary.end()) return bin(std::string(it->second) + sfx + "(" + in(0) + ")");
+    throw CompileError("codegen: no lowering for stablehlo." + n);
+  }
+
+  // stablehlo.gather as index arithmetic: every start index is clamped into
+  // [0, dim - slice] (reference: ops/gather_scatter.cc:233-239).
+  std::string genGather(Op* op, Value* v, const Index& idx) {
+    Value* operand = op->operands[0];
+    Value* indices = op->operands[1];
+    auto& offsetDims = op->ints("offset_dims");
+    auto& collapsed = op->ints("collapsed_slice_dims");
+    auto& obatch = op->ints("operand_batching_dims");
+    auto& ibatch = op->ints("start_indices_batching_dims");
+    auto& sim = op->ints("start_index_map");
+    int64_t ivd = op->integer("index_vector_dim");
+    auto& sizes = op->ints("slice_sizes");
+    auto has = [](const std::vector<int64_t>& a, int64_t x) { return std::find(a.begin(), a.end(), x) != a.end(); };
+    Index m = multi(idx);
+    int rank = v->type.rank();
+    std::vector<IdxDim> batchIdx, offIdx;
+    for (int d = 0; d < rank; ++d) (has(offsetDims, d) ? offIdx : batchIdx).push_back(m.dims[d]);
+    int irank = indices->type.rank();
+    auto indexAt = [&](int k) {
+      std::vector<IdxDim> id(irank);
+      size_t b = 0;
+      for (int d = 0; d < irank; ++d) {
+        if (d == ivd) id[d] = constDim(k);
+        else id[d] = batchIdx.at(b++);
+      }
+      return multiIndex(id, indices->type.dims);
+    };
+    int orank = operand->type.rank();
+    std::vector<IdxDim> od(orank, constDim(0));
+    for (size_t k = 0; k < sim.size(); ++k) {
+      int64_t d = sim[k];
+      int64_t hi = operand->type.dims[d] - sizes[d];
+      if (hi <= 0) continue;
+      Index ii = indexAt((int)k);
+      std::string s = gen(indices, ii);
+      IdxDim st = var("(" + idxT() + ")mn<i64>(mx<i64>((i64)" + s + ", 0), " + std::to_string(hi) + ")", ii.lane());
+      od[d] = st;
+    }
+    // batching dims take the coordinate of the matching batch dim of the indices
+    std::vector<int> idxBatchAxes;
+    for (int d = 0; d < irank; ++d) if (d != ivd) idxBatchAxes.push_back(d);
+    for (size_t k = 0; k < obatch.size(); ++k) {
+      int pos = (int)(std::find(idxBatchAxes.begin(), idxBatchAxes.end(), (int)ibatch[k]) - idxBatchAxes.begin());
+      od[obatch[k]] = addDims(od[obatch[k]], batchIdx.at(pos));
+    }
+    size_t o = 0;
+    for (int d = 0; d < orank; ++d) {
+      if (has(collapsed, d) || has(obatch, d)) continue;
+      od[d] = addDims(od[d], offIdx.at(o++));
+    }
+    return gen(operand, multiIndex(od, operand->type.dims));
+  }
+};
+
+int pickVector(const TensorType& t) {
+  int v = (int)std::max<size_t>(1, 16 / std::max<size_t>(1, dtypeSize(t.dt)));
+  v = std::min(v, 8);
+  int64_t last = t.rank() ? t.dims.back() : 1;
+  // the innermost dim of size 1 carries no information: use the product of trailing dims instead
+  int64_t n = t.numel();
+  int64_t trail = last;
+  for (int d = t.rank() - 2; d >= 0 && trail == 1; --d) trail = t.dims[d];
+  (void)n;
+  while (v > 1 && trail % v != 0) v >>= 1;
+  return v;
+}
+
+bool needs64(const std::vector<Value*>& vals) {
+  for (auto* v : vals) if (v->type.numel() >= (int64_t(1) << 31) - 16) return true;
+  return false;
+}
+
+std::string kernelHeader(const std::vector<Value*>& leaves, const std::vector<std::string>& outs) {
+  std::string s = "extern \"C\" __global__ void __launch_bounds__(256) k(";
+  bool first = true;
+  for (size_t i = 0; i < leaves.size(); ++i) {
+    s += std::string(first ? "" : ", ") + "const " + storageT(leaves[i]->type.dt) + "* __restrict__ in" + std::to_string(i);
+    first = false;
+  }
+  for (auto& o : outs) {
+    s += std::string(first ? "" : ", ") + o;
+    first = false;
+  }
+  return s + ")";
+}
+
+void collectAllValues(Value* root, const LeafPredicate& isLeaf, std::vector<Value*>& out, std::unordered_map<Value*, bool>& seen) {
+  if (seen[root]) return;
+  seen[root] = true;
+  out.push_back(root);
+  if (isLeaf(root) || !root->def) return;
+  for (auto* o : root->def->operands) collectAllValues(o, isLeaf, out, seen);
+}
+
+}  // namespace
+
+bool isFusibleOp(const Op& op) {
+  static const char* names[] = {
+      "add", "subtract", "multiply", "divide", "maximum", "minimum", "power", "remainder", "atan2", "and", "or", "xor",
+      "not", "negate", "abs", "exponential", "exponential_minus_one", "log", "log_plus_one", "sqrt", "rsqrt", "cbrt",
+      "tanh", "tan", "sine", "cosine", "logistic", "floor", "ceil", "sign", "round_nearest_even", "round_nearest_afz",
+      "is_finite", "shift_left", "shift_right_logical", "shift_right_arithmetic", "popcnt", "count_leading_zeros",
+      "compare", "select", "clamp", "convert", "bitcast_convert", "reduce_precision", "constant", "iota", "reshape",
+      "broadcast_in_dim", "transpose", "reverse", "concatenate", "slice", "dynamic_slice", "pad", "gather",
+      "optimization_barrier", "custom_call"};
+  for (auto* n : names) if (op.name == n) return true;
+  return false;
+}
+
+static const char* reduceKind(const Op& reduce) {
+  if (reduce.regions.size() != 1) return nullptr;
+  auto& r = *reduce.regions[0];
+  if (r.args.size() != 2 || r.ops.size() != 2) return nullptr;
+  Op* b = r.ops[0].get();
+  Op* ret = r.ops[1].get();
+  if (ret->name != "return" || ret->operands.size() != 1 || ret->operands[0] != b->result()) return nullptr;
+  if (b->operands.size() != 2) return nullptr;
+  bool uses = (b->operands[0] == r.args[0].get() && b->operands[1] == r.args[1].get()) ||
+              (b->operands[0] == r.args[1].get() && b->operands[1] == r.args[0].get());
+  if (!uses) return nullptr;
+  for (const char* k : {"add", "multiply", "maximum", "minimum", "and", "or"})
+    if (b->name == k) return k;
+  return nullptr;
+}
+
+bool isSimpleReduce(const Op& reduce) { return reduce.operands.size() == 2 && reduceKind(reduce) != nullptr; }
+
+// ------------------------------------------------------------------ loop kernels
+FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf) {
+  std::vector<Value*> all;
+  std::unordered_map<Value*, bool> seen;
+  LeafPredicate inner = [&](Value* v) { return v != root && isLeaf(v); };
+  collectAllValues(root, inner, all, seen);
+  int V = pickVector(root->type);
+  bool i64 = needs64(all);
+  Emitter em(inner, V, i64);
+  int64_t N = root->type.numel();
+  IdxDim lin;
+  lin.isConst = false;
+  lin.base = "base";
+  lin.coef = 1;
+  lin.mult = V;
+  if (V == 1) { lin.coef = 0; }
+  Index idx = em.linearIndex(lin, root->type.dims);
+  std::string val = em.gen(root, idx);
+  DType dt = root->type.dt;
+  std::ostringstream s;
+  s << kPrelude;
+  s << kernelHeader(em.leaves_, {storageT(dt) + "* __restrict__ out0"}) << " {\n";
+  s << "  const " << em.idxT() << " base = ((" << em.idxT() << ")blockIdx.x * 256 + threadIdx.x) * " << V << ";\n";
+  s << "  if (base >= " << N << (i64 ? "ll" : "") << ") return;\n";
+  s << em.pre_;
+  if (V > 1) {
+    s << "  Vec<" << storageT(dt) << ", " << V << "> ov;\n";
+    s << "  #pragma unroll\n  for (int v = 0; v < " << V << "; ++v) {\n";
+    s << em.body_.front();
+    s << "    ov.e[v] = " << storeExpr(dt, val) << ";\n  }\n";
+    s << "  *(Vec<" << storageT(dt) << ", " << V << ">*)(out0 + base) = ov;\n";
+  } else {
+    s << "  {\n    const int v = 0; (void)v;\n" << em.body_.front();
+    s << "    out0[base] = " << storeExpr(dt, val) << ";\n  }\n";
+  }
+  s << "}\n";
+  FusedCode fc;
+  Launch l;
+  l.source = s.str();
+  int64_t threads = (N + V - 1) / V;
+  l.grid[0] = (unsigned)std::max<int64_t>(1, (threads + 255) / 256);
+  l.block[0] = 256;
+  for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
+  KArg o;
+  o.kind = KArg::Out;
+  o.value = root;
+  l.args.push_back(o);
+  fc.launches.push_back(std::move(l));
+  fc.leaves = em.leaves_;
+  return fc;
+}
+
+// -------------------------------------------------- dynamic_update_slice window
+FusedCode generateDusKernel(Op* dus, const LeafPredicate& isLeaf) {
+  Value* operand = dus->operands[0];
+  Value* update = dus->operands[1];
+  Value* result = dus->result();
+  std::vector<Value*> all;
+  std::unordered_map<Value*, bool> seen;
+  collectAllValues(update, isLeaf, all, seen);
+  for (size_t k = 2; k < dus->operands.size(); ++k) collectAllValues(dus->operands[k], isLeaf, all, seen);
+  all.push_back(operand);
+  int V = pickVector(update->type);
+  // the window start along the innermost dim is data dependent, so stores are per lane
+  bool i64 = needs64(all);
+  Emitter em(isLeaf, V, i64);
+  int64_t N = update->type.numel();
+  IdxDim lin;
+  lin.isConst = false;
+  lin.base = "base";
+  lin.coef = V > 1 ? 1 : 0;
+  lin.mult = V;
+  Index idx = em.linearIndex(lin, update->type.dims);
+  std::string val = em.gen(update, idx);
+  Index m = em.multi(idx);
+  std::vector<IdxDim> od(operand->type.rank());
+  for (int d = 0; d < operand->type.rank(); ++d) {
+    int64_t hi = operand->type.dims[d] - update->type.dims[d];
+    if (hi <= 0) { od[d] = m.dims[d]; continue; }
+    std::string sidx = em.gen(dus->operands[2 + d], em.multiIndex({}, {}));
+    IdxDim st = em.var("(" + em.idxT() + ")mn<i64>(mx<i64>((i64)" + sidx + ", 0), " + std::to_string(hi) + ")", false);
+    od[d] = em.addDims(m.dims[d], st);
+  }
+  IdxDim off = em.linearize(od, operand->type.dims);
+  DType dt = result->type.dt;
+  std::ostringstream s;
+  s << kPrelude;
+  s << kernelHeader(em.leaves_, {storageT(dt) + "* out0"}) << " {\n";
+  s << "  const " << em.idxT() << " base = ((" << em.idxT() << ")blockIdx.x * 256 + threadIdx.x) * " << V << ";\n";
+  s << "  if (base >= " << N << (i64 ? "ll" : "") << ") return;\n";
+  s << em.pre_;
+  s << "  #pragma unroll\n  for (int v = 0; v < " << V << "; ++v) {\n";
+  s << em.body_.front();
+  s << "    out0[" << em.dimExpr(off) << "] = " << storeExpr(dt, val) << ";\n  }\n}\n";
+  FusedCode fc;
+  Launch l;
+  l.source = s.str();
+  int64_t threads = (N + V - 1) / V;
+  l.grid[0] = (unsigned)std::max<int64_t>(1, (threads + 255) / 256);
+  l.block[0] = 256;
+  for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
+  KArg o;
+  o.kind = KArg::Out;
+  o.value = result;
+  l.args.push_back(o);
+  fc.launches.push_back(std::move(l));
+  fc.leaves = em.leaves_;
+  return fc;
+}
+
+// --------------------------------------------------------------- reductions
+namespace {
+
+struct RedOp {
+  const char* kind;
+  DType dt;       // element type of the reduce result
+  std::string accT;
+  std::string identity;
+  std::string combine(const std::string& a, const std::string& b) const {
+    std::string k = kind;
+    if (k == "add") return dt == DType::Pred ? "(" + a + " || " + b + ")" : "(" + a + " + " + b + ")";
+    if (k == "multiply") return dt == DType::Pred ? "(" + a + " && " + b + ")" : "(" + a + " * " + b + ")";
+    if (k == "maximum") return dt == DType::Pred ? "(" + a + " || " + b + ")" : "mx<" + accT + ">(" + a + ", " + b + ")";
+    if (k == "minimum") return dt == DType::Pred ? "(" + a + " && " + b + ")" : "mn<" + accT + ">(" + a + ", " + b + ")";
+    if (k == "and") return dt == DType::Pred ? "(" + a + " && " + b + ")" : "(" + accT + ")(" + a + " & " + b + ")";
+    return dt == DType::Pred ? "(" + a + " || " + b + ")" : "(" + accT + ")(" + a + " | " + b + ")";
+  }
+};
+
+RedOp makeRedOp(const Op& reduce) {
+  RedOp r;
+  r.kind = reduceKind(reduce);
+  r.dt = reduce.result()->type.dt;
+  r.accT = computeT(r.dt);
+  std::string k = r.kind;
+  bool f = isFloat(r.dt);
+  if (k == "add" || k == "or") r.identity = r.dt == DType::Pred ? "false" : "(" + r.accT + ")0";
+  else if (k == "multiply") r.identity = r.dt == DType::Pred ? "true" : "(" + r.accT + ")1";
+  else if (k == "and") r.identity = r.dt == DType::Pred ? "true" : "(" + r.accT + ")~(" + r.accT + ")0";
+  else if (k == "maximum") {
+    if (f) r.identity = r.dt == DType::F64 ? "(-__builtin_inf())" : "(-__builtin_inff())";
+    else if (r.dt == DType::Pred) r.identity = "false";
+    else if (isUnsigned(r.dt)) r.identity = "(" + r.accT + ")0";
+    else r.identity = "(" + r.accT + ")(1ull << " + std::to_string(dtypeSize(r.dt) * 8 - 1) + ")";
+  } else {
+    if (f) r.identity = r.dt == DType::F64 ? "__builtin_inf()" : "__builtin_inff()";
+    else if (r.dt == DType::Pred) r.identity = "true";
+    else if (isUnsigned(r.dt)) r.identity = "(" + r.accT + ")~(" + r.accT + ")0";
+    else r.identity = "(" + r.accT + ")((1ull << " + std::to_string(dtypeSize(r.dt) * 8 - 1) + ") - 1ull)";
+  }
+  return r;
+}
+
+// shuffle of an accumulator across the wavefront (64 lanes), by type width
+std::string shflXor(const std::string& accT, const std::string& x, const std::string& lanes) {
+  if (accT == "bool") return "(__shfl_xor((int)" + x + ", " + lanes + ", 64) != 0)";
+  if (accT == "i8" || accT == "u8" || accT == "i16" || accT == "u16") return "(" + accT + ")__shfl_xor((int)" + x + ", " + lanes + ", 64)";
+  return "__shfl_xor(" + x + ", " + lanes + ", 64)";
+}
+
+}  // namespace
+
+FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeaf) {
+  Op* r0 = reduces[0];
+  Value* x0 = r0->operands[0];
+  const std::vector<int64_t>& shape = x0->type.dims;
+  int rank = (int)shape.size();
+  std::vector<int64_t> rdims = r0->ints("dimensions");
+  std::sort(rdims.begin(), rdims.end());
+  std::vector<bool> isRed(rank, false);
+  for (auto d : rdims) isRed[d] = true;
+  std::vector<int64_t> keptShape, redShape;
+  std::vector<int> keptDims, redDims;
+  for (int d = 0; d < rank; ++d) {
+    if (isRed[d]) { redShape.push_back(shape[d]); redDims.push_back(d); }
+    else { keptShape.push_back(shape[d]); keptDims.push_back(d); }
+  }
+  int64_t Kn = 1, Rn = 1;
+  for (auto d : keptShape) Kn *= d;
+  for (auto d : redShape) Rn *= d;
+  size_t nr = reduces.size();
+  std::vector<RedOp> ops;
+  for (auto* r : reduces) ops.push_back(makeRedOp(*r));
+
+  std::vector<Value*> all;
+  std::unordered_map<Value*, bool> seen;
+  for (auto* r : reduces) {
+    collectAllValues(r->operands[0], isLeaf, all, seen);
+    collectAllValues(r->operands[1], isLeaf, all, seen);
+  }
+  bool i64 = needs64(all);
+  std::string IT = i64 ? "i64" : "int";
+
+  // innermost non-unit dim decides the strategy
+  int inner = rank - 1;
+  while (inner > 0 && shape[inner] == 1) --inner;
+  bool rowStyle = rank == 0 || isRed[inner] || Kn == 1;
+  FusedCode fc;
+
+  // ---- common: the final pass that folds partials and the init value
+  auto finalPass = [&](int64_t P, int64_t workStride, std::vector<int64_t> workOff, std::vector<Value*>& initLeaves) -> Launch {
+    // out[k] = combine(init, partial[0..P)[k])
+    Emitter em(isLeaf, 1, i64);
+    std::vector<std::string> inits;
+    for (auto* r : reduces) inits.push_back(em.gen(r->operands[1], em.multiIndex({}, {})));
+    std::ostringstream s;
+    s << kPrelude;
+    std::vector<std::string> outs;
+    for (size_t j = 0; j < nr; ++j) outs.push_back("const " + ops[j].accT + "* __restrict__ part" + std::to_string(j));
+    for (size_t j = 0; j < nr; ++j) outs.push_back(storageT(ops[j].dt) + "* __restrict__ out" + std::to_string(j));
+    s << kernelHeader(em.leaves_, outs) << " {\n";
+    s << "  const " << IT << " kk = (" << IT << ")blockIdx.x * 256 + threadIdx.x;\n  if (kk >= " << Kn << ") return;\n";
+    s << em.pre_;
+    for (size_t j = 0; j < nr; ++j) {
+      s << "  { " << ops[j].accT << " a = " << ops[j].identity << ";\n";
+      s << "    for (" << IT << " p = 0; p < " << P << "; ++p) a = " << ops[j].combine("a", "part" + std::to_string(j) + "[p * " + std::to_string(Kn) + " + kk]") << ";\n";
+      s << "    a = " << ops[j].combine(inits[j], "a") << ";\n";
+      s << "    out" << j << "[kk] = " << storeExpr(ops[j].dt, roundTo(ops[j].dt, "a")) << "; }\n";
+    }
+    s << "}\n";
+    Launch l;
+    l.source = s.str();
+    l.grid[0] = (unsigned)((Kn + 255) / 256);
+    l.block[0] = 256;
+    for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
+    for (size_t j = 0; j < nr; ++j) { KArg a; a.kind = KArg::Work; a.workOffset = workOff[j]; l.args.push_back(a); }
+    for (size_t j = 0; j < nr; ++j) { KArg a; a.kind = KArg::Out; a.value = reduces[j]->result(); l.args.push_back(a); }
+    initLeaves = em.leaves_;
+    (void)workStride;
+    return l;
+  };
+
+  if (rowStyle) {
+    // lanes run along the reduced elements (r, row-major over the reduced dims).  One
+    // wavefront per output when rows are short, one workgroup per output when they
+    // are long, and several workgroups per output (partials) when outputs are few.
+    int V = 1;
+    {
+      int64_t lastRed = redShape.empty() ? 1 : redShape.back();
+      int v = (int)std::min<size_t>(8, std::max<size_t>(1, 16 / std::max<size_t>(1, dtypeSize(x0->type.dt))));
+      bool innerIsLastRed = !redDims.empty() && redDims.back() == inner;
+      while (v > 1 && (!innerIsLastRed || lastRed % v != 0)) v >>= 1;
+      if (Rn < 64 * v) v = 1;
+      V = v;
+    }
+    int64_t vecs = (Rn + V - 1) / V;
+    bool wavePerRow = vecs <= 256 && Kn >= 4;
+    int64_t P = 1;                 // workgroups per output row
+    if (!wavePerRow && Kn < 512 && vecs > 256 * 16) {
+      P = std::min<int64_t>((vecs + 256 * 8 - 1) / (256 * 8), std::max<int64_t>(1, 2048 / Kn));
+    }
+    Emitter em(isLeaf, V, i64);
+    // kept index: lane-invariant
+    IdxDim klin;
+    klin.isConst = false; klin.base = "kk"; klin.coef = 0; klin.mult = 1;
+    auto kd = em.delinearize(klin, keptShape);
+    IdxDim rlin;
+    rlin.isConst = false; rlin.base = "rb"; rlin.coef = V > 1 ? 1 : 0; rlin.mult = V;
+    // everything that depends on rb belongs to the loop body: emit index math there
+    std::string savedPre = em.pre_;
+    em.pre_.clear();
+    auto rd = em.delinearize(rlin, redShape);
+    std::vector<IdxDim> full(rank);
+    for (size_t q = 0; q < keptDims.size(); ++q) full[keptDims[q]] = kd[q];
+    for (size_t q = 0; q < redDims.size(); ++q) full[redDims[q]] = rd[q];
+    Index idx = em.multiIndex(full, shape);
+    std::vector<std::string> vals;
+    for (auto* r : reduces) vals.push_back(em.gen(r->operands[0], idx));
+    std::string loopPre = em.pre_;   // statements that depend on rb (per iteration, lane-invariant)
+    em.pre_ = savedPre;
+    std::vector<std::string> inits;
+    for (auto* r : reduces) inits.push_back(em.gen(r->operands[1], em.multiIndex({}, {})));
+
+    std::ostringstream s;
+    s << kPrelude;
+    std::vector<std::string> outs;
+    bool partial = P > 1;
+    for (size_t j = 0; j < nr; ++j)
+      outs.push_back((partial ? ops[j].accT : storageT(ops[j].dt)) + "* __restrict__ out" + std::to_string(j));
+    s << kernelHeader(em.leaves_, outs) << " {\n";
+    if (wavePerRow) {
+      s << "  const int lane = threadIdx.x & 63;\n";
+      s << "  const " << IT << " kk = (" << IT << ")blockIdx.x * 4 + (threadIdx.x >> 6);\n";
+      s << "  if (kk >= " << Kn << ") return;\n";
+      s << "  const " << IT << " r_begin = 0, r_end = " << vecs << ";\n  const int r_step = 64, r_tid = lane;\n";
+    } else {
+      s << "  const " << IT << " kk = (" << IT << ")blockIdx.x / " << P << ";\n";
+      s << "  const " << IT << " chunk = (" << vecs << " + " << P << " - 1) / " << P << ";\n";
+      s << "  const " << IT << " r_begin = ((" << IT << ")blockIdx.x % " << P << ") * chunk;\n";
+      s << "  const " << IT << " r_end = r_begin + chunk < " << vecs << " ? r_begin + chunk : " << vecs << ";\n";
+      s << "  const int r_step = 256, r_tid = threadIdx.x;\n";
+    }
+    s << em.pre_;
+    for (size_t j = 0; j < nr; ++j) s << "  " << ops[j].accT << " acc" << j << " = " << ops[j].identity << ";\n";
+    s << "  for (" << IT << " rv = r_begin + r_tid; rv < r_end; rv += r_step) {\n";
+    s << "    const " << IT << " rb = rv * " << V << ";\n";
+    s << loopPre;
+    s << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n";
+    s << em.body_.front();
+    for (size_t j = 0; j < nr; ++j) s << "      acc" << j << " = " << ops[j].combine("acc" + std::to_string(j), vals[j]) << ";\n";
+    s << "    }\n  }\n";
+    // wavefront reduction
+    for (size_t j = 0; j < nr; ++j) {
+      s << "  #pragma unroll\n  for (int o = 32; o > 0; o >>= 1) acc" << j << " = "
+        << ops[j].combine("acc" + std::to_string(j), shflXor(ops[j].accT, "acc" + std::to_string(j), "o")) << ";\n";
+    }
+    if (!wavePerRow) {
+      for (size_t j = 0; j < nr; ++j) s << "  __shared__ " << (ops[j].accT == "bool" ? "int" : ops[j].accT) << " sm" << j << "[4];\n";
+      s << "  if ((threadIdx.x & 63) == 0) {";
+      for (size_t j = 0; j < nr; ++j) s << " sm" << j << "[threadIdx.x >> 6] = acc" << j << ";";
+      s << " }\n  __syncthreads();\n  if (threadIdx.x != 0) return;\n";
+      for (size_t j = 0; j < nr; ++j) {
+        s << "  acc" << j << " = (" << ops[j].accT << ")sm" << j << "[0];\n";
+        s << "  for (int w = 1; w < 4; ++w) acc" << j << " = " << ops[j].combine("acc" + std::to_string(j), "(" + ops[j].accT + ")sm" + std::to_string(j) + "[w]") << ";\n";
+      }
+    } else {
+      s << "  if (lane != 0) return;\n";
+    }
+    for (size_t j = 0; j < nr; ++j) {
+      if (partial) s << "  out" << j << "[((" << IT << ")blockIdx.x % " << P << ") * " << Kn << " + kk] = acc" << j << ";\n";
+      else s << "  out" << j << "[kk] = " << storeExpr(ops[j].dt, roundTo(ops[j].dt, ops[j].combine(inits[j], "acc" + std::to_string(j)))) << ";\n";
+    }
+    s << "}\n";
+    Launch l;
+    l.source = s.str();
+    l.grid[0] = (unsigned)(wavePerRow ? (Kn + 3) / 4 : Kn * P);
+    l.block[0] = 256;
+    for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
+    std::vector<int64_t> workOff;
+    int64_t wb = 0;
+    for (size_t j = 0; j < nr; ++j) {
+      KArg a;
+      if (partial) {
+        a.kind = KArg::Work;
+        a.workOffset = wb;
+        workOff.push_back(wb);
+        wb += ((int64_t)P * Kn * 8 + 255) / 256 * 256;
+      } else {
+        a.kind = KArg::Out;
+        a.value = reduces[j]->result();
+      }
+      l.args.push_back(a);
+    }
+    fc.leaves = em.leaves_;
+    fc.launches.push_back(std::move(l));
+    if (partial) {
+      std::vector<Value*> il;
+      fc.launches.push_back(finalPass(P, Kn, workOff, il));
+      for (auto* v : il) if (std::find(fc.leaves.begin(), fc.leaves.end(), v) == fc.leaves.end()) fc.leaves.push_back(v);
+      fc.workspaceBytes = wb;
+    }
+    return fc;
+  }
+
+  // ---- column style: lanes along the kept (contiguous) axis, rows split over
+  // threadIdx.y and, when there are many rows, over blockIdx.y (partials).
+  int V = 1;
+  {
+    int v = (int)std::min<size_t>(8, std::max<size_t>(1, 16 / std::max<size_t>(1, dtypeSize(x0->type.dt))));
+    int64_t lastKept = keptShape.back();
+    bool innerIsLastKept = keptDims.back() == inner;
+    while (v > 1 && (!innerIsLastKept || lastKept % v != 0)) v >>= 1;
+    V = v;
+  }
+  int64_t kvecs = (Kn + V - 1) / V;
+  int TX = 1;
+  while (TX < 64 && TX < kvecs) TX <<= 1;
+  int TY = 256 / TX;
+  int64_t gridX = (kvecs + TX - 1) / TX;
+  int64_t P = 1;
+  if (Rn > (int64_t)TY * 16) P = std::min<int64_t>((Rn + TY * 8 - 1) / (TY * 8), std::max<int64_t>(1, 2048 / gridX));
+  bool partial = P > 1;
+  Emitter em(isLeaf, V, i64);
+  IdxDim klin;
+  klin.isConst = false; klin.base = "kb"; klin.coef = V > 1 ? 1 : 0; klin.mult = V;
+  auto kd = em.delinearize(klin, keptShape);
+  std::string savedPre = em.pre_;
+  em.pre_.clear();
+  IdxDim rlin;
+  rlin.isConst = false; rlin.base = "rr"; rlin.coef = 0; rlin.mult = 1;
+  auto rd = em.delinearize(rlin, redShape);
+  std::vector<IdxDim> full(rank);
+  for (size_t q = 0; q < keptDims.size(); ++q) full[keptDims[q]] = kd[q];
+  for (size_t q = 0; q < redDims.size(); ++q) full[redDims[q]] = rd[q];
+  Index idx = em.multiIndex(full, shape);
+  std::vector<std::string> vals;
+  for (auto* r : reduces) vals.push_back(em.gen(r->operands[0], idx));
+  std::string loopPre = em.pre_;
+  em.pre_ = savedPre;
+  std::vector<std::string> inits;
+  for (auto* r : reduces) inits.push_back(em.gen(r->operands[1], em.multiIndex({}, {})));
+
+  std::ostringstream s;
+  s << kPrelude;
+  std::vector<std::string> outs;
+  for (size_t j = 0; j < nr; ++j)
+    outs.push_back((partial ? ops[j].accT : storageT(ops[j].dt)) + "* __restrict__ out" + std::to_string(j));
+  s << kernelHeader(em.leaves_, outs) << " {\n";
+  s << "  const int tx = threadIdx.x % " << TX << ", ty = threadIdx.x / " << TX << ";\n";
+  s << "  const " << IT << " kb = ((" << IT << ")blockIdx.x * " << TX << " + tx) * " << V << ";\n";
+  s << "  const bool active = kb < " << Kn << ";\n";
+  s << "  const " << IT << " chunk = (" << Rn << " + " << P << " - 1) / " << P << ";\n";
+  s << "  const " << IT << " r_begin = (" << IT << ")blockIdx.y * chunk;\n";
+  s << "  const " << IT << " r_end = r_begin + chunk < " << Rn << " ? r_begin + chunk : " << Rn << ";\n";
+  for (size_t j = 0; j < nr; ++j) {
+    s << "  " << ops[j].accT << " acc" << j << "[" << V << "];\n";
+    s << "  #pragma unroll\n  for (int v = 0; v < " << V << "; ++v) acc" << j << "[v] = " << ops[j].identity << ";\n";
+  }
+  s << "  if (active) {\n";
+  s << em.pre_;
+  s << "  for (" << IT << " rr = r_begin + ty; rr < r_end; rr += " << TY << ") {\n";
+  s << loopPre;
+  s << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n";
+  s << em.body_.front();
+  for (size_t j = 0; j < nr; ++j) s << "      acc" << j << "[v] = " << ops[j].combine("acc" + std::to_string(j) + "[v]", vals[j]) << ";\n";
+  s << "    }\n  }\n  }\n";
+  if (TY > 1) {
+    for (size_t j = 0; j < nr; ++j) {
+      std::string ST = ops[j].accT == "bool" ? "int" : ops[j].accT;
+      s << "  __shared__ " << ST << " sm" << j << "[" << TY << "][" << TX * V << " + 1];\n";
+      s << "  #pragma unroll\n  for (int v = 0; v < " << V << "; ++v) sm" << j << "[ty][tx * " << V << " + v] = acc" << j << "[v];\n";
+    }
+    s << "  __syncthreads();\n  if (ty != 0 || !active) return;\n";
+    for (size_t j = 0; j < nr; ++j) {
+      s << "  for (int y = 1; y < " << TY << "; ++y) {\n    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) acc" << j << "[v] = "
+        << ops[j].combine("acc" + std::to_string(j) + "[v]", "(" + ops[j].accT + ")sm" + std::to_string(j) + "[y][tx * " + std::to_string(V) + " + v]") << ";\n  }\n";
+    }
+  } else {
+    s << "  if (!active) return;\n";
+  }
+  for (size_t j = 0; j < nr; ++j) {
+    s << "  #pragma unroll\n  for (int v = 0; v < " << V << "; ++v) ";
+    if (partial) s << "out" << j << "[(" << IT << ")blockIdx.y * " << Kn << " + kb + v] = acc" << j << "[v];\n";
+    else s << "out" << j << "[kb + v] = " << storeExpr(ops[j].dt, roundTo(ops[j].dt, ops[j].combine(inits[j], "acc" + std::to_string(j) + "[v]"))) << ";\n";
+  }
+  s << "}\n";
+  Launch l;
+  l.source = s.str();
+  l.grid[0] = (unsigned)gridX;
+  l.grid[1] = (unsigned)P;
+  l.block[0] = 256;
+  for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
+  std::vector<int64_t> workOff;
+  int64_t wb = 0;
+  for (size_t j = 0; j < nr; ++j) {
+    KArg a;
+    if (partial) {
+      a.kind = KArg::Work;
+      a.workOffset = wb;
+      workOff.push_back(wb);
+      wb += ((int64_t)P * Kn * 8 + 255) / 256 * 256;
+    } else {
+      a.kind = KArg::Out;
+      a.value = reduces[j]->result();
+    }
+    l.args.push_back(a);
+  }
+  fc.leaves = em.leaves_;
+  fc.launches.push_back(std::move(l));
+  if (partial) {
+    std::vector<Value*> il;
+    fc.launches.push_back(finalPass(P, Kn, workOff, il));
+    for (auto* v : il) if (std::find(fc.leaves.begin(), fc.leaves.end(), v) == fc.leaves.end()) fc.leaves.push_back(v);
+    fc.workspaceBytes = wb;
+  }
+  return fc;
+}
+
+}  // namespace mi355

@@ -1,0 +1,56 @@
+// HIP source generation for fused kernels.
+//
+// A fusion group is a root (an elementwise/indexing value that has to be written
+// to memory, a dynamic_update_slice window, or one or more sibling reductions)
+// plus every producer that is cheap enough to recompute per element.  The
+// generator walks the group once per output element *symbolically* and prints a
+// kernel in which broadcasts, transposes, slices, pads, concatenations, iota,
+// gather and dynamic_slice are index arithmetic, never copies.
+#pragma once
+
+#include <functional>
+#include <string>
+#include <vector>
+
+#include "ir.h"
+
+namespace mi355 {
+
+struct KArg {
+  enum Kind { In, Out, Work } kind = In;
+  Value* value = nullptr;   // In: materialised leaf; Out: root value
+  int64_t workOffset = 0;   // Work: byte offset inside the step's workspace
+};
+
+struct Launch {
+  std::string source;       // complete translation unit; entry point is always `k`
+  unsigned grid[3] = {1, 1, 1};
+  unsigned block[3] = {1, 1, 1};
+  std::vector<KArg> args;
+};
+
+struct FusedCode {
+  std::vector<Launch> launches;
+  int64_t workspaceBytes = 0;
+  std::vector<Value*> leaves;   // distinct materialised inputs
+};
+
+using LeafPredicate = std::function<bool(Value*)>;
+
+// out[i] = f(leaves...) for every element of `root`.
+FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf);
+
+// In-place window write of a dynamic_update_slice: iterates over the update
+// tensor and stores into `dus` result storage (which already holds the operand).
+FusedCode generateDusKernel(Op* dus, const LeafPredicate& isLeaf);
+
+// One or more stablehlo.reduce ops with identical input shape and dimensions.
+// Returns false in `ok` when a reducer body is not a single add/mul/max/min/and/or.
+FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeaf);
+
+// True if codegen can inline `op` into a consumer (elementwise / indexing ops).
+bool isFusibleOp(const Op& op);
+// True if the reducer body of `reduce` is one supported binary op.
+bool isSimpleReduce(const Op& reduce);
+
+}  // namespace mi355

@@ -1,0 +1,92 @@
+// Thin C-ABI layer between the host runtime (plain C++) and HIP.  Only
+// hip_abi.hip and kernels.hip include HIP headers; everything above talks to the
+// GPU through these functions.  All functions return 0 on success or a HIP error
+// code; mi355_last_error() describes the most recent failure of the calling thread.
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* mi355_stream_t;
+typedef void* mi355_event_t;
+typedef void* mi355_function_t;
+
+const char* mi355_last_error(void);
+
+// device
+int mi355_device_count(int* count);
+int mi355_device_init(int device, char* name, size_t name_len, char* arch, size_t arch_len, int* compute_units,
+                      size_t* total_mem);
+int mi355_mem_info(size_t* free_bytes, size_t* total_bytes);
+
+// memory
+int mi355_malloc(void** ptr, size_t bytes);
+int mi355_free(void* ptr);
+int mi355_host_alloc(void** ptr, size_t bytes);   // pinned
+int mi355_host_free(void* ptr);
+int mi355_memcpy_h2d(void* dst, const void* src, size_t bytes, mi355_stream_t s);
+int mi355_memcpy_d2h(void* dst, const void* src, size_t bytes, mi355_stream_t s);
+int mi355_memcpy_d2d(void* dst, const void* src, size_t bytes, mi355_stream_t s);
+
+// streams and events (default priority only)
+int mi355_stream_create(mi355_stream_t* s);
+int mi355_stream_sync(mi355_stream_t s);
+int mi355_event_create(mi355_event_t* e, int timing);
+int mi355_event_destroy(mi355_event_t e);
+int mi355_event_record(mi355_event_t e, mi355_stream_t s);
+int mi355_event_sync(mi355_event_t e);
+int mi355_event_query(mi355_event_t e, int* ready);
+int mi355_event_elapsed_ms(mi355_event_t a, mi355_event_t b, float* ms);
+
+// runtime-compiled kernels: `source` defines extern "C" __global__ void k(...).
+// mi355_rtc_compile is thread-safe (no device state); the code object it returns is
+// malloc'ed and handed to mi355_module_load, which must run on the thread that owns the device.
+int mi355_rtc_compile(const char* source, const char* arch, char** code, size_t* code_size, char* log, size_t log_len);
+int mi355_module_load(const char* code, mi355_function_t* fn);
+int mi355_launch(mi355_function_t fn, const unsigned grid[3], const unsigned block[3], void** arg_ptrs, int num_args,
+                 mi355_stream_t s);
+
+// ahead-of-time kernels (kernels.hip).  dtype codes: 0 f32, 1 bf16, 2 s32, 3 u32.
+typedef struct {
+  int64_t batch0, batch1, M, N, K;
+  int64_t aB0, aB1, aRow, aCol;
+  int64_t bB0, bB1, bRow, bCol;
+  int in_dtype, out_dtype;
+} mi355_gemm_desc;
+int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, mi355_stream_t s);
+
+typedef struct {
+  int nsp;
+  int64_t N, C, O;
+  int64_t in[3], k[3], out[3], stride[3], padLo[3], ldil[3], rdil[3], rev[3];
+  int64_t featureGroups, batchGroups;
+  int64_t lhsB, lhsF, lhsS[3], rhsI, rhsO, rhsS[3], outB, outF, outS[3];
+  int dtype;
+} mi355_conv_desc;
+// `workspace` (may be NULL) is scratch for split-K partial sums; see mi355_conv_workspace_bytes.
+int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace,
+               size_t workspace_bytes, mi355_stream_t s);
+size_t mi355_conv_workspace_bytes(const mi355_conv_desc* d);
+
+typedef struct {
+  int64_t numUpdates, rowElems, operandRows;
+  int kind;        // 0 add, 1 set, 2 mul, 3 min, 4 max
+  int dtype;       // element type code
+  int index_bytes; // 4 or 8
+} mi355_scatter_desc;
+// Deterministic row scatter: updates are applied to each destination row in the order they
+// appear in `indices` (stable sort by row, then one pass per row segment).  `result` already
+// holds the operand.  `workspace` needs mi355_scatter_workspace_bytes(numUpdates) bytes.
+int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* indices, const void* updates,
+                       void* workspace, mi355_stream_t s);
+size_t mi355_scatter_workspace_bytes(int64_t num_updates);
+
+int mi355_copy(void* dst, const void* src, size_t bytes, mi355_stream_t s);   // kernel copy (graph-capturable)
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,479 @@
+// Ahead-of-time HIP kernels for gfx950 (CDNA4): strided batched GEMM on MFMA
+// (fp32 and bf16 inputs, fp32 accumulation), direct convolution for arbitrary
+// StableHLO dimension numbers, deterministic row scatter (stable radix sort +
+// in-order segment fold) and a vector copy.
+//
+// Reference call sites these replace: dot_general -> mlx einsum/matmul
+// (src/pjrt_plugin/ops/linalg.cc:89-250), convolution -> mlx conv_general
+// (linalg.cc:253-550), scatter -> mlx scatter_add with float atomics
+// (ops/gather_scatter.cc:55-77; order-dependent there, ordered here).
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "hip_abi.h"
+
+typedef unsigned short u16;
+typedef unsigned int u32;
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ float bf2f(u16 b) { return __uint_as_float(((u32)b) << 16); }
+__device__ __forceinline__ u16 f2bf(float f) {
+  u32 u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u16)((u >> 16) | 0x40);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (u16)(u >> 16);
+}
+
+// ------------------------------------------------------------------- copy
+__global__ void __launch_bounds__(256) copy_vec16(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n16) dst[i] = src[i];
+}
+__global__ void __launch_bounds__(256) copy_bytes(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst, size_t n) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+// ------------------------------------------------------------------- GEMM
+// Workgroup tile 64x64, four wavefronts in a 2x2 arrangement, each owning a 32x32
+// accumulator held by one MFMA 32x32 instruction.  A and B tiles are staged in LDS
+// k-major (fp32) or k-minor in groups of 8 (bf16) so that every MFMA operand read is a
+// conflict-free row.  Operands are addressed through element strides, so transposed and
+// batched layouts of dot_general need no copies.
+struct GemmArgs {
+  const void* a;
+  const void* b;
+  void* c;
+  long long M, N, K;
+  long long aB0, aB1, aRow, aCol, bB0, bB1, bRow, bCol;
+  int batch1;
+  int outBf16;
+};
+
+__global__ void __launch_bounds__(256) gemm_f32_mfma(GemmArgs g) {
+  constexpr int BM = 64, BN = 64, BK = 16;
+  __shared__ float As[BK][BM + 4];
+  __shared__ float Bs[BK][BN + 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const long long b0 = blockIdx.z / g.batch1, b1 = blockIdx.z % g.batch1;
+  const float* A = (const float*)g.a + b0 * g.aB0 + b1 * g.aB1;
+  const float* B = (const float*)g.b + b0 * g.bB0 + b1 * g.bB1;
+  const long long m0 = (long long)blockIdx.y * BM, n0 = (long long)blockIdx.x * BN;
+  float16v acc = {0};
+  const bool aKfast = g.aCol == 1 || g.aRow != 1;   // walk k fastest when k is the contiguous axis
+  const bool bNfast = g.bCol == 1 || g.bRow != 1;
+  for (long long k0 = 0; k0 < g.K; k0 += BK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int e = tid + 256 * i;
+      int m, k;
+      if (aKfast) { m = e / BK; k = e % BK; } else { k = e / BM; m = e % BM; }
+      long long gm = m0 + m, gk = k0 + k;
+      As[k][m] = (gm < g.M && gk < g.K) ? A[gm * g.aRow + gk * g.aCol] : 0.f;
+      int n, kb;
+      if (bNfast) { kb = e / BN; n = e % BN; } else { n = e / BK; kb = e % BK; }
+      long long gn = n0 + n, gkb = k0 + kb;
+      Bs[kb][n] = (gn < g.N && gkb < g.K) ? B[gkb * g.bRow + gn * g.bCol] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      float av = As[kk + (lane >> 5)][wm * 32 + (lane & 31)];
+      float bv = Bs[kk + (lane >> 5)][wn * 32 + (lane & 31)];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  const long long cBase = (long long)blockIdx.z * g.M * g.N;
+  const long long col = n0 + wn * 32 + (lane & 31);
+  if (col >= g.N) return;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    long long row = m0 + wm * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
+    if (row < g.M) {
+      if (g.outBf16) ((u16*)g.c)[cBase + row * g.N + col] = f2bf(acc[j]);
+      else ((float*)g.c)[cBase + row * g.N + col] = acc[j];
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) gemm_bf16_mfma(GemmArgs g) {
+  constexpr int BM = 64, BN = 64, BK = 32;
+  __shared__ __attribute__((aligned(16))) u16 As[BM][BK + 8];
+  __shared__ __attribute__((aligned(16))) u16 Bs[BN][BK + 8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const long long b0 = blockIdx.z / g.batch1, b1 = blockIdx.z % g.batch1;
+  const u16* A = (const u16*)g.a + b0 * g.aB0 + b1 * g.aB1;
+  const u16* B = (const u16*)g.b + b0 * g.bB0 + b1 * g.bB1;
+  const long long m0 = (long long)blockIdx.y * BM, n0 = (long long)blockIdx.x * BN;
+  float16v acc = {0};
+  const bool aKfast = g.aCol == 1 || g.aRow != 1;
+  const bool bNfast = g.bCol == 1 || g.bRow != 1;
+  for (long long k0 = 0; k0 < g.K; k0 += BK) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int e = tid + 256 * i;
+      int m, k;
+      if (aKfast) { m = e / BK; k = e % BK; } else { k = e / BM; m = e % BM; }
+      long long gm = m0 + m, gk = k0 + k;
+      As[m][k] = (gm < g.M && gk < g.K) ? A[gm * g.aRow + gk * g.aCol] : (u16)0;
+      int n, kb;
+      if (bNfast) { kb = e / BN; n = e % BN; } else { n = e / BK; kb = e % BK; }
+      long long gn = n0 + n, gkb = k0 + kb;
+      Bs[n][kb] = (gn < g.N && gkb < g.K) ? B[gkb * g.bRow + gn * g.bCol] : (u16)0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 16) {
+      bf16x8 av = *(const bf16x8*)&As[wm * 32 + (lane & 31)][kk + (lane >> 5) * 8];
+      bf16x8 bv = *(const bf16x8*)&Bs[wn * 32 + (lane & 31)][kk + (lane >> 5) * 8];
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  const long long cBase = (long long)blockIdx.z * g.M * g.N;
+  const long long col = n0 + wn * 32 + (lane & 31);
+  if (col >= g.N) return;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    long long row = m0 + wm * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
+    if (row < g.M) {
+      if (g.outBf16) ((u16*)g.c)[cBase + row * g.N + col] = f2bf(acc[j]);
+      else ((float*)g.c)[cBase + row * g.N + col] = acc[j];
+    }
+  }
+}
+
+// ------------------------------------------------------------ convolution
+// Direct form: one thread per output element, fp32 accumulation.  Handles every
+// combination the StableHLO op allows (dimension numbers through strides, window
+// strides, negative padding, lhs/rhs dilation, window reversal, feature and batch groups).
+struct ConvArgs {
+  mi355_conv_desc d;
+  const void* lhs;
+  const void* rhs;
+  void* out;
+  long long total;
+};
+
+template <typename T>
+__device__ __forceinline__ float ldf(const T* p);
+template <>
+__device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <>
+__device__ __forceinline__ float ldf<u16>(const u16* p) { return bf2f(*p); }
+
+template <typename T>
+__global__ void __launch_bounds__(256) conv_direct(ConvArgs a) {
+  const mi355_conv_desc& d = a.d;
+  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= a.total) return;
+  // decompose i -> (b, o0, o1, o2, f) with f fastest when outF == 1 (feature-minor outputs), generic otherwise
+  long long r = i;
+  long long f = r % d.O; r /= d.O;
+  long long os[3] = {0, 0, 0};
+  for (int s = d.nsp - 1; s >= 0; --s) { os[s] = r % d.out[s]; r /= d.out[s]; }
+  long long b = r;
+  const long long groups = d.featureGroups > 1 ? d.featureGroups : d.batchGroups;
+  const long long opg = d.O / (groups > 0 ? groups : 1);   // output features per group
+  long long cPerGroup = d.C / d.featureGroups;
+  long long cBase = 0, bBase = b;
+  if (d.featureGroups > 1) cBase = (f / opg) * cPerGroup;
+  if (d.batchGroups > 1) bBase = (f / opg) * d.N + b;
+  const T* L = (const T*)a.lhs;
+  const T* R = (const T*)a.rhs;
+  float acc = 0.f;
+  const long long k0n = d.k[0], k1n = d.nsp > 1 ? d.k[1] : 1, k2n = d.nsp > 2 ? d.k[2] : 1;
+  for (long long k0 = 0; k0 < k0n; ++k0) {
+    long long p0 = os[0] * d.stride[0] - d.padLo[0] + k0 * d.rdil[0];
+    if (p0 < 0 || p0 % d.ldil[0] != 0) continue;
+    p0 /= d.ldil[0];
+    if (p0 >= d.in[0]) continue;
+    long long kk0 = d.rev[0] ? d.k[0] - 1 - k0 : k0;
+    for (long long k1 = 0; k1 < k1n; ++k1) {
+      long long p1 = 0, kk1 = 0;
+      if (d.nsp > 1) {
+        p1 = os[1] * d.stride[1] - d.padLo[1] + k1 * d.rdil[1];
+        if (p1 < 0 || p1 % d.ldil[1] != 0) continue;
+        p1 /= d.ldil[1];
+        if (p1 >= d.in[1]) continue;
+        kk1 = d.rev[1] ? d.k[1] - 1 - k1 : k1;
+      }
+      for (long long k2 = 0; k2 < k2n; ++k2) {
+        long long p2 = 0, kk2 = 0;
+        if (d.nsp > 2) {
+          p2 = os[2] * d.stride[2] - d.padLo[2] + k2 * d.rdil[2];
+          if (p2 < 0 || p2 % d.ldil[2] != 0) continue;
+          p2 /= d.ldil[2];
+          if (p2 >= d.in[2]) continue;
+          kk2 = d.rev[2] ? d.k[2] - 1 - k2 : k2;
+        }
+        const T* lp = L + bBase * d.lhsB + cBase * d.lhsF + p0 * d.lhsS[0] + p1 * d.lhsS[1] + p2 * d.lhsS[2];
+        const T* rp = R + f * d.rhsO + kk0 * d.rhsS[0] + kk1 * d.rhsS[1] + kk2 * d.rhsS[2];
+        for (long long c = 0; c < cPerGroup; ++c) acc += ldf<T>(lp + c * d.lhsF) * ldf<T>(rp + c * d.rhsI);
+      }
+    }
+  }
+  long long off = b * d.outB + f * d.outF + os[0] * d.outS[0] + os[1] * d.outS[1] + os[2] * d.outS[2];
+  if (sizeof(T) == 2) ((u16*)a.out)[off] = f2bf(acc);
+  else ((float*)a.out)[off] = acc;
+}
+
+// ---------------------------------------------------------- row scatter
+// keys[i] = destination row of update i (`rows` if outside the operand: dropped),
+// vals[i] = i.  A stable LSD radix sort by key keeps updates of one row in their
+// original order; every row segment is then folded front to back.
+__global__ void __launch_bounds__(256) scatter_init_keys(const void* idx, int idxBytes, long long n, long long rows, u32* keys, u32* vals) {
+  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  long long r = idxBytes == 8 ? ((const long long*)idx)[i] : (long long)((const int*)idx)[i];
+  keys[i] = (r < 0 || r >= rows) ? (u32)rows : (u32)r;   // rows = "dropped", sorts last
+  vals[i] = (u32)i;
+}
+
+constexpr int kSortBlocks = 64;
+
+__global__ void __launch_bounds__(256) radix_hist(const u32* __restrict__ keys, long long n, int shift, u32* __restrict__ counts) {
+  __shared__ u32 h[256];
+  h[threadIdx.x] = 0;
+  __syncthreads();
+  long long chunk = (n + gridDim.x - 1) / gridDim.x;
+  long long lo = (long long)blockIdx.x * chunk, hi = lo + chunk < n ? lo + chunk : n;
+  for (long long i = lo + threadIdx.x; i < hi; i += 256) atomicAdd(&h[(keys[i] >> shift) & 255u], 1u);
+  __syncthreads();
+  counts[threadIdx.x * gridDim.x + blockIdx.x] = h[threadIdx.x];   // digit-major
+}
+
+__global__ void __launch_bounds__(256) radix_scan(u32* counts, int nblocks) {
+  // exclusive scan over 256*nblocks counters, digit-major; one workgroup
+  __shared__ u32 tot[256];
+  u32 sum = 0;
+  for (int b = 0; b < nblocks; ++b) sum += counts[threadIdx.x * nblocks + b];
+  tot[threadIdx.x] = sum;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    u32 run = 0;
+    for (int d = 0; d < 256; ++d) { u32 t = tot[d]; tot[d] = run; run += t; }
+  }
+  __syncthreads();
+  u32 run = tot[threadIdx.x];
+  for (int b = 0; b < nblocks; ++b) {
+    u32 c = counts[threadIdx.x * nblocks + b];
+    counts[threadIdx.x * nblocks + b] = run;
+    run += c;
+  }
+}
+
+__global__ void __launch_bounds__(256) radix_scatter(const u32* __restrict__ keysIn, const u32* __restrict__ valsIn, long long n, int shift,
+                                                     const u32* __restrict__ offsets, u32* __restrict__ keysOut, u32* __restrict__ valsOut) {
+  __shared__ u32 base[256];          // running output position per digit for this block
+  __shared__ u32 waveCount[4][256];  // per-wave digit counts of the current tile
+  base[threadIdx.x] = offsets[threadIdx.x * gridDim.x + blockIdx.x];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  long long chunk = (n + gridDim.x - 1) / gridDim.x;
+  long long lo = (long long)blockIdx.x * chunk, hi = lo + chunk < n ? lo + chunk : n;
+  for (long long t0 = lo; t0 < hi; t0 += 256) {
+    for (int w = 0; w < 4; ++w) waveCount[w][threadIdx.x] = 0;
+    __syncthreads();
+    long long i = t0 + threadIdx.x;
+    bool valid = i < hi;
+    u32 key = valid ? keysIn[i] : 0u, val = valid ? valsIn[i] : 0u;
+    u32 digit = (key >> shift) & 255u;
+    // lanes of this wavefront holding the same digit
+    unsigned long long peers = __ballot(valid);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      unsigned long long m = __ballot((digit >> b) & 1u);
+      peers &= ((digit >> b) & 1u) ? m : ~m;
+    }
+    unsigned long long lower = peers & ((1ull << lane) - 1ull);
+    u32 rankInWave = (u32)__popcll(lower);
+    if (valid && lower == 0) waveCount[wave][digit] = (u32)__popcll(peers);
+    __syncthreads();
+    if (valid) {
+      u32 pos = base[digit] + rankInWave;
+      for (int w = 0; w < wave; ++w) pos += waveCount[w][digit];
+      keysOut[pos] = key;
+      valsOut[pos] = val;
+    }
+    __syncthreads();
+    base[threadIdx.x] += waveCount[0][threadIdx.x] + waveCount[1][threadIdx.x] + waveCount[2][threadIdx.x] + waveCount[3][threadIdx.x];
+    __syncthreads();
+  }
+}
+
+template <typename T>
+struct ScatterOps;
+template <>
+struct ScatterOps<float> {
+  static __device__ __forceinline__ float apply(int kind, float a, float u) {
+    switch (kind) {
+      case 0: return a + u;
+      case 1: return u;
+      case 2: return a * u;
+      case 3: return (a < u || a != a) ? a : u;
+      default: return (a > u || a != a) ? a : u;
+    }
+  }
+};
+template <>
+struct ScatterOps<int> {
+  static __device__ __forceinline__ int apply(int kind, int a, int u) {
+    switch (kind) {
+      case 0: return a + u;
+      case 1: return u;
+      case 2: return a * u;
+      case 3: return a < u ? a : u;
+      default: return a > u ? a : u;
+    }
+  }
+};
+template <>
+struct ScatterOps<u32> {
+  static __device__ __forceinline__ u32 apply(int kind, u32 a, u32 u) {
+    switch (kind) {
+      case 0: return a + u;
+      case 1: return u;
+      case 2: return a * u;
+      case 3: return a < u ? a : u;
+      default: return a > u ? a : u;
+    }
+  }
+};
+
+// grid.x = update position (only segment heads work), grid.y = column chunk of 256*VEC elements
+template <typename T>
+__global__ void __launch_bounds__(256) scatter_fold(const u32* __restrict__ keys, const u32* __restrict__ vals, long long n, long long rowElems,
+                                                    int kind, T* __restrict__ result, const T* __restrict__ updates, u32 rows) {
+  long long i = blockIdx.x;
+  u32 key = keys[i];
+  if (key >= rows) return;
+  if (i > 0 && keys[i - 1] == key) return;
+  long long col = (long long)blockIdx.y * 256 + threadIdx.x;
+  if (col >= rowElems) return;
+  T acc = result[(long long)key * rowElems + col];
+  for (long long j = i; j < n && keys[j] == key; ++j) acc = ScatterOps<T>::apply(kind, acc, updates[(long long)vals[j] * rowElems + col]);
+  result[(long long)key * rowElems + col] = acc;
+}
+
+__global__ void __launch_bounds__(256) scatter_fold_bf16(const u32* __restrict__ keys, const u32* __restrict__ vals, long long n, long long rowElems,
+                                                         int kind, u16* __restrict__ result, const u16* __restrict__ updates, u32 rows) {
+  long long i = blockIdx.x;
+  u32 key = keys[i];
+  if (key >= rows) return;
+  if (i > 0 && keys[i - 1] == key) return;
+  long long col = (long long)blockIdx.y * 256 + threadIdx.x;
+  if (col >= rowElems) return;
+  float acc = bf2f(result[(long long)key * rowElems + col]);
+  for (long long j = i; j < n && keys[j] == key; ++j)
+    acc = bf2f(f2bf(ScatterOps<float>::apply(kind, acc, bf2f(updates[(long long)vals[j] * rowElems + col]))));
+  result[(long long)key * rowElems + col] = f2bf(acc);
+}
+
+namespace {
+thread_local const char* g_kerr = "";
+int check(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { g_kerr = what; return (int)e; }
+  return 0;
+}
+}  // namespace
+
+extern "C" {
+
+int mi355_copy(void* dst, const void* src, size_t bytes, mi355_stream_t s) {
+  if (bytes == 0 || dst == src) return 0;
+  hipStream_t st = (hipStream_t)s;
+  if (((uintptr_t)dst | (uintptr_t)src | bytes) % 16 == 0) {
+    size_t n16 = bytes / 16;
+    copy_vec16<<<(unsigned)((n16 + 255) / 256), 256, 0, st>>>((const uint4*)src, (uint4*)dst, n16);
+  } else {
+    copy_bytes<<<(unsigned)((bytes + 255) / 256), 256, 0, st>>>((const unsigned char*)src, (unsigned char*)dst, bytes);
+  }
+  return check("copy");
+}
+
+int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, mi355_stream_t s) {
+  if (d->M <= 0 || d->N <= 0 || d->batch0 * d->batch1 <= 0) return 0;
+  GemmArgs g;
+  g.a = a; g.b = b; g.c = c;
+  g.M = d->M; g.N = d->N; g.K = d->K;
+  g.aB0 = d->aB0; g.aB1 = d->aB1; g.aRow = d->aRow; g.aCol = d->aCol;
+  g.bB0 = d->bB0; g.bB1 = d->bB1; g.bRow = d->bRow; g.bCol = d->bCol;
+  g.batch1 = (int)d->batch1;
+  g.outBf16 = d->out_dtype == 1;
+  long long nb = d->batch0 * d->batch1;
+  if (nb > 65535) return 1;   // grid.z limit; callers fold larger batches
+  dim3 grid((unsigned)((d->N + 63) / 64), (unsigned)((d->M + 63) / 64), (unsigned)nb);
+  if (d->in_dtype == 0) gemm_f32_mfma<<<grid, 256, 0, (hipStream_t)s>>>(g);
+  else if (d->in_dtype == 1) gemm_bf16_mfma<<<grid, 256, 0, (hipStream_t)s>>>(g);
+  else return 2;
+  return check("gemm");
+}
+
+size_t mi355_conv_workspace_bytes(const mi355_conv_desc* d) {
+  (void)d;
+  return 0;
+}
+
+int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes,
+               mi355_stream_t s) {
+  (void)workspace;
+  (void)workspace_bytes;
+  ConvArgs a;
+  a.d = *d;
+  a.lhs = lhs; a.rhs = rhs; a.out = out;
+  long long total = d->N * d->O;
+  for (int k = 0; k < d->nsp; ++k) total *= d->out[k];
+  a.total = total;
+  if (total <= 0) return 0;
+  unsigned grid = (unsigned)((total + 255) / 256);
+  if (d->dtype == 0) conv_direct<float><<<grid, 256, 0, (hipStream_t)s>>>(a);
+  else if (d->dtype == 1) conv_direct<u16><<<grid, 256, 0, (hipStream_t)s>>>(a);
+  else return 2;
+  return check("conv");
+}
+
+size_t mi355_scatter_workspace_bytes(int64_t n) {
+  // keys[2][n], vals[2][n], counts[256*kSortBlocks]
+  return (size_t)(4 * n * 4 + 256 * kSortBlocks * 4 + 1024);
+}
+
+int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* indices, const void* updates, void* workspace,
+                       mi355_stream_t s) {
+  long long n = d->numUpdates;
+  if (n <= 0 || d->rowElems <= 0) return 0;
+  hipStream_t st = (hipStream_t)s;
+  u32* keys0 = (u32*)workspace;
+  u32* keys1 = keys0 + n;
+  u32* vals0 = keys1 + n;
+  u32* vals1 = vals0 + n;
+  u32* counts = vals1 + n;
+  unsigned gb = (unsigned)((n + 255) / 256);
+  scatter_init_keys<<<gb, 256, 0, st>>>(indices, d->index_bytes, n, d->operandRows, keys0, vals0);
+  // keys lie in [0, rows]: sort only the bits that can be set
+  int bits = 1;
+  while (bits < 32 && (1ll << bits) <= d->operandRows) ++bits;
+  u32 *kin = keys0, *kout = keys1, *vin = vals0, *vout = vals1;
+  for (int shift = 0; shift < bits; shift += 8) {
+    radix_hist<<<kSortBlocks, 256, 0, st>>>(kin, n, shift, counts);
+    radix_scan<<<1, 256, 0, st>>>(counts, kSortBlocks);
+    radix_scatter<<<kSortBlocks, 256, 0, st>>>(kin, vin, n, shift, counts, kout, vout);
+    u32* t = kin; kin = kout; kout = t;
+    t = vin; vin = vout; vout = t;
+  }
+  dim3 grid((unsigned)n, (unsigned)((d->rowElems + 255) / 256));
+  if (d->dtype == 0) scatter_fold<float><<<grid, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (float*)result, (const float*)updates, (u32)d->operandRows);
+  else if (d->dtype == 2) scatter_fold<int><<<grid, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (int*)result, (const int*)updates, (u32)d->operandRows);
+  else if (d->dtype == 3) scatter_fold<u32><<<grid, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (u32*)result, (const u32*)updates, (u32)d->operandRows);
+  else if (d->dtype == 1) scatter_fold_bf16<<<grid, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (u16*)result, (const u16*)updates, (u32)d->operandRows);
+  else return 2;
+  return check("scatter_rows");
+}
+
+}  // extern "C"

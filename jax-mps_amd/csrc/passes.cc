@@ -1,0 +1,250 @@
+// Module-level passes run once at PJRT_Client_Compile: call inlining, dead-code
+// elimination and the supported-op check.  The reference does the same three
+// things with MLIR's inliner + SymbolDCE and its handler-table scan (reference:
+// src/pjrt_plugin/stablehlo_parser.cc:129-149, 167-184).
+#include <functional>
+#include <set>
+#include <unordered_map>
+#include <unordered_set>
+
+#include "ir.h"
+
+namespace mi355 {
+
+namespace {
+
+using VMap = std::unordered_map<Value*, Value*>;
+
+std::unique_ptr<Op> cloneOp(const Op& src, VMap& map, int& nextId);
+
+std::unique_ptr<Region> cloneRegion(const Region& src, Op* parent, VMap& map, int& nextId) {
+  auto r = std::make_unique<Region>();
+  r->parent = parent;
+  for (auto& a : src.args) {
+    auto v = std::make_unique<Value>();
+    v->id = nextId++;
+    v->type = a->type;
+    v->name = a->name;
+    v->argOf = r.get();
+    v->defIndex = a->defIndex;
+    map[a.get()] = v.get();
+    r->args.push_back(std::move(v));
+  }
+  for (auto& o : src.ops) {
+    auto c = cloneOp(*o, map, nextId);
+    c->parent = r.get();
+    r->ops.push_back(std::move(c));
+  }
+  return r;
+}
+
+std::unique_ptr<Op> cloneOp(const Op& src, VMap& map, int& nextId) {
+  auto op = std::make_unique<Op>();
+  op->name = src.name;
+  op->attrs = src.attrs;
+  op->convDims = src.convDims;
+  op->line = src.line;
+  for (auto* v : src.operands) {
+    auto it = map.find(v);
+    op->operands.push_back(it == map.end() ? v : it->second);
+  }
+  for (auto& r : src.results) {
+    auto v = std::make_unique<Value>();
+    v->id = nextId++;
+    v->type = r->type;
+    v->name = r->name;
+    v->def = op.get();
+    v->defIndex = r->defIndex;
+    map[r.get()] = v.get();
+    op->results.push_back(std::move(v));
+  }
+  for (auto& r : src.regions) op->regions.push_back(cloneRegion(*r, op.get(), map, nextId));
+  return op;
+}
+
+int maxValueId(const Region& r) {
+  int m = -1;
+  for (auto& a : r.args) m = std::max(m, a->id);
+  for (auto& o : r.ops) {
+    for (auto& v : o->results) m = std::max(m, v->id);
+    for (auto& sub : o->regions) m = std::max(m, maxValueId(*sub));
+  }
+  return m;
+}
+
+void applyReplacements(Region& r, const VMap& repl) {
+  auto resolve = [&](Value* v) {
+    auto it = repl.find(v);
+    while (it != repl.end()) {
+      v = it->second;
+      it = repl.find(v);
+    }
+    return v;
+  };
+  for (auto& o : r.ops) {
+    for (auto& v : o->operands) v = resolve(v);
+    for (auto& sub : o->regions) applyReplacements(*sub, repl);
+  }
+}
+
+bool inlineRegion(Module& m, Region& r, VMap& repl, int& nextId, int depth) {
+  if (depth > 64) throw CompileError("call inlining exceeded depth 64 (recursive functions are not supported)");
+  bool any = false;
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) any |= inlineRegion(m, *sub, repl, nextId, depth);
+    if (op->name != "call") continue;
+    Func* callee = m.find(op->str("callee"));
+    if (!callee) throw CompileError("call to unknown function @" + op->str("callee"));
+    if (callee->body.args.size() != op->operands.size()) throw CompileError("call @" + callee->name + ": argument count mismatch");
+    VMap map;
+    for (size_t a = 0; a < op->operands.size(); ++a) map[callee->body.args[a].get()] = op->operands[a];
+    std::vector<std::unique_ptr<Op>> cloned;
+    for (auto& o : callee->body.ops) cloned.push_back(cloneOp(*o, map, nextId));
+    Op* ret = cloned.back().get();
+    if (ret->name != "return" || ret->operands.size() != op->results.size())
+      throw CompileError("call @" + callee->name + ": result count mismatch");
+    for (size_t q = 0; q < op->results.size(); ++q) repl[op->results[q].get()] = ret->operands[q];
+    cloned.pop_back();
+    // keep the call op alive (its result Values are referenced by `repl` keys) but mark it dead
+    op->dead = true;
+    size_t nIns = cloned.size();
+    for (auto& c : cloned) c->parent = &r;
+    r.ops.insert(r.ops.begin() + k, std::make_move_iterator(cloned.begin()), std::make_move_iterator(cloned.end()));
+    // re-scan the inlined ops (they may contain calls themselves)
+    any = true;
+    k += nIns;  // now points at the dead call
+    (void)ret;
+  }
+  return any;
+}
+
+void removeDead(Region& r) {
+  for (auto& o : r.ops) for (auto& sub : o->regions) removeDead(*sub);
+  std::vector<std::unique_ptr<Op>> keep;
+  for (auto& o : r.ops) if (!o->dead) keep.push_back(std::move(o));
+  r.ops.swap(keep);
+}
+
+void collectUses(const Region& r, std::unordered_map<const Value*, int>& uses) {
+  for (auto& o : r.ops) {
+    if (o->dead) continue;
+    for (auto* v : o->operands) uses[v]++;
+    for (auto& sub : o->regions) collectUses(*sub, uses);
+  }
+}
+
+bool sweep(Region& r, std::unordered_map<const Value*, int>& uses) {
+  bool changed = false;
+  for (int k = (int)r.ops.size() - 1; k >= 0; --k) {
+    Op* o = r.ops[k].get();
+    if (o->dead) continue;
+    if (o->name != "return") {
+      bool used = false;
+      for (auto& v : o->results) if (uses[v.get()] > 0) used = true;
+      if (!used) {
+        o->dead = true;
+        std::function<void(Op*)> drop = [&](Op* q) {
+          for (auto* v : q->operands) uses[v]--;
+          for (auto& sub : q->regions) for (auto& qq : sub->ops) if (!qq->dead) drop(qq.get());
+        };
+        drop(o);
+        changed = true;
+        continue;
+      }
+    }
+    for (auto& sub : o->regions) changed |= sweep(*sub, uses);
+  }
+  return changed;
+}
+
+}  // namespace
+
+void inlineCalls(Module& m) {
+  Func* main = m.main();
+  int nextId = 0;
+  for (auto& f : m.funcs) nextId = std::max(nextId, maxValueId(f->body) + 1);
+  VMap repl;
+  for (int iter = 0; iter < 64; ++iter) {
+    if (!inlineRegion(m, main->body, repl, nextId, 0)) break;
+    applyReplacements(main->body, repl);
+    // dead call ops must stay until replacements are resolved, then go
+    removeDead(main->body);
+    repl.clear();
+  }
+}
+
+void eliminateDeadCode(Region& r) {
+  std::unordered_map<const Value*, int> uses;
+  collectUses(r, uses);
+  while (sweep(r, uses)) {}
+  removeDead(r);
+}
+
+void rebuildUses(Region& r) {
+  std::function<void(Region&)> clear = [&](Region& q) {
+    for (auto& a : q.args) a->users.clear();
+    for (auto& o : q.ops) {
+      for (auto& v : o->results) v->users.clear();
+      for (auto& sub : o->regions) clear(*sub);
+    }
+  };
+  std::function<void(Region&)> fill = [&](Region& q) {
+    for (auto& o : q.ops) {
+      for (auto* v : o->operands) v->users.push_back(o.get());
+      for (auto& sub : o->regions) fill(*sub);
+    }
+  };
+  clear(r);
+  fill(r);
+}
+
+int countOps(const Region& r) {
+  int n = 0;
+  for (auto& o : r.ops) {
+    ++n;
+    for (auto& sub : o->regions) n += countOps(*sub);
+  }
+  return n;
+}
+
+static const std::set<std::string>& supportedOps() {
+  static const std::set<std::string> s = {
+      // elementwise (reference: ops/arithmetic.cc:535-607)
+      "add", "subtract", "multiply", "divide", "maximum", "minimum", "power", "remainder", "atan2", "and", "or", "xor",
+      "not", "negate", "abs", "exponential", "exponential_minus_one", "log", "log_plus_one", "sqrt", "rsqrt", "cbrt",
+      "tanh", "tan", "sine", "cosine", "logistic", "floor", "ceil", "sign", "round_nearest_even", "round_nearest_afz",
+      "is_finite", "shift_left", "shift_right_logical", "shift_right_arithmetic", "popcnt", "count_leading_zeros",
+      "compare", "select", "clamp", "convert", "bitcast_convert", "reduce_precision",
+      // shape / slicing (ops/shape.cc:260-270, ops/slice.cc:280-285)
+      "constant", "iota", "reshape", "broadcast_in_dim", "transpose", "reverse", "concatenate", "slice", "dynamic_slice",
+      "dynamic_update_slice", "pad",
+      // heavy ops
+      "reduce", "dot_general", "dot", "convolution", "gather", "scatter",
+      // control flow (ops/control_flow.cc:2364-2376)
+      "while", "case", "return", "optimization_barrier", "custom_call",
+  };
+  return s;
+}
+
+static void scan(const Region& r, std::set<std::string>& bad) {
+  for (auto& o : r.ops) {
+    if (!supportedOps().count(o->name)) bad.insert(o->name);
+    if (o->name == "custom_call") {
+      const std::string& t = o->str("target");
+      if (t != "Sharding" && t != "SPMDFullToShardShape" && t != "SPMDShardToFullShape") bad.insert("custom_call @" + t);
+    }
+    for (auto& sub : o->regions) scan(*sub, bad);
+  }
+}
+
+void checkSupported(const Module& m) {
+  std::set<std::string> bad;
+  scan(m.main()->body, bad);
+  if (bad.empty()) return;
+  std::string msg = "unsupported StableHLO operation(s):";
+  for (auto& b : bad) msg += " " + b;
+  throw CompileError(msg);
+}
+
+}  // namespace mi355

@@ -1,0 +1,116 @@
+// Execution plan: what PJRT_Client_Compile produces from a StableHLO module and
+// what PJRT_LoadedExecutable_Execute replays.  A plan is a list of steps over
+// statically assigned buffers; there is no per-call graph walk (the reference
+// re-dispatches ops through a string-keyed handler table on the first call and
+// replays an MLX-compiled graph afterwards, src/pjrt_plugin/mlx_executable.cc:799-1008).
+#pragma once
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "ir.h"
+
+namespace mi355 {
+
+// Where a materialised value lives during one execution.
+struct BufRef {
+  enum Kind : uint8_t { None, Param, Output, Temp, Const } kind = None;
+  int index = 0;       // parameter / output number
+  int64_t offset = 0;  // byte offset inside the arena (Temp) or the constant pool (Const)
+  bool operator==(const BufRef& o) const { return kind == o.kind && index == o.index && offset == o.offset; }
+  bool operator!=(const BufRef& o) const { return !(*this == o); }
+};
+
+// One generated (runtime-compiled) kernel; identical sources are shared.
+struct GenKernel {
+  std::string name;
+  std::string source;
+  void* function = nullptr;  // hipFunction_t once loaded
+};
+
+struct GemmDesc {   // C[b0,b1] = A[b0,b1] x B[b0,b1]; operands addressed through element strides, C dense row-major
+  int64_t batch0 = 1, batch1 = 1, M = 0, N = 0, K = 0;
+  int64_t aB0 = 0, aB1 = 0, aRow = 0, aCol = 0;   // A(m,k) = a[b0*aB0 + b1*aB1 + m*aRow + k*aCol]
+  int64_t bB0 = 0, bB1 = 0, bRow = 0, bCol = 0;   // B(k,n) = b[b0*bB0 + b1*bB1 + k*bRow + n*bCol]
+  DType inType = DType::F32, outType = DType::F32;
+};
+
+struct ConvDesc {   // StableHLO convolution with arbitrary dimension numbers (<= 3 spatial dims, kernels specialise 2)
+  int nsp = 2;
+  int64_t N = 0, C = 0, O = 0;             // batch (per batch group), input features (total), output features
+  int64_t in[3] = {1, 1, 1}, k[3] = {1, 1, 1}, out[3] = {1, 1, 1};
+  int64_t stride[3] = {1, 1, 1}, padLo[3] = {0, 0, 0}, ldil[3] = {1, 1, 1}, rdil[3] = {1, 1, 1};
+  int64_t rev[3] = {0, 0, 0};
+  int64_t featureGroups = 1, batchGroups = 1;
+  // element strides of each logical dim in the three tensors
+  int64_t lhsB = 0, lhsF = 0, lhsS[3] = {0, 0, 0};
+  int64_t rhsI = 0, rhsO = 0, rhsS[3] = {0, 0, 0};
+  int64_t outB = 0, outF = 0, outS[3] = {0, 0, 0};
+  DType type = DType::F32;
+};
+
+struct ScatterDesc {   // row scatter: operand [rows, rowSize...], one index per update row
+  int64_t numUpdates = 0, rowElems = 0, operandRows = 0;
+  int kind = 0;        // 0 add, 1 set, 2 mul, 3 min, 4 max
+  DType type = DType::F32, indexType = DType::S32;
+};
+
+struct Plan;
+
+struct Step {
+  enum Kind { Kernel, Gemm, Conv, ScatterRows, Copy, Fill, While, Case } kind = Kernel;
+  std::string label;  // op name(s) for profiling ranges and error messages
+
+  // Kernel
+  int kernel = -1;
+  unsigned grid[3] = {1, 1, 1}, block[3] = {1, 1, 1};
+  std::vector<BufRef> args;        // pointer arguments, in kernel order
+  int64_t algoBytes = 0;           // distinct input bytes + output bytes (for bandwidth reports)
+
+  // Gemm / Conv / ScatterRows
+  GemmDesc gemm;
+  ConvDesc conv;
+  ScatterDesc scatter;
+  int64_t workspaceOffset = -1;    // arena offset of split-K / sort scratch
+  int64_t workspaceBytes = 0;
+  int splitK = 1;
+
+  // Copy / Fill
+  BufRef src, dst;
+  int64_t bytes = 0;
+
+  // While / Case
+  std::unique_ptr<Plan> cond;                 // While: evaluates the predicate into predBuf
+  std::vector<std::unique_ptr<Plan>> bodies;  // While: [body]; Case: branches
+  BufRef predBuf;                             // i1 (While) or i32 index (Case)
+  int64_t tripCount = -1;                     // >= 0 when the loop is counted and the count is static
+  DType predType = DType::Pred;
+};
+
+struct Plan {
+  std::vector<Step> steps;
+};
+
+struct OutputInfo {
+  TensorType type;
+};
+
+struct CompiledProgram {
+  std::unique_ptr<Module> module;
+  Plan plan;
+  std::vector<GenKernel> kernels;
+  std::vector<TensorType> paramTypes;
+  std::vector<OutputInfo> outputs;
+  std::vector<uint8_t> constPool;   // host image of the constant pool
+  int64_t arenaBytes = 0;
+  int numOps = 0, numSteps = 0;
+  std::string dump;                 // human-readable plan (MI355X_DUMP_PLAN)
+};
+
+// planner.cc
+std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module);
+
+}  // namespace mi355

@@ -1,0 +1,901 @@
+// StableHLO module -> execution plan.
+//
+//  1. decide which values are written to memory (everything else is recomputed
+//     inside the kernel that needs it),
+//  2. emit one step per materialised root in program order (generated fused
+//     kernels, GEMM / convolution / row-scatter library steps, loops, branches),
+//  3. assign every temporary a fixed offset in one arena by liveness.
+//
+// The chains that end up fused are the ones the reference's pattern pass names
+// (bias-add, softmax, LayerNorm, RMSNorm: src/pjrt_plugin/passes/*.cc) plus
+// whatever else is elementwise; nothing here is pattern-matched by name.
+#include <algorithm>
+#include <functional>
+#include <set>
+#include <sstream>
+#include <unordered_map>
+#include <unordered_set>
+
+#include "codegen.h"
+#include "plan.h"
+
+namespace mi355 {
+
+namespace {
+
+constexpr int64_t kSmallNumel = 8192;   // values at most this big are never materialised just to avoid recomputation
+constexpr int64_t kAlign = 256;
+
+struct Storage {
+  BufRef::Kind kind = BufRef::Temp;
+  int index = 0;          // param / output number
+  int64_t bytes = 0;
+  int64_t offset = -1;    // arena or const-pool offset
+  int first = -1, last = -1;
+  std::vector<int> uses;
+  int values = 0;         // SSA values bound to this storage
+};
+
+bool isExpensive(const std::string& n) {
+  static const std::set<std::string> s = {"exponential", "exponential_minus_one", "log", "log_plus_one", "tanh", "tan",
+                                          "sine", "cosine", "logistic", "power", "atan2", "cbrt", "remainder", "gather"};
+  return s.count(n) != 0;
+}
+
+bool isPassThrough(const Op& op) {
+  return op.name == "optimization_barrier" || op.name == "custom_call";
+}
+
+class Planner {
+ public:
+  explicit Planner(CompiledProgram& p) : P(p) {}
+
+  void run() {
+    Func* main = P.module->main();
+    Region& body = main->body;
+    rebuildUses(body);
+    for (auto& a : body.args) {
+      P.paramTypes.push_back(a->type);
+      int sid = newStorage(a->type.bytes(), BufRef::Param, (int)P.paramTypes.size() - 1);
+      bind(a.get(), sid);
+    }
+    analyze(body);
+    emitRegion(body, P.plan);
+    // program outputs
+    Op* ret = body.terminator();
+    int t = ++time_;
+    for (size_t k = 0; k < ret->operands.size(); ++k) {
+      Value* v = ret->operands[k];
+      OutputInfo oi;
+      oi.type = v->type;
+      P.outputs.push_back(oi);
+      int sid = storageOf(v);
+      Storage& s = st_[sid];
+      if (s.kind == BufRef::Temp && !boundToOutput_.count(sid)) {
+        s.kind = BufRef::Output;
+        s.index = (int)k;
+        boundToOutput_.insert(sid);
+      } else {
+        int out = newStorage(v->type.bytes(), BufRef::Output, (int)k);
+        Step c;
+        c.kind = Step::Copy;
+        c.label = "copy-to-output";
+        c.src = ref(sid, t);
+        c.dst = ref(out, t);
+        c.bytes = (int64_t)v->type.bytes();
+        P.plan.steps.push_back(std::move(c));
+      }
+    }
+    assignArena();
+    patch(P.plan);
+    P.numSteps = countSteps(P.plan);
+    P.numOps = countOps(body);
+    if (getenv("MI355X_DUMP_PLAN")) dumpPlan(P.plan, 0);
+  }
+
+ private:
+  CompiledProgram& P;
+  std::vector<Storage> st_;
+  std::unordered_map<Value*, int> storage_;
+  std::unordered_map<Value*, bool> needMat_;
+  std::unordered_map<std::string, int> kernelIds_;
+  std::unordered_set<int> boundToOutput_;
+  std::vector<std::pair<int, int>> loops_;
+  std::unordered_set<Op*> emitted_;
+  int time_ = 0;
+
+  // ---------------------------------------------------------------- storages
+  int newStorage(size_t bytes, BufRef::Kind kind = BufRef::Temp, int index = 0) {
+    Storage s;
+    s.kind = kind;
+    s.index = index;
+    s.bytes = (int64_t)std::max<size_t>(bytes, 4);
+    st_.push_back(s);
+    return (int)st_.size() - 1;
+  }
+  void bind(Value* v, int sid) {
+    storage_[v] = sid;
+    st_[sid].values++;
+  }
+  bool hasStorage(Value* v) const { return storage_.count(v) != 0; }
+  int storageOf(Value* v) {
+    auto it = storage_.find(v);
+    if (it == storage_.end()) throw CompileError("internal: value " + v->name + " has no storage");
+    return it->second;
+  }
+  BufRef ref(int sid, int t) {
+    Storage& s = st_[sid];
+    s.uses.push_back(t);
+    if (s.first < 0 || t < s.first) s.first = t;
+    if (t > s.last) s.last = t;
+    BufRef r;
+    r.kind = BufRef::Temp;   // patched after arena assignment
+    r.index = sid;
+    return r;
+  }
+
+  // ---------------------------------------------------------------- analysis
+  static Region* regionOf(Value* v) { return v->def ? v->def->parent : v->argOf; }
+
+  static bool forcedBy(Value* v, Op* user) {
+    if (user->name == "gather") return user->operands[0] == v;       // random access needs memory
+    if (isFusibleOp(*user)) return false;
+    if (user->name == "reduce") return !isSimpleReduce(*user);
+    if (user->name == "dynamic_update_slice") return user->operands[0] == v;
+    return true;
+  }
+
+  void analyze(Region& r) {
+    // forward: set of leaves every value depends on (capped)
+    std::unordered_map<Value*, std::vector<Value*>> leaves;
+    auto addLeaf = [](std::vector<Value*>& dst, Value* l) {
+      if (dst.size() < 6 && std::find(dst.begin(), dst.end(), l) == dst.end()) dst.push_back(l);
+    };
+    for (auto& op : r.ops) {
+      for (auto& sub : op->regions) analyze(*sub);
+      if (!isFusibleOp(*op) || op->results.size() != 1) continue;
+      auto& mine = leaves[op->result()];
+      for (auto* o : op->operands) {
+        auto it = leaves.find(o);
+        if (it == leaves.end()) addLeaf(mine, o);
+        else for (auto* l : it->second) addLeaf(mine, l);
+      }
+    }
+    // reverse: materialisation decisions
+    std::unordered_map<Value*, std::vector<Op*>> groups;
+    for (int k = (int)r.ops.size() - 1; k >= 0; --k) {
+      Op* op = r.ops[k].get();
+      if (!isFusibleOp(*op) || op->results.size() != 1) continue;
+      Value* v = op->result();
+      bool forced = false;
+      std::vector<Op*> g;
+      auto addGroup = [&](Op* o) { if (g.size() < 4 && std::find(g.begin(), g.end(), o) == g.end()) g.push_back(o); };
+      for (Op* u : v->users) {
+        if (u->parent != &r) { forced = true; continue; }
+        if (forcedBy(v, u)) { forced = true; continue; }
+        if (u->name == "reduce" || u->name == "dynamic_update_slice") { addGroup(u); continue; }
+        Value* ur = u->result();
+        if (needMat_[ur]) addGroup(u);
+        else for (Op* q : groups[ur]) addGroup(q);
+      }
+      bool mat = forced;
+      if (op->name == "constant") {
+        auto& d = *op->attrs.at("value").dense;
+        if (!d.splat && d.type.numel() > 1) mat = true;
+      }
+      if (!mat && v->type.numel() > kSmallNumel && g.size() >= 2) {
+        int big = 0;
+        for (auto* l : leaves[v]) if (l->type.numel() * 4 >= v->type.numel()) ++big;
+        bool expensive = isExpensive(op->name);
+        for (auto* o : op->operands) if (o->def && !needMat_[o] && isExpensive(o->def->name) && o->def->parent == &r) expensive = true;
+        if (big >= 2 || expensive) mat = true;
+      }
+      needMat_[v] = mat;
+      if (mat) { g.clear(); g.push_back(op); }
+      groups[v] = g;
+    }
+  }
+
+  // ---------------------------------------------------------------- emission
+  LeafPredicate leafPred() {
+    return [this](Value* v) { return storage_.count(v) != 0; };
+  }
+
+  int kernelId(const std::string& source) {
+    auto it = kernelIds_.find(source);
+    if (it != kernelIds_.end()) return it->second;
+    GenKernel k;
+    k.name = "k";
+    k.source = source;
+    P.kernels.push_back(std::move(k));
+    int id = (int)P.kernels.size() - 1;
+    kernelIds_[source] = id;
+    return id;
+  }
+
+  void addFused(Plan& plan, const FusedCode& fc, const std::string& label, const std::vector<Value*>& outs) {
+    int ws = -1;
+    int t0 = time_ + 1;
+    int t1 = time_ + (int)fc.launches.size();
+    if (fc.workspaceBytes > 0) {
+      ws = newStorage((size_t)fc.workspaceBytes);
+      ref(ws, t0);
+      ref(ws, t1);
+      st_[ws].uses.clear();
+    }
+    int64_t bytes = 0;
+    for (auto* l : fc.leaves) bytes += (int64_t)l->type.bytes();
+    for (auto* o : outs) bytes += (int64_t)o->type.bytes();
+    for (auto& l : fc.launches) {
+      int t = ++time_;
+      Step s;
+      s.kind = Step::Kernel;
+      s.label = label;
+      s.kernel = kernelId(l.source);
+      for (int d = 0; d < 3; ++d) { s.grid[d] = l.grid[d]; s.block[d] = l.block[d]; }
+      for (auto& a : l.args) {
+        if (a.kind == KArg::Work) {
+          BufRef r = ref(ws, t);
+          r.offset = a.workOffset;   // added to the storage offset when patched
+          s.args.push_back(r);
+        } else {
+          s.args.push_back(ref(storageOf(a.value), t));
+        }
+      }
+      s.algoBytes = bytes;
+      plan.steps.push_back(std::move(s));
+    }
+  }
+
+  // constant scalar value of an i32/i64/etc. value if it is a compile-time constant
+  static bool constInt(Value* v, int64_t& out) {
+    Op* d = v->def;
+    while (d && (d->name == "reshape" || d->name == "convert" || d->name == "broadcast_in_dim") && d->operands[0]->type.numel() == 1) d = d->operands[0]->def;
+    if (!d || d->name != "constant") return false;
+    auto& dd = *d->attrs.at("value").dense;
+    if (!isInt(dd.type.dt) || dd.type.numel() != 1) return false;
+    int64_t x = 0;
+    size_t sz = dtypeSize(dd.type.dt);
+    memcpy(&x, dd.bytes.data(), sz);
+    if (isSignedInt(dd.type.dt) && sz < 8 && ((x >> (8 * sz - 1)) & 1)) x |= ~((int64_t(1) << (8 * sz)) - 1);
+    out = x;
+    return true;
+  }
+
+  void emitRegion(Region& r, Plan& plan) {
+    for (auto& opPtr : r.ops) {
+      Op* op = opPtr.get();
+      if (emitted_.count(op)) continue;
+      const std::string& n = op->name;
+      if (n == "return") continue;
+      if (isFusibleOp(*op) && op->results.size() == 1) {
+        Value* v = op->result();
+        if (!needMat_[v]) continue;
+        emitMaterialized(op, plan);
+        continue;
+      }
+      if (isPassThrough(*op)) {   // multi-result barrier: results alias operands
+        for (size_t k = 0; k < op->results.size(); ++k) {
+          Value* o = op->operands[k];
+          if (!hasStorage(o)) materializeNow(o, plan);
+          bind(op->results[k].get(), storageOf(o));
+        }
+        continue;
+      }
+      if (n == "reduce") { emitReduce(op, r, plan); continue; }
+      if (n == "dot_general" || n == "dot") { emitDot(op, plan); continue; }
+      if (n == "convolution") { emitConv(op, plan); continue; }
+      if (n == "scatter") { emitScatter(op, plan); continue; }
+      if (n == "dynamic_update_slice") { emitDus(op, plan); continue; }
+      if (n == "while") { emitWhile(op, plan); continue; }
+      if (n == "case") { emitCase(op, plan); continue; }
+      throw CompileError("no lowering for stablehlo." + n);
+    }
+  }
+
+  // a value that analysis left fused but some consumer needs in memory after all
+  void materializeNow(Value* v, Plan& plan) {
+    if (hasStorage(v)) return;
+    if (!v->def || !isFusibleOp(*v->def)) throw CompileError("internal: cannot materialise " + v->name);
+    emitMaterialized(v->def, plan);
+  }
+
+  void emitMaterialized(Op* op, Plan& plan) {
+    Value* v = op->result();
+    if (hasStorage(v)) return;
+    const std::string& n = op->name;
+    if (n == "constant") {
+      auto& d = *op->attrs.at("value").dense;
+      if (!d.splat || d.type.numel() == 1) {
+        int64_t off = ((int64_t)P.constPool.size() + kAlign - 1) / kAlign * kAlign;
+        P.constPool.resize((size_t)off + std::max<size_t>(d.bytes.size(), 4));
+        memcpy(P.constPool.data() + off, d.bytes.data(), d.bytes.size());
+        int sid = newStorage(d.bytes.size(), BufRef::Const);
+        st_[sid].offset = off;
+        bind(v, sid);
+        return;
+      }
+    }
+    if ((n == "reshape" || isPassThrough(*op) || (n == "convert" && op->operands[0]->type.dt == v->type.dt)) && hasStorage(op->operands[0])) {
+      bind(v, storageOf(op->operands[0]));
+      return;
+    }
+    if (v->type.numel() == 0) {
+      bind(v, newStorage(4));
+      return;
+    }
+    FusedCode fc = generateLoopKernel(v, leafPred());
+    int sid = newStorage(v->type.bytes());
+    bind(v, sid);
+    addFused(plan, fc, "fusion:" + n, {v});
+  }
+
+  void collectLeavesOf(Value* v, std::vector<Value*>& out, std::unordered_set<Value*>& seen) {
+    if (!seen.insert(v).second) return;
+    if (hasStorage(v)) { out.push_back(v); return; }
+    if (!v->def || !isFusibleOp(*v->def) || needMat_[v]) { out.push_back(v); return; }
+    for (auto* o : v->def->operands) collectLeavesOf(o, out, seen);
+  }
+
+  void emitReduce(Op* op, Region& r, Plan& plan) {
+    if (!isSimpleReduce(*op)) throw CompileError("stablehlo.reduce with a variadic or non-trivial reducer body is not supported");
+    std::vector<Op*> group{op};
+    std::vector<Value*> myLeaves;
+    {
+      std::unordered_set<Value*> seen;
+      collectLeavesOf(op->operands[0], myLeaves, seen);
+    }
+    // sibling reductions over the same index space that share an input: one pass over memory
+    bool seenSelf = false;
+    for (auto& qp : r.ops) {
+      Op* q = qp.get();
+      if (q == op) { seenSelf = true; continue; }
+      if (!seenSelf || group.size() >= 4) continue;
+      if (q->name != "reduce" || emitted_.count(q) || !isSimpleReduce(*q)) continue;
+      if (q->operands[0]->type.dims != op->operands[0]->type.dims) continue;
+      auto a = q->ints("dimensions"), b = op->ints("dimensions");
+      std::sort(a.begin(), a.end());
+      std::sort(b.begin(), b.end());
+      if (a != b) continue;
+      std::vector<Value*> ql;
+      std::unordered_set<Value*> seen;
+      collectLeavesOf(q->operands[0], ql, seen);
+      collectLeavesOf(q->operands[1], ql, seen);
+      bool ready = true, shares = false;
+      for (auto* l : ql) {
+        if (!hasStorage(l)) ready = false;
+        if (std::find(myLeaves.begin(), myLeaves.end(), l) != myLeaves.end() && l->type.numel() > kSmallNumel) shares = true;
+      }
+      if (ready && shares) group.push_back(q);
+    }
+    for (auto* g : group) {
+      // the init value must be readable
+      std::vector<Value*> il;
+      std::unordered_set<Value*> seen;
+      collectLeavesOf(g->operands[1], il, seen);
+      for (auto* l : il) if (!hasStorage(l)) materializeNow(l, plan);
+    }
+    if (op->result()->type.numel() == 0) {
+      for (auto* g : group) { bind(g->result(), newStorage(4)); emitted_.insert(g); }
+      return;
+    }
+    if (op->operands[0]->type.numel() == 0) {
+      // reducing nothing: the result is the init value broadcast
+      throw CompileError("stablehlo.reduce over an empty tensor is not supported");
+    }
+    FusedCode fc = generateReduceKernel(group, leafPred());
+    std::vector<Value*> outs;
+    for (auto* g : group) {
+      bind(g->result(), newStorage(g->result()->type.bytes()));
+      outs.push_back(g->result());
+      emitted_.insert(g);
+    }
+    addFused(plan, fc, group.size() > 1 ? "reduce x" + std::to_string(group.size()) : "reduce", outs);
+  }
+
+  static std::vector<int64_t> stridesOf(const TensorType& t) {
+    std::vector<int64_t> s(t.rank(), 1);
+    for (int d = t.rank() - 2; d >= 0; --d) s[d] = s[d + 1] * t.dims[d + 1];
+    return s;
+  }
+
+  // merge an ordered list of dims into (size, stride); false if they do not collapse
+  static bool mergeDims(const TensorType& t, const std::vector<int64_t>& dims, int64_t& size, int64_t& stride) {
+    auto st = stridesOf(t);
+    size = 1;
+    stride = 0;
+    bool have = false;
+    int64_t expect = 0;
+    for (size_t k = 0; k < dims.size(); ++k) {
+      int64_t d = dims[k];
+      if (t.dims[d] == 1) continue;
+      if (!have) { have = true; size = t.dims[d]; stride = st[d]; expect = st[d]; continue; }
+      // dims are listed outer to inner: the next one must tile the previous stride exactly
+      if (st[d] * t.dims[d] != expect) return false;
+      size *= t.dims[d];
+      stride = st[d];
+      expect = st[d];
+    }
+    if (!have) stride = 1;
+    return true;
+  }
+
+  void emitDot(Op* op, Plan& plan) {
+    Value* a = op->operands[0];
+    Value* b = op->operands[1];
+    Value* c = op->result();
+    std::vector<int64_t> ab = op->ints("lhs_batch"), bb = op->ints("rhs_batch"), ac = op->ints("lhs_contract"), bc = op->ints("rhs_contract");
+    if (op->name == "dot") { ac = {a->type.rank() - 1}; bc = {0}; }
+    auto has = [](const std::vector<int64_t>& v, int64_t x) { return std::find(v.begin(), v.end(), x) != v.end(); };
+    std::vector<int64_t> af, bf;
+    for (int d = 0; d < a->type.rank(); ++d) if (!has(ab, d) && !has(ac, d)) af.push_back(d);
+    for (int d = 0; d < b->type.rank(); ++d) if (!has(bb, d) && !has(bc, d)) bf.push_back(d);
+    if (!isFloat(a->type.dt) || a->type.dt == DType::F64 || a->type.dt == DType::F16)
+      throw CompileError("dot_general: only f32 and bf16 operands are supported");
+    for (Value* v : {a, b}) if (!hasStorage(v)) materializeNow(v, plan);
+    GemmDesc g;
+    g.inType = a->type.dt;
+    g.outType = c->type.dt;
+    // contraction dims: order both sides by the lhs stride so each side collapses when it can
+    std::vector<size_t> order(ac.size());
+    for (size_t k = 0; k < order.size(); ++k) order[k] = k;
+    auto ast = stridesOf(a->type);
+    std::sort(order.begin(), order.end(), [&](size_t x, size_t y) { return ast[ac[x]] > ast[ac[y]]; });
+    std::vector<int64_t> acs, bcs;
+    for (auto k : order) { acs.push_back(ac[k]); bcs.push_back(bc[k]); }
+    int64_t Ka, Kb, M, N;
+    bool ok = mergeDims(a->type, acs, Ka, g.aCol) && mergeDims(b->type, bcs, Kb, g.bRow) &&
+              mergeDims(a->type, af, M, g.aRow) && mergeDims(b->type, bf, N, g.bCol);
+    g.M = M; g.N = N; g.K = Ka;
+    // batch dims: up to two independent strides per operand
+    std::vector<int64_t> bsz;
+    std::vector<int64_t> abst, bbst;
+    auto bstr = stridesOf(b->type);
+    for (size_t k = 0; k < ab.size(); ++k) {
+      if (a->type.dims[ab[k]] == 1) continue;
+      if (!bsz.empty() && ast[ab[k]] * a->type.dims[ab[k]] == abst.back() && bstr[bb[k]] * b->type.dims[bb[k]] == bbst.back()) {
+        bsz.back() *= a->type.dims[ab[k]];
+        abst.back() = ast[ab[k]];
+        bbst.back() = bstr[bb[k]];
+      } else {
+        bsz.push_back(a->type.dims[ab[k]]);
+        abst.push_back(ast[ab[k]]);
+        bbst.push_back(bstr[bb[k]]);
+      }
+    }
+    if (!ok || bsz.size() > 2 || Ka != Kb)
+      throw CompileError("dot_general: operand layout needs a transposed copy (dims do not collapse to strided 2-D); not supported yet: " + a->type.str() + " x " + b->type.str());
+    if (bsz.size() >= 1) { g.batch0 = bsz[0]; g.aB0 = abst[0]; g.bB0 = bbst[0]; }
+    if (bsz.size() == 2) { g.batch1 = bsz[1]; g.aB1 = abst[1]; g.bB1 = bbst[1]; }
+    int sid = newStorage(c->type.bytes());
+    bind(c, sid);
+    if (c->type.numel() == 0) return;
+    int t = ++time_;
+    Step s;
+    s.kind = Step::Gemm;
+    s.label = "dot_general " + a->type.str() + " x " + b->type.str();
+    s.gemm = g;
+    s.args = {ref(storageOf(a), t), ref(storageOf(b), t), ref(sid, t)};
+    plan.steps.push_back(std::move(s));
+  }
+
+  void emitConv(Op* op, Plan& plan) {
+    Value* lhs = op->operands[0];
+    Value* rhs = op->operands[1];
+    Value* out = op->result();
+    for (Value* v : {lhs, rhs}) if (!hasStorage(v)) materializeNow(v, plan);
+    const ConvDims& cd = op->convDims;
+    int nsp = (int)cd.lhsSpatial.size();
+    if (nsp > 3) throw CompileError("convolution with more than 3 spatial dims is not supported");
+    if (lhs->type.dt != DType::F32 && lhs->type.dt != DType::BF16) throw CompileError("convolution: only f32 and bf16 are supported");
+    ConvDesc c;
+    c.nsp = nsp;
+    c.type = lhs->type.dt;
+    c.featureGroups = op->integer("feature_group_count", 1);
+    c.batchGroups = op->integer("batch_group_count", 1);
+    auto ls = stridesOf(lhs->type), rs = stridesOf(rhs->type), os = stridesOf(out->type);
+    c.N = lhs->type.dims[cd.lhsBatch] / c.batchGroups;
+    c.C = lhs->type.dims[cd.lhsFeature];
+    c.O = rhs->type.dims[cd.rhsOut];
+    c.lhsB = ls[cd.lhsBatch]; c.lhsF = ls[cd.lhsFeature];
+    c.rhsI = rs[cd.rhsIn]; c.rhsO = rs[cd.rhsOut];
+    c.outB = os[cd.outBatch]; c.outF = os[cd.outFeature];
+    auto& stride = op->ints("stride");
+    auto& pad = op->ints("pad");
+    auto& ld = op->ints("lhs_dilate");
+    auto& rd = op->ints("rhs_dilate");
+    auto& rev = op->ints("reverse");
+    for (int d = 0; d < nsp; ++d) {
+      c.in[d] = lhs->type.dims[cd.lhsSpatial[d]];
+      c.k[d] = rhs->type.dims[cd.rhsSpatial[d]];
+      c.out[d] = out->type.dims[cd.outSpatial[d]];
+      c.lhsS[d] = ls[cd.lhsSpatial[d]];
+      c.rhsS[d] = rs[cd.rhsSpatial[d]];
+      c.outS[d] = os[cd.outSpatial[d]];
+      c.stride[d] = stride.empty() ? 1 : stride[d];
+      c.padLo[d] = pad.empty() ? 0 : pad[2 * d];
+      c.ldil[d] = ld.empty() ? 1 : ld[d];
+      c.rdil[d] = rd.empty() ? 1 : rd[d];
+      c.rev[d] = rev.empty() ? 0 : rev[d];
+    }
+    int sid = newStorage(out->type.bytes());
+    bind(out, sid);
+    if (out->type.numel() == 0) return;
+    int t = ++time_;
+    Step s;
+    s.kind = Step::Conv;
+    s.label = "convolution " + lhs->type.str() + " * " + rhs->type.str();
+    s.conv = c;
+    // split-K workspace for shapes with few output tiles (filter gradients)
+    int64_t ws = 0;
+    s.workspaceBytes = ws;
+    s.args = {ref(storageOf(lhs), t), ref(storageOf(rhs), t), ref(sid, t)};
+    plan.steps.push_back(std::move(s));
+  }
+
+  void emitScatter(Op* op, Plan& plan) {
+    if (op->operands.size() != 3) throw CompileError("variadic scatter is not supported");
+    Value* operand = op->operands[0];
+    Value* idx = op->operands[1];
+    Value* upd = op->operands[2];
+    Value* res = op->result();
+    for (Value* v : {operand, idx, upd}) if (!hasStorage(v)) materializeNow(v, plan);
+    auto& uwd = op->ints("update_window_dims");
+    auto& iwd = op->ints("inserted_window_dims");
+    auto& sdo = op->ints("scatter_dims_to_operand_dims");
+    int64_t ivd = op->integer("index_vector_dim");
+    // row scatter: one index per update row, whole rows of the operand's leading dim
+    bool rows = operand->type.rank() >= 1 && iwd == std::vector<int64_t>{0} && sdo == std::vector<int64_t>{0} &&
+                op->ints("input_batching_dims").empty();
+    int64_t nUpd = 1;
+    if (rows) {
+      // scatter dims of updates must be the leading dims, window dims the trailing ones covering the full row
+      int nScatter = upd->type.rank() - (int)uwd.size();
+      for (size_t k = 0; k < uwd.size(); ++k) if (uwd[k] != nScatter + (int64_t)k) rows = false;
+      if ((int)uwd.size() != operand->type.rank() - 1) rows = false;
+      for (size_t k = 0; rows && k < uwd.size(); ++k) if (upd->type.dims[uwd[k]] != operand->type.dims[1 + k]) rows = false;
+      for (int d = 0; rows && d < nScatter; ++d) nUpd *= upd->type.dims[d];
+      int64_t nIdx = idx->type.numel();
+      if (ivd < idx->type.rank() && idx->type.dims[ivd] != 1) rows = false;
+      if (nIdx != nUpd) rows = false;
+    }
+    const char* kind = nullptr;
+    {
+      auto& r = *op->regions.at(0);
+      if (r.ops.size() == 1 && r.ops[0]->operands.size() == 1 && r.ops[0]->operands[0] == r.args[1].get()) kind = "set";
+      else if (r.ops.size() == 2 && r.ops[0]->operands.size() == 2) {
+        Op* b = r.ops[0].get();
+        bool both = (b->operands[0] == r.args[0].get() && b->operands[1] == r.args[1].get()) ||
+                    (b->operands[1] == r.args[0].get() && b->operands[0] == r.args[1].get());
+        if (both && r.ops[1]->operands[0] == b->result()) {
+          if (b->name == "add") kind = "add";
+          else if (b->name == "multiply") kind = "mul";
+          else if (b->name == "minimum") kind = "min";
+          else if (b->name == "maximum") kind = "max";
+        }
+      }
+    }
+    if (!rows || !kind) throw CompileError("stablehlo.scatter: only whole-row scatter along dim 0 with add/set/mul/min/max bodies is supported");
+    if (res->type.dt != DType::F32 && res->type.dt != DType::S32 && res->type.dt != DType::U32 && res->type.dt != DType::BF16)
+      throw CompileError("stablehlo.scatter: element type not supported");
+    if (idx->type.dt != DType::S32 && idx->type.dt != DType::S64 && idx->type.dt != DType::U32) throw CompileError("stablehlo.scatter: index type not supported");
+    // result storage: reuse the operand's buffer when nothing else reads it
+    int osid = storageOf(operand);
+    int sid;
+    int t = ++time_;
+    bool inPlace = st_[osid].kind == BufRef::Temp && st_[osid].values == 1 && operand->users.size() == 1 && !boundToOutput_.count(osid);
+    if (inPlace) {
+      sid = osid;
+    } else {
+      sid = newStorage(res->type.bytes());
+      Step c;
+      c.kind = Step::Copy;
+      c.label = "scatter operand copy";
+      c.src = ref(osid, t);
+      c.dst = ref(sid, t);
+      c.bytes = (int64_t)res->type.bytes();
+      plan.steps.push_back(std::move(c));
+      t = ++time_;
+    }
+    bind(res, sid);
+    if (nUpd == 0) return;
+    Step s;
+    s.kind = Step::ScatterRows;
+    s.label = std::string("scatter-") + kind + " rows";
+    s.scatter.numUpdates = nUpd;
+    s.scatter.operandRows = operand->type.dims[0];
+    s.scatter.rowElems = operand->type.numel() / std::max<int64_t>(1, operand->type.dims[0]);
+    s.scatter.kind = std::string(kind) == "add" ? 0 : std::string(kind) == "set" ? 1 : std::string(kind) == "mul" ? 2 : std::string(kind) == "min" ? 3 : 4;
+    s.scatter.type = res->type.dt;
+    s.scatter.indexType = idx->type.dt;
+    // workspace: sorted keys, permutation, segment heads (4 arrays of numUpdates 4-byte words, double-buffered sort)
+    int64_t wsBytes = ((nUpd * 4 * 6 + 1024) + kAlign - 1) / kAlign * kAlign;
+    int ws = newStorage((size_t)wsBytes);
+    s.workspaceBytes = wsBytes;
+    s.args = {ref(sid, t), ref(storageOf(idx), t), ref(storageOf(upd), t), ref(ws, t)};
+    plan.steps.push_back(std::move(s));
+  }
+
+  void emitDus(Op* op, Plan& plan) {
+    Value* operand = op->operands[0];
+    Value* res = op->result();
+    if (!hasStorage(operand)) materializeNow(operand, plan);
+    int osid = storageOf(operand);
+    // in place when every other reader of the operand buffer has already been issued
+    bool inPlace = st_[osid].kind == BufRef::Temp && !boundToOutput_.count(osid);
+    if (inPlace) {
+      for (Op* u : operand->users) {
+        if (u == op) continue;
+        if (u->parent != op->parent) { inPlace = false; break; }
+        bool before = false;
+        for (auto& q : op->parent->ops) {
+          if (q.get() == u) { before = true; break; }
+          if (q.get() == op) break;
+        }
+        // a fused reader may be inlined into a kernel issued later
+        bool issuesItself = !isFusibleOp(*u) || needMat_[u->result()];
+        if (!before || !issuesItself) { inPlace = false; break; }
+      }
+      if (st_[osid].values > 1 && !operand->argOf) inPlace = false;
+    }
+    int sid = osid;
+    if (!inPlace) {
+      sid = newStorage(res->type.bytes());
+      int t = ++time_;
+      Step c;
+      c.kind = Step::Copy;
+      c.label = "dynamic_update_slice operand copy";
+      c.src = ref(osid, t);
+      c.dst = ref(sid, t);
+      c.bytes = (int64_t)res->type.bytes();
+      plan.steps.push_back(std::move(c));
+    }
+    bind(res, sid);
+    if (op->operands[1]->type.numel() == 0) return;
+    FusedCode fc = generateDusKernel(op, leafPred());
+    addFused(plan, fc, "dynamic_update_slice", {op->operands[1]});
+  }
+
+  // counted loop: cond is `carry_i <cmp> const`, body returns carry_i + const, init is a constant
+  int64_t detectTripCount(Op* op) {
+    Region& cond = *op->regions[0];
+    Region& body = *op->regions[1];
+    Op* ret = cond.terminator();
+    if (!ret || ret->operands.size() != 1) return -1;
+    Op* cmp = ret->operands[0]->def;
+    if (!cmp || cmp->name != "compare") return -1;
+    Value* lhs = cmp->operands[0];
+    Value* rhs = cmp->operands[1];
+    std::string dir = cmp->str("direction");
+    int64_t limit;
+    if (!(lhs->argOf == &cond) || !constInt(rhs, limit)) {
+      if (rhs->argOf == &cond && constInt(lhs, limit)) {
+        std::swap(lhs, rhs);
+        dir = dir == "LT" ? "GT" : dir == "GT" ? "LT" : dir == "LE" ? "GE" : dir == "GE" ? "LE" : dir;
+      } else {
+        return -1;
+      }
+    }
+    int ci = lhs->defIndex;
+    int64_t init;
+    if (!constInt(op->operands[ci], init)) return -1;
+    Value* next = body.terminator()->operands[ci];
+    Op* add = next->def;
+    if (!add || (add->name != "add" && add->name != "subtract")) return -1;
+    int64_t step;
+    Value* barg = body.args[ci].get();
+    if (add->operands[0] == barg && constInt(add->operands[1], step)) {
+      if (add->name == "subtract") step = -step;
+    } else if (add->name == "add" && add->operands[1] == barg && constInt(add->operands[0], step)) {
+    } else {
+      return -1;
+    }
+    if (step == 0) return -1;
+    int64_t n = 0;
+    if (dir == "LT" && step > 0) n = limit > init ? (limit - init + step - 1) / step : 0;
+    else if (dir == "LE" && step > 0) n = limit >= init ? (limit - init) / step + 1 : 0;
+    else if (dir == "GT" && step < 0) n = init > limit ? (init - limit + (-step) - 1) / (-step) : 0;
+    else if (dir == "GE" && step < 0) n = init >= limit ? (init - limit) / (-step) + 1 : 0;
+    else if (dir == "NE" && (limit - init) % step == 0 && (limit - init) / step >= 0) n = (limit - init) / step;
+    else return -1;
+    return n;
+  }
+
+  void copyStep(Plan& plan, int src, int dst, int64_t bytes, const char* label) {
+    if (src == dst) return;
+    int t = ++time_;
+    Step c;
+    c.kind = Step::Copy;
+    c.label = label;
+    c.src = ref(src, t);
+    c.dst = ref(dst, t);
+    c.bytes = bytes;
+    plan.steps.push_back(std::move(c));
+  }
+
+  void emitWhile(Op* op, Plan& plan) {
+    size_t n = op->operands.size();
+    for (auto* v : op->operands) if (!hasStorage(v)) materializeNow(v, plan);
+    int64_t trip = detectTripCount(op);
+    std::vector<int> slots(n);
+    for (size_t i = 0; i < n; ++i) {
+      Value* v = op->operands[i];
+      int osid = storageOf(v);
+      bool reuse = st_[osid].kind == BufRef::Temp && st_[osid].values == 1 && v->users.size() == 1 && !boundToOutput_.count(osid);
+      if (reuse) slots[i] = osid;
+      else {
+        slots[i] = newStorage(v->type.bytes());
+        copyStep(plan, osid, slots[i], (int64_t)v->type.bytes(), "loop carry init");
+      }
+    }
+    int tStart = ++time_;
+    for (size_t i = 0; i < n; ++i) ref(slots[i], tStart);
+    Step w;
+    w.kind = Step::While;
+    w.label = "while";
+    w.tripCount = trip;
+    Region& cond = *op->regions[0];
+    Region& body = *op->regions[1];
+    for (size_t i = 0; i < n; ++i) { bind(cond.args[i].get(), slots[i]); bind(body.args[i].get(), slots[i]); }
+    analyze(cond);
+    analyze(body);
+    w.cond = std::make_unique<Plan>();
+    emitRegion(cond, *w.cond);
+    Value* pred = cond.terminator()->operands.at(0);
+    if (!hasStorage(pred)) materializeNow(pred, *w.cond);
+    w.predBuf = ref(storageOf(pred), ++time_);
+    auto bodyPlan = std::make_unique<Plan>();
+    emitRegion(body, *bodyPlan);
+    Op* ret = body.terminator();
+    if (ret->operands.size() != n) throw CompileError("while: body returns the wrong number of values");
+    std::vector<int> src(n);
+    for (size_t i = 0; i < n; ++i) {
+      Value* v = ret->operands[i];
+      if (!hasStorage(v)) materializeNow(v, *bodyPlan);
+      src[i] = storageOf(v);
+    }
+    // phase 1: values that live in another carry slot are staged through temporaries
+    for (size_t i = 0; i < n; ++i) {
+      if (src[i] == slots[i]) continue;
+      bool isSlot = std::find(slots.begin(), slots.end(), src[i]) != slots.end();
+      if (isSlot || st_[src[i]].kind != BufRef::Temp) {
+        int tmp = newStorage(op->operands[i]->type.bytes());
+        copyStep(*bodyPlan, src[i], tmp, (int64_t)op->operands[i]->type.bytes(), "loop carry stage");
+        src[i] = tmp;
+      }
+    }
+    for (size_t i = 0; i < n; ++i) copyStep(*bodyPlan, src[i], slots[i], (int64_t)op->operands[i]->type.bytes(), "loop carry update");
+    int tEnd = ++time_;
+    for (size_t i = 0; i < n; ++i) ref(slots[i], tEnd);
+    loops_.push_back({tStart, tEnd});
+    w.bodies.push_back(std::move(bodyPlan));
+    for (size_t i = 0; i < n; ++i) bind(op->results[i].get(), slots[i]);
+    plan.steps.push_back(std::move(w));
+  }
+
+  void emitCase(Op* op, Plan& plan) {
+    Value* index = op->operands[0];
+    if (!hasStorage(index)) materializeNow(index, plan);
+    int tStart = ++time_;
+    Step c;
+    c.kind = Step::Case;
+    c.label = "case";
+    c.predBuf = ref(storageOf(index), tStart);
+    c.predType = index->type.dt;
+    std::vector<int> outs;
+    for (auto& r : op->results) outs.push_back(newStorage(r->type.bytes()));
+    for (auto& rg : op->regions) {
+      analyze(*rg);
+      auto bp = std::make_unique<Plan>();
+      emitRegion(*rg, *bp);
+      Op* ret = rg->terminator();
+      for (size_t k = 0; k < op->results.size(); ++k) {
+        Value* v = ret->operands.at(k);
+        if (!hasStorage(v)) materializeNow(v, *bp);
+        copyStep(*bp, storageOf(v), outs[k], (int64_t)v->type.bytes(), "case result");
+      }
+      c.bodies.push_back(std::move(bp));
+    }
+    int tEnd = ++time_;
+    for (auto o : outs) { ref(o, tStart); ref(o, tEnd); }
+    loops_.push_back({tStart, tEnd});
+    for (size_t k = 0; k < op->results.size(); ++k) bind(op->results[k].get(), outs[k]);
+    plan.steps.push_back(std::move(c));
+  }
+
+  // ---------------------------------------------------------------- arena
+  void assignArena() {
+    // a buffer that is used inside a loop but defined outside it lives until the loop ends
+    for (auto& s : st_) {
+      if (s.kind != BufRef::Temp || s.first < 0) continue;
+      for (int u : s.uses) {
+        for (auto& lp : loops_) {
+          if (u > lp.first && u < lp.second && !(s.first > lp.first && s.first < lp.second)) s.last = std::max(s.last, lp.second);
+        }
+      }
+      for (auto& lp : loops_) if (s.last > lp.first && s.last < lp.second && !(s.first > lp.first)) s.last = std::max(s.last, lp.second);
+    }
+    std::vector<int> order;
+    for (int i = 0; i < (int)st_.size(); ++i) if (st_[i].kind == BufRef::Temp && st_[i].first >= 0) order.push_back(i);
+    std::sort(order.begin(), order.end(), [&](int a, int b) { return st_[a].first != st_[b].first ? st_[a].first < st_[b].first : st_[a].bytes > st_[b].bytes; });
+    struct Live { int64_t off, size; int last; };
+    std::vector<Live> live;
+    int64_t peak = 0;
+    for (int id : order) {
+      Storage& s = st_[id];
+      live.erase(std::remove_if(live.begin(), live.end(), [&](const Live& l) { return l.last < s.first; }), live.end());
+      std::sort(live.begin(), live.end(), [](const Live& a, const Live& b) { return a.off < b.off; });
+      int64_t size = (s.bytes + kAlign - 1) / kAlign * kAlign;
+      int64_t off = 0;
+      for (auto& l : live) {
+        if (off + size <= l.off) break;
+        off = std::max(off, l.off + l.size);
+      }
+      s.offset = off;
+      live.push_back({off, size, s.last});
+      peak = std::max(peak, off + size);
+    }
+    P.arenaBytes = peak;
+  }
+
+  BufRef finalRef(const BufRef& r) {
+    if (r.kind == BufRef::None) return r;
+    const Storage& s = st_[r.index];
+    BufRef o;
+    o.kind = s.kind;
+    if (s.kind == BufRef::Param || s.kind == BufRef::Output) { o.index = s.index; o.offset = r.offset; }
+    else { o.index = 0; o.offset = s.offset + r.offset; }
+    return o;
+  }
+
+  void patch(Plan& plan) {
+    for (auto& s : plan.steps) {
+      for (auto& a : s.args) a = finalRef(a);
+      s.src = finalRef(s.src);
+      s.dst = finalRef(s.dst);
+      s.predBuf = finalRef(s.predBuf);
+      if (s.cond) patch(*s.cond);
+      for (auto& b : s.bodies) patch(*b);
+    }
+  }
+
+  static int countSteps(const Plan& p) {
+    int n = 0;
+    for (auto& s : p.steps) {
+      ++n;
+      if (s.cond) n += countSteps(*s.cond);
+      for (auto& b : s.bodies) n += countSteps(*b);
+    }
+    return n;
+  }
+
+  void dumpPlan(const Plan& p, int indent) {
+    std::ostringstream o;
+    static const char* kinds[] = {"kernel", "gemm", "conv", "scatter", "copy", "fill", "while", "case"};
+    for (auto& s : p.steps) {
+      o << std::string(indent, ' ') << kinds[s.kind] << " " << s.label;
+      if (s.kind == Step::Kernel) o << " k" << s.kernel << " grid " << s.grid[0] << "x" << s.grid[1] << " bytes " << s.algoBytes;
+      if (s.kind == Step::While) o << " trip " << s.tripCount;
+      o << "\n";
+      P.dump += o.str();
+      o.str("");
+      if (s.cond) dumpPlan(*s.cond, indent + 2);
+      for (auto& b : s.bodies) dumpPlan(*b, indent + 2);
+    }
+  }
+};
+
+}  // namespace
+
+std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) {
+  auto prog = std::make_unique<CompiledProgram>();
+  inlineCalls(*module);
+  checkSupported(*module);
+  eliminateDeadCode(module->main()->body);
+  prog->module = std::move(module);
+  Planner planner(*prog);
+  planner.run();
+  return prog;
+}
+
+}  // namespace mi355

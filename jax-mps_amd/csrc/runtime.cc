@@ -1,0 +1,476 @@
+// Device singleton, caching allocator, kernel cache, and the plan executor.
+#include "runtime.h"
+
+#include <dlfcn.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <thread>
+
+namespace mi355 {
+
+namespace {
+
+void check(int rc, const char* what) {
+  if (rc != 0) throw RuntimeError(std::string(what) + " failed: " + mi355_last_error());
+}
+
+uint64_t fnv1a(const std::string& s, uint64_t seed) {
+  uint64_t h = seed;
+  for (unsigned char c : s) { h ^= c; h *= 1099511628211ull; }
+  return h;
+}
+
+std::string libraryDir() {
+  Dl_info info;
+  if (dladdr((void*)&fnv1a, &info) && info.dli_fname) {
+    std::string p = info.dli_fname;
+    auto k = p.rfind('/');
+    if (k != std::string::npos) return p.substr(0, k);
+  }
+  return ".";
+}
+
+// On-disk cache of code objects keyed by the kernel source.  Populated at build time
+// (cross-compilation needs no GPU) and at run time for kernels seen for the first time.
+std::string cacheDir() {
+  static std::string dir = [] {
+    const char* e = getenv("MI355X_KERNEL_CACHE_DIR");
+    std::string d = e ? std::string(e) : libraryDir() + "/kcache";
+    if (d == "off" || d.empty()) return std::string();
+    mkdir(d.c_str(), 0755);
+    return d;
+  }();
+  return dir;
+}
+
+std::string cachePath(const std::string& source, const std::string& arch) {
+  std::string d = cacheDir();
+  if (d.empty()) return "";
+  char name[80];
+  snprintf(name, sizeof name, "/%016llx%016llx.hsaco", (unsigned long long)fnv1a(source + arch, 14695981039346656037ull),
+           (unsigned long long)fnv1a(arch + source, 0x9E3779B97F4A7C15ull));
+  return d + name;
+}
+
+bool readFile(const std::string& path, std::vector<char>& out) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f) return false;
+  f.seekg(0, std::ios::end);
+  std::streamsize n = f.tellg();
+  if (n <= 0) return false;
+  f.seekg(0);
+  out.resize((size_t)n);
+  f.read(out.data(), n);
+  return (bool)f;
+}
+
+void writeFileAtomic(const std::string& path, const char* data, size_t n) {
+  std::string tmp = path + ".tmp" + std::to_string((long)getpid()) + "_" + std::to_string((unsigned long)(uintptr_t)data);
+  {
+    std::ofstream f(tmp, std::ios::binary);
+    if (!f) return;
+    f.write(data, (std::streamsize)n);
+    if (!f) { unlink(tmp.c_str()); return; }
+  }
+  if (rename(tmp.c_str(), path.c_str()) != 0) unlink(tmp.c_str());
+}
+
+std::string baseArch(const std::string& arch) {
+  auto k = arch.find(':');
+  return k == std::string::npos ? arch : arch.substr(0, k);
+}
+
+}  // namespace
+
+// Compiles every kernel source that is not cached on disk yet; returns the code objects.
+// Needs no GPU, so the build step can run it ahead of time.
+std::vector<std::vector<char>> compileKernelSources(const std::vector<const std::string*>& sources, const std::string& arch,
+                                                    int* fromDisk, int* compiled) {
+  size_t n = sources.size();
+  std::vector<std::vector<char>> code(n);
+  std::vector<std::string> errors(n);
+  std::atomic<size_t> next{0};
+  std::atomic<int> nDisk{0}, nComp{0};
+  unsigned hw = std::thread::hardware_concurrency();
+  unsigned workers = std::max(1u, std::min<unsigned>({hw ? hw : 4u, 16u, (unsigned)n}));
+  auto work = [&] {
+    while (true) {
+      size_t i = next.fetch_add(1);
+      if (i >= n) break;
+      std::string path = cachePath(*sources[i], arch);
+      if (!path.empty() && readFile(path, code[i])) { nDisk++; continue; }
+      char* buf = nullptr;
+      size_t sz = 0;
+      std::vector<char> log(1 << 14);
+      int rc = mi355_rtc_compile(sources[i]->c_str(), arch.c_str(), &buf, &sz, log.data(), log.size());
+      if (rc != 0) {
+        errors[i] = std::string("kernel compilation failed: ") + mi355_last_error();
+        if (getenv("MI355X_DUMP_KERNELS")) fprintf(stderr, "---- failing kernel ----\n%s\n", sources[i]->c_str());
+        continue;
+      }
+      code[i].assign(buf, buf + sz);
+      free(buf);
+      nComp++;
+      if (!path.empty()) writeFileAtomic(path, code[i].data(), code[i].size());
+    }
+  };
+  std::vector<std::thread> pool;
+  for (unsigned w = 1; w < workers; ++w) pool.emplace_back(work);
+  work();
+  for (auto& t : pool) t.join();
+  for (size_t i = 0; i < n; ++i)
+    if (!errors[i].empty()) throw RuntimeError(errors[i] + "\n---- source ----\n" + *sources[i]);
+  if (fromDisk) *fromDisk = nDisk;
+  if (compiled) *compiled = nComp;
+  return code;
+}
+
+// ---------------------------------------------------------------- Device
+bool Device::available(std::string* why) {
+  int n = 0;
+  if (mi355_device_count(&n) != 0 || n <= 0) {
+    if (why) *why = std::string("no HIP device: ") + mi355_last_error();
+    return false;
+  }
+  return true;
+}
+
+Device& Device::get() {
+  static Device* d = new Device();   // never destroyed: buffers may outlive static destruction order
+  return *d;
+}
+
+Device::Device() {
+  std::string why;
+  if (!available(&why)) throw RuntimeError("MI355X plugin: " + why + " (this plugin has no CPU fallback)");
+  char name[256], arch[256];
+  check(mi355_device_init(0, name, sizeof name, arch, sizeof arch, &cus_, &totalMem_), "device init");
+  name_ = name;
+  arch_ = arch;
+  if (baseArch(arch_) != "gfx950")
+    throw RuntimeError("MI355X plugin: device architecture is " + arch_ + "; the kernels of this library are built for gfx950 only");
+  check(mi355_stream_create(&stream_), "stream create");
+  check(mi355_host_alloc(&pinned_, 4096), "pinned alloc");
+}
+
+void* Device::alloc(size_t bytes) {
+  size_t sz = std::max<size_t>(256, (bytes + 255) / 256 * 256);
+  std::lock_guard<std::mutex> lk(mu_);
+  void* p = nullptr;
+  auto it = free_.lower_bound(sz);
+  // reuse a cached block if it is not wastefully large
+  if (it != free_.end() && it->first <= sz + sz / 4 + 4096) {
+    p = it->second;
+    sz = it->first;
+    free_.erase(it);
+  } else {
+    int rc = mi355_malloc(&p, sz);
+    if (rc != 0) {
+      // give cached blocks back and retry once
+      for (auto& kv : free_) { mi355_free(kv.second); sizes_.erase(kv.second); reserved_ -= (int64_t)kv.first; }
+      free_.clear();
+      check(mi355_malloc(&p, sz), "device allocation");
+    }
+    sizes_[p] = sz;
+    reserved_ += (int64_t)sz;
+  }
+  inUse_ += (int64_t)sz;
+  peak_ = std::max(peak_, inUse_);
+  numAllocs_++;
+  largest_ = std::max<int64_t>(largest_, (int64_t)sz);
+  return p;
+}
+
+void Device::release(void* ptr) {
+  if (!ptr) return;
+  std::lock_guard<std::mutex> lk(mu_);
+  auto it = sizes_.find(ptr);
+  if (it == sizes_.end()) return;
+  inUse_ -= (int64_t)it->second;
+  // All work is issued on one stream, so a recycled block is only touched by work that is
+  // ordered after everything that used it before.
+  free_.emplace(it->second, ptr);
+}
+
+void Device::sync() { check(mi355_stream_sync(stream_), "stream synchronize"); }
+
+mi355_function_t Device::findKernel(const std::string& source) {
+  std::lock_guard<std::mutex> lk(mu_);
+  auto it = kernels_.find(source);
+  return it == kernels_.end() ? nullptr : it->second;
+}
+void Device::storeKernel(const std::string& source, mi355_function_t fn) {
+  std::lock_guard<std::mutex> lk(mu_);
+  kernels_[source] = fn;
+}
+
+DeviceBuffer::~DeviceBuffer() {
+  if (ptr) Device::get().release(ptr);
+}
+
+// ------------------------------------------------------------- Executable
+Executable::Executable(std::unique_ptr<CompiledProgram> prog) : prog_(std::move(prog)) {
+  Device& dev = Device::get();
+  const char* t = getenv("MI355X_TIMING");
+  timingKinds_ = t ? t : "";
+  loadKernels();
+  if (prog_->arenaBytes > 0) arena_ = dev.alloc((size_t)prog_->arenaBytes);
+  if (!prog_->constPool.empty()) {
+    consts_ = dev.alloc(prog_->constPool.size());
+    check(mi355_memcpy_h2d(consts_, prog_->constPool.data(), prog_->constPool.size(), dev.stream()), "constant upload");
+    dev.sync();
+  }
+}
+
+Executable::~Executable() {
+  Device& dev = Device::get();
+  // the arena may still be in use by queued work
+  try { dev.sync(); } catch (...) {}
+  if (arena_) dev.release(arena_);
+  if (consts_) dev.release(consts_);
+  for (auto e : eventPool_) mi355_event_destroy(e);
+  for (auto& p : pending_) { mi355_event_destroy(p.a); mi355_event_destroy(p.b); }
+}
+
+void Executable::loadKernels() {
+  Device& dev = Device::get();
+  auto t0 = std::chrono::steady_clock::now();
+  std::vector<const std::string*> todo;
+  std::vector<size_t> idx;
+  for (size_t i = 0; i < prog_->kernels.size(); ++i) {
+    auto& k = prog_->kernels[i];
+    k.function = dev.findKernel(k.source);
+    if (!k.function) { todo.push_back(&k.source); idx.push_back(i); }
+  }
+  int fromDisk = 0, compiled = 0;
+  auto code = compileKernelSources(todo, baseArch(dev.arch()), &fromDisk, &compiled);
+  for (size_t q = 0; q < idx.size(); ++q) {
+    auto& k = prog_->kernels[idx[q]];
+    mi355_function_t fn = nullptr;
+    check(mi355_module_load(code[q].data(), &fn), "module load");
+    k.function = fn;
+    dev.storeKernel(k.source, fn);
+  }
+  compileSeconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+  if (getenv("MI355X_VERBOSE"))
+    fprintf(stderr, "[mi355x] %zu fused kernels (%d compiled, %d from disk cache, %zu shared) in %.2f s; %d steps, arena %.1f MiB\n",
+            prog_->kernels.size(), compiled, fromDisk, prog_->kernels.size() - idx.size(), compileSeconds, prog_->numSteps,
+            prog_->arenaBytes / 1048576.0);
+}
+
+void* Executable::resolve(const BufRef& r, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) const {
+  switch (r.kind) {
+    case BufRef::Param: return (char*)in[r.index]->ptr + r.offset;
+    case BufRef::Output: return (char*)out[r.index] + r.offset;
+    case BufRef::Temp: return (char*)arena_ + r.offset;
+    case BufRef::Const: return (char*)consts_ + r.offset;
+    default: return nullptr;
+  }
+}
+
+bool Executable::timed(const std::string& kind) const {
+  if (timingKinds_.empty()) return false;
+  if (timingKinds_ == "all" || timingKinds_ == "1") return true;
+  return ("," + timingKinds_ + ",").find("," + kind + ",") != std::string::npos;
+}
+
+mi355_event_t Executable::getEvent() {
+  if (!eventPool_.empty()) {
+    auto e = eventPool_.back();
+    eventPool_.pop_back();
+    return e;
+  }
+  mi355_event_t e;
+  check(mi355_event_create(&e, 1), "event create");
+  return e;
+}
+
+void Executable::resolvePending() {
+  if (pending_.empty()) return;
+  Device::get().sync();
+  for (auto& p : pending_) {
+    float ms = 0;
+    if (mi355_event_elapsed_ms(p.a, p.b, &ms) == 0) {
+      auto& s = stats_[p.kind];
+      s.count++;
+      s.ms += ms;
+      s.flops += p.flops;
+      s.bytes += p.bytes;
+    }
+    eventPool_.push_back(p.a);
+    eventPool_.push_back(p.b);
+  }
+  pending_.clear();
+}
+
+std::map<std::string, KindStat> Executable::timings() {
+  std::lock_guard<std::mutex> lk(mu_);
+  resolvePending();
+  return stats_;
+}
+
+static int dtypeCode(DType d) {
+  switch (d) {
+    case DType::F32: return 0;
+    case DType::BF16: return 1;
+    case DType::S32: return 2;
+    case DType::U32: return 3;
+    default: return -1;
+  }
+}
+
+void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
+  Device& dev = Device::get();
+  mi355_stream_t st = dev.stream();
+  std::string kind;
+  double flops = 0, bytes = 0;
+  switch (s.kind) {
+    case Step::Kernel: kind = s.label.rfind("reduce", 0) == 0 ? "reduce" : "fusion"; bytes = (double)s.algoBytes; break;
+    case Step::Gemm: kind = "gemm"; flops = 2.0 * s.gemm.batch0 * s.gemm.batch1 * s.gemm.M * s.gemm.N * s.gemm.K; break;
+    case Step::Conv: {
+      kind = "conv";
+      double macs = (double)s.conv.N * s.conv.O * (s.conv.C / s.conv.featureGroups);
+      for (int d = 0; d < s.conv.nsp; ++d) macs *= (double)s.conv.out[d] * s.conv.k[d];
+      flops = 2.0 * macs;
+      break;
+    }
+    case Step::ScatterRows: kind = "scatter"; bytes = (double)s.scatter.numUpdates * s.scatter.rowElems * 4; break;
+    case Step::Copy: kind = "copy"; bytes = 2.0 * s.bytes; break;
+    default: break;
+  }
+  bool doTime = !kind.empty() && timed(kind);
+  mi355_event_t ea = nullptr, eb = nullptr;
+  if (doTime) {
+    ea = getEvent();
+    eb = getEvent();
+    mi355_event_record(ea, st);
+  }
+  switch (s.kind) {
+    case Step::Kernel: {
+      void* ptrs[64];
+      void* argv[64];
+      size_t n = s.args.size();
+      if (n > 64) throw RuntimeError("fused kernel with more than 64 arguments");
+      for (size_t i = 0; i < n; ++i) { ptrs[i] = resolve(s.args[i], in, out); argv[i] = &ptrs[i]; }
+      check(mi355_launch((mi355_function_t)prog_->kernels[s.kernel].function, s.grid, s.block, argv, (int)n, st), s.label.c_str());
+      break;
+    }
+    case Step::Gemm: {
+      mi355_gemm_desc d;
+      const GemmDesc& g = s.gemm;
+      d.batch0 = g.batch0; d.batch1 = g.batch1; d.M = g.M; d.N = g.N; d.K = g.K;
+      d.aB0 = g.aB0; d.aB1 = g.aB1; d.aRow = g.aRow; d.aCol = g.aCol;
+      d.bB0 = g.bB0; d.bB1 = g.bB1; d.bRow = g.bRow; d.bCol = g.bCol;
+      d.in_dtype = dtypeCode(g.inType);
+      d.out_dtype = dtypeCode(g.outType);
+      check(mi355_gemm(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), st), "gemm");
+      break;
+    }
+    case Step::Conv: {
+      mi355_conv_desc d;
+      memset(&d, 0, sizeof d);
+      const ConvDesc& c = s.conv;
+      d.nsp = c.nsp; d.N = c.N; d.C = c.C; d.O = c.O;
+      for (int k = 0; k < 3; ++k) {
+        d.in[k] = c.in[k]; d.k[k] = c.k[k]; d.out[k] = c.out[k]; d.stride[k] = c.stride[k]; d.padLo[k] = c.padLo[k];
+        d.ldil[k] = c.ldil[k]; d.rdil[k] = c.rdil[k]; d.rev[k] = c.rev[k];
+        d.lhsS[k] = c.lhsS[k]; d.rhsS[k] = c.rhsS[k]; d.outS[k] = c.outS[k];
+      }
+      d.featureGroups = c.featureGroups; d.batchGroups = c.batchGroups;
+      d.lhsB = c.lhsB; d.lhsF = c.lhsF; d.rhsI = c.rhsI; d.rhsO = c.rhsO; d.outB = c.outB; d.outF = c.outF;
+      d.dtype = dtypeCode(c.type);
+      void* ws = s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
+      check(mi355_conv(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), ws,
+                       (size_t)s.workspaceBytes, st), "convolution");
+      break;
+    }
+    case Step::ScatterRows: {
+      mi355_scatter_desc d;
+      d.numUpdates = s.scatter.numUpdates; d.rowElems = s.scatter.rowElems; d.operandRows = s.scatter.operandRows;
+      d.kind = s.scatter.kind;
+      d.dtype = dtypeCode(s.scatter.type);
+      d.index_bytes = (int)dtypeSize(s.scatter.indexType);
+      check(mi355_scatter_rows(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out),
+                               resolve(s.args[3], in, out), st), "scatter");
+      break;
+    }
+    case Step::Copy:
+      check(mi355_copy(resolve(s.dst, in, out), resolve(s.src, in, out), (size_t)s.bytes, st), "copy");
+      break;
+    case Step::Fill: break;
+    case Step::While: {
+      if (s.tripCount >= 0) {
+        // counted loop: the trip count is known, iterations are queued back to back with no host round trip
+        for (int64_t i = 0; i < s.tripCount; ++i) runPlan(*s.bodies[0], in, out);
+      } else {
+        unsigned char* flag = (unsigned char*)dev.pinnedScratch();
+        while (true) {
+          runPlan(*s.cond, in, out);
+          check(mi355_memcpy_d2h(flag, resolve(s.predBuf, in, out), 1, st), "predicate read-back");
+          dev.sync();
+          if (!*flag) break;
+          runPlan(*s.bodies[0], in, out);
+        }
+      }
+      break;
+    }
+    case Step::Case: {
+      long long idx = 0;
+      size_t sz = dtypeSize(s.predType);
+      void* host = dev.pinnedScratch();
+      check(mi355_memcpy_d2h(host, resolve(s.predBuf, in, out), sz, st), "branch index read-back");
+      dev.sync();
+      if (s.predType == DType::Pred) idx = *(unsigned char*)host ? 1 : 0;
+      else if (sz == 4) idx = *(int*)host;
+      else if (sz == 8) idx = *(long long*)host;
+      else if (sz == 1) idx = *(signed char*)host;
+      else idx = *(short*)host;
+      long long nb = (long long)s.bodies.size();
+      // out-of-range selects the last branch (reference: ops/control_flow.cc:672-675)
+      if (idx < 0 || idx >= nb) idx = nb - 1;
+      runPlan(*s.bodies[(size_t)idx], in, out);
+      break;
+    }
+  }
+  if (doTime) {
+    mi355_event_record(eb, st);
+    pending_.push_back({ea, eb, kind, flops, bytes});
+    if (pending_.size() > 20000) resolvePending();
+  }
+}
+
+void Executable::runPlan(const Plan& plan, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
+  for (auto& s : plan.steps) runStep(s, in, out);
+}
+
+std::vector<std::shared_ptr<DeviceBuffer>> Executable::execute(const std::vector<DeviceBuffer*>& inputs) {
+  std::lock_guard<std::mutex> lk(mu_);
+  Device& dev = Device::get();
+  if (inputs.size() != prog_->paramTypes.size())
+    throw RuntimeError("execute: expected " + std::to_string(prog_->paramTypes.size()) + " arguments, got " + std::to_string(inputs.size()));
+  for (size_t i = 0; i < inputs.size(); ++i) {
+    if (!inputs[i] || inputs[i]->deleted || !inputs[i]->ptr) throw RuntimeError("execute: argument " + std::to_string(i) + " is null or deleted");
+    if (!(inputs[i]->type == prog_->paramTypes[i]))
+      throw RuntimeError("execute: argument " + std::to_string(i) + " has type " + inputs[i]->type.str() + ", executable expects " + prog_->paramTypes[i].str());
+  }
+  std::vector<std::shared_ptr<DeviceBuffer>> outs;
+  std::vector<void*> outPtrs;
+  for (auto& o : prog_->outputs) {
+    auto b = std::make_shared<DeviceBuffer>();
+    b->type = o.type;
+    b->ptr = dev.alloc(std::max<size_t>(o.type.bytes(), 4));
+    outPtrs.push_back(b->ptr);
+    outs.push_back(std::move(b));
+  }
+  runPlan(prog_->plan, inputs, outPtrs);
+  return outs;
+}
+
+}  // namespace mi355

@@ -1,0 +1,112 @@
+// Host runtime: device singleton with a caching allocator and one compute stream,
+// device buffers, and the executor that replays a compiled plan.  Replaces the
+// reference's MlxClient / MlxBuffer / MlxExecutable (src/pjrt_plugin/mlx_client.h:27-31,
+// mlx_buffer.h:46-84, mlx_executable.h:41-77).
+#pragma once
+
+#include <atomic>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "hip_abi.h"
+#include "plan.h"
+
+namespace mi355 {
+
+struct RuntimeError : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+
+class Device {
+ public:
+  static Device& get();            // throws RuntimeError when no GPU is usable
+  static bool available(std::string* why);
+
+  void* alloc(size_t bytes);       // stream-ordered reuse: blocks are recycled without waiting
+  void release(void* ptr);
+  mi355_stream_t stream() const { return stream_; }
+  const std::string& arch() const { return arch_; }
+  const std::string& name() const { return name_; }
+  int computeUnits() const { return cus_; }
+  size_t totalMemory() const { return totalMem_; }
+  void sync();
+
+  // statistics for PJRT_Device_MemoryStats
+  int64_t bytesInUse() const { return inUse_; }
+  int64_t peakBytesInUse() const { return peak_; }
+  int64_t numAllocs() const { return numAllocs_; }
+  int64_t largestAlloc() const { return largest_; }
+  int64_t bytesReserved() const { return reserved_; }
+
+  // compiled-kernel cache shared by all executables (key: source text)
+  mi355_function_t findKernel(const std::string& source);
+  void storeKernel(const std::string& source, mi355_function_t fn);
+
+  void* pinnedScratch() const { return pinned_; }   // 4 KiB pinned host buffer for predicate read-back
+
+ private:
+  Device();
+  std::mutex mu_;
+  mi355_stream_t stream_ = nullptr;
+  std::string arch_, name_;
+  int cus_ = 0;
+  size_t totalMem_ = 0;
+  std::multimap<size_t, void*> free_;
+  std::unordered_map<void*, size_t> sizes_;
+  std::unordered_map<std::string, mi355_function_t> kernels_;
+  int64_t inUse_ = 0, peak_ = 0, numAllocs_ = 0, largest_ = 0, reserved_ = 0;
+  void* pinned_ = nullptr;
+};
+
+struct DeviceBuffer {
+  void* ptr = nullptr;
+  TensorType type;
+  bool deleted = false;
+  ~DeviceBuffer();
+};
+
+struct KindStat {
+  int64_t count = 0;
+  double ms = 0;
+  double flops = 0;
+  double bytes = 0;
+};
+
+class Executable {
+ public:
+  explicit Executable(std::unique_ptr<CompiledProgram> prog);
+  ~Executable();
+
+  const CompiledProgram& program() const { return *prog_; }
+  // Runs the plan on the device stream; returns freshly allocated outputs (enqueued, not awaited).
+  std::vector<std::shared_ptr<DeviceBuffer>> execute(const std::vector<DeviceBuffer*>& inputs);
+  // Aggregated step timings (enabled with MI355X_TIMING=<kinds|all>); resolves pending events.
+  std::map<std::string, KindStat> timings();
+  double compileSeconds = 0;
+
+ private:
+  std::unique_ptr<CompiledProgram> prog_;
+  void* arena_ = nullptr;
+  void* consts_ = nullptr;
+  std::mutex mu_;
+
+  struct Pending { mi355_event_t a, b; std::string kind; double flops, bytes; };
+  std::vector<Pending> pending_;
+  std::vector<mi355_event_t> eventPool_;
+  std::map<std::string, KindStat> stats_;
+  std::string timingKinds_;
+
+  void loadKernels();
+  void* resolve(const BufRef& r, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) const;
+  void runPlan(const Plan& plan, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
+  void runStep(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
+  bool timed(const std::string& kind) const;
+  mi355_event_t getEvent();
+  void resolvePending();
+};
+
+}  // namespace mi355

@@ -427,4 +427,5 @@ def to_device_bytes(arr: np.ndarray, dtype: str) -> np.ndarray:
     """Host array in the element type the module declares (bf16 as uint16 bit patterns)."""
     if dtype == "bf16":
         return f32_to_bf16_bits(np.asarray(arr, np.float32))
-    return np.ascontiguousarray(arr)
+    a = np.asarray(arr)
+    return a if a.flags.c_contiguous else a.copy(order="C")
