@@ -955,14 +955,18 @@ struct RedOp {
   DType dt;       // element type of the reduce result
   std::string accT;
   std::string identity;
+  // Boolean forms use the non-short-circuit operators: the second operand may be a
+  // wavefront shuffle that every lane has to execute.
   std::string combine(const std::string& a, const std::string& b) const {
     std::string k = kind;
-    if (k == "add") return dt == DType::Pred ? "(" + a + " || " + b + ")" : "(" + a + " + " + b + ")";
-    if (k == "multiply") return dt == DType::Pred ? "(" + a + " && " + b + ")" : "(" + a + " * " + b + ")";
-    if (k == "maximum") return dt == DType::Pred ? "(" + a + " || " + b + ")" : "mx<" + accT + ">(" + a + ", " + b + ")";
-    if (k == "minimum") return dt == DType::Pred ? "(" + a + " && " + b + ")" : "mn<" + accT + ">(" + a + ", " + b + ")";
-    if (k == "and") return dt == DType::Pred ? "(" + a + " && " + b + ")" : "(" + accT + ")(" + a + " & " + b + ")";
-    return dt == DType::Pred ? "(" + a + " || " + b + ")" : "(" + accT + ")(" + a + " | " + b + ")";
+    bool p = dt == DType::Pred;
+    std::string band = "(bool)((int)" + a + " & (int)" + b + ")", bor = "(bool)((int)" + a + " | (int)" + b + ")";
+    if (k == "add") return p ? bor : "(" + a + " + " + b + ")";
+    if (k == "multiply") return p ? band : "(" + a + " * " + b + ")";
+    if (k == "maximum") return p ? bor : "mx<" + accT + ">(" + a + ", " + b + ")";
+    if (k == "minimum") return p ? band : "mn<" + accT + ">(" + a + ", " + b + ")";
+    if (k == "and") return p ? band : "(" + accT + ")(" + a + " & " + b + ")";
+    return p ? bor : "(" + accT + ")(" + a + " | " + b + ")";
   }
 };
 

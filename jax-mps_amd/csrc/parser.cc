@@ -461,10 +461,23 @@ class Parser {
         a.i = hexv ? (int64_t)strtoull(tk.c_str(), nullptr, 16) : strtoll(tk.c_str(), nullptr, 10);
         a.f = (double)a.i;
       }
+      // `1 : i64` is a typed literal; in `dim = 0 : (tensor<...>) -> ...` the colon starts the op's type
+      size_t save = i_;
       if (eat(":")) {
-        TensorType t = parseType();
-        if (hexv && t.dt == DType::F32) { uint32_t u = (uint32_t)a.i; float f; memcpy(&f, &u, 4); a.kind = Attr::Float; a.f = f; }
-        else if (isFloat(t.dt) && a.kind == Attr::Int && !hexv) { a.kind = Attr::Float; }
+        ws();
+        bool scalarType = false;
+        if (i_ < n_ && isalpha((unsigned char)s_[i_])) {
+          size_t e = i_;
+          while (e < n_ && isIdentChar(s_[e])) ++e;
+          scalarType = dtypeFromName(std::string(s_ + i_, e - i_)) != DType::Invalid;
+        }
+        if (!scalarType) {
+          i_ = save;
+        } else {
+          TensorType t = parseType();
+          if (hexv && t.dt == DType::F32) { uint32_t u = (uint32_t)a.i; float f; memcpy(&f, &u, 4); a.kind = Attr::Float; a.f = f; }
+          else if (isFloat(t.dt) && a.kind == Attr::Int && !hexv) { a.kind = Attr::Float; }
+        }
       }
       return a;
     }
@@ -605,10 +618,7 @@ class Parser {
     }
     if (eat("->")) {
       if (peekc() == '(') f->resultTypes = typeListParen();
-      else {
-        f->resultTypes.push_back(parseType());
-        if (peekc() == '{') skipBalanced('{', '}');
-      }
+      else f->resultTypes.push_back(parseType());   // attributes on results need the parenthesised form
     }
     if (eatWord("attributes")) skipBalanced('{', '}');
     expect("{");

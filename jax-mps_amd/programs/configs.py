@@ -423,6 +423,24 @@ ALL = {
 }
 
 
+# Reduced instances of the five programs: sizes the CPU oracle finishes in seconds.
+SMALL = {
+    "mlp": dict(batch=8, d_in=12, d_hidden=16),
+    "embedding": dict(vocab=50, dim=8, n_idx=32),
+    "resnet18": dict(batch=4, image=8, width=8, zero_bn2_scale=False),
+    "distilbert": dict(batch=2, seq=8, layers=2, d_model=16, heads=4, d_ff=32, vocab=50, max_pos=16),
+    "lstm": dict(seq=7, batch=4, d_in=6, hidden=8),
+}
+# Mid-size instances: large enough to span several workgroup tiles, still seconds on the oracle.
+MEDIUM = {
+    "mlp": dict(batch=96, d_in=200, d_hidden=130),
+    "embedding": dict(vocab=5000, dim=768, n_idx=2048),
+    "resnet18": dict(batch=8, image=16, width=16, zero_bn2_scale=False),
+    "distilbert": dict(batch=2, seq=40, layers=2, d_model=128, heads=4, d_ff=256, vocab=300, max_pos=64),
+    "lstm": dict(seq=12, batch=16, d_in=40, hidden=72),
+}
+
+
 def to_device_bytes(arr: np.ndarray, dtype: str) -> np.ndarray:
     """Host array in the element type the module declares (bf16 as uint16 bit patterns)."""
     if dtype == "bf16":

@@ -471,7 +471,9 @@ class Builder:
 
     def dynamic_slice(self, x: Val, starts: Sequence[Val], sizes) -> Val:
         v = self._new(sizes, x.dtype)
-        self._emit(f"{v.name} = stablehlo.dynamic_slice {x.name}, {', '.join(s.name for s in starts)}, sizes = [{', '.join(map(str, sizes))}] : ({x.type}, {', '.join(s.type for s in starts)}) -> {v.type}")
+        names = ", ".join([x.name] + [s.name for s in starts])
+        types = ", ".join([x.type] + [s.type for s in starts])
+        self._emit(f"{v.name} = stablehlo.dynamic_slice {names}, sizes = [{', '.join(map(str, sizes))}] : ({types}) -> {v.type}")
 
         def vjp(g):
             z = self.zeros(x.shape, x.dtype)
@@ -481,7 +483,9 @@ class Builder:
 
     def dynamic_update_slice(self, x: Val, upd: Val, starts: Sequence[Val]) -> Val:
         v = self._new(x.shape, x.dtype)
-        self._emit(f"{v.name} = stablehlo.dynamic_update_slice {x.name}, {upd.name}, {', '.join(s.name for s in starts)} : ({x.type}, {upd.type}, {', '.join(s.type for s in starts)}) -> {v.type}")
+        names = ", ".join([x.name, upd.name] + [s.name for s in starts])
+        types = ", ".join([x.type, upd.type] + [s.type for s in starts])
+        self._emit(f"{v.name} = stablehlo.dynamic_update_slice {names} : ({types}) -> {v.type}")
         return v
 
     # ------------------------------------------------------------ reductions
@@ -602,23 +606,35 @@ class Builder:
     def matmul(self, a: Val, b: Val) -> Val:
         return self.dot_general(a, b, ([a.ndim - 1], [0]))
 
-    def conv(self, lhs: Val, rhs: Val, *, strides=(1, 1), padding=((0, 0), (0, 0)), lhs_dilation=(1, 1),
-             rhs_dilation=(1, 1), dn=("b01f", "01io", "b01f"), feature_group_count=1, batch_group_count=1) -> Val:
-        """General 2-D convolution; dimension numbers given as strings like 'b01f','01io','b01f'."""
+    def conv(self, lhs: Val, rhs: Val, *, strides=None, padding=None, lhs_dilation=None,
+             rhs_dilation=None, dn=("b01f", "01io", "b01f"), feature_group_count=1, batch_group_count=1) -> Val:
+        """General N-d convolution; dimension numbers as strings like 'b01f','01io','b01f' (spatial dims are digits)."""
         ls, rs, os_ = dn
-        lb, lf, l0, l1 = ls.index("b"), ls.index("f"), ls.index("0"), ls.index("1")
-        ri, ro, r0, r1 = rs.index("i"), rs.index("o"), rs.index("0"), rs.index("1")
-        ob, of, o0, o1 = os_.index("b"), os_.index("f"), os_.index("0"), os_.index("1")
+        nsp = len(ls) - 2
+        strides = tuple(strides) if strides is not None else (1,) * nsp
+        padding = tuple(tuple(p) for p in padding) if padding is not None else ((0, 0),) * nsp
+        lhs_dilation = tuple(lhs_dilation) if lhs_dilation is not None else (1,) * nsp
+        rhs_dilation = tuple(rhs_dilation) if rhs_dilation is not None else (1,) * nsp
+        lb, lf = ls.index("b"), ls.index("f")
+        ri, ro = rs.index("i"), rs.index("o")
+        ob, of = os_.index("b"), os_.index("f")
+        lsp = [ls.index(str(d)) for d in range(nsp)]
+        rsp = [rs.index(str(d)) for d in range(nsp)]
+        osp = [os_.index(str(d)) for d in range(nsp)]
+        if nsp == 2:
+            l0, l1, r0, r1 = lsp[0], lsp[1], rsp[0], rsp[1]
         out_sp = []
-        for d, (isz, ksz) in enumerate(((lhs.shape[l0], rhs.shape[r0]), (lhs.shape[l1], rhs.shape[r1]))):
+        for d in range(nsp):
+            isz, ksz = lhs.shape[lsp[d]], rhs.shape[rsp[d]]
             din = (isz - 1) * lhs_dilation[d] + 1 if isz > 0 else 0
             dk = (ksz - 1) * rhs_dilation[d] + 1 if ksz > 0 else 0
             padded = din + padding[d][0] + padding[d][1]
             out_sp.append(0 if padded < dk else (padded - dk) // strides[d] + 1)
-        shape = [0] * 4
+        shape = [0] * (nsp + 2)
         shape[ob] = lhs.shape[lb] // batch_group_count
         shape[of] = rhs.shape[ro]
-        shape[o0], shape[o1] = out_sp
+        for d in range(nsp):
+            shape[osp[d]] = out_sp[d]
         v = self._new(shape, lhs.dtype)
 
         def fmt(s):
@@ -632,7 +648,7 @@ class Builder:
             f"precision_config = [#stablehlo<precision DEFAULT>, #stablehlo<precision DEFAULT>]}} : ({lhs.type}, {rhs.type}) -> {v.type}")
 
         def vjp(g):
-            assert feature_group_count == 1 and batch_group_count == 1 and tuple(lhs_dilation) == (1, 1)
+            assert nsp == 2 and feature_group_count == 1 and batch_group_count == 1 and tuple(lhs_dilation) == (1, 1)
             in_sp = (lhs.shape[l0], lhs.shape[l1])
             k_sp = (rhs.shape[r0], rhs.shape[r1])
             # --- input gradient: conv(g dilated by stride, reversed kernel with i<->o swapped)

@@ -293,8 +293,7 @@ class _P:
             tok = m.group(0)
             isf = any(ch in tok for ch in ".eE") and not tok.lower().startswith(("0x", "-0x")) or tok in ("inf", "nan")
             v = float(tok) if isf else int(tok, 0)
-            if self.eat(":"):
-                self.type()
+            self._eat_scalar_type_suffix()
             return v
         if s.startswith("tensor<", self.i):
             return self.type()
@@ -302,6 +301,17 @@ class _P:
         if idn is not None:
             return idn
         self.err("attribute value expected")
+
+    def _eat_scalar_type_suffix(self):
+        """`1 : i64` is a typed literal; `dim = 0 : (tensor<...>)` is not (the colon starts the op's type)."""
+        save = self.i
+        if self.eat(":"):
+            self.ws()
+            m = re.compile(r"(i|ui|si|f|bf)[0-9]+\b|index\b").match(self.s, self.i)
+            if m:
+                self.i = m.end()
+            else:
+                self.i = save
 
     def hash_attr(self):
         """#stablehlo.gather<...>, #stablehlo<precision DEFAULT>, #stablehlo.conv<...> ..."""
@@ -416,7 +426,6 @@ class _P:
                 f.result_types = self.type_list_paren()
             else:
                 f.result_types = [self.type()]
-                self.skip_attr_dict()
         if self.eat("attributes"):
             self.attr_dict()
         self.expect("{")
@@ -463,8 +472,10 @@ class _P:
             self.i = m.end()
             if self.eat(":"):
                 nres = self.integer()
+            end_decl = self.i
             self.expect("=")
-            op.results = [base] if nres == 1 else [f"{base}#{k}" for k in range(nres)]
+            explicit = ":" in self.s[m.end():end_decl]
+            op.results = [base] if (nres == 1 and not explicit) else [f"{base}#{k}" for k in range(nres)]
             has_res = True
         else:
             has_res = False
@@ -820,7 +831,7 @@ def parse(text: str) -> Dict[str, Func]:
 # ----------------------------------------------------------------------------
 # interpreter
 # ----------------------------------------------------------------------------
-def _cast_result(a: np.ndarray, t: TType) -> np.ndarray:
+def _cast_result(a: np.ndarray, t: TType, keep_shape: bool = False) -> np.ndarray:
     a = np.asarray(a)
     if t.dtype == "token":
         return a
@@ -829,7 +840,7 @@ def _cast_result(a: np.ndarray, t: TType) -> np.ndarray:
         a = a.astype(want)
     if t.dtype == "bf16":
         a = round_bf16(a)
-    if a.shape != t.shape:
+    if a.shape != t.shape and not keep_shape:
         a = a.reshape(t.shape)
     return a
 
@@ -856,7 +867,7 @@ class Oracle:
         return [(t.shape, t.dtype) for t in self.main.result_types]
 
     # -- engine
-    def _run_region(self, region: Region, args, outer_env) -> List[np.ndarray]:
+    def _run_region(self, region: Region, args, outer_env, vectorized: bool = False) -> List[np.ndarray]:
         env = dict(outer_env)
         for n, v in zip(region.args, args):
             env[n] = v
@@ -868,7 +879,9 @@ class Oracle:
             if not isinstance(outs, (list, tuple)):
                 outs = [outs]
             for name, val, t in zip(op.results, outs, op.out_types):
-                env[name] = _cast_result(val, t)
+                env[name] = _cast_result(val, t, keep_shape=vectorized)
+                if name.endswith("#0") and len(op.results) == 1:
+                    env[name[:-2]] = env[name]
         return []
 
     def _eval(self, op: Op, ins, env):
@@ -1269,7 +1282,7 @@ class Oracle:
         xt = [np.transpose(x, perm).reshape((-1,) + tuple(x.shape[d] for d in keep)) for x in xs]
         acc = [np.broadcast_to(i, xt[0].shape[1:]).astype(i.dtype).copy() for i in inits]
         for r in range(xt[0].shape[0]):
-            acc = self._run_region(body, acc + [x[r] for x in xt], env)
+            acc = self._run_region(body, acc + [x[r] for x in xt], env, vectorized=True)
         return acc
 
     # ------------------------------------------------------------------

@@ -1,0 +1,357 @@
+"""Per-op parity cases: small StableHLO modules with seeded inputs.
+
+The shapes and edge cases restate the reference's own per-op configs
+(tests/configs/{unary,binary,conversion,shape,slice,matmul,conv,reduction,control_flow}.py):
+each case is one module that goes through PJRT_Client_Compile / Execute and is
+compared with the CPU oracle on the same inputs (bit-exact for integer, boolean
+and data-movement results; 1e-5 relative for f32; 2e-2 for bf16).
+"""
+from __future__ import annotations
+
+import sys
+from dataclasses import dataclass
+from pathlib import Path
+from typing import Callable, List
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parents[1]
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+from jax_mps_amd.shlo.builder import Builder, Val, _NP  # noqa: E402
+
+_MLIR = {np.dtype(v): k for k, v in _NP.items()}
+
+
+@dataclass
+class Case:
+    name: str
+    text: str
+    inputs: List[np.ndarray]
+    dtypes: List[str]
+    exact: bool = False
+
+
+_cases: List[Callable[[], Case]] = []
+
+
+def case(name, fn, *inputs, dtypes=None, exact=False):
+    def make():
+        b = Builder("jit_" + name.replace("-", "_").replace(".", "_"))
+        dts = list(dtypes) if dtypes else [_MLIR[np.asarray(a).dtype] for a in inputs]
+        args = [b.arg(np.asarray(a).shape, d) for a, d in zip(inputs, dts)]
+        out = fn(b, *args)
+        if isinstance(out, Val):
+            out = [out]
+        b.ret(*out)
+        return Case(name, b.text(), [np.asarray(a) for a in inputs], dts, exact)
+    make.case_name = name
+    _cases.append(make)
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def f32(seed, *shape, lo=-2.0, hi=2.0):
+    return rng(seed).uniform(lo, hi, size=shape).astype(np.float32)
+
+
+def i32(seed, *shape, lo=-50, hi=50):
+    return rng(seed).integers(lo, hi, size=shape).astype(np.int32)
+
+
+# ------------------------------------------------------------------ unary (tests/configs/unary.py)
+for k, (op, lo, hi) in enumerate([
+        ("exp", -4, 4), ("log", 0.1, 9), ("sqrt", 0, 9), ("rsqrt", 0.1, 9), ("tanh", -4, 4), ("logistic", -6, 6),
+        ("abs", -3, 3), ("neg", -3, 3), ("sign", -3, 3), ("floor", -3, 3)]):
+    case("unary-" + op, (lambda o: lambda b, x: getattr(b, o)(x))(op), f32(k, 7, 33, lo=lo, hi=hi))
+for k, op in enumerate(["sine", "cosine", "ceil", "log_plus_one", "exponential_minus_one", "round_nearest_even",
+                        "round_nearest_afz", "cbrt", "tan"]):
+    case("unary-" + op, (lambda o: lambda b, x: b._unary(o, x))(op), f32(20 + k, 5, 17, lo=-1.2 if op != "log_plus_one" else -0.5, hi=1.2))
+case("unary-specials", lambda b, x: [b.exp(x), b.sign(x), b.abs(x), b._unary("is_finite", x) if False else b.neg(x)],
+     np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-40, -3.5, 88.0], np.float32))
+case("round-half", lambda b, x: [b._unary("round_nearest_even", x), b._unary("round_nearest_afz", x)],
+     np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.49, -3.51], np.float32), exact=True)
+
+# ------------------------------------------------------------------ binary (tests/configs/binary.py)
+for k, op in enumerate(["add", "sub", "mul", "div", "maximum", "minimum"]):
+    case("binary-" + op, (lambda o: lambda b, x, y: getattr(b, o)(x, y))(op), f32(40 + k, 9, 20), f32(60 + k, 9, 20, lo=0.5, hi=3))
+case("binary-power", lambda b, x, y: b.power(x, y), f32(70, 6, 11, lo=0.2, hi=3), f32(71, 6, 11))
+case("binary-remainder-float", lambda b, x, y: b.remainder(x, y), f32(72, 6, 11, lo=-9, hi=9), f32(73, 6, 11, lo=0.5, hi=3))
+case("binary-atan2", lambda b, x, y: b._binary("atan2", x, y), f32(74, 6, 11), f32(75, 6, 11))
+case("binary-broadcast-scalar", lambda b, x, y: b.add(b.mul(x, 2.5), b.broadcast_in_dim(y, x.shape, [])), f32(76, 3, 5, 8), f32(77))
+case("binary-nan-propagation", lambda b, x, y: [b.maximum(x, y), b.minimum(x, y)],
+     np.array([1.0, np.nan, 3.0, np.nan, -0.0, 0.0], np.float32), np.array([np.nan, 2.0, -np.inf, np.nan, 0.0, -0.0], np.float32))
+# integer semantics (arithmetic.cc:46-83, 496-513; mlx_executable.cc:293-301)
+case("int-arith", lambda b, x, y: [b.add(x, y), b.sub(x, y), b.mul(x, y), b.maximum(x, y), b.minimum(x, y)], i32(80, 6, 9), i32(81, 6, 9), exact=True)
+case("int-div-rem", lambda b, x, y: [b.div(x, y), b.remainder(x, y)],
+     np.array([7, -7, 7, -7, 0, 5, -5, 2147483647, -2147483648], np.int32), np.array([2, 2, -2, -2, 3, 0, 0, -1, 1], np.int32), exact=True)
+case("int-bitwise", lambda b, x, y: [b.and_(x, y), b.or_(x, y), b.xor(x, y), b.not_(x)], i32(82, 33, lo=-2**31, hi=2**31 - 1), i32(83, 33, lo=-2**31, hi=2**31 - 1), exact=True)
+case("int-shifts", lambda b, x, s: [b.shift_left(x, s), b.shift_right_logical(x, s), b._binary("shift_right_arithmetic", x, s)],
+     np.array([1, -1, 12345, -12345, 2**30, -2**31, 7, 7], np.int32), np.array([0, 1, 31, 4, 32, 33, -1, 100], np.int32), exact=True)
+case("uint-shifts", lambda b, x, s: [b.shift_left(x, s), b.shift_right_logical(x, s)],
+     np.array([1, 0xFFFFFFFF, 12345, 2**31], np.uint32), np.array([31, 32, 4, 40], np.uint32), exact=True)
+case("int-popcnt-clz", lambda b, x: [b._unary("popcnt", x), b._unary("count_leading_zeros", x)],
+     np.array([0, 1, -1, 255, 2**30, -2**31, 16777217], np.int32), exact=True)
+case("int-power", lambda b, x, y: b.power(x, y), np.array([2, 3, -2, 1, -1, 5, 0], np.int32), np.array([10, 4, 3, -5, -3, -1, 0], np.int32), exact=True)
+case("bool-logic", lambda b, x, y: [b.and_(x, y), b.or_(x, y), b.xor(x, y), b.not_(x)],
+     np.array([True, True, False, False]), np.array([True, False, True, False]), exact=True)
+
+# ------------------------------------------------------------------ compare / select / clamp
+for d in ["EQ", "NE", "LT", "LE", "GT", "GE"]:
+    case("compare-f32-" + d, (lambda dd: lambda b, x, y: b.compare(x, y, dd))(d),
+         np.array([1.0, 2.0, 2.0, np.nan, -0.0, np.inf], np.float32), np.array([2.0, 2.0, 1.0, 1.0, 0.0, np.inf], np.float32), exact=True)
+case("compare-i32", lambda b, x, y: [b.compare(x, y, "LT"), b.compare(x, y, "GE")], i32(90, 40, lo=-3, hi=3), i32(91, 40, lo=-3, hi=3), exact=True)
+case("compare-u32", lambda b, x, y: b.compare(x, y, "LT"), np.array([1, 0xFFFFFFFF, 5], np.uint32), np.array([0xFFFFFFFF, 1, 5], np.uint32), exact=True)
+case("compare-totalorder", lambda b, x, y: b.compare(x, y, "LT", "TOTALORDER"),
+     np.array([-0.0, 0.0, 1.0, -np.inf, -1.0], np.float32), np.array([0.0, -0.0, 2.0, np.inf, -2.0], np.float32), exact=True)
+case("select", lambda b, p, x, y: b.select(p, x, y), rng(92).integers(0, 2, size=(5, 12)).astype(bool), f32(93, 5, 12), f32(94, 5, 12), exact=True)
+case("select-scalar-pred", lambda b, p, x, y: b.select(b.broadcast_in_dim(p, x.shape, []), x, y), np.array(True), f32(95, 4, 4), f32(96, 4, 4), exact=True)
+case("clamp", lambda b, x: b.clamp(-0.5, x, 0.75), f32(97, 6, 10), exact=True)
+case("clamp-int", lambda b, x: b.clamp(-3, x, 4), i32(98, 30), exact=True)
+
+# ------------------------------------------------------------------ conversions (tests/configs/conversion.py)
+case("convert-f32-i32", lambda b, x: b.convert(x, "i32"),
+     np.array([0.9, -0.9, 1.5, -1.5, 3e9, -3e9, np.nan, np.inf, -np.inf, 2147483520.0], np.float32), exact=True)
+case("convert-f32-u8", lambda b, x: b.convert(x, "ui8"), np.array([0.9, -5.0, 255.9, 300.0, np.nan], np.float32), exact=True)
+case("convert-i32-f32", lambda b, x: b.convert(x, "f32"), np.array([0, 1, -1, 16777217, 2**31 - 1, -2**31], np.int32), exact=True)
+case("convert-f32-bf16-f32", lambda b, x: b.convert(b.convert(x, "bf16"), "f32"), f32(100, 9, 16, lo=-100, hi=100), exact=True)
+case("convert-f32-f16", lambda b, x: b.convert(b.convert(x, "f16"), "f32"), f32(101, 33, lo=-100, hi=100), exact=True)
+case("convert-bool", lambda b, x: [b.convert(x, "i1"), b.convert(b.convert(x, "i1"), "f32")], np.array([0.0, 1.0, -2.0, np.nan, 0.5], np.float32), exact=True)
+case("convert-i64-i32", lambda b, x: b.convert(x, "i32"), np.array([2**40 + 5, -1, 2**31], np.int64), exact=True)
+case("bitcast-f32-i32", lambda b, x: b.bitcast_convert(x, "i32"), np.array([1.0, -0.0, np.inf, 1e-40], np.float32), exact=True)
+case("bitcast-i32-f32", lambda b, x: b.bitcast_convert(x, "f32"), np.array([0x3F800000, 0x7F800000, 1], np.int32), exact=True)
+
+# ------------------------------------------------------------------ shape ops (tests/configs/shape.py)
+case("broadcast_in_dim", lambda b, x: b.broadcast_in_dim(x, (4, 3, 5), [1]), f32(110, 3), exact=True)
+case("broadcast-expand-unit", lambda b, x: b.broadcast_in_dim(x, (4, 3, 5), [0, 1, 2]), f32(111, 4, 1, 5), exact=True)
+case("reshape", lambda b, x: b.reshape(x, (6, 20)), f32(112, 3, 8, 5), exact=True)
+case("reshape-after-transpose", lambda b, x: b.reshape(b.transpose(x, [1, 0, 2]), (8, 15)), f32(113, 3, 8, 5), exact=True)
+case("transpose-2d", lambda b, x: b.transpose(x, [1, 0]), f32(114, 37, 65), exact=True)
+case("transpose-4d", lambda b, x: b.transpose(x, [0, 2, 1, 3]), f32(115, 2, 5, 3, 8), exact=True)
+case("reverse", lambda b, x: b.reverse(x, [0, 2]), f32(116, 3, 4, 5), exact=True)
+case("concatenate", lambda b, x, y, z: b.concatenate([x, y, z], 1), f32(117, 3, 2), f32(118, 3, 5), f32(119, 3, 1), exact=True)
+case("concatenate-dim0", lambda b, x, y: b.concatenate([x, y], 0), f32(120, 3, 8), f32(121, 5, 8), exact=True)
+case("iota", lambda b, x: b.add(x, b.convert(b.iota((4, 6), 1), "f32")), f32(122, 4, 6), exact=True)
+case("slice", lambda b, x: b.slice(x, [1, 0, 2], [3, 4, 8], [1, 2, 3]), f32(123, 4, 4, 9), exact=True)
+case("pad", lambda b, x: b.pad(x, -1.0, [1, 0], [2, 3], [0, 1]), f32(124, 3, 4), exact=True)
+case("pad-negative", lambda b, x: b.pad(x, 0.5, [-1, 2], [1, -2], [0, 0]), f32(125, 4, 6), exact=True)
+case("pad-interior-negative", lambda b, x: b.pad(x, 9.0, [-1, 0], [-1, 1], [2, 0]), f32(126, 4, 3), exact=True)
+case("dynamic_slice", lambda b, x, i, j: b.dynamic_slice(x, [i, j], [2, 3]), f32(127, 5, 7), np.int32(2), np.int32(3), exact=True)
+case("dynamic_slice-clamped", lambda b, x, i, j: b.dynamic_slice(x, [i, j], [2, 3]), f32(128, 5, 7), np.int32(9), np.int32(-4), exact=True)
+case("dynamic_update_slice", lambda b, x, u, i, j: b.dynamic_update_slice(x, u, [i, j]), f32(129, 5, 7), f32(130, 2, 3), np.int32(1), np.int32(2), exact=True)
+case("dynamic_update_slice-clamped", lambda b, x, u, i, j: b.dynamic_update_slice(x, u, [i, j]), f32(131, 5, 7), f32(132, 2, 3), np.int32(7), np.int32(-2), exact=True)
+case("dynamic_update_slice-scalar", lambda b, x, u: b.dynamic_update_slice(x, u, []), f32(133), f32(134), exact=True)
+case("bf16-elementwise", lambda b, x, y: b.add(b.mul(x, y), b.tanh(x)), f32(135, 16, 24), f32(136, 16, 24), dtypes=["bf16", "bf16"])
+
+# ------------------------------------------------------------------ gather (tests/configs/slice.py:33-43,217-240,391-456)
+case("gather-take-rows", lambda b, x, i: b.take_rows(x, i), f32(140, 5, 3), np.array([0, 2, 4], np.int32), exact=True)
+case("gather-take-negative-and-oob", lambda b, x, i: b.take_rows(x, i), f32(141, 5, 3), np.array([-1, 4, 5, -6, 0], np.int32))
+case("gather-multi-index-point", lambda b, x, i: b.gather(x, i, offset_dims=[], collapsed_slice_dims=[0, 1], start_index_map=[0, 1],
+                                                          index_vector_dim=1, slice_sizes=[1, 1]),
+     f32(142, 4, 4), np.stack([np.arange(4), np.arange(4)], 1).astype(np.int32), exact=True)
+case("gather-batched-single-axis", lambda b, x, i: b.gather(x, b.reshape(i, (3, 1)), offset_dims=[], collapsed_slice_dims=[1],
+                                                            operand_batching_dims=[0], start_indices_batching_dims=[0],
+                                                            start_index_map=[1], index_vector_dim=1, slice_sizes=[1, 1]),
+     f32(143, 3, 10), np.array([7, 0, 9], np.int32), exact=True)
+case("gather-partial-reversed-index-map", lambda b, x, i: b.gather(x, i, offset_dims=[1], collapsed_slice_dims=[0, 2], start_index_map=[2, 0],
+                                                                   index_vector_dim=1, slice_sizes=[1, 4, 1]),
+     f32(144, 3, 4, 5), np.array([[3, 2]], np.int32), exact=True)
+case("gather-partial-scalar-indices", lambda b, x, i: b.gather(x, i, offset_dims=[0], collapsed_slice_dims=[0, 2], start_index_map=[0, 2],
+                                                               index_vector_dim=0, slice_sizes=[1, 4, 1]),
+     f32(145, 3, 4, 5), np.array([1, 0], np.int32), exact=True)
+case("gather-multi-dim-no-collapse", lambda b, x, i: b.gather(x, i, offset_dims=[0, 1, 2], collapsed_slice_dims=[], start_index_map=[1, 2],
+                                                              index_vector_dim=1, slice_sizes=[2, 1, 1]) if False else
+     b.gather(x, i, offset_dims=[1, 2, 3], collapsed_slice_dims=[], start_index_map=[1, 2], index_vector_dim=1, slice_sizes=[2, 1, 1]),
+     f32(146, 2, 3, 3), np.array([[0, 1], [1, 2], [0, 0]], np.int32), exact=True)
+case("gather-clamped-window", lambda b, x, i: b.gather(x, i, offset_dims=[1], collapsed_slice_dims=[], start_index_map=[0],
+                                                       index_vector_dim=1, slice_sizes=[3]),
+     f32(147, 8), np.array([[0], [6], [7], [-2]], np.int32), exact=True)
+case("gather-large-int32", lambda b, x, i: b.take_rows(x, i), np.array([[16777217], [2**30], [2**31 - 1]], np.int32), np.array([1, 0, 2], np.int32), exact=True)
+case("gather-large-uint32", lambda b, x, i: b.take_rows(x, i), np.array([[16777217], [2**30], [2**31 - 1]], np.uint32), np.array([1], np.int32), exact=True)
+case("gather-large-int64", lambda b, x, i: b.take_rows(x, i), np.array([[2**40], [2**50], [2**62]], np.int64), np.array([2, 0], np.int32), exact=True)
+
+
+def _row_scatter(body, **kw):
+    def f(b, x, i, u):
+        return b.scatter(x, b.reshape(i, (i.shape[0], 1)), u, update_window_dims=list(range(1, u.ndim)), inserted_window_dims=[0],
+                         scatter_dims_to_operand_dims=[0], index_vector_dim=1, body=body, **kw)
+    return f
+
+
+# ------------------------------------------------------------------ scatter (tests/configs/slice.py:175-216,241-295)
+case("scatter-add", _row_scatter("add"), np.zeros((10, 4), np.float32), np.array([0, 2, 5], np.int32), np.ones((3, 4), np.float32), exact=True)
+case("scatter-add-duplicates", _row_scatter("add"), f32(150, 10, 4), np.array([3, 3, 0, 3, 9, 0, 3], np.int32), f32(151, 7, 4), exact=True)
+case("scatter-add-oob-dropped", _row_scatter("add"), f32(152, 6, 5), np.array([0, 6, -1, 5, 100], np.int32), f32(153, 5, 5), exact=True)
+case("scatter-set", _row_scatter("set"), f32(154, 5, 3), np.array([0, 2], np.int32), f32(155, 2, 3), exact=True)
+case("scatter-mul", _row_scatter("mul", unique_indices=True), np.ones((10, 4), np.float32), np.array([0, 2, 5], np.int32), np.full((3, 4), 2.0, np.float32), exact=True)
+case("scatter-min", _row_scatter("min"), f32(156, 10, 4), np.array([0, 2, 5], np.int32), f32(157, 3, 4), exact=True)
+case("scatter-max", _row_scatter("max"), f32(158, 10, 4), np.array([0, 2, 2], np.int32), f32(159, 3, 4), exact=True)
+case("scatter-large-int32", _row_scatter("set"), np.zeros((5, 1), np.int32), np.array([1], np.int32), np.array([[2**30]], np.int32), exact=True)
+case("scatter-large-uint32", _row_scatter("set"), np.zeros((5, 1), np.uint32), np.array([2], np.int32), np.array([[16777217]], np.uint32), exact=True)
+case("scatter-add-many", _row_scatter("add"), f32(160, 300, 70), rng(161).integers(0, 300, size=1000).astype(np.int32), f32(162, 1000, 70), exact=True)
+
+# ------------------------------------------------------------------ dot_general (tests/configs/matmul.py:19-249)
+case("dot-matmul", lambda b, x, y: b.matmul(x, y), f32(170, 33, 70), f32(171, 70, 45))
+case("dot-vector-matrix", lambda b, x, y: b.dot_general(x, y, ([0], [0])), f32(172, 70), f32(173, 70, 45))
+case("dot-matrix-vector", lambda b, x, y: b.dot_general(x, y, ([1], [0])), f32(174, 33, 70), f32(175, 70))
+case("dot-inner", lambda b, x, y: b.dot_general(x, y, ([0], [0])), f32(176, 129), f32(177, 129))
+case("dot-transposed-lhs", lambda b, x, y: b.dot_general(x, y, ([0], [0])), f32(178, 70, 33), f32(179, 70, 45))
+case("dot-transposed-rhs", lambda b, x, y: b.dot_general(x, y, ([1], [1])), f32(180, 33, 70), f32(181, 45, 70))
+case("dot-batched", lambda b, x, y: b.dot_general(x, y, ([2], [1]), ([0], [0])), f32(182, 5, 17, 40), f32(183, 5, 40, 23))
+case("dot-batched-attention-layout", lambda b, q, k: b.dot_general(q, k, ([3], [3]), ([0, 2], [0, 2])), f32(184, 2, 9, 3, 16), f32(185, 2, 11, 3, 16))
+case("dot-two-contracting", lambda b, x, y: b.dot_general(x, y, ([1, 2], [0, 1])), f32(186, 6, 4, 5), f32(187, 4, 5, 7))
+case("dot-bf16", lambda b, x, y: b.matmul(x, y), f32(188, 40, 96), f32(189, 96, 72), dtypes=["bf16", "bf16"])
+case("dot-bf16-f32-out", lambda b, x, y: b.dot_general(x, y, ([1], [0]), out_dtype="f32"), f32(190, 40, 96), f32(191, 96, 72), dtypes=["bf16", "bf16"])
+case("dot-large-k", lambda b, x, y: b.matmul(x, y), f32(192, 64, 3000, lo=-1, hi=1), f32(193, 3000, 64, lo=-1, hi=1))
+
+
+def _conv(**kw):
+    return lambda b, x, w: b.conv(x, w, **kw)
+
+
+def _same(n, k, s, d=1):
+    out = -(-n // s)
+    tot = max((out - 1) * s + (k - 1) * d + 1 - n, 0)
+    return (tot // 2, tot - tot // 2)
+
+
+# ------------------------------------------------------------------ convolution (tests/configs/conv.py:9-224)
+u = lambda seed, *shape: f32(seed, *shape, lo=-1, hi=1)
+case("conv-SAME", _conv(padding=(_same(8, 3, 1),) * 2), u(200, 2, 8, 8, 3), u(201, 3, 3, 3, 8))
+case("conv-NCHW-OIHW", _conv(padding=(_same(8, 3, 1),) * 2, dn=("bf01", "oi01", "bf01")), u(202, 1, 3, 8, 8), u(203, 16, 3, 3, 3))
+case("conv-1d-NWC", _conv(strides=(2,), padding=(_same(16, 3, 2),), dn=("b0f", "0io", "b0f")), u(204, 2, 16, 3), u(205, 3, 3, 4))
+case("conv-stride2-SAME", _conv(strides=(2, 2), padding=(_same(8, 3, 2),) * 2), u(206, 2, 8, 8, 3), u(207, 3, 3, 3, 8))
+case("conv-stride2-asymmetric", _conv(strides=(2, 2), padding=((1, 0), (1, 0))), u(208, 2, 8, 8, 3), u(209, 3, 3, 3, 8))
+case("conv-5x5-stride2", _conv(strides=(2, 2), padding=(_same(16, 5, 2),) * 2), u(210, 2, 16, 16, 3), u(211, 5, 5, 3, 8))
+case("conv-stride2-dilated", _conv(strides=(2, 2), padding=(_same(16, 3, 2, 2),) * 2, rhs_dilation=(2, 2)), u(212, 2, 16, 16, 3), u(213, 3, 3, 3, 8))
+case("conv-stride2-VALID", _conv(strides=(2, 2)), u(214, 2, 9, 9, 3), u(215, 3, 3, 3, 8))
+case("conv-1d-stride2-dilated", _conv(strides=(2,), padding=(_same(32, 3, 2, 2),), rhs_dilation=(2,), dn=("b0f", "0io", "b0f")), u(216, 2, 32, 3), u(217, 3, 3, 4))
+case("conv-lhs_dilation-neg_padding", _conv(padding=((0, -1), (0, 0)), lhs_dilation=(2, 1)), u(218, 1, 6, 7, 4), u(219, 1, 2, 4, 2))
+case("conv-lhs_dilation-only", _conv(lhs_dilation=(2, 1)), u(220, 1, 6, 7, 4), u(221, 1, 2, 4, 2))
+case("conv-large-kernel", _conv(padding=(_same(4, 8, 1),) * 2), u(222, 1, 4, 4, 3), u(223, 8, 8, 3, 16))
+case("conv-batch_group_count_2", _conv(dn=("bf01", "oi01", "bf01"), batch_group_count=2), u(224, 4, 1, 6, 7), u(225, 2, 1, 1, 2))
+case("conv-batch_group_count_3-multi_filter", _conv(padding=((1, 1), (1, 1)), batch_group_count=3), u(226, 6, 5, 5, 2), u(227, 3, 3, 2, 6))
+case("conv-depthwise", _conv(padding=((1, 1), (1, 1)), feature_group_count=6), u(228, 2, 7, 7, 6), u(229, 3, 3, 1, 12))
+case("conv-grouped", _conv(padding=((1, 1), (1, 1)), feature_group_count=2), u(230, 2, 7, 7, 8), u(231, 3, 3, 4, 6))
+case("conv-1x1", _conv(), u(232, 3, 9, 9, 20), u(233, 1, 1, 20, 24))
+case("conv-resnet-block-shape", _conv(padding=((1, 1), (1, 1))), u(234, 4, 16, 16, 64), u(235, 3, 3, 64, 64))
+case("conv-wgrad-form", lambda b, x, g: b.conv(x, g, strides=(1, 1), padding=((1, 1), (1, 1)), rhs_dilation=(2, 2), dn=("f01b", "i01o", "01bf")),
+     u(236, 4, 16, 16, 24), u(237, 4, 8, 8, 40))
+case("conv-dgrad-form", lambda b, g, w: b.conv(g, b.reverse(w, [0, 1]), strides=(1, 1), padding=((1, 2), (1, 2)), lhs_dilation=(2, 2), dn=("b01f", "01oi", "b01f")),
+     u(238, 4, 8, 8, 40), u(239, 3, 3, 24, 40))
+case("conv-bf16", _conv(padding=((1, 1), (1, 1))), u(240, 2, 8, 8, 16), u(241, 3, 3, 16, 8), dtypes=["bf16", "bf16"])
+
+# ------------------------------------------------------------------ reduce (tests/configs/reduction.py:8-39)
+case("reduce-sum-all", lambda b, x: b.reduce_sum(x, [0, 1]), f32(250, 37, 53))
+case("reduce-sum-rows", lambda b, x: b.reduce_sum(x, [1]), f32(251, 37, 53))
+case("reduce-sum-cols", lambda b, x: b.reduce_sum(x, [0]), f32(252, 37, 53))
+case("reduce-sum-middle", lambda b, x: b.reduce_sum(x, [1]), f32(253, 5, 19, 12))
+case("reduce-sum-outer-two", lambda b, x: b.reduce_sum(x, [0, 1, 2]), f32(254, 4, 9, 9, 16))
+case("reduce-sum-nonadjacent", lambda b, x: b.reduce_sum(x, [0, 2]), f32(255, 6, 7, 8))
+case("reduce-max", lambda b, x: b.reduce_max(x, [1]), f32(256, 21, 130), exact=True)
+case("reduce-min", lambda b, x: b.reduce_min(x, [0]), f32(257, 21, 130), exact=True)
+case("reduce-prod", lambda b, x: b._reduce(x, [1], "multiply", 1.0), f32(258, 9, 12, lo=0.5, hi=1.5))
+case("reduce-sum-int", lambda b, x: b.reduce_sum(x, [0]), i32(259, 100, 7), exact=True)
+case("reduce-and-or", lambda b, x: [b._reduce(x, [1], "and", True), b._reduce(x, [1], "or", False)], rng(260).integers(0, 2, size=(6, 9)).astype(bool), exact=True)
+case("reduce-long-row", lambda b, x: b.reduce_sum(x, [1]), f32(261, 3, 70000, lo=-1, hi=1))
+case("reduce-tall-column", lambda b, x: b.reduce_sum(x, [0]), f32(262, 50000, 24, lo=-1, hi=1))
+case("reduce-full-large", lambda b, x: b.reduce_sum(x, [0]), f32(263, 1 << 20, lo=-1, hi=1))
+case("reduce-siblings", lambda b, x: [b.reduce_sum(x, [0, 1, 2]), b.reduce_sum(b.mul(x, x), [0, 1, 2])], f32(264, 8, 12, 12, 32))
+case("reduce-fused-input", lambda b, x, m: b.reduce_sum(b.mul(b.sub(x, b.broadcast_in_dim(m, x.shape, [1])), 2.0), [0]), f32(265, 300, 40), f32(266, 40))
+case("reduce-bf16", lambda b, x: b.reduce_sum(x, [1]), f32(267, 12, 256), dtypes=["bf16"])
+case("softmax-rows", lambda b, x: __import__("jax_mps_amd.shlo.builder", fromlist=["softmax"]).softmax(b, x, -1), f32(268, 33, 100))
+case("layer-norm", lambda b, x, s, t: __import__("jax_mps_amd.shlo.builder", fromlist=["layer_norm"]).layer_norm(b, x, s, t, 1e-5), f32(269, 20, 96), f32(270, 96), f32(271, 96))
+case("argmax", lambda b, x: b.argmax(x, 1), f32(272, 9, 31), exact=True)
+
+# ------------------------------------------------------------------ control flow (tests/configs/control_flow.py:66-80,232-263,389-458)
+def _sum_to_n(b, n, x):
+    # fori-style loop: i from 0 while i < n; acc += x * i
+    zero = b.constant(0, "i32")
+    out = b.while_loop([zero, b.zeros(x.shape)], lambda i, acc: b.compare(i, n, "LT"),
+                       lambda i, acc: [b.add(i, 1), b.add(acc, b.mul(x, b._bcast_np(b.convert(i, "f32"), x.shape)))])
+    return out[1]
+
+
+case("while-sum-0-4", lambda b, x: _sum_to_n(b, 5, x), np.ones((3,), np.float32), exact=True)
+case("while-130-iterations", lambda b, x: _sum_to_n(b, 130, x), f32(280, 8), )
+case("while-zero-trip", lambda b, x: _sum_to_n(b, 0, x), f32(281, 4), exact=True)
+
+
+def _dynamic_while(b, x, limit):
+    # value-dependent condition: double until the sum exceeds the limit
+    out = b.while_loop([x], lambda v: b.compare(b.reduce_sum(v, [0]), limit, "LT"), lambda v: [b.mul(v, 2.0)])
+    return out[0]
+
+
+case("while-value-dependent", _dynamic_while, np.array([1.0, 2.0, 3.0], np.float32), np.float32(100.0), exact=True)
+
+
+def _traced_bound(b, x, n):
+    zero = b.constant(0, "i32")
+    out = b.while_loop([zero, x], lambda i, v: b.compare(i, n, "LT"), lambda i, v: [b.add(i, 1), b.add(v, 1.5)])
+    return out[1]
+
+
+case("while-traced-bound", _traced_bound, f32(282, 5), np.int32(7), exact=True)
+
+
+def _nested(b, x):
+    zero = b.constant(0, "i32")
+
+    def outer_body(i, acc):
+        inner = b.while_loop([b.constant(0, "i32"), acc], lambda j, a: b.compare(j, 3, "LT"), lambda j, a: [b.add(j, 1), b.add(a, x)])
+        return [b.add(i, 1), b.mul(inner[1], 0.5)]
+    return b.while_loop([zero, b.zeros(x.shape)], lambda i, acc: b.compare(i, 4, "LT"), outer_body)[1]
+
+
+case("while-nested", _nested, f32(283, 6))
+
+
+def _scan_dus(b, xs):
+    # scan that stacks running sums: carries (i, acc, out[T, n])
+    T, n = xs.shape
+    z = b.constant(0, "i32")
+
+    def body(i, acc, out):
+        x_t = b.reshape(b.dynamic_slice(xs, [i, b.constant(0, "i32")], [1, n]), (n,))
+        acc2 = b.add(acc, x_t)
+        return [b.add(i, 1), acc2, b.dynamic_update_slice(out, b.reshape(acc2, (1, n)), [i, b.constant(0, "i32")])]
+    return b.while_loop([z, b.zeros((n,)), b.zeros((T, n))], lambda i, a, o: b.compare(i, T, "LT"), body)[2]
+
+
+case("while-scan-cumsum", _scan_dus, f32(284, 9, 5))
+
+
+def _swap(b, x, y):
+    z = b.constant(0, "i32")
+    r = b.while_loop([z, x, y], lambda i, p, q: b.compare(i, 3, "LT"), lambda i, p, q: [b.add(i, 1), q, b.add(p, 1.0)])
+    return [r[1], r[2]]
+
+
+case("while-swapped-carries", _swap, f32(285, 4), f32(286, 4), exact=True)
+
+
+def _case3(b, idx, x):
+    return b.case(idx, [lambda: b.mul(x, 2.0), lambda: b.add(x, 10.0), lambda: b.neg(x)], [(x.shape, "f32")])[0]
+
+
+for k, v in enumerate([0, 1, 2, 5, -1]):
+    case(f"case-index-{v}", _case3, np.int32(v), f32(290 + k, 4), exact=True)
+
+
+def all_cases() -> List[Case]:
+    return [mk() for mk in _cases]
+
+
+def case_names() -> List[str]:
+    return [mk.case_name for mk in _cases]
+
+
+def get_case(name: str) -> Case:
+    for mk in _cases:
+        if mk.case_name == name:
+            return mk()
+    raise KeyError(name)
