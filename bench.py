@@ -1,0 +1,162 @@
+"""Benchmark: jitted ResNet18 (CIFAR variant) train steps per second, batch 128, fp32, SGD momentum,
+on one MI355X through the plugin's PJRT C API, plus fused-op HBM bandwidth.
+
+Prints ONE JSON line.  `value` is steps/s with all inputs resident in HBM; `roofline` is the
+convolution kernels' achieved fp32 matrix throughput (algorithmic flops / HIP-event time on the
+compute stream, collected by the plugin and read back through PJRT_Executable_GetCostAnalysis);
+`cpu_baseline` is the numpy oracle on a bounded sample of the same workload on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for p in (str(ROOT), str(ROOT / "oracle")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+import numpy as np  # noqa: E402
+
+PEAK_HBM_GBS = 8000.0
+PEAK_F32_MFMA_TFLOPS = 157.3
+
+
+def fused_op_modules():
+    """The fused-op bandwidth shapes (elementwise / reduce chains of the reference's benchmark configs,
+    tests/configs/benchmark.py:14-45, and of the ResNet18 / DistilBERT programs)."""
+    from jax_mps_amd.shlo.builder import Builder, gelu_tanh, layer_norm, softmax
+
+    def mod(name, fn, *specs):
+        b = Builder("fused_" + name)
+        args = [b.arg(s, d) for s, d in specs]
+        out = fn(b, *args)
+        b.ret(*(out if isinstance(out, (list, tuple)) else [out]))
+        return name, b.text()
+
+    n = 10_000_000
+    c = 64
+    act = (128, 32, 32, c)
+    return [
+        mod("add_10M_f32", lambda b, x, y: b.add(x, y), ((n,), "f32"), ((n,), "f32")),
+        mod("exp_10M_f32", lambda b, x: b.exp(x), ((n,), "f32")),
+        mod("sum_10M_f32", lambda b, x: b.reduce_sum(x, [0]), ((n,), "f32")),
+        mod("softmax_10000x1000_f32", lambda b, x: softmax(b, x, -1), ((10000, 1000), "f32")),
+        mod("bn_apply_relu_128x32x32x64_f32",
+            lambda b, x, s, t: b.maximum(b.add(b.mul(x, b.broadcast_in_dim(s, act, [3])), b.broadcast_in_dim(t, act, [3])), 0.0),
+            (act, "f32"), ((c,), "f32"), ((c,), "f32")),
+        mod("bn_stats_128x32x32x64_f32", lambda b, x: [b.reduce_sum(x, [0, 1, 2]), b.reduce_sum(b.mul(x, x), [0, 1, 2])], (act, "f32")),
+        mod("layernorm_4096x768_bf16", lambda b, x, s, t: layer_norm(b, x, s, t, 1e-12), ((4096, 768), "bf16"), ((768,), "bf16"), ((768,), "bf16")),
+        mod("bias_gelu_4096x3072_bf16", lambda b, x, t: gelu_tanh(b, b.add(x, b.broadcast_in_dim(t, (4096, 3072), [1]))), ((4096, 3072), "bf16"), ((3072,), "bf16")),
+    ]
+
+
+_FUSED_BYTES = {   # algorithmic bytes: distinct inputs + outputs, broadcast operands at their own size
+    "add_10M_f32": 120e6, "exp_10M_f32": 80e6, "sum_10M_f32": 40e6, "softmax_10000x1000_f32": 80e6,
+    "bn_apply_relu_128x32x32x64_f32": 2 * 128 * 32 * 32 * 64 * 4, "bn_stats_128x32x32x64_f32": 128 * 32 * 32 * 64 * 4,
+    "layernorm_4096x768_bf16": 2 * 4096 * 768 * 2, "bias_gelu_4096x3072_bf16": 2 * 4096 * 3072 * 2,
+}
+
+
+def bench_fused_ops(client, iters=20):
+    from jax_mps_amd import pjrt, runner
+    from shlo_oracle import parse
+    out = []
+    rng = np.random.default_rng(7)
+    for name, text in fused_op_modules():
+        main = parse(text)["main"]
+        ins = [rng.standard_normal(t.shape).astype(np.float32) for t in main.body.arg_types]
+        dts = [t.dtype for t in main.body.arg_types]
+        exe = client.compile_and_load(text)
+        bufs = runner.upload(client, ins, dts)
+        for _ in range(3):
+            r = exe.execute(bufs)
+        r[0].block_until_ready()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            r = exe.execute(bufs)
+        r[0].block_until_ready()
+        dt = (time.perf_counter() - t0) / iters
+        ca = exe.cost_analysis()
+        # device time of the kernels themselves (HIP events), when the plugin was asked to time them
+        kms = sum(v for k, v in ca.items() if k.endswith(".time_ms"))
+        kcount = sum(v for k, v in ca.items() if k.endswith(".count"))
+        dev = (kms / (iters + 3)) * 1e-3 if kcount else dt
+        gbs = _FUSED_BYTES[name] / dev / 1e9
+        out.append({"op": name, "GB/s": round(gbs, 1), "frac_of_peak": round(gbs / PEAK_HBM_GBS, 4), "us": round(dev * 1e6, 2),
+                    "launches": int(ca.get("steps", 0))})
+    return out
+
+
+def cpu_baseline(sample_batch=16, full_batch=128):
+    """The numpy oracle (float32 BLAS accumulation) on one train step at a reduced batch; steps/s scaled
+    to the full batch linearly."""
+    from jax_mps_amd.programs import configs
+    from shlo_oracle import Oracle
+    p = configs.build_resnet18(batch=sample_batch)
+    o = Oracle(p.text, accum="f32")
+    t0 = time.perf_counter()
+    o.run(*p.inputs)
+    dt = time.perf_counter() - t0
+    return {"value": round((1.0 / dt) * sample_batch / full_batch, 5), "unit": "steps/s", "cores": os.cpu_count(), "kind": "port",
+            "sample": f"1 ResNet18 train step at batch {sample_batch} of {full_batch} ({dt:.1f} s), scaled by {sample_batch}/{full_batch}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-fused", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build drives exactly one GPU (one PJRT device); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    os.environ.setdefault("MI355X_TIMING", "conv")     # HIP-event timing of the convolution launches only
+    from jax_mps_amd import pjrt, runner
+    from jax_mps_amd.programs import configs
+    client = pjrt.get_client()
+    p = configs.build_resnet18()
+    cp = runner.CompiledProgram(p, client)
+    for _ in range(args.warmup):
+        outs = cp.step()
+    outs[-1].block_until_ready()
+    before = cp.exe.cost_analysis()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        outs = cp.step()
+    outs[-1].block_until_ready()
+    dt = time.perf_counter() - t0
+    after = cp.exe.cost_analysis()
+    loss = float(runner.download(outs[-1]))
+    assert np.isfinite(loss), loss
+    conv_ms = after.get("conv.time_ms", 0.0) - before.get("conv.time_ms", 0.0)
+    conv_n = after.get("conv.count", 0.0) - before.get("conv.count", 0.0)
+    conv_flops = p.meta["step_flops"] - 6 * 128 * 512 * 10      # dense head is a GEMM step, not a convolution
+    achieved = conv_flops * args.steps / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else None
+    line = {
+        "metric": "jitted train steps/sec (ResNet18 b128, 1 MI355X); fused-op HBM GB/s vs peak",
+        "value": round(args.steps / dt, 3), "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt / args.steps * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "resnet18_cifar_train_step_batch128_fp32_sgd_momentum", "steps_per_launch_sequence": int(after.get("steps", 0)),
+                   "final_loss": round(loss, 5)},
+        "roofline": {"bound": "mfma", "kernel": "convolution (all launches of one step)", "achieved": None if achieved is None else round(achieved, 3),
+                     "peak": PEAK_F32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": None if achieved is None else round(achieved / PEAK_F32_MFMA_TFLOPS, 4),
+                     "traffic": None, "launches_per_step": conv_n / max(args.steps, 1), "avg_launch_us": round(conv_ms * 1e3 / conv_n, 2) if conv_n else None,
+                     "algorithmic_flops_per_step": conv_flops},
+    }
+    if not args.no_fused:
+        os.environ["MI355X_TIMING"] = "all"
+        line["fused_ops"] = bench_fused_ops(client)
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline()
+        line["speedup_vs_cpu_baseline"] = round(line["value"] / line["cpu_baseline"]["value"], 1)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

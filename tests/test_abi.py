@@ -1,0 +1,80 @@
+"""The C-ABI boundary without a GPU: the library loads, exports exactly the declared symbol, and its
+function table has the populated / NULL entries the header (and the reference's table,
+src/pjrt_plugin/pjrt_api.cc:232-393) prescribes.  No compute calls here."""
+import ctypes as C
+import re
+import subprocess
+from pathlib import Path
+
+import pytest
+
+from jax_mps_amd import pjrt
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = (ROOT / "include" / "pjrt_c_api.h").read_text()
+
+
+@pytest.fixture(scope="module")
+def plugin():
+    return pjrt.Plugin()
+
+
+def test_exports_only_the_declared_symbol():
+    declared = re.findall(r"^const PJRT_Api\* (\w+)\(void\);", HEADER, flags=re.M)
+    assert declared == ["GetPjrtApi"]
+    out = subprocess.run(["nm", "-D", "--defined-only", pjrt.default_library_path()], capture_output=True, text=True, check=True).stdout
+    syms = {line.split()[-1] for line in out.splitlines() if " T " in line or " W " in line}
+    ours = {s for s in syms if "PJRT" in s.upper() or "mi355" in s.lower() or s == "GetPjrtApi"}
+    assert ours == {"GetPjrtApi"}, ours
+
+
+def test_table_header_and_version(plugin):
+    api = plugin.api
+    assert api.struct_size == C.sizeof(pjrt.Api)
+    assert api.pjrt_api_version.major_version == int(re.search(r"#define PJRT_API_MAJOR (\d+)", HEADER).group(1))
+    assert api.pjrt_api_version.minor_version == int(re.search(r"#define PJRT_API_MINOR (\d+)", HEADER).group(1))
+    assert api.extension_start   # profiler extension stub is chained
+
+
+def test_python_table_mirrors_the_header():
+    body = HEADER[HEADER.index("typedef struct PJRT_Api {"):HEADER.index("} PJRT_Api;")]
+    fields = re.findall(r"_PJRT_API_STRUCT_FIELD\((\w+)\);|PJRT_Unimplemented_Fn\* (\w+);", body)
+    names = [a or b for a, b in fields]
+    assert names == pjrt.API_ENTRIES
+    nulls = {b for a, b in fields if b}
+    assert nulls == pjrt.NULL_ENTRIES
+
+
+def test_every_entry_is_populated_or_null_as_declared(plugin):
+    for name in pjrt.API_ENTRIES:
+        ptr = getattr(plugin.api, name)
+        if name in pjrt.NULL_ENTRIES:
+            assert not ptr, f"{name} must be NULL"
+        else:
+            assert ptr, f"{name} must be populated"
+
+
+def test_static_identity_entries(plugin):
+    # entries that need no device
+    a = plugin.call("PJRT_Plugin_Initialize", pjrt.Plugin_Initialize_Args())
+    assert a is not None
+
+
+def test_client_create_without_gpu_is_a_clean_error(plugin):
+    """No CPU fallback: without a device PJRT_Client_Create returns a PJRT_Error (code INTERNAL)."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present; the error path needs a machine without one")
+    with pytest.raises(pjrt.PjrtError) as e:
+        pjrt.Client(plugin)
+    assert "no HIP device" in str(e.value) or "HIP" in str(e.value)
+    assert e.value.code == 13
+
+
+def test_unimplemented_entries_return_the_code(plugin):
+    class A(C.Structure):
+        _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("pad", C.c_void_p * 8)]
+    for name in ("PJRT_Executable_Serialize", "PJRT_Executable_DeserializeAndLoad", "PJRT_Compile", "PJRT_Executable_OptimizedProgram"):
+        with pytest.raises(pjrt.PjrtError) as e:
+            plugin.call(name, A())
+        assert e.value.code == 12, name

@@ -1,0 +1,305 @@
+"""Pins of the CPU oracle that the golden vectors leave open: library routines (torch CPU conv2d /
+conv_transpose2d, numpy einsum), brute force on tiny inputs, IEEE identities, and torch autograd for
+the five benchmark programs (which also pins the StableHLO emitter's VJP rules)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import op_cases
+from jax_mps_amd.programs import configs
+from jax_mps_amd.shlo.builder import Builder
+from shlo_oracle import Oracle, round_bf16, f32_to_bf16_bits, bf16_bits_to_f32
+
+
+def run(fn, *inputs, dtypes=None):
+    b = Builder("pin")
+    dts = dtypes or ["f32" if np.asarray(a).dtype.kind == "f" else "i32" for a in inputs]
+    args = [b.arg(np.asarray(a).shape, d) for a, d in zip(inputs, dts)]
+    out = fn(b, *args)
+    out = out if isinstance(out, (list, tuple)) else [out]
+    b.ret(*out)
+    return Oracle(b.text()).run(*inputs)
+
+
+def rnd(seed, *shape):
+    return np.random.default_rng(seed).uniform(-1, 1, size=shape).astype(np.float32)
+
+
+# ------------------------------------------------------------------ convolution
+@pytest.mark.parametrize("stride,pad,rdil", [(1, 1, 1), (2, 1, 1), (2, 0, 1), (1, 2, 2), (2, 3, 2)])
+def test_conv_forward_vs_torch(stride, pad, rdil):
+    x, w = rnd(1, 2, 9, 10, 3), rnd(2, 3, 3, 3, 5)
+    got = run(lambda b, a, k: b.conv(a, k, strides=(stride, stride), padding=((pad, pad), (pad, pad)), rhs_dilation=(rdil, rdil)), x, w)[0]
+    want = F.conv2d(torch.tensor(x).double().permute(0, 3, 1, 2), torch.tensor(w).double().permute(3, 2, 0, 1), stride=stride, padding=pad, dilation=rdil)
+    np.testing.assert_allclose(got, want.permute(0, 2, 3, 1).numpy(), rtol=1e-6, atol=1e-6)
+
+
+def test_conv_asymmetric_and_negative_padding_vs_torch():
+    x, w = rnd(3, 1, 8, 8, 2), rnd(4, 3, 3, 2, 4)
+    got = run(lambda b, a, k: b.conv(a, k, padding=((2, -1), (0, 1))), x, w)[0]
+    xt = torch.tensor(x).double().permute(0, 3, 1, 2)
+    xt = F.pad(xt, (0, 1, 2, 0))[:, :, :-1, :]          # pad W by (0,1), H by (2,0), then crop one row at the bottom
+    want = F.conv2d(xt, torch.tensor(w).double().permute(3, 2, 0, 1))
+    np.testing.assert_allclose(got, want.permute(0, 2, 3, 1).numpy(), rtol=1e-6, atol=1e-6)
+
+
+def test_conv_lhs_dilation_is_transposed_conv():
+    # lhs dilation by s with padding k-1 and a flipped kernel == conv_transpose2d with stride s
+    x, w = rnd(5, 2, 5, 5, 3), rnd(6, 3, 3, 3, 4)
+    got = run(lambda b, a, k: b.conv(a, b.reverse(k, [0, 1]), padding=((2, 2), (2, 2)), lhs_dilation=(2, 2)), x, w)[0]
+    want = F.conv_transpose2d(torch.tensor(x).double().permute(0, 3, 1, 2), torch.tensor(w).double().permute(2, 3, 0, 1), stride=2)
+    np.testing.assert_allclose(got, want.permute(0, 2, 3, 1).numpy(), rtol=1e-6, atol=1e-6)
+
+
+def test_conv_groups_vs_torch():
+    x, w = rnd(7, 2, 7, 7, 8), rnd(8, 3, 3, 4, 6)
+    got = run(lambda b, a, k: b.conv(a, k, padding=((1, 1), (1, 1)), feature_group_count=2), x, w)[0]
+    want = F.conv2d(torch.tensor(x).double().permute(0, 3, 1, 2), torch.tensor(w).double().permute(3, 2, 0, 1), padding=1, groups=2)
+    np.testing.assert_allclose(got, want.permute(0, 2, 3, 1).numpy(), rtol=1e-6, atol=1e-6)
+
+
+def test_conv_brute_force_general_dimension_numbers():
+    # NCHW input, OIHW kernel, stride (2,1), rhs dilation (1,2), padding ((1,0),(2,1)): seven nested loops
+    x, w = rnd(9, 2, 3, 6, 7), rnd(10, 4, 3, 2, 3)
+    got = run(lambda b, a, k: b.conv(a, k, strides=(2, 1), padding=((1, 0), (2, 1)), rhs_dilation=(1, 2), dn=("bf01", "oi01", "bf01")), x, w)[0]
+    N, C, H, W = x.shape
+    O, _, KH, KW = w.shape
+    OH = (H + 1 + 0 - ((KH - 1) * 1 + 1)) // 2 + 1
+    OW = (W + 2 + 1 - ((KW - 1) * 2 + 1)) // 1 + 1
+    want = np.zeros((N, O, OH, OW))
+    for n in range(N):
+        for o in range(O):
+            for oh in range(OH):
+                for ow in range(OW):
+                    for c in range(C):
+                        for kh in range(KH):
+                            for kw in range(KW):
+                                ih, iw = oh * 2 - 1 + kh, ow - 2 + kw * 2
+                                if 0 <= ih < H and 0 <= iw < W:
+                                    want[n, o, oh, ow] += float(x[n, c, ih, iw]) * float(w[o, c, kh, kw])
+    assert got.shape == want.shape
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+
+
+def test_conv_batch_group_count_brute_force():
+    x, w = rnd(11, 6, 5, 5, 2), rnd(12, 3, 3, 2, 6)
+    got = run(lambda b, a, k: b.conv(a, k, padding=((1, 1), (1, 1)), batch_group_count=3), x, w)[0]
+    # group g uses batch rows [2g, 2g+2) and output features [2g, 2g+2)
+    want = np.zeros((2, 5, 5, 6))
+    for g in range(3):
+        xs = torch.tensor(x[2 * g:2 * g + 2]).double().permute(0, 3, 1, 2)
+        ws = torch.tensor(w[..., 2 * g:2 * g + 2]).double().permute(3, 2, 0, 1)
+        want[..., 2 * g:2 * g + 2] = F.conv2d(xs, ws, padding=1).permute(0, 2, 3, 1).numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+
+
+# ------------------------------------------------------------------ dot_general
+@pytest.mark.parametrize("spec,contract,batch,sa,sb", [
+    ("ik,kj->ij", ([1], [0]), ((), ()), (5, 7), (7, 3)),
+    ("ki,kj->ij", ([0], [0]), ((), ()), (7, 5), (7, 3)),
+    ("ik,jk->ij", ([1], [1]), ((), ()), (5, 7), (3, 7)),
+    ("bik,bkj->bij", ([2], [1]), ([0], [0]), (4, 5, 7), (4, 7, 3)),
+    ("btnh,bsnh->bnts", ([3], [3]), ([0, 2], [0, 2]), (2, 5, 3, 4), (2, 6, 3, 4)),
+    ("ijk,jkl->il", ([1, 2], [0, 1]), ((), ()), (3, 4, 5), (4, 5, 6)),
+    ("k,k->", ([0], [0]), ((), ()), (9,), (9,)),
+])
+def test_dot_general_vs_einsum(spec, contract, batch, sa, sb):
+    a, b_ = rnd(20, *sa), rnd(21, *sb)
+    got = run(lambda b, x, y: b.dot_general(x, y, contract, batch), a, b_)[0]
+    want = np.einsum(spec, a.astype(np.float64), b_.astype(np.float64))
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+
+
+# ------------------------------------------------------------------ reductions / elementwise identities
+def test_reduce_vs_numpy():
+    x = rnd(30, 6, 7, 8)
+    for dims in ([0], [1], [2], [0, 2], [0, 1, 2]):
+        got = run(lambda b, a: b.reduce_sum(a, dims), x)[0]
+        np.testing.assert_allclose(got, x.astype(np.float64).sum(tuple(dims)), rtol=1e-6, atol=1e-6)
+    assert np.array_equal(run(lambda b, a: b.reduce_max(a, [1]), x)[0], x.max(1))
+    assert np.array_equal(run(lambda b, a: b.reduce_min(a, [0, 2]), x)[0], x.min((0, 2)))
+
+
+def test_argmax_first_occurrence():
+    x = np.array([[1, 3, 3, 0], [2, 2, 2, 2], [0, -1, 5, 5]], np.float32)
+    assert np.array_equal(run(lambda b, a: b.argmax(a, 1), x)[0], np.array([1, 0, 2], np.int32))
+
+
+def test_bf16_rounding_is_nearest_even():
+    # 1 + 2^-8 lies exactly between two bf16 values: ties go to the even mantissa
+    x = np.array([1 + 2.0 ** -8, 1 + 3 * 2.0 ** -8, 1 + 2.0 ** -7, 3.0e38, -1e-40], np.float32)
+    r = round_bf16(x)
+    assert r[0] == 1.0 and r[1] == np.float32(1 + 2.0 ** -6) and r[2] == x[2]
+    assert np.array_equal(bf16_bits_to_f32(f32_to_bf16_bits(x)), r)
+    assert np.isinf(round_bf16(np.array([3.4e38], np.float32))[0])
+
+
+def test_convert_float_to_int_saturates():
+    x = np.array([3e9, -3e9, np.nan, 1.9, -1.9], np.float32)
+    assert np.array_equal(run(lambda b, a: b.convert(a, "i32"), x)[0], np.array([2**31 - 1, -2**31, 0, 1, -1], np.int32))
+
+
+def test_total_order_compare():
+    a = np.array([-0.0, 0.0], np.float32)
+    b_ = np.array([0.0, -0.0], np.float32)
+    assert np.array_equal(run(lambda b, x, y: b.compare(x, y, "LT", "TOTALORDER"), a, b_)[0], np.array([True, False]))
+    assert np.array_equal(run(lambda b, x, y: b.compare(x, y, "LT"), a, b_)[0], np.array([False, False]))
+
+
+def test_scatter_is_sequential_in_update_order():
+    # float addition is not associative: only the in-order fold gives this exact value
+    rng = np.random.default_rng(40)
+    idx = rng.integers(0, 7, size=500).astype(np.int32)
+    upd = (rng.standard_normal((500, 3)) * 10 ** rng.uniform(-3, 3, size=(500, 1))).astype(np.float32)
+    op = rng.standard_normal((7, 3)).astype(np.float32)
+    c = op_cases._row_scatter("add")
+    got = run(c, op, idx, upd)[0]
+    want = op.copy()
+    for i, u in zip(idx, upd):
+        want[i] = want[i] + u
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+# ------------------------------------------------------------------ the five programs vs torch autograd
+def test_mlp_program_vs_torch():
+    p = configs.build_mlp(**configs.SMALL["mlp"])
+    out = Oracle(p.text).run(*p.inputs)
+    w1, b1, w2, b2, x, y = [torch.tensor(a) for a in p.inputs]
+    ps = [t.double().requires_grad_(True) for t in (w1, b1, w2, b2)]
+    loss = F.cross_entropy(torch.relu(x.double() @ ps[0] + ps[1]) @ ps[2] + ps[3], y.long())
+    loss.backward()
+    assert abs(float(out[-1]) - loss.item()) < 1e-6
+    for t, o in zip(ps, out):
+        np.testing.assert_allclose(o, (t - 0.01 * t.grad).detach().numpy(), rtol=1e-5, atol=1e-6)
+
+
+def _torch_resnet(p, width):
+    specs = configs.resnet18_param_specs(width, 10)
+    n = len(specs)
+    P = {nm: torch.tensor(a, dtype=torch.float64, requires_grad=True) for (nm, _, _), a in zip(specs, p.inputs[:n])}
+    x = torch.tensor(p.inputs[-2], dtype=torch.float64).permute(0, 3, 1, 2)
+    y = torch.tensor(p.inputs[-1]).long()
+
+    def conv(name, h, stride):
+        w = P[name + ".kernel"].permute(3, 2, 0, 1)
+        k = w.shape[2]
+        n_in = h.shape[2]
+        out = -(-n_in // stride)
+        tot = max((out - 1) * stride + k - n_in, 0)
+        lo, hi = tot // 2, tot - tot // 2
+        return F.conv2d(F.pad(h, (lo, hi, lo, hi)), w, stride=stride)
+
+    def bn(name, h):
+        m = h.mean((0, 2, 3))
+        v = torch.clamp((h * h).mean((0, 2, 3)) - m * m, min=0)
+        return (h - m[None, :, None, None]) * (torch.rsqrt(v + 1e-5) * P[name + ".scale"])[None, :, None, None] + P[name + ".bias"][None, :, None, None]
+
+    h = torch.relu(bn("bn_init", conv("conv_init", x, 1)))
+    cin = width
+    for stage, mult in enumerate((1, 2, 4, 8), 1):
+        cout = width * mult
+        for blk in (1, 2):
+            stride = 2 if (stage > 1 and blk == 1) else 1
+            pn = f"stage{stage}_block{blk}"
+            r = h
+            yv = torch.relu(bn(pn + ".bn1", conv(pn + ".conv1", h, stride)))
+            yv = bn(pn + ".bn2", conv(pn + ".conv2", yv, 1))
+            if cin != cout or stride != 1:
+                r = bn(pn + ".bn_proj", conv(pn + ".conv_proj", r, stride))
+            h = torch.relu(r + yv)
+            cin = cout
+    loss = F.cross_entropy(h.mean((2, 3)) @ P["dense.kernel"] + P["dense.bias"], y)
+    loss.backward()
+    return specs, P, loss
+
+
+def test_resnet18_program_vs_torch():
+    p = configs.build_resnet18(batch=4, image=8, width=8, zero_bn2_scale=False)
+    out = Oracle(p.text).run(*p.inputs)
+    specs, P, loss = _torch_resnet(p, 8)
+    assert abs(float(out[-1]) - loss.item()) < 2e-5
+    n = len(specs)
+    nstat = len(p.inputs) - 2 - 2 * n
+    for i, (nm, _, _) in enumerate(specs):
+        g = P[nm].grad.numpy()
+        mom = out[n + nstat + i]          # new momentum = grad (old momentum is zero)
+        assert np.abs(mom - g).max() <= 2e-5 * (np.abs(g).max() + 1e-12), nm
+        np.testing.assert_allclose(out[i], p.inputs[i] - 0.1 * g, rtol=0, atol=3e-6 * (np.abs(g).max() + 1))
+
+
+def test_embedding_program_vs_numpy():
+    p = configs.build_embedding(**configs.SMALL["embedding"])
+    rows, dtable = Oracle(p.text).run(*p.inputs)
+    table, idx, g = p.inputs
+    assert np.array_equal(rows, table[idx])
+    want = np.zeros_like(table)
+    for i, u in zip(idx, g):
+        want[i] = want[i] + u
+    assert np.array_equal(dtable.view(np.uint32), want.view(np.uint32))
+
+
+def test_lstm_program_vs_torch():
+    kw = configs.SMALL["lstm"]
+    p = configs.build_lstm(**kw)
+    out = Oracle(p.text).run(*p.inputs)
+    H, T, B = kw["hidden"], kw["seq"], kw["batch"]
+    wi, wh, b, wo, bo = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in p.inputs[:5]]
+    xs = torch.tensor(p.inputs[-2], dtype=torch.float64)
+    y = torch.tensor(p.inputs[-1]).long()
+    h = torch.zeros(B, H, dtype=torch.float64)
+    c = torch.zeros(B, H, dtype=torch.float64)
+    for t in range(T):
+        z = xs[t] @ wi + h @ wh + b
+        i, f, g, o = torch.sigmoid(z[:, :H]), torch.sigmoid(z[:, H:2 * H]), torch.tanh(z[:, 2 * H:3 * H]), torch.sigmoid(z[:, 3 * H:])
+        c = f * c + i * g
+        h = o * torch.tanh(c)
+    loss = F.cross_entropy(h @ wo + bo, y)
+    loss.backward()
+    assert abs(float(out[-1]) - loss.item()) < 1e-6
+    for k, t in enumerate((wi, wh, b, wo, bo)):
+        g = t.grad.numpy()
+        m = 0.1 * g
+        np.testing.assert_allclose(out[5 + k], m, rtol=0, atol=2e-6 * np.abs(m).max())
+        step = (m / 0.1) / (np.sqrt(g * g) + 1e-8)     # bias-corrected Adam direction at step 1
+        np.testing.assert_allclose(out[k], t.detach().numpy() - 1e-3 * step, rtol=0, atol=2e-5)
+    assert int(out[15]) == 1
+
+
+def test_distilbert_program_vs_torch():
+    kw = dict(configs.SMALL["distilbert"])
+    p = configs.build_distilbert(dtype="f32", **kw)
+    out = Oracle(p.text).run(*p.inputs)[0]
+    A = {n: torch.tensor(a, dtype=torch.float64) for n, a in zip(p.input_names, p.inputs)}
+    ids = torch.tensor(p.inputs[-2]).long()
+    B, T, D, Hh = kw["batch"], kw["seq"], kw["d_model"], kw["heads"]
+
+    def ln(x, s, b):
+        m = x.mean(-1, keepdim=True)
+        v = ((x * x).mean(-1, keepdim=True) - m * m).clamp(min=0)
+        return (x - m) * torch.rsqrt(v + 1e-12) * s + b
+    x = ln(A["word_emb"][ids] + A["pos_emb"][torch.arange(T)][None], A["emb_ln.scale"], A["emb_ln.bias"])
+    for l in range(kw["layers"]):
+        pf = f"layer{l}."
+        qkv = (x @ A[pf + "qkv.kernel"] + A[pf + "qkv.bias"]).reshape(B, T, 3, Hh, D // Hh)
+        q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+        pr = torch.softmax(torch.einsum("btnh,bsnh->bnts", q, k) / math.sqrt(D // Hh), -1)
+        enc = torch.einsum("bnts,bsnh->btnh", pr, v).reshape(B, T, D)
+        x = ln(x + enc @ A[pf + "out.kernel"] + A[pf + "out.bias"], A[pf + "sa_ln.scale"], A[pf + "sa_ln.bias"])
+        ff = F.gelu(x @ A[pf + "ffn1.kernel"] + A[pf + "ffn1.bias"], approximate="tanh") @ A[pf + "ffn2.kernel"] + A[pf + "ffn2.bias"]
+        x = ln(x + ff, A[pf + "out_ln.scale"], A[pf + "out_ln.bias"])
+    np.testing.assert_allclose(out, x.numpy(), rtol=0, atol=5e-6)
+    # bf16 module: within bf16 resolution of the f32 result
+    pb = configs.build_distilbert(dtype="bf16", **kw)
+    ins = [round_bf16(a) if d == "bf16" else a for a, d in zip(pb.inputs, pb.input_dtypes)]
+    outb = Oracle(pb.text).run(*ins)[0]
+    assert np.abs(outb - x.numpy()).max() <= 2e-2 * np.abs(x.numpy()).max()
+
+
+def test_all_op_cases_run_on_the_oracle():
+    for c in op_cases.all_cases():
+        ins = [round_bf16(a) if d == "bf16" else a for a, d in zip(c.inputs, c.dtypes)]
+        out = Oracle(c.text).run(*ins)
+        assert len(out) >= 1, c.name
