@@ -17,6 +17,7 @@
 #include <unordered_set>
 
 #include "codegen.h"
+#include "hip_abi.h"
 #include "plan.h"
 
 namespace mi355 {
@@ -608,8 +609,8 @@ class Planner {
     s.scatter.kind = std::string(kind) == "add" ? 0 : std::string(kind) == "set" ? 1 : std::string(kind) == "mul" ? 2 : std::string(kind) == "min" ? 3 : 4;
     s.scatter.type = res->type.dt;
     s.scatter.indexType = idx->type.dt;
-    // workspace: sorted keys, permutation, segment heads (4 arrays of numUpdates 4-byte words, double-buffered sort)
-    int64_t wsBytes = ((nUpd * 4 * 6 + 1024) + kAlign - 1) / kAlign * kAlign;
+    // workspace: double-buffered keys and permutation plus the radix-sort counters
+    int64_t wsBytes = ((int64_t)mi355_scatter_workspace_bytes(nUpd) + kAlign - 1) / kAlign * kAlign;
     int ws = newStorage((size_t)wsBytes);
     s.workspaceBytes = wsBytes;
     s.args = {ref(sid, t), ref(storageOf(idx), t), ref(storageOf(upd), t), ref(ws, t)};

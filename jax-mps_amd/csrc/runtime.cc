@@ -397,6 +397,8 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       d.kind = s.scatter.kind;
       d.dtype = dtypeCode(s.scatter.type);
       d.index_bytes = (int)dtypeSize(s.scatter.indexType);
+      if ((size_t)s.workspaceBytes < mi355_scatter_workspace_bytes(d.numUpdates))
+        throw RuntimeError("internal: scatter workspace is smaller than the kernel needs");
       check(mi355_scatter_rows(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out),
                                resolve(s.args[3], in, out), st), "scatter");
       break;
