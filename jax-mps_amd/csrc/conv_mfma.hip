@@ -1,0 +1,428 @@
+// Implicit-GEMM convolution on the fp32 matrix cores of gfx950.
+//
+//   out[b, o0, o1, f] = sum over (k0, k1, c) of lhs[b, pos0, pos1, c] * rhs[k0, k1, c, f]
+//
+// seen as C[M, N] = A[M, K] x B[K, N] with M = batch x output positions, N = output
+// features, K = window taps x input features.  Every tensor is addressed through the
+// element strides of its logical dims, so forward convolutions (NHWC x HWIO), input
+// gradients (lhs dilation, reversed kernel with i/o swapped) and filter gradients
+// (batch and feature swapped, rhs dilation) are the same kernel with different loaders:
+//
+//   A loader  K-vector: features contiguous in lhs      (forward, input gradient)
+//             M-vector: conv-batch dim contiguous in lhs (filter gradient)
+//             scalar  : anything else (3-channel stem, odd strides)
+//   B loader  N-vector: output features contiguous in rhs (forward, filter gradient)
+//             K-vector: input features contiguous in rhs  (input gradient)
+//             scalar  : anything else
+//
+// A workgroup of four wavefronts owns a BM x BN tile (2 x 2 wavefronts, each WM x WN built
+// from 32x32 accumulators of v_mfma_f32_32x32x2_f32).  Tiles of A and B are staged in LDS
+// k-major, so that every MFMA operand is one conflict-free row read; the next k-tile is
+// fetched into registers while the current one is multiplied.  Problems with few output
+// tiles (filter gradients, late stages) split K across blockIdx.z into partial sums that a
+// second kernel folds in a fixed order, which keeps results reproducible.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+
+#include "hip_abi.h"
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int BK = 16;
+
+struct ConvP {
+  const float* lhs;
+  const float* rhs;
+  float* out;       // final output, or partial sums [split][M][N] when splitK > 1
+  int M, N, K;
+  int Nb, C;
+  int in0, in1, k0n, k1n, o0n, o1n;
+  int s0, s1, p0, p1, ld0, ld1, rd0, rd1, rev0, rev1;
+  int lhsB, lhsF, lhsS0, lhsS1, rhsI, rhsO, rhsS0, rhsS1, outB, outF, outS0, outS1;
+  int bFast;            // 1: m = (o0, o1, b) with b fastest; 0: m = (b, o0, o1)
+  int cTiles;           // k-tiles per window tap (tap-chunk tiling)
+  int kTiles;           // total k-tiles
+  int splitK, tilesPerSplit;
+};
+
+struct Row {
+  int base;   // element offset of (b) in lhs; -1 when the row is outside M
+  int i0, i1; // window origin in the dilated, padded input
+};
+
+__device__ __forceinline__ Row makeRow(const ConvP& p, int m) {
+  Row r;
+  if (m >= p.M) { r.base = -1; r.i0 = 0; r.i1 = 0; return r; }
+  int b, o0, o1;
+  if (p.bFast) { b = m % p.Nb; int t = m / p.Nb; o1 = t % p.o1n; o0 = t / p.o1n; }
+  else { o1 = m % p.o1n; int t = m / p.o1n; o0 = t % p.o0n; b = t / p.o0n; }
+  r.base = b * p.lhsB;
+  r.i0 = o0 * p.s0 - p.p0;
+  r.i1 = o1 * p.s1 - p.p1;
+  return r;
+}
+
+// offset of the input element that window tap (k0, k1) touches for this row, or -1 (padding / dilation hole)
+__device__ __forceinline__ int tapOffset(const ConvP& p, const Row& r, int k0, int k1) {
+  if (r.base < 0) return -1;
+  int q0 = r.i0 + k0 * p.rd0, q1 = r.i1 + k1 * p.rd1;
+  if (q0 < 0 || q1 < 0) return -1;
+  if (p.ld0 != 1) { if (q0 % p.ld0) return -1; q0 /= p.ld0; }
+  if (p.ld1 != 1) { if (q1 % p.ld1) return -1; q1 /= p.ld1; }
+  if (q0 >= p.in0 || q1 >= p.in1) return -1;
+  return r.base + q0 * p.lhsS0 + q1 * p.lhsS1;
+}
+
+__device__ __forceinline__ int rhsTapOffset(const ConvP& p, int k0, int k1) {
+  int a = p.rev0 ? p.k0n - 1 - k0 : k0, b = p.rev1 ? p.k1n - 1 - k1 : k1;
+  return a * p.rhsS0 + b * p.rhsS1;
+}
+
+template <int BM, int BN, int AMODE, int BMODE, bool KFLAT>
+__global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+  constexpr int NA4 = BM / 64, NB4 = BN / 64;            // float4 per thread per tile (vector loaders)
+  constexpr int NAS = BM * BK / 256, NBS = BN * BK / 256; // floats per thread per tile (scalar loaders)
+  __shared__ float As[BK][BM + 4];
+  __shared__ float Bs[BK][BN + 4];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const int ktBegin = blockIdx.z * p.tilesPerSplit;
+  const int ktEnd = min(p.kTiles, ktBegin + p.tilesPerSplit);
+
+  // ---- per-thread rows of the A tile (fixed for the whole K loop)
+  Row rowsA[AMODE == 0 ? NAS : NA4];
+  if (AMODE == 1) {
+#pragma unroll
+    for (int i = 0; i < NA4; ++i) rowsA[i] = makeRow(p, m0 + (tid >> 2) + 64 * i);
+  } else if (AMODE == 2) {
+    rowsA[0] = makeRow(p, m0 + 4 * (tid % (BM / 4)));     // 4 consecutive m share (o0, o1); b .. b+3 are contiguous
+#pragma unroll
+    for (int i = 1; i < NA4; ++i) rowsA[i] = rowsA[0];
+  } else {
+#pragma unroll
+    for (int i = 0; i < NAS; ++i) rowsA[i] = makeRow(p, m0 + (tid + 256 * i) / BK);
+  }
+
+  float4 ra[NA4 > 0 ? NA4 : 1];
+  float4 rb[NB4 > 0 ? NB4 : 1];
+  float ras[NAS], rbs[NBS];
+
+  auto loadTile = [&](int kt) {
+    int tap = 0, c0 = 0, k0 = 0, k1 = 0;
+    if (!KFLAT) {
+      tap = kt / p.cTiles;
+      c0 = (kt - tap * p.cTiles) * BK;
+      k0 = tap / p.k1n;
+      k1 = tap - k0 * p.k1n;
+    }
+    // ---------------- A
+    if (AMODE == 1) {
+      const int kq = (tid & 3) * 4;
+#pragma unroll
+      for (int i = 0; i < NA4; ++i) {
+        int off = tapOffset(p, rowsA[i], k0, k1);
+        ra[i] = off >= 0 ? *(const float4*)(p.lhs + off + c0 + kq) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    } else if (AMODE == 2) {
+      int off = tapOffset(p, rowsA[0], k0, k1);
+#pragma unroll
+      for (int i = 0; i < NA4; ++i) {
+        int kr = tid / (BM / 4) + (1024 / BM) * i;
+        ra[i] = off >= 0 ? *(const float4*)(p.lhs + off + (c0 + kr) * p.lhsF) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NAS; ++i) {
+        int k = (tid + 256 * i) % BK;
+        int kk0 = k0, kk1 = k1, c = c0 + k;
+        bool ok = true;
+        if (KFLAT) {
+          int kf = kt * BK + k;
+          ok = kf < p.K;
+          int t = kf / p.C;
+          c = kf - t * p.C;
+          kk0 = t / p.k1n;
+          kk1 = t - kk0 * p.k1n;
+        }
+        int off = ok ? tapOffset(p, rowsA[i], kk0, kk1) : -1;
+        ras[i] = off >= 0 ? p.lhs[off + c * p.lhsF] : 0.f;
+      }
+    }
+    // ---------------- B
+    if (BMODE == 1) {
+      const int nq = 4 * (tid % (BN / 4));
+      const int toff = rhsTapOffset(p, k0, k1);
+#pragma unroll
+      for (int i = 0; i < NB4; ++i) {
+        int kr = tid / (BN / 4) + (1024 / BN) * i;
+        rb[i] = (n0 + nq < p.N) ? *(const float4*)(p.rhs + toff + (c0 + kr) * p.rhsI + n0 + nq) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    } else if (BMODE == 2) {
+      const int kq = (tid & 3) * 4;
+      const int toff = rhsTapOffset(p, k0, k1);
+#pragma unroll
+      for (int i = 0; i < NB4; ++i) {
+        int n = n0 + (tid >> 2) + 64 * i;
+        rb[i] = n < p.N ? *(const float4*)(p.rhs + toff + n * p.rhsO + c0 + kq) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NBS; ++i) {
+        int e = tid + 256 * i;
+        int n = n0 + e % BN, k = e / BN;
+        int kk0 = k0, kk1 = k1, c = c0 + k;
+        bool ok = n < p.N;
+        if (KFLAT) {
+          int kf = kt * BK + k;
+          ok = ok && kf < p.K;
+          int t = kf / p.C;
+          c = kf - t * p.C;
+          kk0 = t / p.k1n;
+          kk1 = t - kk0 * p.k1n;
+        }
+        rbs[i] = ok ? p.rhs[rhsTapOffset(p, kk0, kk1) + c * p.rhsI + n * p.rhsO] : 0.f;
+      }
+    }
+  };
+
+  auto storeTile = [&]() {
+    if (AMODE == 1) {
+      const int kq = (tid & 3) * 4;
+#pragma unroll
+      for (int i = 0; i < NA4; ++i) {
+        int m = (tid >> 2) + 64 * i;
+        As[kq + 0][m] = ra[i].x; As[kq + 1][m] = ra[i].y; As[kq + 2][m] = ra[i].z; As[kq + 3][m] = ra[i].w;
+      }
+    } else if (AMODE == 2) {
+#pragma unroll
+      for (int i = 0; i < NA4; ++i) {
+        int kr = tid / (BM / 4) + (1024 / BM) * i;
+        *(float4*)&As[kr][4 * (tid % (BM / 4))] = ra[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NAS; ++i) { int e = tid + 256 * i; As[e % BK][e / BK] = ras[i]; }
+    }
+    if (BMODE == 1) {
+#pragma unroll
+      for (int i = 0; i < NB4; ++i) {
+        int kr = tid / (BN / 4) + (1024 / BN) * i;
+        *(float4*)&Bs[kr][4 * (tid % (BN / 4))] = rb[i];
+      }
+    } else if (BMODE == 2) {
+      const int kq = (tid & 3) * 4;
+#pragma unroll
+      for (int i = 0; i < NB4; ++i) {
+        int n = (tid >> 2) + 64 * i;
+        Bs[kq + 0][n] = rb[i].x; Bs[kq + 1][n] = rb[i].y; Bs[kq + 2][n] = rb[i].z; Bs[kq + 3][n] = rb[i].w;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NBS; ++i) { int e = tid + 256 * i; Bs[e / BN][e % BN] = rbs[i]; }
+    }
+  };
+
+  float16v acc[TM][TN];
+#pragma unroll
+  for (int a = 0; a < TM; ++a)
+#pragma unroll
+    for (int b = 0; b < TN; ++b) acc[a][b] = (float16v){0};
+
+  if (ktBegin < ktEnd) {
+    loadTile(ktBegin);
+    storeTile();
+    __syncthreads();
+    for (int kt = ktBegin; kt < ktEnd; ++kt) {
+      const bool more = kt + 1 < ktEnd;
+      if (more) loadTile(kt + 1);
+      const int kh = lane >> 5, col = lane & 31;
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += 2) {
+        float av[TM], bv[TN];
+#pragma unroll
+        for (int a = 0; a < TM; ++a) av[a] = As[kk + kh][wm * WM + a * 32 + col];
+#pragma unroll
+        for (int b = 0; b < TN; ++b) bv[b] = Bs[kk + kh][wn * WN + b * 32 + col];
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+          for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[a], bv[b], acc[a][b], 0, 0, 0);
+      }
+      __syncthreads();
+      if (more) {
+        storeTile();
+        __syncthreads();
+      }
+    }
+  }
+
+  // ---- epilogue
+  const bool partial = p.splitK > 1;
+#pragma unroll
+  for (int a = 0; a < TM; ++a) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int m = m0 + wm * WM + a * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
+      if (m >= p.M) continue;
+      long long rowOff;
+      if (partial) {
+        rowOff = ((long long)blockIdx.z * p.M + m) * p.N;
+      } else {
+        int b, o0, o1;
+        if (p.bFast) { b = m % p.Nb; int t = m / p.Nb; o1 = t % p.o1n; o0 = t / p.o1n; }
+        else { o1 = m % p.o1n; int t = m / p.o1n; o0 = t % p.o0n; b = t / p.o0n; }
+        rowOff = (long long)b * p.outB + (long long)o0 * p.outS0 + (long long)o1 * p.outS1;
+      }
+#pragma unroll
+      for (int b = 0; b < TN; ++b) {
+        const int n = n0 + wn * WN + b * 32 + (lane & 31);
+        if (n < p.N) p.out[rowOff + (partial ? n : n * p.outF)] = acc[a][b][j];
+      }
+    }
+  }
+}
+
+// out(m, n) = sum over splits of partial[s][m][n], in split order
+__global__ void __launch_bounds__(256) conv_fold_partials(const float* __restrict__ part, float* __restrict__ out, ConvP p) {
+  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  long long total = (long long)p.M * p.N;
+  if (i >= total) return;
+  int m = (int)(i / p.N), n = (int)(i - (long long)m * p.N);
+  float s = 0.f;
+  for (int z = 0; z < p.splitK; ++z) s += part[(long long)z * total + i];
+  int b, o0, o1;
+  if (p.bFast) { b = m % p.Nb; int t = m / p.Nb; o1 = t % p.o1n; o0 = t / p.o1n; }
+  else { o1 = m % p.o1n; int t = m / p.o1n; o0 = t % p.o0n; b = t / p.o0n; }
+  out[(long long)b * p.outB + (long long)o0 * p.outS0 + (long long)o1 * p.outS1 + (long long)n * p.outF] = s;
+}
+
+struct ConvChoice {
+  bool fast = false;
+  int amode = 0, bmode = 0, bm = 128, bn = 128, splitK = 1, tilesPerSplit = 0, kTiles = 0, cTiles = 0, bFast = 0;
+  bool kflat = false;
+};
+
+bool fitsInt(const mi355_conv_desc* d) {
+  long long lhs = d->N * d->batchGroups * d->C, rhs = d->C * d->O, out = d->N * d->O;
+  for (int k = 0; k < d->nsp; ++k) { lhs *= d->in[k]; rhs *= d->k[k]; out *= d->out[k]; }
+  return lhs < (1ll << 31) && rhs < (1ll << 31) && out < (1ll << 31);
+}
+
+ConvChoice choose(const mi355_conv_desc* d) {
+  ConvChoice c;
+  if (d->dtype != 0 || d->nsp > 2 || d->featureGroups != 1 || d->batchGroups != 1 || !fitsInt(d)) return c;
+  c.fast = true;
+  long long M = d->N, K = d->C;
+  for (int k = 0; k < d->nsp; ++k) { M *= d->out[k]; K *= d->k[k]; }
+  long long N = d->O;
+  bool chunk = d->C % BK == 0;
+  auto mult4 = [](long long x) { return x % 4 == 0; };
+  long long s0 = d->nsp > 0 ? d->lhsS[0] : 0, s1 = d->nsp > 1 ? d->lhsS[1] : 0;
+  long long r0 = d->nsp > 0 ? d->rhsS[0] : 0, r1 = d->nsp > 1 ? d->rhsS[1] : 0;
+  if (chunk && d->lhsF == 1 && mult4(d->lhsB) && mult4(s0) && mult4(s1)) c.amode = 1;
+  else if (chunk && d->lhsB == 1 && d->N % 4 == 0 && mult4(d->lhsF) && mult4(s0) && mult4(s1)) { c.amode = 2; c.bFast = 1; }
+  if (chunk && d->rhsO == 1 && N % 4 == 0 && mult4(d->rhsI) && mult4(r0) && mult4(r1)) c.bmode = 1;
+  else if (chunk && d->rhsI == 1 && mult4(d->rhsO) && mult4(r0) && mult4(r1)) c.bmode = 2;
+  c.kflat = !chunk;
+  long long taps = 1;
+  for (int k = 0; k < d->nsp; ++k) taps *= d->k[k];
+  c.cTiles = chunk ? (int)(d->C / BK) : 1;
+  c.kTiles = chunk ? (int)(taps * c.cTiles) : (int)((K + BK - 1) / BK);
+  long long t128 = ((M + 127) / 128) * ((N + 127) / 128);
+  if (t128 >= 384 && N >= 96) { c.bm = 128; c.bn = 128; }
+  else { c.bm = 64; c.bn = 64; }
+  long long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+  int split = 1;
+  if (tiles < 512) split = (int)std::min<long long>((1024 + tiles - 1) / tiles, std::max(1, c.kTiles / 8));
+  split = std::max(1, std::min(split, 256));
+  c.tilesPerSplit = (c.kTiles + split - 1) / split;
+  c.splitK = (c.kTiles + c.tilesPerSplit - 1) / c.tilesPerSplit;
+  return c;
+}
+
+template <int BM, int BN>
+void launchIgemm(const ConvChoice& c, const ConvP& p, dim3 grid, hipStream_t st) {
+#define CASE(A, B, F) conv_igemm_f32<BM, BN, A, B, F><<<grid, 256, 0, st>>>(p)
+  if (c.kflat) { CASE(0, 0, true); return; }
+  switch (c.amode * 3 + c.bmode) {
+    case 0: CASE(0, 0, false); break;
+    case 1: CASE(0, 1, false); break;
+    case 2: CASE(0, 2, false); break;
+    case 3: CASE(1, 0, false); break;
+    case 4: CASE(1, 1, false); break;
+    case 5: CASE(1, 2, false); break;
+    case 6: CASE(2, 0, false); break;
+    case 7: CASE(2, 1, false); break;
+    case 8: CASE(2, 2, false); break;
+  }
+#undef CASE
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t mi355_conv_workspace_bytes(const mi355_conv_desc* d) {
+  ConvChoice c = choose(d);
+  if (!c.fast || c.splitK <= 1) return 0;
+  long long M = d->N;
+  for (int k = 0; k < d->nsp; ++k) M *= d->out[k];
+  return (size_t)c.splitK * (size_t)M * (size_t)d->O * sizeof(float);
+}
+
+int mi355_conv_direct(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, mi355_stream_t s);
+
+int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes,
+               mi355_stream_t s) {
+  ConvChoice c = choose(d);
+  if (!c.fast) return mi355_conv_direct(d, lhs, rhs, out, s);
+  ConvP p;
+  p.lhs = (const float*)lhs;
+  p.rhs = (const float*)rhs;
+  long long M = d->N, K = d->C;
+  for (int k = 0; k < d->nsp; ++k) { M *= d->out[k]; K *= d->k[k]; }
+  if (M <= 0 || d->O <= 0) return 0;
+  p.M = (int)M; p.N = (int)d->O; p.K = (int)K;
+  p.Nb = (int)d->N; p.C = (int)d->C;
+  auto dim = [&](const int64_t* a, int k, int64_t dflt) { return k < d->nsp ? (int)a[k] : (int)dflt; };
+  p.in0 = dim(d->in, 0, 1); p.in1 = dim(d->in, 1, 1);
+  p.k0n = dim(d->k, 0, 1); p.k1n = dim(d->k, 1, 1);
+  p.o0n = dim(d->out, 0, 1); p.o1n = dim(d->out, 1, 1);
+  p.s0 = dim(d->stride, 0, 1); p.s1 = dim(d->stride, 1, 1);
+  p.p0 = dim(d->padLo, 0, 0); p.p1 = dim(d->padLo, 1, 0);
+  p.ld0 = dim(d->ldil, 0, 1); p.ld1 = dim(d->ldil, 1, 1);
+  p.rd0 = dim(d->rdil, 0, 1); p.rd1 = dim(d->rdil, 1, 1);
+  p.rev0 = dim(d->rev, 0, 0); p.rev1 = dim(d->rev, 1, 0);
+  p.lhsB = (int)d->lhsB; p.lhsF = (int)d->lhsF; p.lhsS0 = dim(d->lhsS, 0, 0); p.lhsS1 = dim(d->lhsS, 1, 0);
+  p.rhsI = (int)d->rhsI; p.rhsO = (int)d->rhsO; p.rhsS0 = dim(d->rhsS, 0, 0); p.rhsS1 = dim(d->rhsS, 1, 0);
+  p.outB = (int)d->outB; p.outF = (int)d->outF; p.outS0 = dim(d->outS, 0, 0); p.outS1 = dim(d->outS, 1, 0);
+  p.bFast = c.bFast;
+  p.cTiles = c.cTiles; p.kTiles = c.kTiles; p.splitK = c.splitK; p.tilesPerSplit = c.tilesPerSplit;
+  if (c.splitK > 1) {
+    size_t need = (size_t)c.splitK * (size_t)M * (size_t)d->O * sizeof(float);
+    if (!workspace || workspace_bytes < need) return 3;   // caller sized the workspace wrong
+    p.out = (float*)workspace;
+  } else {
+    p.out = (float*)out;
+  }
+  hipStream_t st = (hipStream_t)s;
+  dim3 grid((unsigned)((p.M + c.bm - 1) / c.bm), (unsigned)((p.N + c.bn - 1) / c.bn), (unsigned)c.splitK);
+  if (grid.y > 65535) return 4;
+  if (c.bm == 128) launchIgemm<128, 128>(c, p, grid, st);
+  else launchIgemm<64, 64>(c, p, grid, st);
+  if (c.splitK > 1) {
+    long long total = M * d->O;
+    conv_fold_partials<<<(unsigned)((total + 255) / 256), 256, 0, st>>>((const float*)workspace, (float*)out, p);
+  }
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : (int)e;
+}
+
+}  // extern "C"

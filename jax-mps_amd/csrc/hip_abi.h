@@ -71,6 +71,7 @@ typedef struct {
 int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace,
                size_t workspace_bytes, mi355_stream_t s);
 size_t mi355_conv_workspace_bytes(const mi355_conv_desc* d);
+int mi355_conv_direct(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, mi355_stream_t s);
 
 typedef struct {
   int64_t numUpdates, rowElems, operandRows;

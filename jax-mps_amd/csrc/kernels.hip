@@ -416,15 +416,8 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
   return check("gemm");
 }
 
-size_t mi355_conv_workspace_bytes(const mi355_conv_desc* d) {
-  (void)d;
-  return 0;
-}
-
-int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes,
-               mi355_stream_t s) {
-  (void)workspace;
-  (void)workspace_bytes;
+// Direct convolution: the general fallback behind mi355_conv (groups, 3-d windows, bf16).
+int mi355_conv_direct(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, mi355_stream_t s) {
   ConvArgs a;
   a.d = *d;
   a.lhs = lhs; a.rhs = rhs; a.out = out;

@@ -11,6 +11,7 @@
 #include <unordered_map>
 #include <vector>
 
+#include "hip_abi.h"
 #include "ir.h"
 
 namespace mi355 {
@@ -112,5 +113,7 @@ struct CompiledProgram {
 
 // planner.cc
 std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module);
+int abiDtypeCode(DType d);   // element type code of the C-ABI kernel entry points (-1: not supported there)
+mi355_conv_desc toAbi(const ConvDesc& c);
 
 }  // namespace mi355

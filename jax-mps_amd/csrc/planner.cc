@@ -10,6 +10,7 @@
 // (bias-add, softmax, LayerNorm, RMSNorm: src/pjrt_plugin/passes/*.cc) plus
 // whatever else is elementwise; nothing here is pattern-matched by name.
 #include <algorithm>
+#include <cstring>
 #include <functional>
 #include <set>
 #include <sstream>
@@ -444,7 +445,7 @@ class Planner {
     std::sort(order.begin(), order.end(), [&](size_t x, size_t y) { return ast[ac[x]] > ast[ac[y]]; });
     std::vector<int64_t> acs, bcs;
     for (auto k : order) { acs.push_back(ac[k]); bcs.push_back(bc[k]); }
-    int64_t Ka, Kb, M, N;
+    int64_t Ka = 0, Kb = 0, M = 0, N = 0;
     bool ok = mergeDims(a->type, acs, Ka, g.aCol) && mergeDims(b->type, bcs, Kb, g.bRow) &&
               mergeDims(a->type, af, M, g.aRow) && mergeDims(b->type, bf, N, g.bCol);
     g.M = M; g.N = N; g.K = Ka;
@@ -527,10 +528,12 @@ class Planner {
     s.kind = Step::Conv;
     s.label = "convolution " + lhs->type.str() + " * " + rhs->type.str();
     s.conv = c;
-    // split-K workspace for shapes with few output tiles (filter gradients)
-    int64_t ws = 0;
-    s.workspaceBytes = ws;
     s.args = {ref(storageOf(lhs), t), ref(storageOf(rhs), t), ref(sid, t)};
+    // split-K partial sums for shapes with few output tiles (filter gradients, late stages)
+    mi355_conv_desc abi = toAbi(c);
+    int64_t ws = ((int64_t)mi355_conv_workspace_bytes(&abi) + kAlign - 1) / kAlign * kAlign;
+    s.workspaceBytes = ws;
+    if (ws > 0) s.args.push_back(ref(newStorage((size_t)ws), t));
     plan.steps.push_back(std::move(s));
   }
 
@@ -887,6 +890,31 @@ class Planner {
 };
 
 }  // namespace
+
+int abiDtypeCode(DType d) {
+  switch (d) {
+    case DType::F32: return 0;
+    case DType::BF16: return 1;
+    case DType::S32: return 2;
+    case DType::U32: return 3;
+    default: return -1;
+  }
+}
+
+mi355_conv_desc toAbi(const ConvDesc& c) {
+  mi355_conv_desc d;
+  memset(&d, 0, sizeof d);
+  d.nsp = c.nsp; d.N = c.N; d.C = c.C; d.O = c.O;
+  for (int k = 0; k < 3; ++k) {
+    d.in[k] = c.in[k]; d.k[k] = c.k[k]; d.out[k] = c.out[k]; d.stride[k] = c.stride[k]; d.padLo[k] = c.padLo[k];
+    d.ldil[k] = c.ldil[k]; d.rdil[k] = c.rdil[k]; d.rev[k] = c.rev[k];
+    d.lhsS[k] = c.lhsS[k]; d.rhsS[k] = c.rhsS[k]; d.outS[k] = c.outS[k];
+  }
+  d.featureGroups = c.featureGroups; d.batchGroups = c.batchGroups;
+  d.lhsB = c.lhsB; d.lhsF = c.lhsF; d.rhsI = c.rhsI; d.rhsO = c.rhsO; d.outB = c.outB; d.outF = c.outF;
+  d.dtype = abiDtypeCode(c.type);
+  return d;
+}
 
 std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) {
   auto prog = std::make_unique<CompiledProgram>();

@@ -316,15 +316,7 @@ std::map<std::string, KindStat> Executable::timings() {
   return stats_;
 }
 
-static int dtypeCode(DType d) {
-  switch (d) {
-    case DType::F32: return 0;
-    case DType::BF16: return 1;
-    case DType::S32: return 2;
-    case DType::U32: return 3;
-    default: return -1;
-  }
-}
+static int dtypeCode(DType d) { return abiDtypeCode(d); }
 
 void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
   Device& dev = Device::get();
@@ -346,6 +338,8 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
     default: break;
   }
   bool doTime = !kind.empty() && timed(kind);
+  static const bool detail = getenv("MI355X_TIMING_DETAIL") != nullptr;   // one statistics row per step label
+  if (doTime && detail) kind += ":" + s.label;
   mi355_event_t ea = nullptr, eb = nullptr;
   if (doTime) {
     ea = getEvent();
@@ -374,18 +368,7 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       break;
     }
     case Step::Conv: {
-      mi355_conv_desc d;
-      memset(&d, 0, sizeof d);
-      const ConvDesc& c = s.conv;
-      d.nsp = c.nsp; d.N = c.N; d.C = c.C; d.O = c.O;
-      for (int k = 0; k < 3; ++k) {
-        d.in[k] = c.in[k]; d.k[k] = c.k[k]; d.out[k] = c.out[k]; d.stride[k] = c.stride[k]; d.padLo[k] = c.padLo[k];
-        d.ldil[k] = c.ldil[k]; d.rdil[k] = c.rdil[k]; d.rev[k] = c.rev[k];
-        d.lhsS[k] = c.lhsS[k]; d.rhsS[k] = c.rhsS[k]; d.outS[k] = c.outS[k];
-      }
-      d.featureGroups = c.featureGroups; d.batchGroups = c.batchGroups;
-      d.lhsB = c.lhsB; d.lhsF = c.lhsF; d.rhsI = c.rhsI; d.rhsO = c.rhsO; d.outB = c.outB; d.outF = c.outF;
-      d.dtype = dtypeCode(c.type);
+      mi355_conv_desc d = toAbi(s.conv);
       void* ws = s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
       check(mi355_conv(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), ws,
                        (size_t)s.workspaceBytes, st), "convolution");

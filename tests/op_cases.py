@@ -242,6 +242,17 @@ case("conv-wgrad-form", lambda b, x, g: b.conv(x, g, strides=(1, 1), padding=((1
      u(236, 4, 16, 16, 24), u(237, 4, 8, 8, 40))
 case("conv-dgrad-form", lambda b, g, w: b.conv(g, b.reverse(w, [0, 1]), strides=(1, 1), padding=((1, 2), (1, 2)), lhs_dilation=(2, 2), dn=("b01f", "01oi", "b01f")),
      u(238, 4, 8, 8, 40), u(239, 3, 3, 24, 40))
+# shapes that reach the vectorised tile loaders and the split-K path of the implicit-GEMM kernel
+case("conv-fwd-vector-loaders", _conv(padding=((1, 1), (1, 1))), u(242, 8, 12, 12, 32), u(243, 3, 3, 32, 64))
+case("conv-fwd-stride2-vector", _conv(strides=(2, 2), padding=((0, 1), (0, 1))), u(244, 8, 12, 12, 32), u(245, 3, 3, 32, 64))
+case("conv-fwd-128-tile", _conv(padding=((1, 1), (1, 1))), u(246, 16, 32, 32, 16), u(247, 3, 3, 16, 128))
+case("conv-dgrad-vector", lambda b, g, w: b.conv(g, b.reverse(w, [0, 1]), strides=(1, 1), padding=((1, 2), (1, 2)), lhs_dilation=(2, 2), dn=("b01f", "01oi", "b01f")),
+     u(248, 8, 6, 6, 64), u(249, 3, 3, 32, 64))
+case("conv-wgrad-vector", lambda b, x, g: b.conv(x, g, strides=(1, 1), padding=((0, 1), (0, 1)), rhs_dilation=(2, 2), dn=("f01b", "i01o", "01bf")),
+     u(250, 16, 12, 12, 8), u(251, 16, 6, 6, 32))
+case("conv-wgrad-stride1-vector", lambda b, x, g: b.conv(x, g, strides=(1, 1), padding=((1, 1), (1, 1)), dn=("f01b", "i01o", "01bf")),
+     u(252, 32, 8, 8, 64), u(253, 32, 8, 8, 64))
+case("conv-1x1-stride2-vector", _conv(strides=(2, 2)), u(254, 8, 8, 8, 64), u(255, 1, 1, 64, 128))
 case("conv-bf16", _conv(padding=((1, 1), (1, 1))), u(240, 2, 8, 8, 16), u(241, 3, 3, 16, 8), dtypes=["bf16", "bf16"])
 
 # ------------------------------------------------------------------ reduce (tests/configs/reduction.py:8-39)
