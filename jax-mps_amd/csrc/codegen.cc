@@ -30,12 +30,8 @@ typedef unsigned short u16; typedef unsigned int u32; typedef unsigned long long
 typedef signed char i8; typedef unsigned char u8; typedef short i16;
 template <typename T, int N> struct __attribute__((aligned(sizeof(T) * N))) Vec { T e[N]; };
 __device__ __forceinline__ float bf2f(u16 b) { return __uint_as_float(((u32)b) << 16); }
-__device__ __forceinline__ u16 f2bf(float f) {
-  u32 u = __float_as_uint(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u16)((u >> 16) | 0x40);
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return (u16)(u >> 16);
-}
+// gfx950 rounds f32 -> bf16 (nearest even, NaN stays NaN) in one instruction
+__device__ __forceinline__ u16 f2bf(float f) { return __builtin_bit_cast(u16, (__bf16)f); }
 __device__ __forceinline__ float bfr(float f) { return bf2f(f2bf(f)); }
 __device__ __forceinline__ float hfr(float f) { return (float)(_Float16)f; }
 template <typename T> __device__ __forceinline__ T mx(T a, T b) { return (a > b || a != a) ? a : b; }
@@ -58,6 +54,16 @@ template <typename T> __device__ __forceinline__ T ipow(T a, T b) {
 }
 template <typename T> __device__ __forceinline__ T idiv(T a, T b) { return b == (T)0 ? (T)-1 : ((b == (T)-1) ? (T)(0 - a) : (T)(a / b)); }
 template <typename T> __device__ __forceinline__ T irem(T a, T b) { return b == (T)0 ? a : ((b == (T)-1) ? (T)0 : (T)(a % b)); }
+// 16-bit results keep 8 (bf16) or 11 (f16) significand bits: the hardware exponential is exact enough there
+__device__ __forceinline__ float tanh_fast(float x) { float t = __expf(-2.f * fabsf(x)); return copysignf((1.f - t) / (1.f + t), x); }
+// f32 tanh to a few ulp: odd polynomial near 0 (where 1 - exp cancels), exponential form elsewhere
+__device__ __forceinline__ float tanh_f32(float x) {
+  float ax = fabsf(x), x2 = x * x;
+  float p = x * (1.f + x2 * (-0.33333334f + x2 * (0.13333334f + x2 * (-0.05396825f + x2 * (0.021869488f + x2 * -0.008863236f)))));
+  float t = __expf(-2.f * ax);
+  float r = copysignf(__fdividef(1.f - t, 1.f + t), x);
+  return ax < 0.3f ? p : r;
+}
 __device__ __forceinline__ float sgnf(float x) { return (x != x || x == 0.f) ? x : (x > 0.f ? 1.f : -1.f); }
 __device__ __forceinline__ double sgnd(double x) { return (x != x || x == 0.0) ? x : (x > 0.0 ? 1.0 : -1.0); }
 __device__ __forceinline__ int tokey(float f) { int i = __float_as_int(f); return i < 0 ? (i ^ 0x7FFFFFFF) : i; }
@@ -692,6 +698,11 @@ class Emitter {
     if (n == "not") return bin(isP ? "(!" + in(0) + ")" : "(" + T + ")(~" + in(0) + ")");
     if (n == "sign") return bin(isF ? (isD ? "sgnd(" : "sgnf(") + in(0) + ")" : "(" + T + ")((" + in(0) + " > 0) - (" + in(0) + " < 0))");
     if (n == "is_finite") return bin("isfinite(" + in(0) + ")");
+    const bool half = rt.dt == DType::BF16 || rt.dt == DType::F16;
+    if (half && n == "tanh") return bin("tanh_fast(" + in(0) + ")");
+    if (half && n == "exponential") return bin("__expf(" + in(0) + ")");
+    if (rt.dt == DType::F32 && n == "tanh") return bin("tanh_f32(" + in(0) + ")");
+    if (half && n == "logistic") return bin("(1.f / (1.f + __expf(-" + in(0) + ")))");
     if (n == "logistic") return bin(isD ? "(1.0 / (1.0 + exp(-" + in(0) + ")))" : "(1.f / (1.f + expf(-" + in(0) + ")))");
     if (n == "rsqrt") return bin(isD ? "(1.0 / sqrt(" + in(0) + "))" : "(1.f / sqrtf(" + in(0) + "))");
     if (n == "popcnt") return bin(dtypeSize(rt.dt) == 8 ? "(" + T + ")__popcll((u64)" + in(0) + ")" : "(" + T + ")__popc((u32)(" + std::string(dtypeSize(rt.dt) == 4 ? "u32" : dtypeSize(rt.dt) == 2 ? "u16" : "u8") + ")" + in(0) + ")");
@@ -1052,18 +1063,33 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     for (size_t j = 0; j < nr; ++j) outs.push_back("const " + ops[j].accT + "* __restrict__ part" + std::to_string(j));
     for (size_t j = 0; j < nr; ++j) outs.push_back(storageT(ops[j].dt) + "* __restrict__ out" + std::to_string(j));
     s << kernelHeader(em.leaves_, outs) << " {\n";
-    s << "  const " << IT << " kk = (" << IT << ")blockIdx.x * 256 + threadIdx.x;\n  if (kk >= " << Kn << ") return;\n";
+    // many partials per output: one wavefront folds an output (lanes stride over the
+    // partials, then a butterfly); few partials: one lane per output
+    const bool wavePerOut = P >= 16;
+    if (wavePerOut) {
+      s << "  const int lane = threadIdx.x & 63;\n";
+      s << "  const " << IT << " kk = (" << IT << ")blockIdx.x * 4 + (threadIdx.x >> 6);\n  if (kk >= " << Kn << ") return;\n";
+    } else {
+      s << "  const " << IT << " kk = (" << IT << ")blockIdx.x * 256 + threadIdx.x;\n  if (kk >= " << Kn << ") return;\n";
+    }
     s << em.pre_;
     for (size_t j = 0; j < nr; ++j) {
+      std::string part = "part" + std::to_string(j) + "[p * " + std::to_string(Kn) + " + kk]";
       s << "  { " << ops[j].accT << " a = " << ops[j].identity << ";\n";
-      s << "    for (" << IT << " p = 0; p < " << P << "; ++p) a = " << ops[j].combine("a", "part" + std::to_string(j) + "[p * " + std::to_string(Kn) + " + kk]") << ";\n";
+      if (wavePerOut) {
+        s << "    #pragma unroll 4\n    for (" << IT << " p = lane; p < " << P << "; p += 64) a = " << ops[j].combine("a", part) << ";\n";
+        s << "    #pragma unroll\n    for (int o = 32; o > 0; o >>= 1) a = " << ops[j].combine("a", shflXor(ops[j].accT, "a", "o")) << ";\n";
+        s << "    if (lane == 0) {\n";
+      } else {
+        s << "    for (" << IT << " p = 0; p < " << P << "; ++p) a = " << ops[j].combine("a", part) << ";\n    {\n";
+      }
       s << "    a = " << ops[j].combine(inits[j], "a") << ";\n";
-      s << "    out" << j << "[kk] = " << storeExpr(ops[j].dt, roundTo(ops[j].dt, "a")) << "; }\n";
+      s << "    out" << j << "[kk] = " << storeExpr(ops[j].dt, roundTo(ops[j].dt, "a")) << "; } }\n";
     }
     s << "}\n";
     Launch l;
     l.source = s.str();
-    l.grid[0] = (unsigned)((Kn + 255) / 256);
+    l.grid[0] = (unsigned)(wavePerOut ? (Kn + 3) / 4 : (Kn + 255) / 256);
     l.block[0] = 256;
     for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
     for (size_t j = 0; j < nr; ++j) { KArg a; a.kind = KArg::Work; a.workOffset = workOff[j]; l.args.push_back(a); }
@@ -1135,7 +1161,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     }
     s << em.pre_;
     for (size_t j = 0; j < nr; ++j) s << "  " << ops[j].accT << " acc" << j << " = " << ops[j].identity << ";\n";
-    s << "  for (" << IT << " rv = r_begin + r_tid; rv < r_end; rv += r_step) {\n";
+    s << "  #pragma unroll 4\n  for (" << IT << " rv = r_begin + r_tid; rv < r_end; rv += r_step) {\n";
     s << "    const " << IT << " rb = rv * " << V << ";\n";
     s << loopPre;
     s << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n";
@@ -1251,7 +1277,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   }
   s << "  if (active) {\n";
   s << em.pre_;
-  s << "  for (" << IT << " rr = r_begin + ty; rr < r_end; rr += " << TY << ") {\n";
+  s << "  #pragma unroll 4\n  for (" << IT << " rr = r_begin + ty; rr < r_end; rr += " << TY << ") {\n";
   s << loopPre;
   s << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n";
   s << em.body_.front();

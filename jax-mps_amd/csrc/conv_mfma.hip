@@ -25,6 +25,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <cstdlib>
 
 #include "hip_abi.h"
 
@@ -87,8 +88,11 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int NA4 = BM / 64, NB4 = BN / 64;            // float4 per thread per tile (vector loaders)
   constexpr int NAS = BM * BK / 256, NBS = BN * BK / 256; // floats per thread per tile (scalar loaders)
-  __shared__ float As[BK][BM + 4];
-  __shared__ float Bs[BK][BN + 4];
+  // k-major tiles, two stages.  Row padding: 2 floats make the transposing (K-vector) stores
+  // conflict-free, 4 floats keep the float4 stores of the M/N-vector loaders 16-byte aligned.
+  constexpr int PA = AMODE == 1 ? 2 : 4, PB = BMODE == 2 ? 2 : 4;
+  __shared__ __attribute__((aligned(16))) float As[2][BK][BM + PA];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BK][BN + PB];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -114,118 +118,138 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
   float4 rb[NB4 > 0 ? NB4 : 1];
   float ras[NAS], rbs[NBS];
 
+  // Position of the next k-tile to fetch, advanced incrementally (no divisions in the loop):
+  // window tap (nk0, nk1) and first input feature nc.  Row offsets and validity only change
+  // when the tap changes, so they are cached per tap.
+  int nk0 = 0, nk1 = 0, nc = 0;
+  if (!KFLAT) {
+    int tap = ktBegin / p.cTiles;
+    nc = (ktBegin - tap * p.cTiles) * BK;
+    nk0 = tap / p.k1n;
+    nk1 = tap - nk0 * p.k1n;
+  }
+  constexpr int NROW = AMODE == 0 ? NAS : (AMODE == 1 ? NA4 : 1);
+  int offA[NROW];
+  int toffB = 0;
+  auto newTap = [&]() {
+    if (KFLAT) return;
+#pragma unroll
+    for (int i = 0; i < NROW; ++i) offA[i] = tapOffset(p, rowsA[i], nk0, nk1);
+    toffB = rhsTapOffset(p, nk0, nk1);
+  };
+  newTap();
+  // per-thread constants of the loaders
+  const int aKq = (tid & 3) * 4;
+  const int aKr = tid / (BM / 4);
+  const int bNq = 4 * (tid % (BN / 4));
+  const int bKr = tid / (BN / 4);
+  const bool bNok = n0 + bNq < p.N;
+
   auto loadTile = [&](int kt) {
-    int tap = 0, c0 = 0, k0 = 0, k1 = 0;
-    if (!KFLAT) {
-      tap = kt / p.cTiles;
-      c0 = (kt - tap * p.cTiles) * BK;
-      k0 = tap / p.k1n;
-      k1 = tap - k0 * p.k1n;
-    }
     // ---------------- A
     if (AMODE == 1) {
-      const int kq = (tid & 3) * 4;
 #pragma unroll
-      for (int i = 0; i < NA4; ++i) {
-        int off = tapOffset(p, rowsA[i], k0, k1);
-        ra[i] = off >= 0 ? *(const float4*)(p.lhs + off + c0 + kq) : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
+      for (int i = 0; i < NA4; ++i)
+        ra[i] = offA[i] >= 0 ? *(const float4*)(p.lhs + (unsigned)(offA[i] + nc + aKq)) : make_float4(0.f, 0.f, 0.f, 0.f);
     } else if (AMODE == 2) {
-      int off = tapOffset(p, rowsA[0], k0, k1);
 #pragma unroll
       for (int i = 0; i < NA4; ++i) {
-        int kr = tid / (BM / 4) + (1024 / BM) * i;
-        ra[i] = off >= 0 ? *(const float4*)(p.lhs + off + (c0 + kr) * p.lhsF) : make_float4(0.f, 0.f, 0.f, 0.f);
+        int kr = aKr + (1024 / BM) * i;
+        ra[i] = offA[0] >= 0 ? *(const float4*)(p.lhs + (unsigned)(offA[0] + (nc + kr) * p.lhsF)) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
     } else {
 #pragma unroll
       for (int i = 0; i < NAS; ++i) {
         int k = (tid + 256 * i) % BK;
-        int kk0 = k0, kk1 = k1, c = c0 + k;
-        bool ok = true;
+        int off, c = nc + k;
         if (KFLAT) {
           int kf = kt * BK + k;
-          ok = kf < p.K;
           int t = kf / p.C;
           c = kf - t * p.C;
-          kk0 = t / p.k1n;
-          kk1 = t - kk0 * p.k1n;
+          int kk0 = t / p.k1n;
+          off = kf < p.K ? tapOffset(p, rowsA[i], kk0, t - kk0 * p.k1n) : -1;
+        } else {
+          off = offA[i];
         }
-        int off = ok ? tapOffset(p, rowsA[i], kk0, kk1) : -1;
         ras[i] = off >= 0 ? p.lhs[off + c * p.lhsF] : 0.f;
       }
     }
     // ---------------- B
     if (BMODE == 1) {
-      const int nq = 4 * (tid % (BN / 4));
-      const int toff = rhsTapOffset(p, k0, k1);
 #pragma unroll
       for (int i = 0; i < NB4; ++i) {
-        int kr = tid / (BN / 4) + (1024 / BN) * i;
-        rb[i] = (n0 + nq < p.N) ? *(const float4*)(p.rhs + toff + (c0 + kr) * p.rhsI + n0 + nq) : make_float4(0.f, 0.f, 0.f, 0.f);
+        int kr = bKr + (1024 / BN) * i;
+        rb[i] = bNok ? *(const float4*)(p.rhs + (unsigned)(toffB + (nc + kr) * p.rhsI + n0 + bNq)) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
     } else if (BMODE == 2) {
-      const int kq = (tid & 3) * 4;
-      const int toff = rhsTapOffset(p, k0, k1);
 #pragma unroll
       for (int i = 0; i < NB4; ++i) {
         int n = n0 + (tid >> 2) + 64 * i;
-        rb[i] = n < p.N ? *(const float4*)(p.rhs + toff + n * p.rhsO + c0 + kq) : make_float4(0.f, 0.f, 0.f, 0.f);
+        rb[i] = n < p.N ? *(const float4*)(p.rhs + (unsigned)(toffB + n * p.rhsO + nc + aKq)) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
     } else {
 #pragma unroll
       for (int i = 0; i < NBS; ++i) {
         int e = tid + 256 * i;
         int n = n0 + e % BN, k = e / BN;
-        int kk0 = k0, kk1 = k1, c = c0 + k;
+        int c = nc + k, toff = toffB;
         bool ok = n < p.N;
         if (KFLAT) {
           int kf = kt * BK + k;
           ok = ok && kf < p.K;
           int t = kf / p.C;
           c = kf - t * p.C;
-          kk0 = t / p.k1n;
-          kk1 = t - kk0 * p.k1n;
+          int kk0 = t / p.k1n;
+          toff = rhsTapOffset(p, kk0, t - kk0 * p.k1n);
         }
-        rbs[i] = ok ? p.rhs[rhsTapOffset(p, kk0, kk1) + c * p.rhsI + n * p.rhsO] : 0.f;
+        rbs[i] = ok ? p.rhs[toff + c * p.rhsI + n * p.rhsO] : 0.f;
+      }
+    }
+    // ---------------- advance to the following tile
+    if (!KFLAT) {
+      nc += BK;
+      if (nc >= p.C) {
+        nc = 0;
+        if (++nk1 == p.k1n) { nk1 = 0; ++nk0; }
+        newTap();
       }
     }
   };
 
-  auto storeTile = [&]() {
+  auto storeTile = [&](int st) {
     if (AMODE == 1) {
       const int kq = (tid & 3) * 4;
 #pragma unroll
       for (int i = 0; i < NA4; ++i) {
         int m = (tid >> 2) + 64 * i;
-        As[kq + 0][m] = ra[i].x; As[kq + 1][m] = ra[i].y; As[kq + 2][m] = ra[i].z; As[kq + 3][m] = ra[i].w;
+        As[st][kq + 0][m] = ra[i].x; As[st][kq + 1][m] = ra[i].y; As[st][kq + 2][m] = ra[i].z; As[st][kq + 3][m] = ra[i].w;
       }
     } else if (AMODE == 2) {
 #pragma unroll
       for (int i = 0; i < NA4; ++i) {
         int kr = tid / (BM / 4) + (1024 / BM) * i;
-        *(float4*)&As[kr][4 * (tid % (BM / 4))] = ra[i];
+        *(float4*)&As[st][kr][4 * (tid % (BM / 4))] = ra[i];
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < NAS; ++i) { int e = tid + 256 * i; As[e % BK][e / BK] = ras[i]; }
+      for (int i = 0; i < NAS; ++i) { int e = tid + 256 * i; As[st][e % BK][e / BK] = ras[i]; }
     }
     if (BMODE == 1) {
 #pragma unroll
       for (int i = 0; i < NB4; ++i) {
         int kr = tid / (BN / 4) + (1024 / BN) * i;
-        *(float4*)&Bs[kr][4 * (tid % (BN / 4))] = rb[i];
+        *(float4*)&Bs[st][kr][4 * (tid % (BN / 4))] = rb[i];
       }
     } else if (BMODE == 2) {
       const int kq = (tid & 3) * 4;
 #pragma unroll
       for (int i = 0; i < NB4; ++i) {
         int n = (tid >> 2) + 64 * i;
-        Bs[kq + 0][n] = rb[i].x; Bs[kq + 1][n] = rb[i].y; Bs[kq + 2][n] = rb[i].z; Bs[kq + 3][n] = rb[i].w;
+        Bs[st][kq + 0][n] = rb[i].x; Bs[st][kq + 1][n] = rb[i].y; Bs[st][kq + 2][n] = rb[i].z; Bs[st][kq + 3][n] = rb[i].w;
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < NBS; ++i) { int e = tid + 256 * i; Bs[e / BN][e % BN] = rbs[i]; }
+      for (int i = 0; i < NBS; ++i) { int e = tid + 256 * i; Bs[st][e / BN][e % BN] = rbs[i]; }
     }
   };
 
@@ -237,29 +261,28 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
 
   if (ktBegin < ktEnd) {
     loadTile(ktBegin);
-    storeTile();
+    storeTile(0);
     __syncthreads();
+    int cur = 0;
+    const int kh = lane >> 5, col = lane & 31;
     for (int kt = ktBegin; kt < ktEnd; ++kt) {
       const bool more = kt + 1 < ktEnd;
-      if (more) loadTile(kt + 1);
-      const int kh = lane >> 5, col = lane & 31;
+      if (more) loadTile(kt + 1);          // global loads in flight while this tile is multiplied
 #pragma unroll
       for (int kk = 0; kk < BK; kk += 2) {
         float av[TM], bv[TN];
 #pragma unroll
-        for (int a = 0; a < TM; ++a) av[a] = As[kk + kh][wm * WM + a * 32 + col];
+        for (int a = 0; a < TM; ++a) av[a] = As[cur][kk + kh][wm * WM + a * 32 + col];
 #pragma unroll
-        for (int b = 0; b < TN; ++b) bv[b] = Bs[kk + kh][wn * WN + b * 32 + col];
+        for (int b = 0; b < TN; ++b) bv[b] = Bs[cur][kk + kh][wn * WN + b * 32 + col];
 #pragma unroll
         for (int a = 0; a < TM; ++a)
 #pragma unroll
           for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[a], bv[b], acc[a][b], 0, 0, 0);
       }
+      if (more) storeTile(cur ^ 1);         // the other stage: nobody reads it during this iteration
       __syncthreads();
-      if (more) {
-        storeTile();
-        __syncthreads();
-      }
+      cur ^= 1;
     }
   }
 
@@ -335,8 +358,11 @@ ConvChoice choose(const mi355_conv_desc* d) {
   for (int k = 0; k < d->nsp; ++k) taps *= d->k[k];
   c.cTiles = chunk ? (int)(d->C / BK) : 1;
   c.kTiles = chunk ? (int)(taps * c.cTiles) : (int)((K + BK - 1) / BK);
-  long long t128 = ((M + 127) / 128) * ((N + 127) / 128);
-  if (t128 >= 384 && N >= 96) { c.bm = 128; c.bn = 128; }
+  // largest tile that still gives every CU at least two workgroups
+  auto tilesOf = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  static const int forced = getenv("MI355X_CONV_TILE") ? atoi(getenv("MI355X_CONV_TILE")) : 0;
+  if (forced == 128 || (!forced && N >= 128 && tilesOf(128, 128) >= 512)) { c.bm = 128; c.bn = 128; }
+  else if (forced == 12864 || (!forced && tilesOf(128, 64) >= 512)) { c.bm = 128; c.bn = 64; }
   else { c.bm = 64; c.bn = 64; }
   long long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
   int split = 1;
@@ -415,7 +441,8 @@ int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void*
   hipStream_t st = (hipStream_t)s;
   dim3 grid((unsigned)((p.M + c.bm - 1) / c.bm), (unsigned)((p.N + c.bn - 1) / c.bn), (unsigned)c.splitK);
   if (grid.y > 65535) return 4;
-  if (c.bm == 128) launchIgemm<128, 128>(c, p, grid, st);
+  if (c.bm == 128 && c.bn == 128) launchIgemm<128, 128>(c, p, grid, st);
+  else if (c.bm == 128) launchIgemm<128, 64>(c, p, grid, st);
   else launchIgemm<64, 64>(c, p, grid, st);
   if (c.splitK > 1) {
     long long total = M * d->O;

@@ -245,6 +245,7 @@ class Planner {
         }
       }
       s.algoBytes = bytes;
+      bytes = 0;   // the traffic of a multi-launch reduction is counted once
       plan.steps.push_back(std::move(s));
     }
   }
@@ -329,7 +330,7 @@ class Planner {
     FusedCode fc = generateLoopKernel(v, leafPred());
     int sid = newStorage(v->type.bytes());
     bind(v, sid);
-    addFused(plan, fc, "fusion:" + n, {v});
+    addFused(plan, fc, "fusion:" + n + " " + v->type.str(), {v});
   }
 
   void collectLeavesOf(Value* v, std::vector<Value*>& out, std::unordered_set<Value*>& seen) {
@@ -392,7 +393,7 @@ class Planner {
       outs.push_back(g->result());
       emitted_.insert(g);
     }
-    addFused(plan, fc, group.size() > 1 ? "reduce x" + std::to_string(group.size()) : "reduce", outs);
+    addFused(plan, fc, (group.size() > 1 ? "reduce x" + std::to_string(group.size()) : std::string("reduce")) + " " + group[0]->operands[0]->type.str() + " -> " + outs[0]->type.str(), outs);
   }
 
   static std::vector<int64_t> stridesOf(const TensorType& t) {
