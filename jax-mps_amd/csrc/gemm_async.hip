@@ -1,0 +1,319 @@
+// bf16 GEMM for k-contiguous operands (C[m][n] = sum_k A[m][k] * B[n][k]) with an LDS ring
+// filled by direct global->LDS loads (global_load_lds_dwordx4, gfx950), so that several
+// K-slabs are in flight per workgroup without passing through registers.
+//
+// Replaces, for the layouts that qualify, the reference's dot_general lowering to mlx
+// matmul (src/pjrt_plugin/ops/linalg.cc:89-250).
+//
+// Layout of one ring stage: BM rows of A then BN rows of B, each row 64 k = 128 bytes = 8
+// slots of 16 bytes.  A direct load writes lane i of a wavefront at (LDS base + 16*i), i.e.
+// a wavefront instruction fills 8 whole rows; which 16 bytes of global memory a lane fetches
+// is free, so the logical slot kv of row r is kept at physical slot kv ^ ((r >> 1) & 7).
+// With that swizzle the MFMA operand read (32 rows x one slot, ds_read_b128) touches every
+// bank once per 16 lanes.
+//
+// Pipeline per iteration: wait until the oldest stage has landed (vmcnt), barrier, start the
+// loads that refill the stage consumed one iteration ago, multiply the landed stage.  One
+// barrier per 64-wide K-slab; loads are (STAGES-1) slabs ahead of the math.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+
+#include "hip_abi.h"
+
+namespace {
+
+typedef unsigned short u16;
+typedef unsigned int u32;
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+#define GLOBAL_PTR(p) ((__attribute__((address_space(1))) void*)(p))
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+struct AsyncArgs {
+  const u16* a;
+  const u16* b;
+  void* c;
+  long long M, N, K;
+  long long aB0, aB1, aLd, bB0, bB1, bLd;
+  int batch1;
+  int outBf16;
+  int tilesM, tilesN;
+  long long total;
+};
+
+__device__ __forceinline__ u16 to_bf16(float f) { return __builtin_bit_cast(u16, (__bf16)f); }
+
+// s_waitcnt immediate for "at most n vector-memory operations outstanding" (gfx9 encoding:
+// vmcnt in bits 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at their maxima)
+constexpr int vmcntImm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+template <int BM, int BN, int STAGES>
+__global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
+  constexpr int BK = 64;
+  constexpr int TM = BM / 64, TN = BN / 64;
+  constexpr int STAGE_BYTES = (BM + BN) * 128;
+  constexpr int NI = (BM + BN) / 32;          // direct loads per wavefront per stage (8 rows each)
+  static_assert((STAGES - 2) * NI <= 63, "vmcnt range");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  long long id = blockIdx.x;
+  if ((g.total & 7) == 0) id = (id & 7) * (g.total >> 3) + (id >> 3);
+  const long long perBatch = (long long)g.tilesM * g.tilesN;
+  const long long bz = id / perBatch;
+  const int t = (int)(id % perBatch);
+  const int tm = t / g.tilesN, tn = t % g.tilesN;
+  const long long b0 = bz / g.batch1, b1 = bz % g.batch1;
+  const u16* A = g.a + b0 * g.aB0 + b1 * g.aB1;
+  const u16* B = g.b + b0 * g.bB0 + b1 * g.bB1;
+  const long long m0 = (long long)tm * BM, n0 = (long long)tn * BN;
+
+  // per-lane source of each of this wavefront's direct loads (rows past the edge re-read the last row;
+  // their products land in accumulator rows or columns that are never stored)
+  const u16* src[NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    const int c = j * 4 + wave;                       // 8-row group within the stage
+    const int r = c * 8 + (lane >> 3);                // row within [A rows | B rows]
+    const int kv = (lane & 7) ^ ((r >> 1) & 7);       // logical k-slot this lane fetches
+    if (r < BM) {
+      long long gm = m0 + r;
+      if (gm > g.M - 1) gm = g.M - 1;
+      src[j] = A + gm * g.aLd + kv * 8;
+    } else {
+      long long gn = n0 + (r - BM);
+      if (gn > g.N - 1) gn = g.N - 1;
+      src[j] = B + gn * g.bLd + kv * 8;
+    }
+  }
+  const int nk = (int)(g.K / BK);
+  auto issue = [&](int slab) {
+    const int buf = slab % STAGES;
+    const long long k0 = (long long)(slab < nk ? slab : nk - 1) * BK;   // past the end: harmless re-read keeps the count uniform
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      unsigned char* dst = ring + buf * STAGE_BYTES + (j * 4 + wave) * 1024;
+      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[j] + k0), LDS_PTR(dst), 16, 0, 0);
+    }
+  };
+
+  float16v acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) issue(s);
+
+  // fragment addresses: row-dependent part of the swizzle is fixed per lane
+  const int arow = wm * (BM / 2) + (lane & 31);
+  const int brow = BM + wn * (BN / 2) + (lane & 31);
+  const int khalf = lane >> 5;
+  for (int it = 0; it < nk; ++it) {
+    __builtin_amdgcn_s_waitcnt(vmcntImm((STAGES - 2) * NI));
+    __builtin_amdgcn_s_barrier();
+    issue(it + STAGES - 1);
+    const unsigned char* st = ring + (it % STAGES) * STAGE_BYTES;
+    // fragments of k-step kk+1 are requested before the products of k-step kk are issued
+    bf16x8 av[2][TM], bv[2][TN];
+    auto frags = [&](int kk, int p) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int r = arow + i * 32;
+        av[p][i] = *(const bf16x8*)(st + r * 128 + (((kk * 2 + khalf) ^ ((r >> 1) & 7)) << 4));
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int r = brow + j * 32;
+        bv[p][j] = *(const bf16x8*)(st + r * 128 + (((kk * 2 + khalf) ^ ((r >> 1) & 7)) << 4));
+      }
+    };
+    frags(0, 0);
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      if (kk + 1 < 4) frags(kk + 1, (kk + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);   // keep the reads ahead of the products: the scheduler would sink them to save registers
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[kk & 1][i], bv[kk & 1][j], acc[i][j], 0, 0, 0);
+    }
+    // every fragment read of this stage has returned before the next barrier lets a refill start
+    __builtin_amdgcn_s_waitcnt((15) | (3 << 14) | (7 << 4) | (0 << 8));
+  }
+  __builtin_amdgcn_s_waitcnt(vmcntImm(0));   // drain the tail loads before the workgroup's LDS is released
+
+  const long long cBase = bz * g.M * g.N;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const long long col = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
+      if (col >= g.N) continue;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const long long row = m0 + wm * (BM / 2) + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (row >= g.M) continue;
+        if (g.outBf16) ((u16*)g.c)[cBase + row * g.N + col] = to_bf16(acc[i][j][e]);
+        else ((float*)g.c)[cBase + row * g.N + col] = acc[i][j][e];
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int STAGES>
+int launch(const AsyncArgs& g, hipStream_t st) {
+  constexpr int bytes = STAGES * (BM + BN) * 128;
+  static bool configured = false;   // per process; the attribute is per function, not per device state that changes
+  if (!configured) {
+    if (hipFuncSetAttribute((const void*)gemm_bf16_async<BM, BN, STAGES>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return 3;
+    configured = true;
+  }
+  gemm_bf16_async<BM, BN, STAGES><<<dim3((unsigned)g.total), 256, bytes, st>>>(g);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// out[b][x][k] = in[b0, b1][k][x]  (x contiguous in, k contiguous out), 64x64 tiles through LDS
+struct TransposeArgs {
+  const u16* in;
+  u16* out;
+  long long K, X, ld, inB0, inB1;
+  int batch1;
+};
+
+__global__ void __launch_bounds__(256) transpose_bf16(TransposeArgs t) {
+  __shared__ u16 tile[64][64 + 2];
+  const int tid = threadIdx.x;
+  const long long b0 = blockIdx.z / t.batch1, b1 = blockIdx.z % t.batch1;
+  const u16* in = t.in + b0 * t.inB0 + b1 * t.inB1;
+  u16* out = t.out + (long long)blockIdx.z * t.K * t.X;
+  const long long k0 = (long long)blockIdx.y * 64, x0 = (long long)blockIdx.x * 64;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int u = tid + 256 * i, k = u >> 3, xv = (u & 7) * 8;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (k0 + k < t.K && x0 + xv < t.X) v = *(const uint4*)(in + (k0 + k) * t.ld + x0 + xv);
+    const u16* e = (const u16*)&v;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) tile[k][xv + q] = e[q];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int u = tid + 256 * i, x = u >> 3, kv = (u & 7) * 8;
+    if (x0 + x >= t.X || k0 + kv >= t.K) continue;
+    uint4 v;
+    u16* e = (u16*)&v;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) e[q] = tile[kv + q][x];
+    *(uint4*)(out + (x0 + x) * t.K + k0 + kv) = v;
+  }
+}
+
+// How each operand reaches the k-contiguous layout the kernel needs.
+struct OperandPlan {
+  bool ok = false;
+  bool copy = false;     // needs a transposed copy in the workspace
+  long long ld = 0;      // row pitch when used in place
+};
+
+OperandPlan planOperand(long long rowStride, long long kStride, long long rows, long long K, long long other) {
+  OperandPlan p;
+  if (kStride == 1 && rowStride % 8 == 0) { p.ok = true; p.ld = rowStride; return p; }
+  // laid out along the rows: worth a copy only when the other side is large enough to amortise it
+  if (rowStride == 1 && kStride % 8 == 0 && rows % 8 == 0 && other >= 256) { p.ok = true; p.copy = true; p.ld = K; }
+  return p;
+}
+
+bool qualifies(const mi355_gemm_desc* d, OperandPlan& pa, OperandPlan& pb) {
+  if (d->in_dtype != 1 || (d->out_dtype != 0 && d->out_dtype != 1)) return false;
+  const long long nb = d->batch0 * d->batch1;
+  if (d->M <= 0 || d->N <= 0 || d->K <= 0 || nb <= 0 || nb > 65535) return false;
+  if (d->K % 64 != 0) return false;
+  pa = planOperand(d->aRow, d->aCol, d->M, d->K, d->N);
+  pb = planOperand(d->bCol, d->bRow, d->N, d->K, d->M);
+  if (!pa.ok || !pb.ok) return false;
+  if (d->batch0 > 1 && (d->aB0 % 8 || d->bB0 % 8)) return false;
+  if (d->batch1 > 1 && (d->aB1 % 8 || d->bB1 % 8)) return false;
+  return true;
+}
+
+size_t roundUp256(size_t b) { return (b + 255) / 256 * 256; }
+
+int transposeInto(const u16* in, u16* out, long long K, long long X, long long ld, const mi355_gemm_desc* d, long long inB0, long long inB1,
+                  hipStream_t st) {
+  TransposeArgs t;
+  t.in = in; t.out = out; t.K = K; t.X = X; t.ld = ld; t.inB0 = inB0; t.inB1 = inB1; t.batch1 = (int)d->batch1;
+  dim3 grid((unsigned)((X + 63) / 64), (unsigned)((K + 63) / 64), (unsigned)(d->batch0 * d->batch1));
+  transpose_bf16<<<grid, 256, 0, st>>>(t);
+  return hipGetLastError() == hipSuccess ? 0 : 3;
+}
+
+}  // namespace
+
+extern "C" size_t mi355_gemm_workspace_bytes(const mi355_gemm_desc* d) {
+  OperandPlan pa, pb;
+  if (!qualifies(d, pa, pb)) return 0;
+  const size_t nb = (size_t)(d->batch0 * d->batch1);
+  size_t bytes = 0;
+  if (pa.copy) bytes += roundUp256(nb * (size_t)d->M * (size_t)d->K * 2);
+  if (pb.copy) bytes += roundUp256(nb * (size_t)d->N * (size_t)d->K * 2);
+  return bytes;
+}
+
+// 0 = launched, -1 = layout does not qualify, other = launch error.
+extern "C" int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, const void* b, void* c, void* workspace,
+                                     size_t workspace_bytes, mi355_stream_t s) {
+  OperandPlan pa, pb;
+  if (!qualifies(d, pa, pb)) return -1;
+  if (!aligned16(a) || !aligned16(b)) return -1;
+  if ((pa.copy || pb.copy) && (workspace == nullptr || workspace_bytes < mi355_gemm_workspace_bytes(d) || !aligned16(workspace))) return -1;
+  hipStream_t st = (hipStream_t)s;
+  const long long nb = d->batch0 * d->batch1;
+  AsyncArgs g;
+  g.a = (const u16*)a; g.b = (const u16*)b; g.c = c;
+  g.M = d->M; g.N = d->N; g.K = d->K;
+  g.aB0 = d->aB0; g.aB1 = d->aB1; g.aLd = pa.ld;
+  g.bB0 = d->bB0; g.bB1 = d->bB1; g.bLd = pb.ld;
+  g.batch1 = (int)d->batch1;
+  g.outBf16 = d->out_dtype == 1;
+  unsigned char* ws = (unsigned char*)workspace;
+  if (pa.copy) {
+    if (int r = transposeInto((const u16*)a, (u16*)ws, d->K, d->M, d->aCol, d, d->aB0, d->aB1, st)) return r;
+    g.a = (const u16*)ws;
+    g.aB1 = d->M * d->K; g.aB0 = g.aB1 * d->batch1;
+    ws += roundUp256((size_t)nb * (size_t)d->M * (size_t)d->K * 2);
+  }
+  if (pb.copy) {
+    if (int r = transposeInto((const u16*)b, (u16*)ws, d->K, d->N, d->bRow, d, d->bB0, d->bB1, st)) return r;
+    g.b = (const u16*)ws;
+    g.bB1 = d->N * d->K; g.bB0 = g.bB1 * d->batch1;
+  }
+  auto tiles = [&](int bm, int bn) { return ((d->M + bm - 1) / bm) * ((d->N + bn - 1) / bn) * nb; };
+  // the largest tile that still leaves about three workgroups per compute unit
+  int bm = 64, bn = 64;
+  static const char* force = getenv("MI355X_GEMM_TILE");   // "256x128", "128x128", "128x64", "64x64": tuning aid
+  if (force) sscanf(force, "%dx%d", &bm, &bn);
+  else if (d->M > 128 && d->N > 64 && tiles(256, 128) >= 1024) { bm = 256; bn = 128; }
+  else if (d->M > 64 && d->N > 64 && tiles(128, 128) >= 768) { bm = 128; bn = 128; }
+  else if (d->M > 64 && tiles(128, 64) >= 768) { bm = 128; bn = 64; }
+  g.tilesM = (int)((d->M + bm - 1) / bm);
+  g.tilesN = (int)((d->N + bn - 1) / bn);
+  g.total = (long long)g.tilesM * g.tilesN * nb;
+  if (g.total > 0x7FFFFFFFll) return -1;
+  // two ring stages keep two workgroups resident per compute unit, which hides more than a deeper ring does
+  if (bm == 256) return launch<256, 128, 3>(g, st);
+  if (bm == 128 && bn == 128) return launch<128, 128, 2>(g, st);
+  if (bm == 128) return launch<128, 64, 2>(g, st);
+  return launch<64, 64, 2>(g, st);
+}

@@ -398,7 +398,8 @@ int mi355_copy(void* dst, const void* src, size_t bytes, mi355_stream_t s) {
   return check("copy");
 }
 
-int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, mi355_stream_t s) {
+int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, void* workspace, size_t workspace_bytes,
+               mi355_stream_t s) {
   if (d->M <= 0 || d->N <= 0 || d->batch0 * d->batch1 <= 0) return 0;
   GemmArgs g;
   g.a = a; g.b = b; g.c = c;
@@ -408,6 +409,12 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
   g.batch1 = (int)d->batch1;
   g.outBf16 = d->out_dtype == 1;
   long long nb = d->batch0 * d->batch1;
+  if (d->in_dtype == 1) {
+    int r = mi355_gemm_bf16_async(d, a, b, c, workspace, workspace_bytes, s);
+    if (r >= 0) return r;
+    r = mi355_gemm_bf16_tiled(d, a, b, c, s);
+    if (r >= 0) return r;
+  }
   if (nb > 65535) return 1;   // grid.z limit; callers fold larger batches
   dim3 grid((unsigned)((d->N + 63) / 64), (unsigned)((d->M + 63) / 64), (unsigned)nb);
   if (d->in_dtype == 0) gemm_f32_mfma<<<grid, 256, 0, (hipStream_t)s>>>(g);

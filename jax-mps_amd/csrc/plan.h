@@ -115,5 +115,6 @@ struct CompiledProgram {
 std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module);
 int abiDtypeCode(DType d);   // element type code of the C-ABI kernel entry points (-1: not supported there)
 mi355_conv_desc toAbi(const ConvDesc& c);
+mi355_gemm_desc toAbi(const GemmDesc& g);
 
 }  // namespace mi355

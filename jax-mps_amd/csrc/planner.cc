@@ -479,6 +479,11 @@ class Planner {
     s.label = "dot_general " + a->type.str() + " x " + b->type.str();
     s.gemm = g;
     s.args = {ref(storageOf(a), t), ref(storageOf(b), t), ref(sid, t)};
+    // room for a k-contiguous copy of an operand that is laid out along m or n
+    mi355_gemm_desc abi = toAbi(g);
+    int64_t ws = ((int64_t)mi355_gemm_workspace_bytes(&abi) + kAlign - 1) / kAlign * kAlign;
+    s.workspaceBytes = ws;
+    if (ws > 0) s.args.push_back(ref(newStorage((size_t)ws), t));
     plan.steps.push_back(std::move(s));
   }
 
@@ -900,6 +905,16 @@ int abiDtypeCode(DType d) {
     case DType::U32: return 3;
     default: return -1;
   }
+}
+
+mi355_gemm_desc toAbi(const GemmDesc& g) {
+  mi355_gemm_desc d;
+  d.batch0 = g.batch0; d.batch1 = g.batch1; d.M = g.M; d.N = g.N; d.K = g.K;
+  d.aB0 = g.aB0; d.aB1 = g.aB1; d.aRow = g.aRow; d.aCol = g.aCol;
+  d.bB0 = g.bB0; d.bB1 = g.bB1; d.bRow = g.bRow; d.bCol = g.bCol;
+  d.in_dtype = abiDtypeCode(g.inType);
+  d.out_dtype = abiDtypeCode(g.outType);
+  return d;
 }
 
 mi355_conv_desc toAbi(const ConvDesc& c) {

@@ -357,14 +357,10 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       break;
     }
     case Step::Gemm: {
-      mi355_gemm_desc d;
-      const GemmDesc& g = s.gemm;
-      d.batch0 = g.batch0; d.batch1 = g.batch1; d.M = g.M; d.N = g.N; d.K = g.K;
-      d.aB0 = g.aB0; d.aB1 = g.aB1; d.aRow = g.aRow; d.aCol = g.aCol;
-      d.bB0 = g.bB0; d.bB1 = g.bB1; d.bRow = g.bRow; d.bCol = g.bCol;
-      d.in_dtype = dtypeCode(g.inType);
-      d.out_dtype = dtypeCode(g.outType);
-      check(mi355_gemm(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), st), "gemm");
+      mi355_gemm_desc d = toAbi(s.gemm);
+      void* ws = s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
+      check(mi355_gemm(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), ws,
+                       (size_t)s.workspaceBytes, st), "gemm");
       break;
     }
     case Step::Conv: {

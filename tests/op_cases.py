@@ -205,6 +205,19 @@ case("dot-batched-attention-layout", lambda b, q, k: b.dot_general(q, k, ([3], [
 case("dot-two-contracting", lambda b, x, y: b.dot_general(x, y, ([1, 2], [0, 1])), f32(186, 6, 4, 5), f32(187, 4, 5, 7))
 case("dot-bf16", lambda b, x, y: b.matmul(x, y), f32(188, 40, 96), f32(189, 96, 72), dtypes=["bf16", "bf16"])
 case("dot-bf16-f32-out", lambda b, x, y: b.dot_general(x, y, ([1], [0]), out_dtype="f32"), f32(190, 40, 96), f32(191, 96, 72), dtypes=["bf16", "bf16"])
+# bf16 layouts of the tiled MFMA kernel: k-contiguous and m/n-contiguous operands, ragged tiles, batches
+case("dot-bf16-tiled-kn", lambda b, x, y: b.matmul(x, y), f32(1900, 200, 136), f32(1901, 136, 328), dtypes=["bf16", "bf16"])
+case("dot-bf16-tiled-rhs-kmajor", lambda b, x, y: b.dot_general(x, y, ([1], [1])), f32(1902, 150, 72), f32(1903, 90, 72), dtypes=["bf16", "bf16"])
+case("dot-bf16-tiled-lhs-mmajor", lambda b, x, y: b.dot_general(x, y, ([0], [0])), f32(1904, 100, 136), f32(1905, 100, 72), dtypes=["bf16", "bf16"])
+case("dot-bf16-tiled-lhs-mmajor-rhs-kmajor", lambda b, x, y: b.dot_general(x, y, ([0], [1])), f32(1906, 68, 264), f32(1907, 130, 68), dtypes=["bf16", "bf16"])
+case("dot-bf16-tiled-attention-qk", lambda b, q, k: b.dot_general(q, k, ([3], [3]), ([0, 2], [0, 2])), f32(1908, 2, 128, 3, 64), f32(1909, 2, 128, 3, 64), dtypes=["bf16", "bf16"])
+case("dot-bf16-tiled-attention-pv", lambda b, p, v: b.dot_general(p, v, ([3], [1]), ([0, 1], [0, 2])), f32(1910, 2, 3, 128, 128), f32(1911, 2, 128, 3, 64), dtypes=["bf16", "bf16"])
+case("dot-bf16-tiled-big", lambda b, x, y: b.matmul(x, y), f32(1912, 1024, 192, lo=-1, hi=1), f32(1913, 192, 1024, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("dot-bf16-tiled-f32-out", lambda b, x, y: b.dot_general(x, y, ([1], [0]), out_dtype="f32"), f32(1914, 130, 200), f32(1915, 200, 136), dtypes=["bf16", "bf16"])
+case("dot-bf16-async-nt", lambda b, x, y: b.dot_general(x, y, ([1], [1])), f32(1916, 200, 192, lo=-1, hi=1), f32(1917, 328, 192, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("dot-bf16-async-nt-long-k", lambda b, x, y: b.dot_general(x, y, ([1], [1]), out_dtype="f32"), f32(1918, 300, 1024, lo=-1, hi=1), f32(1919, 130, 1024, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("dot-bf16-async-nt-one-slab", lambda b, x, y: b.dot_general(x, y, ([1], [1])), f32(1920, 70, 64), f32(1921, 50, 64), dtypes=["bf16", "bf16"])
+case("dot-bf16-async-nt-big", lambda b, x, y: b.dot_general(x, y, ([1], [1])), f32(1922, 1024, 512, lo=-1, hi=1), f32(1923, 768, 512, lo=-1, hi=1), dtypes=["bf16", "bf16"])
 case("dot-large-k", lambda b, x, y: b.matmul(x, y), f32(192, 64, 3000, lo=-1, hi=1), f32(193, 3000, 64, lo=-1, hi=1))
 
 
