@@ -849,12 +849,19 @@ static const char* reduceKind(const Op& reduce) {
 bool isSimpleReduce(const Op& reduce) { return reduce.operands.size() == 2 && reduceKind(reduce) != nullptr; }
 
 // ------------------------------------------------------------------ loop kernels
-FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf) {
+FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf) { return generateLoopKernel(std::vector<Value*>{root}, isLeaf); }
+
+// One pass over a shared index space that stores several results: all roots have the same
+// dims; a root may feed another root (it is then computed once and both are stored).
+FusedCode generateLoopKernel(const std::vector<Value*>& roots, const LeafPredicate& isLeaf) {
   std::vector<Value*> all;
   std::unordered_map<Value*, bool> seen;
-  LeafPredicate inner = [&](Value* v) { return v != root && isLeaf(v); };
-  collectAllValues(root, inner, all, seen);
-  int V = pickVector(root->type);
+  auto isRoot = [&](Value* v) { return std::find(roots.begin(), roots.end(), v) != roots.end(); };
+  LeafPredicate inner = [&](Value* v) { return !isRoot(v) && isLeaf(v); };
+  for (auto* r : roots) collectAllValues(r, inner, all, seen);
+  Value* root = roots[0];
+  int V = 8;
+  for (auto* r : roots) V = std::min(V, pickVector(r->type));
   bool i64 = needs64(all);
   Emitter em(inner, V, i64);
   int64_t N = root->type.numel();
@@ -865,23 +872,28 @@ FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf) {
   lin.mult = V;
   if (V == 1) { lin.coef = 0; }
   Index idx = em.linearIndex(lin, root->type.dims);
-  std::string val = em.gen(root, idx);
-  DType dt = root->type.dt;
+  std::vector<std::string> vals;
+  for (auto* r : roots) vals.push_back(em.gen(r, idx));
   std::ostringstream s;
   s << kPrelude;
-  s << kernelHeader(em.leaves_, {storageT(dt) + "* __restrict__ out0"}) << " {\n";
+  std::vector<std::string> outs;
+  for (size_t j = 0; j < roots.size(); ++j) outs.push_back(storageT(roots[j]->type.dt) + "* __restrict__ out" + std::to_string(j));
+  s << kernelHeader(em.leaves_, outs) << " {\n";
   s << "  const " << em.idxT() << " base = ((" << em.idxT() << ")blockIdx.x * 256 + threadIdx.x) * " << V << ";\n";
   s << "  if (base >= " << N << (i64 ? "ll" : "") << ") return;\n";
   s << em.pre_;
   if (V > 1) {
-    s << "  Vec<" << storageT(dt) << ", " << V << "> ov;\n";
+    for (size_t j = 0; j < roots.size(); ++j) s << "  Vec<" << storageT(roots[j]->type.dt) << ", " << V << "> ov" << j << ";\n";
     s << "  #pragma unroll\n  for (int v = 0; v < " << V << "; ++v) {\n";
     s << em.body_.front();
-    s << "    ov.e[v] = " << storeExpr(dt, val) << ";\n  }\n";
-    s << "  *(Vec<" << storageT(dt) << ", " << V << ">*)(out0 + base) = ov;\n";
+    for (size_t j = 0; j < roots.size(); ++j) s << "    ov" << j << ".e[v] = " << storeExpr(roots[j]->type.dt, vals[j]) << ";\n";
+    s << "  }\n";
+    for (size_t j = 0; j < roots.size(); ++j)
+      s << "  *(Vec<" << storageT(roots[j]->type.dt) << ", " << V << ">*)(out" << j << " + base) = ov" << j << ";\n";
   } else {
     s << "  {\n    const int v = 0; (void)v;\n" << em.body_.front();
-    s << "    out0[base] = " << storeExpr(dt, val) << ";\n  }\n";
+    for (size_t j = 0; j < roots.size(); ++j) s << "    out" << j << "[base] = " << storeExpr(roots[j]->type.dt, vals[j]) << ";\n";
+    s << "  }\n";
   }
   s << "}\n";
   FusedCode fc;
@@ -891,10 +903,12 @@ FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf) {
   l.grid[0] = (unsigned)std::max<int64_t>(1, (threads + 255) / 256);
   l.block[0] = 256;
   for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
-  KArg o;
-  o.kind = KArg::Out;
-  o.value = root;
-  l.args.push_back(o);
+  for (auto* r : roots) {
+    KArg o;
+    o.kind = KArg::Out;
+    o.value = r;
+    l.args.push_back(o);
+  }
   fc.launches.push_back(std::move(l));
   fc.leaves = em.leaves_;
   return fc;

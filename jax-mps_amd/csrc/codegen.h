@@ -39,6 +39,7 @@ using LeafPredicate = std::function<bool(Value*)>;
 
 // out[i] = f(leaves...) for every element of `root`.
 FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf);
+FusedCode generateLoopKernel(const std::vector<Value*>& roots, const LeafPredicate& isLeaf);
 
 // In-place window write of a dynamic_update_slice: iterates over the update
 // tensor and stores into `dus` result storage (which already holds the operand).

@@ -366,7 +366,7 @@ ConvChoice choose(const mi355_conv_desc* d) {
   else { c.bm = 64; c.bn = 64; }
   long long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
   int split = 1;
-  if (tiles < 512) split = (int)std::min<long long>((1024 + tiles - 1) / tiles, std::max(1, c.kTiles / 8));
+  if (tiles < 512) split = (int)std::min<long long>((1024 + tiles - 1) / tiles, std::max(1, c.kTiles / (tiles < 64 ? 4 : 8)));
   split = std::max(1, std::min(split, 256));
   c.tilesPerSplit = (c.kTiles + split - 1) / split;
   c.splitK = (c.kTiles + c.tilesPerSplit - 1) / c.tilesPerSplit;

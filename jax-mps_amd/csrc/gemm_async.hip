@@ -261,7 +261,7 @@ int transposeInto(const u16* in, u16* out, long long K, long long X, long long l
 
 }  // namespace
 
-extern "C" size_t mi355_gemm_workspace_bytes(const mi355_gemm_desc* d) {
+extern "C" size_t mi355_gemm_bf16_async_workspace_bytes(const mi355_gemm_desc* d) {
   OperandPlan pa, pb;
   if (!qualifies(d, pa, pb)) return 0;
   const size_t nb = (size_t)(d->batch0 * d->batch1);
@@ -277,7 +277,7 @@ extern "C" int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, co
   OperandPlan pa, pb;
   if (!qualifies(d, pa, pb)) return -1;
   if (!aligned16(a) || !aligned16(b)) return -1;
-  if ((pa.copy || pb.copy) && (workspace == nullptr || workspace_bytes < mi355_gemm_workspace_bytes(d) || !aligned16(workspace))) return -1;
+  if ((pa.copy || pb.copy) && (workspace == nullptr || workspace_bytes < mi355_gemm_bf16_async_workspace_bytes(d) || !aligned16(workspace))) return -1;
   hipStream_t st = (hipStream_t)s;
   const long long nb = d->batch0 * d->batch1;
   AsyncArgs g;

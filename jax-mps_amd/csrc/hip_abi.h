@@ -42,6 +42,14 @@ int mi355_event_sync(mi355_event_t e);
 int mi355_event_query(mi355_event_t e, int* ready);
 int mi355_event_elapsed_ms(mi355_event_t a, mi355_event_t b, float* ms);
 
+// Stream capture into an executable graph: work enqueued on `s` between begin and end is recorded,
+// not run; mi355_graph_launch replays it.  Used for the bodies of counted loops.
+typedef void* mi355_graph_t;
+int mi355_capture_begin(mi355_stream_t s);
+int mi355_capture_end(mi355_stream_t s, mi355_graph_t* exec, int* num_nodes);
+int mi355_graph_launch(mi355_graph_t exec, mi355_stream_t s);
+int mi355_graph_destroy(mi355_graph_t exec);
+
 // runtime-compiled kernels: `source` defines extern "C" __global__ void k(...).
 // mi355_rtc_compile is thread-safe (no device state); the code object it returns is
 // malloc'ed and handed to mi355_module_load, which must run on the thread that owns the device.
@@ -65,6 +73,7 @@ size_t mi355_gemm_workspace_bytes(const mi355_gemm_desc* d);
 // bf16, both operands k-contiguous, K % 64 == 0: LDS ring filled by direct global->LDS loads
 int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, const void* b, void* c, void* workspace,
                           size_t workspace_bytes, mi355_stream_t s);
+size_t mi355_gemm_bf16_async_workspace_bytes(const mi355_gemm_desc* d);
 int mi355_gemm_bf16_tiled(const mi355_gemm_desc* d, const void* a, const void* b, void* c, mi355_stream_t s);
 
 typedef struct {
@@ -95,6 +104,8 @@ int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* in
 size_t mi355_scatter_workspace_bytes(int64_t num_updates);
 
 int mi355_copy(void* dst, const void* src, size_t bytes, mi355_stream_t s);   // kernel copy (graph-capturable)
+// up to 16 copies between pairwise disjoint buffers in one launch
+int mi355_copy_multi(int n, void* const* dst, const void* const* src, const size_t* bytes, mi355_stream_t s);
 
 #ifdef __cplusplus
 }

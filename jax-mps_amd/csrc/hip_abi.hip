@@ -90,6 +90,33 @@ int mi355_stream_sync(mi355_stream_t s) {
   HIPCHK(hipStreamSynchronize((hipStream_t)s));
   return 0;
 }
+int mi355_capture_begin(mi355_stream_t s) {
+  HIPCHK(hipStreamBeginCapture((hipStream_t)s, hipStreamCaptureModeThreadLocal));
+  return 0;
+}
+int mi355_capture_end(mi355_stream_t s, mi355_graph_t* exec, int* num_nodes) {
+  hipGraph_t graph = nullptr;
+  HIPCHK(hipStreamEndCapture((hipStream_t)s, &graph));
+  if (!graph) return 1;
+  size_t n = 0;
+  if (hipGraphGetNodes(graph, nullptr, &n) != hipSuccess) n = 0;
+  if (num_nodes) *num_nodes = (int)n;
+  hipGraphExec_t ge = nullptr;
+  hipError_t e = hipGraphInstantiate(&ge, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (e != hipSuccess) return fail(e, "hipGraphInstantiate");
+  *exec = (mi355_graph_t)ge;
+  return 0;
+}
+int mi355_graph_launch(mi355_graph_t exec, mi355_stream_t s) {
+  HIPCHK(hipGraphLaunch((hipGraphExec_t)exec, (hipStream_t)s));
+  return 0;
+}
+int mi355_graph_destroy(mi355_graph_t exec) {
+  HIPCHK(hipGraphExecDestroy((hipGraphExec_t)exec));
+  return 0;
+}
+
 int mi355_event_create(mi355_event_t* e, int timing) {
   hipEvent_t ev;
   HIPCHK(hipEventCreateWithFlags(&ev, timing ? hipEventDefault : hipEventDisableTiming));

@@ -37,6 +37,25 @@ __global__ void __launch_bounds__(256) copy_bytes(const unsigned char* __restric
   if (i < n) dst[i] = src[i];
 }
 
+struct MultiCopyArgs {
+  const unsigned char* src[16];
+  unsigned char* dst[16];
+  unsigned long long bytes[16];
+};
+__global__ void __launch_bounds__(256) copy_multi(MultiCopyArgs a) {
+  const int j = blockIdx.y;
+  const unsigned char* src = a.src[j];
+  unsigned char* dst = a.dst[j];
+  const size_t bytes = a.bytes[j];
+  const size_t stride = (size_t)gridDim.x * 256;
+  if ((((uintptr_t)src | (uintptr_t)dst | bytes) & 15) == 0) {
+    const size_t n16 = bytes / 16;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) ((uint4*)dst)[i] = ((const uint4*)src)[i];
+  } else {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < bytes; i += stride) dst[i] = src[i];
+  }
+}
+
 // ------------------------------------------------------------------- GEMM
 // Workgroup tile 64x64, four wavefronts in a 2x2 arrangement, each owning a 32x32
 // accumulator held by one MFMA 32x32 instruction.  A and B tiles are staged in LDS
@@ -398,6 +417,48 @@ int mi355_copy(void* dst, const void* src, size_t bytes, mi355_stream_t s) {
   return check("copy");
 }
 
+int mi355_copy_multi(int n, void* const* dst, const void* const* src, const size_t* bytes, mi355_stream_t s) {
+  if (n <= 0) return 0;
+  if (n > 16) return 1;
+  MultiCopyArgs a;
+  size_t most = 0;
+  for (int i = 0; i < n; ++i) {
+    a.src[i] = (const unsigned char*)src[i];
+    a.dst[i] = (unsigned char*)dst[i];
+    a.bytes[i] = bytes[i];
+    size_t units = ((((uintptr_t)src[i] | (uintptr_t)dst[i] | bytes[i]) & 15) == 0) ? bytes[i] / 16 : bytes[i];
+    most = units > most ? units : most;
+  }
+  if (most == 0) return 0;
+  unsigned gx = (unsigned)((most + 255) / 256);
+  if (gx > 2048) gx = 2048;
+  copy_multi<<<dim3(gx, (unsigned)n), 256, 0, (hipStream_t)s>>>(a);
+  return check("copy_multi");
+}
+
+// An unbatched fp32 GEMM is a convolution without spatial dims (rows = batch, k = input
+// features, columns = output features): it then runs on the implicit-GEMM kernel with its
+// vector tile loaders, register prefetch and split-K for shapes with few output tiles.
+static bool gemmAsPointwiseConv(const mi355_gemm_desc* d, mi355_conv_desc* c) {
+  if (d->in_dtype != 0 || d->out_dtype != 0 || d->batch0 * d->batch1 != 1 || d->K <= 0) return false;
+  *c = mi355_conv_desc{};
+  c->nsp = 0;
+  c->N = d->M; c->C = d->K; c->O = d->N;
+  c->featureGroups = 1; c->batchGroups = 1;
+  c->lhsB = d->aRow; c->lhsF = d->aCol;
+  c->rhsI = d->bRow; c->rhsO = d->bCol;
+  c->outB = d->N; c->outF = 1;
+  c->dtype = 0;
+  return true;
+}
+
+size_t mi355_gemm_workspace_bytes(const mi355_gemm_desc* d) {
+  if (d->in_dtype == 1) return mi355_gemm_bf16_async_workspace_bytes(d);
+  mi355_conv_desc cd;
+  if (gemmAsPointwiseConv(d, &cd)) return mi355_conv_workspace_bytes(&cd);
+  return 0;
+}
+
 int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, void* workspace, size_t workspace_bytes,
                mi355_stream_t s) {
   if (d->M <= 0 || d->N <= 0 || d->batch0 * d->batch1 <= 0) return 0;
@@ -415,6 +476,8 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
     r = mi355_gemm_bf16_tiled(d, a, b, c, s);
     if (r >= 0) return r;
   }
+  mi355_conv_desc cd;
+  if (gemmAsPointwiseConv(d, &cd)) return mi355_conv(&cd, a, b, c, workspace, workspace_bytes, s);
   if (nb > 65535) return 1;   // grid.z limit; callers fold larger batches
   dim3 grid((unsigned)((d->N + 63) / 64), (unsigned)((d->M + 63) / 64), (unsigned)nb);
   if (d->in_dtype == 0) gemm_f32_mfma<<<grid, 256, 0, (hipStream_t)s>>>(g);

@@ -79,9 +79,11 @@ struct Step {
   int64_t workspaceBytes = 0;
   int splitK = 1;
 
-  // Copy / Fill
+  // Copy / Fill.  A Copy with `copyBytes` set moves several disjoint buffers in one launch:
+  // args = [src0, dst0, src1, dst1, ...], copyBytes[i] = size of pair i.
   BufRef src, dst;
   int64_t bytes = 0;
+  std::vector<int64_t> copyBytes;
 
   // While / Case
   std::unique_ptr<Plan> cond;                 // While: evaluates the predicate into predBuf

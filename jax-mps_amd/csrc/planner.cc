@@ -10,6 +10,7 @@
 // (bias-add, softmax, LayerNorm, RMSNorm: src/pjrt_plugin/passes/*.cc) plus
 // whatever else is elementwise; nothing here is pattern-matched by name.
 #include <algorithm>
+#include <array>
 #include <cstring>
 #include <functional>
 #include <set>
@@ -266,15 +267,15 @@ class Planner {
   }
 
   void emitRegion(Region& r, Plan& plan) {
-    for (auto& opPtr : r.ops) {
-      Op* op = opPtr.get();
+    for (size_t pos = 0; pos < r.ops.size(); ++pos) {
+      Op* op = r.ops[pos].get();
       if (emitted_.count(op)) continue;
       const std::string& n = op->name;
       if (n == "return") continue;
       if (isFusibleOp(*op) && op->results.size() == 1) {
         Value* v = op->result();
         if (!needMat_[v]) continue;
-        emitMaterialized(op, plan);
+        emitLoopGroup(op, r, pos, plan);
         continue;
       }
       if (isPassThrough(*op)) {   // multi-result barrier: results alias operands
@@ -301,6 +302,69 @@ class Planner {
     if (hasStorage(v)) return;
     if (!v->def || !isFusibleOp(*v->def)) throw CompileError("internal: cannot materialise " + v->name);
     emitMaterialized(v->def, plan);
+  }
+
+  // true when materialising `op` takes a kernel (not a constant-pool entry, an alias or nothing)
+  bool takesKernel(Op* op) {
+    Value* v = op->result();
+    const std::string& n = op->name;
+    if (n == "constant") {
+      auto& d = *op->attrs.at("value").dense;
+      if (!d.splat || d.type.numel() == 1) return false;
+    }
+    if ((n == "reshape" || isPassThrough(*op) || (n == "convert" && op->operands[0]->type.dt == v->type.dt)) && hasStorage(op->operands[0])) return false;
+    return v->type.numel() != 0;
+  }
+
+  // Values the loop kernel of `v` would read, given that `roots` are computed in the same kernel.
+  // Returns false when one of them is not in memory yet.
+  bool leavesReady(Value* v, const std::vector<Value*>& roots, std::unordered_set<Value*>& seen, int& count) {
+    for (auto* o : v->def->operands) {
+      if (!seen.insert(o).second) continue;
+      if (std::find(roots.begin(), roots.end(), o) != roots.end()) continue;
+      if (hasStorage(o)) { ++count; continue; }
+      if (!o->def || !isFusibleOp(*o->def) || o->def->results.size() != 1 || needMat_[o]) return false;
+      if (!leavesReady(o, roots, seen, count)) return false;
+    }
+    return true;
+  }
+
+  // Materialised elementwise values with the same dims whose inputs are already in memory are
+  // computed by one kernel with several outputs: later ops of the region are pulled forward
+  // (SSA values are pure, so computing them earlier is always valid).
+  void emitLoopGroup(Op* op, Region& r, size_t pos, Plan& plan) {
+    Value* v = op->result();
+    static const bool multi = !(getenv("MI355X_MULTI_OUTPUT") && getenv("MI355X_MULTI_OUTPUT")[0] == '0');
+    if (hasStorage(v)) return;
+    if (!multi || !takesKernel(op)) { emitMaterialized(op, plan); return; }
+    std::vector<Value*> roots{v};
+    std::vector<Op*> members{op};
+    std::unordered_set<Value*> seen;
+    int leafCount = 0;
+    leavesReady(v, roots, seen, leafCount);
+    const size_t kLookAhead = 96, kMaxRoots = 8;
+    for (size_t q = pos + 1; q < r.ops.size() && q <= pos + kLookAhead && roots.size() < kMaxRoots; ++q) {
+      Op* y = r.ops[q].get();
+      if (emitted_.count(y) || !isFusibleOp(*y) || y->results.size() != 1) continue;
+      Value* w = y->result();
+      if (!needMat_[w] || hasStorage(w)) continue;
+      if (w->type.dims != v->type.dims || dtypeSize(w->type.dt) != dtypeSize(v->type.dt)) continue;
+      if (!takesKernel(y)) continue;
+      std::unordered_set<Value*> seenY = seen;
+      int cnt = leafCount;
+      if (!leavesReady(w, roots, seenY, cnt) || cnt + (int)roots.size() + 1 > 40) continue;
+      seen = std::move(seenY);
+      leafCount = cnt;
+      roots.push_back(w);
+      members.push_back(y);
+    }
+    if (roots.size() == 1) { emitMaterialized(op, plan); return; }
+    FusedCode fc = generateLoopKernel(roots, leafPred());
+    std::string label = "fusion:" + op->name;
+    for (size_t k = 1; k < members.size(); ++k) label += "+" + members[k]->name;
+    for (auto* w : roots) bind(w, newStorage(w->type.bytes()));
+    for (auto* m : members) emitted_.insert(m);
+    addFused(plan, fc, label + " " + v->type.str(), roots);
   }
 
   void emitMaterialized(Op* op, Plan& plan) {
@@ -723,6 +787,27 @@ class Planner {
     plan.steps.push_back(std::move(c));
   }
 
+  // several copies between pairwise disjoint buffers as one launch
+  void multiCopyStep(Plan& plan, const std::vector<std::array<int, 2>>& pairs, const std::vector<int64_t>& bytes, const char* label) {
+    std::vector<size_t> live;
+    for (size_t i = 0; i < pairs.size(); ++i) if (pairs[i][0] != pairs[i][1]) live.push_back(i);
+    for (size_t b = 0; b < live.size(); b += 16) {
+      size_t e = std::min(live.size(), b + 16);
+      if (e - b == 1) { copyStep(plan, pairs[live[b]][0], pairs[live[b]][1], bytes[live[b]], label); continue; }
+      int t = ++time_;
+      Step c;
+      c.kind = Step::Copy;
+      c.label = label;
+      for (size_t k = b; k < e; ++k) {
+        c.args.push_back(ref(pairs[live[k]][0], t));
+        c.args.push_back(ref(pairs[live[k]][1], t));
+        c.copyBytes.push_back(bytes[live[k]]);
+        c.bytes += bytes[live[k]];
+      }
+      plan.steps.push_back(std::move(c));
+    }
+  }
+
   void emitWhile(Op* op, Plan& plan) {
     size_t n = op->operands.size();
     for (auto* v : op->operands) if (!hasStorage(v)) materializeNow(v, plan);
@@ -765,16 +850,25 @@ class Planner {
       src[i] = storageOf(v);
     }
     // phase 1: values that live in another carry slot are staged through temporaries
+    std::vector<std::array<int, 2>> stage, update;
+    std::vector<int64_t> stageBytes, updateBytes;
     for (size_t i = 0; i < n; ++i) {
       if (src[i] == slots[i]) continue;
       bool isSlot = std::find(slots.begin(), slots.end(), src[i]) != slots.end();
       if (isSlot || st_[src[i]].kind != BufRef::Temp) {
         int tmp = newStorage(op->operands[i]->type.bytes());
-        copyStep(*bodyPlan, src[i], tmp, (int64_t)op->operands[i]->type.bytes(), "loop carry stage");
+        stage.push_back({src[i], tmp});
+        stageBytes.push_back((int64_t)op->operands[i]->type.bytes());
         src[i] = tmp;
       }
     }
-    for (size_t i = 0; i < n; ++i) copyStep(*bodyPlan, src[i], slots[i], (int64_t)op->operands[i]->type.bytes(), "loop carry update");
+    multiCopyStep(*bodyPlan, stage, stageBytes, "loop carry stage");
+    // phase 2: sources are temporaries now, destinations are distinct slots: one launch moves them all
+    for (size_t i = 0; i < n; ++i) {
+      update.push_back({src[i], slots[i]});
+      updateBytes.push_back((int64_t)op->operands[i]->type.bytes());
+    }
+    multiCopyStep(*bodyPlan, update, updateBytes, "loop carry update");
     int tEnd = ++time_;
     for (size_t i = 0; i < n; ++i) ref(slots[i], tEnd);
     loops_.push_back({tStart, tEnd});

@@ -7,6 +7,7 @@
 
 #include <algorithm>
 #include <chrono>
+#include <functional>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -220,6 +221,8 @@ Executable::Executable(std::unique_ptr<CompiledProgram> prog) : prog_(std::move(
   Device& dev = Device::get();
   const char* t = getenv("MI355X_TIMING");
   timingKinds_ = t ? t : "";
+  const char* gr = getenv("MI355X_GRAPHS");   // "0" runs loop bodies launch by launch
+  useGraphs_ = !(gr && gr[0] == '0');
   loadKernels();
   if (prog_->arenaBytes > 0) arena_ = dev.alloc((size_t)prog_->arenaBytes);
   if (!prog_->constPool.empty()) {
@@ -235,6 +238,7 @@ Executable::~Executable() {
   try { dev.sync(); } catch (...) {}
   if (arena_) dev.release(arena_);
   if (consts_) dev.release(consts_);
+  for (auto& g : loopGraphs_) for (auto& e : g.second.entries) if (e.exec) mi355_graph_destroy(e.exec);
   for (auto e : eventPool_) mi355_event_destroy(e);
   for (auto& p : pending_) { mi355_event_destroy(p.a); mi355_event_destroy(p.b); }
 }
@@ -383,13 +387,26 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       break;
     }
     case Step::Copy:
+      if (!s.copyBytes.empty()) {
+        const void* srcs[16];
+        void* dsts[16];
+        size_t sizes[16];
+        size_t n = s.copyBytes.size();
+        for (size_t i = 0; i < n; ++i) {
+          srcs[i] = resolve(s.args[2 * i], in, out);
+          dsts[i] = resolve(s.args[2 * i + 1], in, out);
+          sizes[i] = (size_t)s.copyBytes[i];
+        }
+        check(mi355_copy_multi((int)n, dsts, srcs, sizes, st), "copy");
+        break;
+      }
       check(mi355_copy(resolve(s.dst, in, out), resolve(s.src, in, out), (size_t)s.bytes, st), "copy");
       break;
     case Step::Fill: break;
     case Step::While: {
       if (s.tripCount >= 0) {
         // counted loop: the trip count is known, iterations are queued back to back with no host round trip
-        for (int64_t i = 0; i < s.tripCount; ++i) runPlan(*s.bodies[0], in, out);
+        runCountedLoop(s, in, out);
       } else {
         unsigned char* flag = (unsigned char*)dev.pinnedScratch();
         while (true) {
@@ -425,6 +442,93 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
     pending_.push_back({ea, eb, kind, flops, bytes});
     if (pending_.size() > 20000) resolvePending();
   }
+}
+
+bool Executable::capturable(const Plan& p) {
+  auto it = capturable_.find(&p);
+  if (it != capturable_.end()) return it->second;
+  bool ok = true;
+  for (auto& s : p.steps) {
+    switch (s.kind) {
+      case Step::Kernel: case Step::Gemm: case Step::Conv: case Step::ScatterRows: case Step::Copy: case Step::Fill: break;
+      case Step::While: ok = ok && s.tripCount >= 0 && capturable(*s.bodies[0]); break;   // dynamic loops read a flag back on the host
+      default: ok = false; break;
+    }
+  }
+  capturable_[&p] = ok;
+  return ok;
+}
+
+// Iterations of a counted loop are identical launch sequences over fixed addresses (the counter
+// and the carries live in the arena), so after one eager iteration the body is captured into a
+// graph holding several iterations and replayed; the host then issues one launch per replay
+// instead of one per kernel.
+void Executable::runCountedLoop(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
+  Device& dev = Device::get();
+  const Plan& body = *s.bodies[0];
+  const int64_t trip = s.tripCount;
+  const bool graphOk = useGraphs_ && !capturing_ && timingKinds_.empty() && trip >= 4 && !body.steps.empty() && capturable(body);
+  if (!graphOk) {
+    for (int64_t i = 0; i < trip; ++i) runPlan(body, in, out);
+    return;
+  }
+  runPlan(body, in, out);   // first iteration eagerly: finishes lazy one-time set-up outside the capture
+  LoopGraphs& lgs = loopGraphs_[&s];
+  if (!lgs.scanned) {
+    std::function<void(const Plan&)> scan = [&](const Plan& p) {
+      auto add = [&](const BufRef& b) { if (b.kind == BufRef::Param || b.kind == BufRef::Output) lgs.external.push_back(b); };
+      for (auto& st : p.steps) {
+        for (auto& a : st.args) add(a);
+        add(st.src); add(st.dst); add(st.predBuf);
+        if (st.cond) scan(*st.cond);
+        for (auto& b : st.bodies) scan(*b);
+      }
+    };
+    scan(body);
+    lgs.scanned = true;
+  }
+  uint64_t sig = 1469598103934665603ull;
+  for (auto& b : lgs.external) sig = (sig ^ (uint64_t)(uintptr_t)resolve(b, in, out)) * 1099511628211ull;
+  LoopGraph* hit = nullptr;
+  for (auto& e : lgs.entries) if (e.exec && e.signature == sig) hit = &e;
+  if (!hit) {
+    if (lgs.entries.size() < 4) {
+      lgs.entries.emplace_back();
+      hit = &lgs.entries.back();
+    } else {
+      hit = &lgs.entries[0];
+      for (auto& e : lgs.entries) if (e.lastUse < hit->lastUse) hit = &e;
+      // replays of the evicted graph may still be queued
+      dev.sync();
+      mi355_graph_destroy(hit->exec);
+      hit->exec = nullptr;
+    }
+    const int64_t per = std::max<int64_t>(1, std::min<int64_t>(trip - 1, 1024 / (int64_t)body.steps.size()));
+    mi355_stream_t st = dev.stream();
+    check(mi355_capture_begin(st), "graph capture");
+    capturing_ = true;
+    try {
+      for (int64_t i = 0; i < per; ++i) runPlan(body, in, out);
+    } catch (...) {
+      capturing_ = false;
+      mi355_graph_t dead = nullptr;
+      int n = 0;
+      if (mi355_capture_end(st, &dead, &n) == 0 && dead) mi355_graph_destroy(dead);
+      throw;
+    }
+    capturing_ = false;
+    int nodes = 0;
+    check(mi355_capture_end(st, &hit->exec, &nodes), "graph instantiate");
+    hit->signature = sig;
+    hit->itersPerLaunch = per;
+    static const bool verbose = getenv("MI355X_VERBOSE") != nullptr;
+    if (verbose) fprintf(stderr, "[mi355x] loop body captured: %lld iteration(s), %d graph nodes\n", (long long)per, nodes);
+  }
+  hit->lastUse = ++graphClock_;
+  LoopGraph& lg = *hit;
+  int64_t left = trip - 1;
+  for (; left >= lg.itersPerLaunch; left -= lg.itersPerLaunch) check(mi355_graph_launch(lg.exec, dev.stream()), "graph launch");
+  for (; left > 0; --left) runPlan(body, in, out);
 }
 
 void Executable::runPlan(const Plan& plan, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {

@@ -100,6 +100,22 @@ class Executable {
   std::map<std::string, KindStat> stats_;
   std::string timingKinds_;
 
+  // Captured bodies of counted loops.  A graph bakes in the addresses of the call's argument and
+  // result buffers, so it is kept with a signature of those and rebuilt when they change.
+  struct LoopGraph { mi355_graph_t exec = nullptr; uint64_t signature = 0; int64_t itersPerLaunch = 0; uint64_t lastUse = 0; };
+  struct LoopGraphs {
+    bool scanned = false;
+    std::vector<BufRef> external;      // argument / result buffers the body touches
+    std::vector<LoopGraph> entries;    // a few recent address sets (buffers recycle through the allocator)
+  };
+  std::map<const Step*, LoopGraphs> loopGraphs_;
+  uint64_t graphClock_ = 0;
+  std::map<const Plan*, bool> capturable_;
+  bool useGraphs_ = true;
+  bool capturing_ = false;
+  bool capturable(const Plan& p);
+  void runCountedLoop(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
+
   void loadKernels();
   void* resolve(const BufRef& r, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) const;
   void runPlan(const Plan& plan, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
