@@ -19,7 +19,9 @@
 #include <cstring>
 #include <numeric>
 #include <sstream>
+#include <memory>
 #include <unordered_map>
+#include <unordered_set>
 
 namespace mi355 {
 
@@ -204,6 +206,12 @@ class Emitter {
   void pre(const std::string& s) { pre_ += "  " + s + "\n"; }
   void body(const std::string& s) { body_.back() += std::string(2 + 2 * body_.size(), ' ') + s + "\n"; }
   void emit(bool inBody, const std::string& s) { (inBody || guard_ > 0) ? body(s) : pre(s); }
+
+  // Row programs: results of reductions finished earlier in the same kernel, as variables that
+  // hold the value for the row this wavefront / workgroup owns.
+  std::unordered_map<Value*, std::string> rowScalars_;
+  std::vector<IdxDim> rowKept_;           // index of the current row over the kept dims
+  void shareLeavesFrom(const Emitter& o) { leaves_ = o.leaves_; leafIndex_ = o.leafIndex_; }
 
   int leafId(Value* v) {
     auto it = leafIndex_.find(v);
@@ -450,6 +458,18 @@ class Emitter {
   }
 
   std::string genUncached(Value* v, const Index& idx) {
+    auto rs = rowScalars_.find(v);
+    if (rs != rowScalars_.end()) {
+      // only the current row's value exists: the index must be the row index itself
+      Index m = multi(idx);
+      if (m.dims.size() != rowKept_.size()) throw CompileError("row program: reduction result indexed through a reshape");
+      for (size_t q = 0; q < m.dims.size(); ++q) {
+        if (v->type.dims[q] == 1) continue;
+        const IdxDim& d = m.dims[q];
+        if (d.isConst || d.inBody || d.coef != 0 || d.base != rowKept_[q].base) throw CompileError("row program: reduction result read at another row");
+      }
+      return rs->second;
+    }
     if (isLeaf_(v)) return load(v, idx);
     Op* op = v->def;
     if (!op) throw CompileError("codegen: region argument " + v->name + " is not materialised");
@@ -1079,8 +1099,14 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     s << kernelHeader(em.leaves_, outs) << " {\n";
     // many partials per output: one wavefront folds an output (lanes stride over the
     // partials, then a butterfly); few partials: one lane per output
-    const bool wavePerOut = P >= 16;
-    if (wavePerOut) {
+    // a whole workgroup per output when there are hundreds of partials (every lane issues its few
+    // loads at once, so the fold costs one memory round trip)
+    const bool blockPerOut = P >= 256;
+    const bool wavePerOut = !blockPerOut && P >= 16;
+    if (blockPerOut) {
+      s << "  const int lane = threadIdx.x & 63;\n";
+      s << "  const " << IT << " kk = (" << IT << ")blockIdx.x;\n";
+    } else if (wavePerOut) {
       s << "  const int lane = threadIdx.x & 63;\n";
       s << "  const " << IT << " kk = (" << IT << ")blockIdx.x * 4 + (threadIdx.x >> 6);\n  if (kk >= " << Kn << ") return;\n";
     } else {
@@ -1089,8 +1115,17 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     s << em.pre_;
     for (size_t j = 0; j < nr; ++j) {
       std::string part = "part" + std::to_string(j) + "[p * " + std::to_string(Kn) + " + kk]";
+      std::string ST = ops[j].accT == "bool" ? "int" : ops[j].accT;
       s << "  { " << ops[j].accT << " a = " << ops[j].identity << ";\n";
-      if (wavePerOut) {
+      if (blockPerOut) {
+        s << "    #pragma unroll 8\n    for (" << IT << " p = threadIdx.x; p < " << P << "; p += 256) a = " << ops[j].combine("a", part) << ";\n";
+        s << "    #pragma unroll\n    for (int o = 32; o > 0; o >>= 1) a = " << ops[j].combine("a", shflXor(ops[j].accT, "a", "o")) << ";\n";
+        s << "    __shared__ " << ST << " fm" << j << "[4];\n";
+        s << "    if (lane == 0) fm" << j << "[threadIdx.x >> 6] = a;\n    __syncthreads();\n";
+        s << "    if (threadIdx.x == 0) {\n";
+        s << "    a = (" << ops[j].accT << ")fm" << j << "[0];\n";
+        s << "    for (int w = 1; w < 4; ++w) a = " << ops[j].combine("a", "(" + ops[j].accT + ")fm" + std::to_string(j) + "[w]") << ";\n";
+      } else if (wavePerOut) {
         s << "    #pragma unroll 4\n    for (" << IT << " p = lane; p < " << P << "; p += 64) a = " << ops[j].combine("a", part) << ";\n";
         s << "    #pragma unroll\n    for (int o = 32; o > 0; o >>= 1) a = " << ops[j].combine("a", shflXor(ops[j].accT, "a", "o")) << ";\n";
         s << "    if (lane == 0) {\n";
@@ -1103,7 +1138,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     s << "}\n";
     Launch l;
     l.source = s.str();
-    l.grid[0] = (unsigned)(wavePerOut ? (Kn + 3) / 4 : (Kn + 255) / 256);
+    l.grid[0] = (unsigned)(blockPerOut ? Kn : wavePerOut ? (Kn + 3) / 4 : (Kn + 255) / 256);
     l.block[0] = 256;
     for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
     for (size_t j = 0; j < nr; ++j) { KArg a; a.kind = KArg::Work; a.workOffset = workOff[j]; l.args.push_back(a); }
@@ -1346,6 +1381,190 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     for (auto* v : il) if (std::find(fc.leaves.begin(), fc.leaves.end(), v) == fc.leaves.end()) fc.leaves.push_back(v);
     fc.workspaceBytes = wb;
   }
+  return fc;
+}
+
+// ------------------------------------------------------------------ row programs
+// One kernel per group of rows: every phase walks the row once (from HBM the first time, from
+// cache afterwards), phase p may use the reductions finished in phases < p, and the last walk
+// stores the elementwise results.  Softmax is (max | sum of exp | divide), LayerNorm is
+// (sum, sum of squares | normalise); HBM traffic is one read and one write of the tensor.
+FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) {
+  Op* r0 = rp.phases.at(0).at(0);
+  Value* x0 = r0->operands[0];
+  const std::vector<int64_t>& shape = x0->type.dims;
+  int rank = (int)shape.size();
+  std::vector<int64_t> rdims = r0->ints("dimensions");
+  std::sort(rdims.begin(), rdims.end());
+  std::vector<bool> isRed(rank, false);
+  for (auto d : rdims) isRed[d] = true;
+  std::vector<int64_t> keptShape, redShape;
+  std::vector<int> keptDims, redDims;
+  for (int d = 0; d < rank; ++d) {
+    if (isRed[d]) { redShape.push_back(shape[d]); redDims.push_back(d); }
+    else { keptShape.push_back(shape[d]); keptDims.push_back(d); }
+  }
+  for (size_t q = 0; q < redDims.size(); ++q)
+    if (redDims[q] != rank - (int)redDims.size() + (int)q) throw CompileError("row program: reduced dims are not the trailing dims");
+  int64_t Kn = 1, Rn = 1;
+  for (auto d : keptShape) Kn *= d;
+  for (auto d : redShape) Rn *= d;
+
+  std::unordered_set<Value*> inGroup;
+  std::vector<Op*> reduces;
+  for (auto& ph : rp.phases) for (auto* r : ph) { reduces.push_back(r); inGroup.insert(r->result()); }
+  for (auto* v : rp.fullRoots) inGroup.insert(v);
+  for (auto* v : rp.keptRoots) inGroup.insert(v);
+  LeafPredicate inner = [&](Value* v) { return !inGroup.count(v) && isLeaf(v); };
+
+  int V = 8;
+  for (auto* r : reduces) V = std::min(V, pickVector(r->operands[0]->type));
+  for (auto* v : rp.fullRoots) V = std::min(V, pickVector(v->type));
+  while (V > 1 && (redShape.empty() || redShape.back() % V != 0)) V >>= 1;
+  if (Rn < 64 * V) V = 1;
+  const int64_t vecs = (Rn + V - 1) / V;
+  const bool wavePerRow = vecs <= 256;
+  const bool i64 = (double)Kn * (double)Rn >= 2147483000.0;
+  const std::string IT = i64 ? "i64" : "int";
+
+  std::unordered_map<Value*, std::string> scalars;
+  std::ostringstream b;   // kernel body; the header needs the final leaf list
+  if (wavePerRow) {
+    b << "  const int r_tid = threadIdx.x & 63, r_step = 64;\n";
+    b << "  const " << IT << " kk = (" << IT << ")blockIdx.x * 4 + (threadIdx.x >> 6);\n";
+    b << "  if (kk >= " << Kn << ") return;\n";
+  } else {
+    b << "  const int r_tid = threadIdx.x, r_step = 256;\n";
+    b << "  const " << IT << " kk = (" << IT << ")blockIdx.x;\n";
+  }
+  b << "  const int r_end = " << vecs << ";\n";
+  std::vector<RedOp> ops;
+  for (size_t i = 0; i < reduces.size(); ++i) {
+    ops.push_back(makeRedOp(*reduces[i]));
+    b << "  " << ops[i].accT << " red" << i << ";\n";
+  }
+
+  // per phase: a fresh emitter (own temporaries inside its own scope) over the shared leaf list
+  std::unique_ptr<Emitter> prev;
+  auto newEmitter = [&]() {
+    auto em = std::make_unique<Emitter>(inner, V, i64);
+    if (prev) em->shareLeavesFrom(*prev);
+    em->rowScalars_ = scalars;
+    return em;
+  };
+  // index of element (row kk, position rb + v) and of the row itself
+  auto rowIndex = [&](Emitter& em, std::string& loopPre, Index& full, Index& keptIdx) {
+    IdxDim klin;
+    klin.isConst = false; klin.base = "kk"; klin.coef = 0; klin.mult = 1;
+    auto kd = em.delinearize(klin, keptShape);
+    em.rowKept_ = kd;
+    keptIdx = em.multiIndex(kd, keptShape);
+    std::string savedPre = em.pre_;
+    em.pre_.clear();
+    IdxDim rlin;
+    rlin.isConst = false; rlin.base = "rb"; rlin.coef = V > 1 ? 1 : 0; rlin.mult = V;
+    auto rd = em.delinearize(rlin, redShape);
+    std::vector<IdxDim> dims(rank);
+    for (size_t q = 0; q < keptDims.size(); ++q) dims[keptDims[q]] = kd[q];
+    for (size_t q = 0; q < redDims.size(); ++q) dims[redDims[q]] = rd[q];
+    full = em.multiIndex(dims, shape);
+    loopPre = em.pre_;
+    em.pre_ = savedPre;
+  };
+
+  size_t base = 0;
+  for (size_t p = 0; p < rp.phases.size(); ++p) {
+    auto& ph = rp.phases[p];
+    auto em = newEmitter();
+    std::string idxPre;
+    Index full, keptIdx;
+    rowIndex(*em, idxPre, full, keptIdx);
+    std::string savedPre = em->pre_;
+    em->pre_.clear();
+    std::vector<std::string> vals;
+    for (auto* r : ph) vals.push_back(em->gen(r->operands[0], full));
+    std::string loopPre = idxPre + em->pre_;
+    em->pre_ = savedPre;
+    std::vector<std::string> inits;
+    for (auto* r : ph) inits.push_back(em->gen(r->operands[1], em->multiIndex({}, {})));
+    b << "  {\n" << em->pre_;
+    for (size_t j = 0; j < ph.size(); ++j) b << "  " << ops[base + j].accT << " acc" << j << " = " << ops[base + j].identity << ";\n";
+    b << "  #pragma unroll 4\n  for (int rv = r_tid; rv < r_end; rv += r_step) {\n";
+    b << "    const int rb = rv * " << V << ";\n" << loopPre;
+    b << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n" << em->body_.front();
+    for (size_t j = 0; j < ph.size(); ++j) b << "      acc" << j << " = " << ops[base + j].combine("acc" + std::to_string(j), vals[j]) << ";\n";
+    b << "    }\n  }\n";
+    for (size_t j = 0; j < ph.size(); ++j) {
+      const RedOp& o = ops[base + j];
+      std::string a = "acc" + std::to_string(j);
+      b << "  #pragma unroll\n  for (int o = 32; o > 0; o >>= 1) " << a << " = " << o.combine(a, shflXor(o.accT, a, "o")) << ";\n";
+      if (!wavePerRow) {
+        std::string ST = o.accT == "bool" ? "int" : o.accT;
+        std::string sm = "sm" + std::to_string(base + j);
+        b << "  __shared__ " << ST << " " << sm << "[4];\n";
+        b << "  if ((threadIdx.x & 63) == 0) " << sm << "[threadIdx.x >> 6] = " << a << ";\n  __syncthreads();\n";
+        b << "  " << a << " = (" << o.accT << ")" << sm << "[0];\n";
+        b << "  for (int w = 1; w < 4; ++w) " << a << " = " << o.combine(a, "(" + o.accT + ")" + sm + "[w]") << ";\n";
+      }
+      b << "  red" << (base + j) << " = " << roundTo(o.dt, o.combine(inits[j], a)) << ";\n";
+    }
+    b << "  }\n";
+    for (size_t j = 0; j < ph.size(); ++j) scalars[ph[j]->result()] = "red" + std::to_string(base + j);
+    base += ph.size();
+    prev = std::move(em);
+  }
+
+  // last walk: elementwise results of the full shape, then the per-row results
+  {
+    auto em = newEmitter();
+    std::string idxPre;
+    Index full, keptIdx;
+    rowIndex(*em, idxPre, full, keptIdx);
+    std::string savedPre = em->pre_;
+    em->pre_.clear();
+    std::vector<std::string> vals;
+    for (auto* v : rp.fullRoots) vals.push_back(em->gen(v, full));
+    std::string loopPre = idxPre + em->pre_;
+    em->pre_ = savedPre;
+    std::vector<std::string> kvals;
+    for (auto* v : rp.keptRoots) kvals.push_back(em->gen(v, keptIdx));
+    b << "  {\n" << em->pre_;
+    if (!rp.fullRoots.empty()) {
+      b << "  #pragma unroll 2\n  for (int rv = r_tid; rv < r_end; rv += r_step) {\n";
+      b << "    const int rb = rv * " << V << ";\n" << loopPre;
+      for (size_t j = 0; j < rp.fullRoots.size(); ++j) b << "    Vec<" << storageT(rp.fullRoots[j]->type.dt) << ", " << V << "> ov" << j << ";\n";
+      b << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n" << em->body_.front();
+      for (size_t j = 0; j < rp.fullRoots.size(); ++j) b << "      ov" << j << ".e[v] = " << storeExpr(rp.fullRoots[j]->type.dt, vals[j]) << ";\n";
+      b << "    }\n";
+      for (size_t j = 0; j < rp.fullRoots.size(); ++j)
+        b << "    *(Vec<" << storageT(rp.fullRoots[j]->type.dt) << ", " << V << ">*)(outF" << j << " + (" << IT << ")kk * " << Rn << " + rb) = ov" << j << ";\n";
+      b << "  }\n";
+    }
+    b << "  if (r_tid == 0) {\n";
+    for (size_t j = 0; j < rp.keptRoots.size(); ++j) b << "    outK" << j << "[kk] = " << storeExpr(rp.keptRoots[j]->type.dt, kvals[j]) << ";\n";
+    for (size_t i = 0; i < reduces.size(); ++i) b << "    outR" << i << "[kk] = " << storeExpr(ops[i].dt, "red" + std::to_string(i)) << ";\n";
+    b << "  }\n  }\n";
+    prev = std::move(em);
+  }
+
+  std::vector<std::string> outs;
+  for (size_t j = 0; j < rp.fullRoots.size(); ++j) outs.push_back(storageT(rp.fullRoots[j]->type.dt) + "* __restrict__ outF" + std::to_string(j));
+  for (size_t j = 0; j < rp.keptRoots.size(); ++j) outs.push_back(storageT(rp.keptRoots[j]->type.dt) + "* __restrict__ outK" + std::to_string(j));
+  for (size_t i = 0; i < reduces.size(); ++i) outs.push_back(storageT(ops[i].dt) + "* __restrict__ outR" + std::to_string(i));
+  if (prev->leaves_.size() + outs.size() > 60) throw CompileError("row program: too many kernel arguments");
+  std::ostringstream s;
+  s << kPrelude << kernelHeader(prev->leaves_, outs) << " {\n" << b.str() << "}\n";
+  FusedCode fc;
+  Launch l;
+  l.source = s.str();
+  l.grid[0] = (unsigned)(wavePerRow ? (Kn + 3) / 4 : Kn);
+  l.block[0] = 256;
+  for (auto* v : prev->leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
+  for (auto* v : rp.fullRoots) { KArg a; a.kind = KArg::Out; a.value = v; l.args.push_back(a); }
+  for (auto* v : rp.keptRoots) { KArg a; a.kind = KArg::Out; a.value = v; l.args.push_back(a); }
+  for (auto* r : reduces) { KArg a; a.kind = KArg::Out; a.value = r->result(); l.args.push_back(a); }
+  fc.leaves = prev->leaves_;
+  fc.launches.push_back(std::move(l));
   return fc;
 }
 

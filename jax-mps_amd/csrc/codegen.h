@@ -41,6 +41,15 @@ using LeafPredicate = std::function<bool(Value*)>;
 FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf);
 FusedCode generateLoopKernel(const std::vector<Value*>& roots, const LeafPredicate& isLeaf);
 
+// Reductions over the trailing dims in dependency phases plus the elementwise values that
+// consume them, computed row by row in one kernel.
+struct RowProgram {
+  std::vector<std::vector<Op*>> phases;   // phase p may read the results of phases < p
+  std::vector<Value*> fullRoots;          // stored values of the unreduced shape
+  std::vector<Value*> keptRoots;          // stored values of the reduced (per-row) shape
+};
+FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf);
+
 // In-place window write of a dynamic_update_slice: iterates over the update
 // tensor and stores into `dus` result storage (which already holds the operand).
 FusedCode generateDusKernel(Op* dus, const LeafPredicate& isLeaf);

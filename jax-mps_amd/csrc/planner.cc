@@ -286,7 +286,7 @@ class Planner {
         }
         continue;
       }
-      if (n == "reduce") { emitReduce(op, r, plan); continue; }
+      if (n == "reduce") { if (!tryRowProgram(op, r, pos, plan)) emitReduce(op, r, plan); continue; }
       if (n == "dot_general" || n == "dot") { emitDot(op, plan); continue; }
       if (n == "convolution") { emitConv(op, plan); continue; }
       if (n == "scatter") { emitScatter(op, plan); continue; }
@@ -402,6 +402,134 @@ class Planner {
     if (hasStorage(v)) { out.push_back(v); return; }
     if (!v->def || !isFusibleOp(*v->def) || needMat_[v]) { out.push_back(v); return; }
     for (auto* o : v->def->operands) collectLeavesOf(o, out, seen);
+  }
+
+  // Softmax / LayerNorm shaped subgraphs: reductions over the trailing dims, elementwise values
+  // that read them back through a broadcast, possibly further reductions of those, all computed
+  // in one kernel that owns whole rows (reference: the mps.softmax / mps.layer_norm custom calls
+  // its fusion passes produce, passes/fuse_softmax.cc:174-247, passes/fuse_layer_norm.cc:229-354).
+  bool tryRowProgram(Op* op, Region& r, size_t pos, Plan& plan) {
+    static const bool enabled = !(getenv("MI355X_ROW_PROGRAMS") && getenv("MI355X_ROW_PROGRAMS")[0] == '0');
+    if (!enabled || !isSimpleReduce(*op)) return false;
+    const TensorType& xt = op->operands[0]->type;
+    std::vector<int64_t> rd = op->ints("dimensions");
+    std::sort(rd.begin(), rd.end());
+    int rank = xt.rank();
+    if (rd.empty() || (int)rd.size() >= rank) return false;
+    for (size_t q = 0; q < rd.size(); ++q) if (rd[q] != rank - (int)rd.size() + (int)q) return false;
+    std::vector<int64_t> keptShape(xt.dims.begin(), xt.dims.end() - rd.size());
+    int64_t Kn = 1, Rn = 1;
+    for (auto d : keptShape) Kn *= d;
+    for (size_t q = keptShape.size(); q < xt.dims.size(); ++q) Rn *= xt.dims[q];
+    if (Kn < 256 || Rn < 2 || Rn > 32768) return false;
+
+    RowProgram rp;
+    std::unordered_map<Value*, int> phaseOf;
+    std::unordered_set<Op*> inlined;      // fusible ops evaluated inside the kernel
+    std::vector<Op*> rootOps, candidates;
+    std::vector<std::vector<Op*>> candidateDeps;
+    // can `v` be evaluated in the kernel?  dep = 1 + the latest phase it needs
+    std::function<bool(Value*, int&, std::vector<Op*>&)> can = [&](Value* v, int& dep, std::vector<Op*>& seen) -> bool {
+      if (hasStorage(v)) return true;
+      auto ph = phaseOf.find(v);
+      if (ph != phaseOf.end()) { dep = std::max(dep, ph->second + 1); return true; }
+      Op* d = v->def;
+      if (!d || !isFusibleOp(*d) || d->results.size() != 1 || d->parent != &r) return false;
+      if (std::find(seen.begin(), seen.end(), d) != seen.end()) return true;
+      seen.push_back(d);
+      if (seen.size() > 256) return false;
+      for (auto* o : d->operands) if (!can(o, dep, seen)) return false;
+      return true;
+    };
+    const size_t kWindow = 96;
+    for (size_t q = pos; q < r.ops.size() && q <= pos + kWindow; ++q) {
+      Op* y = r.ops[q].get();
+      if (emitted_.count(y)) continue;
+      if (y->name == "reduce") {
+        if (!isSimpleReduce(*y) || y->operands[0]->type.dims != xt.dims) { if (y == op) return false; continue; }
+        std::vector<int64_t> yd = y->ints("dimensions");
+        std::sort(yd.begin(), yd.end());
+        if (yd != rd) continue;
+        int dep = 0;
+        std::vector<Op*> seen;
+        if (!can(y->operands[0], dep, seen) || !can(y->operands[1], dep, seen)) { if (y == op) return false; continue; }
+        if (dep > (int)rp.phases.size()) continue;
+        if (dep == (int)rp.phases.size()) rp.phases.emplace_back();
+        if (rp.phases[dep].size() >= 4) continue;
+        rp.phases[dep].push_back(y);
+        phaseOf[y->result()] = dep;
+        for (auto* z : seen) inlined.insert(z);
+        continue;
+      }
+      if (rp.phases.empty()) return false;
+      if (!isFusibleOp(*y) || y->results.size() != 1) continue;
+      Value* w = y->result();
+      if (!needMat_[w] || hasStorage(w) || !takesKernel(y)) continue;
+      if (w->type.dims != xt.dims && w->type.dims != keptShape) continue;
+      int dep = 0;
+      std::vector<Op*> seen;
+      if (!can(w, dep, seen) || dep == 0) continue;
+      candidates.push_back(y);
+      candidateDeps.push_back(std::move(seen));
+    }
+    if (rp.phases.empty() || rp.phases[0].empty() || rp.phases[0][0] != op) return false;
+    // Candidates in reverse program order: one whose readers are all inside the kernel is not
+    // stored (it is recomputed where needed); the others become outputs.
+    std::unordered_set<Op*> members(inlined.begin(), inlined.end());
+    for (auto& ph : rp.phases) for (auto* y : ph) members.insert(y);
+    std::vector<Op*> dropped;
+    for (int c = (int)candidates.size() - 1; c >= 0; --c) {
+      Op* y = candidates[c];
+      Value* w = y->result();
+      bool inside = !w->users.empty();
+      for (Op* u : w->users) if (!members.count(u)) inside = false;
+      if (inside) continue;   // stays an inlined intermediate if a member reads it, otherwise untouched
+      if (rp.fullRoots.size() + rp.keptRoots.size() >= 8) continue;
+      (w->type.dims == xt.dims ? rp.fullRoots : rp.keptRoots).push_back(w);
+      rootOps.push_back(y);
+      members.insert(y);
+      for (auto* z : candidateDeps[c]) { inlined.insert(z); members.insert(z); }
+    }
+    if (rp.phases.size() == 1 && rp.fullRoots.empty()) return false;   // plain reductions: the partial-sum kernels do better
+    // inlined values that were going to be written to memory: dropped when every reader is in the kernel
+    for (auto* z : inlined) {
+      Value* w = z->result();
+      if (!needMat_[w] || hasStorage(w)) continue;
+      if (std::find(rootOps.begin(), rootOps.end(), z) != rootOps.end()) continue;
+      bool inside = true;
+      for (Op* u : w->users) if (!members.count(u)) inside = false;
+      if (inside) { dropped.push_back(z); continue; }
+      bool full = w->type.dims == xt.dims, kept = w->type.dims == keptShape;
+      if ((!full && !kept) || !takesKernel(z) || rp.fullRoots.size() + rp.keptRoots.size() >= 10) return false;
+      (full ? rp.fullRoots : rp.keptRoots).push_back(w);
+      rootOps.push_back(z);
+    }
+    FusedCode fc;
+    try {
+      fc = generateRowProgram(rp, leafPred());
+    } catch (const CompileError&) {
+      return false;
+    }
+    std::vector<Value*> outs;
+    std::string label = "rows:";
+    for (auto& ph : rp.phases) {
+      for (auto* y : ph) {
+        bind(y->result(), newStorage(y->result()->type.bytes()));
+        outs.push_back(y->result());
+        emitted_.insert(y);
+        label += "reduce,";
+      }
+      label += "|";
+    }
+    for (auto* y : rootOps) {
+      bind(y->result(), newStorage(y->result()->type.bytes()));
+      outs.push_back(y->result());
+      emitted_.insert(y);
+      label += y->name + ",";
+    }
+    for (auto* z : dropped) emitted_.insert(z);
+    addFused(plan, fc, label + " " + xt.str(), outs);
+    return true;
   }
 
   void emitReduce(Op* op, Region& r, Plan& plan) {
