@@ -16,6 +16,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <numeric>
 #include <sstream>
@@ -57,13 +58,13 @@ template <typename T> __device__ __forceinline__ T ipow(T a, T b) {
 template <typename T> __device__ __forceinline__ T idiv(T a, T b) { return b == (T)0 ? (T)-1 : ((b == (T)-1) ? (T)(0 - a) : (T)(a / b)); }
 template <typename T> __device__ __forceinline__ T irem(T a, T b) { return b == (T)0 ? a : ((b == (T)-1) ? (T)0 : (T)(a % b)); }
 // 16-bit results keep 8 (bf16) or 11 (f16) significand bits: the hardware exponential is exact enough there
-__device__ __forceinline__ float tanh_fast(float x) { float t = __expf(-2.f * fabsf(x)); return copysignf((1.f - t) / (1.f + t), x); }
+__device__ __forceinline__ float tanh_fast(float x) { float t = __expf(-2.f * fabsf(x)); return copysignf((1.f - t) * __builtin_amdgcn_rcpf(1.f + t), x); }
 // f32 tanh to a few ulp: odd polynomial near 0 (where 1 - exp cancels), exponential form elsewhere
 __device__ __forceinline__ float tanh_f32(float x) {
   float ax = fabsf(x), x2 = x * x;
   float p = x * (1.f + x2 * (-0.33333334f + x2 * (0.13333334f + x2 * (-0.05396825f + x2 * (0.021869488f + x2 * -0.008863236f)))));
   float t = __expf(-2.f * ax);
-  float r = copysignf(__fdividef(1.f - t, 1.f + t), x);
+  float r = copysignf((1.f - t) * __builtin_amdgcn_rcpf(1.f + t), x);
   return ax < 0.3f ? p : r;
 }
 __device__ __forceinline__ float sgnf(float x) { return (x != x || x == 0.f) ? x : (x > 0.f ? 1.f : -1.f); }
@@ -431,9 +432,14 @@ class Emitter {
   std::unordered_map<std::string, std::string> vecLoads_;
   std::vector<std::unordered_map<std::string, std::string>> cache_;
 
-  std::string def(const TensorType& t, const std::string& expr, bool inBody) {
+  // 16-bit float results are computed in fp32.  Inside a fused chain they are rounded to their
+  // own precision only where the program asks for the narrowing (convert and friends) or where
+  // they are stored; rounding after every arithmetic op (MI355X_STRICT_BF16=1) costs two
+  // instructions per op and only loses accuracy.
+  std::string def(const TensorType& t, const std::string& expr, bool inBody, bool narrowing = true) {
+    static const bool strict = getenv("MI355X_STRICT_BF16") && getenv("MI355X_STRICT_BF16")[0] == '1';
     std::string name = fresh("t");
-    emit(inBody, "const " + computeT(t.dt) + " " + name + " = " + roundTo(t.dt, expr) + ";");
+    emit(inBody, "const " + computeT(t.dt) + " " + name + " = " + ((strict || narrowing) ? roundTo(t.dt, expr) : expr) + ";");
     return name;
   }
 
@@ -477,7 +483,9 @@ class Emitter {
     const TensorType& rt = v->type;
     bool inB = idx.lane();
     auto in = [&](int k) { return gen(op->operands[k], idx); };
-    auto bin = [&](const std::string& e) { return def(rt, e, inB); };
+    const bool narrowing = n == "convert" || n == "reduce_precision" || n == "bitcast_convert" || n == "iota" || n == "round_nearest_even" ||
+                           n == "round_nearest_afz" || n == "floor" || n == "ceil";
+    auto bin = [&](const std::string& e) { return def(rt, e, inB, narrowing); };
     DType odt = op->operands.empty() ? rt.dt : op->operands[0]->type.dt;
     bool isF = isFloat(rt.dt), isD = rt.dt == DType::F64, isP = rt.dt == DType::Pred;
     std::string sfx = isD ? "" : "f";
@@ -1427,6 +1435,10 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
   const bool i64 = (double)Kn * (double)Rn >= 2147483000.0;
   const std::string IT = i64 ? "i64" : "int";
 
+  // short rows are walked by fully unrolled loops: the compiler then keeps the row (and pure
+  // functions of it) in registers from one phase to the next instead of re-reading it
+  const int64_t walks = (vecs + (wavePerRow ? 64 : 256) - 1) / (wavePerRow ? 64 : 256);
+  const int walkUnroll = walks <= 8 ? (int)walks : 4;
   std::unordered_map<Value*, std::string> scalars;
   std::ostringstream b;   // kernel body; the header needs the final leaf list
   if (wavePerRow) {
@@ -1489,7 +1501,7 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
     for (auto* r : ph) inits.push_back(em->gen(r->operands[1], em->multiIndex({}, {})));
     b << "  {\n" << em->pre_;
     for (size_t j = 0; j < ph.size(); ++j) b << "  " << ops[base + j].accT << " acc" << j << " = " << ops[base + j].identity << ";\n";
-    b << "  #pragma unroll 4\n  for (int rv = r_tid; rv < r_end; rv += r_step) {\n";
+    b << "  #pragma unroll " << walkUnroll << "\n  for (int rv = r_tid; rv < r_end; rv += r_step) {\n";
     b << "    const int rb = rv * " << V << ";\n" << loopPre;
     b << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n" << em->body_.front();
     for (size_t j = 0; j < ph.size(); ++j) b << "      acc" << j << " = " << ops[base + j].combine("acc" + std::to_string(j), vals[j]) << ";\n";
@@ -1530,7 +1542,7 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
     for (auto* v : rp.keptRoots) kvals.push_back(em->gen(v, keptIdx));
     b << "  {\n" << em->pre_;
     if (!rp.fullRoots.empty()) {
-      b << "  #pragma unroll 2\n  for (int rv = r_tid; rv < r_end; rv += r_step) {\n";
+      b << "  #pragma unroll " << walkUnroll << "\n  for (int rv = r_tid; rv < r_end; rv += r_step) {\n";
       b << "    const int rb = rv * " << V << ";\n" << loopPre;
       for (size_t j = 0; j < rp.fullRoots.size(); ++j) b << "    Vec<" << storageT(rp.fullRoots[j]->type.dt) << ", " << V << "> ov" << j << ";\n";
       b << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n" << em->body_.front();

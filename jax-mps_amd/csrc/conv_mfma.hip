@@ -25,6 +25,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <vector>
 #include <cstdlib>
 
 #include "hip_abi.h"
@@ -42,6 +43,7 @@ struct ConvP {
   int M, N, K;
   int Nb, C;
   int in0, in1, k0n, k1n, o0n, o1n;
+  int kb0, ks0, kc0, kb1, ks1, kc1;   // window taps visited: kb + ks * t, t < kc (all of them unless a dilation class narrows it)
   int s0, s1, p0, p1, ld0, ld1, rd0, rd1, rev0, rev1;
   int lhsB, lhsF, lhsS0, lhsS1, rhsI, rhsO, rhsS0, rhsS1, outB, outF, outS0, outS1;
   int bFast;            // 1: m = (o0, o1, b) with b fastest; 0: m = (b, o0, o1)
@@ -125,8 +127,8 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
   if (!KFLAT) {
     int tap = ktBegin / p.cTiles;
     nc = (ktBegin - tap * p.cTiles) * BK;
-    nk0 = tap / p.k1n;
-    nk1 = tap - nk0 * p.k1n;
+    nk0 = tap / p.kc1;
+    nk1 = tap - nk0 * p.kc1;
   }
   constexpr int NROW = AMODE == 0 ? NAS : (AMODE == 1 ? NA4 : 1);
   int offA[NROW];
@@ -134,8 +136,8 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
   auto newTap = [&]() {
     if (KFLAT) return;
 #pragma unroll
-    for (int i = 0; i < NROW; ++i) offA[i] = tapOffset(p, rowsA[i], nk0, nk1);
-    toffB = rhsTapOffset(p, nk0, nk1);
+    for (int i = 0; i < NROW; ++i) offA[i] = tapOffset(p, rowsA[i], p.kb0 + p.ks0 * nk0, p.kb1 + p.ks1 * nk1);
+    toffB = rhsTapOffset(p, p.kb0 + p.ks0 * nk0, p.kb1 + p.ks1 * nk1);
   };
   newTap();
   // per-thread constants of the loaders
@@ -210,7 +212,7 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
       nc += BK;
       if (nc >= p.C) {
         nc = 0;
-        if (++nk1 == p.k1n) { nk1 = 0; ++nk0; }
+        if (++nk1 == p.kc1) { nk1 = 0; ++nk0; }
         newTap();
       }
     }
@@ -312,18 +314,53 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
   }
 }
 
-// out(m, n) = sum over splits of partial[s][m][n], in split order
+// out(m, n) = sum over splits of partial[s][m][n].  32 consecutive outputs per workgroup, the
+// splits dealt round-robin to 8 groups of lanes whose sums are then added in group order, so
+// the result depends only on the split count, never on timing.
 __global__ void __launch_bounds__(256) conv_fold_partials(const float* __restrict__ part, float* __restrict__ out, ConvP p) {
-  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
-  long long total = (long long)p.M * p.N;
-  if (i >= total) return;
-  int m = (int)(i / p.N), n = (int)(i - (long long)m * p.N);
+  __shared__ float sm[8][33];
+  const int lane = threadIdx.x & 31, grp = threadIdx.x >> 5;
+  const long long total = (long long)p.M * p.N;
+  const long long i = (long long)blockIdx.x * 32 + lane;
   float s = 0.f;
-  for (int z = 0; z < p.splitK; ++z) s += part[(long long)z * total + i];
+  if (i < total) {
+#pragma unroll 4
+    for (int z = grp; z < p.splitK; z += 8) s += part[(long long)z * total + i];
+  }
+  sm[grp][lane] = s;
+  __syncthreads();
+  if (grp != 0 || i >= total) return;
+#pragma unroll
+  for (int g = 1; g < 8; ++g) s += sm[g][lane];
+  int m = (int)(i / p.N), n = (int)(i - (long long)m * p.N);
   int b, o0, o1;
   if (p.bFast) { b = m % p.Nb; int t = m / p.Nb; o1 = t % p.o1n; o0 = t / p.o1n; }
   else { o1 = m % p.o1n; int t = m / p.o1n; o0 = t % p.o0n; b = t / p.o0n; }
   out[(long long)b * p.outB + (long long)o0 * p.outS0 + (long long)o1 * p.outS1 + (long long)n * p.outF] = s;
+}
+
+// Filter laid out with the contracted feature contiguous (data gradients): rewritten once per call
+// as [tap][contracted feature][output feature] so that the B tile loads are 16-byte rows along n.
+__global__ void __launch_bounds__(256) conv_repack_filter(const float* __restrict__ src, float* __restrict__ dst, ConvP p, int taps) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
+  const int tap = blockIdx.z;
+  const int t0 = tap / p.k1n, t1 = tap % p.k1n;
+  const float* s = src + (long long)t0 * p.rhsS0 + (long long)t1 * p.rhsS1;
+  float* d = dst + (long long)tap * p.C * p.N;
+  const int c0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
+  (void)taps;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int n = n0 + ty + 8 * r, c = c0 + tx;   // source: c contiguous (rhsI == 1)
+    tile[ty + 8 * r][tx] = (n < p.N && c < p.C) ? s[(long long)c * p.rhsI + (long long)n * p.rhsO] : 0.f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int c = c0 + ty + 8 * r, n = n0 + tx;
+    if (c < p.C && n < p.N) d[(long long)c * p.N + n] = tile[tx][ty + 8 * r];
+  }
 }
 
 struct ConvChoice {
@@ -338,7 +375,7 @@ bool fitsInt(const mi355_conv_desc* d) {
   return lhs < (1ll << 31) && rhs < (1ll << 31) && out < (1ll << 31);
 }
 
-ConvChoice choose(const mi355_conv_desc* d) {
+ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
   ConvChoice c;
   if (d->dtype != 0 || d->nsp > 2 || d->featureGroups != 1 || d->batchGroups != 1 || !fitsInt(d)) return c;
   c.fast = true;
@@ -356,6 +393,7 @@ ConvChoice choose(const mi355_conv_desc* d) {
   c.kflat = !chunk;
   long long taps = 1;
   for (int k = 0; k < d->nsp; ++k) taps *= d->k[k];
+  if (tapsVisited >= 0 && chunk) taps = tapsVisited;
   c.cTiles = chunk ? (int)(d->C / BK) : 1;
   c.kTiles = chunk ? (int)(taps * c.cTiles) : (int)((K + BK - 1) / BK);
   // largest tile that still gives every CU at least two workgroups
@@ -391,24 +429,95 @@ void launchIgemm(const ConvChoice& c, const ConvP& p, dim3 grid, hipStream_t st)
 #undef CASE
 }
 
+// One launch of the implicit-GEMM kernel: the whole convolution, or one residue class of an
+// input-dilated one.  With lhs dilation L (the data gradient of a stride-L convolution) an
+// output position o only meets real input where (o - pad + tap) is a multiple of L, so the
+// outputs with o = c (mod L) all use the same subset of the taps (tap = (pad - c) mod L,
+// step L).  Run per class, no product with an inserted zero is ever formed: a 3x3 filter
+// with L = 2 does 9 tap-products per 4 outputs instead of 36.
+struct ConvPart {
+  mi355_conv_desc d;
+  int kb[2] = {0, 0}, ks[2] = {1, 1}, kc[2] = {1, 1};
+  long long outOffset = 0;
+  long long taps() const { return (long long)kc[0] * kc[1]; }
+};
+
+std::vector<ConvPart> partsOf(const mi355_conv_desc* d) {
+  std::vector<ConvPart> parts;
+  ConvPart whole;
+  whole.d = *d;
+  for (int k = 0; k < 2; ++k) whole.kc[k] = k < d->nsp ? (int)d->k[k] : 1;
+  bool dilated = false, eligible = d->nsp == 2 && d->C % BK == 0 && d->dtype == 0 && d->featureGroups == 1 && d->batchGroups == 1;
+  for (int k = 0; k < d->nsp && k < 2; ++k) {
+    if (d->ldil[k] > 1) dilated = true;
+    if (d->stride[k] != 1 || d->rdil[k] != 1 || d->k[k] < d->ldil[k] || d->out[k] < d->ldil[k]) eligible = false;
+  }
+  static const bool off = getenv("MI355X_CONV_CLASSES") && getenv("MI355X_CONV_CLASSES")[0] == '0';
+  if (!dilated || !eligible || off) { parts.push_back(whole); return parts; }
+  const int L0 = (int)d->ldil[0], L1 = (int)d->ldil[1];
+  for (int c0 = 0; c0 < L0; ++c0) {
+    for (int c1 = 0; c1 < L1; ++c1) {
+      ConvPart p = whole;
+      const int cls[2] = {c0, c1};
+      for (int k = 0; k < 2; ++k) {
+        const int L = (int)d->ldil[k];
+        p.d.out[k] = (d->out[k] - cls[k] + L - 1) / L;          // outputs o = cls + L * j
+        p.d.stride[k] = L;                                      // input coordinate of j: j * L + cls - pad
+        p.d.padLo[k] = d->padLo[k] - cls[k];
+        p.d.outS[k] = d->outS[k] * L;
+        p.outOffset += (long long)cls[k] * d->outS[k];
+        p.kb[k] = (int)((((d->padLo[k] - cls[k]) % L) + L) % L);
+        p.ks[k] = L;
+        p.kc[k] = (int)((d->k[k] - p.kb[k] + L - 1) / L);
+      }
+      parts.push_back(p);
+    }
+  }
+  return parts;
+}
+
+// A filter whose contracted feature is the contiguous one (the layout data gradients see) is
+// worth rewriting when the GEMM has many rows: returns the bytes of the rewritten copy and
+// the descriptor that addresses it, or 0.
+size_t repackedFilter(const mi355_conv_desc* d, mi355_conv_desc* out) {
+  if (d->dtype != 0 || d->nsp > 2 || d->featureGroups != 1 || d->batchGroups != 1 || !fitsInt(d)) return 0;
+  if (d->rhsI != 1 || d->rhsO == 1 || d->C % BK != 0 || d->O % 4 != 0) return 0;
+  long long M = d->N, taps = 1;
+  for (int k = 0; k < d->nsp; ++k) { M *= d->out[k]; taps *= d->k[k]; }
+  if (M < 2048) return 0;
+  *out = *d;
+  out->rhsO = 1;
+  out->rhsI = d->O;
+  if (d->nsp > 1) out->rhsS[1] = d->C * d->O;
+  if (d->nsp > 0) out->rhsS[0] = (d->nsp > 1 ? d->k[1] : 1) * d->C * d->O;
+  size_t bytes = (size_t)taps * (size_t)d->C * (size_t)d->O * sizeof(float);
+  return (bytes + 255) / 256 * 256;
+}
+
 }  // namespace
 
 extern "C" {
 
 size_t mi355_conv_workspace_bytes(const mi355_conv_desc* d) {
-  ConvChoice c = choose(d);
-  if (!c.fast || c.splitK <= 1) return 0;
-  long long M = d->N;
-  for (int k = 0; k < d->nsp; ++k) M *= d->out[k];
-  return (size_t)c.splitK * (size_t)M * (size_t)d->O * sizeof(float);
+  mi355_conv_desc d2;
+  size_t repack = repackedFilter(d, &d2);
+  if (repack) d = &d2;
+  size_t most = 0;
+  for (const ConvPart& part : partsOf(d)) {
+    ConvChoice c = choose(&part.d, part.taps());
+    if (!c.fast || c.splitK <= 1) continue;
+    long long M = part.d.N;
+    for (int k = 0; k < part.d.nsp; ++k) M *= part.d.out[k];
+    most = std::max(most, (size_t)c.splitK * (size_t)M * (size_t)d->O * sizeof(float));
+  }
+  return repack + most;
 }
 
 int mi355_conv_direct(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, mi355_stream_t s);
 
-int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes,
-               mi355_stream_t s) {
-  ConvChoice c = choose(d);
-  if (!c.fast) return mi355_conv_direct(d, lhs, rhs, out, s);
+static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  const mi355_conv_desc* d = &part.d;
+  ConvChoice c = choose(d, part.taps());
   ConvP p;
   p.lhs = (const float*)lhs;
   p.rhs = (const float*)rhs;
@@ -420,6 +529,8 @@ int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void*
   auto dim = [&](const int64_t* a, int k, int64_t dflt) { return k < d->nsp ? (int)a[k] : (int)dflt; };
   p.in0 = dim(d->in, 0, 1); p.in1 = dim(d->in, 1, 1);
   p.k0n = dim(d->k, 0, 1); p.k1n = dim(d->k, 1, 1);
+  p.kb0 = part.kb[0]; p.ks0 = part.ks[0]; p.kc0 = part.kc[0];
+  p.kb1 = part.kb[1]; p.ks1 = part.ks[1]; p.kc1 = part.kc[1];
   p.o0n = dim(d->out, 0, 1); p.o1n = dim(d->out, 1, 1);
   p.s0 = dim(d->stride, 0, 1); p.s1 = dim(d->stride, 1, 1);
   p.p0 = dim(d->padLo, 0, 0); p.p1 = dim(d->padLo, 1, 0);
@@ -431,14 +542,14 @@ int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void*
   p.outB = (int)d->outB; p.outF = (int)d->outF; p.outS0 = dim(d->outS, 0, 0); p.outS1 = dim(d->outS, 1, 0);
   p.bFast = c.bFast;
   p.cTiles = c.cTiles; p.kTiles = c.kTiles; p.splitK = c.splitK; p.tilesPerSplit = c.tilesPerSplit;
+  float* dst = (float*)out + part.outOffset;
   if (c.splitK > 1) {
     size_t need = (size_t)c.splitK * (size_t)M * (size_t)d->O * sizeof(float);
     if (!workspace || workspace_bytes < need) return 3;   // caller sized the workspace wrong
     p.out = (float*)workspace;
   } else {
-    p.out = (float*)out;
+    p.out = dst;
   }
-  hipStream_t st = (hipStream_t)s;
   dim3 grid((unsigned)((p.M + c.bm - 1) / c.bm), (unsigned)((p.N + c.bn - 1) / c.bn), (unsigned)c.splitK);
   if (grid.y > 65535) return 4;
   if (c.bm == 128 && c.bn == 128) launchIgemm<128, 128>(c, p, grid, st);
@@ -446,10 +557,39 @@ int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void*
   else launchIgemm<64, 64>(c, p, grid, st);
   if (c.splitK > 1) {
     long long total = M * d->O;
-    conv_fold_partials<<<(unsigned)((total + 255) / 256), 256, 0, st>>>((const float*)workspace, (float*)out, p);
+    conv_fold_partials<<<(unsigned)((total + 31) / 32), 256, 0, st>>>((const float*)workspace, dst, p);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
+}
+
+int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes,
+               mi355_stream_t s) {
+  hipStream_t st = (hipStream_t)s;
+  mi355_conv_desc d2;
+  size_t repack = repackedFilter(d, &d2);
+  if (repack) {
+    if (!workspace || workspace_bytes < repack) return 3;   // caller sized the workspace wrong
+    ConvP q;
+    q.C = (int)d->C; q.N = (int)d->O;
+    q.k1n = d->nsp > 1 ? (int)d->k[1] : 1;
+    q.rhsI = (int)d->rhsI; q.rhsO = (int)d->rhsO;
+    q.rhsS0 = d->nsp > 0 ? (int)d->rhsS[0] : 0; q.rhsS1 = d->nsp > 1 ? (int)d->rhsS[1] : 0;
+    int taps = 1;
+    for (int k = 0; k < d->nsp; ++k) taps *= (int)d->k[k];
+    dim3 grid((unsigned)((d->C + 31) / 32), (unsigned)((d->O + 31) / 32), (unsigned)taps);
+    conv_repack_filter<<<grid, 256, 0, st>>>((const float*)rhs, (float*)workspace, q, taps);
+    rhs = workspace;
+    workspace = (char*)workspace + repack;
+    workspace_bytes -= repack;
+    d = &d2;
+  }
+  if (!choose(d).fast) return mi355_conv_direct(d, lhs, rhs, out, s);
+  for (const ConvPart& part : partsOf(d)) {
+    // parts run back to back on the stream, so they can share the split-K scratch
+    if (int r = launchPart(part, lhs, rhs, out, workspace, workspace_bytes, st)) return r;
+  }
+  return 0;
 }
 
 }  // extern "C"

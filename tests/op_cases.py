@@ -261,6 +261,12 @@ case("conv-fwd-stride2-vector", _conv(strides=(2, 2), padding=((0, 1), (0, 1))),
 case("conv-fwd-128-tile", _conv(padding=((1, 1), (1, 1))), u(246, 16, 32, 32, 16), u(247, 3, 3, 16, 128))
 case("conv-dgrad-vector", lambda b, g, w: b.conv(g, b.reverse(w, [0, 1]), strides=(1, 1), padding=((1, 2), (1, 2)), lhs_dilation=(2, 2), dn=("b01f", "01oi", "b01f")),
      u(248, 8, 6, 6, 64), u(249, 3, 3, 32, 64))
+# input-dilated convolutions run one launch per residue class of the output positions
+case("conv-dgrad-classes-odd", lambda b, g, w: b.conv(g, b.reverse(w, [0, 1]), strides=(1, 1), padding=((1, 1), (2, 1)), lhs_dilation=(2, 3), dn=("b01f", "01oi", "b01f")),
+     u(1300, 4, 7, 5, 32), u(1301, 3, 3, 16, 32))
+case("conv-dgrad-classes-repacked", lambda b, g, w: b.conv(g, b.reverse(w, [0, 1]), strides=(1, 1), padding=((1, 2), (1, 2)), lhs_dilation=(2, 2), dn=("b01f", "01oi", "b01f")),
+     u(1302, 16, 8, 8, 32), u(1303, 3, 3, 16, 32))
+case("conv-dilated-5x5-classes", _conv(padding=((2, 2), (0, 3)), lhs_dilation=(2, 2)), u(1304, 2, 9, 6, 16), u(1305, 5, 5, 16, 8))
 case("conv-wgrad-vector", lambda b, x, g: b.conv(x, g, strides=(1, 1), padding=((0, 1), (0, 1)), rhs_dilation=(2, 2), dn=("f01b", "i01o", "01bf")),
      u(250, 16, 12, 12, 8), u(251, 16, 6, 6, 32))
 case("conv-wgrad-stride1-vector", lambda b, x, g: b.conv(x, g, strides=(1, 1), padding=((1, 1), (1, 1)), dn=("f01b", "i01o", "01bf")),
