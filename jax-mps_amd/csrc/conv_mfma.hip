@@ -403,8 +403,12 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
   else if (forced == 12864 || (!forced && tilesOf(128, 64) >= 512)) { c.bm = 128; c.bn = 64; }
   else { c.bm = 64; c.bn = 64; }
   long long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+  // Split K until there are about `target` workgroups: several per CU, so that a tile count that is
+  // not a multiple of the CU count costs little, without exceeding it (a few stragglers would
+  // take a whole extra workgroup time).
+  static const int target = getenv("MI355X_CONV_BLOCKS") ? atoi(getenv("MI355X_CONV_BLOCKS")) : 768;
   int split = 1;
-  if (tiles < 512) split = (int)std::min<long long>((1024 + tiles - 1) / tiles, std::max(1, c.kTiles / (tiles < 64 ? 4 : 8)));
+  if (tiles * 2 <= target) split = (int)std::min<long long>(target / tiles, std::max(1, c.kTiles / (tiles < 64 ? 4 : 8)));
   split = std::max(1, std::min(split, 256));
   c.tilesPerSplit = (c.kTiles + split - 1) / split;
   c.splitK = (c.kTiles + c.tilesPerSplit - 1) / c.tilesPerSplit;

@@ -140,7 +140,18 @@ class Planner {
   // ---------------------------------------------------------------- analysis
   static Region* regionOf(Value* v) { return v->def ? v->def->parent : v->argOf; }
 
+  // stablehlo.reverse of a filter over its window dims only: the convolution kernels take a
+  // per-dim "window reversal" flag, so the flipped copy is never made
+  static bool isWindowReverse(Value* v, Op* conv) {
+    if (!v->def || v->def->name != "reverse" || conv->name != "convolution" || conv->operands.size() < 2 || conv->operands[1] != v) return false;
+    if (v->users.size() != 1) return false;
+    for (auto d : v->def->ints("dims"))
+      if (std::find(conv->convDims.rhsSpatial.begin(), conv->convDims.rhsSpatial.end(), d) == conv->convDims.rhsSpatial.end()) return false;
+    return true;
+  }
+
   static bool forcedBy(Value* v, Op* user) {
+    if (isWindowReverse(v, user)) return false;
     if (user->name == "gather") return user->operands[0] == v;       // random access needs memory
     if (isFusibleOp(*user)) return false;
     if (user->name == "reduce") return !isSimpleReduce(*user);
@@ -683,6 +694,11 @@ class Planner {
     Value* lhs = op->operands[0];
     Value* rhs = op->operands[1];
     Value* out = op->result();
+    std::vector<int64_t> flipped;
+    if (!hasStorage(rhs) && isWindowReverse(rhs, op)) {
+      flipped = rhs->def->ints("dims");
+      rhs = rhs->def->operands[0];
+    }
     for (Value* v : {lhs, rhs}) if (!hasStorage(v)) materializeNow(v, plan);
     const ConvDims& cd = op->convDims;
     int nsp = (int)cd.lhsSpatial.size();
@@ -717,6 +733,7 @@ class Planner {
       c.ldil[d] = ld.empty() ? 1 : ld[d];
       c.rdil[d] = rd.empty() ? 1 : rd[d];
       c.rev[d] = rev.empty() ? 0 : rev[d];
+      if (std::find(flipped.begin(), flipped.end(), cd.rhsSpatial[d]) != flipped.end()) c.rev[d] = !c.rev[d];
     }
     int sid = newStorage(out->type.bytes());
     bind(out, sid);
