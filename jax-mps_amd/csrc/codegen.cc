@@ -1056,7 +1056,12 @@ std::string shflXor(const std::string& accT, const std::string& x, const std::st
 
 }  // namespace
 
-FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeaf) {
+FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeafOuter, const std::vector<Value*>& epilogue) {
+  // values computed from the results right where they are finished (second pass only)
+  std::unordered_set<Value*> own;
+  for (auto* r : reduces) own.insert(r->result());
+  for (auto* v : epilogue) own.insert(v);
+  LeafPredicate isLeaf = [&](Value* v) { return !own.count(v) && isLeafOuter(v); };
   Op* r0 = reduces[0];
   Value* x0 = r0->operands[0];
   const std::vector<int64_t>& shape = x0->type.dims;
@@ -1099,12 +1104,11 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     Emitter em(isLeaf, 1, i64);
     std::vector<std::string> inits;
     for (auto* r : reduces) inits.push_back(em.gen(r->operands[1], em.multiIndex({}, {})));
-    std::ostringstream s;
-    s << kPrelude;
+    std::ostringstream s;   // body; the header follows once the epilogue has named its inputs
     std::vector<std::string> outs;
     for (size_t j = 0; j < nr; ++j) outs.push_back("const " + ops[j].accT + "* __restrict__ part" + std::to_string(j));
     for (size_t j = 0; j < nr; ++j) outs.push_back(storageT(ops[j].dt) + "* __restrict__ out" + std::to_string(j));
-    s << kernelHeader(em.leaves_, outs) << " {\n";
+    for (size_t q = 0; q < epilogue.size(); ++q) outs.push_back(storageT(epilogue[q]->type.dt) + "* __restrict__ outE" + std::to_string(q));
     // many partials per output: one wavefront folds an output (lanes stride over the
     // partials, then a butterfly); few partials: one lane per output
     // a whole workgroup per output when there are hundreds of partials (every lane issues its few
@@ -1120,37 +1124,59 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     } else {
       s << "  const " << IT << " kk = (" << IT << ")blockIdx.x * 256 + threadIdx.x;\n  if (kk >= " << Kn << ") return;\n";
     }
-    s << em.pre_;
+    const std::string initPre = em.pre_;
+    s << initPre;
     for (size_t j = 0; j < nr; ++j) {
       std::string part = "part" + std::to_string(j) + "[p * " + std::to_string(Kn) + " + kk]";
       std::string ST = ops[j].accT == "bool" ? "int" : ops[j].accT;
-      s << "  { " << ops[j].accT << " a = " << ops[j].identity << ";\n";
+      std::string a = "a" + std::to_string(j);
+      s << "  " << ops[j].accT << " " << a << " = " << ops[j].identity << ";\n";
       if (blockPerOut) {
-        s << "    #pragma unroll 8\n    for (" << IT << " p = threadIdx.x; p < " << P << "; p += 256) a = " << ops[j].combine("a", part) << ";\n";
-        s << "    #pragma unroll\n    for (int o = 32; o > 0; o >>= 1) a = " << ops[j].combine("a", shflXor(ops[j].accT, "a", "o")) << ";\n";
-        s << "    __shared__ " << ST << " fm" << j << "[4];\n";
-        s << "    if (lane == 0) fm" << j << "[threadIdx.x >> 6] = a;\n    __syncthreads();\n";
-        s << "    if (threadIdx.x == 0) {\n";
-        s << "    a = (" << ops[j].accT << ")fm" << j << "[0];\n";
-        s << "    for (int w = 1; w < 4; ++w) a = " << ops[j].combine("a", "(" + ops[j].accT + ")fm" + std::to_string(j) + "[w]") << ";\n";
+        s << "  #pragma unroll 8\n  for (" << IT << " p = threadIdx.x; p < " << P << "; p += 256) " << a << " = " << ops[j].combine(a, part) << ";\n";
+        s << "  #pragma unroll\n  for (int o = 32; o > 0; o >>= 1) " << a << " = " << ops[j].combine(a, shflXor(ops[j].accT, a, "o")) << ";\n";
+        s << "  __shared__ " << ST << " fm" << j << "[4];\n";
+        s << "  if (lane == 0) fm" << j << "[threadIdx.x >> 6] = " << a << ";\n";
       } else if (wavePerOut) {
-        s << "    #pragma unroll 4\n    for (" << IT << " p = lane; p < " << P << "; p += 64) a = " << ops[j].combine("a", part) << ";\n";
-        s << "    #pragma unroll\n    for (int o = 32; o > 0; o >>= 1) a = " << ops[j].combine("a", shflXor(ops[j].accT, "a", "o")) << ";\n";
-        s << "    if (lane == 0) {\n";
+        s << "  #pragma unroll 4\n  for (" << IT << " p = lane; p < " << P << "; p += 64) " << a << " = " << ops[j].combine(a, part) << ";\n";
+        s << "  #pragma unroll\n  for (int o = 32; o > 0; o >>= 1) " << a << " = " << ops[j].combine(a, shflXor(ops[j].accT, a, "o")) << ";\n";
       } else {
-        s << "    for (" << IT << " p = 0; p < " << P << "; ++p) a = " << ops[j].combine("a", part) << ";\n    {\n";
+        s << "  for (" << IT << " p = 0; p < " << P << "; ++p) " << a << " = " << ops[j].combine(a, part) << ";\n";
       }
-      s << "    a = " << ops[j].combine(inits[j], "a") << ";\n";
-      s << "    out" << j << "[kk] = " << storeExpr(ops[j].dt, roundTo(ops[j].dt, "a")) << "; } }\n";
+    }
+    if (blockPerOut) s << "  __syncthreads();\n  if (threadIdx.x != 0) return;\n";
+    else if (wavePerOut) s << "  if (lane != 0) return;\n";
+    for (size_t j = 0; j < nr; ++j) {
+      std::string a = "a" + std::to_string(j);
+      if (blockPerOut) {
+        s << "  " << a << " = (" << ops[j].accT << ")fm" << j << "[0];\n";
+        s << "  for (int w = 1; w < 4; ++w) " << a << " = " << ops[j].combine(a, "(" + ops[j].accT + ")fm" + std::to_string(j) + "[w]") << ";\n";
+      }
+      s << "  const " << ops[j].accT << " res" << j << " = " << roundTo(ops[j].dt, ops[j].combine(inits[j], a)) << ";\n";
+      s << "  out" << j << "[kk] = " << storeExpr(ops[j].dt, "res" + std::to_string(j)) << ";\n";
+    }
+    if (!epilogue.empty()) {
+      // per-output values that only need the finished results: computed by the lane that holds them
+      for (size_t j = 0; j < nr; ++j) em.rowScalars_[reduces[j]->result()] = "res" + std::to_string(j);
+      IdxDim klin;
+      klin.isConst = false; klin.base = "kk"; klin.coef = 0; klin.mult = 1;
+      em.pre_.clear();
+      auto kd = em.delinearize(klin, keptShape);
+      em.rowKept_ = kd;
+      Index kidx = em.multiIndex(kd, keptShape);
+      std::vector<std::string> ev;
+      for (auto* v : epilogue) ev.push_back(em.gen(v, kidx));
+      s << em.pre_;
+      for (size_t q = 0; q < epilogue.size(); ++q) s << "  outE" << q << "[kk] = " << storeExpr(epilogue[q]->type.dt, ev[q]) << ";\n";
     }
     s << "}\n";
     Launch l;
-    l.source = s.str();
+    l.source = std::string(kPrelude) + kernelHeader(em.leaves_, outs) + " {\n" + s.str();
     l.grid[0] = (unsigned)(blockPerOut ? Kn : wavePerOut ? (Kn + 3) / 4 : (Kn + 255) / 256);
     l.block[0] = 256;
     for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
     for (size_t j = 0; j < nr; ++j) { KArg a; a.kind = KArg::Work; a.workOffset = workOff[j]; l.args.push_back(a); }
     for (size_t j = 0; j < nr; ++j) { KArg a; a.kind = KArg::Out; a.value = reduces[j]->result(); l.args.push_back(a); }
+    for (auto* v : epilogue) { KArg a; a.kind = KArg::Out; a.value = v; l.args.push_back(a); }
     initLeaves = em.leaves_;
     (void)workStride;
     return l;
@@ -1272,6 +1298,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     if (partial) {
       std::vector<Value*> il;
       fc.launches.push_back(finalPass(P, Kn, workOff, il));
+      fc.epilogueFused = !epilogue.empty();
       for (auto* v : il) if (std::find(fc.leaves.begin(), fc.leaves.end(), v) == fc.leaves.end()) fc.leaves.push_back(v);
       fc.workspaceBytes = wb;
     }
@@ -1386,6 +1413,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   if (partial) {
     std::vector<Value*> il;
     fc.launches.push_back(finalPass(P, Kn, workOff, il));
+      fc.epilogueFused = !epilogue.empty();
     for (auto* v : il) if (std::find(fc.leaves.begin(), fc.leaves.end(), v) == fc.leaves.end()) fc.leaves.push_back(v);
     fc.workspaceBytes = wb;
   }

@@ -32,6 +32,7 @@ struct Launch {
 struct FusedCode {
   std::vector<Launch> launches;
   int64_t workspaceBytes = 0;
+  bool epilogueFused = false;
   std::vector<Value*> leaves;   // distinct materialised inputs
 };
 
@@ -56,7 +57,9 @@ FusedCode generateDusKernel(Op* dus, const LeafPredicate& isLeaf);
 
 // One or more stablehlo.reduce ops with identical input shape and dimensions.
 // Returns false in `ok` when a reducer body is not a single add/mul/max/min/and/or.
-FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeaf);
+// `epilogue`: values of the result shape computed from the results (and other inputs of that shape); they are
+// produced by the pass that folds partial sums when there is one (FusedCode::epilogueFused), otherwise ignored.
+FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeaf, const std::vector<Value*>& epilogue = {});
 
 // True if codegen can inline `op` into a consumer (elementwise / indexing ops).
 bool isFusibleOp(const Op& op);

@@ -589,14 +589,55 @@ class Planner {
       // reducing nothing: the result is the init value broadcast
       throw CompileError("stablehlo.reduce over an empty tensor is not supported");
     }
-    FusedCode fc = generateReduceKernel(group, leafPred());
+    // Per-output values that need nothing but the results and inputs of the result shape (a mean, a
+    // variance, a reciprocal square root ...) ride along in the pass that folds the partial sums.
+    std::vector<Value*> epilogue;
+    std::vector<Op*> epilogueOps;
+    {
+      std::unordered_set<Value*> results;
+      for (auto* g : group) results.insert(g->result());
+      const auto& keptDims = op->result()->type.dims;
+      std::function<bool(Value*, bool&, int&)> can = [&](Value* v, bool& usesResult, int& budget) -> bool {
+        if (results.count(v) || std::find(epilogue.begin(), epilogue.end(), v) != epilogue.end()) { usesResult = true; return true; }
+        if (hasStorage(v)) return v->type.numel() <= op->result()->type.numel();   // nothing bigger than the result shape
+        Op* d = v->def;
+        if (!d || !isFusibleOp(*d) || d->results.size() != 1 || d->parent != &r || needMat_[v] || --budget < 0) return false;
+        for (auto* o : d->operands) if (!can(o, usesResult, budget)) return false;
+        return true;
+      };
+      size_t pos = 0;
+      while (pos < r.ops.size() && r.ops[pos].get() != op) ++pos;
+      for (size_t q = pos + 1; q < r.ops.size() && q <= pos + 64 && epilogue.size() < 6; ++q) {
+        Op* y = r.ops[q].get();
+        if (emitted_.count(y) || !isFusibleOp(*y) || y->results.size() != 1) continue;
+        Value* w = y->result();
+        if (!needMat_[w] || hasStorage(w) || !takesKernel(y) || w->type.dims != keptDims) continue;
+        bool uses = false;
+        int budget = 64;
+        bool ok = true;
+        for (auto* o : y->operands) if (!can(o, uses, budget)) ok = false;
+        if (!ok || !uses) continue;
+        epilogue.push_back(w);
+        epilogueOps.push_back(y);
+      }
+    }
+    FusedCode fc = generateReduceKernel(group, leafPred(), epilogue);
     std::vector<Value*> outs;
     for (auto* g : group) {
       bind(g->result(), newStorage(g->result()->type.bytes()));
       outs.push_back(g->result());
       emitted_.insert(g);
     }
-    addFused(plan, fc, (group.size() > 1 ? "reduce x" + std::to_string(group.size()) : std::string("reduce")) + " " + group[0]->operands[0]->type.str() + " -> " + outs[0]->type.str(), outs);
+    std::string label = (group.size() > 1 ? "reduce x" + std::to_string(group.size()) : std::string("reduce"));
+    if (fc.epilogueFused) {
+      for (size_t k = 0; k < epilogue.size(); ++k) {
+        bind(epilogue[k], newStorage(epilogue[k]->type.bytes()));
+        outs.push_back(epilogue[k]);
+        emitted_.insert(epilogueOps[k]);
+        label += "+" + epilogueOps[k]->name;
+      }
+    }
+    addFused(plan, fc, label + " " + group[0]->operands[0]->type.str() + " -> " + outs[0]->type.str(), outs);
   }
 
   static std::vector<int64_t> stridesOf(const TensorType& t) {
