@@ -111,6 +111,11 @@ def cpu_baseline(budget_s=12.0, batch=128):
             "sample": f"{n} ResNet18 train step(s) at batch {batch} in {dt:.1f} s (numpy/BLAS float32 interpreter of the same module)"}
 
 
+# HBM bytes per conv_igemm_f32 launch of this workload: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by
+# what the same counter reads for a 256 MiB copy (profiles/conv_igemm_f32_resnet18_b128_hbm_traffic.md).
+CONV_HBM_BYTES_PER_LAUNCH = 101.5e6
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -118,11 +123,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fused", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a 256 MiB device copy (kernel copy_vec16) a few times: the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives exactly one GPU (one PJRT device); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
-    os.environ.setdefault("MI355X_TIMING", "conv")     # HIP-event timing of the convolution launches only
+    os.environ.setdefault("MI355X_TIMING", "conv")     # HIP-event timing of the convolution launches only,
+    every = int(os.environ.setdefault("MI355X_TIMING_EVERY", "5"))   # on one step in five: the events cost ~5 us per launch
     from jax_mps_amd import pjrt, runner
     from jax_mps_amd.programs import configs
     client = pjrt.get_client()
@@ -143,7 +151,8 @@ def main():
     conv_ms = after.get("conv.time_ms", 0.0) - before.get("conv.time_ms", 0.0)
     conv_n = after.get("conv.count", 0.0) - before.get("conv.count", 0.0)
     conv_flops = p.meta["step_flops"] - 6 * 128 * 512 * 10      # dense head is a GEMM step, not a convolution
-    achieved = conv_flops * args.steps / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else None
+    timed_steps = sum(1 for i in range(args.warmup, args.warmup + args.steps) if i % every == 0)   # execute calls the plugin sampled
+    achieved = conv_flops * timed_steps / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else None
     line = {
         "metric": "jitted train steps/sec (ResNet18 b128, 1 MI355X); fused-op HBM GB/s vs peak",
         "value": round(args.steps / dt, 3), "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -153,11 +162,23 @@ def main():
                    "final_loss": round(loss, 5)},
         "roofline": {"bound": "mfma", "kernel": "convolution (all launches of one step)", "achieved": None if achieved is None else round(achieved, 3),
                      "peak": PEAK_F32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": None if achieved is None else round(achieved / PEAK_F32_MFMA_TFLOPS, 4),
-                     "traffic": None, "launches_per_step": conv_n / max(args.steps, 1), "avg_launch_us": round(conv_ms * 1e3 / conv_n, 2) if conv_n else None,
+                     "traffic": CONV_HBM_BYTES_PER_LAUNCH, "launches_per_step": conv_n / max(timed_steps, 1), "timed_steps": timed_steps, "avg_launch_us": round(conv_ms * 1e3 / conv_n, 2) if conv_n else None,
                      "algorithmic_flops_per_step": conv_flops},
     }
+    if args.copy_calibration:
+        from jax_mps_amd.shlo.builder import Builder
+        b = Builder("copy_calibration")
+        x = b.arg((64 * 1024 * 1024,), "f32")
+        b.ret(x)                                   # an argument returned as a result is one copy_vec16 launch of 256 MiB
+        exe = client.compile_and_load(b.text())
+        buf = client.buffer_from_pyval(np.zeros(64 * 1024 * 1024, np.float32))
+        for _ in range(5):
+            o = exe.execute([buf])
+        o[0].block_until_ready()
+        line["copy_calibration"] = {"kernel": "copy_vec16", "bytes_read": 256 * 1024 * 1024, "bytes_written": 256 * 1024 * 1024, "launches": 5}
     if not args.no_fused:
         os.environ["MI355X_TIMING"] = "all"
+        os.environ["MI355X_TIMING_EVERY"] = "1"
         line["fused_ops"] = bench_fused_ops(client)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()

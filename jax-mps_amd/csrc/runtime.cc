@@ -221,6 +221,8 @@ Executable::Executable(std::unique_ptr<CompiledProgram> prog) : prog_(std::move(
   Device& dev = Device::get();
   const char* t = getenv("MI355X_TIMING");
   timingKinds_ = t ? t : "";
+  const char* every = getenv("MI355X_TIMING_EVERY");   // time one execute call in N (sampling keeps the events' own cost small)
+  timingEvery_ = every ? std::max(1, atoi(every)) : 1;
   const char* gr = getenv("MI355X_GRAPHS");   // "0" runs loop bodies launch by launch
   useGraphs_ = !(gr && gr[0] == '0');
   loadKernels();
@@ -341,7 +343,7 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
     case Step::Copy: kind = "copy"; bytes = 2.0 * s.bytes; break;
     default: break;
   }
-  bool doTime = !kind.empty() && timed(kind);
+  bool doTime = !kind.empty() && timedCall_ && timed(kind);
   static const bool detail = getenv("MI355X_TIMING_DETAIL") != nullptr;   // one statistics row per step label
   if (doTime && detail) kind += ":" + s.label;
   mi355_event_t ea = nullptr, eb = nullptr;
@@ -554,6 +556,7 @@ std::vector<std::shared_ptr<DeviceBuffer>> Executable::execute(const std::vector
     outPtrs.push_back(b->ptr);
     outs.push_back(std::move(b));
   }
+  timedCall_ = (executeCount_++ % timingEvery_) == 0;
   runPlan(prog_->plan, inputs, outPtrs);
   return outs;
 }

@@ -99,6 +99,9 @@ class Executable {
   std::vector<mi355_event_t> eventPool_;
   std::map<std::string, KindStat> stats_;
   std::string timingKinds_;
+  int timingEvery_ = 1;
+  uint64_t executeCount_ = 0;
+  bool timedCall_ = true;
 
   // Captured bodies of counted loops.  A graph bakes in the addresses of the call's argument and
   // result buffers, so it is kept with a signature of those and rebuilt when they change.
