@@ -365,33 +365,132 @@ struct ScatterOps<u32> {
   }
 };
 
-// grid.x = update position (only segment heads work), grid.y = column chunk of 256*VEC elements
+// Segment fold.  After the stable sort, the updates of one destination row are a run of equal
+// keys whose values (update numbers) ascend; applying them in that order to the row is exactly
+// what a sequential scatter does, bit for bit, and rows are independent of each other.
+//
+// Storage / accumulator policies (bf16 rounds after every application, like a bf16 loop would).
 template <typename T>
-__global__ void __launch_bounds__(256) scatter_fold(const u32* __restrict__ keys, const u32* __restrict__ vals, long long n, long long rowElems,
-                                                    int kind, T* __restrict__ result, const T* __restrict__ updates, u32 rows) {
-  long long i = blockIdx.x;
-  u32 key = keys[i];
+struct Plain {
+  typedef T S;
+  typedef T A;
+  static __device__ __forceinline__ A load(S s) { return s; }
+  static __device__ __forceinline__ S store(A a) { return a; }
+  static __device__ __forceinline__ A apply(int kind, A a, S u) { return ScatterOps<T>::apply(kind, a, u); }
+};
+struct Bf16 {
+  typedef u16 S;
+  typedef float A;
+  static __device__ __forceinline__ A load(S s) { return bf2f(s); }
+  static __device__ __forceinline__ S store(A a) { return f2bf(a); }
+  static __device__ __forceinline__ A apply(int kind, A a, S u) { return bf2f(f2bf(ScatterOps<float>::apply(kind, a, bf2f(u)))); }
+};
+
+constexpr int kLongSegment = 16;   // runs at least this long go to the column-parallel kernel
+
+// Short runs (the common case): one workgroup per run head and chunk of 256 columns; every
+// lane fetches all (< 16) updates of its column at once, then applies them in order.
+template <typename P>
+__global__ void __launch_bounds__(256) scatter_fold_short(const u32* __restrict__ keys, const u32* __restrict__ vals, long long n, long long rowElems,
+                                                          int kind, typename P::S* __restrict__ result, const typename P::S* __restrict__ updates, u32 rows) {
+  const long long i = blockIdx.x;
+  const u32 key = keys[i];
   if (key >= rows) return;
   if (i > 0 && keys[i - 1] == key) return;
-  long long col = (long long)blockIdx.y * 256 + threadIdx.x;
+  if (i + kLongSegment - 1 < n && keys[i + kLongSegment - 1] == key) return;   // long run: other kernel
+  const long long col = (long long)blockIdx.y * 256 + threadIdx.x;
   if (col >= rowElems) return;
-  T acc = result[(long long)key * rowElems + col];
-  for (long long j = i; j < n && keys[j] == key; ++j) acc = ScatterOps<T>::apply(kind, acc, updates[(long long)vals[j] * rowElems + col]);
-  result[(long long)key * rowElems + col] = acc;
+  int cnt = 1;
+  while (cnt < kLongSegment && i + cnt < n && keys[i + cnt] == key) ++cnt;
+  typename P::S u[kLongSegment];
+#pragma unroll
+  for (int q = 0; q < kLongSegment - 1; ++q)
+    if (q < cnt) u[q] = updates[(long long)vals[i + q] * rowElems + col];
+  typename P::A acc = P::load(result[(long long)key * rowElems + col]);
+#pragma unroll
+  for (int q = 0; q < kLongSegment - 1; ++q)
+    if (q < cnt) acc = P::apply(kind, acc, u[q]);
+  result[(long long)key * rowElems + col] = P::store(acc);
 }
 
-__global__ void __launch_bounds__(256) scatter_fold_bf16(const u32* __restrict__ keys, const u32* __restrict__ vals, long long n, long long rowElems,
-                                                         int kind, u16* __restrict__ result, const u16* __restrict__ updates, u32 rows) {
-  long long i = blockIdx.x;
-  u32 key = keys[i];
+template <typename P, int KIND>
+__device__ __forceinline__ void foldStaged(typename P::A& acc, const typename P::S* column, int m) {
+  int r = 0;
+  for (; r + 16 <= m; r += 16) {
+    typename P::S v[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) v[q] = column[(r + q) * 64];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc = P::apply(KIND, acc, v[q]);
+  }
+  for (; r < m; ++r) acc = P::apply(KIND, acc, column[r * 64]);
+}
+
+// Long runs (hot rows of a skewed index distribution): the row is cut into chunks of 64 columns,
+// one workgroup each, so that one hot row keeps many CUs and many loads busy.  Four wavefronts
+// fetch 128 updates x 64 columns per round into LDS (32 independent loads per lane); the first
+// wavefront then applies the 128 staged values of its column in order.  A run of length >= 16
+// contains a multiple of 16, so only those positions get a workgroup, and the first of them
+// inside the run does the work (the run's head is found by bisection in the sorted keys).
+template <typename P>
+__global__ void __launch_bounds__(256) scatter_fold_long(const u32* __restrict__ keys, const u32* __restrict__ vals, long long n, long long rowElems,
+                                                          int kind, typename P::S* __restrict__ result, const typename P::S* __restrict__ updates, u32 rows) {
+  typedef typename P::S S;
+  constexpr int kWaves = 4, kPerLane = 32, kRound = kWaves * kPerLane;   // 128 updates x 64 columns staged per round
+  __shared__ u32 sval[256];
+  __shared__ S stage[kRound][64];
+  const long long p = (long long)blockIdx.x * kLongSegment;
+  if (p >= n) return;
+  const u32 key = keys[p];
   if (key >= rows) return;
-  if (i > 0 && keys[i - 1] == key) return;
-  long long col = (long long)blockIdx.y * 256 + threadIdx.x;
-  if (col >= rowElems) return;
-  float acc = bf2f(result[(long long)key * rowElems + col]);
-  for (long long j = i; j < n && keys[j] == key; ++j)
-    acc = bf2f(f2bf(ScatterOps<float>::apply(kind, acc, bf2f(updates[(long long)vals[j] * rowElems + col]))));
-  result[(long long)key * rowElems + col] = f2bf(acc);
+  long long lo = 0, hi = p;           // first position holding `key`
+  while (lo < hi) {
+    long long mid = (lo + hi) >> 1;
+    if (keys[mid] < key) lo = mid + 1; else hi = mid;
+  }
+  const long long head = lo;
+  if (p - head >= kLongSegment) return;                                             // an earlier workgroup owns this run
+  if (head + kLongSegment - 1 >= n || keys[head + kLongSegment - 1] != key) return;   // short run
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const long long col = (long long)blockIdx.y * 64 + lane;
+  const bool active = col < rowElems;
+  typename P::A acc = typename P::A();
+  if (w == 0 && active) acc = P::load(result[(long long)key * rowElems + col]);
+  for (long long base = head;; base += 256) {
+    const long long j = base + threadIdx.x;
+    const bool mine = j < n && keys[j] == key;
+    __syncthreads();
+    sval[threadIdx.x] = mine ? vals[j] : 0u;
+    const int cnt = __syncthreads_count(mine);   // sorted: the matches are a prefix of the tile
+    for (int t0 = 0; t0 < cnt; t0 += kRound) {
+      const int m = cnt - t0 < kRound ? cnt - t0 : kRound;
+      S u[kPerLane];
+#pragma unroll
+      for (int q = 0; q < kPerLane; ++q) {
+        const int r = w + kWaves * q;
+        if (r < m && active) u[q] = updates[(long long)sval[t0 + r] * rowElems + col];
+      }
+#pragma unroll
+      for (int q = 0; q < kPerLane; ++q) {
+        const int r = w + kWaves * q;
+        if (r < m && active) stage[r][lane] = u[q];
+      }
+      __syncthreads();
+      if (w == 0 && active) {
+        // the combiner is fixed outside the loop so that the LDS reads of a column pipeline
+        switch (kind) {
+          case 0: foldStaged<P, 0>(acc, &stage[0][lane], m); break;
+          case 1: foldStaged<P, 1>(acc, &stage[0][lane], m); break;
+          case 2: foldStaged<P, 2>(acc, &stage[0][lane], m); break;
+          case 3: foldStaged<P, 3>(acc, &stage[0][lane], m); break;
+          default: foldStaged<P, 4>(acc, &stage[0][lane], m); break;
+        }
+      }
+      __syncthreads();
+    }
+    if (cnt < 256) break;
+  }
+  if (w == 0 && active) result[(long long)key * rowElems + col] = P::store(acc);
 }
 
 namespace {
@@ -523,19 +622,28 @@ int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* in
   int bits = 1;
   while (bits < 32 && (1ll << bits) <= d->operandRows) ++bits;
   u32 *kin = keys0, *kout = keys1, *vin = vals0, *vout = vals1;
+  // few keys: few sorting workgroups, so that the single-workgroup scan over their histograms stays short
+  int sortBlocks = (int)((n + 2047) / 2048);
+  sortBlocks = sortBlocks < 1 ? 1 : (sortBlocks > kSortBlocks ? kSortBlocks : sortBlocks);
   for (int shift = 0; shift < bits; shift += 8) {
-    radix_hist<<<kSortBlocks, 256, 0, st>>>(kin, n, shift, counts);
-    radix_scan<<<1, 256, 0, st>>>(counts, kSortBlocks);
-    radix_scatter<<<kSortBlocks, 256, 0, st>>>(kin, vin, n, shift, counts, kout, vout);
+    radix_hist<<<sortBlocks, 256, 0, st>>>(kin, n, shift, counts);
+    radix_scan<<<1, 256, 0, st>>>(counts, sortBlocks);
+    radix_scatter<<<sortBlocks, 256, 0, st>>>(kin, vin, n, shift, counts, kout, vout);
     u32* t = kin; kin = kout; kout = t;
     t = vin; vin = vout; vout = t;
   }
-  dim3 grid((unsigned)n, (unsigned)((d->rowElems + 255) / 256));
-  if (d->dtype == 0) scatter_fold<float><<<grid, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (float*)result, (const float*)updates, (u32)d->operandRows);
-  else if (d->dtype == 2) scatter_fold<int><<<grid, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (int*)result, (const int*)updates, (u32)d->operandRows);
-  else if (d->dtype == 3) scatter_fold<u32><<<grid, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (u32*)result, (const u32*)updates, (u32)d->operandRows);
-  else if (d->dtype == 1) scatter_fold_bf16<<<grid, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (u16*)result, (const u16*)updates, (u32)d->operandRows);
+  dim3 gridShort((unsigned)n, (unsigned)((d->rowElems + 255) / 256));
+  dim3 gridLong((unsigned)((n + kLongSegment - 1) / kLongSegment), (unsigned)((d->rowElems + 63) / 64));
+#define FOLD(P) do { \
+    scatter_fold_short<P><<<gridShort, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (typename P::S*)result, (const typename P::S*)updates, (u32)d->operandRows); \
+    if (n >= kLongSegment) scatter_fold_long<P><<<gridLong, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (typename P::S*)result, (const typename P::S*)updates, (u32)d->operandRows); \
+  } while (0)
+  if (d->dtype == 0) FOLD(Plain<float>);
+  else if (d->dtype == 2) FOLD(Plain<int>);
+  else if (d->dtype == 3) FOLD(Plain<u32>);
+  else if (d->dtype == 1) FOLD(Bf16);
   else return 2;
+#undef FOLD
   return check("scatter_rows");
 }
 

@@ -193,6 +193,17 @@ case("scatter-large-int32", _row_scatter("set"), np.zeros((5, 1), np.int32), np.
 case("scatter-large-uint32", _row_scatter("set"), np.zeros((5, 1), np.uint32), np.array([2], np.int32), np.array([[16777217]], np.uint32), exact=True)
 case("scatter-add-many", _row_scatter("add"), f32(160, 300, 70), rng(161).integers(0, 300, size=1000).astype(np.int32), f32(162, 1000, 70), exact=True)
 
+# hot rows: runs of equal indices longer than the LDS index tile (256) and the staging round (128), next to short runs
+def _hot(seed, n, rows):
+    r = rng(seed)
+    idx = np.where(r.random(n) < 0.7, r.integers(0, 3, size=n) * 7, r.integers(0, rows, size=n))
+    return idx.astype(np.int32)
+case("scatter-add-hot-rows", _row_scatter("add"), f32(163, 40, 100), _hot(164, 1500, 40), f32(165, 1500, 100), exact=True)
+case("scatter-add-hot-rows-int", _row_scatter("add"), rng(166).integers(-5, 5, size=(30, 70)).astype(np.int32), _hot(167, 900, 30),
+     rng(168).integers(-1000, 1000, size=(900, 70)).astype(np.int32), exact=True)
+case("scatter-max-hot-rows", _row_scatter("max"), f32(169, 25, 64), _hot(1690, 600, 25), f32(1691, 600, 64), exact=True)
+case("scatter-add-hot-rows-exactly-16", _row_scatter("add"), f32(1692, 8, 33), np.array([5] * 16 + [2] * 15 + [7] * 17, np.int32), f32(1693, 48, 33), exact=True)
+
 # ------------------------------------------------------------------ dot_general (tests/configs/matmul.py:19-249)
 case("dot-matmul", lambda b, x, y: b.matmul(x, y), f32(170, 33, 70), f32(171, 70, 45))
 case("dot-vector-matrix", lambda b, x, y: b.dot_general(x, y, ([0], [0])), f32(172, 70), f32(173, 70, 45))
