@@ -339,6 +339,25 @@ __global__ void __launch_bounds__(256) conv_fold_partials(const float* __restric
   out[(long long)b * p.outB + (long long)o0 * p.outS0 + (long long)o1 * p.outS1 + (long long)n * p.outF] = s;
 }
 
+// Few splits: one lane per four consecutive outputs (16-byte reads of every partial), splits added in order.
+__global__ void __launch_bounds__(256) conv_fold_few(const float* __restrict__ part, float* __restrict__ out, ConvP p) {
+  const long long total = (long long)p.M * p.N;   // p.N % 4 == 0 (checked by the launcher)
+  const long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= total) return;
+  float4 s = *(const float4*)(part + i);
+  for (int z = 1; z < p.splitK; ++z) {
+    float4 v = *(const float4*)(part + (long long)z * total + i);
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  const int m = (int)(i / p.N), n = (int)(i - (long long)m * p.N);
+  int b, o0, o1;
+  if (p.bFast) { b = m % p.Nb; int t = m / p.Nb; o1 = t % p.o1n; o0 = t / p.o1n; }
+  else { o1 = m % p.o1n; int t = m / p.o1n; o0 = t % p.o0n; b = t / p.o0n; }
+  float* o = out + (long long)b * p.outB + (long long)o0 * p.outS0 + (long long)o1 * p.outS1 + (long long)n * p.outF;
+  if (p.outF == 1 && (((uintptr_t)o) & 15) == 0) *(float4*)o = s;
+  else { o[0] = s.x; o[p.outF] = s.y; o[2 * (long long)p.outF] = s.z; o[3 * (long long)p.outF] = s.w; }
+}
+
 // Filter laid out with the contracted feature contiguous (data gradients): rewritten once per call
 // as [tap][contracted feature][output feature] so that the B tile loads are 16-byte rows along n.
 __global__ void __launch_bounds__(256) conv_repack_filter(const float* __restrict__ src, float* __restrict__ dst, ConvP p, int taps) {
@@ -561,7 +580,10 @@ static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, vo
   else launchIgemm<64, 64>(c, p, grid, st);
   if (c.splitK > 1) {
     long long total = M * d->O;
-    conv_fold_partials<<<(unsigned)((total + 31) / 32), 256, 0, st>>>((const float*)workspace, dst, p);
+    if (c.splitK <= 8 && p.N % 4 == 0 && ((uintptr_t)workspace & 15) == 0)
+      conv_fold_few<<<(unsigned)((total / 4 + 255) / 256), 256, 0, st>>>((const float*)workspace, dst, p);
+    else
+      conv_fold_partials<<<(unsigned)((total + 31) / 32), 256, 0, st>>>((const float*)workspace, dst, p);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
