@@ -415,11 +415,12 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
   if (tapsVisited >= 0 && chunk) taps = tapsVisited;
   c.cTiles = chunk ? (int)(d->C / BK) : 1;
   c.kTiles = chunk ? (int)(taps * c.cTiles) : (int)((K + BK - 1) / BK);
-  // largest tile that still gives every CU at least two workgroups
+  // largest tile that still leaves minTiles output tiles (split-K then multiplies the workgroups); tuned on the ResNet18 step
   auto tilesOf = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   static const int forced = getenv("MI355X_CONV_TILE") ? atoi(getenv("MI355X_CONV_TILE")) : 0;
-  if (forced == 128 || (!forced && N >= 128 && tilesOf(128, 128) >= 512)) { c.bm = 128; c.bn = 128; }
-  else if (forced == 12864 || (!forced && tilesOf(128, 64) >= 512)) { c.bm = 128; c.bn = 64; }
+  static const int minTiles = getenv("MI355X_CONV_MIN_TILES") ? atoi(getenv("MI355X_CONV_MIN_TILES")) : 128;
+  if (forced == 128 || (!forced && N >= 128 && tilesOf(128, 128) >= minTiles)) { c.bm = 128; c.bn = 128; }
+  else if (forced == 12864 || (!forced && tilesOf(128, 64) >= minTiles)) { c.bm = 128; c.bn = 64; }
   else { c.bm = 64; c.bn = 64; }
   long long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
   // Split K until there are about `target` workgroups: several per CU, so that a tile count that is
