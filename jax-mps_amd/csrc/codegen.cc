@@ -213,6 +213,7 @@ class Emitter {
   std::unordered_map<Value*, std::string> rowScalars_;
   std::vector<IdxDim> rowKept_;           // index of the current row over the kept dims
   void shareLeavesFrom(const Emitter& o) { leaves_ = o.leaves_; leafIndex_ = o.leafIndex_; }
+  void startTemporariesAt(int n) { tmp_ = n; }   // keeps the names of nested emitters apart
 
   int leafId(Value* v) {
     auto it = leafIndex_.find(v);
@@ -1417,6 +1418,127 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     for (auto* v : il) if (std::find(fc.leaves.begin(), fc.leaves.end(), v) == fc.leaves.end()) fc.leaves.push_back(v);
     fc.workspaceBytes = wb;
   }
+  return fc;
+}
+
+// ------------------------------------------------------------ reductions with any body
+// stablehlo.reduce over n inputs with an arbitrary reducer region (argmax / argmin as JAX
+// lowers them: a (value, index) pair with a compare-select body; reference: the argmax/argmin
+// pattern of ops/reduction.cc:83-162).  The region is generated as straight-line code over
+// the accumulator tuple.  One wavefront per output: lanes stride over the reduced elements,
+// then a butterfly over the tuple.  Every lane starts from the init tuple, which the
+// operation allows to be combined any number of times.
+FusedCode generateRegionReduce(Op* reduce, const LeafPredicate& isLeaf) {
+  const size_t n = reduce->operands.size() / 2;
+  if (n == 0 || reduce->operands.size() != 2 * n || reduce->results.size() != n || reduce->regions.size() != 1)
+    throw CompileError("stablehlo.reduce: malformed operands");
+  Region& body = *reduce->regions[0];
+  if (body.args.size() != 2 * n || !body.terminator() || body.terminator()->operands.size() != n)
+    throw CompileError("stablehlo.reduce: the reducer region does not match the operands");
+  for (auto& op : body.ops)
+    if (op->name != "return" && (!isFusibleOp(*op) || op->results.size() != 1 || !op->regions.empty()))
+      throw CompileError("stablehlo.reduce: reducer body op stablehlo." + op->name + " is not supported");
+  Value* x0 = reduce->operands[0];
+  const std::vector<int64_t>& shape = x0->type.dims;
+  for (size_t j = 1; j < n; ++j)
+    if (reduce->operands[j]->type.dims != shape) throw CompileError("stablehlo.reduce: inputs of different shapes");
+  int rank = (int)shape.size();
+  std::vector<int64_t> rdims = reduce->ints("dimensions");
+  std::sort(rdims.begin(), rdims.end());
+  std::vector<bool> isRed(rank, false);
+  for (auto d : rdims) isRed[d] = true;
+  std::vector<int64_t> keptShape, redShape;
+  std::vector<int> keptDims, redDims;
+  for (int d = 0; d < rank; ++d) {
+    if (isRed[d]) { redShape.push_back(shape[d]); redDims.push_back(d); }
+    else { keptShape.push_back(shape[d]); keptDims.push_back(d); }
+  }
+  int64_t Kn = 1, Rn = 1;
+  for (auto d : keptShape) Kn *= d;
+  for (auto d : redShape) Rn *= d;
+  const bool i64 = x0->type.numel() >= (int64_t(1) << 31) - 16;
+  const std::string IT = i64 ? "i64" : "int";
+
+  Emitter em(isLeaf, 1, i64);
+  IdxDim klin;
+  klin.isConst = false; klin.base = "kk"; klin.coef = 0; klin.mult = 1;
+  auto kd = em.delinearize(klin, keptShape);
+  std::string savedPre = em.pre_;
+  em.pre_.clear();
+  IdxDim rlin;
+  rlin.isConst = false; rlin.base = "rb"; rlin.coef = 0; rlin.mult = 1;
+  auto rd = em.delinearize(rlin, redShape);
+  std::vector<IdxDim> full(rank);
+  for (size_t q = 0; q < keptDims.size(); ++q) full[keptDims[q]] = kd[q];
+  for (size_t q = 0; q < redDims.size(); ++q) full[redDims[q]] = rd[q];
+  Index idx = em.multiIndex(full, shape);
+  std::vector<std::string> vals;
+  for (size_t j = 0; j < n; ++j) vals.push_back(em.gen(reduce->operands[j], idx));
+  std::string loopPre = em.pre_;
+  em.pre_ = savedPre;
+  std::vector<std::string> inits;
+  for (size_t j = 0; j < n; ++j) inits.push_back(em.gen(reduce->operands[n + j], em.multiIndex({}, {})));
+
+  std::vector<DType> dts;
+  std::vector<std::string> accT;
+  for (size_t j = 0; j < n; ++j) { dts.push_back(reduce->results[j]->type.dt); accT.push_back(computeT(dts[j])); }
+
+  // (acc tuple) = body(acc tuple, other tuple), as a block of straight-line code
+  int site = 0;
+  auto combine = [&](const std::vector<std::string>& other, const std::string& indent) {
+    Emitter b(isLeaf, 1, i64);
+    b.shareLeavesFrom(em);
+    b.startTemporariesAt(100000 * (site + 1));
+    for (size_t j = 0; j < n; ++j) {
+      b.rowScalars_[body.args[j].get()] = "acc" + std::to_string(j);
+      b.rowScalars_[body.args[n + j].get()] = other[j];
+    }
+    std::vector<std::string> res;
+    for (size_t j = 0; j < n; ++j) res.push_back(b.gen(body.terminator()->operands[j], b.multiIndex({}, {})));
+    if (b.leaves_.size() != em.leaves_.size()) throw CompileError("stablehlo.reduce: the reducer region reads values defined outside it");
+    std::ostringstream o;
+    o << indent << "{\n" << b.pre_;
+    for (size_t j = 0; j < n; ++j) o << indent << "  const " << accT[j] << " nx" << site << "_" << j << " = " << roundTo(dts[j], res[j]) << ";\n";
+    for (size_t j = 0; j < n; ++j) o << indent << "  acc" << j << " = nx" << site << "_" << j << ";\n";
+    o << indent << "}\n";
+    ++site;
+    return o.str();
+  };
+
+  std::ostringstream s;
+  s << "  const int lane = threadIdx.x & 63;\n";
+  s << "  const " << IT << " kk = (" << IT << ")blockIdx.x * 4 + (threadIdx.x >> 6);\n";
+  s << "  if (kk >= " << Kn << ") return;\n";
+  s << em.pre_;
+  for (size_t j = 0; j < n; ++j) s << "  " << accT[j] << " acc" << j << " = " << inits[j] << ";\n";
+  s << "  for (" << IT << " rb = lane; rb < " << Rn << "; rb += 64) {\n";
+  s << loopPre;
+  s << "    { const int v = 0; (void)v;\n" << em.body_.front();
+  s << combine(vals, "    ");
+  s << "    }\n  }\n";
+  s << "  #pragma unroll\n  for (int o = 32; o > 0; o >>= 1) {\n";
+  std::vector<std::string> peers;
+  for (size_t j = 0; j < n; ++j) {
+    s << "    const " << accT[j] << " pr" << j << " = " << shflXor(accT[j], "acc" + std::to_string(j), "o") << ";\n";
+    peers.push_back("pr" + std::to_string(j));
+  }
+  s << combine(peers, "    ");
+  s << "  }\n";
+  s << "  if (lane != 0) return;\n";
+  for (size_t j = 0; j < n; ++j) s << "  out" << j << "[kk] = " << storeExpr(dts[j], "acc" + std::to_string(j)) << ";\n";
+  s << "}\n";
+
+  std::vector<std::string> outs;
+  for (size_t j = 0; j < n; ++j) outs.push_back(storageT(dts[j]) + "* __restrict__ out" + std::to_string(j));
+  FusedCode fc;
+  Launch l;
+  l.source = std::string(kPrelude) + kernelHeader(em.leaves_, outs) + " {\n" + s.str();
+  l.grid[0] = (unsigned)((Kn + 3) / 4);
+  l.block[0] = 256;
+  for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
+  for (size_t j = 0; j < n; ++j) { KArg a; a.kind = KArg::Out; a.value = reduce->results[j].get(); l.args.push_back(a); }
+  fc.leaves = em.leaves_;
+  fc.launches.push_back(std::move(l));
   return fc;
 }
 

@@ -42,6 +42,9 @@ using LeafPredicate = std::function<bool(Value*)>;
 FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf);
 FusedCode generateLoopKernel(const std::vector<Value*>& roots, const LeafPredicate& isLeaf);
 
+// stablehlo.reduce with several inputs and/or an arbitrary reducer region (argmax, argmin, ...).
+FusedCode generateRegionReduce(Op* reduce, const LeafPredicate& isLeaf);
+
 // Reductions over the trailing dims in dependency phases plus the elementwise values that
 // consume them, computed row by row in one kernel.
 struct RowProgram {

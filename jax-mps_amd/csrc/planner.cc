@@ -154,7 +154,7 @@ class Planner {
     if (isWindowReverse(v, user)) return false;
     if (user->name == "gather") return user->operands[0] == v;       // random access needs memory
     if (isFusibleOp(*user)) return false;
-    if (user->name == "reduce") return !isSimpleReduce(*user);
+    if (user->name == "reduce") return false;   // every reduce kernel evaluates its inputs in place
     if (user->name == "dynamic_update_slice") return user->operands[0] == v;
     return true;
   }
@@ -543,8 +543,30 @@ class Planner {
     return true;
   }
 
+  void emitRegionReduce(Op* op, Plan& plan) {
+    size_t n = op->operands.size() / 2;
+    for (size_t j = 0; j < n; ++j) {
+      // init values must be readable
+      std::vector<Value*> il;
+      std::unordered_set<Value*> seen;
+      collectLeavesOf(op->operands[n + j], il, seen);
+      for (auto* l : il) if (!hasStorage(l)) materializeNow(l, plan);
+    }
+    std::vector<Value*> outs;
+    for (auto& r : op->results) outs.push_back(r.get());
+    if (outs.empty() || outs[0]->type.numel() == 0) {
+      for (auto* o : outs) bind(o, newStorage(4));
+      return;
+    }
+    if (op->operands[0]->type.numel() == 0) throw CompileError("stablehlo.reduce over an empty tensor is not supported");
+    FusedCode fc = generateRegionReduce(op, leafPred());
+    for (auto* o : outs) bind(o, newStorage(o->type.bytes()));
+    emitted_.insert(op);
+    addFused(plan, fc, "reduce(region) " + op->operands[0]->type.str() + " -> " + outs[0]->type.str(), outs);
+  }
+
   void emitReduce(Op* op, Region& r, Plan& plan) {
-    if (!isSimpleReduce(*op)) throw CompileError("stablehlo.reduce with a variadic or non-trivial reducer body is not supported");
+    if (!isSimpleReduce(*op)) { emitRegionReduce(op, plan); return; }
     std::vector<Op*> group{op};
     std::vector<Value*> myLeaves;
     {

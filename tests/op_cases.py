@@ -306,6 +306,12 @@ case("reduce-bf16", lambda b, x: b.reduce_sum(x, [1]), f32(267, 12, 256), dtypes
 case("softmax-rows", lambda b, x: __import__("jax_mps_amd.shlo.builder", fromlist=["softmax"]).softmax(b, x, -1), f32(268, 33, 100))
 case("layer-norm", lambda b, x, s, t: __import__("jax_mps_amd.shlo.builder", fromlist=["layer_norm"]).layer_norm(b, x, s, t, 1e-5), f32(269, 20, 96), f32(270, 96), f32(271, 96))
 case("argmax", lambda b, x: b.argmax(x, 1), f32(272, 9, 31), exact=True)
+case("argmax-leading-dim", lambda b, x: b.argmax(x, 0), f32(2720, 150, 7), exact=True)
+case("argmax-middle-dim-long", lambda b, x: b.argmax(x, 1), f32(2721, 3, 1000, 5), exact=True)
+case("argmax-ties-first-occurrence", lambda b, x: b.argmax(x, 1),
+     np.array([[1, 3, 3, 2], [5, 5, 5, 5], [-1, -2, -1, -3], [0, -0.0, 0, 0]], np.float32), exact=True)
+case("argmax-nan-wins", lambda b, x: b.argmax(x, 1), np.array([[1, np.nan, 3, np.nan], [np.inf, 2, np.inf, 1], [-np.inf, -np.inf, -np.inf, -np.inf]], np.float32), exact=True)
+case("argmax-of-fused-input", lambda b, x, y: b.argmax(b.add(b.mul(x, y), 1.0), 1), f32(2722, 64, 10), f32(2723, 64, 10), exact=True)
 
 # ------------------------------------------------------------------ control flow (tests/configs/control_flow.py:66-80,232-263,389-458)
 def _sum_to_n(b, n, x):

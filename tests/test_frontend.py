@@ -30,14 +30,12 @@ def test_every_op_case_plans():
     bad = []
     for c in op_cases.all_cases():
         r = plan(c.text)
-        if r.returncode != 0 and c.name != "argmax":
+        if r.returncode != 0:
             bad.append((c.name, r.stderr[-300:]))
     assert not bad, bad
 
 
 def test_unsupported_ops_are_named():
-    r = plan(op_cases.get_case("argmax").text)
-    assert r.returncode != 0 and "variadic" in r.stderr
     r = plan("module { func.func public @main(%a: tensor<4xf32>) -> tensor<4xf32> {\n %0 = stablehlo.fft %a : tensor<4xf32>\n return %0 : tensor<4xf32> } }")
     assert r.returncode != 0 and ("fft" in r.stderr)
     r = plan("module { func.func public @main(%a: tensor<4xf64>) -> tensor<4xf64> {\n return %a : tensor<4xf64> } }")

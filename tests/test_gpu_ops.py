@@ -14,8 +14,8 @@ pytestmark = pytest.mark.gpu
 
 F32_TOL = 1e-5
 BF16_TOL = 2e-2
-# the plan compiler rejects these (the error text is checked in test_frontend.py)
-UNSUPPORTED = {"argmax"}
+# cases the plan compiler rejects (none at present; the error texts are checked in test_frontend.py)
+UNSUPPORTED = set()
 
 
 @pytest.mark.parametrize("name", [n for n in op_cases.case_names() if n not in UNSUPPORTED])
