@@ -141,6 +141,7 @@ std::unique_ptr<Module> parseStableHLOText(const char* data, size_t size);
 
 // Passes (passes.cc)
 void inlineCalls(Module& m);          // replaces every "call" by the callee body
+void lowerIntegerDots(Module& m);    // integer / boolean dot_general -> broadcast, multiply, reduce
 void eliminateDeadCode(Region& r);    // removes ops whose results are unused (recursively)
 void rebuildUses(Region& r);          // recompute Value::users for a region tree
 void checkSupported(const Module& m); // throws CompileError naming unsupported ops

@@ -174,6 +174,147 @@ void inlineCalls(Module& m) {
   }
 }
 
+// ---- integer / boolean dot_general ---------------------------------------------------------
+// The matrix cores have no exact 32-bit integer mode, and integer contractions are rare and
+// small on this path, so they are rewritten into ops the fused-reduction generator already
+// handles exactly:  broadcast both operands to [batch..., lhs free..., rhs free..., contracting...],
+// multiply (and for i1), reduce with add (or for i1) over the trailing dims.  Wrap-around
+// arithmetic, no detour through floats (the reference round-trips through f32 and is exact
+// only below 2^24: ops/linalg.cc:196-250).
+namespace {
+
+Value* addResult(Op* op, const TensorType& t, int& nextId) {
+  auto v = std::make_unique<Value>();
+  v->id = nextId++;
+  v->type = t;
+  v->def = op;
+  v->defIndex = (int)op->results.size();
+  v->name = "%lowered" + std::to_string(v->id);
+  op->results.push_back(std::move(v));
+  return op->results.back().get();
+}
+
+std::unique_ptr<Op> makeOp(const std::string& name, std::vector<Value*> operands, Region* parent, int line) {
+  auto op = std::make_unique<Op>();
+  op->name = name;
+  op->operands = std::move(operands);
+  op->parent = parent;
+  op->line = line;
+  return op;
+}
+
+Attr intsAttr(const std::vector<int64_t>& v) {
+  Attr a;
+  a.kind = Attr::Ints;
+  a.ints = v;
+  return a;
+}
+
+void lowerIntegerDotsIn(Region& r, int& nextId) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) lowerIntegerDotsIn(*sub, nextId);
+    if (op->name != "dot_general" && op->name != "dot") continue;
+    Value* a = op->operands[0];
+    Value* b = op->operands[1];
+    if (isFloat(a->type.dt)) continue;
+    Value* c = op->result();
+    const DType et = c->type.dt;
+    const bool pred = et == DType::Pred;
+    std::vector<int64_t> ab = op->ints("lhs_batch"), bb = op->ints("rhs_batch"), ac = op->ints("lhs_contract"), bc = op->ints("rhs_contract");
+    if (op->name == "dot") { ac = {a->type.rank() - 1}; bc = {0}; }
+    auto has = [](const std::vector<int64_t>& v, int64_t x) { return std::find(v.begin(), v.end(), x) != v.end(); };
+    std::vector<int64_t> af, bf;
+    for (int d = 0; d < a->type.rank(); ++d) if (!has(ab, d) && !has(ac, d)) af.push_back(d);
+    for (int d = 0; d < b->type.rank(); ++d) if (!has(bb, d) && !has(bc, d)) bf.push_back(d);
+    // the common index space and where each operand dim sits in it
+    std::vector<int64_t> space, aMap(a->type.rank()), bMap(b->type.rank());
+    for (size_t q = 0; q < ab.size(); ++q) { aMap[ab[q]] = (int64_t)space.size(); bMap[bb[q]] = (int64_t)space.size(); space.push_back(a->type.dims[ab[q]]); }
+    for (auto d : af) { aMap[d] = (int64_t)space.size(); space.push_back(a->type.dims[d]); }
+    for (auto d : bf) { bMap[d] = (int64_t)space.size(); space.push_back(b->type.dims[d]); }
+    std::vector<int64_t> redDims;
+    for (size_t q = 0; q < ac.size(); ++q) {
+      aMap[ac[q]] = (int64_t)space.size(); bMap[bc[q]] = (int64_t)space.size();
+      redDims.push_back((int64_t)space.size());
+      space.push_back(a->type.dims[ac[q]]);
+    }
+    std::vector<std::unique_ptr<Op>> made;
+    auto emit = [&](std::unique_ptr<Op> o, const TensorType& t) { Value* v = addResult(o.get(), t, nextId); made.push_back(std::move(o)); return v; };
+    auto widen = [&](Value* v) {   // operands take the result's element type first (preferred_element_type)
+      if (v->type.dt == et) return v;
+      TensorType t = v->type;
+      t.dt = et;
+      return emit(makeOp("convert", {v}, &r, op->line), t);
+    };
+    TensorType st;
+    st.dt = et;
+    st.dims = space;
+    auto spread = [&](Value* v, const std::vector<int64_t>& map) {
+      auto o = makeOp("broadcast_in_dim", {v}, &r, op->line);
+      o->attrs["dims"] = intsAttr(map);
+      return emit(std::move(o), st);
+    };
+    Value* A = spread(widen(a), aMap);
+    Value* B = spread(widen(b), bMap);
+    Value* prod = emit(makeOp(pred ? "and" : "multiply", {A, B}, &r, op->line), st);
+    // init: zero of the element type
+    auto zero = makeOp("constant", {}, &r, op->line);
+    Attr dv;
+    dv.kind = Attr::Dense;
+    dv.dense = std::make_shared<DenseData>();
+    dv.dense->type.dt = et;
+    dv.dense->splat = true;
+    dv.dense->bytes.assign(dtypeSize(et), 0);
+    zero->attrs["value"] = dv;
+    TensorType scalar;
+    scalar.dt = et;
+    Value* z = emit(std::move(zero), scalar);
+    // the reduce takes over the dot's result value, so its users need no rewiring
+    auto red = makeOp("reduce", {prod, z}, &r, op->line);
+    red->attrs["dimensions"] = intsAttr(redDims);
+    auto body = std::make_unique<Region>();
+    body->parent = red.get();
+    for (int q = 0; q < 2; ++q) {
+      auto arg = std::make_unique<Value>();
+      arg->id = nextId++;
+      arg->type = scalar;
+      arg->argOf = body.get();
+      arg->defIndex = q;
+      arg->name = "%lowered_arg" + std::to_string(arg->id);
+      body->args.push_back(std::move(arg));
+    }
+    auto comb = makeOp(pred ? "or" : "add", {body->args[0].get(), body->args[1].get()}, body.get(), op->line);
+    Value* cv = addResult(comb.get(), scalar, nextId);
+    auto ret = makeOp("return", {cv}, body.get(), op->line);
+    body->ops.push_back(std::move(comb));
+    body->ops.push_back(std::move(ret));
+    red->regions.push_back(std::move(body));
+    red->results = std::move(op->results);
+    for (auto& v : red->results) v->def = red.get();
+    if (redDims.empty()) {
+      // nothing to contract: the product is the result
+      red->name = "reshape";
+      red->operands = {prod};
+      red->regions.clear();
+      red->attrs.clear();
+    }
+    made.push_back(std::move(red));
+    size_t nIns = made.size();
+    r.ops.erase(r.ops.begin() + k);
+    r.ops.insert(r.ops.begin() + k, std::make_move_iterator(made.begin()), std::make_move_iterator(made.end()));
+    k += nIns - 1;
+  }
+}
+
+}  // namespace
+
+void lowerIntegerDots(Module& m) {
+  Func* f = m.main();
+  if (!f) return;
+  int nextId = maxValueId(f->body) + 1;
+  lowerIntegerDotsIn(f->body, nextId);
+}
+
 void eliminateDeadCode(Region& r) {
   std::unordered_map<const Value*, int> uses;
   collectUses(r, uses);

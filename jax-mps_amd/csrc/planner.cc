@@ -1237,6 +1237,7 @@ mi355_conv_desc toAbi(const ConvDesc& c) {
 std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) {
   auto prog = std::make_unique<CompiledProgram>();
   inlineCalls(*module);
+  lowerIntegerDots(*module);
   checkSupported(*module);
   eliminateDeadCode(module->main()->body);
   prog->module = std::move(module);

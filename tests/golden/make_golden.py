@@ -126,6 +126,11 @@ add("sign_keeps_nan_and_zero", lambda b, x: b.sign(x), [np.array([-3.0, 0.0, 5.0
 # dot_general of small integers exact in float (matmul.py:221-249 restated in f32)
 a = np.array([[1, 2, 3], [4, 5, 6]], np.float32); bb = np.array([[7, 8], [9, 10], [11, 12]], np.float32)
 add("matmul_2x3_3x2", lambda b, x, y: b.matmul(x, y), [a, bb], np.array([[58, 64], [139, 154]], np.float32), "tests/configs/matmul.py:19-30")
+# integer and boolean contractions with the literal operands of the reference's tests (matmul.py:221-249)
+add("dot_int32", lambda b, x, y: b.dot_general(x, y, ([0], [0])), [np.array([1, 2, 3], np.int32), np.array([4, 5, 6], np.int32)], np.array(32, np.int32), "tests/configs/matmul.py:221-228")
+add("matmul_int32", lambda b, x, y: b.matmul(x, y), [np.array([[1, 2], [3, 4]], np.int32), np.array([[5, 6], [7, 8]], np.int32)], np.array([[19, 22], [43, 50]], np.int32), "tests/configs/matmul.py:229-235")
+add("dot_bool", lambda b, x, y: b.dot_general(x, y, ([0], [0])), [np.array([True, False, True]), np.array([True, True, False])], np.array(True), "tests/configs/matmul.py:236-242")
+add("matmul_uint32", lambda b, x, y: b.matmul(x, y), [np.array([[1, 2], [3, 4]], np.uint32), np.array([[5, 6], [7, 8]], np.uint32)], np.array([[19, 22], [43, 50]], np.uint32), "tests/configs/matmul.py:243-249")
 add("pad_edge_and_interior", lambda b, x: b.pad(x, 0.0, [1], [2], [1]), [np.array([1, 2, 3], np.float32)], np.array([0, 1, 0, 2, 0, 3, 0, 0], np.float32), "src/pjrt_plugin/ops/slice.cc:202-276")
 add("pad_negative_crops", lambda b, x: b.pad(x, 9.0, [-1], [1], [0]), [np.array([1, 2, 3], np.float32)], np.array([2, 3, 9], np.float32), "src/pjrt_plugin/ops/slice.cc:202-276")
 

@@ -229,6 +229,13 @@ case("dot-bf16-async-nt", lambda b, x, y: b.dot_general(x, y, ([1], [1])), f32(1
 case("dot-bf16-async-nt-long-k", lambda b, x, y: b.dot_general(x, y, ([1], [1]), out_dtype="f32"), f32(1918, 300, 1024, lo=-1, hi=1), f32(1919, 130, 1024, lo=-1, hi=1), dtypes=["bf16", "bf16"])
 case("dot-bf16-async-nt-one-slab", lambda b, x, y: b.dot_general(x, y, ([1], [1])), f32(1920, 70, 64), f32(1921, 50, 64), dtypes=["bf16", "bf16"])
 case("dot-bf16-async-nt-big", lambda b, x, y: b.dot_general(x, y, ([1], [1])), f32(1922, 1024, 512, lo=-1, hi=1), f32(1923, 768, 512, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+# integer contractions are lowered to broadcast-multiply-reduce (exact, wrap-around)
+def i32(seed, *shape, lo=-1000, hi=1000):
+    return rng(seed).integers(lo, hi, size=shape).astype(np.int32)
+case("dot-int32-matmul", lambda b, x, y: b.matmul(x, y), i32(1930, 33, 70), i32(1931, 70, 45), exact=True)
+case("dot-int32-batched-attention-layout", lambda b, q, k: b.dot_general(q, k, ([3], [3]), ([0, 2], [0, 2])), i32(1932, 2, 9, 3, 16), i32(1933, 2, 11, 3, 16), exact=True)
+case("dot-int32-wraps", lambda b, x, y: b.matmul(x, y), i32(1934, 8, 300, lo=-2**30, hi=2**30), i32(1935, 300, 8, lo=-2**30, hi=2**30), exact=True)
+case("dot-uint32-above-2p24", lambda b, x, y: b.matmul(x, y), rng(1936).integers(0, 2**20, size=(5, 40)).astype(np.uint32), rng(1937).integers(0, 2**11, size=(40, 6)).astype(np.uint32), exact=True)
 case("dot-large-k", lambda b, x, y: b.matmul(x, y), f32(192, 64, 3000, lo=-1, hi=1), f32(193, 3000, 64, lo=-1, hi=1))
 
 
