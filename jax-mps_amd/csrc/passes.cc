@@ -3,6 +3,7 @@
 // things with MLIR's inliner + SymbolDCE and its handler-table scan (reference:
 // src/pjrt_plugin/stablehlo_parser.cc:129-149, 167-184).
 #include <functional>
+#include <cstring>
 #include <set>
 #include <unordered_map>
 #include <unordered_set>
@@ -313,6 +314,206 @@ void lowerIntegerDots(Module& m) {
   if (!f) return;
   int nextId = maxValueId(f->body) + 1;
   lowerIntegerDotsIn(f->body, nextId);
+}
+
+// ---- general scatter -------------------------------------------------------------------------
+// A scatter that is not "whole rows along dim 0" is rewritten into that form over single
+// elements: every update element gets the linear index of the operand element it lands on
+// (computed with iota / slice / broadcast / multiply-add, i.e. one fused kernel), or an
+// out-of-range key when its window does not fit the operand; the flattened operand is then
+// scattered one element per "row".  The ordered fold of the row scatter therefore gives the
+// sequential update order for every scatter form (reference: DetectScatterType / ApplyScatter,
+// ops/gather_scatter.cc:296-699, which leaves the order to float atomics).
+namespace {
+
+bool isRowScatter(const Op& op) {
+  if (op.operands.size() != 3) return false;
+  const TensorType& operand = op.operands[0]->type;
+  const TensorType& idx = op.operands[1]->type;
+  const TensorType& upd = op.operands[2]->type;
+  auto& uwd = op.ints("update_window_dims");
+  if (operand.rank() < 1 || op.ints("inserted_window_dims") != std::vector<int64_t>{0} ||
+      op.ints("scatter_dims_to_operand_dims") != std::vector<int64_t>{0} || !op.ints("input_batching_dims").empty())
+    return false;
+  int nScatter = upd.rank() - (int)uwd.size();
+  for (size_t k = 0; k < uwd.size(); ++k) if (uwd[k] != nScatter + (int64_t)k) return false;
+  if ((int)uwd.size() != operand.rank() - 1) return false;
+  for (size_t k = 0; k < uwd.size(); ++k) if (upd.dims[uwd[k]] != operand.dims[1 + k]) return false;
+  int64_t nUpd = 1;
+  for (int d = 0; d < nScatter; ++d) nUpd *= upd.dims[d];
+  int64_t ivd = op.integer("index_vector_dim");
+  if (ivd < idx.rank() && idx.dims[ivd] != 1) return false;
+  return idx.numel() == nUpd;
+}
+
+void lowerScattersIn(Region& r, int& nextId) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) lowerScattersIn(*sub, nextId);
+    if (op->name != "scatter" || op->operands.size() != 3 || isRowScatter(*op)) continue;
+    Value* operand = op->operands[0];
+    Value* idx = op->operands[1];
+    Value* upd = op->operands[2];
+    const TensorType ot = operand->type, it = idx->type, ut = upd->type;
+    const int64_t P = ot.numel(), n = ut.numel();
+    if (P >= (int64_t(1) << 32) - 1) throw CompileError("stablehlo.scatter: operand too large for element-wise lowering");
+    auto uwd = op->ints("update_window_dims"), iwd = op->ints("inserted_window_dims"), ibd = op->ints("input_batching_dims"),
+         sibd = op->ints("scatter_indices_batching_dims"), sdo = op->ints("scatter_dims_to_operand_dims");
+    const int64_t ivd = op->has("index_vector_dim") ? op->integer("index_vector_dim") : it.rank();
+    auto has = [](const std::vector<int64_t>& v, int64_t x) { return std::find(v.begin(), v.end(), x) != v.end(); };
+    std::vector<int64_t> sd;                       // scatter dims of the updates, in order
+    for (int d = 0; d < ut.rank(); ++d) if (!has(uwd, d)) sd.push_back(d);
+    std::vector<int64_t> idxBatchAxes;             // dims of the index tensor except the vector dim
+    for (int d = 0; d < it.rank(); ++d) if (d != ivd) idxBatchAxes.push_back(d);
+    if (idxBatchAxes.size() != sd.size()) throw CompileError("stablehlo.scatter: index and update ranks do not agree");
+    std::vector<int64_t> winDims;                  // operand dims that carry a window coordinate
+    for (int d = 0; d < ot.rank(); ++d) if (!has(iwd, d) && !has(ibd, d)) winDims.push_back(d);
+    if (winDims.size() != uwd.size()) throw CompileError("stablehlo.scatter: update_window_dims do not match the operand");
+
+    std::vector<std::unique_ptr<Op>> made;
+    auto emit = [&](std::unique_ptr<Op> o, const TensorType& t) { Value* v = addResult(o.get(), t, nextId); made.push_back(std::move(o)); return v; };
+    TensorType i64u;                // int64 over the update index space
+    i64u.dt = DType::S64;
+    i64u.dims = ut.dims;
+    TensorType predu = i64u;
+    predu.dt = DType::Pred;
+    auto splat = [&](int64_t x) {
+      auto c = makeOp("constant", {}, &r, op->line);
+      Attr dv;
+      dv.kind = Attr::Dense;
+      dv.dense = std::make_shared<DenseData>();
+      dv.dense->type.dt = DType::S64;
+      dv.dense->type.dims = ut.dims;
+      dv.dense->splat = true;
+      dv.dense->bytes.resize(8);
+      memcpy(dv.dense->bytes.data(), &x, 8);
+      c->attrs["value"] = dv;
+      return emit(std::move(c), i64u);
+    };
+    auto iota = [&](int64_t dim) {
+      auto o = makeOp("iota", {}, &r, op->line);
+      Attr a;
+      a.kind = Attr::Int;
+      a.i = dim;
+      o->attrs["dim"] = a;
+      return emit(std::move(o), i64u);
+    };
+    auto binary = [&](const char* name, Value* a, Value* b, const TensorType& t) { return emit(makeOp(name, {a, b}, &r, op->line), t); };
+    auto compare = [&](const char* dir, Value* a, Value* b) {
+      auto o = makeOp("compare", {a, b}, &r, op->line);
+      Attr d;
+      d.kind = Attr::Str;
+      d.s = dir;
+      o->attrs["direction"] = d;
+      return emit(std::move(o), predu);
+    };
+    // component q of the index vector, spread over the update index space
+    auto component = [&](int64_t q) {
+      Value* v = idx;
+      if (ivd < it.rank()) {
+        auto sl = makeOp("slice", {idx}, &r, op->line);
+        std::vector<int64_t> st(it.rank(), 0), lim = it.dims, sr(it.rank(), 1);
+        st[ivd] = q;
+        lim[ivd] = q + 1;
+        sl->attrs["start"] = intsAttr(st);
+        sl->attrs["limit"] = intsAttr(lim);
+        sl->attrs["strides"] = intsAttr(sr);
+        TensorType t = it;
+        t.dims[ivd] = 1;
+        v = emit(std::move(sl), t);
+      }
+      TensorType bt;
+      bt.dt = it.dt;
+      for (auto a : idxBatchAxes) bt.dims.push_back(it.dims[a]);
+      v = emit(makeOp("reshape", {v}, &r, op->line), bt);
+      TensorType ct = bt;
+      ct.dt = DType::S64;
+      if (bt.dt != DType::S64) v = emit(makeOp("convert", {v}, &r, op->line), ct);
+      auto bc = makeOp("broadcast_in_dim", {v}, &r, op->line);
+      bc->attrs["dims"] = intsAttr(sd);
+      return emit(std::move(bc), i64u);
+    };
+    std::vector<int64_t> stride(ot.rank(), 1);
+    for (int d = ot.rank() - 2; d >= 0; --d) stride[d] = stride[d + 1] * ot.dims[d + 1];
+    Value* lin = splat(0);
+    Value* inb = nullptr;
+    for (int d = 0; d < ot.rank(); ++d) {
+      Value* coord = nullptr;
+      auto add = [&](Value* v) { coord = coord ? binary("add", coord, v, i64u) : v; };
+      auto sIt = std::find(sdo.begin(), sdo.end(), (int64_t)d);
+      int64_t ws = 1;
+      auto wIt = std::find(winDims.begin(), winDims.end(), (int64_t)d);
+      if (wIt != winDims.end()) ws = ut.dims[uwd[wIt - winDims.begin()]];
+      if (sIt != sdo.end()) {
+        Value* start = component(sIt - sdo.begin());
+        Value* ok = binary("and", compare("GE", start, splat(0)), compare("LE", start, splat(ot.dims[d] - ws)), predu);
+        inb = inb ? binary("and", inb, ok, predu) : ok;
+        add(start);
+      }
+      if (wIt != winDims.end()) add(iota(uwd[wIt - winDims.begin()]));
+      auto bIt = std::find(ibd.begin(), ibd.end(), (int64_t)d);
+      if (bIt != ibd.end()) {
+        int64_t ib = sibd.at(bIt - ibd.begin());
+        auto pos = std::find(idxBatchAxes.begin(), idxBatchAxes.end(), ib);
+        if (pos == idxBatchAxes.end()) throw CompileError("stablehlo.scatter: scatter_indices_batching_dims names the index vector dim");
+        add(iota(sd[pos - idxBatchAxes.begin()]));
+      }
+      if (!coord) continue;
+      lin = binary("add", lin, stride[d] == 1 ? coord : binary("multiply", coord, splat(stride[d]), i64u), i64u);
+    }
+    Value* key64 = lin;
+    if (inb) {
+      auto sel = makeOp("select", {inb, lin, splat(P)}, &r, op->line);
+      key64 = emit(std::move(sel), i64u);
+    }
+    TensorType keyT = i64u;
+    keyT.dt = DType::U32;
+    Value* key = emit(makeOp("convert", {key64}, &r, op->line), keyT);
+    TensorType flatKey;
+    flatKey.dt = DType::U32;
+    flatKey.dims = {n};
+    key = emit(makeOp("reshape", {key}, &r, op->line), flatKey);
+    TensorType flatUpd;
+    flatUpd.dt = ut.dt;
+    flatUpd.dims = {n};
+    Value* fu = emit(makeOp("reshape", {upd}, &r, op->line), flatUpd);
+    TensorType flatOp;
+    flatOp.dt = ot.dt;
+    flatOp.dims = {P};
+    Value* fo = emit(makeOp("reshape", {operand}, &r, op->line), flatOp);
+    // the element scatter keeps the original body
+    auto sc = makeOp("scatter", {fo, key, fu}, &r, op->line);
+    sc->attrs["update_window_dims"] = intsAttr({});
+    sc->attrs["inserted_window_dims"] = intsAttr({0});
+    sc->attrs["scatter_dims_to_operand_dims"] = intsAttr({0});
+    Attr one;
+    one.kind = Attr::Int;
+    one.i = 1;
+    sc->attrs["index_vector_dim"] = one;
+    for (auto& kv : op->attrs)
+      if (kv.first == "unique_indices" || kv.first == "indices_are_sorted") sc->attrs[kv.first] = kv.second;
+    sc->regions = std::move(op->regions);
+    for (auto& rg : sc->regions) rg->parent = sc.get();
+    Value* flatRes = emit(std::move(sc), flatOp);
+    // a reshape takes over the original result value
+    auto back = makeOp("reshape", {flatRes}, &r, op->line);
+    back->results = std::move(op->results);
+    for (auto& v : back->results) v->def = back.get();
+    made.push_back(std::move(back));
+    size_t nIns = made.size();
+    r.ops.erase(r.ops.begin() + k);
+    r.ops.insert(r.ops.begin() + k, std::make_move_iterator(made.begin()), std::make_move_iterator(made.end()));
+    k += nIns - 1;
+  }
+}
+
+}  // namespace
+
+void lowerGeneralScatters(Module& m) {
+  Func* f = m.main();
+  if (!f) return;
+  int nextId = maxValueId(f->body) + 1;
+  lowerScattersIn(f->body, nextId);
 }
 
 void eliminateDeadCode(Region& r) {

@@ -1238,6 +1238,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   auto prog = std::make_unique<CompiledProgram>();
   inlineCalls(*module);
   lowerIntegerDots(*module);
+  lowerGeneralScatters(*module);
   checkSupported(*module);
   eliminateDeadCode(module->main()->body);
   prog->module = std::move(module);

@@ -193,6 +193,21 @@ case("scatter-large-int32", _row_scatter("set"), np.zeros((5, 1), np.int32), np.
 case("scatter-large-uint32", _row_scatter("set"), np.zeros((5, 1), np.uint32), np.array([2], np.int32), np.array([[16777217]], np.uint32), exact=True)
 case("scatter-add-many", _row_scatter("add"), f32(160, 300, 70), rng(161).integers(0, 300, size=1000).astype(np.int32), f32(162, 1000, 70), exact=True)
 
+# scatter forms other than whole rows along dim 0 (lowered to an element scatter with computed keys)
+case("scatter-point-2d-add", lambda b, x, i, u: b.scatter(x, i, u, update_window_dims=[], inserted_window_dims=[0, 1], scatter_dims_to_operand_dims=[0, 1], index_vector_dim=1),
+     f32(1940, 6, 7), np.array([[0, 0], [5, 6], [2, 3], [2, 3], [6, 0], [-1, 2], [2, 3]], np.int32), f32(1941, 7), exact=True)
+case("scatter-along-dim1-set", lambda b, x, i, u: b.scatter(x, i, u, update_window_dims=[0], inserted_window_dims=[1], scatter_dims_to_operand_dims=[1], index_vector_dim=1, body="set"),
+     f32(1942, 5, 8), np.array([[7], [0], [3]], np.int32), f32(1943, 5, 3), exact=True)
+case("scatter-window-2x3-add", lambda b, x, i, u: b.scatter(x, i, u, update_window_dims=[1, 2], inserted_window_dims=[], scatter_dims_to_operand_dims=[0, 1], index_vector_dim=1),
+     f32(1944, 10, 12), np.array([[0, 0], [8, 9], [3, 4], [4, 5], [9, 9], [8, 10]], np.int32), f32(1945, 6, 2, 3), exact=True)
+case("scatter-index-vector-dim0-max", lambda b, x, i, u: b.scatter(x, i, u, update_window_dims=[], inserted_window_dims=[0, 1], scatter_dims_to_operand_dims=[1, 0], index_vector_dim=0, body="max"),
+     f32(1946, 4, 9), np.array([[8, 0, 3, 3, 8], [3, 0, 1, 1, 3]], np.int32), f32(1947, 5), exact=True)
+case("scatter-batched-dims-add", lambda b, x, i, u: b.scatter(x, i, u, update_window_dims=[], inserted_window_dims=[1], scatter_dims_to_operand_dims=[1], index_vector_dim=2,
+                                                              input_batching_dims=[0], scatter_indices_batching_dims=[0]),
+     f32(1948, 3, 10), rng(1949).integers(0, 10, size=(3, 6, 1)).astype(np.int32), f32(1950, 3, 6), exact=True)
+case("scatter-point-int32-many", lambda b, x, i, u: b.scatter(x, i, u, update_window_dims=[], inserted_window_dims=[0, 1], scatter_dims_to_operand_dims=[0, 1], index_vector_dim=1),
+     rng(1951).integers(-9, 9, size=(20, 30)).astype(np.int32), rng(1952).integers(0, 20, size=(2000, 2)).astype(np.int32), rng(1953).integers(-100, 100, size=(2000,)).astype(np.int32), exact=True)
+
 # hot rows: runs of equal indices longer than the LDS index tile (256) and the staging round (128), next to short runs
 def _hot(seed, n, rows):
     r = rng(seed)
