@@ -73,7 +73,11 @@ struct PJRT_Executable {
   std::vector<PJRT_NamedValue> cost;
   std::vector<std::string> costNames;
   std::string fingerprint;
+  std::string source;            // program text as compiled (what Serialize hands out)
   bool ownedByLoaded = false;
+};
+struct PJRT_SerializedExecutable {
+  std::string bytes;
 };
 struct PJRT_LoadedExecutable {
   PJRT_Executable* executable = nullptr;
@@ -366,27 +370,33 @@ void fillExecutableMetadata(PJRT_Executable* e) {
   e->fingerprint = fp;
 }
 
+// text -> plan -> loaded executable (shared by Compile and DeserializeAndLoad)
+PJRT_LoadedExecutable* compileAndLoad(PJRT_Client* client, const char* code, size_t size) {
+  auto module = parseStableHLOText(code, size);
+  auto prog = compileProgram(std::move(module));
+  auto* ex = new PJRT_Executable();
+  try {
+    ex->exe = std::make_shared<Executable>(std::move(prog));
+  } catch (...) {
+    delete ex;
+    throw;
+  }
+  ex->source.assign(code, size);
+  ex->ownedByLoaded = true;
+  fillExecutableMetadata(ex);
+  auto* le = new PJRT_LoadedExecutable();
+  le->executable = ex;
+  le->client = client;
+  return le;
+}
+
 PJRT_Error* Client_Compile(PJRT_Client_Compile_Args* a) {
   return guard([&]() -> PJRT_Error* {
     std::lock_guard<std::recursive_mutex> lk(apiMutex());
     if (!a->program || !a->program->code) return makeError("null program", PJRT_Error_Code_INVALID_ARGUMENT);
     std::string format(a->program->format ? a->program->format : "", a->program->format ? a->program->format_size : 0);
     if (format != "mlir") return makeError("unsupported program format '" + format + "' (expected 'mlir')", PJRT_Error_Code_INVALID_ARGUMENT);
-    auto module = parseStableHLOText(a->program->code, a->program->code_size);
-    auto prog = compileProgram(std::move(module));
-    auto* ex = new PJRT_Executable();
-    try {
-      ex->exe = std::make_shared<Executable>(std::move(prog));
-    } catch (...) {
-      delete ex;
-      throw;
-    }
-    ex->ownedByLoaded = true;
-    fillExecutableMetadata(ex);
-    auto* le = new PJRT_LoadedExecutable();
-    le->executable = ex;
-    le->client = a->client;
-    a->executable = le;
+    a->executable = compileAndLoad(a->client, a->program->code, a->program->code_size);
     return nullptr;
   });
 }
@@ -572,7 +582,26 @@ PJRT_Error* Executable_OutputMemoryKinds(PJRT_Executable_OutputMemoryKinds_Args*
   return nullptr;
 }
 PJRT_Error* Executable_OptimizedProgram(PJRT_Executable_OptimizedProgram_Args*) { return unimplemented("PJRT_Executable_OptimizedProgram"); }
-PJRT_Error* Executable_Serialize(PJRT_Executable_Serialize_Args*) { return unimplemented("PJRT_Executable_Serialize"); }
+// A serialized executable is the program text behind a small header: loading it again replans
+// (milliseconds) and finds every generated kernel in the on-disk code-object cache, so nothing
+// is recompiled.  The reference leaves both entry points unimplemented (pjrt_executable.cc:101-107,
+// 269-271); with them JAX's persistent compilation cache works.
+constexpr char kSerialMagic[] = "MI355X-PJRT-EXE\x01";
+PJRT_Error* Executable_Serialize(PJRT_Executable_Serialize_Args* a) {
+  return guard([&]() -> PJRT_Error* {
+    if (!a->executable) return makeError("null executable", PJRT_Error_Code_INVALID_ARGUMENT);
+    auto* out = new PJRT_SerializedExecutable();
+    out->bytes.assign(kSerialMagic, sizeof(kSerialMagic) - 1);
+    uint64_t n = a->executable->source.size();
+    out->bytes.append((const char*)&n, sizeof n);
+    out->bytes += a->executable->source;
+    a->serialized_executable = out;
+    a->serialized_bytes = out->bytes.data();
+    a->serialized_bytes_size = out->bytes.size();
+    a->serialized_executable_deleter = [](PJRT_SerializedExecutable* p) { delete p; };
+    return nullptr;
+  });
+}
 PJRT_Error* Executable_OutputElementTypes(PJRT_Executable_OutputElementTypes_Args* a) {
   a->output_types = a->executable->outTypes.data();
   a->num_output_types = a->executable->outTypes.size();
@@ -591,7 +620,19 @@ PJRT_Error* Executable_Fingerprint(PJRT_Executable_Fingerprint_Args* a) {
 }
 PJRT_Error* Executable_GetCompiledMemoryStats(PJRT_Executable_GetCompiledMemoryStats_Args*) { return unimplemented("PJRT_Executable_GetCompiledMemoryStats"); }
 PJRT_Error* Executable_GetCompileOptions(PJRT_Executable_GetCompileOptions_Args*) { return unimplemented("PJRT_Executable_GetCompileOptions"); }
-PJRT_Error* Executable_DeserializeAndLoad(PJRT_Executable_DeserializeAndLoad_Args*) { return unimplemented("PJRT_Executable_DeserializeAndLoad"); }
+PJRT_Error* Executable_DeserializeAndLoad(PJRT_Executable_DeserializeAndLoad_Args* a) {
+  return guard([&]() -> PJRT_Error* {
+    std::lock_guard<std::recursive_mutex> lk(apiMutex());
+    const size_t head = sizeof(kSerialMagic) - 1 + sizeof(uint64_t);
+    if (!a->serialized_executable || a->serialized_executable_size < head || memcmp(a->serialized_executable, kSerialMagic, sizeof(kSerialMagic) - 1) != 0)
+      return makeError("not an executable serialized by this plugin", PJRT_Error_Code_INVALID_ARGUMENT);
+    uint64_t n = 0;
+    memcpy(&n, a->serialized_executable + sizeof(kSerialMagic) - 1, sizeof n);
+    if (n != a->serialized_executable_size - head) return makeError("serialized executable is truncated", PJRT_Error_Code_INVALID_ARGUMENT);
+    a->loaded_executable = compileAndLoad(a->client, a->serialized_executable + head, (size_t)n);
+    return nullptr;
+  });
+}
 
 PJRT_Error* LoadedExecutable_Destroy(PJRT_LoadedExecutable_Destroy_Args* a) {
   std::lock_guard<std::recursive_mutex> lk(apiMutex());

@@ -48,6 +48,12 @@ class Program(C.Structure):
 Client_Compile_Args = _args("Client_Compile_Args", [
     ("client", _P), ("program", C.POINTER(Program)), ("compile_options", C.c_char_p), ("compile_options_size", _SZ),
     ("executable", _P)])
+Executable_Serialize_Args = _args("Executable_Serialize_Args", [
+    ("executable", _P), ("serialized_bytes", _P), ("serialized_bytes_size", _SZ), ("serialized_executable", _P),
+    ("serialized_executable_deleter", C.CFUNCTYPE(None, _P))])
+Executable_DeserializeAndLoad_Args = _args("Executable_DeserializeAndLoad_Args", [
+    ("client", _P), ("serialized_executable", C.c_char_p), ("serialized_executable_size", _SZ), ("loaded_executable", _P),
+    ("overridden_serialized_compile_options", C.c_char_p), ("overridden_serialized_compile_options_size", _SZ)])
 BufferFromHostBuffer_Args = _args("BufferFromHostBuffer_Args", [
     ("client", _P), ("data", _P), ("type", C.c_int), ("dims", C.POINTER(C.c_int64)), ("num_dims", _SZ),
     ("byte_strides", C.POINTER(C.c_int64)), ("num_byte_strides", _SZ), ("host_buffer_semantics", C.c_int),
@@ -321,6 +327,14 @@ class LoadedExecutable:
             p.call("PJRT_Event_Destroy", Event_Args(event=events[0]))
         return [Buffer(self.client, out_arr[i]) for i in range(self.num_outputs)]
 
+    def serialize(self) -> bytes:
+        """PJRT_Executable_Serialize: bytes that `Client.deserialize_and_load` turns back into a loaded executable."""
+        a = self.client.plugin.call("PJRT_Executable_Serialize", Executable_Serialize_Args(executable=self.exe))
+        data = C.string_at(a.serialized_bytes, a.serialized_bytes_size)
+        if a.serialized_executable_deleter:
+            a.serialized_executable_deleter(a.serialized_executable)
+        return data
+
     def cost_analysis(self) -> dict:
         a = self.client.plugin.call("PJRT_Executable_GetCostAnalysis", Executable_GetCostAnalysis_Args(executable=self.exe))
         out = {}
@@ -376,6 +390,12 @@ class Client:
         a = Client_Compile_Args(client=self.handle, program=C.pointer(prog), compile_options=None, compile_options_size=0)
         self.plugin.call("PJRT_Client_Compile", a)
         return LoadedExecutable(self, a.executable)
+
+    def deserialize_and_load(self, data: bytes) -> LoadedExecutable:
+        a = Executable_DeserializeAndLoad_Args(client=self.handle, serialized_executable=data, serialized_executable_size=len(data),
+                                               overridden_serialized_compile_options=None, overridden_serialized_compile_options_size=0)
+        self.plugin.call("PJRT_Executable_DeserializeAndLoad", a)
+        return LoadedExecutable(self, a.loaded_executable)
 
     def buffer_from_pyval(self, x, dtype_code: Optional[int] = None) -> Buffer:
         arr = np.asarray(x)

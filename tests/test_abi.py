@@ -74,7 +74,18 @@ def test_client_create_without_gpu_is_a_clean_error(plugin):
 def test_unimplemented_entries_return_the_code(plugin):
     class A(C.Structure):
         _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("pad", C.c_void_p * 8)]
-    for name in ("PJRT_Executable_Serialize", "PJRT_Executable_DeserializeAndLoad", "PJRT_Compile", "PJRT_Executable_OptimizedProgram"):
+    for name in ("PJRT_Compile", "PJRT_Executable_OptimizedProgram", "PJRT_TopologyDescription_Serialize"):
         with pytest.raises(pjrt.PjrtError) as e:
             plugin.call(name, A())
         assert e.value.code == 12, name
+
+
+def test_serialization_entries_reject_bad_arguments(plugin):
+    """Serialize / DeserializeAndLoad are implemented; without valid arguments they answer INVALID_ARGUMENT, not a crash."""
+    with pytest.raises(pjrt.PjrtError) as e:
+        plugin.call("PJRT_Executable_Serialize", pjrt.Executable_Serialize_Args(executable=None))
+    assert e.value.code == 3
+    with pytest.raises(pjrt.PjrtError) as e:
+        plugin.call("PJRT_Executable_DeserializeAndLoad", pjrt.Executable_DeserializeAndLoad_Args(
+            client=None, serialized_executable=b"junk", serialized_executable_size=4))
+    assert e.value.code == 3

@@ -178,6 +178,28 @@ def test_error_paths(client):
     assert stats["bytes_in_use"] > 0 and stats["bytes_limit"] > 2**36
 
 
+def test_serialize_round_trip(client):
+    """PJRT_Executable_Serialize -> PJRT_Executable_DeserializeAndLoad gives an executable with the same results
+    (the reference leaves both unimplemented: pjrt_executable.cc:101-107, 269-271)."""
+    from jax_mps_amd import pjrt, runner
+    from jax_mps_amd.programs import configs
+    p = configs.build_mlp(**configs.SMALL["mlp"])
+    cp = runner.CompiledProgram(p, client)
+    want = cp.run_once()
+    blob = cp.exe.serialize()
+    assert blob.startswith(b"MI355X-PJRT-EXE") and p.text.encode() in blob
+    exe2 = client.deserialize_and_load(blob)
+    got = [runner.download(o) for o in exe2.execute(cp.state)]
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+    with pytest.raises(pjrt.PjrtError) as e:
+        client.deserialize_and_load(b"not an executable")
+    assert e.value.code == 3   # INVALID_ARGUMENT
+    with pytest.raises(pjrt.PjrtError):
+        client.deserialize_and_load(blob[:-5])
+
+
 def test_strided_host_buffer(client):
     x = np.arange(24, dtype=np.float32).reshape(4, 6).T   # non-contiguous host view
     buf = client.buffer_from_pyval(x)
