@@ -424,3 +424,29 @@ def get_case(name: str) -> Case:
         if mk.case_name == name:
             return mk()
     raise KeyError(name)
+
+
+# ------------------------------------------------------------------ threefry2x32 as JAX lowers it without a custom call:
+# plain ui32 adds, xors and rotations (reference kernel text: src/pjrt_plugin/ops/control_flow.cc:1351-1390); the whole
+# block cipher fuses into one generated kernel.  Inputs are the Random123 known-answer vectors.
+def threefry2x32(b, k0, k1, c0, c1):
+    u = lambda x: b.constant(np.uint32(x), "ui32", k0.shape)
+    rotl = lambda x, r: b.or_(b.shift_left(x, u(r)), b.shift_right_logical(x, u(32 - r)))
+    ks = [k0, k1, b.xor(b.xor(k0, k1), u(0x1BD11BDA))]
+    x0, x1 = b.add(c0, ks[0]), b.add(c1, ks[1])
+    rots = [(13, 15, 26, 6), (17, 29, 16, 24)]
+    for blk in range(5):
+        for r in rots[blk % 2]:
+            x0 = b.add(x0, x1)
+            x1 = b.xor(x0, rotl(x1, r))
+        x0 = b.add(x0, ks[(blk + 1) % 3])
+        x1 = b.add(x1, b.add(ks[(blk + 2) % 3], u(blk + 1)))
+    return x0, x1
+
+
+THREEFRY_KAT = dict(
+    key0=np.array([0x00000000, 0xFFFFFFFF, 0x13198A2E], np.uint32), key1=np.array([0x00000000, 0xFFFFFFFF, 0x03707344], np.uint32),
+    ctr0=np.array([0x00000000, 0xFFFFFFFF, 0x243F6A88], np.uint32), ctr1=np.array([0x00000000, 0xFFFFFFFF, 0x85A308D3], np.uint32),
+    out0=np.array([0x6B200159, 0x1CB996FC, 0xC4923A9C], np.uint32), out1=np.array([0x99BA4EFE, 0xBB002BE7, 0x483DF7A0], np.uint32))
+case("threefry2x32-known-answers", threefry2x32, THREEFRY_KAT["key0"], THREEFRY_KAT["key1"], THREEFRY_KAT["ctr0"], THREEFRY_KAT["ctr1"], exact=True)
+case("threefry2x32-stream", threefry2x32, np.full(5000, 42, np.uint32), np.full(5000, 7, np.uint32), np.arange(5000, dtype=np.uint32), np.zeros(5000, np.uint32), exact=True)

@@ -303,3 +303,13 @@ def test_all_op_cases_run_on_the_oracle():
         ins = [round_bf16(a) if d == "bf16" else a for a, d in zip(c.inputs, c.dtypes)]
         out = Oracle(c.text).run(*ins)
         assert len(out) >= 1, c.name
+
+
+def test_threefry2x32_known_answer_vectors():
+    """Random123 KATs (the vectors JAX's own tests use): key (0,0) ctr (0,0) -> 6b200159 99ba4efe; all ones -> 1cb996fc bb002be7;
+    key (13198a2e, 03707344) ctr (243f6a88, 85a308d3) -> c4923a9c 483df7a0.  Pins ui32 add / xor / shifts of the oracle."""
+    import op_cases
+    c = op_cases.get_case("threefry2x32-known-answers")
+    out = Oracle(c.text).run(*c.inputs)
+    assert np.array_equal(out[0], op_cases.THREEFRY_KAT["out0"])
+    assert np.array_equal(out[1], op_cases.THREEFRY_KAT["out1"])
