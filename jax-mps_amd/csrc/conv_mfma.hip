@@ -428,7 +428,9 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
   // take a whole extra workgroup time).
   static const int target = getenv("MI355X_CONV_BLOCKS") ? atoi(getenv("MI355X_CONV_BLOCKS")) : 768;
   int split = 1;
-  if (tiles * 2 <= target) split = (int)std::min<long long>(target / tiles, std::max(1, c.kTiles / (tiles < 64 ? 4 : 8)));
+  static const int minSplitTiles = getenv("MI355X_CONV_MIN_SPLIT_KTILES") ? atoi(getenv("MI355X_CONV_MIN_SPLIT_KTILES")) : 1;
+  // (measured: splitting pays even for a short K, the shorter dependent chain per workgroup outweighs the fold launch)
+  if (tiles * 2 <= target && c.kTiles >= minSplitTiles) split = (int)std::min<long long>(target / tiles, std::max(1, c.kTiles / (tiles < 64 ? 4 : 8)));
   split = std::max(1, std::min(split, 256));
   c.tilesPerSplit = (c.kTiles + split - 1) / split;
   c.splitK = (c.kTiles + c.tilesPerSplit - 1) / c.tilesPerSplit;

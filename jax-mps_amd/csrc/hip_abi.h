@@ -53,6 +53,8 @@ int mi355_graph_destroy(mi355_graph_t exec);
 // runtime-compiled kernels: `source` defines extern "C" __global__ void k(...).
 // mi355_rtc_compile is thread-safe (no device state); the code object it returns is
 // malloc'ed and handed to mi355_module_load, which must run on the thread that owns the device.
+// identifies the compiler build and the options mi355_rtc_compile uses (part of the on-disk cache key)
+const char* mi355_rtc_fingerprint(void);
 int mi355_rtc_compile(const char* source, const char* arch, char** code, size_t* code_size, char* log, size_t log_len);
 int mi355_module_load(const char* code, mi355_function_t* fn);
 int mi355_launch(mi355_function_t fn, const unsigned grid[3], const unsigned block[3], void** arg_ptrs, int num_args,

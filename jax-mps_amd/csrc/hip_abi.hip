@@ -146,6 +146,16 @@ int mi355_event_elapsed_ms(mi355_event_t a, mi355_event_t b, float* ms) {
   return 0;
 }
 
+const char* mi355_rtc_fingerprint(void) {
+  static char buf[96];
+  if (!buf[0]) {
+    int major = 0, minor = 0;
+    if (hiprtcVersion(&major, &minor) != HIPRTC_SUCCESS) major = minor = -1;
+    snprintf(buf, sizeof buf, "hiprtc-%d.%d -O3 -ffp-contract=off -packed-fp32-ops", major, minor);
+  }
+  return buf;
+}
+
 int mi355_rtc_compile(const char* source, const char* arch, char** code, size_t* code_size, char* log, size_t log_len) {
   hiprtcProgram prog;
   if (log && log_len) log[0] = 0;

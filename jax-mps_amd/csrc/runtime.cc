@@ -55,8 +55,9 @@ std::string cachePath(const std::string& source, const std::string& arch) {
   std::string d = cacheDir();
   if (d.empty()) return "";
   char name[80];
-  snprintf(name, sizeof name, "/%016llx%016llx.hsaco", (unsigned long long)fnv1a(source + arch, 14695981039346656037ull),
-           (unsigned long long)fnv1a(arch + source, 0x9E3779B97F4A7C15ull));
+  const std::string target = arch + "|" + mi355_rtc_fingerprint();   // a code object is only valid for the compiler that made it
+  snprintf(name, sizeof name, "/%016llx%016llx.hsaco", (unsigned long long)fnv1a(source + target, 14695981039346656037ull),
+           (unsigned long long)fnv1a(target + source, 0x9E3779B97F4A7C15ull));
   return d + name;
 }
 
