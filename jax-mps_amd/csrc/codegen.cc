@@ -208,6 +208,26 @@ class Emitter {
   void body(const std::string& s) { body_.back() += std::string(2 + 2 * body_.size(), ' ') + s + "\n"; }
   void emit(bool inBody, const std::string& s) { (inBody || guard_ > 0) ? body(s) : pre(s); }
 
+  // Names declared inside the lane loop.  An expression that mentions one of them has to be emitted
+  // there too, whatever its index looks like (with one element per lane nothing is lane-dependent
+  // by index, yet guarded loads, concatenations and their consumers still live in the loop body).
+  std::unordered_set<std::string> bodyNames_;
+  bool mentionsBody(const std::string& e) const {
+    if (bodyNames_.empty()) return false;
+    size_t i = 0, n = e.size();
+    while (i < n) {
+      if (isalpha((unsigned char)e[i]) || e[i] == '_') {
+        size_t j = i;
+        while (j < n && (isalnum((unsigned char)e[j]) || e[j] == '_')) ++j;
+        if (bodyNames_.count(e.substr(i, j - i))) return true;
+        i = j;
+      } else {
+        ++i;
+      }
+    }
+    return false;
+  }
+
   // Row programs: results of reductions finished earlier in the same kernel, as variables that
   // hold the value for the row this wavefront / workgroup owns.
   std::unordered_map<Value*, std::string> rowScalars_;
@@ -235,11 +255,16 @@ class Emitter {
   IdxDim var(const std::string& expr, bool inBody, int64_t coef = 0, int64_t mult = 1) {
     IdxDim d;
     d.isConst = false;
-    d.inBody = inBody || guard_ > 0;
+    const bool forced = !inBody && mentionsBody(expr);
+    d.inBody = inBody || guard_ > 0 || forced;
     d.base = fresh("ix");
     d.coef = d.inBody ? 0 : coef;
     d.mult = mult;
-    emit(d.inBody, "const " + idxT() + " " + d.base + " = " + expr + ";");
+    // a lane-dependent value (expr + coef * v) that is forced into the lane loop by a guarded scope
+    // becomes a plain per-lane variable: its lane term has to be part of the expression
+    const std::string full = (!inBody && (guard_ > 0 || forced) && coef != 0) ? "(" + expr + " + " + std::to_string(coef) + " * v)" : expr;
+    emit(d.inBody, "const " + idxT() + " " + d.base + " = " + full + ";");
+    if (d.inBody) bodyNames_.insert(d.base);
     return d;
   }
 
@@ -250,6 +275,7 @@ class Emitter {
     r.isConst = false;
     r.inBody = true;
     r.base = fresh("ix");
+    bodyNames_.insert(r.base);
     body("const " + idxT() + " " + r.base + " = " + dimExpr(d) + ";");
     return r;
   }
@@ -319,7 +345,9 @@ class Emitter {
     int n = (int)shape.size();
     std::vector<int64_t> stride(n, 1);
     for (int d = n - 2; d >= 0; --d) stride[d] = stride[d + 1] * shape[d + 1];
-    bool anyBody = false, allConst = true;
+    // inside a guarded scope every new index variable lives in the lane loop, so the per-lane
+    // term of each component has to be spelled out
+    bool anyBody = guard_ > 0, allConst = true;
     int64_t cst = 0;
     for (int d = 0; d < n; ++d) {
       if (dims[d].isConst) cst += dims[d].cval * stride[d];
@@ -407,6 +435,7 @@ class Emitter {
       pre("const " + computeT(dt) + " " + t + " = " + loadExpr(dt, ptr + "[" + (off.isConst ? off.base : off.base) + "]") + ";");
       return t;
     }
+    bodyNames_.insert(t);
     body("const " + computeT(dt) + " " + t + " = " + loadExpr(dt, ptr + "[" + dimExpr(off) + "]") + ";");
     return t;
   }
@@ -440,7 +469,9 @@ class Emitter {
   std::string def(const TensorType& t, const std::string& expr, bool inBody, bool narrowing = true) {
     static const bool strict = getenv("MI355X_STRICT_BF16") && getenv("MI355X_STRICT_BF16")[0] == '1';
     std::string name = fresh("t");
-    emit(inBody, "const " + computeT(t.dt) + " " + name + " = " + ((strict || narrowing) ? roundTo(t.dt, expr) : expr) + ";");
+    const bool inB = inBody || guard_ > 0 || mentionsBody(expr);
+    if (inB) bodyNames_.insert(name);
+    emit(inB, "const " + computeT(t.dt) + " " + name + " = " + ((strict || narrowing) ? roundTo(t.dt, expr) : expr) + ";");
     return name;
   }
 
@@ -448,6 +479,7 @@ class Emitter {
   template <typename F>
   std::string guarded(const TensorType& t, const std::string& cond, F inner, const std::string& other) {
     std::string name = fresh("t");
+    bodyNames_.insert(name);
     body(computeT(t.dt) + " " + name + " = " + other + ";");
     body("if (" + cond + ") {");
     body_.emplace_back();
@@ -609,6 +641,7 @@ class Emitter {
       IdxDim pos = toBody(m.dims[dim]);
       std::string e = dimExpr(pos);
       std::string name = fresh("t");
+      bodyNames_.insert(name);
       body(computeT(rt.dt) + " " + name + ";");
       int64_t off = 0;
       for (size_t k = 0; k < op->operands.size(); ++k) {

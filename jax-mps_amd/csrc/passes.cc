@@ -509,6 +509,286 @@ void lowerScattersIn(Region& r, int& nextId) {
 
 }  // namespace
 
+// ---- reduce_window / select_and_scatter (pooling) ----------------------------------------------
+// A window reduction with a small window is the combination of one strided slice of the padded
+// operand per window tap; the rewrite emits exactly that (pad, k slices, k-1 combiner ops) and
+// the fusion planner turns it back into a single kernel whose index arithmetic walks the
+// window.  select_and_scatter (the gradient of max pooling) becomes: find the selected tap of
+// every window with a running compare over the same slices (first occurrence wins, as the
+// sequential definition does), then add, per tap, the source values whose window selected
+// that tap, dilated by the stride and shifted into operand coordinates with a pad.
+// (reference: ops/reduction.cc:165-626 pooling tier.)
+namespace {
+
+std::vector<int64_t> denseInts(const Attr& a, size_t n) {
+  std::vector<int64_t> out(n, 0);
+  if (a.kind == Attr::Ints) { for (size_t i = 0; i < n && i < a.ints.size(); ++i) out[i] = a.ints[i]; return out; }
+  if (a.kind != Attr::Dense || !a.dense) return out;
+  const DenseData& d = *a.dense;
+  size_t esz = dtypeSize(d.type.dt);
+  for (size_t i = 0; i < n; ++i) {
+    const uint8_t* p = d.bytes.data() + (d.splat ? 0 : i * esz);
+    if ((d.splat ? esz : (i + 1) * esz) > d.bytes.size()) break;
+    int64_t v = 0;
+    if (esz == 8) memcpy(&v, p, 8);
+    else if (esz == 4) { int32_t t; memcpy(&t, p, 4); v = t; }
+    else if (esz == 1) v = (int8_t)p[0];
+    out[i] = v;
+  }
+  return out;
+}
+
+// name of the single binary op a two-argument region applies to its arguments, or ""
+std::string regionBinaryOp(const Region& r) {
+  if (r.args.size() != 2 || r.ops.size() != 2) return "";
+  Op* b = r.ops[0].get();
+  Op* ret = r.ops[1].get();
+  if (ret->name != "return" || ret->operands.size() != 1 || ret->operands[0] != b->result() || b->operands.size() != 2) return "";
+  bool uses = (b->operands[0] == r.args[0].get() && b->operands[1] == r.args[1].get()) ||
+              (b->operands[0] == r.args[1].get() && b->operands[1] == r.args[0].get());
+  return uses ? b->name : "";
+}
+
+struct WindowSpec {
+  int rank = 0;
+  std::vector<int64_t> size, stride, baseDil, winDil, padLo, padHi;
+  int64_t taps = 1;
+};
+
+WindowSpec windowSpec(const Op& op, int rank) {
+  WindowSpec w;
+  w.rank = rank;
+  auto get = [&](const char* name, int64_t dflt) {
+    std::vector<int64_t> v(rank, dflt);
+    auto it = op.attrs.find(name);
+    if (it != op.attrs.end()) { auto x = denseInts(it->second, rank); if (!it->second.ints.empty() || it->second.kind == Attr::Dense) v = x; }
+    return v;
+  };
+  w.size = get("window_dimensions", 1);
+  w.stride = get("window_strides", 1);
+  w.baseDil = get("base_dilations", 1);
+  w.winDil = get("window_dilations", 1);
+  w.padLo.assign(rank, 0);
+  w.padHi.assign(rank, 0);
+  auto it = op.attrs.find("padding");
+  if (it != op.attrs.end()) {
+    auto p = denseInts(it->second, 2 * (size_t)rank);
+    for (int d = 0; d < rank; ++d) { w.padLo[d] = p[2 * d]; w.padHi[d] = p[2 * d + 1]; }
+  }
+  for (auto k : w.size) w.taps *= k;
+  return w;
+}
+
+struct Rewriter {
+  Region& r;
+  int& nextId;
+  int line;
+  std::vector<std::unique_ptr<Op>> made;
+  Value* emit(std::unique_ptr<Op> o, const TensorType& t) { Value* v = addResult(o.get(), t, nextId); made.push_back(std::move(o)); return v; }
+  Value* unary(const char* name, Value* a, const TensorType& t) { return emit(makeOp(name, {a}, &r, line), t); }
+  Value* binary(const std::string& name, Value* a, Value* b, const TensorType& t) { return emit(makeOp(name, {a, b}, &r, line), t); }
+  Value* broadcastScalar(Value* s, const TensorType& t) {
+    auto o = makeOp("broadcast_in_dim", {s}, &r, line);
+    o->attrs["dims"] = intsAttr({});
+    return emit(std::move(o), t);
+  }
+  Value* pad(Value* x, Value* padValue, const std::vector<int64_t>& lo, const std::vector<int64_t>& hi, const std::vector<int64_t>& interior) {
+    bool trivial = true;
+    TensorType t = x->type;
+    for (int d = 0; d < t.rank(); ++d) {
+      if (lo[d] || hi[d] || interior[d]) trivial = false;
+      t.dims[d] = std::max<int64_t>(0, (x->type.dims[d] > 0 ? (x->type.dims[d] - 1) * (interior[d] + 1) + 1 : 0) + lo[d] + hi[d]);
+    }
+    if (trivial) return x;
+    auto o = makeOp("pad", {x, padValue}, &r, line);
+    o->attrs["low"] = intsAttr(lo);
+    o->attrs["high"] = intsAttr(hi);
+    o->attrs["interior"] = intsAttr(interior);
+    return emit(std::move(o), t);
+  }
+  Value* slice(Value* x, const std::vector<int64_t>& start, const std::vector<int64_t>& count, const std::vector<int64_t>& stride) {
+    TensorType t = x->type;
+    std::vector<int64_t> limit(start.size());
+    bool whole = true;
+    for (size_t d = 0; d < start.size(); ++d) {
+      t.dims[d] = count[d];
+      limit[d] = start[d] + (count[d] > 0 ? (count[d] - 1) * stride[d] + 1 : 0);
+      if (start[d] != 0 || stride[d] != 1 || count[d] != x->type.dims[d]) whole = false;
+    }
+    if (whole) return x;
+    auto o = makeOp("slice", {x}, &r, line);
+    o->attrs["start"] = intsAttr(start);
+    o->attrs["limit"] = intsAttr(limit);
+    o->attrs["strides"] = intsAttr(stride);
+    return emit(std::move(o), t);
+  }
+  Value* splat(DType dt, const std::vector<int64_t>& dims, const void* bytes) {
+    auto c = makeOp("constant", {}, &r, line);
+    Attr dv;
+    dv.kind = Attr::Dense;
+    dv.dense = std::make_shared<DenseData>();
+    dv.dense->type.dt = dt;
+    dv.dense->type.dims = dims;
+    dv.dense->splat = true;
+    dv.dense->bytes.assign((const uint8_t*)bytes, (const uint8_t*)bytes + dtypeSize(dt));
+    c->attrs["value"] = dv;
+    TensorType t;
+    t.dt = dt;
+    t.dims = dims;
+    return emit(std::move(c), t);
+  }
+  // replaces op k of the region by the ops made so far; `last` takes over the results of the replaced op
+  void finish(size_t& k, Op* replaced, std::unique_ptr<Op> last) {
+    last->results = std::move(replaced->results);
+    for (auto& v : last->results) v->def = last.get();
+    made.push_back(std::move(last));
+    size_t nIns = made.size();
+    r.ops.erase(r.ops.begin() + k);
+    r.ops.insert(r.ops.begin() + k, std::make_move_iterator(made.begin()), std::make_move_iterator(made.end()));
+    k += nIns - 1;
+    made.clear();
+  }
+};
+
+constexpr int64_t kMaxWindowTaps = 64;
+
+// the slices of the padded operand, one per window tap in row-major tap order
+std::vector<Value*> tapSlices(Rewriter& rw, Value* padded, const WindowSpec& w, const std::vector<int64_t>& outDims) {
+  std::vector<Value*> taps;
+  std::vector<int64_t> t(w.rank, 0);
+  for (int64_t n = 0; n < w.taps; ++n) {
+    std::vector<int64_t> start(w.rank);
+    for (int d = 0; d < w.rank; ++d) start[d] = t[d] * w.winDil[d];
+    taps.push_back(rw.slice(padded, start, outDims, w.stride));
+    for (int d = w.rank - 1; d >= 0; --d) { if (++t[d] < w.size[d]) break; t[d] = 0; }
+  }
+  return taps;
+}
+
+void lowerWindowOpsIn(Region& r, int& nextId) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) lowerWindowOpsIn(*sub, nextId);
+    if (op->name == "reduce_window") {
+      if (op->operands.size() != 2 || op->regions.size() != 1) throw CompileError("stablehlo.reduce_window with several inputs is not supported");
+      Value* x = op->operands[0];
+      Value* init = op->operands[1];
+      const TensorType rt = op->result()->type;
+      std::string comb = regionBinaryOp(*op->regions[0]);
+      static const std::set<std::string> ok = {"add", "multiply", "maximum", "minimum", "and", "or", "xor"};
+      if (!ok.count(comb)) throw CompileError("stablehlo.reduce_window: the reducer must be a single add / multiply / maximum / minimum / and / or / xor");
+      WindowSpec w = windowSpec(*op, x->type.rank());
+      if (w.taps > kMaxWindowTaps) throw CompileError("stablehlo.reduce_window: windows of more than 64 elements (cumulative sums and the like) are not supported");
+      Rewriter rw{r, nextId, op->line, {}};
+      std::vector<int64_t> interior(w.rank);
+      for (int d = 0; d < w.rank; ++d) interior[d] = w.baseDil[d] - 1;
+      Value* padded = rw.pad(x, init, w.padLo, w.padHi, interior);
+      auto taps = tapSlices(rw, padded, w, rt.dims);
+      Value* acc = rw.broadcastScalar(init, rt);
+      for (size_t t = 0; t + 1 < taps.size() + 1 && t < taps.size(); ++t) {
+        if (t + 1 == taps.size()) break;
+        acc = rw.binary(comb, acc, taps[t], rt);
+      }
+      auto last = makeOp(comb, {acc, taps.back()}, &r, op->line);
+      rw.finish(k, op, std::move(last));
+      continue;
+    }
+    if (op->name == "select_and_scatter") {
+      if (op->operands.size() != 3 || op->regions.size() != 2) throw CompileError("stablehlo.select_and_scatter: malformed");
+      Value* x = op->operands[0];
+      Value* src = op->operands[1];
+      Value* init = op->operands[2];
+      const TensorType rt = op->result()->type;
+      if (!isFloat(x->type.dt)) throw CompileError("stablehlo.select_and_scatter: only floating-point operands are supported");
+      // select region: one compare of its two arguments
+      Region& sel = *op->regions[0];
+      std::string dir;
+      if (sel.args.size() == 2 && sel.ops.size() == 2 && sel.ops[0]->name == "compare" && sel.ops[0]->operands.size() == 2 &&
+          sel.ops[0]->operands[0] == sel.args[0].get() && sel.ops[0]->operands[1] == sel.args[1].get() && sel.ops[1]->name == "return" &&
+          sel.ops[1]->operands.size() == 1 && sel.ops[1]->operands[0] == sel.ops[0]->result())
+        dir = sel.ops[0]->str("direction");
+      if (dir != "GE" && dir != "GT" && dir != "LE" && dir != "LT") throw CompileError("stablehlo.select_and_scatter: the select region must be one GE / GT / LE / LT compare");
+      if (regionBinaryOp(*op->regions[1]) != "add") throw CompileError("stablehlo.select_and_scatter: the scatter region must be an add");
+      WindowSpec w = windowSpec(*op, x->type.rank());
+      if (w.taps > kMaxWindowTaps) throw CompileError("stablehlo.select_and_scatter: windows of more than 64 elements are not supported");
+      for (int d = 0; d < w.rank; ++d) if (w.baseDil[d] != 1 || w.winDil[d] != 1) throw CompileError("stablehlo.select_and_scatter: dilations are not supported");
+      Rewriter rw{r, nextId, op->line, {}};
+      // padding never wins the selection
+      const bool wantsLarge = dir == "GE" || dir == "GT";
+      float losingF = wantsLarge ? -__builtin_inff() : __builtin_inff();
+      uint16_t losingBf = wantsLarge ? 0xFF80 : 0x7F80;
+      uint16_t losingH = wantsLarge ? 0xFC00 : 0x7C00;
+      double losingD = wantsLarge ? -__builtin_inf() : __builtin_inf();
+      const void* lp = x->type.dt == DType::F32 ? (const void*)&losingF : x->type.dt == DType::BF16 ? (const void*)&losingBf
+                       : x->type.dt == DType::F16 ? (const void*)&losingH : (const void*)&losingD;
+      Value* losing = rw.splat(x->type.dt, {}, lp);
+      std::vector<int64_t> zeros(w.rank, 0);
+      Value* padded = rw.pad(x, losing, w.padLo, w.padHi, zeros);
+      auto taps = tapSlices(rw, padded, w, src->type.dims);
+      // running selection over the taps: select(best, candidate) false -> the candidate takes over
+      TensorType idxT = src->type;
+      idxT.dt = DType::S32;
+      TensorType predT = src->type;
+      predT.dt = DType::Pred;
+      int32_t zero32 = 0;
+      Value* bestVal = taps[0];
+      Value* bestIdx = rw.splat(DType::S32, src->type.dims, &zero32);
+      for (size_t t = 1; t < taps.size(); ++t) {
+        auto cmp = makeOp("compare", {bestVal, taps[t]}, &r, op->line);
+        Attr d;
+        d.kind = Attr::Str;
+        d.s = dir;
+        cmp->attrs["direction"] = d;
+        Value* keep = rw.emit(std::move(cmp), predT);
+        int32_t ti = (int32_t)t;
+        Value* tv = rw.splat(DType::S32, src->type.dims, &ti);
+        bestVal = rw.emit(makeOp("select", {keep, bestVal, taps[t]}, &r, op->line), src->type.dt == x->type.dt ? taps[t]->type : taps[t]->type);
+        bestIdx = rw.emit(makeOp("select", {keep, bestIdx, tv}, &r, op->line), idxT);
+      }
+      // per tap: the sources whose window selected it, moved to operand coordinates
+      uint64_t zeroBits = 0;
+      Value* zeroScalar = rw.splat(src->type.dt, {}, &zeroBits);
+      Value* zeroSrc = rw.splat(src->type.dt, src->type.dims, &zeroBits);
+      Value* acc = rw.broadcastScalar(init, rt);
+      std::vector<int64_t> t(w.rank, 0), interior(w.rank);
+      for (int d = 0; d < w.rank; ++d) interior[d] = w.stride[d] - 1;
+      std::unique_ptr<Op> lastOp;
+      for (int64_t n = 0; n < w.taps; ++n) {
+        int32_t ti = (int32_t)n;
+        Value* tv = rw.splat(DType::S32, src->type.dims, &ti);
+        auto eq = makeOp("compare", {bestIdx, tv}, &r, op->line);
+        Attr d;
+        d.kind = Attr::Str;
+        d.s = "EQ";
+        eq->attrs["direction"] = d;
+        Value* hit = rw.emit(std::move(eq), predT);
+        Value* contrib = rw.emit(makeOp("select", {hit, src, zeroSrc}, &r, op->line), src->type);
+        std::vector<int64_t> lo(w.rank), hi(w.rank);
+        for (int dd = 0; dd < w.rank; ++dd) {
+          lo[dd] = t[dd] - w.padLo[dd];
+          int64_t span = src->type.dims[dd] > 0 ? (src->type.dims[dd] - 1) * w.stride[dd] + 1 : 0;
+          hi[dd] = rt.dims[dd] - span - lo[dd];
+        }
+        Value* placed = rw.pad(contrib, zeroScalar, lo, hi, interior);
+        if (n + 1 < w.taps) acc = rw.binary("add", acc, placed, rt);
+        else lastOp = makeOp("add", {acc, placed}, &r, op->line);
+        for (int dd = w.rank - 1; dd >= 0; --dd) { if (++t[dd] < w.size[dd]) break; t[dd] = 0; }
+      }
+      rw.finish(k, op, std::move(lastOp));
+      continue;
+    }
+  }
+}
+
+}  // namespace
+
+void lowerWindowOps(Module& m) {
+  Func* f = m.main();
+  if (!f) return;
+  int nextId = maxValueId(f->body) + 1;
+  lowerWindowOpsIn(f->body, nextId);
+}
+
 void lowerGeneralScatters(Module& m) {
   Func* f = m.main();
   if (!f) return;
@@ -562,7 +842,7 @@ static const std::set<std::string>& supportedOps() {
       "constant", "iota", "reshape", "broadcast_in_dim", "transpose", "reverse", "concatenate", "slice", "dynamic_slice",
       "dynamic_update_slice", "pad",
       // heavy ops
-      "reduce", "dot_general", "dot", "convolution", "gather", "scatter",
+      "reduce", "dot_general", "dot", "convolution", "gather", "scatter", "reduce_window", "select_and_scatter",
       // control flow (ops/control_flow.cc:2364-2376)
       "while", "case", "return", "optimization_barrier", "custom_call",
   };

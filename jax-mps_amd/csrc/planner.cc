@@ -1239,6 +1239,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   inlineCalls(*module);
   lowerIntegerDots(*module);
   lowerGeneralScatters(*module);
+  lowerWindowOps(*module);
   checkSupported(*module);
   eliminateDeadCode(module->main()->body);
   prog->module = std::move(module);

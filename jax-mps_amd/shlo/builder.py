@@ -746,6 +746,69 @@ class Builder:
         self._emit(f"}}) : ({operand.type}, {indices.type}, {updates.type}) -> {v.type}")
         return v
 
+    def _window_attr_text(self, window, strides, padding, base_dilation=None, window_dilation=None):
+        rank = len(window)
+        f = lambda t: ", ".join(map(str, t))
+        arr = lambda t: f"array<i64: {f(t)}>" if len(t) else "array<i64>"
+        pad = [[int(a), int(b)] for a, b in padding]
+        attrs = []
+        if base_dilation is not None:
+            attrs.append(f"base_dilations = {arr(base_dilation)}")
+        if any(a or b for a, b in pad):
+            rows = ", ".join("[" + f(p) + "]" for p in pad)
+            attrs.append(f"padding = dense<[{rows}]> : tensor<{rank}x2xi64>")
+        if window_dilation is not None:
+            attrs.append(f"window_dilations = {arr(window_dilation)}")
+        attrs.append(f"window_dimensions = {arr(window)}")
+        attrs.append(f"window_strides = {arr(strides)}")
+        return ", ".join(attrs)
+
+    def reduce_window(self, x: Val, init, kind: str, window, strides=None, padding=None, base_dilation=None, window_dilation=None) -> Val:
+        """`lax.reduce_window` with an add / max / min / mul reducer, printed in the generic form JAX uses."""
+        rank = len(x.shape)
+        strides = list(strides) if strides is not None else [1] * rank
+        padding = [tuple(p) for p in padding] if padding is not None else [(0, 0)] * rank
+        bd = list(base_dilation) if base_dilation is not None else [1] * rank
+        wdl = list(window_dilation) if window_dilation is not None else [1] * rank
+        out = []
+        for d in range(rank):
+            dil = (x.shape[d] - 1) * bd[d] + 1 if x.shape[d] > 0 else 0
+            span = (window[d] - 1) * wdl[d] + 1
+            out.append(max(0, (dil + padding[d][0] + padding[d][1] - span) // strides[d] + 1))
+        iv = init if isinstance(init, Val) else self.constant(init, x.dtype)
+        v = self._new(out, x.dtype)
+        st = ttype((), x.dtype)
+        n0 = self._n
+        a0, a1, r = f"%warg{n0}_0", f"%warg{n0}_1", f"%wres{n0}"
+        ind = "  " * self._blk.indent
+        opn = {"add": "add", "max": "maximum", "min": "minimum", "mul": "multiply"}[kind]
+        self._emit(f'{v.name} = "stablehlo.reduce_window"({x.name}, {iv.name}) <{{{self._window_attr_text(window, strides, padding, base_dilation, window_dilation)}}}> ({{')
+        self._blk.lines.append(f"{ind}^bb0({a0}: {st}, {a1}: {st}):")
+        self._blk.lines.append(f"{ind}  {r} = stablehlo.{opn} {a0}, {a1} : {st}")
+        self._blk.lines.append(f"{ind}  stablehlo.return {r} : {st}")
+        self._emit(f"}}) : ({x.type}, {st}) -> {v.type}")
+        return v
+
+    def select_and_scatter(self, operand: Val, source: Val, init, window, strides, padding=None, direction="GE") -> Val:
+        """The op JAX emits for the gradient of max (GE) / min (LE) pooling."""
+        rank = len(operand.shape)
+        padding = [tuple(p) for p in padding] if padding is not None else [(0, 0)] * rank
+        iv = init if isinstance(init, Val) else self.constant(init, operand.dtype)
+        v = self._new(operand.shape, operand.dtype)
+        st = ttype((), operand.dtype)
+        n0 = self._n
+        ind = "  " * self._blk.indent
+        self._emit(f'{v.name} = "stablehlo.select_and_scatter"({operand.name}, {source.name}, {iv.name}) <{{{self._window_attr_text(window, strides, padding)}}}> ({{')
+        self._blk.lines.append(f"{ind}^bb0(%ssa{n0}: {st}, %ssb{n0}: {st}):")
+        self._blk.lines.append(f"{ind}  %ssc{n0} = stablehlo.compare  {direction}, %ssa{n0}, %ssb{n0},  FLOAT : ({st}, {st}) -> tensor<i1>")
+        self._blk.lines.append(f"{ind}  stablehlo.return %ssc{n0} : tensor<i1>")
+        self._blk.lines.append(f"{ind}}}, {{")
+        self._blk.lines.append(f"{ind}^bb0(%ssd{n0}: {st}, %sse{n0}: {st}):")
+        self._blk.lines.append(f"{ind}  %ssf{n0} = stablehlo.add %ssd{n0}, %sse{n0} : {st}")
+        self._blk.lines.append(f"{ind}  stablehlo.return %ssf{n0} : {st}")
+        self._emit(f"}}) : ({operand.type}, {source.type}, {st}) -> {v.type}")
+        return v
+
     def take_rows(self, table: Val, idx: Val) -> Val:
         """`jnp.take(table, idx, axis=0)` in the default (fill) mode: negative
         indices wrap, then rows outside [0, n) read as NaN (the mask JAX adds

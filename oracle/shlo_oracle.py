@@ -1243,6 +1243,71 @@ class Oracle:
         return out
 
     # ------------------------------------------------------------------
+    # window reductions (reference: ops/reduction.cc:165-626)
+    # ------------------------------------------------------------------
+    @staticmethod
+    def _window_attrs(op, rank):
+        def ints(name, dflt):
+            v = op.attrs.get(name)
+            if v is None:
+                return [dflt] * rank
+            v = np.asarray(v).reshape(-1)
+            return [int(x) for x in (v if v.size == rank else np.full(rank, v[0] if v.size else dflt))]
+        pad = op.attrs.get("padding")
+        if isinstance(pad, tuple):      # dense literal: (values, type)
+            pad = pad[0]
+        if pad is None:
+            pad = np.zeros((rank, 2), np.int64)
+        pad = np.asarray(pad)
+        pad = np.broadcast_to(pad.reshape(-1, 2) if pad.size == 2 * rank else np.full((rank, 2), int(pad.reshape(-1)[0]) if pad.size else 0), (rank, 2))
+        return ints("window_dimensions", 1), ints("window_strides", 1), ints("base_dilations", 1), ints("window_dilations", 1), pad.astype(np.int64)
+
+    def op_reduce_window(self, op, ins, env):
+        """Every output element is the reducer folded, in row-major window order and starting from the
+        init value, over its window of the operand padded (and base-dilated) with the init value.
+        Evaluated one output element at a time with the reducer region itself."""
+        x, init = ins
+        rank = x.ndim
+        wd, ws, bd, wdil, pad = self._window_attrs(op, rank)
+        body = op.regions[0]
+        dil = [d + max(d - 1, 0) * (b - 1) for d, b in zip(x.shape, bd)]
+        P = np.full([dil[d] + int(pad[d, 0]) + int(pad[d, 1]) for d in range(rank)], init, dtype=x.dtype)
+        valid = np.zeros(P.shape, dtype=bool)
+        P[tuple(slice(int(pad[d, 0]), int(pad[d, 0]) + dil[d], bd[d]) for d in range(rank))] = x
+        out_shape = op.out_types[0].shape
+        out = np.empty(out_shape, dtype=x.dtype)
+        import itertools
+        for o in itertools.product(*[range(n) for n in out_shape]):
+            acc = np.asarray(init)
+            for t in itertools.product(*[range(k) for k in wd]):
+                pos = tuple(o[d] * ws[d] + t[d] * wdil[d] for d in range(rank))
+                acc = np.asarray(self._run_region(body, [acc, np.asarray(P[pos])], env)[0])
+            out[o] = acc
+        return out
+
+    def op_select_and_scatter(self, op, ins, env):
+        """For every window of the operand (row-major), the select region picks one element by a running
+        comparison over the in-bounds window elements; the scatter region adds the window's source value
+        to that element of the result, which starts as the init value."""
+        x, src, init = ins
+        rank = x.ndim
+        wd, ws, _, _, pad = self._window_attrs(op, rank)
+        select, scatter = op.regions
+        out = np.full(x.shape, init, dtype=x.dtype)
+        import itertools
+        for w in itertools.product(*[range(n) for n in src.shape]):
+            best = None
+            for t in itertools.product(*[range(k) for k in wd]):
+                pos = tuple(w[d] * ws[d] - int(pad[d, 0]) + t[d] for d in range(rank))
+                if any(p < 0 or p >= x.shape[d] for d, p in enumerate(pos)):
+                    continue
+                if best is None or not bool(np.asarray(self._run_region(select, [np.asarray(x[best]), np.asarray(x[pos])], env)[0])):
+                    best = pos
+            if best is not None:
+                out[best] = np.asarray(self._run_region(scatter, [np.asarray(out[best]), np.asarray(src[w])], env)[0])
+        return out
+
+    # ------------------------------------------------------------------
     # reductions (reference: ops/reduction.cc:83-162)
     # ------------------------------------------------------------------
     def op_reduce(self, op, ins, env):

@@ -131,6 +131,22 @@ add("dot_int32", lambda b, x, y: b.dot_general(x, y, ([0], [0])), [np.array([1, 
 add("matmul_int32", lambda b, x, y: b.matmul(x, y), [np.array([[1, 2], [3, 4]], np.int32), np.array([[5, 6], [7, 8]], np.int32)], np.array([[19, 22], [43, 50]], np.int32), "tests/configs/matmul.py:229-235")
 add("dot_bool", lambda b, x, y: b.dot_general(x, y, ([0], [0])), [np.array([True, False, True]), np.array([True, True, False])], np.array(True), "tests/configs/matmul.py:236-242")
 add("matmul_uint32", lambda b, x, y: b.matmul(x, y), [np.array([[1, 2], [3, 4]], np.uint32), np.array([[5, 6], [7, 8]], np.uint32)], np.array([[19, 22], [43, 50]], np.uint32), "tests/configs/matmul.py:243-249")
+# pooling with tied values (reduction.py:296-342: "maxpool2d-tied-grad", "maxpool2d-overlapping-tied-grad", "maxpool1d-tied-grad")
+tied = np.array([[[[0.0], [0.0], [1.0], [0.0]], [[0.0], [0.0], [0.0], [0.0]], [[2.0], [0.0], [0.0], [0.0]], [[0.0], [0.0], [0.0], [3.0]]]], np.float32)
+add("maxpool2d_tied", lambda b, x: b.reduce_window(x, float("-inf"), "max", (1, 2, 2, 1), (1, 2, 2, 1)), [tied],
+    np.array([[[[0.0], [1.0]], [[2.0], [3.0]]]], np.float32), "tests/configs/reduction.py:296-313")
+# gradient of the same pooling for an all-ones cotangent: each window's first maximum receives it
+tied_grad = np.zeros((1, 4, 4, 1), np.float32)
+for pos in [(0, 0), (0, 2), (2, 0), (3, 3)]:
+    tied_grad[0, pos[0], pos[1], 0] = 1.0
+add("maxpool2d_tied_grad", lambda b, x, g: b.select_and_scatter(x, g, 0.0, (1, 2, 2, 1), (1, 2, 2, 1)), [tied, np.ones((1, 2, 2, 1), np.float32)],
+    tied_grad, "tests/configs/reduction.py:296-313")
+over = np.zeros((1, 5, 5, 1), np.float32)
+over[0, 1, 1, 0] = over[0, 1, 2, 0] = over[0, 2, 1, 0] = 5.0
+add("maxpool2d_overlapping_tied", lambda b, x: b.reduce_window(x, float("-inf"), "max", (1, 3, 3, 1), (1, 1, 1, 1)), [over],
+    np.array([[5, 5, 5], [5, 5, 5], [5, 5, 0]], np.float32).reshape(1, 3, 3, 1), "tests/configs/reduction.py:315-332")
+add("maxpool1d_tied", lambda b, x: b.reduce_window(x, float("-inf"), "max", (1, 2), (1, 2)), [np.array([[0, 0, 1, 1, 0, 0, 2, 0]], np.float32)],
+    np.array([[0, 1, 0, 2]], np.float32), "tests/configs/reduction.py:334-342")
 add("pad_edge_and_interior", lambda b, x: b.pad(x, 0.0, [1], [2], [1]), [np.array([1, 2, 3], np.float32)], np.array([0, 1, 0, 2, 0, 3, 0, 0], np.float32), "src/pjrt_plugin/ops/slice.cc:202-276")
 add("pad_negative_crops", lambda b, x: b.pad(x, 9.0, [-1], [1], [0]), [np.array([1, 2, 3], np.float32)], np.array([2, 3, 9], np.float32), "src/pjrt_plugin/ops/slice.cc:202-276")
 

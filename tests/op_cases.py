@@ -450,3 +450,17 @@ THREEFRY_KAT = dict(
     out0=np.array([0x6B200159, 0x1CB996FC, 0xC4923A9C], np.uint32), out1=np.array([0x99BA4EFE, 0xBB002BE7, 0x483DF7A0], np.uint32))
 case("threefry2x32-known-answers", threefry2x32, THREEFRY_KAT["key0"], THREEFRY_KAT["key1"], THREEFRY_KAT["ctr0"], THREEFRY_KAT["ctr1"], exact=True)
 case("threefry2x32-stream", threefry2x32, np.full(5000, 42, np.uint32), np.full(5000, 7, np.uint32), np.arange(5000, dtype=np.uint32), np.zeros(5000, np.uint32), exact=True)
+
+
+# ------------------------------------------------------------------ pooling: reduce_window / select_and_scatter (tests/configs/reduction.py:87-342)
+NHWC_PAD1 = [(0, 0), (1, 1), (1, 1), (0, 0)]
+case("maxpool-3x3-s2-pad1", lambda b, x: b.reduce_window(x, float("-inf"), "max", (1, 3, 3, 1), (1, 2, 2, 1), NHWC_PAD1), f32(3000, 4, 17, 15, 24), exact=True)
+case("sumpool-2x2-s2", lambda b, x: b.reduce_window(x, 0.0, "add", (1, 2, 2, 1), (1, 2, 2, 1)), f32(3001, 2, 16, 16, 8))
+case("minpool-dilated-window", lambda b, x: b.reduce_window(x, float("inf"), "min", (1, 2, 3, 1), (1, 1, 2, 1), [(0, 0), (1, 0), (2, 1), (0, 0)], window_dilation=(1, 2, 2, 1)), f32(3002, 2, 9, 11, 3), exact=True)
+case("sumpool-base-dilation", lambda b, x: b.reduce_window(x, 0.0, "add", (2, 3), (1, 1), [(1, 1), (0, 2)], base_dilation=(2, 3)), f32(3003, 5, 6))
+case("reduce_window-scalar", lambda b, x: b.reduce_window(x, 0.0, "add", (), (), []), np.float32(2.5), exact=True)
+case("maxpool-bf16", lambda b, x: b.reduce_window(x, float("-inf"), "max", (1, 3, 3, 1), (1, 2, 2, 1), NHWC_PAD1), f32(3004, 2, 8, 8, 16), dtypes=["bf16"], exact=True)
+case("maxpool-grad-3x3-s2-pad1", lambda b, x, g: b.select_and_scatter(x, g, 0.0, (1, 3, 3, 1), (1, 2, 2, 1), NHWC_PAD1), f32(3005, 2, 9, 8, 6), f32(3006, 2, 5, 4, 6))
+case("maxpool-grad-ties", lambda b, x, g: b.select_and_scatter(x, g, 0.0, (1, 2, 2, 1), (1, 1, 1, 1)),
+     np.round(f32(3007, 1, 6, 6, 2) * 2).astype(np.float32), f32(3008, 1, 5, 5, 2))
+case("minpool-grad", lambda b, x, g: b.select_and_scatter(x, g, 0.0, (1, 2, 2, 1), (1, 2, 2, 1), direction="LE"), f32(3009, 2, 6, 6, 4), f32(3010, 2, 3, 3, 4))

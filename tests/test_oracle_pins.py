@@ -313,3 +313,29 @@ def test_threefry2x32_known_answer_vectors():
     out = Oracle(c.text).run(*c.inputs)
     assert np.array_equal(out[0], op_cases.THREEFRY_KAT["out0"])
     assert np.array_equal(out[1], op_cases.THREEFRY_KAT["out1"])
+
+
+def test_pooling_against_torch():
+    """reduce_window (max / sum) and select_and_scatter (gradient of max pooling, first maximum wins) against
+    torch.nn.functional.max_pool2d / avg_pool2d and torch autograd, NHWC <-> NCHW."""
+    import torch
+    from jax_mps_amd.shlo.builder import Builder
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((2, 9, 8, 3)).astype(np.float32)
+    pad = [(0, 0), (1, 1), (1, 1), (0, 0)]
+    b = Builder()
+    b.ret(b.reduce_window(b.arg(x.shape), float("-inf"), "max", (1, 3, 3, 1), (1, 2, 2, 1), pad))
+    t = torch.nn.functional.max_pool2d(torch.tensor(x).permute(0, 3, 1, 2), 3, 2, 1).permute(0, 2, 3, 1).numpy()
+    assert np.array_equal(Oracle(b.text()).run(x)[0], t)
+    b = Builder()
+    b.ret(b.reduce_window(b.arg(x.shape), 0.0, "add", (1, 2, 2, 1), (1, 2, 2, 1)))
+    t = 4 * torch.nn.functional.avg_pool2d(torch.tensor(x).permute(0, 3, 1, 2), 2, 2).permute(0, 2, 3, 1).numpy()
+    assert np.allclose(Oracle(b.text()).run(x)[0], t, rtol=1e-6, atol=1e-6)
+    xt = torch.tensor(x).permute(0, 3, 1, 2).clone().requires_grad_(True)
+    y = torch.nn.functional.max_pool2d(xt, 3, 2, 1)
+    g = torch.tensor(rng.standard_normal(tuple(y.shape)).astype(np.float32))
+    y.backward(g)
+    b = Builder()
+    b.ret(b.select_and_scatter(b.arg(x.shape), b.arg((2, 5, 4, 3)), 0.0, (1, 3, 3, 1), (1, 2, 2, 1), pad))
+    got = Oracle(b.text()).run(x, g.permute(0, 2, 3, 1).numpy().copy())[0]
+    assert np.allclose(got, xt.grad.permute(0, 2, 3, 1).numpy(), rtol=1e-6, atol=1e-6)
