@@ -678,8 +678,42 @@ void lowerWindowOpsIn(Region& r, int& nextId) {
       static const std::set<std::string> ok = {"add", "multiply", "maximum", "minimum", "and", "or", "xor"};
       if (!ok.count(comb)) throw CompileError("stablehlo.reduce_window: the reducer must be a single add / multiply / maximum / minimum / and / or / xor");
       WindowSpec w = windowSpec(*op, x->type.rank());
-      if (w.taps > kMaxWindowTaps) throw CompileError("stablehlo.reduce_window: windows of more than 64 elements (cumulative sums and the like) are not supported");
       Rewriter rw{r, nextId, op->line, {}};
+      if (w.taps > kMaxWindowTaps) {
+        // Cumulative pattern (cumsum / cumprod / cummax as JAX lowers them): the window spans one whole
+        // dim, padded by n-1 on one side.  Computed as a Hillis-Steele scan: log2(n) passes of
+        // "combine with a copy of yourself shifted by s", each pass kept in memory.
+        int axis = -1;
+        bool cumulative = true;
+        for (int d = 0; d < w.rank; ++d) {
+          if (w.stride[d] != 1 || w.baseDil[d] != 1 || w.winDil[d] != 1) cumulative = false;
+          if (w.size[d] == 1) { if (w.padLo[d] || w.padHi[d]) cumulative = false; continue; }
+          if (axis >= 0 || w.size[d] != x->type.dims[d]) cumulative = false;
+          axis = d;
+        }
+        const int64_t n = axis >= 0 ? x->type.dims[axis] : 0;
+        const bool forward = cumulative && axis >= 0 && w.padLo[axis] == n - 1 && w.padHi[axis] == 0;
+        const bool backward = cumulative && axis >= 0 && w.padLo[axis] == 0 && w.padHi[axis] == n - 1;
+        if (!forward && !backward)
+          throw CompileError("stablehlo.reduce_window: windows of more than 64 elements are supported only in the cumulative form (one whole dim, padded by n-1 on one side)");
+        Value* cur = x;
+        std::vector<int64_t> zeros(w.rank, 0);
+        for (int64_t sft = 1; sft < n; sft *= 2) {
+          std::vector<int64_t> lo = zeros, hi = zeros;
+          lo[axis] = forward ? sft : -sft;
+          hi[axis] = forward ? -sft : sft;
+          Value* shifted = rw.pad(cur, init, lo, hi, zeros);
+          auto step = makeOp(comb, {cur, shifted}, &r, op->line);
+          Attr flag;
+          flag.kind = Attr::Bool;
+          flag.b = true;
+          step->attrs["force_materialize"] = flag;   // each pass reads the previous one at two places: recomputing it would double the work per pass
+          cur = rw.emit(std::move(step), rt);
+        }
+        auto last = makeOp(comb, {rw.broadcastScalar(init, rt), cur}, &r, op->line);
+        rw.finish(k, op, std::move(last));
+        continue;
+      }
       std::vector<int64_t> interior(w.rank);
       for (int d = 0; d < w.rank; ++d) interior[d] = w.baseDil[d] - 1;
       Value* padded = rw.pad(x, init, w.padLo, w.padHi, interior);

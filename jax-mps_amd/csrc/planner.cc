@@ -192,7 +192,7 @@ class Planner {
         if (needMat_[ur]) addGroup(u);
         else for (Op* q : groups[ur]) addGroup(q);
       }
-      bool mat = forced;
+      bool mat = forced || op->has("force_materialize");
       if (op->name == "constant") {
         auto& d = *op->attrs.at("value").dense;
         if (!d.splat && d.type.numel() > 1) mat = true;
@@ -332,7 +332,11 @@ class Planner {
   bool leavesReady(Value* v, const std::vector<Value*>& roots, std::unordered_set<Value*>& seen, int& count) {
     for (auto* o : v->def->operands) {
       if (!seen.insert(o).second) continue;
-      if (std::find(roots.begin(), roots.end(), o) != roots.end()) continue;
+      if (std::find(roots.begin(), roots.end(), o) != roots.end()) {
+        // a value that must live in memory (it is read at shifted positions) cannot feed a kernel that also computes it
+        if (o->def && o->def->has("force_materialize")) return false;
+        continue;
+      }
       if (hasStorage(o)) { ++count; continue; }
       if (!o->def || !isFusibleOp(*o->def) || o->def->results.size() != 1 || needMat_[o]) return false;
       if (!leavesReady(o, roots, seen, count)) return false;

@@ -464,3 +464,9 @@ case("maxpool-grad-3x3-s2-pad1", lambda b, x, g: b.select_and_scatter(x, g, 0.0,
 case("maxpool-grad-ties", lambda b, x, g: b.select_and_scatter(x, g, 0.0, (1, 2, 2, 1), (1, 1, 1, 1)),
      np.round(f32(3007, 1, 6, 6, 2) * 2).astype(np.float32), f32(3008, 1, 5, 5, 2))
 case("minpool-grad", lambda b, x, g: b.select_and_scatter(x, g, 0.0, (1, 2, 2, 1), (1, 2, 2, 1), direction="LE"), f32(3009, 2, 6, 6, 4), f32(3010, 2, 3, 3, 4))
+
+# cumulative reductions as JAX lowers them: a reduce_window over one whole dim padded by n-1 (tests/configs/reduction.py:41-77)
+case("cumsum-axis1", lambda b, x: b.reduce_window(x, 0.0, "add", (1, 300), (1, 1), [(0, 0), (299, 0)]), f32(3020, 7, 300))
+case("cumsum-axis0-int", lambda b, x: b.reduce_window(x, 0, "add", (200, 1), (1, 1), [(199, 0), (0, 0)]), rng(3021).integers(-50, 50, size=(200, 9)).astype(np.int32), exact=True)
+case("cummax-reverse", lambda b, x: b.reduce_window(x, float("-inf"), "max", (1, 1, 130), (1, 1, 1), [(0, 0), (0, 0), (0, 129)]), f32(3022, 3, 4, 130), exact=True)
+case("cumprod-axis1", lambda b, x: b.reduce_window(x, 1.0, "mul", (1, 100), (1, 1), [(0, 0), (99, 0)]), f32(3023, 5, 100, lo=0.9, hi=1.1))
