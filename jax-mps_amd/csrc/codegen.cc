@@ -1762,5 +1762,57 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
   fc.launches.push_back(std::move(l));
   return fc;
 }
+// Horizontal batching: independent one-dimensional kernels become the segments of one
+// launch.  Every generated kernel is kPrelude + one header + body, and addresses its grid
+// through blockIdx.x only, so a segment is that body as a device function of the block index.
+bool batchableKernel(const std::string& source) {
+  const size_t pre = strlen(kPrelude);
+  if (source.compare(0, pre, kPrelude) != 0) return false;
+  if (source.find("blockIdx.y", pre) != std::string::npos || source.find("blockIdx.z", pre) != std::string::npos) return false;
+  if (source.find("gridDim", pre) != std::string::npos) return false;
+  return source.compare(pre, 10, "extern \"C\"") == 0;
+}
+
+std::string combineKernels(const std::vector<const std::string*>& sources, const std::vector<unsigned>& gridX) {
+  const size_t pre = strlen(kPrelude);
+  static const std::string head = "extern \"C\" __global__ void __launch_bounds__(256) k(";
+  std::ostringstream segs, params, dispatch;
+  size_t argNo = 0;
+  unsigned start = 0;
+  for (size_t k = 0; k < sources.size(); ++k) {
+    const std::string& src = *sources[k];
+    if (!batchableKernel(src) || src.compare(pre, head.size(), head) != 0) return "";
+    size_t p0 = pre + head.size();
+    size_t p1 = src.find(") {\n", p0);
+    size_t end = src.rfind('}');
+    if (p1 == std::string::npos || end == std::string::npos || end < p1) return "";
+    std::string plist = src.substr(p0, p1 - p0);
+    std::string body = src.substr(p1 + 4, end - (p1 + 4));
+    for (size_t at = body.find("blockIdx.x"); at != std::string::npos; at = body.find("blockIdx.x", at)) body.replace(at, 10, "seg_bx");
+    segs << "static __device__ __forceinline__ void seg" << k << "(const unsigned seg_bx" << (plist.empty() ? "" : ", ") << plist << ") {\n" << body << "}\n";
+    dispatch << "  if (b < " << (start + gridX[k]) << "u) { seg" << k << "(b - " << start << "u";
+    // each parameter is "<type> <name>"; the wrapper renames them a<N> and drops the no-alias promise,
+    // which holds inside one segment but not across segments that read the same buffer
+    size_t pos = 0;
+    while (pos < plist.size()) {
+      size_t comma = plist.find(", ", pos);
+      std::string one = plist.substr(pos, comma == std::string::npos ? std::string::npos : comma - pos);
+      pos = comma == std::string::npos ? plist.size() : comma + 2;
+      size_t sp = one.rfind(' ');
+      if (sp == std::string::npos) return "";
+      std::string type = one.substr(0, sp);
+      size_t r = type.find(" __restrict__");
+      if (r != std::string::npos) type.erase(r, 13);
+      params << (argNo ? ", " : "") << type << " a" << argNo;
+      dispatch << ", a" << argNo;
+      ++argNo;
+    }
+    dispatch << "); return; }\n";
+    start += gridX[k];
+  }
+  std::ostringstream s;
+  s << kPrelude << segs.str() << head << params.str() << ") {\n  const unsigned b = blockIdx.x;\n" << dispatch.str() << "}\n";
+  return s.str();
+}
 
 }  // namespace mi355

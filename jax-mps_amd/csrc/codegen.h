@@ -58,6 +58,12 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf);
 // tensor and stores into `dus` result storage (which already holds the operand).
 FusedCode generateDusKernel(Op* dus, const LeafPredicate& isLeaf);
 
+// Several independent kernels with one-dimensional grids as the segments of one launch: block b
+// runs the kernel whose block range holds b.  Arguments are the kernels' arguments, concatenated.
+// Returns "" when one of the sources cannot take part (batchableKernel is the cheap test).
+bool batchableKernel(const std::string& source);
+std::string combineKernels(const std::vector<const std::string*>& sources, const std::vector<unsigned>& gridX);
+
 // One or more stablehlo.reduce ops with identical input shape and dimensions.
 // Returns false in `ok` when a reducer body is not a single add/mul/max/min/and/or.
 // `epilogue`: values of the result shape computed from the results (and other inputs of that shape); they are

@@ -120,6 +120,64 @@ __global__ void __launch_bounds__(256) gemm_f32_mfma(GemmArgs g) {
   }
 }
 
+// fp32 GEMMs with few output elements (recurrent cells, classifier heads, per-step projections):
+// one workgroup per TxT output tile, the four waves split K between them and fold their partial
+// tiles through LDS, so the whole product is one short launch with no split-K workspace.  Operands
+// are read straight from memory in the MFMA operand layout (one element per lane per step).
+template <int T>
+__global__ void __launch_bounds__(256) gemm_f32_small(GemmArgs g) {
+  constexpr int KS = T == 16 ? 4 : 2;         // k values per MFMA
+  constexpr int NACC = T == 16 ? 4 : 16;
+  typedef float accv __attribute__((ext_vector_type(NACC)));
+  __shared__ float red[4][T * T];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const long long b0 = blockIdx.z / g.batch1, b1 = blockIdx.z % g.batch1;
+  const float* A = (const float*)g.a + b0 * g.aB0 + b1 * g.aB1;
+  const float* B = (const float*)g.b + b0 * g.bB0 + b1 * g.bB1;
+  const long long m0 = (long long)blockIdx.y * T, n0 = (long long)blockIdx.x * T;
+  const int r = lane % T, kl = lane / T;
+  const bool mOk = m0 + r < g.M, nOk = n0 + r < g.N;
+  const float* ap = A + (m0 + r) * g.aRow;
+  const float* bp = B + (n0 + r) * g.bCol;
+  const long long steps = (g.K + KS - 1) / KS, per = (steps + 3) / 4;
+  const long long s0 = w * per, s1 = s0 + per < steps ? s0 + per : steps;
+  accv acc = {0};
+  constexpr int U = 8;
+  long long s = s0;
+  for (; s + U <= s1; s += U) {
+    float av[U], bv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const long long k = (s + u) * KS + kl;
+      av[u] = (mOk && k < g.K) ? ap[k * g.aCol] : 0.f;
+      bv[u] = (nOk && k < g.K) ? bp[k * g.bRow] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if constexpr (T == 16) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u], acc, 0, 0, 0);
+      else acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u], bv[u], acc, 0, 0, 0);
+    }
+  }
+  for (; s < s1; ++s) {
+    const long long k = s * KS + kl;
+    const float a1 = (mOk && k < g.K) ? ap[k * g.aCol] : 0.f;
+    const float b1v = (nOk && k < g.K) ? bp[k * g.bRow] : 0.f;
+    if constexpr (T == 16) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1v, acc, 0, 0, 0);
+    else acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1v, acc, 0, 0, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < NACC; ++i) {
+    const int row = T == 16 ? kl * 4 + i : (i >> 2) * 8 + kl * 4 + (i & 3);
+    red[w][row * T + r] = acc[i];
+  }
+  __syncthreads();
+  float* C = (float*)g.c + (long long)blockIdx.z * g.M * g.N;
+  for (int e = threadIdx.x; e < T * T; e += 256) {
+    const long long row = m0 + e / T, col = n0 + e % T;
+    if (row < g.M && col < g.N) C[row * g.N + col] = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
+  }
+}
+
 __global__ void __launch_bounds__(256) gemm_bf16_mfma(GemmArgs g) {
   constexpr int BM = 64, BN = 64, BK = 32;
   __shared__ __attribute__((aligned(16))) u16 As[BM][BK + 8];
@@ -551,8 +609,26 @@ static bool gemmAsPointwiseConv(const mi355_gemm_desc* d, mi355_conv_desc* c) {
   return true;
 }
 
+// Tile edge of the small-product kernel for this GEMM, 0 when the product is big enough to want
+// the tiled kernels (enough output tiles to fill the chip, or a long K per tile).
+static int smallGemmTile(const mi355_gemm_desc* d) {
+  if (d->in_dtype != 0 || d->out_dtype != 0 || d->K <= 0) return 0;
+  static const int off = getenv("MI355X_SMALL_GEMM") ? atoi(getenv("MI355X_SMALL_GEMM")) == 0 : 0;
+  if (off) return 0;
+  const long long nb = d->batch0 * d->batch1;
+  if (nb > 65535) return 0;
+  const double flops = 2.0 * (double)nb * (double)d->M * (double)d->N * (double)d->K;
+  if (flops > 3.0e8) return 0;
+  const long long t16 = ((d->M + 15) / 16) * ((d->N + 15) / 16) * nb;
+  const long long t32 = ((d->M + 31) / 32) * ((d->N + 31) / 32) * nb;
+  if (t16 <= 1024) return 16;
+  if (t32 <= 2048) return 32;
+  return 0;
+}
+
 size_t mi355_gemm_workspace_bytes(const mi355_gemm_desc* d) {
   if (d->in_dtype == 1) return mi355_gemm_bf16_async_workspace_bytes(d);
+  if (smallGemmTile(d)) return 0;
   mi355_conv_desc cd;
   if (gemmAsPointwiseConv(d, &cd)) return mi355_conv_workspace_bytes(&cd);
   return 0;
@@ -574,6 +650,12 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
     if (r >= 0) return r;
     r = mi355_gemm_bf16_tiled(d, a, b, c, s);
     if (r >= 0) return r;
+  }
+  if (const int t = smallGemmTile(d)) {
+    dim3 grid((unsigned)((d->N + t - 1) / t), (unsigned)((d->M + t - 1) / t), (unsigned)nb);
+    if (t == 16) gemm_f32_small<16><<<grid, 256, 0, (hipStream_t)s>>>(g);
+    else gemm_f32_small<32><<<grid, 256, 0, (hipStream_t)s>>>(g);
+    return check("gemm");
   }
   mi355_conv_desc cd;
   if (gemmAsPointwiseConv(d, &cd)) return mi355_conv(&cd, a, b, c, workspace, workspace_bytes, s);

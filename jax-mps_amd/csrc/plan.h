@@ -70,6 +70,8 @@ struct Step {
   unsigned grid[3] = {1, 1, 1}, block[3] = {1, 1, 1};
   std::vector<BufRef> args;        // pointer arguments, in kernel order
   int64_t algoBytes = 0;           // distinct input bytes + output bytes (for bandwidth reports)
+  std::vector<uint8_t> argWrites;  // planning only: 1 where the kernel writes the argument's buffer
+  int time = 0;                    // planning only: position in the buffer-lifetime clock
 
   // Gemm / Conv / ScatterRows
   GemmDesc gemm;

@@ -89,6 +89,8 @@ class Planner {
         P.plan.steps.push_back(std::move(c));
       }
     }
+    static const bool batching = !getenv("MI355X_BATCH_KERNELS") || atoi(getenv("MI355X_BATCH_KERNELS")) != 0;
+    if (batching) batchKernels(P.plan);
     assignArena();
     patch(P.plan);
     P.numSteps = countSteps(P.plan);
@@ -202,7 +204,9 @@ class Planner {
         for (auto* l : leaves[v]) if (l->type.numel() * 4 >= v->type.numel()) ++big;
         bool expensive = isExpensive(op->name);
         for (auto* o : op->operands) if (o->def && !needMat_[o] && isExpensive(o->def->name) && o->def->parent == &r) expensive = true;
-        if (big >= 2 || expensive) mat = true;
+        // g consumers each re-reading `big` leaves move g*big tensors; materialising moves big + 1 + g and costs a launch
+        static const int limit = getenv("MI355X_RECOMPUTE_LIMIT") ? atoi(getenv("MI355X_RECOMPUTE_LIMIT")) : 1;
+        if ((big >= 2 && ((int)g.size() - 1) * (big - 1) > limit) || expensive) mat = true;
       }
       needMat_[v] = mat;
       if (mat) { g.clear(); g.push_back(op); }
@@ -255,7 +259,9 @@ class Planner {
         } else {
           s.args.push_back(ref(storageOf(a.value), t));
         }
+        s.argWrites.push_back(a.kind != KArg::In);
       }
+      s.time = t;
       s.algoBytes = bytes;
       bytes = 0;   // the traffic of a multi-launch reduction is counted once
       plan.steps.push_back(std::move(s));
@@ -1117,6 +1123,72 @@ class Planner {
     loops_.push_back({tStart, tEnd});
     for (size_t k = 0; k < op->results.size(); ++k) bind(op->results[k].get(), outs[k]);
     plan.steps.push_back(std::move(c));
+  }
+
+  // ---------------------------------------------------------------- horizontal batching
+  // Consecutive kernel steps that touch disjoint buffers (or only read the shared ones) run as
+  // the segments of one launch: small kernels cost a launch each whatever their size, and the
+  // optimiser updates of a training step or the bookkeeping of a loop body come in such runs.
+  static constexpr unsigned kBatchMaxBlocks = 4096;   // bigger kernels fill the chip on their own
+  static constexpr size_t kBatchMaxArgs = 192;
+  static constexpr size_t kBatchMaxSegments = 24;
+
+  bool batchCandidate(const Step& s) const {
+    return s.kind == Step::Kernel && s.grid[1] == 1 && s.grid[2] == 1 && s.block[0] == 256 && s.block[1] == 1 && s.block[2] == 1 &&
+           s.grid[0] <= kBatchMaxBlocks && s.argWrites.size() == s.args.size() && batchableKernel(P.kernels[s.kernel].source);
+  }
+
+  static bool independent(const Step& a, const Step& b) {
+    for (size_t i = 0; i < a.args.size(); ++i)
+      for (size_t j = 0; j < b.args.size(); ++j)
+        if (a.args[i].index == b.args[j].index && (a.argWrites[i] || b.argWrites[j])) return false;
+    return true;
+  }
+
+  void batchKernels(Plan& plan) {
+    std::vector<Step> out;
+    auto& steps = plan.steps;
+    size_t i = 0;
+    while (i < steps.size()) {
+      for (auto& b : steps[i].bodies) batchKernels(*b);
+      if (!batchCandidate(steps[i])) { out.push_back(std::move(steps[i++])); continue; }
+      size_t j = i + 1, nargs = steps[i].args.size();
+      while (j < steps.size() && j - i < kBatchMaxSegments && batchCandidate(steps[j]) && nargs + steps[j].args.size() <= kBatchMaxArgs) {
+        bool ok = true;
+        for (size_t k = i; k < j && ok; ++k) ok = independent(steps[k], steps[j]);
+        if (!ok) break;
+        nargs += steps[j].args.size();
+        ++j;
+      }
+      if (j - i < 2) { out.push_back(std::move(steps[i++])); continue; }
+      std::vector<const std::string*> sources;
+      std::vector<unsigned> grids;
+      for (size_t k = i; k < j; ++k) { sources.push_back(&P.kernels[steps[k].kernel].source); grids.push_back(steps[k].grid[0]); }
+      std::string combined = combineKernels(sources, grids);
+      if (combined.empty()) { out.push_back(std::move(steps[i++])); continue; }
+      Step m;
+      m.kind = Step::Kernel;
+      m.kernel = kernelId(combined);
+      m.block[0] = 256;
+      m.grid[0] = 0;
+      m.time = steps[i].time;
+      m.label = "batch[" + std::to_string(j - i) + "]:" + steps[i].label;
+      const int tFirst = steps[i].time, tLast = steps[j - 1].time;
+      for (size_t k = i; k < j; ++k) {
+        m.grid[0] += steps[k].grid[0];
+        m.algoBytes += steps[k].algoBytes;
+        for (size_t a = 0; a < steps[k].args.size(); ++a) {
+          m.args.push_back(steps[k].args[a]);
+          m.argWrites.push_back(steps[k].argWrites[a]);
+          // every buffer of the group is live for the whole group: the segments run concurrently
+          ref(steps[k].args[a].index, tFirst);
+          ref(steps[k].args[a].index, tLast);
+        }
+      }
+      out.push_back(std::move(m));
+      i = j;
+    }
+    steps = std::move(out);
   }
 
   // ---------------------------------------------------------------- arena

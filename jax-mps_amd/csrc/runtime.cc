@@ -355,10 +355,10 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
   }
   switch (s.kind) {
     case Step::Kernel: {
-      void* ptrs[64];
-      void* argv[64];
+      void* ptrs[256];
+      void* argv[256];
       size_t n = s.args.size();
-      if (n > 64) throw RuntimeError("fused kernel with more than 64 arguments");
+      if (n > 256) throw RuntimeError("fused kernel with more than 256 arguments");
       for (size_t i = 0; i < n; ++i) { ptrs[i] = resolve(s.args[i], in, out); argv[i] = &ptrs[i]; }
       check(mi355_launch((mi355_function_t)prog_->kernels[s.kernel].function, s.grid, s.block, argv, (int)n, st), s.label.c_str());
       break;

@@ -252,6 +252,12 @@ case("dot-int32-batched-attention-layout", lambda b, q, k: b.dot_general(q, k, (
 case("dot-int32-wraps", lambda b, x, y: b.matmul(x, y), i32(1934, 8, 300, lo=-2**30, hi=2**30), i32(1935, 300, 8, lo=-2**30, hi=2**30), exact=True)
 case("dot-uint32-above-2p24", lambda b, x, y: b.matmul(x, y), rng(1936).integers(0, 2**20, size=(5, 40)).astype(np.uint32), rng(1937).integers(0, 2**11, size=(40, 6)).astype(np.uint32), exact=True)
 case("dot-large-k", lambda b, x, y: b.matmul(x, y), f32(192, 64, 3000, lo=-1, hi=1), f32(193, 3000, 64, lo=-1, hi=1))
+# fp32 products by size class: small ones run on the K-split-in-workgroup kernel (16- or 32-wide tiles), larger
+# unbatched ones on the implicit-GEMM kernel, larger batched ones on the strided tile kernel
+case("dot-f32-small-tile32-batched", lambda b, x, y: b.dot_general(x, y, ([2], [1]), ([0], [0])), f32(1940, 6, 300, 200, lo=-1, hi=1), f32(1941, 6, 200, 300, lo=-1, hi=1))
+case("dot-f32-small-tile32-transposed", lambda b, x, y: b.dot_general(x, y, ([0], [1])), f32(1942, 77, 500, lo=-1, hi=1), f32(1943, 610, 77, lo=-1, hi=1))
+case("dot-f32-igemm", lambda b, x, y: b.matmul(x, y), f32(1944, 520, 384, lo=-1, hi=1), f32(1945, 384, 1030, lo=-1, hi=1))
+case("dot-f32-strided-batched", lambda b, x, y: b.dot_general(x, y, ([2], [1]), ([0], [0])), f32(1946, 8, 330, 256, lo=-1, hi=1), f32(1947, 8, 256, 330, lo=-1, hi=1))
 
 
 def _conv(**kw):
