@@ -12,6 +12,13 @@
 // With that swizzle the MFMA operand read (32 rows x one slot, ds_read_b128) touches every
 // bank once per 16 lanes.
 //
+// B may also be given n-contiguous ([K][N] rows, the layout of a dense layer's weights): its
+// stage then holds 64 k-rows of BN columns, and the MFMA operand (8 consecutive k per lane) is
+// assembled by two transposing LDS reads (ds_read_b64_tr_b16: within 16 lanes, lane d receives
+// element d%4 of the 8 bytes addressed by lanes d/4, d/4+4, d/4+8, d/4+12), so no transposed
+// copy of the weights is made.  The 16-byte slots of a k-row are XOR-swizzled by the row number
+// so that the four rows one such read touches fall into different banks.
+//
 // Pipeline per iteration: wait until the oldest stage has landed (vmcnt), barrier, start the
 // loads that refill the stage consumed one iteration ago, multiply the landed stage.  One
 // barrier per 64-wide K-slab; loads are (STAGES-1) slabs ahead of the math.
@@ -29,6 +36,8 @@ typedef unsigned short u16;
 typedef unsigned int u32;
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
 
 #define GLOBAL_PTR(p) ((__attribute__((address_space(1))) void*)(p))
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -51,7 +60,11 @@ __device__ __forceinline__ u16 to_bf16(float f) { return __builtin_bit_cast(u16,
 // vmcnt in bits 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at their maxima)
 constexpr int vmcntImm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
-template <int BM, int BN, int STAGES>
+// slot swizzle of an n-contiguous B stage: rows k .. k+3 of one 32-column block land in distinct banks
+template <int BN>
+__device__ __forceinline__ int swzB(int k) { return BN == 64 ? ((k >> 1) & 1) << 2 : (k & 3) << 2; }
+
+template <int BM, int BN, int STAGES, bool BNN>
 __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
   constexpr int BK = 64;
   constexpr int TM = BM / 64, TN = BN / 64;
@@ -85,6 +98,14 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
       long long gm = m0 + r;
       if (gm > g.M - 1) gm = g.M - 1;
       src[j] = A + gm * g.aLd + kv * 8;
+    } else if (BNN) {
+      constexpr int PR = BN / 8;                      // 16-byte slots per k-row
+      const int q = (c - BM / 8) * 64 + lane;         // physical slot within the B part
+      const int k = q / PR;
+      const int pcol = (q % PR) ^ swzB<BN>(k);        // logical slot kept there
+      long long gn = n0 + pcol * 8;
+      if (gn > g.N - 8) gn = g.N - 8;                 // columns past the edge are never stored
+      src[j] = B + (long long)k * g.bLd + gn;
     } else {
       long long gn = n0 + (r - BM);
       if (gn > g.N - 1) gn = g.N - 1;
@@ -98,7 +119,9 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
       unsigned char* dst = ring + buf * STAGE_BYTES + (j * 4 + wave) * 1024;
-      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[j] + k0), LDS_PTR(dst), 16, 0, 0);
+      // loads j >= BM/32 fill the B part; an n-contiguous B advances by rows
+      const long long step = (BNN && j >= BM / 32) ? k0 * g.bLd : k0;
+      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[j] + step), LDS_PTR(dst), 16, 0, 0);
     }
   };
 
@@ -117,6 +140,19 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
   const int arow = wm * (BM / 2) + (lane & 31);
   const int brow = BM + wn * (BN / 2) + (lane & 31);
   const int khalf = lane >> 5;
+  // n-contiguous B: per-lane byte offset of its transposing reads inside a stage.  Lane d of a 16-lane group
+  // addresses k-row khalf*8 + d/4 (+ a multiple of 4 per read, which leaves the swizzle unchanged) and
+  // the 4 columns 4*(d%4) .. +3 of the group's 16.
+  int bOff[TN];
+  if (BNN) {
+    const int d = lane & 15, nhalf = (lane >> 4) & 1;
+    const int kLane = khalf * 8 + (d >> 2);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int slot = ((wn * (BN / 2) + j * 32) >> 3) + nhalf * 2 + ((d & 3) >> 1);
+      bOff[j] = BM * 128 + kLane * (BN * 2) + ((slot ^ swzB<BN>(kLane)) << 4) + ((d & 1) << 3);
+    }
+  }
   for (int it = 0; it < nk; ++it) {
     __builtin_amdgcn_s_waitcnt(vmcntImm((STAGES - 2) * NI));
     __builtin_amdgcn_s_barrier();
@@ -132,8 +168,17 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const int r = brow + j * 32;
-        bv[p][j] = *(const bf16x8*)(st + r * 128 + (((kk * 2 + khalf) ^ ((r >> 1) & 7)) << 4));
+        if (BNN) {
+          short4v h[2];
+#pragma unroll
+          for (int q = 0; q < 2; ++q)   // the step-dependent part of the address is a compile-time offset
+            h[q] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v*)(st + bOff[j] + (kk * 16 + q * 4) * (BN * 2)));
+          short8v both = __builtin_shufflevector(h[0], h[1], 0, 1, 2, 3, 4, 5, 6, 7);
+          bv[p][j] = __builtin_bit_cast(bf16x8, both);
+        } else {
+          const int r = brow + j * 32;
+          bv[p][j] = *(const bf16x8*)(st + r * 128 + (((kk * 2 + khalf) ^ ((r >> 1) & 7)) << 4));
+        }
       }
     };
     frags(0, 0);
@@ -169,15 +214,15 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
   }
 }
 
-template <int BM, int BN, int STAGES>
+template <int BM, int BN, int STAGES, bool BNN>
 int launch(const AsyncArgs& g, hipStream_t st) {
   constexpr int bytes = STAGES * (BM + BN) * 128;
   static bool configured = false;   // per process; the attribute is per function, not per device state that changes
   if (!configured) {
-    if (hipFuncSetAttribute((const void*)gemm_bf16_async<BM, BN, STAGES>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return 3;
+    if (hipFuncSetAttribute((const void*)gemm_bf16_async<BM, BN, STAGES, BNN>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return 3;
     configured = true;
   }
-  gemm_bf16_async<BM, BN, STAGES><<<dim3((unsigned)g.total), 256, bytes, st>>>(g);
+  gemm_bf16_async<BM, BN, STAGES, BNN><<<dim3((unsigned)g.total), 256, bytes, st>>>(g);
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 
@@ -224,6 +269,7 @@ __global__ void __launch_bounds__(256) transpose_bf16(TransposeArgs t) {
 struct OperandPlan {
   bool ok = false;
   bool copy = false;     // needs a transposed copy in the workspace
+  bool rowsOfK = false;  // used in place as [K][rows] (B only): the kernel transposes while reading LDS
   long long ld = 0;      // row pitch when used in place
 };
 
@@ -242,6 +288,19 @@ bool qualifies(const mi355_gemm_desc* d, OperandPlan& pa, OperandPlan& pb) {
   if (d->K % 64 != 0) return false;
   pa = planOperand(d->aRow, d->aCol, d->M, d->K, d->N);
   pb = planOperand(d->bCol, d->bRow, d->N, d->K, d->M);
+  // An n-contiguous B is read in place when that beats a transposed copy: the in-place kernel runs about a
+  // sixth slower than the k-contiguous one on large products (measured), the copy costs a launch plus one pass over B.
+  // MI355X_GEMM_NN=0 always copies, =2 never does.
+  static const int nnMode = getenv("MI355X_GEMM_NN") ? atoi(getenv("MI355X_GEMM_NN")) : 1;
+  if (nnMode != 0 && d->bCol == 1 && d->bRow % 8 == 0 && d->N % 8 == 0 && d->N >= 8 && d->bRow >= d->N) {
+    const double nbd = (double)nb;
+    const double gemmSeconds = 2.0 * nbd * (double)d->M * (double)d->N * (double)d->K / 450e12;
+    const double copySeconds = 5e-6 + 4.0 * nbd * (double)d->N * (double)d->K / 5e12;
+    if (nnMode == 2 || !pb.ok || 0.15 * gemmSeconds < copySeconds) {
+      pb = OperandPlan();
+      pb.ok = true; pb.rowsOfK = true; pb.ld = d->bRow;
+    }
+  }
   if (!pa.ok || !pb.ok) return false;
   if (d->batch0 > 1 && (d->aB0 % 8 || d->bB0 % 8)) return false;
   if (d->batch1 > 1 && (d->aB1 % 8 || d->bB1 % 8)) return false;
@@ -312,8 +371,14 @@ extern "C" int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, co
   g.total = (long long)g.tilesM * g.tilesN * nb;
   if (g.total > 0x7FFFFFFFll) return -1;
   // two ring stages keep two workgroups resident per compute unit, which hides more than a deeper ring does
-  if (bm == 256) return launch<256, 128, 3>(g, st);
-  if (bm == 128 && bn == 128) return launch<128, 128, 2>(g, st);
-  if (bm == 128) return launch<128, 64, 2>(g, st);
-  return launch<64, 64, 2>(g, st);
+  if (pb.rowsOfK) {
+    if (bm == 256) return launch<256, 128, 3, true>(g, st);
+    if (bm == 128 && bn == 128) return launch<128, 128, 2, true>(g, st);
+    if (bm == 128) return launch<128, 64, 2, true>(g, st);
+    return launch<64, 64, 2, true>(g, st);
+  }
+  if (bm == 256) return launch<256, 128, 3, false>(g, st);
+  if (bm == 128 && bn == 128) return launch<128, 128, 2, false>(g, st);
+  if (bm == 128) return launch<128, 64, 2, false>(g, st);
+  return launch<64, 64, 2, false>(g, st);
 }

@@ -247,6 +247,13 @@ case("dot-bf16-async-nt-big", lambda b, x, y: b.dot_general(x, y, ([1], [1])), f
 # integer contractions are lowered to broadcast-multiply-reduce (exact, wrap-around)
 def i32(seed, *shape, lo=-1000, hi=1000):
     return rng(seed).integers(lo, hi, size=shape).astype(np.int32)
+# n-contiguous rhs (a dense layer's [in, out] weights) read in place by the LDS-ring kernel, one case per tile shape
+case("dot-bf16-async-nn-edges", lambda b, x, y: b.matmul(x, y), f32(1950, 200, 128, lo=-1, hi=1), f32(1951, 128, 328, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("dot-bf16-async-nn-narrow", lambda b, x, y: b.matmul(x, y), f32(1952, 300, 64, lo=-1, hi=1), f32(1953, 64, 72, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("dot-bf16-async-nn-batched", lambda b, x, y: b.dot_general(x, y, ([2], [1]), ([0], [0])), f32(1954, 3, 130, 64, lo=-1, hi=1), f32(1955, 3, 64, 136, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("dot-bf16-async-nn-128x64", lambda b, x, y: b.matmul(x, y), f32(1956, 2048, 128, lo=-1, hi=1), f32(1957, 128, 3072, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("dot-bf16-async-nn-128x128", lambda b, x, y: b.dot_general(x, y, ([1], [0]), out_dtype="f32"), f32(1958, 2048, 128, lo=-1, hi=1), f32(1959, 128, 6144, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("dot-bf16-async-nn-256x128", lambda b, x, y: b.matmul(x, y), f32(1960, 4096, 192, lo=-1, hi=1), f32(1961, 192, 8200, lo=-1, hi=1), dtypes=["bf16", "bf16"])
 case("dot-int32-matmul", lambda b, x, y: b.matmul(x, y), i32(1930, 33, 70), i32(1931, 70, 45), exact=True)
 case("dot-int32-batched-attention-layout", lambda b, q, k: b.dot_general(q, k, ([3], [3]), ([0, 2], [0, 2])), i32(1932, 2, 9, 3, 16), i32(1933, 2, 11, 3, 16), exact=True)
 case("dot-int32-wraps", lambda b, x, y: b.matmul(x, y), i32(1934, 8, 300, lo=-2**30, hi=2**30), i32(1935, 300, 8, lo=-2**30, hi=2**30), exact=True)
