@@ -60,7 +60,10 @@ _FUSED_BYTES = {   # algorithmic bytes: distinct inputs + outputs, broadcast ope
 }
 
 
-def bench_fused_ops(client, iters=20):
+FUSED_REPEAT = 20   # launches of each fused kernel between one pair of HIP events
+
+
+def bench_fused_ops(client, iters=10):
     from jax_mps_amd import pjrt, runner
     from shlo_oracle import parse
     out = []
@@ -80,13 +83,16 @@ def bench_fused_ops(client, iters=20):
         r[0].block_until_ready()
         dt = (time.perf_counter() - t0) / iters
         ca = exe.cost_analysis()
-        # device time of the kernels themselves (HIP events), when the plugin was asked to time them
+        # device time of the kernels themselves: HIP events around FUSED_REPEAT back-to-back launches of each
+        # kernel of the program (the event pair alone costs a few microseconds, as much as a small kernel)
         kms = sum(v for k, v in ca.items() if k.endswith(".time_ms"))
         kcount = sum(v for k, v in ca.items() if k.endswith(".count"))
-        dev = (kms / (iters + 3)) * 1e-3 if kcount else dt
+        steps = int(ca.get("steps", 0))
+        passes = kcount / max(steps, 1)                       # how many times the whole program was timed
+        dev = (kms / passes) * 1e-3 if kcount else dt
         gbs = _FUSED_BYTES[name] / dev / 1e9
         out.append({"op": name, "GB/s": round(gbs, 1), "frac_of_peak": round(gbs / PEAK_HBM_GBS, 4), "us": round(dev * 1e6, 2),
-                    "launches": int(ca.get("steps", 0))})
+                    "launches": steps, "us_per_call_wall": round(dt * 1e6 / FUSED_REPEAT, 2)})
     return out
 
 
@@ -179,6 +185,7 @@ def main():
     if not args.no_fused:
         os.environ["MI355X_TIMING"] = "all"
         os.environ["MI355X_TIMING_EVERY"] = "1"
+        os.environ["MI355X_TIMING_REPEAT"] = str(FUSED_REPEAT)
         line["fused_ops"] = bench_fused_ops(client)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()

@@ -224,6 +224,8 @@ Executable::Executable(std::unique_ptr<CompiledProgram> prog) : prog_(std::move(
   timingKinds_ = t ? t : "";
   const char* every = getenv("MI355X_TIMING_EVERY");   // time one execute call in N (sampling keeps the events' own cost small)
   timingEvery_ = every ? std::max(1, atoi(every)) : 1;
+  const char* repeat = getenv("MI355X_TIMING_REPEAT");   // launches of a timed fused kernel per event pair
+  timingRepeat_ = repeat ? std::max(1, atoi(repeat)) : 1;
   const char* gr = getenv("MI355X_GRAPHS");   // "0" runs loop bodies launch by launch
   useGraphs_ = !(gr && gr[0] == '0');
   loadKernels();
@@ -306,7 +308,7 @@ void Executable::resolvePending() {
     float ms = 0;
     if (mi355_event_elapsed_ms(p.a, p.b, &ms) == 0) {
       auto& s = stats_[p.kind];
-      s.count++;
+      s.count += (int64_t)p.launches;
       s.ms += ms;
       s.flops += p.flops;
       s.bytes += p.bytes;
@@ -360,7 +362,12 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       size_t n = s.args.size();
       if (n > 256) throw RuntimeError("fused kernel with more than 256 arguments");
       for (size_t i = 0; i < n; ++i) { ptrs[i] = resolve(s.args[i], in, out); argv[i] = &ptrs[i]; }
-      check(mi355_launch((mi355_function_t)prog_->kernels[s.kernel].function, s.grid, s.block, argv, (int)n, st), s.label.c_str());
+      // A timed fused kernel may be launched several times between its two events: the kernels are pure
+      // functions of their inputs (or rewrite the same window in place), so the result is unchanged, and
+      // the cost of the event pair is spread over the launches.
+      const int launches = doTime ? timingRepeat_ : 1;
+      for (int r = 0; r < launches; ++r)
+        check(mi355_launch((mi355_function_t)prog_->kernels[s.kernel].function, s.grid, s.block, argv, (int)n, st), s.label.c_str());
       break;
     }
     case Step::Gemm: {
@@ -442,7 +449,8 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
   }
   if (doTime) {
     mi355_event_record(eb, st);
-    pending_.push_back({ea, eb, kind, flops, bytes});
+    const double launches = s.kind == Step::Kernel ? (double)timingRepeat_ : 1.0;
+    pending_.push_back({ea, eb, kind, flops * launches, bytes * launches, launches});
     if (pending_.size() > 20000) resolvePending();
   }
 }

@@ -94,12 +94,13 @@ class Executable {
   void* consts_ = nullptr;
   std::mutex mu_;
 
-  struct Pending { mi355_event_t a, b; std::string kind; double flops, bytes; };
+  struct Pending { mi355_event_t a, b; std::string kind; double flops, bytes, launches; };
   std::vector<Pending> pending_;
   std::vector<mi355_event_t> eventPool_;
   std::map<std::string, KindStat> stats_;
   std::string timingKinds_;
   int timingEvery_ = 1;
+  int timingRepeat_ = 1;
   uint64_t executeCount_ = 0;
   bool timedCall_ = true;
 
