@@ -46,6 +46,7 @@ struct AsyncArgs {
   const u16* a;
   const u16* b;
   void* c;
+  const void* bias;   // N values of the output type, or null
   long long M, N, K;
   long long aB0, aB1, aLd, bB0, bB1, bLd;
   int batch1;
@@ -203,12 +204,20 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
     for (int j = 0; j < TN; ++j) {
       const long long col = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
       if (col >= g.N) continue;
+      // bias epilogue: the product is rounded to the output type first, as the separate add would see it
+      float bias = 0.f;
+      if (g.bias) bias = g.outBf16 ? __uint_as_float((u32)((const u16*)g.bias)[col] << 16) : ((const float*)g.bias)[col];
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const long long row = m0 + wm * (BM / 2) + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
         if (row >= g.M) continue;
-        if (g.outBf16) ((u16*)g.c)[cBase + row * g.N + col] = to_bf16(acc[i][j][e]);
-        else ((float*)g.c)[cBase + row * g.N + col] = acc[i][j][e];
+        if (g.outBf16) {
+          u16 r = to_bf16(acc[i][j][e]);
+          if (g.bias) r = to_bf16(__uint_as_float((u32)r << 16) + bias);
+          ((u16*)g.c)[cBase + row * g.N + col] = r;
+        } else {
+          ((float*)g.c)[cBase + row * g.N + col] = acc[i][j][e] + bias;
+        }
       }
     }
   }
@@ -331,7 +340,7 @@ extern "C" size_t mi355_gemm_bf16_async_workspace_bytes(const mi355_gemm_desc* d
 }
 
 // 0 = launched, -1 = layout does not qualify, other = launch error.
-extern "C" int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, const void* b, void* c, void* workspace,
+extern "C" int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, const void* b, void* c, const void* bias, void* workspace,
                                      size_t workspace_bytes, mi355_stream_t s) {
   OperandPlan pa, pb;
   if (!qualifies(d, pa, pb)) return -1;
@@ -341,6 +350,7 @@ extern "C" int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, co
   const long long nb = d->batch0 * d->batch1;
   AsyncArgs g;
   g.a = (const u16*)a; g.b = (const u16*)b; g.c = c;
+  g.bias = bias;
   g.M = d->M; g.N = d->N; g.K = d->K;
   g.aB0 = d->aB0; g.aB1 = d->aB1; g.aLd = pa.ld;
   g.bB0 = d->bB0; g.bB1 = d->bB1; g.bLd = pb.ld;

@@ -68,12 +68,14 @@ typedef struct {
   int in_dtype, out_dtype;
 } mi355_gemm_desc;
 // `workspace` (may be NULL) holds k-contiguous copies of bf16 operands; see mi355_gemm_workspace_bytes.
-int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, void* workspace, size_t workspace_bytes,
-               mi355_stream_t s);
+// `bias` (may be NULL): N values of the output type added to every row of C after the product has been rounded to
+// the output type, i.e. exactly dot_general followed by add(broadcast(bias)).
+int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, const void* bias, void* workspace,
+               size_t workspace_bytes, mi355_stream_t s);
 size_t mi355_gemm_workspace_bytes(const mi355_gemm_desc* d);
 // bf16 operands with 16-byte-loadable layouts on 128x128 / 128x64 / 64x64 tiles; -1 = layout does not qualify
 // bf16, both operands k-contiguous, K % 64 == 0: LDS ring filled by direct global->LDS loads
-int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, const void* b, void* c, void* workspace,
+int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, const void* b, void* c, const void* bias, void* workspace,
                           size_t workspace_bytes, mi355_stream_t s);
 size_t mi355_gemm_bf16_async_workspace_bytes(const mi355_gemm_desc* d);
 int mi355_gemm_bf16_tiled(const mi355_gemm_desc* d, const void* a, const void* b, void* c, mi355_stream_t s);

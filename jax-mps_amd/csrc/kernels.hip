@@ -70,7 +70,17 @@ struct GemmArgs {
   long long aB0, aB1, aRow, aCol, bB0, bB1, bRow, bCol;
   int batch1;
   int outBf16;
+  const void* bias;   // N values of the output type, or null
 };
+
+// c[r][n] += bias[n] for kernels without a bias epilogue of their own (c is already rounded to its type)
+template <typename T>
+__global__ void __launch_bounds__(256) gemm_add_bias(T* c, const T* bias, long long total, long long N) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  if constexpr (sizeof(T) == 2) c[i] = f2bf(bf2f(c[i]) + bf2f(bias[i % N]));
+  else c[i] = c[i] + bias[i % N];
+}
 
 __global__ void __launch_bounds__(256) gemm_f32_mfma(GemmArgs g) {
   constexpr int BM = 64, BN = 64, BK = 16;
@@ -174,7 +184,10 @@ __global__ void __launch_bounds__(256) gemm_f32_small(GemmArgs g) {
   float* C = (float*)g.c + (long long)blockIdx.z * g.M * g.N;
   for (int e = threadIdx.x; e < T * T; e += 256) {
     const long long row = m0 + e / T, col = n0 + e % T;
-    if (row < g.M && col < g.N) C[row * g.N + col] = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
+    if (row < g.M && col < g.N) {
+      const float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
+      C[row * g.N + col] = g.bias ? sum + ((const float*)g.bias)[col] : sum;
+    }
   }
 }
 
@@ -634,8 +647,17 @@ size_t mi355_gemm_workspace_bytes(const mi355_gemm_desc* d) {
   return 0;
 }
 
-int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, void* workspace, size_t workspace_bytes,
-               mi355_stream_t s) {
+static int addBias(const mi355_gemm_desc* d, void* c, const void* bias, mi355_stream_t s) {
+  if (!bias) return 0;
+  const long long total = d->batch0 * d->batch1 * d->M * d->N;
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  if (d->out_dtype == 1) gemm_add_bias<u16><<<grid, 256, 0, (hipStream_t)s>>>((u16*)c, (const u16*)bias, total, d->N);
+  else gemm_add_bias<float><<<grid, 256, 0, (hipStream_t)s>>>((float*)c, (const float*)bias, total, d->N);
+  return check("gemm bias");
+}
+
+int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, const void* bias, void* workspace,
+               size_t workspace_bytes, mi355_stream_t s) {
   if (d->M <= 0 || d->N <= 0 || d->batch0 * d->batch1 <= 0) return 0;
   GemmArgs g;
   g.a = a; g.b = b; g.c = c;
@@ -644,12 +666,13 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
   g.bB0 = d->bB0; g.bB1 = d->bB1; g.bRow = d->bRow; g.bCol = d->bCol;
   g.batch1 = (int)d->batch1;
   g.outBf16 = d->out_dtype == 1;
+  g.bias = bias;
   long long nb = d->batch0 * d->batch1;
   if (d->in_dtype == 1) {
-    int r = mi355_gemm_bf16_async(d, a, b, c, workspace, workspace_bytes, s);
+    int r = mi355_gemm_bf16_async(d, a, b, c, bias, workspace, workspace_bytes, s);
     if (r >= 0) return r;
     r = mi355_gemm_bf16_tiled(d, a, b, c, s);
-    if (r >= 0) return r;
+    if (r >= 0) return r ? r : addBias(d, c, bias, s);
   }
   if (const int t = smallGemmTile(d)) {
     dim3 grid((unsigned)((d->N + t - 1) / t), (unsigned)((d->M + t - 1) / t), (unsigned)nb);
@@ -658,13 +681,18 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
     return check("gemm");
   }
   mi355_conv_desc cd;
-  if (gemmAsPointwiseConv(d, &cd)) return mi355_conv(&cd, a, b, c, workspace, workspace_bytes, s);
+  // strided views may start anywhere; the implicit-GEMM loaders issue 16-byte loads
+  if (gemmAsPointwiseConv(d, &cd) && (((uintptr_t)a | (uintptr_t)b) & 15) == 0) {
+    int r = mi355_conv(&cd, a, b, c, workspace, workspace_bytes, s);
+    return r ? r : addBias(d, c, bias, s);
+  }
   if (nb > 65535) return 1;   // grid.z limit; callers fold larger batches
   dim3 grid((unsigned)((d->N + 63) / 64), (unsigned)((d->M + 63) / 64), (unsigned)nb);
   if (d->in_dtype == 0) gemm_f32_mfma<<<grid, 256, 0, (hipStream_t)s>>>(g);
   else if (d->in_dtype == 1) gemm_bf16_mfma<<<grid, 256, 0, (hipStream_t)s>>>(g);
   else return 2;
-  return check("gemm");
+  if (int r = check("gemm")) return r;
+  return addBias(d, c, bias, s);
 }
 
 // Direct convolution: the general fallback behind mi355_conv (groups, 3-d windows, bf16).

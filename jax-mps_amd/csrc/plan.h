@@ -77,6 +77,7 @@ struct Step {
   GemmDesc gemm;
   ConvDesc conv;
   ScatterDesc scatter;
+  BufRef bias;                     // Gemm: per-column values added to the product (kind None: no bias)
   int64_t workspaceOffset = -1;    // arena offset of split-K / sort scratch
   int64_t workspaceBytes = 0;
   int splitK = 1;

@@ -154,6 +154,7 @@ class Planner {
 
   static bool forcedBy(Value* v, Op* user) {
     if (isWindowReverse(v, user)) return false;
+    if (dotTakesView(v, user)) return false;
     if (user->name == "gather") return user->operands[0] == v;       // random access needs memory
     if (isFusibleOp(*user)) return false;
     if (user->name == "reduce") return false;   // every reduce kernel evaluates its inputs in place
@@ -680,7 +681,9 @@ class Planner {
 
   // merge an ordered list of dims into (size, stride); false if they do not collapse
   static bool mergeDims(const TensorType& t, const std::vector<int64_t>& dims, int64_t& size, int64_t& stride) {
-    auto st = stridesOf(t);
+    return mergeDims(t, stridesOf(t), dims, size, stride);
+  }
+  static bool mergeDims(const TensorType& t, const std::vector<int64_t>& st, const std::vector<int64_t>& dims, int64_t& size, int64_t& stride) {
     size = 1;
     stride = 0;
     bool have = false;
@@ -699,6 +702,126 @@ class Planner {
     return true;
   }
 
+  // ---------------------------------------------------------------- strided views
+  // A dot_general operand that is a slice / reshape / transpose chain over a buffer is read through
+  // element strides and a base offset instead of being copied out first (the split of a fused QKV
+  // projection into heads is such a chain).
+  struct View {
+    Value* root = nullptr;          // value that owns the memory
+    int64_t offset = 0;             // elements from the root's first element
+    std::vector<int64_t> strides;   // per dim of the viewed value
+  };
+
+  // strides of `newDims` over memory laid out as (oldDims, oldStrides), if no copy is needed
+  static bool reshapeStrides(const std::vector<int64_t>& oldDims, const std::vector<int64_t>& oldStrides, const std::vector<int64_t>& newDims,
+                             std::vector<int64_t>& out) {
+    std::vector<int64_t> od, os;
+    for (size_t i = 0; i < oldDims.size(); ++i) if (oldDims[i] != 1) { od.push_back(oldDims[i]); os.push_back(oldStrides[i]); }
+    out.assign(newDims.size(), 0);
+    size_t oi = 0, ni = 0;
+    while (ni < newDims.size()) {
+      if (newDims[ni] == 1) { out[ni++] = 0; continue; }
+      if (oi >= od.size()) return false;
+      // grow a group of old dims and a group of new dims until their sizes agree
+      size_t o0 = oi, n0 = ni;
+      int64_t op = od[oi++], np = newDims[ni++];
+      while (op != np) {
+        if (op < np) { if (oi >= od.size()) return false; op *= od[oi++]; }
+        else {
+          while (ni < newDims.size() && newDims[ni] == 1) out[ni++] = 0;
+          if (ni >= newDims.size()) return false;
+          np *= newDims[ni++];
+        }
+      }
+      // the old group must itself be contiguous in its own strides
+      for (size_t k = o0; k + 1 < oi; ++k) if (os[k] != os[k + 1] * od[k + 1]) return false;
+      int64_t st = os[oi - 1];
+      for (size_t k = ni; k-- > n0;) {
+        if (newDims[k] == 1) { out[k] = 0; continue; }
+        out[k] = st;
+        st *= newDims[k];
+      }
+    }
+    return oi == od.size();
+  }
+
+  static bool isViewOp(const Op* d) { return d && d->results.size() == 1 && (d->name == "reshape" || d->name == "slice" || d->name == "transpose"); }
+
+  // `ownsMemory(v)`: the caller's notion of "v is (or will be) in memory".
+  template <typename F>
+  static bool resolveView(Value* v, const F& ownsMemory, View& out) {
+    if (ownsMemory(v)) {
+      out.root = v;
+      out.offset = 0;
+      out.strides = stridesOf(v->type);
+      return true;
+    }
+    Op* d = v->def;
+    if (!isViewOp(d) || v->type.numel() == 0) return false;
+    View in;
+    if (!resolveView(d->operands[0], ownsMemory, in)) return false;
+    const TensorType& xt = d->operands[0]->type;
+    out.root = in.root;
+    out.offset = in.offset;
+    if (d->name == "slice") {
+      auto& start = d->ints("start");
+      auto& stride = d->ints("strides");
+      out.strides.resize(xt.rank());
+      for (int k = 0; k < xt.rank(); ++k) {
+        out.offset += start[k] * in.strides[k];
+        out.strides[k] = in.strides[k] * (stride.empty() ? 1 : stride[k]);
+      }
+      return true;
+    }
+    if (d->name == "transpose") {
+      auto& perm = d->ints("dims");
+      out.strides.resize(perm.size());
+      for (size_t k = 0; k < perm.size(); ++k) out.strides[k] = in.strides[perm[k]];
+      return true;
+    }
+    return reshapeStrides(xt.dims, in.strides, v->type.dims, out.strides);
+  }
+
+  // the add that emitDot folds into its product as a bias epilogue, or null
+  static Op* foldedBiasAdd(Op* dot) {
+    static const bool fuseBias = !getenv("MI355X_GEMM_BIAS") || atoi(getenv("MI355X_GEMM_BIAS")) != 0;
+    if (!fuseBias || (dot->name != "dot_general" && dot->name != "dot")) return nullptr;
+    Value* c = dot->result();
+    if (c->users.size() != 1 || c->users[0]->name != "add" || c->users[0]->parent != dot->parent || c->type.numel() == 0 || c->type.rank() == 0) return nullptr;
+    // exactly one free rhs dim, so that the last result dim is the GEMM's column index
+    Value* b = dot->operands[1];
+    int64_t used = (int64_t)dot->ints("rhs_batch").size() + (int64_t)dot->ints("rhs_contract").size();
+    if (dot->name == "dot") used = 1;
+    if (b->type.rank() - used != 1) return nullptr;
+    Op* add = c->users[0];
+    Value* other = add->operands[0] == c ? add->operands[1] : add->operands[0];
+    Op* bc = other->def;
+    if (other == c || !bc || bc->name != "broadcast_in_dim" || bc->parent != dot->parent) return nullptr;
+    Value* bias = bc->operands[0];
+    if (bias->type.rank() != 1 || bias->type.dt != c->type.dt || bias->type.dims[0] != c->type.dims.back()) return nullptr;
+    if (bc->ints("dims") != std::vector<int64_t>{(int64_t)c->type.rank() - 1}) return nullptr;
+    return add;
+  }
+
+  // values that are in memory whatever the fusion analysis decides: arguments, results of ops that
+  // are steps of their own, and bias sums folded into their product
+  static bool alwaysInMemory(Value* v) {
+    if (!v->def) return true;
+    if (!isFusibleOp(*v->def)) return v->def->name != "return";
+    if (v->def->name == "add")
+      for (auto* o : v->def->operands)
+        if (o->def && (o->def->name == "dot_general" || o->def->name == "dot") && foldedBiasAdd(o->def) == v->def) return true;
+    return false;
+  }
+
+  static bool dotTakesView(Value* v, Op* user) {
+    static const bool views = !getenv("MI355X_GEMM_VIEWS") || atoi(getenv("MI355X_GEMM_VIEWS")) != 0;
+    if (!views || (user->name != "dot_general" && user->name != "dot") || !isViewOp(v->def)) return false;
+    if (v->type.dt != DType::F32 && v->type.dt != DType::BF16) return false;
+    View vw;
+    return resolveView(v, alwaysInMemory, vw);
+  }
+
   void emitDot(Op* op, Plan& plan) {
     Value* a = op->operands[0];
     Value* b = op->operands[1];
@@ -711,25 +834,32 @@ class Planner {
     for (int d = 0; d < b->type.rank(); ++d) if (!has(bb, d) && !has(bc, d)) bf.push_back(d);
     if (!isFloat(a->type.dt) || a->type.dt == DType::F64 || a->type.dt == DType::F16)
       throw CompileError("dot_general: only f32 and bf16 operands are supported");
-    for (Value* v : {a, b}) if (!hasStorage(v)) materializeNow(v, plan);
+    View va, vb;
+    auto stored = [this](Value* v) { return hasStorage(v); };
+    for (Value* v : {a, b}) {
+      View& vw = v == a ? va : vb;
+      if (!hasStorage(v) && !(dotTakesView(v, op) && resolveView(v, stored, vw))) materializeNow(v, plan);
+      if (hasStorage(v)) { vw.root = v; vw.offset = 0; vw.strides = stridesOf(v->type); }
+    }
+    if (b == a) vb = va;
     GemmDesc g;
     g.inType = a->type.dt;
     g.outType = c->type.dt;
     // contraction dims: order both sides by the lhs stride so each side collapses when it can
     std::vector<size_t> order(ac.size());
     for (size_t k = 0; k < order.size(); ++k) order[k] = k;
-    auto ast = stridesOf(a->type);
+    const std::vector<int64_t>& ast = va.strides;
     std::sort(order.begin(), order.end(), [&](size_t x, size_t y) { return ast[ac[x]] > ast[ac[y]]; });
     std::vector<int64_t> acs, bcs;
     for (auto k : order) { acs.push_back(ac[k]); bcs.push_back(bc[k]); }
     int64_t Ka = 0, Kb = 0, M = 0, N = 0;
-    bool ok = mergeDims(a->type, acs, Ka, g.aCol) && mergeDims(b->type, bcs, Kb, g.bRow) &&
-              mergeDims(a->type, af, M, g.aRow) && mergeDims(b->type, bf, N, g.bCol);
+    bool ok = mergeDims(a->type, va.strides, acs, Ka, g.aCol) && mergeDims(b->type, vb.strides, bcs, Kb, g.bRow) &&
+              mergeDims(a->type, va.strides, af, M, g.aRow) && mergeDims(b->type, vb.strides, bf, N, g.bCol);
     g.M = M; g.N = N; g.K = Ka;
     // batch dims: up to two independent strides per operand
     std::vector<int64_t> bsz;
     std::vector<int64_t> abst, bbst;
-    auto bstr = stridesOf(b->type);
+    const std::vector<int64_t>& bstr = vb.strides;
     for (size_t k = 0; k < ab.size(); ++k) {
       if (a->type.dims[ab[k]] == 1) continue;
       if (!bsz.empty() && ast[ab[k]] * a->type.dims[ab[k]] == abst.back() && bstr[bb[k]] * b->type.dims[bb[k]] == bbst.back()) {
@@ -746,15 +876,34 @@ class Planner {
       throw CompileError("dot_general: operand layout needs a transposed copy (dims do not collapse to strided 2-D); not supported yet: " + a->type.str() + " x " + b->type.str());
     if (bsz.size() >= 1) { g.batch0 = bsz[0]; g.aB0 = abst[0]; g.bB0 = bbst[0]; }
     if (bsz.size() == 2) { g.batch1 = bsz[1]; g.aB1 = abst[1]; g.bB1 = bbst[1]; }
+    // dot_general -> add(broadcast(bias over the last dim)) with no other reader of the product: the kernels add the
+    // bias while they store the result (the reference fuses the same pair into one addmm, passes/fuse_bias_add.cc:120-171)
+    Value* biasV = nullptr;
+    Op* biasAdd = foldedBiasAdd(op);
+    if (biasAdd) {
+      Value* other = biasAdd->operands[0] == c ? biasAdd->operands[1] : biasAdd->operands[0];
+      biasV = other->def->operands[0];
+      if (!hasStorage(biasV)) {
+        if (biasV->def && isFusibleOp(*biasV->def)) materializeNow(biasV, plan);
+        else biasAdd = nullptr, biasV = nullptr;
+      }
+    }
     int sid = newStorage(c->type.bytes());
     bind(c, sid);
     if (c->type.numel() == 0) return;
     int t = ++time_;
     Step s;
     s.kind = Step::Gemm;
-    s.label = "dot_general " + a->type.str() + " x " + b->type.str();
+    s.label = "dot_general " + a->type.str() + " x " + b->type.str() + (biasV ? " + bias" : "");
     s.gemm = g;
-    s.args = {ref(storageOf(a), t), ref(storageOf(b), t), ref(sid, t)};
+    s.args = {ref(storageOf(va.root), t), ref(storageOf(vb.root), t), ref(sid, t)};
+    s.args[0].offset = va.offset * (int64_t)dtypeSize(a->type.dt);
+    s.args[1].offset = vb.offset * (int64_t)dtypeSize(b->type.dt);
+    if (biasV) {
+      s.bias = ref(storageOf(biasV), t);
+      bind(biasAdd->result(), sid);   // the step writes the sum; nothing reads the bare product
+      emitted_.insert(biasAdd);
+    }
     // room for a k-contiguous copy of an operand that is laid out along m or n
     mi355_gemm_desc abi = toAbi(g);
     int64_t ws = ((int64_t)mi355_gemm_workspace_bytes(&abi) + kAlign - 1) / kAlign * kAlign;
@@ -1241,6 +1390,7 @@ class Planner {
       for (auto& a : s.args) a = finalRef(a);
       s.src = finalRef(s.src);
       s.dst = finalRef(s.dst);
+      s.bias = finalRef(s.bias);
       s.predBuf = finalRef(s.predBuf);
       if (s.cond) patch(*s.cond);
       for (auto& b : s.bodies) patch(*b);

@@ -373,7 +373,8 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
     case Step::Gemm: {
       mi355_gemm_desc d = toAbi(s.gemm);
       void* ws = s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
-      check(mi355_gemm(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), ws,
+      const void* bias = s.bias.kind == BufRef::None ? nullptr : resolve(s.bias, in, out);
+      check(mi355_gemm(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), bias, ws,
                        (size_t)s.workspaceBytes, st), "gemm");
       break;
     }
@@ -490,7 +491,7 @@ void Executable::runCountedLoop(const Step& s, const std::vector<DeviceBuffer*>&
       auto add = [&](const BufRef& b) { if (b.kind == BufRef::Param || b.kind == BufRef::Output) lgs.external.push_back(b); };
       for (auto& st : p.steps) {
         for (auto& a : st.args) add(a);
-        add(st.src); add(st.dst); add(st.predBuf);
+        add(st.src); add(st.dst); add(st.predBuf); add(st.bias);
         if (st.cond) scan(*st.cond);
         for (auto& b : st.bodies) scan(*b);
       }

@@ -254,6 +254,41 @@ case("dot-bf16-async-nn-batched", lambda b, x, y: b.dot_general(x, y, ([2], [1])
 case("dot-bf16-async-nn-128x64", lambda b, x, y: b.matmul(x, y), f32(1956, 2048, 128, lo=-1, hi=1), f32(1957, 128, 3072, lo=-1, hi=1), dtypes=["bf16", "bf16"])
 case("dot-bf16-async-nn-128x128", lambda b, x, y: b.dot_general(x, y, ([1], [0]), out_dtype="f32"), f32(1958, 2048, 128, lo=-1, hi=1), f32(1959, 128, 6144, lo=-1, hi=1), dtypes=["bf16", "bf16"])
 case("dot-bf16-async-nn-256x128", lambda b, x, y: b.matmul(x, y), f32(1960, 4096, 192, lo=-1, hi=1), f32(1961, 192, 8200, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+# bias added by the GEMM kernels' own epilogue (dot_general -> add(broadcast(bias)) with no other reader of the product)
+def _linear(b, x, w, bias):
+    y = b.dot_general(x, w, ([x.ndim - 1], [0]))
+    return b.add(y, b.broadcast_in_dim(bias, y.shape, [y.ndim - 1]))
+
+
+case("dot-bias-f32-small", _linear, f32(1970, 33, 70), f32(1971, 70, 45), f32(1972, 45))
+case("dot-bias-f32-igemm", _linear, f32(1973, 520, 384, lo=-1, hi=1), f32(1974, 384, 1030, lo=-1, hi=1), f32(1975, 1030))
+case("dot-bias-f32-3d", _linear, f32(1976, 4, 9, 70), f32(1977, 70, 24), f32(1978, 24))
+case("dot-bias-bf16-async", _linear, f32(1979, 200, 128, lo=-1, hi=1), f32(1980, 128, 328, lo=-1, hi=1), f32(1981, 328), dtypes=["bf16", "bf16", "bf16"])
+case("dot-bias-bf16-tiled", _linear, f32(1982, 200, 136, lo=-1, hi=1), f32(1983, 136, 328, lo=-1, hi=1), f32(1984, 328), dtypes=["bf16", "bf16", "bf16"])
+case("dot-bias-bf16-odd", _linear, f32(1985, 37, 50, lo=-1, hi=1), f32(1986, 50, 29, lo=-1, hi=1), f32(1987, 29), dtypes=["bf16", "bf16", "bf16"])
+case("dot-bias-computed", lambda b, x, w, c: _linear(b, x, w, b.mul(c, c)), f32(1988, 33, 70), f32(1989, 70, 45), f32(1990, 45))
+case("dot-bias-product-read-twice", lambda b, x, w, c: (lambda y: b.mul(b.add(y, b.broadcast_in_dim(c, y.shape, [1])), y))(b.matmul(x, w)),
+     f32(1991, 33, 70), f32(1992, 70, 45), f32(1993, 45))
+
+
+# operands that are slice / reshape / transpose chains over a buffer are read through strides (no copy kernel)
+def _qkv_attention_logits(b, x, w, bias, heads):
+    bt, s, _ = x.shape
+    hd = w.shape[1] // (3 * heads)
+    qkv = b.reshape(_linear(b, x, w, bias), (bt, s, 3, heads, hd))
+    q, k, v = (b.reshape(b.slice(qkv, [0, 0, i, 0, 0], [bt, s, i + 1, heads, hd]), (bt, s, heads, hd)) for i in range(3))
+    logits = b.dot_general(q, k, ([3], [3]), ([0, 2], [0, 2]))      # B H T S
+    return b.dot_general(logits, v, ([3], [1]), ([0, 1], [0, 2]))   # B H T D
+
+
+case("dot-view-qkv-split-f32", lambda b, x, w, c: _qkv_attention_logits(b, x, w, c, 2), f32(2000, 3, 10, 24, lo=-1, hi=1), f32(2001, 24, 48, lo=-1, hi=1), f32(2002, 48))
+case("dot-view-qkv-split-bf16", lambda b, x, w, c: _qkv_attention_logits(b, x, w, c, 3), f32(2003, 2, 128, 64, lo=-1, hi=1), f32(2004, 64, 576, lo=-0.3, hi=0.3), f32(2005, 576, lo=-0.3, hi=0.3),
+     dtypes=["bf16", "bf16", "bf16"])
+case("dot-view-strided-slice-of-argument", lambda b, x, y: b.matmul(b.slice(x, [1, 2], [33, 70], [2, 1]), b.slice(y, [0, 3], [68, 45], [1, 2])), f32(2006, 33, 70), f32(2007, 70, 45))
+case("dot-view-transpose-of-argument", lambda b, x, y: b.matmul(b.transpose(x, [1, 0]), b.transpose(y, [1, 0])), f32(2008, 70, 33), f32(2009, 45, 70))
+case("dot-view-reshape-merging-dims", lambda b, x, y: b.matmul(b.reshape(b.slice(x, [0, 0, 0], [4, 6, 35]), (24, 35)), y), f32(2010, 4, 6, 40), f32(2011, 35, 12))
+case("dot-view-reshape-not-a-view", lambda b, x, y: b.matmul(b.reshape(b.slice(x, [0, 0, 0], [4, 5, 35]), (20, 35)), y), f32(2012, 4, 6, 35), f32(2013, 35, 12))
+case("dot-view-same-buffer-twice", lambda b, x: b.dot_general(b.slice(x, [0, 0], [16, 40]), b.slice(x, [16, 0], [32, 40]), ([1], [1])), f32(2014, 32, 40))
 case("dot-int32-matmul", lambda b, x, y: b.matmul(x, y), i32(1930, 33, 70), i32(1931, 70, 45), exact=True)
 case("dot-int32-batched-attention-layout", lambda b, q, k: b.dot_general(q, k, ([3], [3]), ([0, 2], [0, 2])), i32(1932, 2, 9, 3, 16), i32(1933, 2, 11, 3, 16), exact=True)
 case("dot-int32-wraps", lambda b, x, y: b.matmul(x, y), i32(1934, 8, 300, lo=-2**30, hi=2**30), i32(1935, 300, 8, lo=-2**30, hi=2**30), exact=True)
