@@ -134,46 +134,63 @@ __global__ void __launch_bounds__(256) gemm_f32_mfma(GemmArgs g) {
 // one workgroup per TxT output tile, the four waves split K between them and fold their partial
 // tiles through LDS, so the whole product is one short launch with no split-K workspace.  Operands
 // are read straight from memory in the MFMA operand layout (one element per lane per step).
+// Up to two products of the same shape are summed into one result (x*Wi + h*Wh of a recurrent cell).
+struct SmallPair {
+  const float* a;
+  const float* b;
+  long long K, aB0, aB1, aRow, aCol, bB0, bB1, bRow, bCol;
+};
+struct SmallArgs {
+  SmallPair p[2];
+  int pairs;
+  float* c;
+  const float* bias;   // N values or null
+  long long M, N;
+  int batch1;
+};
+
 template <int T>
-__global__ void __launch_bounds__(256) gemm_f32_small(GemmArgs g) {
+__global__ void __launch_bounds__(256) gemm_f32_small(SmallArgs g) {
   constexpr int KS = T == 16 ? 4 : 2;         // k values per MFMA
   constexpr int NACC = T == 16 ? 4 : 16;
   typedef float accv __attribute__((ext_vector_type(NACC)));
   __shared__ float red[4][T * T];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const long long b0 = blockIdx.z / g.batch1, b1 = blockIdx.z % g.batch1;
-  const float* A = (const float*)g.a + b0 * g.aB0 + b1 * g.aB1;
-  const float* B = (const float*)g.b + b0 * g.bB0 + b1 * g.bB1;
   const long long m0 = (long long)blockIdx.y * T, n0 = (long long)blockIdx.x * T;
   const int r = lane % T, kl = lane / T;
   const bool mOk = m0 + r < g.M, nOk = n0 + r < g.N;
-  const float* ap = A + (m0 + r) * g.aRow;
-  const float* bp = B + (n0 + r) * g.bCol;
-  const long long steps = (g.K + KS - 1) / KS, per = (steps + 3) / 4;
-  const long long s0 = w * per, s1 = s0 + per < steps ? s0 + per : steps;
   accv acc = {0};
-  constexpr int U = 8;
-  long long s = s0;
-  for (; s + U <= s1; s += U) {
-    float av[U], bv[U];
+  for (int q = 0; q < g.pairs; ++q) {
+    const SmallPair& pr = g.p[q];
+    const float* ap = pr.a + b0 * pr.aB0 + b1 * pr.aB1 + (m0 + r) * pr.aRow;
+    const float* bp = pr.b + b0 * pr.bB0 + b1 * pr.bB1 + (n0 + r) * pr.bCol;
+    const long long K = pr.K, aCol = pr.aCol, bRow = pr.bRow;
+    const long long steps = (K + KS - 1) / KS, per = (steps + 3) / 4;
+    const long long s0 = w * per, s1 = s0 + per < steps ? s0 + per : steps;
+    constexpr int U = 8;
+    long long s = s0;
+    for (; s + U <= s1; s += U) {
+      float av[U], bv[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const long long k = (s + u) * KS + kl;
-      av[u] = (mOk && k < g.K) ? ap[k * g.aCol] : 0.f;
-      bv[u] = (nOk && k < g.K) ? bp[k * g.bRow] : 0.f;
-    }
+      for (int u = 0; u < U; ++u) {
+        const long long k = (s + u) * KS + kl;
+        av[u] = (mOk && k < K) ? ap[k * aCol] : 0.f;
+        bv[u] = (nOk && k < K) ? bp[k * bRow] : 0.f;
+      }
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if constexpr (T == 16) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u], acc, 0, 0, 0);
-      else acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u], bv[u], acc, 0, 0, 0);
+      for (int u = 0; u < U; ++u) {
+        if constexpr (T == 16) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u], acc, 0, 0, 0);
+        else acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u], bv[u], acc, 0, 0, 0);
+      }
     }
-  }
-  for (; s < s1; ++s) {
-    const long long k = s * KS + kl;
-    const float a1 = (mOk && k < g.K) ? ap[k * g.aCol] : 0.f;
-    const float b1v = (nOk && k < g.K) ? bp[k * g.bRow] : 0.f;
-    if constexpr (T == 16) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1v, acc, 0, 0, 0);
-    else acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1v, acc, 0, 0, 0);
+    for (; s < s1; ++s) {
+      const long long k = s * KS + kl;
+      const float a1 = (mOk && k < K) ? ap[k * aCol] : 0.f;
+      const float b1v = (nOk && k < K) ? bp[k * bRow] : 0.f;
+      if constexpr (T == 16) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1v, acc, 0, 0, 0);
+      else acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1v, acc, 0, 0, 0);
+    }
   }
 #pragma unroll
   for (int i = 0; i < NACC; ++i) {
@@ -181,12 +198,12 @@ __global__ void __launch_bounds__(256) gemm_f32_small(GemmArgs g) {
     red[w][row * T + r] = acc[i];
   }
   __syncthreads();
-  float* C = (float*)g.c + (long long)blockIdx.z * g.M * g.N;
+  float* C = g.c + (long long)blockIdx.z * g.M * g.N;
   for (int e = threadIdx.x; e < T * T; e += 256) {
     const long long row = m0 + e / T, col = n0 + e % T;
     if (row < g.M && col < g.N) {
       const float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
-      C[row * g.N + col] = g.bias ? sum + ((const float*)g.bias)[col] : sum;
+      C[row * g.N + col] = g.bias ? sum + g.bias[col] : sum;
     }
   }
 }
@@ -647,6 +664,38 @@ size_t mi355_gemm_workspace_bytes(const mi355_gemm_desc* d) {
   return 0;
 }
 
+static SmallPair smallPair(const mi355_gemm_desc* d, const void* a, const void* b) {
+  SmallPair p;
+  p.a = (const float*)a; p.b = (const float*)b;
+  p.K = d->K;
+  p.aB0 = d->aB0; p.aB1 = d->aB1; p.aRow = d->aRow; p.aCol = d->aCol;
+  p.bB0 = d->bB0; p.bB1 = d->bB1; p.bRow = d->bRow; p.bCol = d->bCol;
+  return p;
+}
+
+int mi355_gemm_is_small(const mi355_gemm_desc* d) { return smallGemmTile(d) != 0; }
+
+// C = A1 x B1 (+ A2 x B2 when d2 is given: same M, N and batch dims) (+ bias), both products small fp32 ones.
+int mi355_gemm_small_sum(const mi355_gemm_desc* d1, const void* a1, const void* b1, const mi355_gemm_desc* d2, const void* a2,
+                         const void* b2, void* c, const void* bias, mi355_stream_t s) {
+  const int t = smallGemmTile(d1);
+  if (!t) return -1;
+  if (d2 && (!smallGemmTile(d2) || d2->M != d1->M || d2->N != d1->N || d2->batch0 != d1->batch0 || d2->batch1 != d1->batch1)) return -1;
+  if (d1->M <= 0 || d1->N <= 0 || d1->batch0 * d1->batch1 <= 0) return 0;
+  SmallArgs g;
+  g.p[0] = smallPair(d1, a1, b1);
+  g.p[1] = d2 ? smallPair(d2, a2, b2) : g.p[0];
+  g.pairs = d2 ? 2 : 1;
+  g.c = (float*)c;
+  g.bias = (const float*)bias;
+  g.M = d1->M; g.N = d1->N;
+  g.batch1 = (int)d1->batch1;
+  dim3 grid((unsigned)((d1->N + t - 1) / t), (unsigned)((d1->M + t - 1) / t), (unsigned)(d1->batch0 * d1->batch1));
+  if (t == 16) gemm_f32_small<16><<<grid, 256, 0, (hipStream_t)s>>>(g);
+  else gemm_f32_small<32><<<grid, 256, 0, (hipStream_t)s>>>(g);
+  return check("gemm");
+}
+
 static int addBias(const mi355_gemm_desc* d, void* c, const void* bias, mi355_stream_t s) {
   if (!bias) return 0;
   const long long total = d->batch0 * d->batch1 * d->M * d->N;
@@ -674,12 +723,7 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
     r = mi355_gemm_bf16_tiled(d, a, b, c, s);
     if (r >= 0) return r ? r : addBias(d, c, bias, s);
   }
-  if (const int t = smallGemmTile(d)) {
-    dim3 grid((unsigned)((d->N + t - 1) / t), (unsigned)((d->M + t - 1) / t), (unsigned)nb);
-    if (t == 16) gemm_f32_small<16><<<grid, 256, 0, (hipStream_t)s>>>(g);
-    else gemm_f32_small<32><<<grid, 256, 0, (hipStream_t)s>>>(g);
-    return check("gemm");
-  }
+  if (smallGemmTile(d)) return mi355_gemm_small_sum(d, a, b, nullptr, nullptr, nullptr, c, bias, s);
   mi355_conv_desc cd;
   // strided views may start anywhere; the implicit-GEMM loaders issue 16-byte loads
   if (gemmAsPointwiseConv(d, &cd) && (((uintptr_t)a | (uintptr_t)b) & 15) == 0) {

@@ -75,6 +75,8 @@ struct Step {
 
   // Gemm / Conv / ScatterRows
   GemmDesc gemm;
+  GemmDesc gemm2;                  // dual: second product summed into the same result; args = [a, b, c, a2, b2]
+  bool dual = false;
   ConvDesc conv;
   ScatterDesc scatter;
   BufRef bias;                     // Gemm: per-column values added to the product (kind None: no bias)

@@ -107,6 +107,7 @@ class Planner {
   std::unordered_set<int> boundToOutput_;
   std::vector<std::pair<int, int>> loops_;
   std::unordered_set<Op*> emitted_;
+  std::unordered_map<Op*, Op*> heldDots_;   // later product of add(dot, dot) -> the earlier one waiting for it
   int time_ = 0;
 
   // ---------------------------------------------------------------- storages
@@ -305,7 +306,22 @@ class Planner {
         continue;
       }
       if (n == "reduce") { if (!tryRowProgram(op, r, pos, plan)) emitReduce(op, r, plan); continue; }
-      if (n == "dot_general" || n == "dot") { emitDot(op, plan); continue; }
+      if (n == "dot_general" || n == "dot") {
+        // add(dot, dot): the earlier product waits for the later one when nothing that writes in place lies between
+        auto held = heldDots_.find(op);
+        if (held != heldDots_.end()) { emitDot(op, plan, held->second); continue; }
+        if (Op* partner = sumPartner(op)) {
+          size_t q = pos + 1;
+          bool clear = true;
+          for (; q < r.ops.size() && r.ops[q].get() != partner; ++q) {
+            const std::string& between = r.ops[q]->name;
+            if (!isFusibleOp(*r.ops[q]) && between != "dot_general" && between != "dot" && between != "reduce" && between != "convolution") clear = false;
+          }
+          if (clear && q < r.ops.size() && !emitted_.count(partner) && !heldDots_.count(partner)) { heldDots_[partner] = op; continue; }
+        }
+        emitDot(op, plan);
+        continue;
+      }
       if (n == "convolution") { emitConv(op, plan); continue; }
       if (n == "scatter") { emitScatter(op, plan); continue; }
       if (n == "dynamic_update_slice") { emitDus(op, plan); continue; }
@@ -782,25 +798,15 @@ class Planner {
     return reshapeStrides(xt.dims, in.strides, v->type.dims, out.strides);
   }
 
-  // the add that emitDot folds into its product as a bias epilogue, or null
+  // the add that emitDot folds into the product of `dot` as a bias epilogue, or null
   static Op* foldedBiasAdd(Op* dot) {
-    static const bool fuseBias = !getenv("MI355X_GEMM_BIAS") || atoi(getenv("MI355X_GEMM_BIAS")) != 0;
-    if (!fuseBias || (dot->name != "dot_general" && dot->name != "dot")) return nullptr;
-    Value* c = dot->result();
-    if (c->users.size() != 1 || c->users[0]->name != "add" || c->users[0]->parent != dot->parent || c->type.numel() == 0 || c->type.rank() == 0) return nullptr;
+    if (dot->name != "dot_general" && dot->name != "dot") return nullptr;
     // exactly one free rhs dim, so that the last result dim is the GEMM's column index
     Value* b = dot->operands[1];
     int64_t used = (int64_t)dot->ints("rhs_batch").size() + (int64_t)dot->ints("rhs_contract").size();
     if (dot->name == "dot") used = 1;
     if (b->type.rank() - used != 1) return nullptr;
-    Op* add = c->users[0];
-    Value* other = add->operands[0] == c ? add->operands[1] : add->operands[0];
-    Op* bc = other->def;
-    if (other == c || !bc || bc->name != "broadcast_in_dim" || bc->parent != dot->parent) return nullptr;
-    Value* bias = bc->operands[0];
-    if (bias->type.rank() != 1 || bias->type.dt != c->type.dt || bias->type.dims[0] != c->type.dims.back()) return nullptr;
-    if (bc->ints("dims") != std::vector<int64_t>{(int64_t)c->type.rank() - 1}) return nullptr;
-    return add;
+    return biasAddOf(dot->result());
   }
 
   // values that are in memory whatever the fusion analysis decides: arguments, results of ops that
@@ -822,7 +828,14 @@ class Planner {
     return resolveView(v, alwaysInMemory, vw);
   }
 
-  void emitDot(Op* op, Plan& plan) {
+  struct DotPlan {
+    GemmDesc g;
+    View va, vb;
+    size_t rhsFreeDims = 0;
+  };
+
+  // materialises or resolves the operands of a dot_general and collapses its dims to one strided batched GEMM
+  DotPlan prepareDot(Op* op, Plan& plan) {
     Value* a = op->operands[0];
     Value* b = op->operands[1];
     Value* c = op->result();
@@ -842,7 +855,8 @@ class Planner {
       if (hasStorage(v)) { vw.root = v; vw.offset = 0; vw.strides = stridesOf(v->type); }
     }
     if (b == a) vb = va;
-    GemmDesc g;
+    DotPlan dp;
+    GemmDesc& g = dp.g;
     g.inType = a->type.dt;
     g.outType = c->type.dt;
     // contraction dims: order both sides by the lhs stride so each side collapses when it can
@@ -876,12 +890,79 @@ class Planner {
       throw CompileError("dot_general: operand layout needs a transposed copy (dims do not collapse to strided 2-D); not supported yet: " + a->type.str() + " x " + b->type.str());
     if (bsz.size() >= 1) { g.batch0 = bsz[0]; g.aB0 = abst[0]; g.bB0 = bbst[0]; }
     if (bsz.size() == 2) { g.batch1 = bsz[1]; g.aB1 = abst[1]; g.bB1 = bbst[1]; }
-    // dot_general -> add(broadcast(bias over the last dim)) with no other reader of the product: the kernels add the
+    dp.va = va;
+    dp.vb = vb;
+    dp.rhsFreeDims = bf.size();
+    return dp;
+  }
+
+  // value-level form of the bias pattern: the add that follows `c` and only adds a broadcast 1-D bias over c's last dim
+  static Op* biasAddOf(Value* c) {
+    static const bool fuseBias = !getenv("MI355X_GEMM_BIAS") || atoi(getenv("MI355X_GEMM_BIAS")) != 0;
+    if (!fuseBias || !c->def || c->users.size() != 1 || c->users[0]->name != "add" || c->users[0]->parent != c->def->parent) return nullptr;
+    if (c->type.numel() == 0 || c->type.rank() == 0) return nullptr;
+    Op* add = c->users[0];
+    Value* other = add->operands[0] == c ? add->operands[1] : add->operands[0];
+    Op* bc = other->def;
+    if (other == c || !bc || bc->name != "broadcast_in_dim" || bc->parent != c->def->parent) return nullptr;
+    Value* bias = bc->operands[0];
+    if (bias->type.rank() != 1 || bias->type.dt != c->type.dt || bias->type.dims[0] != c->type.dims.back()) return nullptr;
+    if (bc->ints("dims") != std::vector<int64_t>{(int64_t)c->type.rank() - 1}) return nullptr;
+    return add;
+  }
+
+  // add(dot_general, dot_general) of two single-use f32 products with one result type: the other product, or null
+  static Op* sumPartner(Op* dot) {
+    static const bool on = !getenv("MI355X_GEMM_SUM") || atoi(getenv("MI355X_GEMM_SUM")) != 0;
+    if (!on || dot->name != "dot_general") return nullptr;
+    Value* c = dot->result();
+    if (c->type.dt != DType::F32 || c->users.size() != 1 || c->users[0]->name != "add" || c->users[0]->parent != dot->parent) return nullptr;
+    Op* add = c->users[0];
+    Value* o = add->operands[0] == c ? add->operands[1] : add->operands[0];
+    if (o == c || !o->def || o->def->name != "dot_general" || o->def->parent != dot->parent || o->users.size() != 1) return nullptr;
+    if (!(o->type == c->type) || o->def->operands[0]->type.dt != DType::F32 || dot->operands[0]->type.dt != DType::F32) return nullptr;
+    return o->def;
+  }
+
+  // `first` (may be null) is an earlier product that was held back because add(first, op) can be one launch
+  void emitDot(Op* op, Plan& plan, Op* first = nullptr) {
+    if (first) {
+      DotPlan d1 = prepareDot(first, plan), d2 = prepareDot(op, plan);
+      mi355_gemm_desc a1 = toAbi(d1.g), a2 = toAbi(d2.g);
+      bool both = mi355_gemm_is_small(&a1) && mi355_gemm_is_small(&a2) && d1.g.M == d2.g.M && d1.g.N == d2.g.N &&
+                  d1.g.batch0 == d2.g.batch0 && d1.g.batch1 == d2.g.batch1;
+      if (!both) {
+        emitDotStep(first, plan, d1, nullptr, nullptr);
+        emitDotStep(op, plan, d2, nullptr, nullptr);
+        return;
+      }
+      emitDotStep(first, plan, d1, op, &d2);
+      return;
+    }
+    DotPlan d = prepareDot(op, plan);
+    emitDotStep(op, plan, d, nullptr, nullptr);
+  }
+
+  void emitDotStep(Op* op, Plan& plan, const DotPlan& dp, Op* second, const DotPlan* dp2) {
+    Value* a = op->operands[0];
+    Value* b = op->operands[1];
+    Value* c = op->result();
+    const GemmDesc& g = dp.g;
+    const View& va = dp.va;
+    const View& vb = dp.vb;
+    // the value the step produces: the product, or the sum of the two products
+    Value* produced = c;
+    Op* sumAdd = nullptr;
+    if (second) {
+      sumAdd = c->users[0];
+      produced = sumAdd->result();
+    }
+    // product -> add(broadcast(bias over the last dim)) with no other reader of the product: the kernels add the
     // bias while they store the result (the reference fuses the same pair into one addmm, passes/fuse_bias_add.cc:120-171)
     Value* biasV = nullptr;
-    Op* biasAdd = foldedBiasAdd(op);
+    Op* biasAdd = dp.rhsFreeDims == 1 ? biasAddOf(produced) : nullptr;
     if (biasAdd) {
-      Value* other = biasAdd->operands[0] == c ? biasAdd->operands[1] : biasAdd->operands[0];
+      Value* other = biasAdd->operands[0] == produced ? biasAdd->operands[1] : biasAdd->operands[0];
       biasV = other->def->operands[0];
       if (!hasStorage(biasV)) {
         if (biasV->def && isFusibleOp(*biasV->def)) materializeNow(biasV, plan);
@@ -889,12 +970,14 @@ class Planner {
       }
     }
     int sid = newStorage(c->type.bytes());
-    bind(c, sid);
+    bind(produced, sid);
+    if (sumAdd) emitted_.insert(sumAdd);
     if (c->type.numel() == 0) return;
     int t = ++time_;
     Step s;
     s.kind = Step::Gemm;
-    s.label = "dot_general " + a->type.str() + " x " + b->type.str() + (biasV ? " + bias" : "");
+    s.label = "dot_general " + a->type.str() + " x " + b->type.str() + (second ? " + " + second->operands[0]->type.str() + " x " + second->operands[1]->type.str() : "") +
+              (biasV ? " + bias" : "");
     s.gemm = g;
     s.args = {ref(storageOf(va.root), t), ref(storageOf(vb.root), t), ref(sid, t)};
     s.args[0].offset = va.offset * (int64_t)dtypeSize(a->type.dt);
@@ -903,6 +986,16 @@ class Planner {
       s.bias = ref(storageOf(biasV), t);
       bind(biasAdd->result(), sid);   // the step writes the sum; nothing reads the bare product
       emitted_.insert(biasAdd);
+    }
+    if (second) {
+      s.gemm2 = dp2->g;
+      s.dual = true;
+      s.args.push_back(ref(storageOf(dp2->va.root), t));
+      s.args.push_back(ref(storageOf(dp2->vb.root), t));
+      s.args[3].offset = dp2->va.offset * 4;
+      s.args[4].offset = dp2->vb.offset * 4;
+      plan.steps.push_back(std::move(s));
+      return;
     }
     // room for a k-contiguous copy of an operand that is laid out along m or n
     mi355_gemm_desc abi = toAbi(g);

@@ -334,7 +334,7 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
   double flops = 0, bytes = 0;
   switch (s.kind) {
     case Step::Kernel: kind = s.label.rfind("reduce", 0) == 0 ? "reduce" : "fusion"; bytes = (double)s.algoBytes; break;
-    case Step::Gemm: kind = "gemm"; flops = 2.0 * s.gemm.batch0 * s.gemm.batch1 * s.gemm.M * s.gemm.N * s.gemm.K; break;
+    case Step::Gemm: kind = "gemm"; flops = 2.0 * s.gemm.batch0 * s.gemm.batch1 * s.gemm.M * s.gemm.N * (s.gemm.K + (s.dual ? s.gemm2.K : 0)); break;
     case Step::Conv: {
       kind = "conv";
       double macs = (double)s.conv.N * s.conv.O * (s.conv.C / s.conv.featureGroups);
@@ -372,8 +372,14 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
     }
     case Step::Gemm: {
       mi355_gemm_desc d = toAbi(s.gemm);
-      void* ws = s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
       const void* bias = s.bias.kind == BufRef::None ? nullptr : resolve(s.bias, in, out);
+      if (s.dual) {
+        mi355_gemm_desc d2 = toAbi(s.gemm2);
+        check(mi355_gemm_small_sum(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), &d2, resolve(s.args[3], in, out),
+                                   resolve(s.args[4], in, out), resolve(s.args[2], in, out), bias, st), "gemm (sum of two products)");
+        break;
+      }
+      void* ws = s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
       check(mi355_gemm(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), bias, ws,
                        (size_t)s.workspaceBytes, st), "gemm");
       break;

@@ -271,6 +271,16 @@ case("dot-bias-product-read-twice", lambda b, x, w, c: (lambda y: b.mul(b.add(y,
      f32(1991, 33, 70), f32(1992, 70, 45), f32(1993, 45))
 
 
+# add(dot, dot) of two small fp32 products is one launch (the recurrent cell's x*Wi + h*Wh), with the bias on top
+case("dot-sum-two-products", lambda b, x, wi, h, wh: b.add(b.matmul(x, wi), b.matmul(h, wh)), f32(2020, 33, 70), f32(2021, 70, 45), f32(2022, 33, 19), f32(2023, 19, 45))
+case("dot-sum-two-products-bias", lambda b, x, wi, h, wh, c: (lambda y: b.add(y, b.broadcast_in_dim(c, y.shape, [1])))(b.add(b.matmul(x, wi), b.matmul(h, wh))),
+     f32(2024, 64, 128), f32(2025, 128, 200), f32(2026, 64, 256), f32(2027, 256, 200), f32(2028, 200))
+case("dot-sum-two-products-work-between", lambda b, x, wi, h, wh: b.add(b.matmul(x, wi), b.matmul(b.tanh(b.add(h, h)), wh)), f32(2029, 33, 70), f32(2030, 70, 45), f32(2031, 33, 19), f32(2032, 19, 45))
+case("dot-sum-two-products-transposed", lambda b, x, wi, h, wh: b.add(b.dot_general(x, wi, ([0], [1])), b.dot_general(h, wh, ([1], [1]))), f32(2033, 70, 33), f32(2034, 45, 70), f32(2035, 33, 19), f32(2036, 45, 19))
+case("dot-sum-one-product-large", lambda b, x, wi, h, wh: b.add(b.matmul(x, wi), b.matmul(h, wh)), f32(2037, 520, 384, lo=-1, hi=1), f32(2038, 384, 1030, lo=-1, hi=1), f32(2039, 520, 16), f32(2040, 16, 1030))
+case("dot-sum-product-read-twice", lambda b, x, wi, h, wh: (lambda p, q: b.mul(b.add(p, q), q))(b.matmul(x, wi), b.matmul(h, wh)), f32(2041, 33, 70), f32(2042, 70, 45), f32(2043, 33, 19), f32(2044, 19, 45))
+
+
 # operands that are slice / reshape / transpose chains over a buffer are read through strides (no copy kernel)
 def _qkv_attention_logits(b, x, w, bias, heads):
     bt, s, _ = x.shape
