@@ -150,14 +150,14 @@ struct SmallArgs {
 };
 
 template <int T>
-__global__ void __launch_bounds__(256) gemm_f32_small(SmallArgs g) {
+__device__ __forceinline__ void smallGemmTileBody(const SmallArgs& g, unsigned bx, unsigned by, unsigned bz) {
   constexpr int KS = T == 16 ? 4 : 2;         // k values per MFMA
   constexpr int NACC = T == 16 ? 4 : 16;
   typedef float accv __attribute__((ext_vector_type(NACC)));
   __shared__ float red[4][T * T];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const long long b0 = blockIdx.z / g.batch1, b1 = blockIdx.z % g.batch1;
-  const long long m0 = (long long)blockIdx.y * T, n0 = (long long)blockIdx.x * T;
+  const long long b0 = bz / g.batch1, b1 = bz % g.batch1;
+  const long long m0 = (long long)by * T, n0 = (long long)bx * T;
   const int r = lane % T, kl = lane / T;
   const bool mOk = m0 + r < g.M, nOk = n0 + r < g.N;
   accv acc = {0};
@@ -198,7 +198,7 @@ __global__ void __launch_bounds__(256) gemm_f32_small(SmallArgs g) {
     red[w][row * T + r] = acc[i];
   }
   __syncthreads();
-  float* C = g.c + (long long)blockIdx.z * g.M * g.N;
+  float* C = g.c + (long long)bz * g.M * g.N;
   for (int e = threadIdx.x; e < T * T; e += 256) {
     const long long row = m0 + e / T, col = n0 + e % T;
     if (row < g.M && col < g.N) {
@@ -206,6 +206,30 @@ __global__ void __launch_bounds__(256) gemm_f32_small(SmallArgs g) {
       C[row * g.N + col] = g.bias ? sum + g.bias[col] : sum;
     }
   }
+}
+
+template <int T>
+__global__ void __launch_bounds__(256) gemm_f32_small(SmallArgs g) {
+  smallGemmTileBody<T>(g, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+// several independent small products in one launch: workgroup b belongs to the problem whose tile range holds b
+constexpr int kMaxSmallGroup = 4;
+struct SmallGroupArgs {
+  SmallArgs prob[kMaxSmallGroup];
+  unsigned first[kMaxSmallGroup + 1];   // first workgroup of each problem
+  unsigned tilesN[kMaxSmallGroup], tilesM[kMaxSmallGroup];
+  int n;
+};
+
+template <int T>
+__global__ void __launch_bounds__(256) gemm_f32_small_group(SmallGroupArgs g) {
+  const unsigned b = blockIdx.x;
+  int p = 0;
+  while (p + 1 < g.n && b >= g.first[p + 1]) ++p;
+  const unsigned local = b - g.first[p];
+  const unsigned tx = local % g.tilesN[p], rest = local / g.tilesN[p];
+  smallGemmTileBody<T>(g.prob[p], tx, rest % g.tilesM[p], rest / g.tilesM[p]);
 }
 
 __global__ void __launch_bounds__(256) gemm_bf16_mfma(GemmArgs g) {
@@ -673,7 +697,50 @@ static SmallPair smallPair(const mi355_gemm_desc* d, const void* a, const void* 
   return p;
 }
 
-int mi355_gemm_is_small(const mi355_gemm_desc* d) { return smallGemmTile(d) != 0; }
+int mi355_gemm_is_small(const mi355_gemm_desc* d) { return smallGemmTile(d); }
+
+static bool fillSmall(SmallArgs& g, const mi355_gemm_desc* d1, const void* a1, const void* b1, const mi355_gemm_desc* d2, const void* a2,
+                      const void* b2, void* c, const void* bias) {
+  if (!smallGemmTile(d1)) return false;
+  if (d2 && (!smallGemmTile(d2) || d2->M != d1->M || d2->N != d1->N || d2->batch0 != d1->batch0 || d2->batch1 != d1->batch1)) return false;
+  g.p[0] = smallPair(d1, a1, b1);
+  g.p[1] = d2 ? smallPair(d2, a2, b2) : g.p[0];
+  g.pairs = d2 ? 2 : 1;
+  g.c = (float*)c;
+  g.bias = (const float*)bias;
+  g.M = d1->M; g.N = d1->N;
+  g.batch1 = (int)d1->batch1;
+  return true;
+}
+
+// n <= 4 independent problems of one tile class (mi355_gemm_is_small gives it), each C = A1 x B1 (+ A2 x B2) (+ bias);
+// d2[i] may be NULL.
+int mi355_gemm_small_group(int n, const mi355_gemm_desc* const* d1, const void* const* a1, const void* const* b1,
+                           const mi355_gemm_desc* const* d2, const void* const* a2, const void* const* b2, void* const* c,
+                           const void* const* bias, mi355_stream_t s) {
+  if (n <= 0) return 0;
+  if (n > kMaxSmallGroup) return -1;
+  SmallGroupArgs g;
+  const int t = smallGemmTile(d1[0]);
+  unsigned total = 0;
+  int k = 0;
+  for (int i = 0; i < n; ++i) {
+    if (smallGemmTile(d1[i]) != t || !fillSmall(g.prob[k], d1[i], a1[i], b1[i], d2[i], a2[i], b2[i], c[i], bias[i])) return -1;
+    const long long nb = d1[i]->batch0 * d1[i]->batch1;
+    if (d1[i]->M <= 0 || d1[i]->N <= 0 || nb <= 0) continue;
+    g.first[k] = total;
+    g.tilesN[k] = (unsigned)((d1[i]->N + t - 1) / t);
+    g.tilesM[k] = (unsigned)((d1[i]->M + t - 1) / t);
+    total += g.tilesN[k] * g.tilesM[k] * (unsigned)nb;
+    ++k;
+  }
+  if (k == 0) return 0;
+  g.first[k] = total;
+  g.n = k;
+  if (t == 16) gemm_f32_small_group<16><<<total, 256, 0, (hipStream_t)s>>>(g);
+  else gemm_f32_small_group<32><<<total, 256, 0, (hipStream_t)s>>>(g);
+  return check("gemm group");
+}
 
 // C = A1 x B1 (+ A2 x B2 when d2 is given: same M, N and batch dims) (+ bias), both products small fp32 ones.
 int mi355_gemm_small_sum(const mi355_gemm_desc* d1, const void* a1, const void* b1, const mi355_gemm_desc* d2, const void* a2,

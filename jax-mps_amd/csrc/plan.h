@@ -62,7 +62,7 @@ struct ScatterDesc {   // row scatter: operand [rows, rowSize...], one index per
 struct Plan;
 
 struct Step {
-  enum Kind { Kernel, Gemm, Conv, ScatterRows, Copy, Fill, While, Case } kind = Kernel;
+  enum Kind { Kernel, Gemm, Conv, ScatterRows, Copy, Fill, While, Case, GemmGroup } kind = Kernel;
   std::string label;  // op name(s) for profiling ranges and error messages
 
   // Kernel
@@ -77,6 +77,7 @@ struct Step {
   GemmDesc gemm;
   GemmDesc gemm2;                  // dual: second product summed into the same result; args = [a, b, c, a2, b2]
   bool dual = false;
+  std::vector<Step> parts;         // GemmGroup: independent small products launched together (each a Gemm step)
   ConvDesc conv;
   ScatterDesc scatter;
   BufRef bias;                     // Gemm: per-column values added to the product (kind None: no bias)

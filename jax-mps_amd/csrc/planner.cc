@@ -90,6 +90,7 @@ class Planner {
       }
     }
     static const bool batching = !getenv("MI355X_BATCH_KERNELS") || atoi(getenv("MI355X_BATCH_KERNELS")) != 0;
+    groupSmallGemms(P.plan);
     if (batching) batchKernels(P.plan);
     assignArena();
     patch(P.plan);
@@ -976,6 +977,7 @@ class Planner {
     int t = ++time_;
     Step s;
     s.kind = Step::Gemm;
+    s.time = t;
     s.label = "dot_general " + a->type.str() + " x " + b->type.str() + (second ? " + " + second->operands[0]->type.str() + " x " + second->operands[1]->type.str() : "") +
               (biasV ? " + bias" : "");
     s.gemm = g;
@@ -1433,6 +1435,65 @@ class Planner {
     steps = std::move(out);
   }
 
+  // Consecutive small fp32 products that do not depend on each other (the weight and input gradients of a
+  // recurrent step, say) share one launch.
+  static int smallClass(const Step& s) {
+    if (s.kind != Step::Gemm || s.workspaceBytes != 0 || s.gemm.inType != DType::F32 || s.gemm.outType != DType::F32) return 0;
+    mi355_gemm_desc d = toAbi(s.gemm);
+    int t = mi355_gemm_is_small(&d);
+    if (t && s.dual) { mi355_gemm_desc d2 = toAbi(s.gemm2); if (mi355_gemm_is_small(&d2) == 0) return 0; }
+    return t;
+  }
+
+  static bool gemmsIndependent(const Step& a, const Step& b) {
+    auto reads = [](const Step& s) {
+      std::vector<int> r{s.args[0].index, s.args[1].index};
+      if (s.dual) { r.push_back(s.args[3].index); r.push_back(s.args[4].index); }
+      if (s.bias.kind != BufRef::None) r.push_back(s.bias.index);
+      return r;
+    };
+    const int wa = a.args[2].index, wb = b.args[2].index;
+    if (wa == wb) return false;
+    for (int x : reads(a)) if (x == wb) return false;
+    for (int x : reads(b)) if (x == wa) return false;
+    return true;
+  }
+
+  void groupSmallGemms(Plan& plan) {
+    static const bool on = !getenv("MI355X_GEMM_GROUPS") || atoi(getenv("MI355X_GEMM_GROUPS")) != 0;
+    if (!on) return;
+    std::vector<Step> out;
+    auto& steps = plan.steps;
+    size_t i = 0;
+    while (i < steps.size()) {
+      for (auto& b : steps[i].bodies) groupSmallGemms(*b);
+      const int cls = smallClass(steps[i]);
+      size_t j = i + 1;
+      if (cls) {
+        while (j < steps.size() && j - i < 4 && smallClass(steps[j]) == cls) {
+          bool ok = true;
+          for (size_t k = i; k < j && ok; ++k) ok = gemmsIndependent(steps[k], steps[j]);
+          if (!ok) break;
+          ++j;
+        }
+      }
+      if (j - i < 2) { out.push_back(std::move(steps[i++])); continue; }
+      Step m;
+      m.kind = Step::GemmGroup;
+      m.time = steps[i].time;
+      m.label = "small products x" + std::to_string(j - i);
+      const int tFirst = steps[i].time, tLast = steps[j - 1].time;
+      for (size_t k = i; k < j; ++k) {
+        for (auto& a : steps[k].args) { ref(a.index, tFirst); ref(a.index, tLast); }
+        if (steps[k].bias.kind != BufRef::None) { ref(steps[k].bias.index, tFirst); ref(steps[k].bias.index, tLast); }
+        m.parts.push_back(std::move(steps[k]));
+      }
+      out.push_back(std::move(m));
+      i = j;
+    }
+    steps = std::move(out);
+  }
+
   // ---------------------------------------------------------------- arena
   void assignArena() {
     // a buffer that is used inside a loop but defined outside it lives until the loop ends
@@ -1480,6 +1541,10 @@ class Planner {
 
   void patch(Plan& plan) {
     for (auto& s : plan.steps) {
+      for (auto& part : s.parts) {
+        for (auto& a : part.args) a = finalRef(a);
+        part.bias = finalRef(part.bias);
+      }
       for (auto& a : s.args) a = finalRef(a);
       s.src = finalRef(s.src);
       s.dst = finalRef(s.dst);
@@ -1502,7 +1567,7 @@ class Planner {
 
   void dumpPlan(const Plan& p, int indent) {
     std::ostringstream o;
-    static const char* kinds[] = {"kernel", "gemm", "conv", "scatter", "copy", "fill", "while", "case"};
+    static const char* kinds[] = {"kernel", "gemm", "conv", "scatter", "copy", "fill", "while", "case", "gemm-group"};
     for (auto& s : p.steps) {
       o << std::string(indent, ' ') << kinds[s.kind] << " " << s.label;
       if (s.kind == Step::Kernel) o << " k" << s.kernel << " grid " << s.grid[0] << "x" << s.grid[1] << " bytes " << s.algoBytes;
@@ -1512,6 +1577,7 @@ class Planner {
       o.str("");
       if (s.cond) dumpPlan(*s.cond, indent + 2);
       for (auto& b : s.bodies) dumpPlan(*b, indent + 2);
+      for (auto& part : s.parts) { P.dump += std::string(indent + 2, ' ') + part.label + "\n"; }
     }
   }
 };

@@ -335,6 +335,10 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
   switch (s.kind) {
     case Step::Kernel: kind = s.label.rfind("reduce", 0) == 0 ? "reduce" : "fusion"; bytes = (double)s.algoBytes; break;
     case Step::Gemm: kind = "gemm"; flops = 2.0 * s.gemm.batch0 * s.gemm.batch1 * s.gemm.M * s.gemm.N * (s.gemm.K + (s.dual ? s.gemm2.K : 0)); break;
+    case Step::GemmGroup:
+      kind = "gemm";
+      for (auto& part : s.parts) flops += 2.0 * part.gemm.batch0 * part.gemm.batch1 * part.gemm.M * part.gemm.N * (part.gemm.K + (part.dual ? part.gemm2.K : 0));
+      break;
     case Step::Conv: {
       kind = "conv";
       double macs = (double)s.conv.N * s.conv.O * (s.conv.C / s.conv.featureGroups);
@@ -382,6 +386,30 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       void* ws = s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
       check(mi355_gemm(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), bias, ws,
                        (size_t)s.workspaceBytes, st), "gemm");
+      break;
+    }
+    case Step::GemmGroup: {
+      const int n = (int)s.parts.size();
+      mi355_gemm_desc d1[4], d2[4];
+      const mi355_gemm_desc *p1[4], *p2[4];
+      const void *a1[4], *b1[4], *a2[4], *b2[4], *bias[4];
+      void* c[4];
+      if (n > 4) throw RuntimeError("gemm group of more than 4 products");
+      for (int i = 0; i < n; ++i) {
+        const Step& part = s.parts[(size_t)i];
+        d1[i] = toAbi(part.gemm);
+        p1[i] = &d1[i];
+        a1[i] = resolve(part.args[0], in, out); b1[i] = resolve(part.args[1], in, out); c[i] = resolve(part.args[2], in, out);
+        if (part.dual) {
+          d2[i] = toAbi(part.gemm2);
+          p2[i] = &d2[i];
+          a2[i] = resolve(part.args[3], in, out); b2[i] = resolve(part.args[4], in, out);
+        } else {
+          p2[i] = nullptr; a2[i] = nullptr; b2[i] = nullptr;
+        }
+        bias[i] = part.bias.kind == BufRef::None ? nullptr : resolve(part.bias, in, out);
+      }
+      check(mi355_gemm_small_group(n, p1, a1, b1, p2, a2, b2, c, bias, st), "gemm group");
       break;
     }
     case Step::Conv: {
@@ -468,7 +496,7 @@ bool Executable::capturable(const Plan& p) {
   bool ok = true;
   for (auto& s : p.steps) {
     switch (s.kind) {
-      case Step::Kernel: case Step::Gemm: case Step::Conv: case Step::ScatterRows: case Step::Copy: case Step::Fill: break;
+      case Step::Kernel: case Step::Gemm: case Step::GemmGroup: case Step::Conv: case Step::ScatterRows: case Step::Copy: case Step::Fill: break;
       case Step::While: ok = ok && s.tripCount >= 0 && capturable(*s.bodies[0]); break;   // dynamic loops read a flag back on the host
       default: ok = false; break;
     }
@@ -497,6 +525,7 @@ void Executable::runCountedLoop(const Step& s, const std::vector<DeviceBuffer*>&
       auto add = [&](const BufRef& b) { if (b.kind == BufRef::Param || b.kind == BufRef::Output) lgs.external.push_back(b); };
       for (auto& st : p.steps) {
         for (auto& a : st.args) add(a);
+        for (auto& part : st.parts) { for (auto& a : part.args) add(a); add(part.bias); }
         add(st.src); add(st.dst); add(st.predBuf); add(st.bias);
         if (st.cond) scan(*st.cond);
         for (auto& b : st.bodies) scan(*b);

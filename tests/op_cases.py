@@ -281,6 +281,12 @@ case("dot-sum-one-product-large", lambda b, x, wi, h, wh: b.add(b.matmul(x, wi),
 case("dot-sum-product-read-twice", lambda b, x, wi, h, wh: (lambda p, q: b.mul(b.add(p, q), q))(b.matmul(x, wi), b.matmul(h, wh)), f32(2041, 33, 70), f32(2042, 70, 45), f32(2043, 33, 19), f32(2044, 19, 45))
 
 
+# independent small products next to each other share one launch (the gradients of one recurrent step)
+case("dot-group-three-independent", lambda b, dz, wh, h, x: [b.dot_general(dz, wh, ([1], [1])), b.dot_general(h, dz, ([0], [0])), b.dot_general(x, dz, ([0], [0]))],
+     f32(2050, 20, 96), f32(2051, 40, 96), f32(2052, 20, 40), f32(2053, 20, 24))
+case("dot-group-second-reads-first", lambda b, x, w1, w2: (lambda y: [y, b.matmul(y, w2)])(b.matmul(x, w1)), f32(2054, 20, 30), f32(2055, 30, 40), f32(2056, 40, 10))
+
+
 # operands that are slice / reshape / transpose chains over a buffer are read through strides (no copy kernel)
 def _qkv_attention_logits(b, x, w, bias, heads):
     bt, s, _ = x.shape
