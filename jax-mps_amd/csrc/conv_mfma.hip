@@ -270,6 +270,7 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
     for (int kt = ktBegin; kt < ktEnd; ++kt) {
       const bool more = kt + 1 < ktEnd;
       if (more) loadTile(kt + 1);          // global loads in flight while this tile is multiplied
+      __builtin_amdgcn_s_setprio(2);       // a wavefront that has its operands wins the matrix pipe over ones still fetching
 #pragma unroll
       for (int kk = 0; kk < BK; kk += 2) {
         float av[TM], bv[TN];
@@ -282,6 +283,7 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
 #pragma unroll
           for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[a], bv[b], acc[a][b], 0, 0, 0);
       }
+      __builtin_amdgcn_s_setprio(0);
       if (more) storeTile(cur ^ 1);         // the other stage: nobody reads it during this iteration
       __syncthreads();
       cur ^= 1;
