@@ -983,6 +983,18 @@ class Parser {
       fnType(op, outs);
       return;
     }
+    if (n == "rng_bit_generator") {
+      // %state, %bits = stablehlo.rng_bit_generator %state0, algorithm = THREE_FRY : (tensor<2xui64>) -> (tensor<2xui64>, tensor<8xui32>)
+      op->operands = ssaUseList();
+      expect(",");
+      expect("algorithm");
+      expect("=");
+      setStr(op, "rng_algorithm", ident());
+      if (peekc() == '{') skipBalanced('{', '}');
+      expect(":");
+      fnType(op, outs);
+      return;
+    }
     if (n == "optimization_barrier") {
       if (peekc() == '%') op->operands = ssaUseList();
       expect(":");

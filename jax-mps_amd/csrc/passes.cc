@@ -814,7 +814,109 @@ void lowerWindowOpsIn(Region& r, int& nextId) {
   }
 }
 
+
+// stablehlo.rng_bit_generator -> plain integer ops.  The bits are implementation-defined by the specification
+// (the reference draws them from MLX's generator and says so, src/pjrt_plugin/ops/control_flow.cc:2301-2360); what
+// callers rely on is the state rule the reference keeps: state = [key, counter] as ui64[2], the counter grows by
+// ceil(output bytes / 16).  Here element i of the output is word 0 (and word 1 for 64-bit types) of
+// threefry2x32(key = the two halves of state[0], counter = (i, low half of state[1])), which the planner fuses
+// into one kernel like any other integer chain.
+void lowerRngIn(Region& r, int& nextId) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) lowerRngIn(*sub, nextId);
+    if (op->name != "rng_bit_generator") continue;
+    if (op->operands.size() != 1 || op->results.size() != 2) throw CompileError("stablehlo.rng_bit_generator: expected one state operand and two results");
+    Value* state = op->operands[0];
+    const TensorType st = state->type;
+    const TensorType ot = op->results[1]->type;
+    if (st.dt != DType::U64 || st.rank() != 1 || st.dims[0] < 2 || !(op->results[0]->type == st))
+      throw CompileError("stablehlo.rng_bit_generator: the state must be tensor<Nxui64> with N >= 2, got " + st.str());
+    const size_t esz = dtypeSize(ot.dt);
+    if (!(isInt(ot.dt) || ot.dt == DType::U8 || ot.dt == DType::U16 || ot.dt == DType::U32 || ot.dt == DType::U64) || ot.numel() >= (int64_t(1) << 32))
+      throw CompileError("stablehlo.rng_bit_generator: unsupported output type " + ot.str());
+    Rewriter rw{r, nextId, op->line, {}};
+    auto ty = [](DType dt, std::vector<int64_t> dims) { TensorType t; t.dt = dt; t.dims = std::move(dims); return t; };
+    const int64_t N = st.dims[0];
+    // ---- new state: counter (element 1) + ceil(bytes / 16)
+    const uint64_t incr = ((uint64_t)ot.numel() * esz + 15) / 16;
+    Value* head = rw.slice(state, {0}, {1}, {1});
+    Value* ctr = rw.slice(state, {1}, {1}, {1});
+    Value* ctrNew = rw.binary("add", ctr, rw.splat(DType::U64, {1}, &incr), ty(DType::U64, {1}));
+    std::vector<Value*> parts{head, ctrNew};
+    if (N > 2) parts.push_back(rw.slice(state, {2}, {N - 2}, {1}));
+    auto cat = makeOp("concatenate", parts, &r, op->line);
+    Attr dimA;
+    dimA.kind = Attr::Int;
+    dimA.i = 0;
+    cat->attrs["dim"] = dimA;
+    // ---- bits
+    const TensorType u32t = ty(DType::U32, ot.dims), u64s = ty(DType::U64, {}), u32s = ty(DType::U32, {});
+    auto scalarOf = [&](Value* one) { return rw.unary("reshape", one, u64s); };
+    const uint64_t sh32 = 32;
+    Value* key64 = scalarOf(head);
+    Value* ctr64 = scalarOf(ctr);
+    Value* k0s = rw.unary("convert", key64, u32s);
+    Value* k1s = rw.unary("convert", rw.binary("shift_right_logical", key64, rw.splat(DType::U64, {}, &sh32), u64s), u32s);
+    Value* c1s = rw.unary("convert", ctr64, u32s);
+    Value* k0 = rw.broadcastScalar(k0s, u32t);
+    Value* k1 = rw.broadcastScalar(k1s, u32t);
+    Value* c1 = rw.broadcastScalar(c1s, u32t);
+    // element index: iota over the flattened output, reshaped to the output dims
+    auto io = makeOp("iota", {}, &r, op->line);
+    Attr zero;
+    zero.kind = Attr::Int;
+    zero.i = 0;
+    io->attrs["dim"] = zero;
+    Value* flat = rw.emit(std::move(io), ty(DType::U32, {ot.numel()}));
+    Value* c0 = ot.rank() == 1 ? flat : rw.unary("reshape", flat, u32t);
+    auto cu = [&](uint32_t x) { return rw.splat(DType::U32, ot.dims, &x); };
+    auto bin = [&](const char* n, Value* a, Value* b) { return rw.binary(n, a, b, u32t); };
+    auto rotl = [&](Value* x, uint32_t rbits) { return bin("or", bin("shift_left", x, cu(rbits)), bin("shift_right_logical", x, cu(32 - rbits))); };
+    Value* ks[3] = {k0, k1, bin("xor", bin("xor", k0, k1), cu(0x1BD11BDAu))};
+    Value* x0 = bin("add", c0, ks[0]);
+    Value* x1 = bin("add", c1, ks[1]);
+    static const uint32_t rots[2][4] = {{13, 15, 26, 6}, {17, 29, 16, 24}};
+    for (uint32_t blk = 0; blk < 5; ++blk) {
+      for (uint32_t rr : rots[blk % 2]) {
+        x0 = bin("add", x0, x1);
+        x1 = bin("xor", rotl(x1, rr), x0);
+      }
+      x0 = bin("add", x0, ks[(blk + 1) % 3]);
+      x1 = bin("add", bin("add", x1, ks[(blk + 2) % 3]), cu(blk + 1));
+    }
+    std::unique_ptr<Op> last;
+    if (esz == 8) {
+      const TensorType u64t = ty(DType::U64, ot.dims);
+      Value* lo = rw.unary("convert", x0, u64t);
+      Value* hi = rw.binary("shift_left", rw.unary("convert", x1, u64t), rw.splat(DType::U64, ot.dims, &sh32), u64t);
+      Value* both = rw.binary("or", lo, hi, u64t);
+      last = makeOp(ot.dt == DType::U64 ? "reshape" : "bitcast_convert", {both}, &r, op->line);
+    } else {
+      last = makeOp(ot.dt == DType::U32 ? "reshape" : (esz == 4 ? "bitcast_convert" : "convert"), {x0}, &r, op->line);
+    }
+    // the two results move to the two final ops
+    cat->results.push_back(std::move(op->results[0]));
+    cat->results[0]->def = cat.get();
+    last->results.push_back(std::move(op->results[1]));
+    last->results[0]->def = last.get();
+    rw.made.push_back(std::move(cat));
+    rw.made.push_back(std::move(last));
+    size_t nIns = rw.made.size();
+    r.ops.erase(r.ops.begin() + k);
+    r.ops.insert(r.ops.begin() + k, std::make_move_iterator(rw.made.begin()), std::make_move_iterator(rw.made.end()));
+    k += nIns - 1;
+  }
+}
+
 }  // namespace
+
+void lowerRng(Module& m) {
+  Func* f = m.main();
+  if (!f) return;
+  int nextId = maxValueId(f->body) + 1;
+  lowerRngIn(f->body, nextId);
+}
 
 void lowerWindowOps(Module& m) {
   Func* f = m.main();

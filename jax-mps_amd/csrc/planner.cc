@@ -1625,6 +1625,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   lowerIntegerDots(*module);
   lowerGeneralScatters(*module);
   lowerWindowOps(*module);
+  lowerRng(*module);
   checkSupported(*module);
   eliminateDeadCode(module->main()->body);
   prog->module = std::move(module);

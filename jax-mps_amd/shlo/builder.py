@@ -809,6 +809,13 @@ class Builder:
         self._emit(f"}}) : ({operand.type}, {source.type}, {st}) -> {v.type}")
         return v
 
+    def rng_bit_generator(self, state: Val, shape, dtype="ui32", algorithm="DEFAULT"):
+        """`jax.random.bits` under the rbg / unsafe_rbg PRNG implementations: (new state, bits)."""
+        name = self._fresh()
+        shape = tuple(int(x) for x in shape)
+        self._emit(f"{name}:2 = stablehlo.rng_bit_generator {state.name}, algorithm = {algorithm} : ({state.type}) -> ({state.type}, {ttype(shape, dtype)})")
+        return Val(self, f"{name}#0", state.shape, state.dtype, self._blk), Val(self, f"{name}#1", shape, dtype, self._blk)
+
     def take_rows(self, table: Val, idx: Val) -> Val:
         """`jnp.take(table, idx, axis=0)` in the default (fill) mode: negative
         indices wrap, then rows outside [0, n) read as NaN (the mask JAX adds

@@ -607,6 +607,15 @@ class _P:
             self.expect(":")
             self.fn_type(op)
             return
+        if short == "rng_bit_generator":
+            op.operands = self.ssa_list()
+            self.expect(",")
+            self.expect("algorithm")
+            self.expect("=")
+            op.attrs["rng_algorithm"] = self.ident()
+            self.expect(":")
+            self.fn_type(op)
+            return
         if short == "optimization_barrier":
             op.operands = self.ssa_list() if self.peek("%") else []
             self.expect(":")
@@ -1607,11 +1616,56 @@ class Oracle:
 
     def op_optimization_barrier(self, op, ins, env): return list(ins)
 
+    def op_rng_bit_generator(self, op, ins, env):
+        """State rule of the reference (src/pjrt_plugin/ops/control_flow.cc:2301-2360): state = [key, counter, ...] as
+        ui64, the counter grows by ceil(output bytes / 16).  The bits themselves are implementation-defined (the
+        reference takes MLX's); this build defines element i as threefry2x32(key halves; (i, low half of the counter)),
+        word 0 for types up to 32 bits (truncated), both words for 64-bit types.  PARITY UNPINNED for the bit values."""
+        state = np.asarray(ins[0], dtype=np.uint64)
+        t = op.out_types[1]
+        n = int(np.prod(t.shape, dtype=np.int64))
+        dt = _NP[t.dtype]
+        esz = np.dtype(dt).itemsize
+        new_state = state.copy()
+        new_state[1] = np.uint64((int(state[1]) + (n * esz + 15) // 16) & ((1 << 64) - 1))
+        k0 = np.uint32(int(state[0]) & 0xFFFFFFFF)
+        k1 = np.uint32(int(state[0]) >> 32)
+        c0 = np.arange(n, dtype=np.uint32)
+        c1 = np.full(n, int(state[1]) & 0xFFFFFFFF, dtype=np.uint32)
+        x0, x1 = threefry2x32(k0, k1, c0, c1)
+        if esz == 8:
+            bits = (x0.astype(np.uint64) | (x1.astype(np.uint64) << np.uint64(32))).view(dt)
+        elif esz == 4:
+            bits = x0.view(dt)
+        else:
+            bits = x0.astype(np.dtype("u%d" % esz)).view(dt)
+        return [new_state, bits.reshape(t.shape)]
+
     def op_custom_call(self, op, ins, env):
         tgt = op.attrs.get("call_target_name")
         if tgt in ("Sharding", "SPMDFullToShardShape", "SPMDShardToFullShape"):
             return ins[0]
         raise NotImplementedError(f"oracle: custom_call {tgt}")
+
+
+def threefry2x32(k0, k1, c0, c1):
+    """Threefry-2x32 with 20 rounds (Salmon et al., Random123), on uint32 arrays; checked against the published
+    known-answer vectors in tests/test_oracle_pins.py."""
+    with np.errstate(over="ignore"):
+        k0 = np.asarray(k0, np.uint32); k1 = np.asarray(k1, np.uint32)
+        x0 = np.asarray(c0, np.uint32).copy(); x1 = np.asarray(c1, np.uint32).copy()
+        ks = [k0, k1, k0 ^ k1 ^ np.uint32(0x1BD11BDA)]
+        rotl = lambda x, r: (x << np.uint32(r)) | (x >> np.uint32(32 - r))
+        x0 = x0 + ks[0]
+        x1 = x1 + ks[1]
+        rots = [(13, 15, 26, 6), (17, 29, 16, 24)]
+        for blk in range(5):
+            for r in rots[blk % 2]:
+                x0 = x0 + x1
+                x1 = rotl(x1, r) ^ x0
+            x0 = x0 + ks[(blk + 1) % 3]
+            x1 = x1 + ks[(blk + 2) % 3] + np.uint32(blk + 1)
+        return x0, x1
 
 
 def run_text(text: str, *args, accum="f64"):

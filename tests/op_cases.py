@@ -490,6 +490,21 @@ def get_case(name: str) -> Case:
     raise KeyError(name)
 
 
+# ------------------------------------------------------------------ rng_bit_generator: counter update as the reference
+# keeps it (src/pjrt_plugin/ops/control_flow.cc:2343-2355); bits = threefry2x32 of (key halves; element index, counter)
+_RNG_STATE = np.array([0x0123456789ABCDEF, 41], dtype=np.uint64)
+case("rng-bits-u32", lambda b, st: list(b.rng_bit_generator(st, (1000,), "ui32", "THREE_FRY")), _RNG_STATE, exact=True)
+case("rng-bits-u32-2d-default", lambda b, st: list(b.rng_bit_generator(st, (7, 33), "ui32")), _RNG_STATE, exact=True)
+case("rng-bits-u64", lambda b, st: list(b.rng_bit_generator(st, (129,), "ui64", "PHILOX")), _RNG_STATE, exact=True)
+case("rng-bits-u8", lambda b, st: list(b.rng_bit_generator(st, (50,), "ui8")), _RNG_STATE, exact=True)
+case("rng-bits-i32", lambda b, st: list(b.rng_bit_generator(st, (64,), "i32")), _RNG_STATE, exact=True)
+case("rng-bits-chained", lambda b, st: (lambda s1, b1: (lambda s2, b2: [s2, b1, b2])(*b.rng_bit_generator(s1, (16,), "ui32")))(*b.rng_bit_generator(st, (16,), "ui32")),
+     np.array([7, 0xFFFFFFFFFFFFFFFF], dtype=np.uint64), exact=True)
+case("rng-uniform-floats", lambda b, st: (lambda s1, bits: b.sub(b.bitcast_convert(b.or_(b.shift_right_logical(bits, b.constant(np.uint32(9), "ui32", bits.shape)),
+                                                                                        b.constant(np.uint32(0x3F800000), "ui32", bits.shape)), "f32"),
+                                                               b.constant(np.float32(1), "f32", bits.shape)))(*b.rng_bit_generator(st, (4096,), "ui32")), _RNG_STATE, exact=True)
+
+
 # ------------------------------------------------------------------ threefry2x32 as JAX lowers it without a custom call:
 # plain ui32 adds, xors and rotations (reference kernel text: src/pjrt_plugin/ops/control_flow.cc:1351-1390); the whole
 # block cipher fuses into one generated kernel.  Inputs are the Random123 known-answer vectors.

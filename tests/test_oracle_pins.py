@@ -315,6 +315,38 @@ def test_threefry2x32_known_answer_vectors():
     assert np.array_equal(out[1], op_cases.THREEFRY_KAT["out1"])
 
 
+def test_rng_bit_generator_state_rule_and_bits():
+    """State: key unchanged, counter += ceil(output bytes / 16) (reference: src/pjrt_plugin/ops/control_flow.cc:2343-2355),
+    wrapping at 2^64.  Bits: the oracle's threefry helper reproduces the Random123 known answers, element i of a draw is
+    threefry(key halves; (i, counter low half)), and the stream looks uniform (bit balance, byte chi-square)."""
+    import op_cases
+    import shlo_oracle
+    kat = op_cases.THREEFRY_KAT
+    x0, x1 = shlo_oracle.threefry2x32(kat["key0"], kat["key1"], kat["ctr0"], kat["ctr1"])
+    assert np.array_equal(x0, kat["out0"]) and np.array_equal(x1, kat["out1"])
+    for name, nbytes in (("rng-bits-u32", 4000), ("rng-bits-u64", 129 * 8), ("rng-bits-u8", 50), ("rng-bits-u32-2d-default", 7 * 33 * 4)):
+        c = op_cases.get_case(name)
+        state, bits = Oracle(c.text).run(*c.inputs)
+        assert state[0] == c.inputs[0][0] and int(state[1]) == int(c.inputs[0][1]) + (nbytes + 15) // 16, name
+    c = op_cases.get_case("rng-bits-chained")
+    s2, b1, b2 = Oracle(c.text).run(*c.inputs)
+    assert int(s2[0]) == 7 and int(s2[1]) == 7            # key untouched; counter (2^64 - 1) + 4 + 4 wraps to 7
+    assert not np.array_equal(b1, b2)                      # the second draw uses the advanced counter
+    c = op_cases.get_case("rng-bits-u32")
+    _, bits = Oracle(c.text).run(*c.inputs)
+    k0, k1 = np.uint32(0x89ABCDEF), np.uint32(0x01234567)
+    want, _ = shlo_oracle.threefry2x32(k0, k1, np.arange(1000, dtype=np.uint32), np.full(1000, 41, np.uint32))
+    assert np.array_equal(bits, want)
+    ones = np.unpackbits(bits.view(np.uint8)).mean()
+    assert abs(ones - 0.5) < 0.01
+    counts = np.bincount(bits.view(np.uint8), minlength=256)
+    chi2 = ((counts - counts.mean()) ** 2 / counts.mean()).sum()
+    assert chi2 < 340                                      # 255 degrees of freedom: P(chi2 > 340) < 3e-4
+    c = op_cases.get_case("rng-uniform-floats")
+    u = Oracle(c.text).run(*c.inputs)[0]
+    assert u.min() >= 0.0 and u.max() < 1.0 and abs(u.mean() - 0.5) < 0.02 and abs(u.var() - 1 / 12) < 0.01
+
+
 def test_pooling_against_torch():
     """reduce_window (max / sum) and select_and_scatter (gradient of max pooling, first maximum wins) against
     torch.nn.functional.max_pool2d / avg_pool2d and torch autograd, NHWC <-> NCHW."""
