@@ -1762,6 +1762,123 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
   fc.launches.push_back(std::move(l));
   return fc;
 }
+// stablehlo.sort: one workgroup per slice along the sorted dim.  The operands of the slice are staged in LDS
+// and a permutation is sorted by a bitonic network whose order is "comparator(a, b), else not comparator(b, a)
+// and a came first", a strict total order, so the result is the stable sort whatever network produces it
+// (reference: src/pjrt_plugin/ops/sort_fft_complex.cc:145-216, which sorts by the first operand only; here the
+// comparator region itself is compiled, so multi-key and custom orders work).
+int64_t sortLdsBytes(Op* sort) {
+  int64_t L = sort->operands[0]->type.dims.empty() ? 1 : sort->operands[0]->type.dims[(size_t)sort->integer("dimension")];
+  int64_t P = 1;
+  while (P < L) P <<= 1;
+  int64_t per = 4;
+  for (auto* o : sort->operands) per += (int64_t)dtypeSize(o->type.dt);
+  return P * per;
+}
+
+FusedCode generateSortKernel(Op* sort, const LeafPredicate& isLeaf) {
+  const size_t n = sort->operands.size();
+  if (n == 0 || sort->results.size() != n || sort->regions.size() != 1) throw CompileError("stablehlo.sort: malformed operands");
+  Region& body = *sort->regions[0];
+  if (body.args.size() != 2 * n || !body.terminator() || body.terminator()->operands.size() != 1)
+    throw CompileError("stablehlo.sort: the comparator region does not match the operands");
+  for (auto& op : body.ops)
+    if (op->name != "return" && (!isFusibleOp(*op) || op->results.size() != 1 || !op->regions.empty()))
+      throw CompileError("stablehlo.sort: comparator op stablehlo." + op->name + " is not supported");
+  const TensorType& t0 = sort->operands[0]->type;
+  for (auto* o : sort->operands) if (o->type.dims != t0.dims) throw CompileError("stablehlo.sort: operands of different shapes");
+  const int rank = t0.rank();
+  int64_t dim = rank == 0 ? 0 : sort->integer("dimension");
+  if (dim < 0) dim += rank;
+  int64_t L = rank == 0 ? 1 : t0.dims[(size_t)dim], inner = 1, outer = 1;
+  for (int d = 0; d < rank; ++d) { if (d < dim) outer *= t0.dims[(size_t)d]; if (d > dim) inner *= t0.dims[(size_t)d]; }
+  int64_t P = 1;
+  while (P < L) P <<= 1;
+  // slices too long for LDS are sorted in place in a workspace by the same network, one workgroup per slice
+  // (values are read from the operands through the permutation; slower, but any length works)
+  const bool inLds = sortLdsBytes(sort) <= 60 * 1024;
+  if (t0.numel() >= (int64_t(1) << 31) || outer * inner * P >= (int64_t(1) << 31)) throw CompileError("stablehlo.sort: tensor too large");
+
+  // comparator as straight-line code over named scalars
+  Emitter b(isLeaf, 1, false);
+  for (size_t j = 0; j < n; ++j) {
+    b.rowScalars_[body.args[2 * j].get()] = "ca" + std::to_string(j);
+    b.rowScalars_[body.args[2 * j + 1].get()] = "cb" + std::to_string(j);
+  }
+  std::string res = b.gen(body.terminator()->operands[0], b.multiIndex({}, {}));
+  if (!b.leaves_.empty()) throw CompileError("stablehlo.sort: the comparator reads values defined outside it");
+
+  std::ostringstream s;
+  s << "  const int row = blockIdx.x;\n";
+  s << "  const int base = (row / " << inner << ") * " << (L * inner) << " + (row % " << inner << ");\n";
+  if (inLds) {
+    for (size_t j = 0; j < n; ++j) s << "  __shared__ " << storageT(sort->operands[j]->type.dt) << " sv" << j << "[" << P << "];\n";
+    s << "  __shared__ int perm[" << P << "];\n";
+  } else {
+    s << "  int* perm = work + (long long)row * " << P << ";\n";
+  }
+  s << "  for (int e = threadIdx.x; e < " << P << "; e += 256) {\n";
+  s << "    perm[e] = e;\n";
+  if (inLds) {
+    s << "    if (e < " << L << ") {\n";
+    for (size_t j = 0; j < n; ++j) s << "      sv" << j << "[e] = in" << j << "[base + e * " << inner << "];\n";
+    s << "    }\n";
+  }
+  s << "  }\n  __syncthreads();\n";
+  auto elem = [&](size_t j, const std::string& i) {
+    return inLds ? "sv" + std::to_string(j) + "[" + i + "]" : "in" + std::to_string(j) + "[base + " + i + " * " + std::to_string(inner) + "]";
+  };
+  // before(a, b): a sorts strictly before b
+  s << "  auto cmp = [&](int a, int b) -> bool {\n";
+  for (size_t j = 0; j < n; ++j) {
+    DType dt = sort->operands[j]->type.dt;
+    s << "    const " << computeT(dt) << " ca" << j << " = " << loadExpr(dt, elem(j, "a")) << ";\n";
+    s << "    const " << computeT(dt) << " cb" << j << " = " << loadExpr(dt, elem(j, "b")) << ";\n";
+  }
+  s << "    const int v = 0; (void)v;\n";
+  s << b.pre_;
+  s << "    return " << res << ";\n  };\n";
+  s << "  auto before = [&](int a, int b) -> bool {\n";
+  s << "    if (a >= " << L << " || b >= " << L << ") return a < b;   // padding sorts last\n";
+  s << "    if (cmp(a, b)) return true;\n";
+  s << "    if (cmp(b, a)) return false;\n";
+  s << "    return a < b;\n  };\n";
+  s << "  for (int k = 2; k <= " << P << "; k <<= 1) {\n";
+  s << "    for (int j = k >> 1; j > 0; j >>= 1) {\n";
+  s << "      for (int t = threadIdx.x; t < " << (P / 2) << "; t += 256) {\n";
+  s << "        const int i = ((t / j) * 2 * j) + (t % j), l = i + j;\n";
+  s << "        const int a = perm[i], c = perm[l];\n";
+  s << "        const bool up = (i & k) == 0;\n";
+  s << "        if (up ? before(c, a) : before(a, c)) { perm[i] = c; perm[l] = a; }\n";
+  s << "      }\n      __syncthreads();\n    }\n  }\n";
+  s << "  for (int e = threadIdx.x; e < " << L << "; e += 256) {\n";
+  s << "    const int src = perm[e];\n";
+  for (size_t j = 0; j < n; ++j) s << "    out" << j << "[base + e * " << inner << "] = " << elem(j, "src") << ";\n";
+  s << "  }\n}\n";
+
+  std::vector<Value*> leaves(sort->operands.begin(), sort->operands.end());
+  std::vector<std::string> outs;
+  for (size_t j = 0; j < n; ++j) outs.push_back(storageT(sort->results[j]->type.dt) + "* __restrict__ out" + std::to_string(j));
+  if (!inLds) outs.push_back("int* __restrict__ work");
+  FusedCode fc;
+  Launch l;
+  l.source = std::string(kPrelude) + kernelHeader(leaves, outs) + " {\n" + s.str();
+  l.grid[0] = (unsigned)std::max<int64_t>(1, outer * inner);
+  l.block[0] = 256;
+  for (auto* v : leaves) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
+  for (auto& r : sort->results) { KArg a; a.kind = KArg::Out; a.value = r.get(); l.args.push_back(a); }
+  if (!inLds) {
+    KArg a;
+    a.kind = KArg::Work;
+    a.workOffset = 0;
+    l.args.push_back(a);
+    fc.workspaceBytes = outer * inner * P * 4;
+  }
+  fc.leaves = leaves;
+  fc.launches.push_back(std::move(l));
+  return fc;
+}
+
 // Horizontal batching: independent one-dimensional kernels become the segments of one
 // launch.  Every generated kernel is kPrelude + one header + body, and addresses its grid
 // through blockIdx.x only, so a segment is that body as a device function of the block index.

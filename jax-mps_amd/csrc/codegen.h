@@ -58,6 +58,11 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf);
 // tensor and stores into `dus` result storage (which already holds the operand).
 FusedCode generateDusKernel(Op* dus, const LeafPredicate& isLeaf);
 
+// stablehlo.sort of a dim that fits LDS (sortLdsBytes <= 60 KiB): one workgroup per slice, comparator region compiled.
+// All operands must be in memory.
+int64_t sortLdsBytes(Op* sort);
+FusedCode generateSortKernel(Op* sort, const LeafPredicate& isLeaf);
+
 // Several independent kernels with one-dimensional grids as the segments of one launch: block b
 // runs the kernel whose block range holds b.  Arguments are the kernels' arguments, concatenated.
 // Returns "" when one of the sources cannot take part (batchableKernel is the cheap test).

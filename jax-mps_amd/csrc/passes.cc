@@ -978,7 +978,7 @@ static const std::set<std::string>& supportedOps() {
       "constant", "iota", "reshape", "broadcast_in_dim", "transpose", "reverse", "concatenate", "slice", "dynamic_slice",
       "dynamic_update_slice", "pad",
       // heavy ops
-      "reduce", "dot_general", "dot", "convolution", "gather", "scatter", "reduce_window", "select_and_scatter",
+      "reduce", "dot_general", "dot", "convolution", "gather", "scatter", "reduce_window", "select_and_scatter", "sort",
       // control flow (ops/control_flow.cc:2364-2376)
       "while", "case", "return", "optimization_barrier", "custom_call",
   };

@@ -325,6 +325,7 @@ class Planner {
       }
       if (n == "convolution") { emitConv(op, plan); continue; }
       if (n == "scatter") { emitScatter(op, plan); continue; }
+      if (n == "sort") { emitSort(op, plan); continue; }
       if (n == "dynamic_update_slice") { emitDus(op, plan); continue; }
       if (n == "while") { emitWhile(op, plan); continue; }
       if (n == "case") { emitCase(op, plan); continue; }
@@ -827,6 +828,20 @@ class Planner {
     if (v->type.dt != DType::F32 && v->type.dt != DType::BF16) return false;
     View vw;
     return resolveView(v, alwaysInMemory, vw);
+  }
+
+  void emitSort(Op* op, Plan& plan) {
+    for (auto* v : op->operands) if (!hasStorage(v)) materializeNow(v, plan);
+    std::vector<Value*> outs;
+    for (auto& r : op->results) outs.push_back(r.get());
+    if (outs.empty() || outs[0]->type.numel() == 0) {
+      for (auto* o : outs) bind(o, newStorage(4));
+      return;
+    }
+    FusedCode fc = generateSortKernel(op, leafPred());
+    for (auto* o : outs) bind(o, newStorage(o->type.bytes()));
+    emitted_.insert(op);
+    addFused(plan, fc, "sort " + op->operands[0]->type.str() + " dim " + std::to_string(op->integer("dimension")), outs);
   }
 
   struct DotPlan {

@@ -809,6 +809,42 @@ class Builder:
         self._emit(f"}}) : ({operand.type}, {source.type}, {st}) -> {v.type}")
         return v
 
+    def sort(self, operands: Sequence[Val], dimension: int = -1, num_keys: int = 1, descending: bool = False, is_stable: bool = True,
+             comparator: Optional[Callable] = None) -> List[Val]:
+        """`lax.sort` as JAX lowers it: a lexicographic comparator over the first `num_keys` operands (floats in
+        total order, so NaNs sort last), or a caller-built `comparator(b, lhs, rhs) -> i1 Val` over scalar block arguments."""
+        operands = list(operands)
+        rank = operands[0].ndim
+        dimension = dimension % rank if rank else 0
+        name = self._fresh()
+        n0 = self._n
+        ind = self._blk.indent
+        self._emit(f'{name}:{len(operands)} = "stablehlo.sort"({", ".join(o.name for o in operands)}) <{{dimension = {dimension} : i64, is_stable = {"true" if is_stable else "false"}}}> ({{')
+        blk = _Block(ind + 1)
+        self._blocks.append(blk)
+        lhs = [Val(self, f"%sl{n0}_{k}", (), o.dtype, blk) for k, o in enumerate(operands)]
+        rhs = [Val(self, f"%sr{n0}_{k}", (), o.dtype, blk) for k, o in enumerate(operands)]
+        hdr = ", ".join(f"{a.name}: {a.type}, {b_.name}: {b_.type}" for a, b_ in zip(lhs, rhs))
+        if comparator is not None:
+            res = comparator(self, lhs, rhs)
+        else:
+            res = None
+            for k in reversed(range(num_keys)):
+                a, c = lhs[k], rhs[k]
+                kind = "TOTALORDER" if a.dtype in FLOAT_TYPES else None
+                first = self.compare(a, c, "GT" if descending else "LT", kind)
+                if res is None:
+                    res = first
+                else:
+                    res = self.or_(first, self.and_(self.compare(a, c, "EQ", kind), res))
+        self._emit(f"stablehlo.return {res.name} : {res.type}")
+        self._blocks.pop()
+        self._blk.lines.append("  " * (ind + 1) + f"^bb0({hdr}):")
+        self._blk.lines.extend(blk.lines)
+        ts = ", ".join(o.type for o in operands)
+        self._emit(f"}}) : ({ts}) -> ({ts})")
+        return [Val(self, f"{name}#{k}", o.shape, o.dtype, self._blk) for k, o in enumerate(operands)]
+
     def rng_bit_generator(self, state: Val, shape, dtype="ui32", algorithm="DEFAULT"):
         """`jax.random.bits` under the rbg / unsafe_rbg PRNG implementations: (new state, bits)."""
         name = self._fresh()

@@ -1616,6 +1616,46 @@ class Oracle:
 
     def op_optimization_barrier(self, op, ins, env): return list(ins)
 
+    def op_sort(self, op, ins, env):
+        """stablehlo.sort: the comparator region decides, ties keep their order (the reference sorts by the first
+        operand with a direction read off the comparator, src/pjrt_plugin/ops/sort_fft_complex.cc:145-216; for the
+        comparators JAX emits both agree).  Evaluated without a sorting routine: the comparator is run on all pairs
+        of a slice at once, and element i lands at (number of j before i) where j is before i if cmp(j, i), or
+        neither cmp(j, i) nor cmp(i, j) and j < i."""
+        dim = int(op.attrs["dimension"])
+        xs = [np.asarray(x) for x in ins]
+        if xs[0].ndim == 0:
+            return [x.copy() for x in xs]
+        if dim < 0:
+            dim += xs[0].ndim
+        moved = [np.moveaxis(x, dim, -1) for x in xs]
+        L = moved[0].shape[-1]
+        lead = moved[0].shape[:-1]
+        flat = [m.reshape(-1, L) for m in moved]
+        outs = [np.empty_like(f) for f in flat]
+        body = op.regions[0]
+        idx = np.arange(L)
+        step = max(1, min(L, (1 << 23) // max(L, 1)))      # rows of the all-pairs table evaluated at once
+        for r in range(flat[0].shape[0]):
+            pos = np.empty(L, dtype=np.int64)
+            for i0 in range(0, L, step):
+                i1 = min(L, i0 + step)
+                fwd, rev = [], []
+                for f in flat:
+                    xi = np.broadcast_to(f[r][i0:i1, None], (i1 - i0, L))
+                    xj = np.broadcast_to(f[r][None, :], (i1 - i0, L))
+                    fwd += [xi, xj]
+                    rev += [xj, xi]
+                lt_ij = np.asarray(self._run_region(body, fwd, env, vectorized=True)[0]).astype(bool)   # cmp(x_i, x_j)
+                lt_ji = np.asarray(self._run_region(body, rev, env, vectorized=True)[0]).astype(bool)   # cmp(x_j, x_i)
+                before = lt_ji | (~lt_ij & ~lt_ji & (idx[None, :] < idx[i0:i1, None]))                   # j sorts before i
+                pos[i0:i1] = before.sum(axis=1)
+            perm = np.empty(L, dtype=np.int64)
+            perm[pos] = idx
+            for f, o in zip(flat, outs):
+                o[r] = f[r][perm]
+        return [np.moveaxis(o.reshape(lead + (L,)), -1, dim) for o in outs]
+
     def op_rng_bit_generator(self, op, ins, env):
         """State rule of the reference (src/pjrt_plugin/ops/control_flow.cc:2301-2360): state = [key, counter, ...] as
         ui64, the counter grows by ceil(output bytes / 16).  The bits themselves are implementation-defined (the

@@ -490,6 +490,35 @@ def get_case(name: str) -> Case:
     raise KeyError(name)
 
 
+# ------------------------------------------------------------------ sort (reference tests: tests/configs/sort.py:13-135 use
+# random inputs against JAX-CPU; here the same forms, checked bit-for-bit against the oracle, which tests/test_oracle_pins.py
+# pins to numpy's stable sorts)
+def _with_ties(seed, *shape):
+    return (np.round(f32(seed, *shape, lo=-3, hi=3) * 2) / 2 + np.float32(0.0)).astype(np.float32)   # + 0.0: no negative zeros (total order tells them apart)
+
+
+_SORT_NAN = np.array([[3.0, np.nan, -1.0, 2.0, -np.inf, np.inf, -0.0, 0.0, np.nan, 2.0]], np.float32)
+case("sort-1d", lambda b, x: b.sort([x]), f32(2100, 1000), exact=True)
+case("sort-1d-odd-length", lambda b, x: b.sort([x]), f32(2101, 777), exact=True)
+case("sort-2d-axis0", lambda b, x: b.sort([x], dimension=0), f32(2102, 37, 20), exact=True)
+case("sort-3d-axis1", lambda b, x: b.sort([x], dimension=1), f32(2103, 3, 50, 7), exact=True)
+case("sort-descending", lambda b, x: b.sort([x], descending=True), _with_ties(2104, 4, 64), exact=True)
+case("sort-nan-and-signed-zero-total-order", lambda b, x: b.sort([x]), _SORT_NAN, exact=True)
+case("sort-int32", lambda b, x: b.sort([x]), i32(2105, 5, 300, lo=-1000, hi=1000), exact=True)
+case("sort-uint8", lambda b, x: b.sort([x], descending=True), rng(2106).integers(0, 256, size=(3, 100)).astype(np.uint8), exact=True)
+case("sort-bool", lambda b, x: b.sort([x]), rng(2107).integers(0, 2, size=(2, 33)).astype(np.bool_), exact=True)
+case("sort-key-val-stable-ties", lambda b, k, v: b.sort([k, v], dimension=1), _with_ties(2108, 4, 200), f32(2109, 4, 200), exact=True)
+case("sort-argsort-descending-ties", lambda b, k: b.sort([k, b.iota(k.shape, 1, "i32")], dimension=1, descending=True), _with_ties(2110, 6, 129), exact=True)
+case("sort-two-keys-lexicographic", lambda b, k0, k1, v: b.sort([k0, k1, v], dimension=0, num_keys=2),
+     rng(2111).integers(0, 4, size=(500,)).astype(np.int32), _with_ties(2112, 500), f32(2113, 500), exact=True)
+case("sort-custom-comparator-abs", lambda b, x: b.sort([x], comparator=lambda bb, l, r: bb.compare(bb.abs(l[0]), bb.abs(r[0]), "LT")), _with_ties(2114, 3, 100), exact=True)
+case("sort-bf16-keys", lambda b, k, v: b.sort([k, v]), f32(2115, 2, 256), i32(2116, 2, 256), dtypes=["bf16", "i32"], exact=True)
+case("sort-4096", lambda b, x: b.sort([x]), f32(2117, 2, 4096), exact=True)
+case("sort-long-slice-in-memory", lambda b, x: b.sort([x]), f32(2119, 20000), exact=True)
+case("sort-long-key-val-in-memory", lambda b, k, v: b.sort([k, v], dimension=0, descending=True), _with_ties(2120, 9000, 2), i32(2121, 9000, 2), exact=True)
+case("sort-fused-producer-and-consumer", lambda b, x: b.mul(b.sort([b.neg(x)])[0], 2.0), f32(2118, 8, 100), exact=True)
+
+
 # ------------------------------------------------------------------ rng_bit_generator: counter update as the reference
 # keeps it (src/pjrt_plugin/ops/control_flow.cc:2343-2355); bits = threefry2x32 of (key halves; element index, counter)
 _RNG_STATE = np.array([0x0123456789ABCDEF, 41], dtype=np.uint64)

@@ -315,6 +315,45 @@ def test_threefry2x32_known_answer_vectors():
     assert np.array_equal(out[1], op_cases.THREEFRY_KAT["out1"])
 
 
+def test_sort_against_numpy_stable_sorts():
+    """The oracle's sort (comparator on all pairs, no sorting routine) against numpy: np.sort for values, stable
+    np.argsort for key/value and descending ties (JAX's descending sort is a stable sort under GT, so equal keys keep
+    their original order), np.lexsort for two keys, total order for NaN and signed zero."""
+    import op_cases
+    def run(name):
+        c = op_cases.get_case(name)
+        ins = [round_bf16(a) if d == "bf16" else a for a, d in zip(c.inputs, c.dtypes)]
+        return ins, Oracle(c.text).run(*ins)
+    for name, axis in (("sort-1d", 0), ("sort-1d-odd-length", 0), ("sort-2d-axis0", 0), ("sort-3d-axis1", 1), ("sort-int32", 1), ("sort-bool", 1), ("sort-4096", 1), ("sort-long-slice-in-memory", 0)):
+        ins, out = run(name)
+        assert np.array_equal(out[0], np.sort(ins[0], axis=axis, kind="stable")), name
+    ins, out = run("sort-descending")
+    assert np.array_equal(out[0], -np.sort(-ins[0], axis=1, kind="stable"))
+    ins, out = run("sort-uint8")
+    assert np.array_equal(out[0], np.sort(ins[0], axis=1)[:, ::-1])
+    ins, out = run("sort-nan-and-signed-zero-total-order")
+    want = np.array([[-np.inf, -1.0, -0.0, 0.0, 2.0, 2.0, 3.0, np.inf, np.nan, np.nan]], np.float32)
+    assert np.array_equal(out[0].view(np.uint32), want.view(np.uint32))       # -0.0 before +0.0, NaNs last
+    ins, out = run("sort-key-val-stable-ties")
+    order = np.argsort(ins[0], axis=1, kind="stable")
+    assert np.array_equal(out[0], np.take_along_axis(ins[0], order, 1)) and np.array_equal(out[1], np.take_along_axis(ins[1], order, 1))
+    ins, out = run("sort-argsort-descending-ties")
+    order = np.argsort(-ins[0], axis=1, kind="stable")
+    assert np.array_equal(out[1], order.astype(np.int32)) and np.array_equal(out[0], np.take_along_axis(ins[0], order, 1))
+    ins, out = run("sort-long-key-val-in-memory")
+    order = np.argsort(-ins[0], axis=0, kind="stable")
+    assert np.array_equal(out[0], np.take_along_axis(ins[0], order, 0)) and np.array_equal(out[1], np.take_along_axis(ins[1], order, 0))
+    ins, out = run("sort-two-keys-lexicographic")
+    order = np.lexsort((ins[1], ins[0]))                                       # last key is the primary one; lexsort is stable
+    assert all(np.array_equal(o, i[order]) for o, i in zip(out, ins))
+    ins, out = run("sort-custom-comparator-abs")
+    order = np.argsort(np.abs(ins[0]), axis=1, kind="stable")
+    assert np.array_equal(out[0], np.take_along_axis(ins[0], order, 1))
+    ins, out = run("sort-bf16-keys")
+    order = np.argsort(ins[0], axis=1, kind="stable")
+    assert np.array_equal(out[1], np.take_along_axis(ins[1], order, 1))
+
+
 def test_rng_bit_generator_state_rule_and_bits():
     """State: key unchanged, counter += ceil(output bytes / 16) (reference: src/pjrt_plugin/ops/control_flow.cc:2343-2355),
     wrapping at 2^64.  Bits: the oracle's threefry helper reproduces the Random123 known answers, element i of a draw is
