@@ -142,6 +142,7 @@ std::unique_ptr<Module> parseStableHLOText(const char* data, size_t size);
 // Passes (passes.cc)
 void inlineCalls(Module& m);          // replaces every "call" by the callee body
 void lowerIntegerDots(Module& m);    // integer / boolean dot_general -> broadcast, multiply, reduce
+void lowerTopK(Module& m);           // chlo.top_k -> stable descending sort of (value, position) + slice
 void lowerRng(Module& m);            // rng_bit_generator -> counter update + threefry2x32 as plain ui32 ops
 void lowerWindowOps(Module& m);      // reduce_window / select_and_scatter with small windows -> pad, strided slices, elementwise ops
 void lowerGeneralScatters(Module& m); // scatter forms other than whole rows along dim 0 -> element scatter with computed keys

@@ -983,6 +983,22 @@ class Parser {
       fnType(op, outs);
       return;
     }
+    if (n == "chlo.top_k") {
+      // %values, %indices = chlo.top_k(%x, k = 3) : tensor<16xf32> -> (tensor<3xf32>, tensor<3xi32>)
+      expect("(");
+      op->operands = ssaUseList();
+      expect(",");
+      expect("k");
+      expect("=");
+      setInt(op, "k", integer());
+      expect(")");
+      if (peekc() == '{') skipBalanced('{', '}');
+      expect(":");
+      parseType();
+      expect("->");
+      outs = typeListParen();
+      return;
+    }
     if (n == "rng_bit_generator") {
       // %state, %bits = stablehlo.rng_bit_generator %state0, algorithm = THREE_FRY : (tensor<2xui64>) -> (tensor<2xui64>, tensor<8xui32>)
       op->operands = ssaUseList();

@@ -909,7 +909,100 @@ void lowerRngIn(Region& r, int& nextId) {
   }
 }
 
+// chlo.top_k(x, k) -> the first k entries of a stable descending sort of (x, position) along the last dim: largest
+// values first, equal values in ascending position (the tie rule the reference keeps, src/pjrt_plugin/ops/
+// sort_fft_complex.cc:40-82); floats compare in total order.
+void lowerTopKIn(Region& r, int& nextId) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) lowerTopKIn(*sub, nextId);
+    if (op->name != "chlo.top_k") continue;
+    if (op->operands.size() != 1 || op->results.size() != 2) throw CompileError("chlo.top_k: expected one operand and two results");
+    Value* x = op->operands[0];
+    const TensorType xt = x->type;
+    if (xt.rank() < 1) throw CompileError("chlo.top_k: the operand must have at least one dim");
+    const int64_t kk = op->integer("k");
+    const int last = xt.rank() - 1;
+    if (kk < 0 || kk > xt.dims[(size_t)last]) throw CompileError("chlo.top_k: k is out of range");
+    const DType it = op->results[1]->type.dt;
+    Rewriter rw{r, nextId, op->line, {}};
+    TensorType idxT = xt;
+    idxT.dt = it;
+    auto io = makeOp("iota", {}, &r, op->line);
+    Attr dimA;
+    dimA.kind = Attr::Int;
+    dimA.i = last;
+    io->attrs["dim"] = dimA;
+    Value* pos = rw.emit(std::move(io), idxT);
+    // sort with the comparator "lhs > rhs" on the values
+    auto so = makeOp("sort", {x, pos}, &r, op->line);
+    Attr lastA = dimA;
+    so->attrs["dimension"] = lastA;
+    auto region = std::make_unique<Region>();
+    region->parent = so.get();
+    TensorType scalarV, scalarI, pred;
+    scalarV.dt = xt.dt; scalarI.dt = it; pred.dt = DType::Pred;
+    const TensorType argTypes[4] = {scalarV, scalarV, scalarI, scalarI};
+    for (int a = 0; a < 4; ++a) {
+      auto v = std::make_unique<Value>();
+      v->id = nextId++;
+      v->type = argTypes[a];
+      v->argOf = region.get();
+      v->defIndex = a;
+      v->name = "%topk_arg" + std::to_string(v->id);
+      region->args.push_back(std::move(v));
+    }
+    auto cmp = makeOp("compare", {region->args[0].get(), region->args[1].get()}, region.get(), op->line);
+    Attr dir;
+    dir.kind = Attr::Str;
+    dir.s = "GT";
+    cmp->attrs["direction"] = dir;
+    if (isFloat(xt.dt)) {
+      Attr ct;
+      ct.kind = Attr::Str;
+      ct.s = "TOTALORDER";
+      cmp->attrs["compare_type"] = ct;
+    }
+    Value* gt = addResult(cmp.get(), pred, nextId);
+    auto ret = makeOp("return", {gt}, region.get(), op->line);
+    region->ops.push_back(std::move(cmp));
+    region->ops.push_back(std::move(ret));
+    so->regions.push_back(std::move(region));
+    Value* sortedV = addResult(so.get(), xt, nextId);
+    Value* sortedI = addResult(so.get(), idxT, nextId);
+    rw.made.push_back(std::move(so));
+    // first k along the last dim
+    auto firstK = [&](Value* v) {
+      auto sl = makeOp("slice", {v}, &r, op->line);
+      std::vector<int64_t> start((size_t)xt.rank(), 0), limit = xt.dims, stride((size_t)xt.rank(), 1);
+      limit[(size_t)last] = kk;
+      sl->attrs["start"] = intsAttr(start);
+      sl->attrs["limit"] = intsAttr(limit);
+      sl->attrs["strides"] = intsAttr(stride);
+      return sl;
+    };
+    auto sv = firstK(sortedV), si = firstK(sortedI);
+    sv->results.push_back(std::move(op->results[0]));
+    sv->results[0]->def = sv.get();
+    si->results.push_back(std::move(op->results[1]));
+    si->results[0]->def = si.get();
+    rw.made.push_back(std::move(sv));
+    rw.made.push_back(std::move(si));
+    size_t nIns = rw.made.size();
+    r.ops.erase(r.ops.begin() + k);
+    r.ops.insert(r.ops.begin() + k, std::make_move_iterator(rw.made.begin()), std::make_move_iterator(rw.made.end()));
+    k += nIns - 1;
+  }
+}
+
 }  // namespace
+
+void lowerTopK(Module& m) {
+  Func* f = m.main();
+  if (!f) return;
+  int nextId = maxValueId(f->body) + 1;
+  lowerTopKIn(f->body, nextId);
+}
 
 void lowerRng(Module& m) {
   Func* f = m.main();

@@ -1641,6 +1641,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   lowerGeneralScatters(*module);
   lowerWindowOps(*module);
   lowerRng(*module);
+  lowerTopK(*module);
   checkSupported(*module);
   eliminateDeadCode(module->main()->body);
   prog->module = std::move(module);

@@ -845,6 +845,13 @@ class Builder:
         self._emit(f"}}) : ({ts}) -> ({ts})")
         return [Val(self, f"{name}#{k}", o.shape, o.dtype, self._blk) for k, o in enumerate(operands)]
 
+    def top_k(self, x: Val, k: int):
+        """`lax.top_k`: (values, i32 indices) of the k largest entries along the last dim."""
+        name = self._fresh()
+        shape = tuple(x.shape[:-1]) + (int(k),)
+        self._emit(f"{name}:2 = chlo.top_k({x.name}, k = {int(k)}) : {x.type} -> ({ttype(shape, x.dtype)}, {ttype(shape, 'i32')})")
+        return Val(self, f"{name}#0", shape, x.dtype, self._blk), Val(self, f"{name}#1", shape, "i32", self._blk)
+
     def rng_bit_generator(self, state: Val, shape, dtype="ui32", algorithm="DEFAULT"):
         """`jax.random.bits` under the rbg / unsafe_rbg PRNG implementations: (new state, bits)."""
         name = self._fresh()

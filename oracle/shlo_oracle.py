@@ -607,6 +607,19 @@ class _P:
             self.expect(":")
             self.fn_type(op)
             return
+        if op.name == "chlo.top_k":
+            self.expect("(")
+            op.operands = self.ssa_list()
+            self.expect(",")
+            self.expect("k")
+            self.expect("=")
+            op.attrs["k"] = self.integer()
+            self.expect(")")
+            self.expect(":")
+            op.in_types = [self.type()]
+            self.expect("->")
+            op.out_types = self.type_list_paren()
+            return
         if short == "rng_bit_generator":
             op.operands = self.ssa_list()
             self.expect(",")
@@ -1656,6 +1669,22 @@ class Oracle:
                 o[r] = f[r][perm]
         return [np.moveaxis(o.reshape(lead + (L,)), -1, dim) for o in outs]
 
+    def op_chlo_top_k(self, op, ins, env):
+        """Largest k along the last dim, equal values in ascending position (reference: TopKImplFn,
+        src/pjrt_plugin/ops/sort_fft_complex.cc:40-82); floats in total order (NaN above +inf, -0.0 below +0.0).
+        Selection by counting: element i has rank #{j: x_j > x_i} + #{j < i: x_j == x_i}."""
+        x = np.asarray(ins[0])
+        k = int(op.attrs["k"])
+        key = _total_order_key(x) if x.dtype.kind == "f" else x
+        a, b = key[..., :, None], key[..., None, :]
+        L = x.shape[-1]
+        idx = np.arange(L)
+        rank = (b > a).sum(-1) + ((b == a) & (idx[None, :] < idx[:, None])).sum(-1)
+        order = np.empty(x.shape, dtype=np.int64)
+        np.put_along_axis(order, rank, np.broadcast_to(idx, x.shape), axis=-1)
+        order = order[..., :k]
+        return [np.take_along_axis(x, order, -1), order.astype(_NP[op.out_types[1].dtype])]
+
     def op_rng_bit_generator(self, op, ins, env):
         """State rule of the reference (src/pjrt_plugin/ops/control_flow.cc:2301-2360): state = [key, counter, ...] as
         ui64, the counter grows by ceil(output bytes / 16).  The bits themselves are implementation-defined (the
@@ -1686,6 +1715,15 @@ class Oracle:
         if tgt in ("Sharding", "SPMDFullToShardShape", "SPMDShardToFullShape"):
             return ins[0]
         raise NotImplementedError(f"oracle: custom_call {tgt}")
+
+
+def _total_order_key(x):
+    """Signed integer key whose order is the IEEE total order of the floats (sign-magnitude bits made monotonic)."""
+    x = np.asarray(x)
+    bits = {2: np.int16, 4: np.int32, 8: np.int64}[x.dtype.itemsize]
+    i = x.view(bits).astype(np.int64)
+    top = np.int64(1) << (8 * x.dtype.itemsize - 1)
+    return np.where(i < 0, -(i + top) - 1, i)
 
 
 def threefry2x32(k0, k1, c0, c1):

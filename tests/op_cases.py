@@ -519,6 +519,19 @@ case("sort-long-key-val-in-memory", lambda b, k, v: b.sort([k, v], dimension=0, 
 case("sort-fused-producer-and-consumer", lambda b, x: b.mul(b.sort([b.neg(x)])[0], 2.0), f32(2118, 8, 100), exact=True)
 
 
+# top_k (reference tests: tests/configs/sort.py:140-210): shapes of the reference's cases plus ties, NaN and a vocabulary-sized row
+case("top-k-1d", lambda b, x: list(b.top_k(x, 3)), f32(2130, 16), exact=True)
+case("top-k-2d-k1", lambda b, x: list(b.top_k(x, 1)), f32(2131, 4, 8), exact=True)
+case("top-k-2d-k5", lambda b, x: list(b.top_k(x, 5)), f32(2132, 4, 8), exact=True)
+case("top-k-4d", lambda b, x: list(b.top_k(x, 3)), f32(2133, 2, 2, 4, 8), exact=True)
+case("top-k-transposed-input", lambda b, x: list(b.top_k(b.transpose(x, [2, 1, 0]), 2)), f32(2134, 2, 4, 8), exact=True)
+case("top-k-equals-size", lambda b, x: list(b.top_k(x, 8)), f32(2135, 4, 8), exact=True)
+case("top-k-ties-lowest-index-first", lambda b, x: list(b.top_k(x, 6)), _with_ties(2136, 5, 40), exact=True)
+case("top-k-nan-first", lambda b, x: list(b.top_k(x, 4)), _SORT_NAN, exact=True)
+case("top-k-int32", lambda b, x: list(b.top_k(x, 7)), i32(2137, 3, 100), exact=True)
+case("top-k-vocabulary-row", lambda b, x: list(b.top_k(x, 50)), f32(2138, 2, 8000), exact=True)
+
+
 # ------------------------------------------------------------------ rng_bit_generator: counter update as the reference
 # keeps it (src/pjrt_plugin/ops/control_flow.cc:2343-2355); bits = threefry2x32 of (key halves; element index, counter)
 _RNG_STATE = np.array([0x0123456789ABCDEF, 41], dtype=np.uint64)

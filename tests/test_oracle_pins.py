@@ -354,6 +354,23 @@ def test_sort_against_numpy_stable_sorts():
     assert np.array_equal(out[1], np.take_along_axis(ins[1], order, 1))
 
 
+def test_top_k_against_numpy():
+    """top_k of the oracle (rank counting) against a stable numpy argsort of the negated values, and the literal tie /
+    NaN expectations: equal values come out in ascending position, NaN ranks above +inf (total order)."""
+    import op_cases
+    for name in ("top-k-1d", "top-k-2d-k5", "top-k-4d", "top-k-equals-size", "top-k-ties-lowest-index-first", "top-k-int32", "top-k-vocabulary-row"):
+        c = op_cases.get_case(name)
+        vals, idx = Oracle(c.text).run(*c.inputs)
+        x = c.inputs[0]
+        k = vals.shape[-1]
+        order = np.argsort(-x.astype(np.float64), axis=-1, kind="stable")[..., :k]
+        assert np.array_equal(idx, order.astype(np.int32)), name
+        assert np.array_equal(vals, np.take_along_axis(x, order, -1)), name
+    c = op_cases.get_case("top-k-nan-first")
+    vals, idx = Oracle(c.text).run(*c.inputs)
+    assert np.array_equal(idx, np.array([[1, 8, 5, 0]], np.int32)) and np.isnan(vals[0, :2]).all() and vals[0, 2] == np.inf and vals[0, 3] == 3.0
+
+
 def test_rng_bit_generator_state_rule_and_bits():
     """State: key unchanged, counter += ceil(output bytes / 16) (reference: src/pjrt_plugin/ops/control_flow.cc:2343-2355),
     wrapping at 2^64.  Bits: the oracle's threefry helper reproduces the Random123 known answers, element i of a draw is
