@@ -909,6 +909,7 @@ static const char* reduceKind(const Op& reduce) {
 }
 
 bool isSimpleReduce(const Op& reduce) { return reduce.operands.size() == 2 && reduceKind(reduce) != nullptr; }
+const char* simpleReduceKind(const Op& reduce) { return reduce.operands.size() == 2 ? reduceKind(reduce) : nullptr; }
 
 // ------------------------------------------------------------------ loop kernels
 FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf) { return generateLoopKernel(std::vector<Value*>{root}, isLeaf); }

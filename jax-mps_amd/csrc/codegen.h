@@ -79,5 +79,6 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
 bool isFusibleOp(const Op& op);
 // True if the reducer body of `reduce` is one supported binary op.
 bool isSimpleReduce(const Op& reduce);
+const char* simpleReduceKind(const Op& reduce);   // "add", "maximum", ... for a one-input reduce with a single-op reducer, else null
 
 }  // namespace mi355

@@ -89,6 +89,18 @@ int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, const void* b
 size_t mi355_gemm_bf16_async_workspace_bytes(const mi355_gemm_desc* d);
 int mi355_gemm_bf16_tiled(const mi355_gemm_desc* d, const void* a, const void* b, void* c, mi355_stream_t s);
 
+// softmax(scale * Q K^T, masked positions replaced by `masked`) V for bf16 tensors addressed through element strides
+// (head dim contiguous): q[b, n, t, :H], k[b, n, s, :H], v[b, n, s, :H], out[b, n, t, :H]; mask (may be NULL) is one byte
+// per position addressed by mB / mN / mT / mS (0 = broadcast), non-zero = keep.
+typedef struct {
+  int64_t B, N, T, S, H;
+  int64_t qB, qN, qT, kB, kN, kS, vB, vN, vS, oB, oN, oT, mB, mN, mT, mS;
+  float scale, masked;
+} mi355_attention_desc;
+int mi355_attention_supported(const mi355_attention_desc* d);
+int mi355_attention(const mi355_attention_desc* d, const void* q, const void* k, const void* v, const void* mask, void* out,
+                    mi355_stream_t s);
+
 typedef struct {
   int nsp;
   int64_t N, C, O;

@@ -59,10 +59,17 @@ struct ScatterDesc {   // row scatter: operand [rows, rowSize...], one index per
   DType type = DType::F32, indexType = DType::S32;
 };
 
+struct AttentionDesc {   // softmax(scale * Q K^T, masked -> `masked`) V, tensors addressed as [b, n, t|s, h] through element strides
+  int64_t B = 0, N = 0, T = 0, S = 0, H = 0;
+  int64_t qB = 0, qN = 0, qT = 0, kB = 0, kN = 0, kS = 0, vB = 0, vN = 0, vS = 0, oB = 0, oN = 0, oT = 0, mB = 0, mN = 0, mT = 0, mS = 0;
+  float scale = 1.f, masked = 0.f;
+  bool hasMask = false;
+};
+
 struct Plan;
 
 struct Step {
-  enum Kind { Kernel, Gemm, Conv, ScatterRows, Copy, Fill, While, Case, GemmGroup } kind = Kernel;
+  enum Kind { Kernel, Gemm, Conv, ScatterRows, Copy, Fill, While, Case, GemmGroup, Attention } kind = Kernel;
   std::string label;  // op name(s) for profiling ranges and error messages
 
   // Kernel
@@ -75,6 +82,7 @@ struct Step {
 
   // Gemm / Conv / ScatterRows
   GemmDesc gemm;
+  AttentionDesc attn;              // Attention: args = [q, k, v, out, (mask)]
   GemmDesc gemm2;                  // dual: second product summed into the same result; args = [a, b, c, a2, b2]
   bool dual = false;
   std::vector<Step> parts;         // GemmGroup: independent small products launched together (each a Gemm step)
@@ -124,5 +132,6 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module);
 int abiDtypeCode(DType d);   // element type code of the C-ABI kernel entry points (-1: not supported there)
 mi355_conv_desc toAbi(const ConvDesc& c);
 mi355_gemm_desc toAbi(const GemmDesc& g);
+mi355_attention_desc toAbi(const AttentionDesc& a);
 
 }  // namespace mi355

@@ -287,16 +287,50 @@ class Planner {
   }
 
   void emitRegion(Region& r, Plan& plan) {
+    // attention chains: everything between the two products is skipped, the second product emits the fused step
+    std::unordered_map<Op*, AttnMatch> attention;   // keyed by the second product
+    std::unordered_set<Op*> attentionInner;
+    for (auto& o : r.ops) {
+      AttnMatch m;
+      if (o->name == "dot_general" && matchAttention(o.get(), m)) {
+        bool fresh = true;
+        for (Op* a : m.absorbed) if (attentionInner.count(a)) fresh = false;
+        if (!fresh) continue;
+        for (Op* a : m.absorbed) if (a != m.pv) attentionInner.insert(a);
+        attention[o.get()] = m;
+      }
+    }
     for (size_t pos = 0; pos < r.ops.size(); ++pos) {
       Op* op = r.ops[pos].get();
       if (emitted_.count(op)) continue;
+      if (attentionInner.count(op)) continue;
+      {
+        auto am = attention.find(op);
+        if (am != attention.end()) {
+          if (emitAttention(am->second, plan)) continue;
+          // not eligible after all: emit the chain the ordinary way, in program order, then this product
+          for (size_t q = 0; q < pos; ++q) {
+            Op* inner = r.ops[q].get();
+            if (std::find(am->second.absorbed.begin(), am->second.absorbed.end(), inner) == am->second.absorbed.end()) continue;
+            attentionInner.erase(inner);
+            emitOne(inner, r, q, plan);
+          }
+        }
+      }
+      emitOne(op, r, pos, plan);
+    }
+  }
+
+  void emitOne(Op* op, Region& r, size_t pos, Plan& plan) {
+    {
+      if (emitted_.count(op)) return;
       const std::string& n = op->name;
-      if (n == "return") continue;
+      if (n == "return") return;
       if (isFusibleOp(*op) && op->results.size() == 1) {
         Value* v = op->result();
-        if (!needMat_[v]) continue;
+        if (!needMat_[v]) return;
         emitLoopGroup(op, r, pos, plan);
-        continue;
+        return;
       }
       if (isPassThrough(*op)) {   // multi-result barrier: results alias operands
         for (size_t k = 0; k < op->results.size(); ++k) {
@@ -304,13 +338,13 @@ class Planner {
           if (!hasStorage(o)) materializeNow(o, plan);
           bind(op->results[k].get(), storageOf(o));
         }
-        continue;
+        return;
       }
-      if (n == "reduce") { if (!tryRowProgram(op, r, pos, plan)) emitReduce(op, r, plan); continue; }
+      if (n == "reduce") { if (!tryRowProgram(op, r, pos, plan)) emitReduce(op, r, plan); return; }
       if (n == "dot_general" || n == "dot") {
         // add(dot, dot): the earlier product waits for the later one when nothing that writes in place lies between
         auto held = heldDots_.find(op);
-        if (held != heldDots_.end()) { emitDot(op, plan, held->second); continue; }
+        if (held != heldDots_.end()) { emitDot(op, plan, held->second); return; }
         if (Op* partner = sumPartner(op)) {
           size_t q = pos + 1;
           bool clear = true;
@@ -318,17 +352,17 @@ class Planner {
             const std::string& between = r.ops[q]->name;
             if (!isFusibleOp(*r.ops[q]) && between != "dot_general" && between != "dot" && between != "reduce" && between != "convolution") clear = false;
           }
-          if (clear && q < r.ops.size() && !emitted_.count(partner) && !heldDots_.count(partner)) { heldDots_[partner] = op; continue; }
+          if (clear && q < r.ops.size() && !emitted_.count(partner) && !heldDots_.count(partner)) { heldDots_[partner] = op; return; }
         }
         emitDot(op, plan);
-        continue;
+        return;
       }
-      if (n == "convolution") { emitConv(op, plan); continue; }
-      if (n == "scatter") { emitScatter(op, plan); continue; }
-      if (n == "sort") { emitSort(op, plan); continue; }
-      if (n == "dynamic_update_slice") { emitDus(op, plan); continue; }
-      if (n == "while") { emitWhile(op, plan); continue; }
-      if (n == "case") { emitCase(op, plan); continue; }
+      if (n == "convolution") { emitConv(op, plan); return; }
+      if (n == "scatter") { emitScatter(op, plan); return; }
+      if (n == "sort") { emitSort(op, plan); return; }
+      if (n == "dynamic_update_slice") { emitDus(op, plan); return; }
+      if (n == "while") { emitWhile(op, plan); return; }
+      if (n == "case") { emitCase(op, plan); return; }
       throw CompileError("no lowering for stablehlo." + n);
     }
   }
@@ -828,6 +862,199 @@ class Planner {
     if (v->type.dt != DType::F32 && v->type.dt != DType::BF16) return false;
     View vw;
     return resolveView(v, alwaysInMemory, vw);
+  }
+
+  // ---------------------------------------------------------------- fused attention
+  // dot_general(q, k) -> [* scale] -> [select(mask, ., c)] -> softmax over the keys -> convert -> dot_general(., v)
+  // [-> transpose that merges the heads], every intermediate read by this chain only: one launch of the fused
+  // kernel.  Matching starts from the second product and walks up.
+  struct AttnMatch {
+    Op* qk = nullptr;
+    Op* pv = nullptr;
+    Op* merge = nullptr;          // transpose [0, 2, 1, 3] of the result, if it is the only reader
+    Value* mask = nullptr;        // i1, rank 4, dims 1 or full
+    float scale = 1.f, masked = 0.f;
+    std::vector<Op*> absorbed;    // ops between the two products (and the products)
+  };
+
+  static bool splatFloat(Value* v, float& out) {
+    Op* d = v->def;
+    while (d && (d->name == "broadcast_in_dim" || d->name == "reshape") && d->operands[0]->type.numel() == 1) d = d->operands[0]->def;
+    if (!d || d->name != "constant") return false;
+    auto& dd = *d->attrs.at("value").dense;
+    if (dd.type.dt != DType::F32 || (!dd.splat && dd.type.numel() != 1)) return false;
+    memcpy(&out, dd.bytes.data(), 4);
+    return true;
+  }
+
+  // v = broadcast_in_dim(r, dims = [0, 1, 2]) of a reduce over dim 3 of `x` with the given reducer
+  static Op* rowReduceOf(Value* v, Value* x, const char* kind, std::vector<Op*>& absorbed) {
+    Op* bc = v->def;
+    if (!bc || bc->name != "broadcast_in_dim" || v->users.size() != 1 || bc->ints("dims") != std::vector<int64_t>{0, 1, 2}) return nullptr;
+    Op* red = bc->operands[0]->def;
+    if (!red || red->name != "reduce" || bc->operands[0]->users.size() != 1 || red->operands[0] != x) return nullptr;
+    const char* k = simpleReduceKind(*red);
+    if (!k || std::string(k) != kind || red->ints("dimensions") != std::vector<int64_t>{3}) return nullptr;
+    float init = 0.f;
+    if (!splatFloat(red->operands[1], init)) return nullptr;
+    if (std::string(kind) == "add" ? init != 0.f : !(init == -__builtin_inff())) return nullptr;
+    absorbed.push_back(bc);
+    absorbed.push_back(red);
+    return red;
+  }
+
+  static bool matchAttention(Op* pv, AttnMatch& m) {
+    static const bool on = !getenv("MI355X_ATTENTION") || atoi(getenv("MI355X_ATTENTION")) != 0;
+    if (!on || pv->name != "dot_general") return false;
+    Value* p = pv->operands[0];
+    Value* v = pv->operands[1];
+    if (p->type.dt != DType::BF16 || v->type.dt != DType::BF16 || pv->result()->type.dt != DType::BF16) return false;
+    if (p->type.rank() != 4 || v->type.rank() != 4) return false;
+    if (pv->ints("lhs_batch") != std::vector<int64_t>{0, 1} || pv->ints("lhs_contract") != std::vector<int64_t>{3}) return false;
+    if (pv->ints("rhs_batch").size() != 2 || pv->ints("rhs_contract").size() != 1) return false;
+    // the free dim of v must be its last one (the head dim, contiguous)
+    {
+      std::vector<bool> used(4, false);
+      for (auto d : pv->ints("rhs_batch")) used[(size_t)d] = true;
+      used[(size_t)pv->ints("rhs_contract")[0]] = true;
+      if (used[3]) return false;
+    }
+    m.pv = pv;
+    Op* cv = p->def;
+    if (!cv || cv->name != "convert" || p->users.size() != 1 || cv->operands[0]->type.dt != DType::F32) return false;
+    Value* probs = cv->operands[0];
+    Op* dv = probs->def;
+    if (!dv || dv->name != "divide" || probs->users.size() != 1) return false;
+    Value* e = dv->operands[0];
+    Op* ex = e->def;
+    if (!ex || ex->name != "exponential" || e->users.size() != 2) return false;
+    m.absorbed = {pv, cv, dv, ex};
+    if (!rowReduceOf(dv->operands[1], e, "add", m.absorbed)) return false;
+    Value* centred = ex->operands[0];
+    Op* sb = centred->def;
+    if (!sb || sb->name != "subtract" || centred->users.size() != 1) return false;
+    m.absorbed.push_back(sb);
+    Value* x = sb->operands[0];
+    if (x->users.size() != 2 || !rowReduceOf(sb->operands[1], x, "maximum", m.absorbed)) return false;
+    if (x->def && x->def->name == "select" && x->type.dt == DType::F32) {
+      Op* sel = x->def;
+      Op* mb = sel->operands[0]->def;
+      float neg = 0.f;
+      if (!mb || mb->name != "broadcast_in_dim" || sel->operands[0]->users.size() != 1 || mb->ints("dims") != std::vector<int64_t>{0, 1, 2, 3}) return false;
+      if (!splatFloat(sel->operands[2], neg)) return false;
+      Value* ms = mb->operands[0];
+      if (ms->type.dt != DType::Pred || ms->type.rank() != 4) return false;
+      for (int d = 0; d < 4; ++d) if (ms->type.dims[(size_t)d] != 1 && ms->type.dims[(size_t)d] != x->type.dims[(size_t)d]) return false;
+      m.mask = ms;
+      m.masked = neg;
+      m.absorbed.push_back(sel);
+      m.absorbed.push_back(mb);
+      x = sel->operands[1];
+      if (x->users.size() != 1) return false;
+    }
+    if (x->def && x->def->name == "multiply") {
+      Op* mu = x->def;
+      float sc = 1.f;
+      Value* other = nullptr;
+      if (splatFloat(mu->operands[1], sc)) other = mu->operands[0];
+      else if (splatFloat(mu->operands[0], sc)) other = mu->operands[1];
+      else return false;
+      m.scale = sc;
+      m.absorbed.push_back(mu);
+      x = other;
+      if (x->users.size() != 1) return false;
+    }
+    Op* qk = x->def;
+    if (!qk || qk->name != "dot_general" || x->type.dt != DType::F32 || qk->parent != pv->parent) return false;
+    Value* q = qk->operands[0];
+    Value* k = qk->operands[1];
+    if (q->type.dt != DType::BF16 || k->type.dt != DType::BF16 || q->type.rank() != 4 || k->type.rank() != 4) return false;
+    if (qk->ints("lhs_batch").size() != 2 || qk->ints("rhs_batch").size() != 2) return false;
+    if (qk->ints("lhs_contract") != std::vector<int64_t>{3} || qk->ints("rhs_contract") != std::vector<int64_t>{3}) return false;
+    m.qk = qk;
+    m.absorbed.push_back(qk);
+    for (Op* o : m.absorbed) if (o->parent != pv->parent) return false;
+    // result read only by the head-merging transpose: write it in that layout
+    Value* out = pv->result();
+    if (out->users.size() == 1 && out->users[0]->name == "transpose" && out->users[0]->parent == pv->parent &&
+        out->users[0]->ints("dims") == std::vector<int64_t>{0, 2, 1, 3})
+      m.merge = out->users[0];
+    return true;
+  }
+
+  // dims of a rank-4 operand of a batched product: its two batch dims in result order, then the remaining non-contracted dim
+  static void attnDims(Op* dot, bool lhs, int& db, int& dn, int& dfree) {
+    auto& batch = dot->ints(lhs ? "lhs_batch" : "rhs_batch");
+    int64_t contract = dot->ints(lhs ? "lhs_contract" : "rhs_contract")[0];
+    db = (int)batch[0];
+    dn = (int)batch[1];
+    dfree = -1;
+    for (int d = 0; d < 4; ++d) if (d != db && d != dn && d != contract) dfree = d;
+  }
+
+  bool emitAttention(const AttnMatch& m, Plan& plan) {
+    Value* q = m.qk->operands[0];
+    Value* k = m.qk->operands[1];
+    Value* v = m.pv->operands[1];
+    Value* out = m.merge ? m.merge->result() : m.pv->result();
+    auto stored = [this](Value* x) { return hasStorage(x); };
+    View vq, vk, vv;
+    Value* ops3[3] = {q, k, v};
+    View* views[3] = {&vq, &vk, &vv};
+    Op* users[3] = {m.qk, m.qk, m.pv};
+    for (int i = 0; i < 3; ++i) {
+      Value* x = ops3[i];
+      if (!hasStorage(x) && !(dotTakesView(x, users[i]) && resolveView(x, stored, *views[i]))) materializeNow(x, plan);
+      if (hasStorage(x)) { views[i]->root = x; views[i]->offset = 0; views[i]->strides = stridesOf(x->type); }
+    }
+    AttentionDesc a;
+    int db, dn, df;
+    attnDims(m.qk, true, db, dn, df);          // q: [b, n] batch, free dim = queries, dim 3 = head
+    if (df < 0 || df == 3 || vq.strides[3] != 1) return false;
+    a.B = q->type.dims[(size_t)db]; a.N = q->type.dims[(size_t)dn]; a.T = q->type.dims[(size_t)df]; a.H = q->type.dims[3];
+    a.qB = vq.strides[(size_t)db]; a.qN = vq.strides[(size_t)dn]; a.qT = vq.strides[(size_t)df];
+    attnDims(m.qk, false, db, dn, df);
+    if (df < 0 || df == 3 || vk.strides[3] != 1) return false;
+    a.S = k->type.dims[(size_t)df];
+    a.kB = vk.strides[(size_t)db]; a.kN = vk.strides[(size_t)dn]; a.kS = vk.strides[(size_t)df];
+    {
+      auto& batch = m.pv->ints("rhs_batch");
+      int64_t contract = m.pv->ints("rhs_contract")[0];
+      if (vv.strides[3] != 1 || v->type.dims[3] != a.H || v->type.dims[(size_t)contract] != a.S) return false;
+      a.vB = vv.strides[(size_t)batch[0]]; a.vN = vv.strides[(size_t)batch[1]]; a.vS = vv.strides[(size_t)contract];
+    }
+    // result [b, n, t, h] dense, or [b, t, n, h] after the head merge
+    if (m.merge) { a.oB = a.T * a.N * a.H; a.oT = a.N * a.H; a.oN = a.H; }
+    else { a.oB = a.N * a.T * a.H; a.oN = a.T * a.H; a.oT = a.H; }
+    a.scale = m.scale;
+    a.masked = m.masked;
+    a.hasMask = m.mask != nullptr;
+    if (m.mask) {
+      if (!hasStorage(m.mask)) materializeNow(m.mask, plan);
+      auto ms = stridesOf(m.mask->type);
+      auto md = m.mask->type.dims;
+      a.mB = md[0] == 1 ? 0 : ms[0]; a.mN = md[1] == 1 ? 0 : ms[1]; a.mT = md[2] == 1 ? 0 : ms[2]; a.mS = md[3] == 1 ? 0 : ms[3];
+    }
+    mi355_attention_desc abi = toAbi(a);
+    if (!mi355_attention_supported(&abi)) return false;
+    if ((vq.offset | vk.offset | vv.offset) % 8 != 0) return false;
+    int sid = newStorage(out->type.bytes());
+    bind(out, sid);
+    int t = ++time_;
+    Step s;
+    s.kind = Step::Attention;
+    s.time = t;
+    s.label = "attention " + q->type.str() + (m.mask ? " masked" : "") + (m.merge ? " + head merge" : "");
+    s.attn = a;
+    s.args = {ref(storageOf(vq.root), t), ref(storageOf(vk.root), t), ref(storageOf(vv.root), t), ref(sid, t)};
+    s.args[0].offset = vq.offset * 2;
+    s.args[1].offset = vk.offset * 2;
+    s.args[2].offset = vv.offset * 2;
+    if (m.mask) s.args.push_back(ref(storageOf(m.mask), t));
+    plan.steps.push_back(std::move(s));
+    for (Op* o : m.absorbed) emitted_.insert(o);
+    if (m.merge) emitted_.insert(m.merge);
+    return true;
   }
 
   void emitSort(Op* op, Plan& plan) {
@@ -1582,7 +1809,7 @@ class Planner {
 
   void dumpPlan(const Plan& p, int indent) {
     std::ostringstream o;
-    static const char* kinds[] = {"kernel", "gemm", "conv", "scatter", "copy", "fill", "while", "case", "gemm-group"};
+    static const char* kinds[] = {"kernel", "gemm", "conv", "scatter", "copy", "fill", "while", "case", "gemm-group", "attention"};
     for (auto& s : p.steps) {
       o << std::string(indent, ' ') << kinds[s.kind] << " " << s.label;
       if (s.kind == Step::Kernel) o << " k" << s.kernel << " grid " << s.grid[0] << "x" << s.grid[1] << " bytes " << s.algoBytes;
@@ -1616,6 +1843,15 @@ mi355_gemm_desc toAbi(const GemmDesc& g) {
   d.bB0 = g.bB0; d.bB1 = g.bB1; d.bRow = g.bRow; d.bCol = g.bCol;
   d.in_dtype = abiDtypeCode(g.inType);
   d.out_dtype = abiDtypeCode(g.outType);
+  return d;
+}
+
+mi355_attention_desc toAbi(const AttentionDesc& a) {
+  mi355_attention_desc d;
+  d.B = a.B; d.N = a.N; d.T = a.T; d.S = a.S; d.H = a.H;
+  d.qB = a.qB; d.qN = a.qN; d.qT = a.qT; d.kB = a.kB; d.kN = a.kN; d.kS = a.kS; d.vB = a.vB; d.vN = a.vN; d.vS = a.vS;
+  d.oB = a.oB; d.oN = a.oN; d.oT = a.oT; d.mB = a.mB; d.mN = a.mN; d.mT = a.mT; d.mS = a.mS;
+  d.scale = a.scale; d.masked = a.masked;
   return d;
 }
 

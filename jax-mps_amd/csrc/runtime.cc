@@ -335,6 +335,7 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
   switch (s.kind) {
     case Step::Kernel: kind = s.label.rfind("reduce", 0) == 0 ? "reduce" : "fusion"; bytes = (double)s.algoBytes; break;
     case Step::Gemm: kind = "gemm"; flops = 2.0 * s.gemm.batch0 * s.gemm.batch1 * s.gemm.M * s.gemm.N * (s.gemm.K + (s.dual ? s.gemm2.K : 0)); break;
+    case Step::Attention: kind = "attention"; flops = 4.0 * s.attn.B * s.attn.N * s.attn.T * s.attn.S * s.attn.H; break;
     case Step::GemmGroup:
       kind = "gemm";
       for (auto& part : s.parts) flops += 2.0 * part.gemm.batch0 * part.gemm.batch1 * part.gemm.M * part.gemm.N * (part.gemm.K + (part.dual ? part.gemm2.K : 0));
@@ -386,6 +387,15 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       void* ws = s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
       check(mi355_gemm(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), bias, ws,
                        (size_t)s.workspaceBytes, st), "gemm");
+      break;
+    }
+    case Step::Attention: {
+      mi355_attention_desc d = toAbi(s.attn);
+      const void* mask = s.args.size() > 4 ? resolve(s.args[4], in, out) : nullptr;
+      int r = mi355_attention(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), mask,
+                              resolve(s.args[3], in, out), st);
+      if (r < 0) throw RuntimeError("attention: operands are not aligned as planned");
+      check(r, "attention");
       break;
     }
     case Step::GemmGroup: {
@@ -496,7 +506,7 @@ bool Executable::capturable(const Plan& p) {
   bool ok = true;
   for (auto& s : p.steps) {
     switch (s.kind) {
-      case Step::Kernel: case Step::Gemm: case Step::GemmGroup: case Step::Conv: case Step::ScatterRows: case Step::Copy: case Step::Fill: break;
+      case Step::Kernel: case Step::Gemm: case Step::GemmGroup: case Step::Attention: case Step::Conv: case Step::ScatterRows: case Step::Copy: case Step::Fill: break;
       case Step::While: ok = ok && s.tripCount >= 0 && capturable(*s.bodies[0]); break;   // dynamic loops read a flag back on the host
       default: ok = false; break;
     }

@@ -281,6 +281,47 @@ case("dot-sum-one-product-large", lambda b, x, wi, h, wh: b.add(b.matmul(x, wi),
 case("dot-sum-product-read-twice", lambda b, x, wi, h, wh: (lambda p, q: b.mul(b.add(p, q), q))(b.matmul(x, wi), b.matmul(h, wh)), f32(2041, 33, 70), f32(2042, 70, 45), f32(2043, 33, 19), f32(2044, 19, 45))
 
 
+# softmax(scale * q k^T [masked]) v as JAX's XLA path spells it: one fused launch when the operands are bf16 (tests/
+# test_gpu_ops.py holds bf16 results to 2e-2); layouts, tails, masks and head sizes the fused kernel has to get right
+def _sdpa(b, q, k, v, mask=None, scale=None, layout="BTNH", merge=True):
+    import math as _m
+    if layout == "BTNH":
+        logits = b.dot_general(q, k, ([3], [3]), ([0, 2], [0, 2]), out_dtype="f32")          # B N T S
+    else:
+        logits = b.dot_general(q, k, ([3], [3]), ([0, 1], [0, 1]), out_dtype="f32")
+    if scale is not None:
+        logits = b.mul(logits, float(scale))
+    if mask is not None:
+        keep = b.compare(mask, 0, "NE")
+        logits = b.select(b.broadcast_in_dim(keep, logits.shape, [0, 1, 2, 3]), logits, b.full_like(logits, float(-0.7 * np.finfo(np.float32).max)))
+    from jax_mps_amd.programs.configs import softmax as _softmax
+    probs = b.convert(_softmax(b, logits, -1), q.dtype)
+    if layout == "BTNH":
+        enc = b.dot_general(probs, v, ([3], [1]), ([0, 1], [0, 2]))                             # B N T H
+    else:
+        enc = b.dot_general(probs, v, ([3], [2]), ([0, 1], [0, 1]))
+    if merge:
+        bt, n, t, h = enc.shape
+        enc = b.reshape(b.transpose(enc, [0, 2, 1, 3]), (bt, t, n * h))
+    return enc
+
+
+_B16 = ["bf16", "bf16", "bf16"]
+case("attention-bf16-128x128-h64", lambda b, q, k, v: _sdpa(b, q, k, v, scale=0.125), f32(2200, 2, 128, 3, 64, lo=-1, hi=1), f32(2201, 2, 128, 3, 64, lo=-1, hi=1), f32(2202, 2, 128, 3, 64, lo=-1, hi=1), dtypes=_B16)
+case("attention-bf16-tails", lambda b, q, k, v: _sdpa(b, q, k, v, scale=0.125), f32(2203, 2, 50, 2, 64, lo=-1, hi=1), f32(2204, 2, 70, 2, 64, lo=-1, hi=1), f32(2205, 2, 70, 2, 64, lo=-1, hi=1), dtypes=_B16)
+case("attention-bf16-key-mask", lambda b, q, k, v, m: _sdpa(b, q, k, v, mask=m, scale=0.125), f32(2206, 3, 40, 2, 64, lo=-1, hi=1), f32(2207, 3, 96, 2, 64, lo=-1, hi=1),
+     f32(2208, 3, 96, 2, 64, lo=-1, hi=1), (rng(2209).uniform(size=(3, 1, 1, 96)) < 0.7).astype(np.int32), dtypes=_B16 + ["i32"])
+case("attention-bf16-full-mask", lambda b, q, k, v, m: _sdpa(b, q, k, v, mask=m, scale=0.2), f32(2210, 2, 64, 2, 64, lo=-1, hi=1), f32(2211, 2, 64, 2, 64, lo=-1, hi=1),
+     f32(2212, 2, 64, 2, 64, lo=-1, hi=1), np.tril(np.ones((64, 64), np.int32))[None, None].repeat(2, 0), dtypes=_B16 + ["i32"])
+case("attention-bf16-h128-long-keys", lambda b, q, k, v: _sdpa(b, q, k, v, scale=0.09), f32(2213, 1, 200, 2, 128, lo=-1, hi=1), f32(2214, 1, 300, 2, 128, lo=-1, hi=1), f32(2215, 1, 300, 2, 128, lo=-1, hi=1), dtypes=_B16)
+case("attention-bf16-bnth-no-merge-no-scale", lambda b, q, k, v: _sdpa(b, q, k, v, layout="BNTH", merge=False), f32(2216, 2, 3, 72, 64, lo=-0.5, hi=0.5), f32(2217, 2, 3, 100, 64, lo=-0.5, hi=0.5),
+     f32(2218, 2, 3, 100, 64, lo=-0.5, hi=0.5), dtypes=_B16)
+case("attention-bf16-h32-not-fused", lambda b, q, k, v: _sdpa(b, q, k, v, scale=0.18), f32(2219, 2, 64, 2, 32, lo=-1, hi=1), f32(2220, 2, 64, 2, 32, lo=-1, hi=1), f32(2221, 2, 64, 2, 32, lo=-1, hi=1), dtypes=_B16)
+case("attention-bf16-probabilities-read-twice", lambda b, q, k, v: (lambda lg: [b.convert(lg, "bf16"), b.dot_general(b.convert(lg, "bf16"), v, ([3], [1]), ([0, 1], [0, 2]))])(
+     __import__("jax_mps_amd.programs.configs", fromlist=["softmax"]).softmax(b, b.dot_general(q, k, ([3], [3]), ([0, 2], [0, 2]), out_dtype="f32"), -1)),
+     f32(2222, 2, 64, 2, 64, lo=-1, hi=1), f32(2223, 2, 64, 2, 64, lo=-1, hi=1), f32(2224, 2, 64, 2, 64, lo=-1, hi=1), dtypes=_B16)
+
+
 # independent small products next to each other share one launch (the gradients of one recurrent step)
 case("dot-group-three-independent", lambda b, dz, wh, h, x: [b.dot_general(dz, wh, ([1], [1])), b.dot_general(h, dz, ([0], [0])), b.dot_general(x, dz, ([0], [0]))],
      f32(2050, 20, 96), f32(2051, 40, 96), f32(2052, 20, 40), f32(2053, 20, 24))
