@@ -252,7 +252,7 @@ case("dot-bf16-async-nn-edges", lambda b, x, y: b.matmul(x, y), f32(1950, 200, 1
 case("dot-bf16-async-nn-narrow", lambda b, x, y: b.matmul(x, y), f32(1952, 300, 64, lo=-1, hi=1), f32(1953, 64, 72, lo=-1, hi=1), dtypes=["bf16", "bf16"])
 case("dot-bf16-async-nn-batched", lambda b, x, y: b.dot_general(x, y, ([2], [1]), ([0], [0])), f32(1954, 3, 130, 64, lo=-1, hi=1), f32(1955, 3, 64, 136, lo=-1, hi=1), dtypes=["bf16", "bf16"])
 case("dot-bf16-async-nn-128x64", lambda b, x, y: b.matmul(x, y), f32(1956, 2048, 128, lo=-1, hi=1), f32(1957, 128, 3072, lo=-1, hi=1), dtypes=["bf16", "bf16"])
-case("dot-bf16-async-nn-128x128", lambda b, x, y: b.dot_general(x, y, ([1], [0]), out_dtype="f32"), f32(1958, 2048, 128, lo=-1, hi=1), f32(1959, 128, 6144, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("dot-bf16-async-nn-128x128", lambda b, x, y: b.dot_general(x, y, ([1], [0]), out_dtype="f32"), f32(1958, 4096, 128, lo=-1, hi=1), f32(1959, 128, 6144, lo=-1, hi=1), dtypes=["bf16", "bf16"])
 case("dot-bf16-async-nn-256x128", lambda b, x, y: b.matmul(x, y), f32(1960, 4096, 192, lo=-1, hi=1), f32(1961, 192, 8200, lo=-1, hi=1), dtypes=["bf16", "bf16"])
 # bias added by the GEMM kernels' own epilogue (dot_general -> add(broadcast(bias)) with no other reader of the product)
 def _linear(b, x, w, bias):
