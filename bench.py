@@ -122,6 +122,36 @@ def cpu_baseline(budget_s=12.0, batch=128):
 CONV_HBM_BYTES_PER_LAUNCH = 101.5e6
 
 
+# Algorithmic work of the other four benchmark programs (the figures the design notes quote): flops of the MFMA
+# part for the GEMM-bound one, bytes for the HBM-bound one, launches for the two that are bound by launch latency.
+def time_config(client, name, steps, warmup):
+    from jax_mps_amd import runner
+    from jax_mps_amd.programs import configs
+    p = configs.ALL[name]()
+    cp = runner.CompiledProgram(p, client)
+    for _ in range(warmup):
+        outs = cp.step()
+    outs[-1].block_until_ready()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        outs = cp.step()
+    outs[-1].block_until_ready()
+    dt = (time.perf_counter() - t0) / steps
+    ca = cp.exe.cost_analysis()
+    rec = {"config": name, "ms_per_step": round(dt * 1e3, 4), "steps_per_s": round(1 / dt, 1), "plan_steps": int(ca.get("steps", 0))}
+    if name == "distilbert":
+        rec["roofline"] = {"bound": "mfma", "unit": "TFLOP/s", "achieved": round(p.meta["flops"] / dt / 1e12, 1), "peak": 2500.0,
+                           "frac": round(p.meta["flops"] / dt / 2.5e15, 4), "note": "whole forward pass (GEMM flops / wall time), bf16"}
+    elif name == "embedding":
+        nbytes = 50.4e6 + 178.8e6      # gather: indices + rows read + rows written; scatter-add: dense result + updates + indices
+        rec["roofline"] = {"bound": "hbm", "unit": "GB/s", "achieved": round(nbytes / dt / 1e9, 1), "peak": PEAK_HBM_GBS,
+                           "frac": round(nbytes / dt / 1e9 / PEAK_HBM_GBS, 4), "note": "gather + sorted scatter-add of 8192 Zipf rows"}
+    else:
+        rec["note"] = "launch-latency bound: us per plan step = %.2f" % (dt * 1e6 / max(rec["plan_steps"], 1)) if name == "mlp" else \
+            "launch-latency bound: 2 x 100 loop iterations replayed from HIP graphs"
+    return rec
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -129,6 +159,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fused", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true")
+    ap.add_argument("--config", default=None, help="time only this benchmark program (mlp, embedding, distilbert, lstm) and print its record")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device copy (kernel copy_vec16) a few times: the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -140,6 +172,10 @@ def main():
     from jax_mps_amd import pjrt, runner
     from jax_mps_amd.programs import configs
     client = pjrt.get_client()
+    if args.config:
+        os.environ.pop("MI355X_TIMING", None)
+        print(json.dumps(time_config(client, args.config, args.steps, args.warmup)))
+        return
     p = configs.build_resnet18()
     cp = runner.CompiledProgram(p, client)
     for _ in range(args.warmup):
@@ -182,6 +218,9 @@ def main():
             o = exe.execute([buf])
         o[0].block_until_ready()
         line["copy_calibration"] = {"kernel": "copy_vec16", "bytes_read": 256 * 1024 * 1024, "bytes_written": 256 * 1024 * 1024, "launches": 5}
+    if not args.no_other_configs:
+        os.environ.pop("MI355X_TIMING", None)      # timing events would keep counted loops off their captured graphs
+        line["other_configs"] = [time_config(client, n, 50, 5) for n in ("mlp", "embedding", "distilbert", "lstm")]
     if not args.no_fused:
         os.environ["MI355X_TIMING"] = "all"
         os.environ["MI355X_TIMING_EVERY"] = "1"

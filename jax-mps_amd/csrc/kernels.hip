@@ -139,6 +139,7 @@ struct SmallPair {
   const float* a;
   const float* b;
   long long K, aB0, aB1, aRow, aCol, bB0, bB1, bRow, bCol;
+  int aVec, bVec;   // k is the contiguous, 16-byte aligned axis of the operand: four k values per load
 };
 struct SmallArgs {
   SmallPair p[2];
@@ -149,9 +150,68 @@ struct SmallArgs {
   int batch1;
 };
 
+// The MFMA contraction does not care which k a lane's operand slot stands for as long as A and B agree, so a
+// lane takes four consecutive k per "super-step" (one 16-byte load where k is contiguous, four strided loads
+// otherwise) and feeds them to four products: lane kl of a row covers k = 4 * KS * s + 4 * kl + j in product j.
+template <int T, bool AVEC, bool BVEC, typename ACC>
+__device__ __forceinline__ void smallGemmPair(const SmallPair& pr, ACC& acc, long long b0, long long b1, long long m0, long long n0, int r, int kl,
+                                              int w, bool mOk, bool nOk) {
+  constexpr int KS = T == 16 ? 4 : 2;         // k values per MFMA
+  constexpr int KSS = 4 * KS;                 // k values per super-step
+  const float* ap = pr.a + b0 * pr.aB0 + b1 * pr.aB1 + (m0 + r) * pr.aRow;
+  const float* bp = pr.b + b0 * pr.bB0 + b1 * pr.bB1 + (n0 + r) * pr.bCol;
+  const long long K = pr.K, aCol = pr.aCol, bRow = pr.bRow;
+  const long long steps = (K + KSS - 1) / KSS, per = (steps + 3) / 4;
+  const long long s0 = w * per, s1 = s0 + per < steps ? s0 + per : steps;
+  auto fetchA = [&](long long kb, float (&x)[4]) {
+    if constexpr (AVEC) {
+      const float4 t = mOk ? *(const float4*)(ap + kb) : make_float4(0.f, 0.f, 0.f, 0.f);
+      x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) x[j] = (mOk && kb + j < K) ? ap[(kb + j) * aCol] : 0.f;
+    }
+  };
+  auto fetchB = [&](long long kb, float (&x)[4]) {
+    if constexpr (BVEC) {
+      const float4 t = nOk ? *(const float4*)(bp + kb) : make_float4(0.f, 0.f, 0.f, 0.f);
+      x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) x[j] = (nOk && kb + j < K) ? bp[(kb + j) * bRow] : 0.f;
+    }
+  };
+  auto products = [&](const float (&av)[4], const float (&bv)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if constexpr (T == 16) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j], acc, 0, 0, 0);
+      else acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j], bv[j], acc, 0, 0, 0);
+    }
+  };
+  constexpr int U = 4;
+  long long s = s0;
+  for (; s + U <= s1; s += U) {
+    float av[U][4], bv[U][4];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const long long kb = (s + u) * KSS + 4 * kl;
+      fetchA(kb, av[u]);
+      fetchB(kb, bv[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) products(av[u], bv[u]);
+  }
+  for (; s < s1; ++s) {
+    float av[4], bv[4];
+    const long long kb = s * KSS + 4 * kl;
+    fetchA(kb, av);
+    fetchB(kb, bv);
+    products(av, bv);
+  }
+}
+
 template <int T>
 __device__ __forceinline__ void smallGemmTileBody(const SmallArgs& g, unsigned bx, unsigned by, unsigned bz) {
-  constexpr int KS = T == 16 ? 4 : 2;         // k values per MFMA
   constexpr int NACC = T == 16 ? 4 : 16;
   typedef float accv __attribute__((ext_vector_type(NACC)));
   __shared__ float red[4][T * T];
@@ -163,33 +223,11 @@ __device__ __forceinline__ void smallGemmTileBody(const SmallArgs& g, unsigned b
   accv acc = {0};
   for (int q = 0; q < g.pairs; ++q) {
     const SmallPair& pr = g.p[q];
-    const float* ap = pr.a + b0 * pr.aB0 + b1 * pr.aB1 + (m0 + r) * pr.aRow;
-    const float* bp = pr.b + b0 * pr.bB0 + b1 * pr.bB1 + (n0 + r) * pr.bCol;
-    const long long K = pr.K, aCol = pr.aCol, bRow = pr.bRow;
-    const long long steps = (K + KS - 1) / KS, per = (steps + 3) / 4;
-    const long long s0 = w * per, s1 = s0 + per < steps ? s0 + per : steps;
-    constexpr int U = 8;
-    long long s = s0;
-    for (; s + U <= s1; s += U) {
-      float av[U], bv[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const long long k = (s + u) * KS + kl;
-        av[u] = (mOk && k < K) ? ap[k * aCol] : 0.f;
-        bv[u] = (nOk && k < K) ? bp[k * bRow] : 0.f;
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        if constexpr (T == 16) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], bv[u], acc, 0, 0, 0);
-        else acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u], bv[u], acc, 0, 0, 0);
-      }
-    }
-    for (; s < s1; ++s) {
-      const long long k = s * KS + kl;
-      const float a1 = (mOk && k < K) ? ap[k * aCol] : 0.f;
-      const float b1v = (nOk && k < K) ? bp[k * bRow] : 0.f;
-      if constexpr (T == 16) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b1v, acc, 0, 0, 0);
-      else acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1v, acc, 0, 0, 0);
+    switch (pr.aVec * 2 + pr.bVec) {   // uniform; the loaders are compile-time so that their loads batch
+      case 0: smallGemmPair<T, false, false>(pr, acc, b0, b1, m0, n0, r, kl, w, mOk, nOk); break;
+      case 1: smallGemmPair<T, false, true>(pr, acc, b0, b1, m0, n0, r, kl, w, mOk, nOk); break;
+      case 2: smallGemmPair<T, true, false>(pr, acc, b0, b1, m0, n0, r, kl, w, mOk, nOk); break;
+      default: smallGemmPair<T, true, true>(pr, acc, b0, b1, m0, n0, r, kl, w, mOk, nOk); break;
     }
   }
 #pragma unroll
@@ -694,6 +732,11 @@ static SmallPair smallPair(const mi355_gemm_desc* d, const void* a, const void* 
   p.K = d->K;
   p.aB0 = d->aB0; p.aB1 = d->aB1; p.aRow = d->aRow; p.aCol = d->aCol;
   p.bB0 = d->bB0; p.bB1 = d->bB1; p.bRow = d->bRow; p.bCol = d->bCol;
+  // 16-byte loads along k: k contiguous, every row / batch offset a multiple of 4 floats, no ragged last super-step
+  const bool whole = d->K % 16 == 0;
+  auto mult4 = [](long long x) { return x % 4 == 0; };
+  p.aVec = whole && d->aCol == 1 && mult4(d->aRow) && mult4(d->aB0) && mult4(d->aB1) && ((uintptr_t)a & 15) == 0;
+  p.bVec = whole && d->bRow == 1 && mult4(d->bCol) && mult4(d->bB0) && mult4(d->bB1) && ((uintptr_t)b & 15) == 0;
   return p;
 }
 
