@@ -1512,6 +1512,91 @@ class Planner {
     }
   }
 
+  // ---------------------------------------------------------------- loop carries written in place
+  // A value a loop body yields normally lands in a temporary and is copied to the carry's slot at the end of the
+  // iteration.  The kernel that produces it may write the slot directly when nothing still needs the old carry:
+  // no step after the producer reads the slot, and the producer itself reads it (if at all) element for element
+  // at the position it writes (c' = f * c + i * g).
+  static bool sameShapeElementwise(const Op& op) {
+    static const std::set<std::string> moves = {"broadcast_in_dim", "reshape", "transpose", "slice", "dynamic_slice", "pad", "concatenate", "gather",
+                                                "reverse", "iota", "dynamic_update_slice", "bitcast_convert", "constant"};
+    if (!isFusibleOp(op) || op.results.size() != 1 || moves.count(op.name)) return false;
+    for (auto* o : op.operands) if (o->type.dims != op.results[0]->type.dims) return false;
+    return true;
+  }
+
+  // the kernel step `w` reads `carryArg` only at the element it computes: every path from a value the step writes
+  // down to the carry (through the values fused into the kernel) consists of same-shape elementwise ops
+  bool writerReadsAligned(Step& w, Value* carryArg) {
+    std::unordered_set<int> written;
+    forEachRef(w, [&](BufRef& r, bool wr) { if (wr) written.insert(r.index); });
+    std::vector<Value*> roots;
+    for (auto& kv : storage_) if (written.count(kv.second) && kv.first->def) roots.push_back(kv.first);
+    std::set<std::pair<Value*, bool>> seen;
+    std::function<bool(Value*, bool, int)> walk = [&](Value* v, bool aligned, int depth) -> bool {
+      if (v == carryArg) return aligned;
+      if (depth > 0 && hasStorage(v)) return true;      // another buffer: a leaf of the kernel
+      if (!seen.insert({v, aligned}).second) return true;
+      Op* d = v->def;
+      if (!d || !isFusibleOp(*d) || depth > 256) return d == nullptr || !isFusibleOp(*d) ? true : false;
+      const bool ew = sameShapeElementwise(*d);
+      for (auto* o : d->operands) if (!walk(o, aligned && ew, depth + 1)) return false;
+      return true;
+    };
+    for (auto* r : roots) if (!walk(r, true, 0)) return false;
+    return true;
+  }
+
+  static void forEachRef(Step& s, const std::function<void(BufRef&, bool)>& f) {
+    for (size_t i = 0; i < s.args.size(); ++i) {
+      bool writes = true;   // unknown layouts count as writes
+      if (s.kind == Step::Kernel) writes = i < s.argWrites.size() ? s.argWrites[i] != 0 : true;
+      else if (s.kind == Step::Gemm) writes = i == 2;
+      else if (s.kind == Step::Conv) writes = i >= 2;
+      else if (s.kind == Step::Attention) writes = i == 3;
+      else if (s.kind == Step::Copy) writes = (i & 1) != 0;
+      f(s.args[i], writes);
+    }
+    if (s.src.kind != BufRef::None) f(s.src, false);
+    if (s.dst.kind != BufRef::None) f(s.dst, true);
+    if (s.bias.kind != BufRef::None) f(s.bias, false);
+    if (s.predBuf.kind != BufRef::None) f(s.predBuf, false);
+    for (auto& part : s.parts) forEachRef(part, f);
+  }
+
+  // true if the yielded storage `from` was redirected to the carry slot `slot` throughout `body`
+  bool carryInPlace(Plan& body, int from, int slot, Value* carryArg) {
+    auto dbg = [&](const char* why) { if (getenv("MI355X_VERBOSE")) fprintf(stderr, "[mi355x] carry %s (%s) stays copied: %s\n", carryArg->name.c_str(), carryArg->type.str().c_str(), why); };
+    static const bool on = !getenv("MI355X_CARRY_IN_PLACE") || atoi(getenv("MI355X_CARRY_IN_PLACE")) != 0;
+    if (!on || st_[from].kind != BufRef::Temp || boundToOutput_.count(from)) { dbg("not a temp"); return false; }
+    int writer = -1;
+    for (size_t k = 0; k < body.steps.size(); ++k) {
+      Step& s = body.steps[k];
+      if (s.cond || !s.bodies.empty()) { dbg("nested"); return false; }
+      bool writesFrom = false;
+      forEachRef(s, [&](BufRef& r, bool w) { if (r.index == from && w) writesFrom = true; });
+      if (writesFrom) {
+        if (writer >= 0) { dbg("two writers"); return false; }
+        writer = (int)k;
+      }
+    }
+    if (writer < 0) { dbg("no writer"); return false; }
+    Step& w = body.steps[(size_t)writer];
+    if (w.kind != Step::Kernel && w.kind != Step::Gemm) { dbg("writer kind"); return false; }
+    bool writerReadsSlot = false, laterReadsSlot = false, partial = false;
+    forEachRef(w, [&](BufRef& r, bool) { if (r.index == slot) writerReadsSlot = true; if (r.index == from && r.offset != 0) partial = true; });
+    for (size_t k = (size_t)writer + 1; k < body.steps.size(); ++k)
+      forEachRef(body.steps[k], [&](BufRef& r, bool) { if (r.index == slot) laterReadsSlot = true; });
+    if (laterReadsSlot || partial) { dbg(laterReadsSlot ? "later step reads the slot" : "partial"); return false; }
+    if (writerReadsSlot && (w.kind != Step::Kernel || !writerReadsAligned(w, carryArg))) { dbg("writer reads the slot unaligned"); return false; }
+    for (auto& s : body.steps)
+      forEachRef(s, [&](BufRef& r, bool) { if (r.index == from) r.index = slot; });
+    st_[from].first = -1;   // no longer used: keep it out of the arena
+    st_[from].last = -1;
+    st_[from].uses.clear();
+    return true;
+  }
+
   void emitWhile(Op* op, Plan& plan) {
     size_t n = op->operands.size();
     for (auto* v : op->operands) if (!hasStorage(v)) materializeNow(v, plan);
@@ -1552,6 +1637,20 @@ class Planner {
       Value* v = ret->operands[i];
       if (!hasStorage(v)) materializeNow(v, *bodyPlan);
       src[i] = storageOf(v);
+    }
+    // carries whose producer can write the slot itself need no copy
+    for (size_t i = 0; i < n; ++i) {
+      if (src[i] == slots[i]) continue;
+      if (std::count(src.begin(), src.end(), src[i]) != 1) continue;
+      if (std::find(slots.begin(), slots.end(), src[i]) != slots.end()) continue;
+      // another carry receives the old value of this slot (a swap): the copies at the end still need it
+      bool slotIsSource = false;
+      for (size_t j = 0; j < n; ++j) if (j != i && src[j] == slots[i]) slotIsSource = true;
+      if (slotIsSource) continue;
+      if (carryInPlace(*bodyPlan, src[i], slots[i], body.args[i].get())) {
+        storage_[ret->operands[i]] = slots[i];
+        src[i] = slots[i];
+      }
     }
     // phase 1: values that live in another carry slot are staged through temporaries
     std::vector<std::array<int, 2>> stage, update;

@@ -508,6 +508,24 @@ def _swap(b, x, y):
 case("while-swapped-carries", _swap, f32(285, 4), f32(286, 4), exact=True)
 
 
+# loop carries written in place by their producer: the cases where that is and is not allowed
+def _loop(b, init, body, trips=5):
+    z = b.constant(0, "i32")
+    r = b.while_loop([z] + list(init), lambda i, *c: b.compare(i, trips, "LT"), lambda i, *c: [b.add(i, 1)] + list(body(i, *c)))
+    return r[1:]
+
+
+case("while-carry-in-place-elementwise", lambda b, c, f: _loop(b, [c], lambda i, cc: [b.add(b.mul(cc, f), 1.0)]), f32(2300, 6, 40), f32(2301, 6, 40, lo=0.5, hi=1.0), exact=True)
+case("while-carry-two-updated-together", lambda b, x, y: _loop(b, [x, y], lambda i, p, q: [b.add(p, q), b.sub(p, q)]), f32(2302, 33), f32(2303, 33, lo=-0.1, hi=0.1))
+case("while-carry-read-shifted-by-producer", lambda b, x: _loop(b, [x], lambda i, p: [b.add(p, b.reverse(p, [0]))]), f32(2304, 64, lo=-0.1, hi=0.1))
+case("while-carry-rolled", lambda b, x: _loop(b, [x], lambda i, p: [b.concatenate([b.slice(p, [1], [50]), b.slice(p, [0], [1])], 0)]), f32(2305, 50), exact=True)
+case("while-carry-old-value-read-after-producer", lambda b, x, w: _loop(b, [x, b.zeros((8, 8))], lambda i, p, acc: (lambda pn: [pn, b.add(acc, b.matmul(p, w))])(b.add(p, 1.0))),
+     f32(2306, 8, 8, lo=-0.5, hi=0.5), f32(2307, 8, 8, lo=-0.5, hi=0.5))
+case("while-carry-new-value-read-after-producer", lambda b, x, w: _loop(b, [x, b.zeros((8, 8))], lambda i, p, acc: (lambda pn: [pn, b.add(acc, b.matmul(pn, w))])(b.mul(p, 0.9))),
+     f32(2308, 8, 8, lo=-0.5, hi=0.5), f32(2309, 8, 8, lo=-0.5, hi=0.5))
+case("while-carry-broadcast-row-of-itself", lambda b, x: _loop(b, [x], lambda i, p: [b.add(p, b.broadcast_in_dim(b.reshape(b.slice(p, [0, 0], [1, 16]), (16,)), (4, 16), [1]))]), f32(2310, 4, 16, lo=-0.1, hi=0.1))
+
+
 def _case3(b, idx, x):
     return b.case(idx, [lambda: b.mul(x, 2.0), lambda: b.add(x, 10.0), lambda: b.neg(x)], [(x.shape, "f32")])[0]
 
