@@ -1208,7 +1208,10 @@ class Planner {
       Value* other = biasAdd->operands[0] == produced ? biasAdd->operands[1] : biasAdd->operands[0];
       biasV = other->def->operands[0];
       if (!hasStorage(biasV)) {
-        if (biasV->def && isFusibleOp(*biasV->def)) materializeNow(biasV, plan);
+        // a computed bias is materialised here only when everything it reads is already in memory
+        std::unordered_set<Value*> seen;
+        int leaves = 0;
+        if (biasV->def && isFusibleOp(*biasV->def) && biasV->def->results.size() == 1 && leavesReady(biasV, {}, seen, leaves)) materializeNow(biasV, plan);
         else biasAdd = nullptr, biasV = nullptr;
       }
     }

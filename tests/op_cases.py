@@ -267,6 +267,8 @@ case("dot-bias-bf16-async", _linear, f32(1979, 200, 128, lo=-1, hi=1), f32(1980,
 case("dot-bias-bf16-tiled", _linear, f32(1982, 200, 136, lo=-1, hi=1), f32(1983, 136, 328, lo=-1, hi=1), f32(1984, 328), dtypes=["bf16", "bf16", "bf16"])
 case("dot-bias-bf16-odd", _linear, f32(1985, 37, 50, lo=-1, hi=1), f32(1986, 50, 29, lo=-1, hi=1), f32(1987, 29), dtypes=["bf16", "bf16", "bf16"])
 case("dot-bias-computed", lambda b, x, w, c: _linear(b, x, w, b.mul(c, c)), f32(1988, 33, 70), f32(1989, 70, 45), f32(1990, 45))
+case("dot-bias-depends-on-a-later-product", lambda b, x, w, v: (lambda y, z: b.add(y, b.broadcast_in_dim(b.neg(b.reshape(z, (45,))), y.shape, [1])))(b.matmul(x, w), b.matmul(v, w)),
+     f32(1994, 33, 70), f32(1995, 70, 45), f32(1996, 1, 70))
 case("dot-bias-product-read-twice", lambda b, x, w, c: (lambda y: b.mul(b.add(y, b.broadcast_in_dim(c, y.shape, [1])), y))(b.matmul(x, w)),
      f32(1991, 33, 70), f32(1992, 70, 45), f32(1993, 45))
 
