@@ -98,7 +98,11 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  // Workgroups go to the eight XCDs round-robin by linear id; tiles that are neighbours along M share window rows,
+  // so each XCD (one L2) takes a contiguous band of M tiles when the grid allows it.
+  int bx = blockIdx.x;
+  if ((gridDim.x & 7) == 0) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);
+  const int m0 = bx * BM, n0 = blockIdx.y * BN;
   const int ktBegin = blockIdx.z * p.tilesPerSplit;
   const int ktEnd = min(p.kTiles, ktBegin + p.tilesPerSplit);
 
