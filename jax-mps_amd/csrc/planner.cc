@@ -1726,6 +1726,12 @@ class Planner {
            s.grid[0] <= kBatchMaxBlocks && s.argWrites.size() == s.args.size() && batchableKernel(P.kernels[s.kernel].source);
   }
 
+  // the shared prelude never declares LDS, so any __shared__ after the kernel header belongs to the body
+  static bool ldsInBody(const std::string& source) {
+    size_t header = source.find("extern \"C\" __global__");
+    return header != std::string::npos && source.find("__shared__", header) != std::string::npos;
+  }
+
   static bool independent(const Step& a, const Step& b) {
     for (size_t i = 0; i < a.args.size(); ++i)
       for (size_t j = 0; j < b.args.size(); ++j)
@@ -1741,7 +1747,11 @@ class Planner {
       for (auto& b : steps[i].bodies) batchKernels(*b);
       if (!batchCandidate(steps[i])) { out.push_back(std::move(steps[i++])); continue; }
       size_t j = i + 1, nargs = steps[i].args.size();
+      // static LDS of the segments adds up in the combined kernel: at most four segments that use any
+      auto usesLds = [&](const Step& st) { return ldsInBody(P.kernels[st.kernel].source); };
+      size_t ldsSegments = usesLds(steps[i]) ? 1 : 0;
       while (j < steps.size() && j - i < kBatchMaxSegments && batchCandidate(steps[j]) && nargs + steps[j].args.size() <= kBatchMaxArgs) {
+        if (usesLds(steps[j])) { if (ldsSegments >= 4) break; ++ldsSegments; }
         bool ok = true;
         for (size_t k = i; k < j && ok; ++k) ok = independent(steps[k], steps[j]);
         if (!ok) break;
