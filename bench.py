@@ -161,6 +161,7 @@ def main():
     ap.add_argument("--no-fused", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true")
     ap.add_argument("--config", default=None, help="time only this benchmark program (mlp, embedding, distilbert, lstm) and print its record")
+    ap.add_argument("--fused-only", action="store_true", help="time only the fused-op bandwidth shapes and print their records")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device copy (kernel copy_vec16) a few times: the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -172,6 +173,12 @@ def main():
     from jax_mps_amd import pjrt, runner
     from jax_mps_amd.programs import configs
     client = pjrt.get_client()
+    if args.fused_only:
+        os.environ["MI355X_TIMING"] = "all"
+        os.environ["MI355X_TIMING_EVERY"] = "1"
+        os.environ["MI355X_TIMING_REPEAT"] = str(FUSED_REPEAT)
+        print(json.dumps({"fused_ops": bench_fused_ops(client)}))
+        return
     if args.config:
         os.environ.pop("MI355X_TIMING", None)
         print(json.dumps(time_config(client, args.config, args.steps, args.warmup)))

@@ -231,7 +231,16 @@ class Emitter {
   // Row programs: results of reductions finished earlier in the same kernel, as variables that
   // hold the value for the row this wavefront / workgroup owns.
   std::unordered_map<Value*, std::string> rowScalars_;
+  std::unordered_map<std::string, std::string> rowRcp_;   // row scalar variable -> variable holding its reciprocal
   std::vector<IdxDim> rowKept_;           // index of the current row over the kept dims
+  // Row programs with unrolled walks: values an earlier walk computed at the same element, as the
+  // expression that reads them back from the registers they were kept in.  A lookup that lands on one
+  // stops there (the walk is top-down, so the hits are the values closest to the roots) and is recorded.
+  std::unordered_map<std::string, std::string> seeded_;
+  std::unordered_set<std::string> seededUsed_;
+  int seededCap_ = 0;
+  std::unordered_map<std::string, Value*> keyValue_;
+  const std::unordered_map<std::string, std::string>& unguardedValues() const { return cache_.front(); }
   void shareLeavesFrom(const Emitter& o) { leaves_ = o.leaves_; leafIndex_ = o.leafIndex_; }
   void startTemporariesAt(int n) { tmp_ = n; }   // keeps the names of nested emitters apart
 
@@ -447,6 +456,14 @@ class Emitter {
       auto it = cache_[s].find(key);
       if (it != cache_[s].end()) return it->second;
     }
+    if (!seeded_.empty()) {
+      auto sd = seeded_.find(key);
+      if (sd != seeded_.end() && (seededUsed_.count(key) || (int)seededUsed_.size() < seededCap_)) {
+        seededUsed_.insert(key);
+        return sd->second;
+      }
+    }
+    keyValue_[key] = v;
     std::string r = genUncached(v, idx);
     // values emitted into the lane-invariant prologue are visible everywhere
     bool laneInv = !idx.lane() && guard_ == 0;
@@ -735,7 +752,15 @@ class Emitter {
     if (n == "add") return bin(isP ? "(" + in(0) + " || " + in(1) + ")" : "(" + in(0) + " + " + in(1) + ")");
     if (n == "subtract") return bin("(" + in(0) + " - " + in(1) + ")");
     if (n == "multiply") return bin(isP ? "(" + in(0) + " && " + in(1) + ")" : "(" + in(0) + " * " + in(1) + ")");
-    if (n == "divide") return bin(isF ? "(" + in(0) + " / " + in(1) + ")" : "idiv<" + T + ">(" + in(0) + ", " + in(1) + ")");
+    if (n == "divide") {
+      // a divisor that is one number per row (softmax's sum) is inverted once per row, not once per element
+      if (isF && !isD) {
+        std::string d = in(1);
+        auto rc = rowRcp_.find(d);
+        if (rc != rowRcp_.end()) return bin("(" + in(0) + " * " + rc->second + ")");
+      }
+      return bin(isF ? "(" + in(0) + " / " + in(1) + ")" : "idiv<" + T + ">(" + in(0) + ", " + in(1) + ")");
+    }
     if (n == "remainder") return bin(isF ? "fmod" + sfx + "(" + in(0) + ", " + in(1) + ")" : "irem<" + T + ">(" + in(0) + ", " + in(1) + ")");
     if (n == "maximum") return bin(isP ? "(" + in(0) + " || " + in(1) + ")" : "mx<" + T + ">(" + in(0) + ", " + in(1) + ")");
     if (n == "minimum") return bin(isP ? "(" + in(0) + " && " + in(1) + ")" : "mn<" + T + ">(" + in(0) + ", " + in(1) + ")");
@@ -1623,7 +1648,17 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
   // functions of it) in registers from one phase to the next instead of re-reading it
   const int64_t walks = (vecs + (wavePerRow ? 64 : 256) - 1) / (wavePerRow ? 64 : 256);
   const int walkUnroll = walks <= 8 ? (int)walks : 4;
+  // Rows of at most eight walks: the walks are unrolled with the walk number a constant, and what one walk
+  // computed per element (loaded operands, exponentials, differences) is kept in registers for the later
+  // walks that need it instead of being loaded or computed again.
+  static const bool carryOff = getenv("MI355X_ROW_CARRY") && atoi(getenv("MI355X_ROW_CARRY")) == 0;
+  const bool carry = !carryOff && walks <= 8 && walks * V <= 32;
+  const int maxCarried = 4;
+  struct Kept { std::string name, expr, type; size_t phase; bool used; };
+  std::unordered_map<std::string, Kept> kept;   // by "value|index" key
+  int keptNames = 0, keptUsed = 0;
   std::unordered_map<Value*, std::string> scalars;
+  std::unordered_map<std::string, std::string> rcps;
   std::ostringstream b;   // kernel body; the header needs the final leaf list
   if (wavePerRow) {
     b << "  const int r_tid = threadIdx.x & 63, r_step = 64;\n";
@@ -1638,7 +1673,18 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
   for (size_t i = 0; i < reduces.size(); ++i) {
     ops.push_back(makeRedOp(*reduces[i]));
     b << "  " << ops[i].accT << " red" << i << ";\n";
+    if (ops[i].accT == "float") b << "  float rcp" << i << ";\n";
   }
+  auto walkOpen = [&](std::ostringstream& o) {
+    if (carry) {
+      o << "  #pragma unroll\n  for (int it = 0; it < " << walks << "; ++it) {\n";
+      o << "    const int rv = r_tid + it * r_step;\n";
+      o << "    if (it + 1 < " << walks << " || rv < r_end) {\n";
+    } else {
+      o << "  #pragma unroll " << walkUnroll << "\n  for (int rv = r_tid; rv < r_end; rv += r_step) {\n";
+    }
+  };
+  auto walkClose = [&](std::ostringstream& o) { o << (carry ? "    }\n  }\n" : "  }\n"); };
 
   // per phase: a fresh emitter (own temporaries inside its own scope) over the shared leaf list
   std::unique_ptr<Emitter> prev;
@@ -1646,6 +1692,14 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
     auto em = std::make_unique<Emitter>(inner, V, i64);
     if (prev) em->shareLeavesFrom(*prev);
     em->rowScalars_ = scalars;
+    em->rowRcp_ = rcps;
+    if (carry) {
+      for (auto& kv : kept) {
+        em->seeded_[kv.first] = kv.second.name + "[it][v]";
+        em->bodyNames_.insert(kv.second.name);
+      }
+      em->seededCap_ = maxCarried - keptUsed;
+    }
     return em;
   };
   // index of element (row kk, position rb + v) and of the row itself
@@ -1667,6 +1721,34 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
     loopPre = em.pre_;
     em.pre_ = savedPre;
   };
+  // the text of a walk is final only when the later walks have said what they want kept
+  std::vector<std::string> walkHead, walkTail, keepStores;
+  // after a walk was generated: note what later walks took from registers, offer what this one computed
+  auto settle = [&](Emitter& em, const Index& full, size_t phase) {
+    if (!carry) return;
+    std::vector<std::string> usedKeys(em.seededUsed_.begin(), em.seededUsed_.end());
+    std::sort(usedKeys.begin(), usedKeys.end());
+    for (auto& key : usedKeys) {
+      Kept& k = kept.at(key);
+      if (k.used) continue;
+      k.used = true;
+      ++keptUsed;
+      keepStores[k.phase] += "      " + k.name + "[it][v] = " + k.expr + ";\n";
+    }
+    const std::string suffix = "|" + full.sig;
+    std::vector<std::pair<std::string, std::string>> fresh(em.unguardedValues().begin(), em.unguardedValues().end());
+    std::sort(fresh.begin(), fresh.end());   // names must not depend on hash order: the source text is the cache key
+    for (auto& kv : fresh) {
+      const std::string& key = kv.first;
+      if (key.size() <= suffix.size() || key.compare(key.size() - suffix.size(), suffix.size(), suffix) != 0 || kept.count(key)) continue;
+      auto vi = em.keyValue_.find(key);
+      if (vi == em.keyValue_.end()) continue;
+      Value* v = vi->second;
+      if (v->type.dims != shape || scalars.count(v)) continue;
+      if (v->def && (v->def->name == "constant" || v->def->name == "iota" || v->def->name == "broadcast_in_dim")) continue;
+      kept[key] = Kept{"cr" + std::to_string(keptNames++), kv.second, computeT(v->type.dt), phase, false};
+    }
+  };
 
   size_t base = 0;
   for (size_t p = 0; p < rp.phases.size(); ++p) {
@@ -1683,29 +1765,39 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
     em->pre_ = savedPre;
     std::vector<std::string> inits;
     for (auto* r : ph) inits.push_back(em->gen(r->operands[1], em->multiIndex({}, {})));
-    b << "  {\n" << em->pre_;
-    for (size_t j = 0; j < ph.size(); ++j) b << "  " << ops[base + j].accT << " acc" << j << " = " << ops[base + j].identity << ";\n";
-    b << "  #pragma unroll " << walkUnroll << "\n  for (int rv = r_tid; rv < r_end; rv += r_step) {\n";
-    b << "    const int rb = rv * " << V << ";\n" << loopPre;
-    b << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n" << em->body_.front();
-    for (size_t j = 0; j < ph.size(); ++j) b << "      acc" << j << " = " << ops[base + j].combine("acc" + std::to_string(j), vals[j]) << ";\n";
-    b << "    }\n  }\n";
+    std::ostringstream h, t;
+    h << "  {\n" << em->pre_;
+    for (size_t j = 0; j < ph.size(); ++j) h << "  " << ops[base + j].accT << " acc" << j << " = " << ops[base + j].identity << ";\n";
+    walkOpen(h);
+    h << "    const int rb = rv * " << V << ";\n" << loopPre;
+    h << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n" << em->body_.front();
+    for (size_t j = 0; j < ph.size(); ++j) t << "      acc" << j << " = " << ops[base + j].combine("acc" + std::to_string(j), vals[j]) << ";\n";
+    t << "    }\n";
+    walkClose(t);
     for (size_t j = 0; j < ph.size(); ++j) {
       const RedOp& o = ops[base + j];
       std::string a = "acc" + std::to_string(j);
-      b << "  #pragma unroll\n  for (int o = 32; o > 0; o >>= 1) " << a << " = " << o.combine(a, shflXor(o.accT, a, "o")) << ";\n";
+      t << "  #pragma unroll\n  for (int o = 32; o > 0; o >>= 1) " << a << " = " << o.combine(a, shflXor(o.accT, a, "o")) << ";\n";
       if (!wavePerRow) {
         std::string ST = o.accT == "bool" ? "int" : o.accT;
         std::string sm = "sm" + std::to_string(base + j);
-        b << "  __shared__ " << ST << " " << sm << "[4];\n";
-        b << "  if ((threadIdx.x & 63) == 0) " << sm << "[threadIdx.x >> 6] = " << a << ";\n  __syncthreads();\n";
-        b << "  " << a << " = (" << o.accT << ")" << sm << "[0];\n";
-        b << "  for (int w = 1; w < 4; ++w) " << a << " = " << o.combine(a, "(" + o.accT + ")" + sm + "[w]") << ";\n";
+        t << "  __shared__ " << ST << " " << sm << "[4];\n";
+        t << "  if ((threadIdx.x & 63) == 0) " << sm << "[threadIdx.x >> 6] = " << a << ";\n  __syncthreads();\n";
+        t << "  " << a << " = (" << o.accT << ")" << sm << "[0];\n";
+        t << "  for (int w = 1; w < 4; ++w) " << a << " = " << o.combine(a, "(" + o.accT + ")" + sm + "[w]") << ";\n";
       }
-      b << "  red" << (base + j) << " = " << roundTo(o.dt, o.combine(inits[j], a)) << ";\n";
+      t << "  red" << (base + j) << " = " << roundTo(o.dt, o.combine(inits[j], a)) << ";\n";
+      if (o.accT == "float") t << "  rcp" << (base + j) << " = 1.f / red" << (base + j) << ";\n";
     }
-    b << "  }\n";
-    for (size_t j = 0; j < ph.size(); ++j) scalars[ph[j]->result()] = "red" + std::to_string(base + j);
+    t << "  }\n";
+    walkHead.push_back(h.str());
+    walkTail.push_back(t.str());
+    keepStores.emplace_back();
+    settle(*em, full, p);
+    for (size_t j = 0; j < ph.size(); ++j) {
+      scalars[ph[j]->result()] = "red" + std::to_string(base + j);
+      if (ops[base + j].accT == "float") rcps["red" + std::to_string(base + j)] = "rcp" + std::to_string(base + j);
+    }
     base += ph.size();
     prev = std::move(em);
   }
@@ -1724,24 +1816,32 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
     em->pre_ = savedPre;
     std::vector<std::string> kvals;
     for (auto* v : rp.keptRoots) kvals.push_back(em->gen(v, keptIdx));
-    b << "  {\n" << em->pre_;
+    std::ostringstream h, t;
+    h << "  {\n" << em->pre_;
     if (!rp.fullRoots.empty()) {
-      b << "  #pragma unroll " << walkUnroll << "\n  for (int rv = r_tid; rv < r_end; rv += r_step) {\n";
-      b << "    const int rb = rv * " << V << ";\n" << loopPre;
-      for (size_t j = 0; j < rp.fullRoots.size(); ++j) b << "    Vec<" << storageT(rp.fullRoots[j]->type.dt) << ", " << V << "> ov" << j << ";\n";
-      b << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n" << em->body_.front();
-      for (size_t j = 0; j < rp.fullRoots.size(); ++j) b << "      ov" << j << ".e[v] = " << storeExpr(rp.fullRoots[j]->type.dt, vals[j]) << ";\n";
-      b << "    }\n";
+      walkOpen(h);
+      h << "    const int rb = rv * " << V << ";\n" << loopPre;
+      for (size_t j = 0; j < rp.fullRoots.size(); ++j) h << "    Vec<" << storageT(rp.fullRoots[j]->type.dt) << ", " << V << "> ov" << j << ";\n";
+      h << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n" << em->body_.front();
+      for (size_t j = 0; j < rp.fullRoots.size(); ++j) h << "      ov" << j << ".e[v] = " << storeExpr(rp.fullRoots[j]->type.dt, vals[j]) << ";\n";
+      h << "    }\n";
       for (size_t j = 0; j < rp.fullRoots.size(); ++j)
-        b << "    *(Vec<" << storageT(rp.fullRoots[j]->type.dt) << ", " << V << ">*)(outF" << j << " + (" << IT << ")kk * " << Rn << " + rb) = ov" << j << ";\n";
-      b << "  }\n";
+        h << "    *(Vec<" << storageT(rp.fullRoots[j]->type.dt) << ", " << V << ">*)(outF" << j << " + (" << IT << ")kk * " << Rn << " + rb) = ov" << j << ";\n";
+      walkClose(h);
     }
-    b << "  if (r_tid == 0) {\n";
-    for (size_t j = 0; j < rp.keptRoots.size(); ++j) b << "    outK" << j << "[kk] = " << storeExpr(rp.keptRoots[j]->type.dt, kvals[j]) << ";\n";
-    for (size_t i = 0; i < reduces.size(); ++i) b << "    outR" << i << "[kk] = " << storeExpr(ops[i].dt, "red" + std::to_string(i)) << ";\n";
-    b << "  }\n  }\n";
+    h << "  if (r_tid == 0) {\n";
+    for (size_t j = 0; j < rp.keptRoots.size(); ++j) h << "    outK" << j << "[kk] = " << storeExpr(rp.keptRoots[j]->type.dt, kvals[j]) << ";\n";
+    for (size_t i = 0; i < reduces.size(); ++i) h << "    outR" << i << "[kk] = " << storeExpr(ops[i].dt, "red" + std::to_string(i)) << ";\n";
+    h << "  }\n  }\n";
+    walkHead.push_back(h.str());
+    walkTail.push_back("");
+    keepStores.emplace_back();
+    settle(*em, full, rp.phases.size());
     prev = std::move(em);
   }
+  for (auto& kv : kept)
+    if (kv.second.used) b << "  " << kv.second.type << " " << kv.second.name << "[" << walks << "][" << V << "];\n";
+  for (size_t p = 0; p < walkHead.size(); ++p) b << walkHead[p] << keepStores[p] << walkTail[p];
 
   std::vector<std::string> outs;
   for (size_t j = 0; j < rp.fullRoots.size(); ++j) outs.push_back(storageT(rp.fullRoots[j]->type.dt) + "* __restrict__ outF" + std::to_string(j));

@@ -180,6 +180,40 @@ class Planner {
         else for (auto* l : it->second) addLeaf(mine, l);
       }
     }
+    // Small values that a much larger kernel reads through a broadcast (per-channel scales, reciprocal standard
+    // deviations, gradient coefficients): recomputing their chain for every element of the large tensor makes a
+    // memory-bound kernel arithmetic-bound, while storing them costs a few hundred bytes and usually no launch
+    // (they ride in the pass that folds the partial sums they are computed from).
+    std::unordered_set<Value*> smallStored;
+    {
+      static const bool off = getenv("MI355X_STORE_SMALL") && atoi(getenv("MI355X_STORE_SMALL")) == 0;
+      std::unordered_map<Value*, int> cost;   // arithmetic between a value and the stored values below it
+      auto opCost = [](const std::string& n) {
+        if (n == "divide" || n == "sqrt" || n == "rsqrt" || isExpensive(n)) return 100;
+        if (n == "constant" || n == "reshape" || n == "broadcast_in_dim" || n == "convert" || n == "transpose" || n == "slice") return 0;
+        return 1;
+      };
+      for (auto& op : r.ops) {
+        if (!isFusibleOp(*op) || op->results.size() != 1) continue;
+        Value* v = op->result();
+        int c = opCost(op->name);
+        for (auto* o : op->operands) {
+          auto it = cost.find(o);
+          if (it != cost.end()) c += it->second;
+        }
+        c = std::min(c, 10000);
+        const int64_t n = v->type.numel();
+        bool feedsBig = false;
+        if (!off && n >= 2 && n <= kSmallNumel)
+          for (Op* u : v->users)
+            if (u->name == "broadcast_in_dim" && u->parent == &r && u->result()->type.numel() > kSmallNumel && u->result()->type.numel() >= 16 * n) feedsBig = true;
+        if (feedsBig && c >= 100) {   // at least one division, square root or transcendental per element saved
+          smallStored.insert(v);
+          c = 0;
+        }
+        cost[v] = c;
+      }
+    }
     // reverse: materialisation decisions
     std::unordered_map<Value*, std::vector<Op*>> groups;
     for (int k = (int)r.ops.size() - 1; k >= 0; --k) {
@@ -197,7 +231,7 @@ class Planner {
         if (needMat_[ur]) addGroup(u);
         else for (Op* q : groups[ur]) addGroup(q);
       }
-      bool mat = forced || op->has("force_materialize");
+      bool mat = forced || op->has("force_materialize") || smallStored.count(v) != 0;
       if (op->name == "constant") {
         auto& d = *op->attrs.at("value").dense;
         if (!d.splat && d.type.numel() > 1) mat = true;
@@ -682,11 +716,14 @@ class Planner {
       std::unordered_set<Value*> results;
       for (auto* g : group) results.insert(g->result());
       const auto& keptDims = op->result()->type.dims;
+      std::unordered_set<Value*> counted;
       std::function<bool(Value*, bool&, int&)> can = [&](Value* v, bool& usesResult, int& budget) -> bool {
         if (results.count(v) || std::find(epilogue.begin(), epilogue.end(), v) != epilogue.end()) { usesResult = true; return true; }
         if (hasStorage(v)) return v->type.numel() <= op->result()->type.numel();   // nothing bigger than the result shape
         Op* d = v->def;
-        if (!d || !isFusibleOp(*d) || d->results.size() != 1 || d->parent != &r || needMat_[v] || --budget < 0) return false;
+        if (!d || !isFusibleOp(*d) || d->results.size() != 1 || d->parent != &r || needMat_[v]) return false;
+        if (!counted.insert(v).second) return true;   // a shared subexpression is generated once
+        if (--budget < 0) return false;
         for (auto* o : d->operands) if (!can(o, usesResult, budget)) return false;
         return true;
       };
@@ -700,6 +737,7 @@ class Planner {
         bool uses = false;
         int budget = 64;
         bool ok = true;
+        counted.clear();
         for (auto* o : y->operands) if (!can(o, uses, budget)) ok = false;
         if (!ok || !uses) continue;
         epilogue.push_back(w);
