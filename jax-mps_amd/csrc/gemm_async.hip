@@ -22,6 +22,12 @@
 // Pipeline per iteration: wait until the oldest stage has landed (vmcnt), barrier, start the
 // loads that refill the stage consumed one iteration ago, multiply the landed stage.  One
 // barrier per 64-wide K-slab; loads are (STAGES-1) slabs ahead of the math.
+//
+// Every ring stage is an LDS array of its own and the K loop is unrolled by the ring length, so each
+// direct load and each operand read names its stage at compile time.  The compiler has to order LDS
+// reads after direct loads into LDS that may alias them; with one array for the whole ring it cannot
+// tell the stage being refilled from the stage being read and waits for every outstanding load
+// (vmcnt(0)) before the first operand read of each iteration, which serialises load and math.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -65,6 +71,16 @@ constexpr int vmcntImm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | 
 template <int BN>
 __device__ __forceinline__ int swzB(int k) { return BN == 64 ? ((k >> 1) & 1) << 2 : (k & 3) << 2; }
 
+// one LDS array per (size, stage): distinct objects, so accesses to different stages provably do not alias
+template <int BYTES, int S>
+__device__ __forceinline__ unsigned char* stageBase() {
+  __shared__ __attribute__((aligned(1024))) unsigned char buf[BYTES];
+  return buf;
+}
+
+template <int N>
+struct Const { static constexpr int value = N; };
+
 template <int BM, int BN, int STAGES, bool BNN>
 __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
   constexpr int BK = 64;
@@ -72,7 +88,6 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
   constexpr int STAGE_BYTES = (BM + BN) * 128;
   constexpr int NI = (BM + BN) / 32;          // direct loads per wavefront per stage (8 rows each)
   static_assert((STAGES - 2) * NI <= 63, "vmcnt range");
-  extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
 
@@ -114,12 +129,12 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
     }
   }
   const int nk = (int)(g.K / BK);
-  auto issue = [&](int slab) {
-    const int buf = slab % STAGES;
+  auto issue = [&](auto stage, int slab) {   // stage == slab % STAGES, as a compile-time constant
+    unsigned char* ring = stageBase<STAGE_BYTES, decltype(stage)::value>();
     const long long k0 = (long long)(slab < nk ? slab : nk - 1) * BK;   // past the end: harmless re-read keeps the count uniform
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
-      unsigned char* dst = ring + buf * STAGE_BYTES + (j * 4 + wave) * 1024;
+      unsigned char* dst = ring + (j * 4 + wave) * 1024;
       // loads j >= BM/32 fill the B part; an n-contiguous B advances by rows
       const long long step = (BNN && j >= BM / 32) ? k0 * g.bLd : k0;
       __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[j] + step), LDS_PTR(dst), 16, 0, 0);
@@ -134,8 +149,10 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-#pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s) issue(s);
+  issue(Const<0>(), 0);
+  if constexpr (STAGES > 2) issue(Const<1>(), 1);
+  if constexpr (STAGES > 3) issue(Const<2>(), 2);
+  static_assert(STAGES >= 2 && STAGES <= 4, "ring length");
 
   // fragment addresses: row-dependent part of the swizzle is fixed per lane
   const int arow = wm * (BM / 2) + (lane & 31);
@@ -154,11 +171,12 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
       bOff[j] = BM * 128 + kLane * (BN * 2) + ((slot ^ swzB<BN>(kLane)) << 4) + ((d & 1) << 3);
     }
   }
-  for (int it = 0; it < nk; ++it) {
+  auto step = [&](auto stage, int it) {
+    constexpr int S = decltype(stage)::value;
     __builtin_amdgcn_s_waitcnt(vmcntImm((STAGES - 2) * NI));
     __builtin_amdgcn_s_barrier();
-    issue(it + STAGES - 1);
-    const unsigned char* st = ring + (it % STAGES) * STAGE_BYTES;
+    issue(Const<(S + STAGES - 1) % STAGES>(), it + STAGES - 1);
+    const unsigned char* st = stageBase<STAGE_BYTES, S>();
     // fragments of k-step kk+1 are requested before the products of k-step kk are issued
     bf16x8 av[2][TM], bv[2][TN];
     auto frags = [&](int kk, int p) {
@@ -194,7 +212,18 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
     }
     // every fragment read of this stage has returned before the next barrier lets a refill start
     __builtin_amdgcn_s_waitcnt((15) | (3 << 14) | (7 << 4) | (0 << 8));
+  };
+  int it = 0;
+  for (; it + STAGES <= nk; it += STAGES) {   // whole turns of the ring, no branches inside
+    step(Const<0>(), it);
+    step(Const<1>(), it + 1);
+    if constexpr (STAGES > 2) step(Const<2>(), it + 2);
+    if constexpr (STAGES > 3) step(Const<3>(), it + 3);
   }
+  // the last partial turn (nk is uniform, so every wavefront takes the same steps)
+  if (it < nk) step(Const<0>(), it);
+  if (it + 1 < nk) step(Const<1>(), it + 1);
+  if constexpr (STAGES > 3) { if (it + 2 < nk) step(Const<2>(), it + 2); }
   __builtin_amdgcn_s_waitcnt(vmcntImm(0));   // drain the tail loads before the workgroup's LDS is released
 
   const long long cBase = bz * g.M * g.N;
@@ -225,13 +254,7 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
 
 template <int BM, int BN, int STAGES, bool BNN>
 int launch(const AsyncArgs& g, hipStream_t st) {
-  constexpr int bytes = STAGES * (BM + BN) * 128;
-  static bool configured = false;   // per process; the attribute is per function, not per device state that changes
-  if (!configured) {
-    if (hipFuncSetAttribute((const void*)gemm_bf16_async<BM, BN, STAGES, BNN>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return 3;
-    configured = true;
-  }
-  gemm_bf16_async<BM, BN, STAGES, BNN><<<dim3((unsigned)g.total), 256, bytes, st>>>(g);
+  gemm_bf16_async<BM, BN, STAGES, BNN><<<dim3((unsigned)g.total), 256, 0, st>>>(g);   // the ring is static LDS
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 
@@ -382,7 +405,21 @@ extern "C" int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, co
   g.tilesN = (int)((d->N + bn - 1) / bn);
   g.total = (long long)g.tilesM * g.tilesN * nb;
   if (g.total > 0x7FFFFFFFll) return -1;
-  // two ring stages keep two workgroups resident per compute unit, which hides more than a deeper ring does
+  // two ring stages keep three workgroups of 128x64 resident per compute unit; deeper rings (MI355X_GEMM_STAGES=3|4, a tuning aid)
+  // leave room for fewer and measured slower on the benchmark shapes: twelve resident wavefronts hide more than a third stage
+  static const int stagesEnv = getenv("MI355X_GEMM_STAGES") ? atoi(getenv("MI355X_GEMM_STAGES")) : 0;
+  if (pb.rowsOfK && stagesEnv) {
+    if (bm == 128 && bn == 128) {
+      if (stagesEnv == 3) return launch<128, 128, 3, true>(g, st);
+      if (stagesEnv == 4) return launch<128, 128, 4, true>(g, st);
+    } else if (bm == 128) {
+      if (stagesEnv == 3) return launch<128, 64, 3, true>(g, st);
+      if (stagesEnv == 4) return launch<128, 64, 4, true>(g, st);
+    } else if (bm == 64) {
+      if (stagesEnv == 3) return launch<64, 64, 3, true>(g, st);
+      if (stagesEnv == 4) return launch<64, 64, 4, true>(g, st);
+    }
+  }
   if (pb.rowsOfK) {
     if (bm == 256) return launch<256, 128, 3, true>(g, st);
     if (bm == 128 && bn == 128) return launch<128, 128, 2, true>(g, st);
