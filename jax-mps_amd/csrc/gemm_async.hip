@@ -59,6 +59,8 @@ struct AsyncArgs {
   int outBf16;
   int tilesM, tilesN;
   long long total;
+  int act;                 // 1: y = actA * x * (1 + tanh(actC * (x + actB * x^3))) on the stored value (bf16 results)
+  float actA, actB, actC;
 };
 
 __device__ __forceinline__ u16 to_bf16(float f) { return __builtin_bit_cast(u16, (__bf16)f); }
@@ -243,6 +245,12 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
         if (g.outBf16) {
           u16 r = to_bf16(acc[i][j][e]);
           if (g.bias) r = to_bf16(__uint_as_float((u32)r << 16) + bias);
+          if (g.act == 1) {
+            const float x = __uint_as_float((u32)r << 16);
+            const float u = g.actC * (x + g.actB * (x * x * x));
+            const float ex = __expf(2.f * fminf(u, 20.f));   // 1 + tanh(u) = 2 e^(2u) / (1 + e^(2u)): no cancellation for negative u
+            r = to_bf16(g.actA * x * (2.f * ex * __builtin_amdgcn_rcpf(1.f + ex)));
+          }
           ((u16*)g.c)[cBase + row * g.N + col] = r;
         } else {
           ((float*)g.c)[cBase + row * g.N + col] = acc[i][j][e] + bias;
@@ -379,6 +387,8 @@ extern "C" int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, co
   g.bB0 = d->bB0; g.bB1 = d->bB1; g.bLd = pb.ld;
   g.batch1 = (int)d->batch1;
   g.outBf16 = d->out_dtype == 1;
+  if (d->act && !g.outBf16) return -1;
+  g.act = d->act; g.actA = d->act_a; g.actB = d->act_b; g.actC = d->act_c;
   unsigned char* ws = (unsigned char*)workspace;
   if (pa.copy) {
     if (int r = transposeInto((const u16*)a, (u16*)ws, d->K, d->M, d->aCol, d, d->aB0, d->aB1, st)) return r;

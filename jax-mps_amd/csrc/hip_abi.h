@@ -66,6 +66,10 @@ typedef struct {
   int64_t aB0, aB1, aRow, aCol;
   int64_t bB0, bB1, bRow, bCol;
   int in_dtype, out_dtype;
+  // act 1 (bf16 results only): after the bias, y = act_a * x * (1 + tanh(act_c * (x + act_b * x^3))) on the stored
+  // (rounded) value x, computed in fp32 and rounded again: the tanh form of GELU with the program's own constants
+  int act;
+  float act_a, act_b, act_c;
 } mi355_gemm_desc;
 // `workspace` (may be NULL) holds k-contiguous copies of bf16 operands; see mi355_gemm_workspace_bytes.
 // `bias` (may be NULL): N values of the output type added to every row of C after the product has been rounded to

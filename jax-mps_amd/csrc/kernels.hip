@@ -73,13 +73,25 @@ struct GemmArgs {
   const void* bias;   // N values of the output type, or null
 };
 
-// c[r][n] += bias[n] for kernels without a bias epilogue of their own (c is already rounded to its type)
+// c[r][n] += bias[n], then the activation, for kernels without an epilogue of their own (c is already rounded to its type)
+struct ActArgs { int act; float a, b, c; };
+__device__ __forceinline__ float geluTanh(float x, const ActArgs& k) {
+  const float u = k.c * (x + k.b * (x * x * x));
+  const float e = __expf(2.f * fminf(u, 20.f));          // 1 + tanh(u) = 2 e^(2u) / (1 + e^(2u)): no cancellation for negative u
+  return k.a * x * (2.f * e * __builtin_amdgcn_rcpf(1.f + e));
+}
 template <typename T>
-__global__ void __launch_bounds__(256) gemm_add_bias(T* c, const T* bias, long long total, long long N) {
+__global__ void __launch_bounds__(256) gemm_add_bias(T* c, const T* bias, long long total, long long N, ActArgs act) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i >= total) return;
-  if constexpr (sizeof(T) == 2) c[i] = f2bf(bf2f(c[i]) + bf2f(bias[i % N]));
-  else c[i] = c[i] + bias[i % N];
+  if constexpr (sizeof(T) == 2) {
+    u16 r = c[i];
+    if (bias) r = f2bf(bf2f(r) + bf2f(bias[i % N]));
+    if (act.act == 1) r = f2bf(geluTanh(bf2f(r), act));
+    c[i] = r;
+  } else {
+    if (bias) c[i] = c[i] + bias[i % N];
+  }
 }
 
 __global__ void __launch_bounds__(256) gemm_f32_mfma(GemmArgs g) {
@@ -807,11 +819,13 @@ int mi355_gemm_small_sum(const mi355_gemm_desc* d1, const void* a1, const void* 
 }
 
 static int addBias(const mi355_gemm_desc* d, void* c, const void* bias, mi355_stream_t s) {
-  if (!bias) return 0;
+  if (d->act && d->out_dtype != 1) return 2;   // the activation epilogue exists for bf16 results only
+  if (!bias && !d->act) return 0;
+  const ActArgs act{d->act, d->act_a, d->act_b, d->act_c};
   const long long total = d->batch0 * d->batch1 * d->M * d->N;
   const unsigned grid = (unsigned)((total + 255) / 256);
-  if (d->out_dtype == 1) gemm_add_bias<u16><<<grid, 256, 0, (hipStream_t)s>>>((u16*)c, (const u16*)bias, total, d->N);
-  else gemm_add_bias<float><<<grid, 256, 0, (hipStream_t)s>>>((float*)c, (const float*)bias, total, d->N);
+  if (d->out_dtype == 1) gemm_add_bias<u16><<<grid, 256, 0, (hipStream_t)s>>>((u16*)c, (const u16*)bias, total, d->N, act);
+  else gemm_add_bias<float><<<grid, 256, 0, (hipStream_t)s>>>((float*)c, (const float*)bias, total, d->N, act);
   return check("gemm bias");
 }
 
@@ -833,6 +847,7 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
     r = mi355_gemm_bf16_tiled(d, a, b, c, s);
     if (r >= 0) return r ? r : addBias(d, c, bias, s);
   }
+  if (d->act && d->out_dtype != 1) return 2;
   if (smallGemmTile(d)) return mi355_gemm_small_sum(d, a, b, nullptr, nullptr, nullptr, c, bias, s);
   mi355_conv_desc cd;
   // strided views may start anywhere; the implicit-GEMM loaders issue 16-byte loads

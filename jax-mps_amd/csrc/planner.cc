@@ -13,6 +13,7 @@
 #include <array>
 #include <cstring>
 #include <functional>
+#include <cmath>
 #include <set>
 #include <sstream>
 #include <unordered_map>
@@ -902,6 +903,123 @@ class Planner {
     return resolveView(v, alwaysInMemory, vw);
   }
 
+
+  // ---------------------------------------------------------------- activation epilogue of a product
+  // The elementwise chain that follows a bf16 product (after its bias) is recognised by what it computes, not by
+  // how it is written: the chain is evaluated on the host at a handful of points as a function of the one value
+  // it reads, and accepted when y = a x (1 + tanh(c (x + b x^3))) fits, with a, b, c read off the evaluations
+  // (the tanh form of GELU; jax.nn.gelu(approximate=True) and hand-written variants associate the products
+  // differently and carry their constants in the tensor's own precision).
+  struct ActMatch {
+    Value* out = nullptr;
+    std::vector<Op*> ops;
+    float a = 0.f, b = 0.f, c = 0.f;
+  };
+
+  static bool splatNumber(Op* cst, double& out) {
+    auto& dd = *cst->attrs.at("value").dense;
+    if (!dd.splat && dd.type.numel() != 1) return false;
+    const uint8_t* p = dd.bytes.data();
+    switch (dd.type.dt) {
+      case DType::F32: { float f; memcpy(&f, p, 4); out = f; return true; }
+      case DType::BF16: { uint16_t h; memcpy(&h, p, 2); uint32_t u = (uint32_t)h << 16; float f; memcpy(&f, &u, 4); out = f; return true; }
+      case DType::F16: { _Float16 h; memcpy(&h, p, 2); out = (double)h; return true; }
+      case DType::S32: { int32_t i; memcpy(&i, p, 4); out = i; return true; }
+      default: return false;
+    }
+  }
+
+  // value of `v` when `x` holds `at`; false when the chain leaves the ops a scalar evaluation covers
+  static bool evalChain(Value* v, Value* x, double at, std::unordered_map<Value*, double>& memo, double& out) {
+    if (v == x) { out = at; return true; }
+    auto it = memo.find(v);
+    if (it != memo.end()) { out = it->second; return true; }
+    Op* d = v->def;
+    if (!d || d->results.size() != 1) return false;
+    const std::string& n = d->name;
+    double a = 0, b = 0;
+    bool ok = true;
+    if (n == "constant") ok = splatNumber(d, out);
+    else if (n == "broadcast_in_dim" || n == "reshape" || n == "convert") ok = evalChain(d->operands[0], x, at, memo, out);
+    else if (n == "add" || n == "subtract" || n == "multiply" || n == "divide" || n == "power") {
+      ok = evalChain(d->operands[0], x, at, memo, a) && evalChain(d->operands[1], x, at, memo, b);
+      out = n == "add" ? a + b : n == "subtract" ? a - b : n == "multiply" ? a * b : n == "divide" ? a / b : std::pow(a, b);
+    } else if (n == "tanh" || n == "negate" || n == "exponential" || n == "logistic") {
+      ok = evalChain(d->operands[0], x, at, memo, a);
+      out = n == "tanh" ? std::tanh(a) : n == "negate" ? -a : n == "exponential" ? std::exp(a) : 1.0 / (1.0 + std::exp(-a));
+    } else ok = false;
+    if (ok) memo[v] = out;
+    return ok;
+  }
+
+  // the chain of same-shape elementwise ops that is the only reader of `x` and has one value read from outside
+  bool matchActivation(Value* x, ActMatch& m) {
+    static const bool on = !getenv("MI355X_GEMM_ACT") || atoi(getenv("MI355X_GEMM_ACT")) != 0;
+    if (!on || x->type.dt != DType::BF16 || x->users.empty() || !x->def) return false;
+    Region* r = x->def->parent;
+    std::unordered_set<Op*> in;
+    std::vector<Op*> order;
+    std::vector<Value*> work{x};
+    while (!work.empty()) {
+      Value* v = work.back();
+      work.pop_back();
+      for (Op* u : v->users) {
+        if (in.count(u)) continue;
+        static const std::set<std::string> el = {"add", "subtract", "multiply", "divide", "power", "tanh", "negate", "exponential", "logistic", "convert"};
+        if (u->parent != r || !el.count(u->name) || u->results.size() != 1 || u->result()->type.dims != x->type.dims) {
+          if (v == x) return false;     // the product itself is read from outside the chain: it has to exist in memory
+          continue;                     // a reader outside the chain: v is a candidate for the chain's result
+        }
+        if (in.size() >= 32) return false;
+        in.insert(u);
+        order.push_back(u);
+        work.push_back(u->result());
+      }
+    }
+    if (in.empty()) return false;
+    // exactly one value of the chain is read from outside, and it has no reader inside
+    Value* out = nullptr;
+    for (Op* o : order) {
+      bool outside = false, inside = false;
+      for (Op* u : o->result()->users) (in.count(u) ? inside : outside) = true;
+      if (o->result()->users.empty()) outside = true;
+      if (outside && inside) return false;
+      if (outside) {
+        if (out) return false;
+        out = o->result();
+      }
+    }
+    if (!out || out->type.dt != DType::BF16) return false;
+    // every other input of the chain is a constant (checked by the evaluation); fit the three constants
+    auto f = [&](double at, double& y) {
+      std::unordered_map<Value*, double> memo;
+      return evalChain(out, x, at, memo, y);
+    };
+    double yBig, y1, y2;
+    if (!f(12.0, yBig) || !f(0.5, y1) || !f(1.0, y2)) return false;
+    const double a = yBig / (2.0 * 12.0);
+    if (!(a > 0.05 && a < 20.0)) return false;
+    const double r1 = y1 / (a * 0.5) - 1.0, r2 = y2 / (a * 1.0) - 1.0;
+    if (!(std::fabs(r1) < 1.0 && std::fabs(r2) < 1.0)) return false;
+    const double u1 = std::atanh(r1), u2 = std::atanh(r2);      // c (x + b x^3) at 0.5 and 1
+    // u1 = c (0.5 + 0.125 b), u2 = c (1 + b)  =>  b = (0.5 u2 - u1) / (u1 - 0.125 u2), c = u2 / (1 + b)
+    const double den = u1 - 0.125 * u2;
+    if (std::fabs(den) < 1e-9) return false;
+    const double b = (0.5 * u2 - u1) / den;
+    const double c = u2 / (1.0 + b);
+    if (!(c > 0.0) || !std::isfinite(b) || !std::isfinite(c)) return false;
+    for (double at : {-6.0, -3.0, -1.5, -0.7, -0.1, 0.0, 0.2, 0.9, 1.7, 2.5, 4.0, 7.0}) {
+      double y;
+      if (!f(at, y)) return false;
+      const double want = a * at * (1.0 + std::tanh(c * (at + b * at * at * at)));
+      if (!(std::fabs(y - want) <= 1e-6 * (1.0 + std::fabs(want)))) return false;
+    }
+    m.out = out;
+    m.ops = order;
+    m.a = (float)a; m.b = (float)b; m.c = (float)c;
+    return true;
+  }
+
   // ---------------------------------------------------------------- fused attention
   // dot_general(q, k) -> [* scale] -> [select(mask, ., c)] -> softmax over the keys -> convert -> dot_general(., v)
   // [-> transpose that merges the heads], every intermediate read by this chain only: one launch of the fused
@@ -1253,6 +1371,10 @@ class Planner {
         else biasAdd = nullptr, biasV = nullptr;
       }
     }
+    // ... -> tanh-form GELU read by nothing else: applied while the result is stored (bf16 products)
+    ActMatch act;
+    const bool fuseAct = !second && c->type.numel() > 0 && g.inType == DType::BF16 && g.outType == DType::BF16 &&
+                         matchActivation(biasAdd ? biasAdd->result() : produced, act);
     int sid = newStorage(c->type.bytes());
     bind(produced, sid);
     if (sumAdd) emitted_.insert(sumAdd);
@@ -1262,8 +1384,14 @@ class Planner {
     s.kind = Step::Gemm;
     s.time = t;
     s.label = "dot_general " + a->type.str() + " x " + b->type.str() + (second ? " + " + second->operands[0]->type.str() + " x " + second->operands[1]->type.str() : "") +
-              (biasV ? " + bias" : "");
+              (biasV ? " + bias" : "") + (fuseAct ? " + gelu" : "");
     s.gemm = g;
+    if (fuseAct) {
+      s.gemm.act = 1;
+      s.gemm.actA = act.a; s.gemm.actB = act.b; s.gemm.actC = act.c;
+      bind(act.out, sid);   // the step writes the activation; the chain's other values are never needed
+      for (Op* o : act.ops) emitted_.insert(o);
+    }
     s.args = {ref(storageOf(va.root), t), ref(storageOf(vb.root), t), ref(sid, t)};
     s.args[0].offset = va.offset * (int64_t)dtypeSize(a->type.dt);
     s.args[1].offset = vb.offset * (int64_t)dtypeSize(b->type.dt);
@@ -1993,6 +2121,7 @@ mi355_gemm_desc toAbi(const GemmDesc& g) {
   d.bB0 = g.bB0; d.bB1 = g.bB1; d.bRow = g.bRow; d.bCol = g.bCol;
   d.in_dtype = abiDtypeCode(g.inType);
   d.out_dtype = abiDtypeCode(g.outType);
+  d.act = g.act; d.act_a = g.actA; d.act_b = g.actB; d.act_c = g.actC;
   return d;
 }
 

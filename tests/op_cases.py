@@ -272,6 +272,34 @@ case("dot-bias-depends-on-a-later-product", lambda b, x, w, v: (lambda y, z: b.a
 case("dot-bias-product-read-twice", lambda b, x, w, c: (lambda y: b.mul(b.add(y, b.broadcast_in_dim(c, y.shape, [1])), y))(b.matmul(x, w)),
      f32(1991, 33, 70), f32(1992, 70, 45), f32(1993, 45))
 
+# tanh-form GELU after a bf16 product: applied by the GEMM kernels while they store (recognised by what the chain computes)
+def _gelu_builder(b, y):
+    from jax_mps_amd.shlo.builder import gelu_tanh
+    return gelu_tanh(b, y)
+
+
+def _gelu_jax_order(b, y):   # jax.nn.gelu(approximate=True): x * (0.5 * (1 + tanh(c * (x + 0.044715 * x^3))))
+    inner = b.mul(b.add(y, b.mul(b.mul(b.mul(y, y), y), 0.044715)), 0.7978845608028654)
+    return b.mul(y, b.mul(b.add(b.tanh(inner), 1.0), 0.5))
+
+
+case("dot-gelu-bf16-async", lambda b, x, w, c: _gelu_builder(b, _linear(b, x, w, c)), f32(2101, 256, 128, lo=-1, hi=1), f32(2102, 128, 320, lo=-1, hi=1), f32(2103, 320),
+     dtypes=["bf16", "bf16", "bf16"])
+case("dot-gelu-bf16-jax-order-no-bias", lambda b, x, w: _gelu_jax_order(b, b.matmul(x, w)), f32(2104, 200, 128, lo=-1, hi=1), f32(2105, 128, 328, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("dot-gelu-bf16-tiled", lambda b, x, w, c: _gelu_builder(b, _linear(b, x, w, c)), f32(2106, 200, 136, lo=-1, hi=1), f32(2107, 136, 328, lo=-1, hi=1), f32(2108, 328),
+     dtypes=["bf16", "bf16", "bf16"])
+case("dot-gelu-bf16-odd", lambda b, x, w, c: _gelu_jax_order(b, _linear(b, x, w, c)), f32(2109, 37, 50, lo=-2, hi=2), f32(2110, 50, 29, lo=-2, hi=2), f32(2111, 29), dtypes=["bf16", "bf16", "bf16"])
+case("dot-gelu-bf16-3d-wide-range", lambda b, x, w, c: _gelu_builder(b, _linear(b, x, w, c)), f32(2112, 4, 64, 64, lo=-3, hi=3), f32(2113, 64, 128, lo=-3, hi=3), f32(2114, 128, lo=-8, hi=8),
+     dtypes=["bf16", "bf16", "bf16"])
+case("dot-gelu-bf16-zero-cubic-term", lambda b, x, w, c: (lambda y: b.mul(b.mul(y, 0.5), b.add(b.tanh(b.mul(y, 0.8)), 1.0)))(_linear(b, x, w, c)), f32(2124, 128, 128, lo=-1, hi=1),
+     f32(2125, 128, 128, lo=-1, hi=1), f32(2126, 128), dtypes=["bf16", "bf16", "bf16"])
+# chains that must stay kernels of their own: the sum is read twice; the function is not a GELU; the result is f32
+case("dot-gelu-bf16-sum-read-twice", lambda b, x, w, c: (lambda y: b.add(_gelu_builder(b, y), y))(_linear(b, x, w, c)), f32(2115, 128, 128, lo=-1, hi=1), f32(2116, 128, 128, lo=-1, hi=1),
+     f32(2117, 128), dtypes=["bf16", "bf16", "bf16"])
+case("dot-not-gelu-bf16", lambda b, x, w, c: (lambda y: b.mul(y, b.tanh(y)))(_linear(b, x, w, c)), f32(2118, 128, 128, lo=-1, hi=1),
+     f32(2119, 128, 128, lo=-1, hi=1), f32(2120, 128), dtypes=["bf16", "bf16", "bf16"])
+case("dot-gelu-f32", lambda b, x, w, c: _gelu_builder(b, _linear(b, x, w, c)), f32(2121, 33, 70), f32(2122, 70, 45), f32(2123, 45))
+
 
 # add(dot, dot) of two small fp32 products is one launch (the recurrent cell's x*Wi + h*Wh), with the bias on top
 case("dot-sum-two-products", lambda b, x, wi, h, wh: b.add(b.matmul(x, wi), b.matmul(h, wh)), f32(2020, 33, 70), f32(2021, 70, 45), f32(2022, 33, 19), f32(2023, 19, 45))
