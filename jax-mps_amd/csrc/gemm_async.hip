@@ -93,13 +93,16 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
 
-  long long id = blockIdx.x;
-  if ((g.total & 7) == 0) id = (id & 7) * (g.total >> 3) + (id >> 3);
-  const long long perBatch = (long long)g.tilesM * g.tilesN;
-  const long long bz = id / perBatch;
-  const int t = (int)(id % perBatch);
-  const int tm = t / g.tilesN, tn = t % g.tilesN;
-  const long long b0 = bz / g.batch1, b1 = bz % g.batch1;
+  // tile decode in 32-bit arithmetic (the launcher keeps the grid below 2^31): 64-bit divisions cost hundreds of cycles each
+  unsigned id = blockIdx.x;
+  const unsigned total = (unsigned)g.total;
+  if ((total & 7u) == 0) id = (id & 7u) * (total >> 3) + (id >> 3);
+  const unsigned perBatch = (unsigned)g.tilesM * (unsigned)g.tilesN;
+  const unsigned bzu = id / perBatch;
+  const unsigned t = id - bzu * perBatch;
+  const int tm = (int)(t / (unsigned)g.tilesN), tn = (int)(t - (unsigned)tm * (unsigned)g.tilesN);
+  const long long bz = bzu;
+  const long long b0 = bzu / (unsigned)g.batch1, b1 = bzu - (unsigned)b0 * (unsigned)g.batch1;
   const u16* A = g.a + b0 * g.aB0 + b1 * g.aB1;
   const u16* B = g.b + b0 * g.bB0 + b1 * g.bB1;
   const long long m0 = (long long)tm * BM, n0 = (long long)tn * BN;
@@ -151,6 +154,14 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+  // the bias values this lane adds at the end are fetched now, behind the first slabs
+  float biasv[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const long long col = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
+    biasv[j] = 0.f;
+    if (g.bias && col < g.N) biasv[j] = g.outBf16 ? __uint_as_float((u32)((const u16*)g.bias)[col] << 16) : ((const float*)g.bias)[col];
+  }
   issue(Const<0>(), 0);
   if constexpr (STAGES > 2) issue(Const<1>(), 1);
   if constexpr (STAGES > 3) issue(Const<2>(), 2);
@@ -229,31 +240,61 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
   __builtin_amdgcn_s_waitcnt(vmcntImm(0));   // drain the tail loads before the workgroup's LDS is released
 
   const long long cBase = bz * g.M * g.N;
+  // value of accumulator element e of tile (i, j) as it is stored: bias added to the rounded product, then the activation
+  auto finish16 = [&](float v, float bias) -> u16 {
+    u16 r = to_bf16(v);
+    if (g.bias) r = to_bf16(__uint_as_float((u32)r << 16) + bias);
+    if (g.act == 1) {
+      const float x = __uint_as_float((u32)r << 16);
+      const float u = g.actC * (x + g.actB * (x * x * x));
+      const float ex = __expf(2.f * fminf(u, 20.f));   // 1 + tanh(u) = 2 e^(2u) / (1 + e^(2u)): no cancellation for negative u
+      r = to_bf16(g.actA * x * (2.f * ex * __builtin_amdgcn_rcpf(1.f + ex)));
+    }
+    return r;
+  };
+  if (g.outBf16 && (g.N & 7) == 0 && ((uintptr_t)g.c & 15) == 0) {
+    // bf16 results leave through LDS: an accumulator lane holds 16 rows of one column, so direct stores are
+    // 2-byte writes, 64 of them per instruction.  Each 64-row band of the tile is transposed through a ring
+    // stage (free by now) and written as 16-byte row segments, whole cache lines per row.
+    constexpr int LDW = BN + 8;   // staged row in elements: 16-byte aligned, consecutive rows 4 banks apart
+    static_assert(64 * LDW * 2 <= STAGE_BYTES, "a band fits one stage");
+    __syncthreads();              // every wavefront has read its last operands; all direct loads have landed
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i) {
+      u16* band = (u16*)((i & 1) ? stageBase<STAGE_BYTES, 1>() : stageBase<STAGE_BYTES, 0>());
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const long long col = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
-      if (col >= g.N) continue;
-      // bias epilogue: the product is rounded to the output type first, as the separate add would see it
-      float bias = 0.f;
-      if (g.bias) bias = g.outBf16 ? __uint_as_float((u32)((const u16*)g.bias)[col] << 16) : ((const float*)g.bias)[col];
+      for (int j = 0; j < TN; ++j) {
+        const int lc = wn * (BN / 2) + j * 32 + (lane & 31);
+        const float bias = biasv[j];
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const long long row = m0 + wm * (BM / 2) + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        if (row >= g.M) continue;
-        if (g.outBf16) {
-          u16 r = to_bf16(acc[i][j][e]);
-          if (g.bias) r = to_bf16(__uint_as_float((u32)r << 16) + bias);
-          if (g.act == 1) {
-            const float x = __uint_as_float((u32)r << 16);
-            const float u = g.actC * (x + g.actB * (x * x * x));
-            const float ex = __expf(2.f * fminf(u, 20.f));   // 1 + tanh(u) = 2 e^(2u) / (1 + e^(2u)): no cancellation for negative u
-            r = to_bf16(g.actA * x * (2.f * ex * __builtin_amdgcn_rcpf(1.f + ex)));
-          }
-          ((u16*)g.c)[cBase + row * g.N + col] = r;
-        } else {
-          ((float*)g.c)[cBase + row * g.N + col] = acc[i][j][e] + bias;
+        for (int e = 0; e < 16; ++e) {
+          const int lr = wm * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          band[lr * LDW + lc] = finish16(acc[i][j][e], bias);
+        }
+      }
+      __syncthreads();   // also orders this band's reads of the other buffer's previous use before its next writes
+      for (int sg = tid; sg < 64 * (BN / 8); sg += 256) {
+        const int lr = sg / (BN / 8), cs = sg % (BN / 8);
+        const long long row = m0 + (lr >> 5) * (BM / 2) + i * 32 + (lr & 31);
+        const long long col = n0 + cs * 8;
+        if (row < g.M && col < g.N) *(uint4*)((u16*)g.c + cBase + row * g.N + col) = *(const uint4*)(band + lr * LDW + cs * 8);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const long long col = n0 + wn * (BN / 2) + j * 32 + (lane & 31);
+        if (col >= g.N) continue;
+        // bias epilogue: the product is rounded to the output type first, as the separate add would see it
+        const float bias = biasv[j];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const long long row = m0 + wm * (BM / 2) + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          if (row >= g.M) continue;
+          if (g.outBf16) ((u16*)g.c)[cBase + row * g.N + col] = finish16(acc[i][j][e], bias);
+          else ((float*)g.c)[cBase + row * g.N + col] = acc[i][j][e] + bias;
         }
       }
     }
