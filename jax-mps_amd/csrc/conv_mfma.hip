@@ -47,6 +47,8 @@ struct ConvP {
   int s0, s1, p0, p1, ld0, ld1, rd0, rd1, rev0, rev1;
   int lhsB, lhsF, lhsS0, lhsS1, rhsI, rhsO, rhsS0, rhsS1, outB, outF, outS0, outS1;
   int bFast;            // 1: m = (o0, o1, b) with b fastest; 0: m = (b, o0, o1)
+  long long outRow;     // > 0: output row m starts at m * outRow (the usual dense layouts): no index decode when storing
+  int outVec;           // columns are contiguous and every row of the destination (output or partial sums) starts 16-byte aligned: float4 stores
   int cTiles;           // k-tiles per window tap (tap-chunk tiling)
   int kTiles;           // total k-tiles
   int splitK, tilesPerSplit;
@@ -285,7 +287,7 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
 #pragma unroll
         for (int a = 0; a < TM; ++a)
 #pragma unroll
-          for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[a], bv[b], acc[a][b], 0, 0, 0);
+          for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[b], av[a], acc[a][b], 0, 0, 0);   // operands swapped: the transposed tile
       }
       __builtin_amdgcn_s_setprio(0);
       if (more) storeTile(cur ^ 1);         // the other stage: nobody reads it during this iteration
@@ -295,26 +297,40 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
   }
 
   // ---- epilogue
+  // The products were issued with their operands swapped, so a lane holds the transposed tile: one output row
+  // (lane & 31) and, per group of four accumulator registers, four consecutive output columns.  A lane decodes one
+  // row per 32-row block instead of sixteen, and stores 16 bytes at a time where the layout allows.
   const bool partial = p.splitK > 1;
+  const bool vec = p.outVec != 0;
 #pragma unroll
   for (int a = 0; a < TM; ++a) {
+    const int m = m0 + wm * WM + a * 32 + (lane & 31);
+    if (m >= p.M) continue;
+    long long rowOff;
+    if (partial) {
+      rowOff = ((long long)blockIdx.z * p.M + m) * p.N;
+    } else if (p.outRow > 0) {
+      rowOff = (long long)m * p.outRow;
+    } else {
+      int b, o0, o1;
+      if (p.bFast) { b = m % p.Nb; int t = m / p.Nb; o1 = t % p.o1n; o0 = t / p.o1n; }
+      else { o1 = m % p.o1n; int t = m / p.o1n; o0 = t % p.o0n; b = t / p.o0n; }
+      rowOff = (long long)b * p.outB + (long long)o0 * p.outS0 + (long long)o1 * p.outS1;
+    }
+    const long long colStride = partial ? 1 : p.outF;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const int m = m0 + wm * WM + a * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
-      if (m >= p.M) continue;
-      long long rowOff;
-      if (partial) {
-        rowOff = ((long long)blockIdx.z * p.M + m) * p.N;
-      } else {
-        int b, o0, o1;
-        if (p.bFast) { b = m % p.Nb; int t = m / p.Nb; o1 = t % p.o1n; o0 = t / p.o1n; }
-        else { o1 = m % p.o1n; int t = m / p.o1n; o0 = t % p.o0n; b = t / p.o0n; }
-        rowOff = (long long)b * p.outB + (long long)o0 * p.outS0 + (long long)o1 * p.outS1;
-      }
+    for (int b = 0; b < TN; ++b) {
 #pragma unroll
-      for (int b = 0; b < TN; ++b) {
-        const int n = n0 + wn * WN + b * 32 + (lane & 31);
-        if (n < p.N) p.out[rowOff + (partial ? n : n * p.outF)] = acc[a][b][j];
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int n = n0 + wn * WN + b * 32 + g4 * 8 + (lane >> 5) * 4;
+        if (n >= p.N) continue;
+        if (vec) {
+          *(float4*)(p.out + rowOff + n) = make_float4(acc[a][b][4 * g4], acc[a][b][4 * g4 + 1], acc[a][b][4 * g4 + 2], acc[a][b][4 * g4 + 3]);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < p.N) p.out[rowOff + (n + r) * colStride] = acc[a][b][4 * g4 + r];
+        }
       }
     }
   }
@@ -573,14 +589,32 @@ static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, vo
   p.rhsI = (int)d->rhsI; p.rhsO = (int)d->rhsO; p.rhsS0 = dim(d->rhsS, 0, 0); p.rhsS1 = dim(d->rhsS, 1, 0);
   p.outB = (int)d->outB; p.outF = (int)d->outF; p.outS0 = dim(d->outS, 0, 0); p.outS1 = dim(d->outS, 1, 0);
   p.bFast = c.bFast;
+  {
+    // Is the offset of output row m linear in m?  It is a mixed-radix function of m, so agreement at the carries decides.
+    auto rowOff = [&](long long m) {
+      long long b, o0, o1;
+      if (p.bFast) { b = m % p.Nb; long long t = m / p.Nb; o1 = t % p.o1n; o0 = t / p.o1n; }
+      else { o1 = m % p.o1n; long long t = m / p.o1n; o0 = t % p.o0n; b = t / p.o0n; }
+      return b * (long long)p.outB + o0 * (long long)p.outS0 + o1 * (long long)p.outS1;
+    };
+    const long long unit = M > 1 ? rowOff(1) : 1;
+    const long long inner = p.bFast ? p.Nb : p.o1n, mid = inner * (p.bFast ? p.o1n : p.o0n);
+    bool linear = unit > 0;
+    for (long long m : {inner - 1, inner, mid - 1, mid, mid + inner, M - 1})
+      if (m > 0 && m < M && rowOff(m) != m * unit) linear = false;
+    p.outRow = linear ? unit : 0;
+  }
   p.cTiles = c.cTiles; p.kTiles = c.kTiles; p.splitK = c.splitK; p.tilesPerSplit = c.tilesPerSplit;
   float* dst = (float*)out + part.outOffset;
   if (c.splitK > 1) {
     size_t need = (size_t)c.splitK * (size_t)M * (size_t)d->O * sizeof(float);
     if (!workspace || workspace_bytes < need) return 3;   // caller sized the workspace wrong
     p.out = (float*)workspace;
+    p.outVec = (p.N & 3) == 0 && ((uintptr_t)workspace & 15) == 0;
   } else {
     p.out = dst;
+    auto mult4 = [](long long x) { return (x & 3) == 0; };
+    p.outVec = p.outF == 1 && mult4(p.N) && mult4(p.outB) && mult4(p.outS0) && mult4(p.outS1) && ((uintptr_t)dst & 15) == 0;
   }
   dim3 grid((unsigned)((p.M + c.bm - 1) / c.bm), (unsigned)((p.N + c.bn - 1) / c.bn), (unsigned)c.splitK);
   if (grid.y > 65535) return 4;
