@@ -445,10 +445,10 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
   else if (forced == 12864 || (!forced && tilesOf(128, 64) >= minTiles)) { c.bm = 128; c.bn = 64; }
   else { c.bm = 64; c.bn = 64; }
   long long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
-  // Split K until there are about `target` workgroups: several per CU, so that a tile count that is
-  // not a multiple of the CU count costs little, without exceeding it (a few stragglers would
-  // take a whole extra workgroup time).
-  static const int target = getenv("MI355X_CONV_BLOCKS") ? atoi(getenv("MI355X_CONV_BLOCKS")) : 768;
+  // Split K until there are about `target` workgroups: four per CU, which is what stays resident, so that a
+  // tile count that is not a multiple of the CU count costs little, without exceeding it (a fifth
+  // workgroup per CU waits for a whole workgroup time: 1280 measured a tenth slower than 1024).
+  static const int target = getenv("MI355X_CONV_BLOCKS") ? atoi(getenv("MI355X_CONV_BLOCKS")) : 1024;
   int split = 1;
   static const int minSplitTiles = getenv("MI355X_CONV_MIN_SPLIT_KTILES") ? atoi(getenv("MI355X_CONV_MIN_SPLIT_KTILES")) : 1;
   // (measured: splitting pays even for a short K, the shorter dependent chain per workgroup outweighs the fold launch)
