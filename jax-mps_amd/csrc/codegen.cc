@@ -1283,13 +1283,11 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     std::vector<std::string> inits;
     for (auto* r : reduces) inits.push_back(em.gen(r->operands[1], em.multiIndex({}, {})));
 
-    std::ostringstream s;
-    s << kPrelude;
+    std::ostringstream s;   // body; the header follows once an epilogue has named its inputs
     std::vector<std::string> outs;
     bool partial = P > 1;
     for (size_t j = 0; j < nr; ++j)
       outs.push_back((partial ? ops[j].accT : storageT(ops[j].dt)) + "* __restrict__ out" + std::to_string(j));
-    s << kernelHeader(em.leaves_, outs) << " {\n";
     if (wavePerRow) {
       s << "  const int lane = threadIdx.x & 63;\n";
       s << "  const " << IT << " kk = (" << IT << ")blockIdx.x * 4 + (threadIdx.x >> 6);\n";
@@ -1330,11 +1328,33 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     }
     for (size_t j = 0; j < nr; ++j) {
       if (partial) s << "  out" << j << "[((" << IT << ")blockIdx.x % " << P << ") * " << Kn << " + kk] = acc" << j << ";\n";
-      else s << "  out" << j << "[kk] = " << storeExpr(ops[j].dt, roundTo(ops[j].dt, ops[j].combine(inits[j], "acc" + std::to_string(j)))) << ";\n";
+      else {
+        s << "  const " << ops[j].accT << " res" << j << " = " << roundTo(ops[j].dt, ops[j].combine(inits[j], "acc" + std::to_string(j))) << ";\n";
+        s << "  out" << j << "[kk] = " << storeExpr(ops[j].dt, "res" + std::to_string(j)) << ";\n";
+      }
+    }
+    // one pass: the lane that holds a finished result also computes the per-output values that need nothing else
+    std::string header = kernelHeader(em.leaves_, outs);
+    if (!partial && !epilogue.empty()) {
+      for (size_t j = 0; j < nr; ++j) em.rowScalars_[reduces[j]->result()] = "res" + std::to_string(j);
+      em.rowKept_ = kd;
+      Index kidx = em.multiIndex(kd, keptShape);
+      std::string savedPre2 = em.pre_;
+      em.pre_.clear();
+      std::vector<std::string> ev;
+      for (auto* v : epilogue) ev.push_back(em.gen(v, kidx));
+      s << em.pre_;
+      em.pre_ = savedPre2;
+      for (size_t q = 0; q < epilogue.size(); ++q) {
+        s << "  outE" << q << "[kk] = " << storeExpr(epilogue[q]->type.dt, ev[q]) << ";\n";
+        outs.push_back(storageT(epilogue[q]->type.dt) + "* __restrict__ outE" + std::to_string(q));
+      }
+      header = kernelHeader(em.leaves_, outs);
+      fc.epilogueFused = true;
     }
     s << "}\n";
     Launch l;
-    l.source = s.str();
+    l.source = std::string(kPrelude) + header + " {\n" + s.str();
     l.grid[0] = (unsigned)(wavePerRow ? (Kn + 3) / 4 : Kn * P);
     l.block[0] = 256;
     for (auto* v : em.leaves_) { KArg a; a.kind = KArg::In; a.value = v; l.args.push_back(a); }
@@ -1353,6 +1373,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
       }
       l.args.push_back(a);
     }
+    if (!partial) for (auto* v : epilogue) { KArg a; a.kind = KArg::Out; a.value = v; l.args.push_back(a); }
     fc.leaves = em.leaves_;
     fc.launches.push_back(std::move(l));
     if (partial) {
