@@ -166,31 +166,46 @@ struct SmallArgs {
 // lane takes four consecutive k per "super-step" (one 16-byte load where k is contiguous, four strided loads
 // otherwise) and feeds them to four products: lane kl of a row covers k = 4 * KS * s + 4 * kl + j in product j.
 template <int T, bool AVEC, bool BVEC, typename ACC>
-__device__ __forceinline__ void smallGemmPair(const SmallPair& pr, ACC& acc, long long b0, long long b1, long long m0, long long n0, int r, int kl,
-                                              int w, bool mOk, bool nOk) {
+__device__ __forceinline__ void smallGemmPair(const SmallPair& pr, ACC& acc, long long b0, long long b1, long long rowA, long long rowB, int kl,
+                                              int w) {
   constexpr int KS = T == 16 ? 4 : 2;         // k values per MFMA
   constexpr int KSS = 4 * KS;                 // k values per super-step
-  const float* ap = pr.a + b0 * pr.aB0 + b1 * pr.aB1 + (m0 + r) * pr.aRow;
-  const float* bp = pr.b + b0 * pr.bB0 + b1 * pr.bB1 + (n0 + r) * pr.bCol;
-  const long long K = pr.K, aCol = pr.aCol, bRow = pr.bRow;
-  const long long steps = (K + KSS - 1) / KSS, per = (steps + 3) / 4;
-  const long long s0 = w * per, s1 = s0 + per < steps ? s0 + per : steps;
-  auto fetchA = [&](long long kb, float (&x)[4]) {
+  // rowA / rowB are clamped to the operand's last row: a row of A only reaches its own row of the result and a
+  // column of B its own column, and results outside M x N are never stored, so whatever the clamped lanes load
+  // is harmless and every load of a whole super-step is unconditional (a predicated load is a branch around the
+  // load: a batch of twenty of them took 1 700 cycles to issue).  Only the one ragged super-step at the end of
+  // K selects zeros, for the k beyond K.
+  const float* ap = pr.a + b0 * pr.aB0 + b1 * pr.aB1 + rowA * pr.aRow;
+  const float* bp = pr.b + b0 * pr.bB0 + b1 * pr.bB1 + rowB * pr.bCol;
+  const int K = (int)pr.K;
+  const long long aCol = pr.aCol, bRow = pr.bRow;
+  const int fullSteps = K / KSS, steps = (K + KSS - 1) / KSS, per = (steps + 3) / 4;
+  const int s0 = w * per, s1 = s0 + per < steps ? s0 + per : steps;
+  const int sFull = s1 < fullSteps ? s1 : fullSteps;
+  auto fetch = [&](int kb, float (&xa)[4], float (&xb)[4]) {
     if constexpr (AVEC) {
-      const float4 t = mOk ? *(const float4*)(ap + kb) : make_float4(0.f, 0.f, 0.f, 0.f);
-      x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
+      const float4 t = *(const float4*)(ap + kb);
+      xa[0] = t.x; xa[1] = t.y; xa[2] = t.z; xa[3] = t.w;
     } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) x[j] = (mOk && kb + j < K) ? ap[(kb + j) * aCol] : 0.f;
+      for (int j = 0; j < 4; ++j) xa[j] = ap[(kb + j) * aCol];
+    }
+    if constexpr (BVEC) {
+      const float4 t = *(const float4*)(bp + kb);
+      xb[0] = t.x; xb[1] = t.y; xb[2] = t.z; xb[3] = t.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xb[j] = bp[(kb + j) * bRow];
     }
   };
-  auto fetchB = [&](long long kb, float (&x)[4]) {
-    if constexpr (BVEC) {
-      const float4 t = nOk ? *(const float4*)(bp + kb) : make_float4(0.f, 0.f, 0.f, 0.f);
-      x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
-    } else {
+  auto fetchRagged = [&](int kb, float (&xa)[4], float (&xb)[4]) {   // never the vector layouts: those need K % 16 == 0
 #pragma unroll
-      for (int j = 0; j < 4; ++j) x[j] = (nOk && kb + j < K) ? bp[(kb + j) * bRow] : 0.f;
+    for (int j = 0; j < 4; ++j) {
+      const bool in = kb + j < K;
+      const int k = in ? kb + j : K - 1;
+      const float va = ap[k * aCol], vb = bp[k * bRow];
+      xa[j] = in ? va : 0.f;
+      xb[j] = in ? vb : 0.f;
     }
   };
   auto products = [&](const float (&av)[4], const float (&bv)[4]) {
@@ -201,23 +216,22 @@ __device__ __forceinline__ void smallGemmPair(const SmallPair& pr, ACC& acc, lon
     }
   };
   constexpr int U = 4;
-  long long s = s0;
-  for (; s + U <= s1; s += U) {
+  int s = s0;
+  for (; s + U <= sFull; s += U) {
     float av[U][4], bv[U][4];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const long long kb = (s + u) * KSS + 4 * kl;
-      fetchA(kb, av[u]);
-      fetchB(kb, bv[u]);
-    }
+    for (int u = 0; u < U; ++u) fetch((s + u) * KSS + 4 * kl, av[u], bv[u]);
 #pragma unroll
     for (int u = 0; u < U; ++u) products(av[u], bv[u]);
   }
+  for (; s < sFull; ++s) {
+    float av[4], bv[4];
+    fetch(s * KSS + 4 * kl, av, bv);
+    products(av, bv);
+  }
   for (; s < s1; ++s) {
     float av[4], bv[4];
-    const long long kb = s * KSS + 4 * kl;
-    fetchA(kb, av);
-    fetchB(kb, bv);
+    fetchRagged(s * KSS + 4 * kl, av, bv);
     products(av, bv);
   }
 }
@@ -232,14 +246,15 @@ __device__ __forceinline__ void smallGemmTileBody(const SmallArgs& g, unsigned b
   const long long m0 = (long long)by * T, n0 = (long long)bx * T;
   const int r = lane % T, kl = lane / T;
   const bool mOk = m0 + r < g.M, nOk = n0 + r < g.N;
+  const long long rowA = mOk ? m0 + r : g.M - 1, rowB = nOk ? n0 + r : g.N - 1;
   accv acc = {0};
   for (int q = 0; q < g.pairs; ++q) {
     const SmallPair& pr = g.p[q];
     switch (pr.aVec * 2 + pr.bVec) {   // uniform; the loaders are compile-time so that their loads batch
-      case 0: smallGemmPair<T, false, false>(pr, acc, b0, b1, m0, n0, r, kl, w, mOk, nOk); break;
-      case 1: smallGemmPair<T, false, true>(pr, acc, b0, b1, m0, n0, r, kl, w, mOk, nOk); break;
-      case 2: smallGemmPair<T, true, false>(pr, acc, b0, b1, m0, n0, r, kl, w, mOk, nOk); break;
-      default: smallGemmPair<T, true, true>(pr, acc, b0, b1, m0, n0, r, kl, w, mOk, nOk); break;
+      case 0: smallGemmPair<T, false, false>(pr, acc, b0, b1, rowA, rowB, kl, w); break;
+      case 1: smallGemmPair<T, false, true>(pr, acc, b0, b1, rowA, rowB, kl, w); break;
+      case 2: smallGemmPair<T, true, false>(pr, acc, b0, b1, rowA, rowB, kl, w); break;
+      default: smallGemmPair<T, true, true>(pr, acc, b0, b1, rowA, rowB, kl, w); break;
     }
   }
 #pragma unroll
