@@ -215,9 +215,17 @@ __device__ __forceinline__ void smallGemmPair(const SmallPair& pr, ACC& acc, lon
       else acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j], bv[j], acc, 0, 0, 0);
     }
   };
-  constexpr int U = 4;
-  int s = s0;
-  for (; s + U <= sFull; s += U) {
+  int s = s0;   // batches of eight, then four, super-steps of loads in flight (sixteen measured slower)
+  for (; s + 8 <= sFull; s += 8) {
+    constexpr int U = 8;
+    float av[U][4], bv[U][4];
+#pragma unroll
+    for (int u = 0; u < U; ++u) fetch((s + u) * KSS + 4 * kl, av[u], bv[u]);
+#pragma unroll
+    for (int u = 0; u < U; ++u) products(av[u], bv[u]);
+  }
+  for (; s + 4 <= sFull; s += 4) {
+    constexpr int U = 4;
     float av[U][4], bv[U][4];
 #pragma unroll
     for (int u = 0; u < U; ++u) fetch((s + u) * KSS + 4 * kl, av[u], bv[u]);
