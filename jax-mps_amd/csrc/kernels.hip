@@ -573,6 +573,20 @@ struct Bf16 {
 
 constexpr int kLongSegment = 16;   // runs at least this long go to the column-parallel kernel
 
+template <typename P, int C>
+__device__ __forceinline__ void foldShortRun(typename P::A& acc, const u32* __restrict__ vals, int cnt, const typename P::S* __restrict__ updates,
+                                             long long rowElems, long long col, int kind) {
+  u32 src[C];
+#pragma unroll
+  for (int q = 0; q < C; ++q) src[q] = vals[q < cnt ? q : cnt - 1];
+  typename P::S u[C];
+#pragma unroll
+  for (int q = 0; q < C; ++q) u[q] = updates[(long long)src[q] * rowElems + col];
+#pragma unroll
+  for (int q = 0; q < C; ++q)
+    if (q < cnt) acc = P::apply(kind, acc, u[q]);
+}
+
 // Short runs (the common case): one workgroup per run head and chunk of 256 columns; every
 // lane fetches all (< 16) updates of its column at once, then applies them in order.
 template <typename P>
@@ -587,14 +601,15 @@ __global__ void __launch_bounds__(256) scatter_fold_short(const u32* __restrict_
   if (col >= rowElems) return;
   int cnt = 1;
   while (cnt < kLongSegment && i + cnt < n && keys[i + cnt] == key) ++cnt;
-  typename P::S u[kLongSegment];
-#pragma unroll
-  for (int q = 0; q < kLongSegment - 1; ++q)
-    if (q < cnt) u[q] = updates[(long long)vals[i + q] * rowElems + col];
   typename P::A acc = P::load(result[(long long)key * rowElems + col]);
-#pragma unroll
-  for (int q = 0; q < kLongSegment - 1; ++q)
-    if (q < cnt) acc = P::apply(kind, acc, u[q]);
+  // The run length is the same for the whole workgroup; by length class, all loads of the class are issued
+  // unconditionally (positions past the run repeat its last update and are not applied), so they are in flight
+  // together instead of one branch and one round trip per update.
+  if (cnt <= 1) foldShortRun<P, 1>(acc, vals + i, cnt, updates, rowElems, col, kind);
+  else if (cnt <= 2) foldShortRun<P, 2>(acc, vals + i, cnt, updates, rowElems, col, kind);
+  else if (cnt <= 4) foldShortRun<P, 4>(acc, vals + i, cnt, updates, rowElems, col, kind);
+  else if (cnt <= 8) foldShortRun<P, 8>(acc, vals + i, cnt, updates, rowElems, col, kind);
+  else foldShortRun<P, kLongSegment - 1>(acc, vals + i, cnt, updates, rowElems, col, kind);
   result[(long long)key * rowElems + col] = P::store(acc);
 }
 
@@ -639,6 +654,7 @@ __global__ void __launch_bounds__(256) scatter_fold_long(const u32* __restrict__
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const long long col = (long long)blockIdx.y * 64 + lane;
   const bool active = col < rowElems;
+  const long long colc = active ? col : rowElems - 1;
   typename P::A acc = typename P::A();
   if (w == 0 && active) acc = P::load(result[(long long)key * rowElems + col]);
   for (long long base = head;; base += 256) {
@@ -649,17 +665,14 @@ __global__ void __launch_bounds__(256) scatter_fold_long(const u32* __restrict__
     const int cnt = __syncthreads_count(mine);   // sorted: the matches are a prefix of the tile
     for (int t0 = 0; t0 < cnt; t0 += kRound) {
       const int m = cnt - t0 < kRound ? cnt - t0 : kRound;
+      // All 32 loads of a lane are unconditional (a predicated load is a branch around it, and 32 branches issue
+      // far slower than 32 loads): positions past the run read update row sval[..] = 0 and columns past the row
+      // read the last column; neither is ever folded or stored.
       S u[kPerLane];
 #pragma unroll
-      for (int q = 0; q < kPerLane; ++q) {
-        const int r = w + kWaves * q;
-        if (r < m && active) u[q] = updates[(long long)sval[t0 + r] * rowElems + col];
-      }
+      for (int q = 0; q < kPerLane; ++q) u[q] = updates[(long long)sval[t0 + w + kWaves * q] * rowElems + colc];
 #pragma unroll
-      for (int q = 0; q < kPerLane; ++q) {
-        const int r = w + kWaves * q;
-        if (r < m && active) stage[r][lane] = u[q];
-      }
+      for (int q = 0; q < kPerLane; ++q) stage[w + kWaves * q][lane] = u[q];
       __syncthreads();
       if (w == 0 && active) {
         // the combiner is fixed outside the loop so that the LDS reads of a column pipeline
