@@ -444,6 +444,10 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
   if (forced == 128 || (!forced && N >= 128 && tilesOf(128, 128) >= minTiles)) { c.bm = 128; c.bn = 128; }
   else if (forced == 12864 || (!forced && tilesOf(128, 64) >= minTiles)) { c.bm = 128; c.bn = 64; }
   else { c.bm = 64; c.bn = 64; }
+  // At most 256 tiles of 128x128 would be split four ways or more to fill the chip; 128x64 tiles need half the split,
+  // which halves the partial sums written and folded (measured: 0.7 % of a ResNet step; 64x64 tiles with no split lose).
+  // The long-K filter gradients keep the wide tile: their output is small and their K loop is all that matters.
+  if (!forced && c.bm == 128 && c.bn == 128 && tilesOf(128, 128) <= 256 && c.kTiles < 2048) c.bn = 64;
   long long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
   // Split K until there are about `target` workgroups: four per CU, which is what stays resident, so that a
   // tile count that is not a multiple of the CU count costs little, without exceeding it (a fifth
