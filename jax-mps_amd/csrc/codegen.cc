@@ -1258,8 +1258,10 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     int64_t vecs = (Rn + V - 1) / V;
     bool wavePerRow = vecs <= 256 && Kn >= 4;
     int64_t P = 1;                 // workgroups per output row
+    static const int perThread = getenv("MI355X_REDUCE_PER_THREAD") ? atoi(getenv("MI355X_REDUCE_PER_THREAD")) : 16;
+    static const int rowUnroll = getenv("MI355X_REDUCE_UNROLL") ? atoi(getenv("MI355X_REDUCE_UNROLL")) : 4;
     if (!wavePerRow && Kn < 512 && vecs > 256 * 16) {
-      P = std::min<int64_t>((vecs + 256 * 8 - 1) / (256 * 8), std::max<int64_t>(1, 2048 / Kn));
+      P = std::min<int64_t>((vecs + 256 * perThread - 1) / (256 * perThread), std::max<int64_t>(1, 8192 / Kn));
     }
     Emitter em(isLeaf, V, i64);
     // kept index: lane-invariant
@@ -1302,7 +1304,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     }
     s << em.pre_;
     for (size_t j = 0; j < nr; ++j) s << "  " << ops[j].accT << " acc" << j << " = " << ops[j].identity << ";\n";
-    s << "  #pragma unroll 4\n  for (" << IT << " rv = r_begin + r_tid; rv < r_end; rv += r_step) {\n";
+    s << "  #pragma unroll " << rowUnroll << "\n  for (" << IT << " rv = r_begin + r_tid; rv < r_end; rv += r_step) {\n";
     s << "    const " << IT << " rb = rv * " << V << ";\n";
     s << loopPre;
     s << "    #pragma unroll\n    for (int v = 0; v < " << V << "; ++v) {\n";
@@ -1402,7 +1404,8 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   int TY = 256 / TX;
   int64_t gridX = (kvecs + TX - 1) / TX;
   int64_t P = 1;
-  if (Rn > (int64_t)TY * 16) P = std::min<int64_t>((Rn + TY * 8 - 1) / (TY * 8), std::max<int64_t>(1, 2048 / gridX));
+  static const int colPerThread = getenv("MI355X_REDUCE_COL_PER_THREAD") ? atoi(getenv("MI355X_REDUCE_COL_PER_THREAD")) : 8;
+  if (Rn > (int64_t)TY * 16) P = std::min<int64_t>((Rn + TY * colPerThread - 1) / (TY * colPerThread), std::max<int64_t>(1, 2048 / gridX));
   bool partial = P > 1;
   Emitter em(isLeaf, V, i64);
   IdxDim klin;
