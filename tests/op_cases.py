@@ -462,6 +462,40 @@ case("reduce-fused-input", lambda b, x, m: b.reduce_sum(b.mul(b.sub(x, b.broadca
 case("reduce-bf16", lambda b, x: b.reduce_sum(x, [1]), f32(267, 12, 256), dtypes=["bf16"])
 case("softmax-rows", lambda b, x: __import__("jax_mps_amd.shlo.builder", fromlist=["softmax"]).softmax(b, x, -1), f32(268, 33, 100))
 case("layer-norm", lambda b, x, s, t: __import__("jax_mps_amd.shlo.builder", fromlist=["layer_norm"]).layer_norm(b, x, s, t, 1e-5), f32(269, 20, 96), f32(270, 96), f32(271, 96))
+# row programs at row lengths that take the different walk forms: several unrolled walks with values kept in registers
+# between them (the last one ragged), one element per lane, long rows walked by loops, 16-bit rows
+def _softmax_of(b, x):
+    from jax_mps_amd.shlo.builder import softmax
+    return softmax(b, x, -1)
+
+
+def _layer_norm_of(b, x, s, t):
+    from jax_mps_amd.shlo.builder import layer_norm
+    return layer_norm(b, x, s, t, 1e-5)
+
+
+case("softmax-rows-1000", _softmax_of, f32(2730, 37, 1000, lo=-6, hi=6))
+case("softmax-rows-777", _softmax_of, f32(2731, 19, 777, lo=-6, hi=6))
+case("softmax-rows-5000", _softmax_of, f32(2732, 7, 5000, lo=-6, hi=6))
+case("softmax-rows-bf16-768", _softmax_of, f32(2733, 24, 768, lo=-4, hi=4), dtypes=["bf16"])
+case("layer-norm-768-bf16", _layer_norm_of, f32(2734, 40, 768), f32(2735, 768), f32(2736, 768), dtypes=["bf16", "bf16", "bf16"])
+case("layer-norm-1536", _layer_norm_of, f32(2737, 12, 1536), f32(2738, 1536), f32(2739, 1536))
+# per-channel chains with a division and a square root that a large kernel reads through a broadcast: stored by the pass
+# that folds the sums they depend on, or by a kernel of their own when they depend on no reduction
+def _bn_like(b, x, g):
+    n = float(x.shape[0] * x.shape[1])
+    mean = b.div(b.reduce_sum(x, [0, 1]), n)
+    var = b.sub(b.div(b.reduce_sum(b.mul(x, x), [0, 1]), n), b.mul(mean, mean))
+    scale = b.div(g, b.sqrt(b.add(b.maximum(var, 0.0), 1e-5)))
+    return b.mul(b.sub(x, b.broadcast_in_dim(mean, x.shape, [2])), b.broadcast_in_dim(scale, x.shape, [2]))
+
+
+case("per-channel-chain-after-reduce", _bn_like, f32(2740, 96, 50, 64), f32(2741, 64, lo=0.5, hi=1.5))
+case("per-channel-chain-no-reduce", lambda b, x, g, v: b.mul(x, b.broadcast_in_dim(b.div(g, b.sqrt(b.add(v, 1e-3))), x.shape, [2])),
+     f32(2742, 96, 50, 64), f32(2743, 64, lo=0.5, hi=1.5), f32(2744, 64, lo=0.1, hi=2.0))
+# a reduction finished in one launch whose per-output values ride in the same launch
+case("reduce-then-scale-one-pass", lambda b, x: b.div(b.reduce_sum(x, [0]), 300.0), f32(2745, 300, lo=-1, hi=1))
+case("reduce-rows-then-scale-one-pass", lambda b, x, w: b.mul(b.reduce_sum(x, [1]), w), f32(2746, 70, 90, lo=-1, hi=1), f32(2747, 70))
 case("argmax", lambda b, x: b.argmax(x, 1), f32(272, 9, 31), exact=True)
 case("argmax-leading-dim", lambda b, x: b.argmax(x, 0), f32(2720, 150, 7), exact=True)
 case("argmax-middle-dim-long", lambda b, x: b.argmax(x, 1), f32(2721, 3, 1000, 5), exact=True)
