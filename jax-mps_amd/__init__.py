@@ -27,41 +27,58 @@ class Mi355xPluginError(RuntimeError):
     pass
 
 
+def _candidate_libraries():
+    yield _PKG_DIR / LIB_NAME
+    yield _PKG_DIR / "lib" / LIB_NAME
+    yield Path("/usr/local/lib") / LIB_NAME
+
+
 def find_library() -> str | None:
-    """Environment override first, then next to this package (reference: __init__.py:37-61)."""
-    env = os.environ.get("MI355X_PJRT_LIBRARY_PATH")
-    if env is not None:
-        if Path(env).exists():
-            return env
-        raise Mi355xPluginError(f"MI355X_PJRT_LIBRARY_PATH is set to '{env}', but the file does not exist.")
-    for cand in (_PKG_DIR / LIB_NAME, _PKG_DIR / "lib" / LIB_NAME, Path("/usr/local/lib") / LIB_NAME):
-        if cand.exists():
-            return str(cand)
-    return None
+    """Path of the plugin library, or None.  `MI355X_PJRT_LIBRARY_PATH` wins over the search next to this
+    package and must then name an existing file (same precedence as the reference's MPS_LIBRARY_PATH,
+    src/jax_plugins/mps/__init__.py:37-61)."""
+    override = os.environ.get("MI355X_PJRT_LIBRARY_PATH")
+    if override is None:
+        return next((str(c) for c in _candidate_libraries() if c.exists()), None)
+    if not Path(override).is_file():
+        raise Mi355xPluginError(f"MI355X_PJRT_LIBRARY_PATH={override!r} names no file")
+    return override
+
+
+def _register(xla_bridge, library_path: str) -> None:
+    try:
+        xla_bridge.register_plugin(PLATFORM_NAME, priority=500, library_path=library_path, options=None)
+    except Exception as e:   # a second initialize() in one process finds the platform registered already
+        text = str(e)
+        if "ALREADY_EXISTS" in text and PLATFORM_NAME in text.lower():
+            return
+        raise Mi355xPluginError(f"jax refused the {PLATFORM_NAME} plugin at {library_path}: {e}") from e
 
 
 def initialize() -> None:
-    """Register the plugin with JAX (raises Mi355xPluginError when that is impossible)."""
+    """Entry point of the `jax_plugins` group: make `JAX_PLATFORMS=mi355x` resolve to this library.
+
+    Needs jax with `xla_bridge.register_plugin`; anything missing raises Mi355xPluginError so that jax's
+    plugin discovery reports it instead of silently running elsewhere."""
     library_path = find_library()
     if library_path is None:
-        raise Mi355xPluginError(f"Could not find {LIB_NAME} next to {_PKG_DIR}; set MI355X_PJRT_LIBRARY_PATH or build the library.")
-    try:
-        from jax._src import xla_bridge as xb
-    except ImportError as e:
-        raise Mi355xPluginError(f"Failed to import JAX xla_bridge: {e}") from e
-    if not hasattr(xb, "register_plugin"):
-        raise Mi355xPluginError("JAX version does not support register_plugin API.")
+        raise Mi355xPluginError(f"{LIB_NAME} is neither next to {_PKG_DIR} nor named by MI355X_PJRT_LIBRARY_PATH; "
+                                "build it with __graft_entry__.build()")
     try:
         import jax
-        # the front end reads StableHLO, not the sdy dialect (reference: __init__.py:120-131)
-        jax.config.update("jax_use_shardy_partitioner", False)
-    except Exception:
-        pass
+        from jax._src import xla_bridge
+    except ImportError as e:
+        raise Mi355xPluginError(f"jax is not importable here ({e}); the plugin can still be driven through jax_mps_amd.pjrt") from e
+    register = getattr(xla_bridge, "register_plugin", None)
+    if register is None:
+        raise Mi355xPluginError(f"jax {getattr(jax, '__version__', '?')} predates xla_bridge.register_plugin; a newer jax is needed")
+    # the front end reads the stablehlo dialect; with shardy on, jax would emit sdy ops instead
+    # (reference: src/jax_plugins/mps/__init__.py:120-131)
     try:
-        xb.register_plugin(PLATFORM_NAME, priority=500, library_path=library_path, options=None)
-    except Exception as e:
-        if not ("ALREADY_EXISTS" in str(e) and PLATFORM_NAME in str(e).lower()):
-            raise Mi355xPluginError(f"Failed to register the {PLATFORM_NAME} plugin with JAX: {e}") from e
+        jax.config.update("jax_use_shardy_partitioner", False)
+    except (AttributeError, KeyError, ValueError):
+        pass
+    _register(xla_bridge, library_path)
 
 
 def build_library(force: bool = True, jobs: int = 8) -> str:

@@ -802,7 +802,11 @@ class Emitter {
     static const std::unordered_map<std::string, const char*> unary = {
         {"exponential", "exp"}, {"exponential_minus_one", "expm1"}, {"log", "log"}, {"log_plus_one", "log1p"},
         {"sqrt", "sqrt"}, {"cbrt", "cbrt"}, {"tanh", "tanh"}, {"tan", "tan"}, {"sine", "sin"}, {"cosine", "cos"},
-        {"floor", "floor"}, {"ceil", "ceil"}, {"round_nearest_even", "rint"}, {"round_nearest_afz", "round"}};
+        {"floor", "floor"}, {"ceil", "ceil"}, {"round_nearest_even", "rint"}, {"round_nearest_afz", "round"},
+        // chlo unary ops, also reached as custom_call @mhlo.<name> (reference: ops/control_flow.cc:53-63)
+        {"chlo.asin", "asin"}, {"chlo.acos", "acos"}, {"chlo.atan", "atan"}, {"chlo.sinh", "sinh"}, {"chlo.cosh", "cosh"},
+        {"chlo.asinh", "asinh"}, {"chlo.acosh", "acosh"}, {"chlo.atanh", "atanh"}, {"chlo.erf", "erf"},
+        {"chlo.erf_inv", "erfinv"}};
     auto it = unary.find(n);
     if (it != unary.end()) return bin(std::string(it->second) + sfx + "(" + in(0) + ")");
     throw CompileError("codegen: no lowering for stablehlo." + n);
@@ -912,7 +916,8 @@ bool isFusibleOp(const Op& op) {
       "is_finite", "shift_left", "shift_right_logical", "shift_right_arithmetic", "popcnt", "count_leading_zeros",
       "compare", "select", "clamp", "convert", "bitcast_convert", "reduce_precision", "constant", "iota", "reshape",
       "broadcast_in_dim", "transpose", "reverse", "concatenate", "slice", "dynamic_slice", "pad", "gather",
-      "optimization_barrier", "custom_call"};
+      "optimization_barrier", "custom_call", "chlo.asin", "chlo.acos", "chlo.atan", "chlo.sinh", "chlo.cosh", "chlo.asinh",
+      "chlo.acosh", "chlo.atanh", "chlo.erf", "chlo.erf_inv"};
   for (auto* n : names) if (op.name == n) return true;
   return false;
 }

@@ -79,7 +79,7 @@ class Parser {
 
   std::unique_ptr<Module> parseModule() {
     auto m = std::make_unique<Module>();
-    ws();
+    skipAliasLines();
     bool wrapped = false;
     if (eatWord("module")) {
       wrapped = true;
@@ -93,12 +93,17 @@ class Parser {
       if (eatWord("attributes")) skipBalanced('{', '}');
       expect("{");
     }
+    skipAliasLines();
     while (true) {
       ws();
       if (i_ >= n_) break;
       if (wrapped && eat("}")) break;
+      skipAliasLines();
+      if (i_ >= n_) break;
       m->funcs.push_back(parseFunc());
     }
+    if (wrapped) skipLoc();
+    skipAliasLines();
     if (!m->main()) {
       // a module with a single function is accepted under any name
       if (m->funcs.size() == 1) m->funcs[0]->name = "main";
@@ -122,10 +127,13 @@ class Parser {
     for (auto& c : ctx) if (c == '\n') c = ' ';
     throw CompileError("StableHLO parse error at line " + std::to_string(line) + ": " + msg + " near '" + ctx + "'");
   }
-  int currentLine() const {
-    int line = 1;
-    for (size_t k = 0; k < i_ && k < n_; ++k) if (s_[k] == '\n') ++line;
-    return line;
+  // line of the read position; positions only move forward between calls, so the count resumes where it stopped
+  size_t lineScanned_ = 0;
+  int lineAtScan_ = 1;
+  int currentLine() {
+    if (i_ < lineScanned_) { lineScanned_ = 0; lineAtScan_ = 1; }
+    for (; lineScanned_ < i_ && lineScanned_ < n_; ++lineScanned_) if (s_[lineScanned_] == '\n') ++lineAtScan_;
+    return lineAtScan_;
   }
   void ws() {
     while (i_ < n_) {
@@ -167,6 +175,12 @@ class Parser {
     }
     if (b == i_) fail("identifier expected");
     return std::string(s_ + b, i_ - b);
+  }
+  // the name after `@`: bare identifier or quoted string
+  std::string symbolName() {
+    ws();
+    if (i_ < n_ && s_[i_] == '"') return stringLit();
+    return ident();
   }
   std::string ssaName() {
     ws();
@@ -219,6 +233,34 @@ class Parser {
       out.push_back(integer());
       if (eat(c)) return out;
       expect(",");
+    }
+  }
+  // `loc(...)` after an op, a block argument or a function signature: debug information only
+  void skipLoc() {
+    size_t save = i_;
+    ws();
+    if (i_ + 4 <= n_ && memcmp(s_ + i_, "loc(", 4) == 0) {
+      i_ += 3;
+      skipBalanced('(', ')');
+      return;
+    }
+    i_ = save;
+  }
+  // `#loc3 = loc("f.py":12:4)` and other `#alias = ...` definitions outside functions: read to the end of the
+  // definition (brackets and strings balanced) and dropped, since only locations are ever referred to by alias here
+  void skipAliasLines() {
+    while (true) {
+      ws();
+      if (i_ >= n_ || s_[i_] != '#') return;
+      int depth = 0;
+      while (i_ < n_) {
+        char c = s_[i_];
+        if (c == '"') { stringLit(); continue; }
+        if (c == '(' || c == '[' || c == '{' || c == '<') ++depth;
+        else if (c == ')' || c == ']' || c == '}' || c == '>') --depth;
+        else if (c == '\n' && depth <= 0) break;
+        ++i_;
+      }
     }
   }
   void skipBalanced(char open, char close) {
@@ -427,7 +469,7 @@ class Parser {
       return a;
     }
     if (c == '#') return parseHashAttr();
-    if (c == '@') { ++i_; a.kind = Attr::Str; a.s = ident(); return a; }
+    if (c == '@') { ++i_; a.kind = Attr::Str; a.s = symbolName(); return a; }
     if (peek("dense<")) return parseDense();
     if (peek("array<")) {
       i_ += 6;
@@ -599,7 +641,7 @@ class Parser {
     else if (eatWord("private")) f->isPublic = false;
     else f->isPublic = true;
     expect("@");
-    f->name = ident();
+    f->name = symbolName();
     scopes_.emplace_back();
     expect("(");
     if (!eat(")")) {
@@ -612,6 +654,7 @@ class Parser {
         define(nm, {v.get()});
         f->body.args.push_back(std::move(v));
         if (peekc() == '{') skipBalanced('{', '}');
+        skipLoc();
         if (eat(")")) break;
         expect(",");
       }
@@ -624,6 +667,7 @@ class Parser {
     expect("{");
     parseBlockOps(f->body);
     expect("}");
+    skipLoc();
     scopes_.pop_back();
     return f;
   }
@@ -674,6 +718,7 @@ class Parser {
             v->defIndex = (int)r->args.size();
             define(nm, {v.get()});
             r->args.push_back(std::move(v));
+            skipLoc();
             if (eat(")")) break;
             expect(",");
           }
@@ -709,6 +754,12 @@ class Parser {
       else outs.push_back(parseType());
     } else {
       outs.push_back(parseType());
+      // chlo's pretty form: `chlo.erf %x : tensor<4xf32> -> tensor<4xf32>`
+      if (eat("->")) {
+        outs.clear();
+        if (peekc() == '(') outs = typeListParen();
+        else outs.push_back(parseType());
+      }
     }
   }
 
@@ -718,13 +769,22 @@ class Parser {
     ws();
     std::string base;
     int declared = 0;
+    // `%a = op`, `%a:2 = op` or `%a, %b = op` (each name stands for `count` consecutive results)
+    std::vector<std::pair<std::string, int>> resultNames;
     if (peekc() == '%') {
-      size_t b = i_++;
-      while (i_ < n_ && (isIdentChar(s_[i_]) || s_[i_] == '-')) ++i_;
-      base = std::string(s_ + b, i_ - b);
-      declared = 1;
-      if (eat(":")) declared = (int)integer();
-      if (peekc() == ',') fail("comma-separated result lists are not supported; use %name:N");
+      while (true) {
+        ws();
+        if (i_ >= n_ || s_[i_] != '%') fail("result name expected");
+        size_t b = i_++;
+        while (i_ < n_ && (isIdentChar(s_[i_]) || s_[i_] == '-')) ++i_;
+        std::string nm(s_ + b, i_ - b);
+        int cnt = 1;
+        if (eat(":")) cnt = (int)integer();
+        resultNames.emplace_back(nm, cnt);
+        declared += cnt;
+        if (!eat(",")) break;
+      }
+      base = resultNames[0].first;
       expect("=");
     }
     ws();
@@ -746,7 +806,7 @@ class Parser {
       } else if (op->name == "call") {
         expect("@");
         op->attrs["callee"].kind = Attr::Str;
-        op->attrs["callee"].s = ident();
+        op->attrs["callee"].s = symbolName();
         expect("(");
         if (peekc() != ')') op->operands = ssaUseList();
         expect(")");
@@ -760,7 +820,16 @@ class Parser {
         parsePrettyOp(op.get(), outs);
       }
     }
-    setResults(op.get(), outs, base, base.empty() ? -1 : declared);
+    setResults(op.get(), outs, resultNames.size() > 1 ? std::string() : base, base.empty() ? -1 : declared);
+    if (resultNames.size() > 1) {
+      size_t at = 0;
+      for (auto& rn : resultNames) {
+        std::vector<Value*> vals;
+        for (int k = 0; k < rn.second && at < op->results.size(); ++k) vals.push_back(op->results[at++].get());
+        define(rn.first, vals);
+      }
+    }
+    skipLoc();
     return op;
   }
 
@@ -1017,7 +1086,37 @@ class Parser {
       outs = typesBare();
       return;
     }
-    if (n == "composite") fail("stablehlo.composite is not supported");
+    if (n == "composite") {
+      // %0 = stablehlo.composite "chlo.asin" %x {decomposition = @chlo.asin.impl} : (tensor<4xf32>) -> tensor<4xf32>
+      setStr(op, "name", stringLit());
+      if (peekc() == '%') op->operands = ssaUseList();
+      if (peekc() == '{') {
+        auto d = parseAttrDict();
+        for (auto& kv : d) op->attrs[kv.first] = kv.second;
+      }
+      expect(":");
+      fnType(op, outs);
+      if (!op->has("decomposition")) fail("stablehlo.composite without a decomposition function");
+      return;
+    }
+    if (n == "reduce_precision") {
+      // %0 = stablehlo.reduce_precision %x, format = e5m10 : tensor<16xf32>
+      op->operands = ssaUseList();
+      expect(",");
+      expect("format");
+      expect("=");
+      ws();
+      if (i_ >= n_ || s_[i_] != 'e') fail("expected a format of the form e<exponent bits>m<mantissa bits>");
+      ++i_;
+      setInt(op, "exponent_bits", integer());
+      if (i_ >= n_ || s_[i_] != 'm') fail("expected a format of the form e<exponent bits>m<mantissa bits>");
+      ++i_;
+      setInt(op, "mantissa_bits", integer());
+      if (peekc() == '{') skipBalanced('{', '}');
+      expect(":");
+      fnType(op, outs);
+      return;
+    }
     // common pretty form: operands, keyword attributes, optional attr dict, type
     if (peekc() == '%') op->operands = ssaUseList();
     if (n == "slice") {

@@ -94,9 +94,11 @@ bool inlineRegion(Module& m, Region& r, VMap& repl, int& nextId, int depth) {
   for (size_t k = 0; k < r.ops.size(); ++k) {
     Op* op = r.ops[k].get();
     for (auto& sub : op->regions) any |= inlineRegion(m, *sub, repl, nextId, depth);
-    if (op->name != "call") continue;
-    Func* callee = m.find(op->str("callee"));
-    if (!callee) throw CompileError("call to unknown function @" + op->str("callee"));
+    // a composite runs its decomposition function (reference: ops/control_flow.cc:2242-2262)
+    if (op->name != "call" && op->name != "composite") continue;
+    const std::string& target = op->name == "call" ? op->str("callee") : op->str("decomposition");
+    Func* callee = m.find(target);
+    if (!callee) throw CompileError(op->name + " of unknown function @" + target);
     if (callee->body.args.size() != op->operands.size()) throw CompileError("call @" + callee->name + ": argument count mismatch");
     VMap map;
     for (size_t a = 0; a < op->operands.size(); ++a) map[callee->body.args[a].get()] = op->operands[a];
@@ -159,6 +161,18 @@ bool sweep(Region& r, std::unordered_map<const Value*, int>& uses) {
   return changed;
 }
 
+// custom_call @mhlo.asin(%x) and its siblings are the chlo unary ops under another spelling
+// (reference: ops/control_flow.cc:53-63, 1417-1440)
+void renameUnaryCustomCalls(Region& r) {
+  static const std::set<std::string> unary = {"asin", "acos", "atan", "sinh", "cosh", "asinh", "acosh", "atanh", "erf", "erf_inv"};
+  for (auto& o : r.ops) {
+    for (auto& sub : o->regions) renameUnaryCustomCalls(*sub);
+    if (o->name != "custom_call" || o->operands.size() != 1 || o->results.size() != 1) continue;
+    const std::string& t = o->str("target");
+    if (t.rfind("mhlo.", 0) == 0 && unary.count(t.substr(5))) o->name = "chlo." + t.substr(5);
+  }
+}
+
 }  // namespace
 
 void inlineCalls(Module& m) {
@@ -173,6 +187,7 @@ void inlineCalls(Module& m) {
     removeDead(main->body);
     repl.clear();
   }
+  renameUnaryCustomCalls(main->body);
 }
 
 // ---- integer / boolean dot_general ---------------------------------------------------------
@@ -1074,13 +1089,36 @@ static const std::set<std::string>& supportedOps() {
       "reduce", "dot_general", "dot", "convolution", "gather", "scatter", "reduce_window", "select_and_scatter", "sort",
       // control flow (ops/control_flow.cc:2364-2376)
       "while", "case", "return", "optimization_barrier", "custom_call",
+      // chlo unary ops (reference: ops/control_flow.cc:53-63)
+      "chlo.asin", "chlo.acos", "chlo.atan", "chlo.sinh", "chlo.cosh", "chlo.asinh", "chlo.acosh", "chlo.atanh", "chlo.erf",
+      "chlo.erf_inv",
   };
   return s;
+}
+
+// Attributes without which an op has no meaning.  The accessors of Op return 0 / an empty list for a missing key,
+// which is right only where StableHLO defines that default, so the others are checked here once.
+static void checkRequiredAttrs(const Op& o) {
+  static const std::map<std::string, std::vector<const char*>> required = {
+      {"iota", {"dim"}}, {"concatenate", {"dim"}}, {"broadcast_in_dim", {"dims"}}, {"transpose", {"dims"}},
+      {"reverse", {"dims"}}, {"reduce", {"dimensions"}}, {"slice", {"start", "limit"}}, {"dynamic_slice", {"sizes"}},
+      {"pad", {"low", "high"}}, {"compare", {"direction"}}, {"reduce_precision", {"exponent_bits", "mantissa_bits"}},
+      {"constant", {"value"}}, {"gather", {"slice_sizes", "index_vector_dim", "start_index_map"}},
+      {"scatter", {"index_vector_dim", "scatter_dims_to_operand_dims"}}, {"chlo.top_k", {"k"}},
+      {"dot_general", {"lhs_contract", "rhs_contract"}}, {"custom_call", {"target"}}};
+  auto it = required.find(o.name);
+  if (it == required.end()) return;
+  for (const char* k : it->second)
+    if (!o.has(k))
+      throw CompileError("stablehlo." + o.name + " at line " + std::to_string(o.line) + " lacks its '" + k + "' attribute");
+  if (o.name == "reduce_precision" && (o.integer("exponent_bits") < 1 || o.integer("mantissa_bits") < 0))
+    throw CompileError("stablehlo.reduce_precision at line " + std::to_string(o.line) + ": exponent_bits must be at least 1 and mantissa_bits non-negative");
 }
 
 static void scan(const Region& r, std::set<std::string>& bad) {
   for (auto& o : r.ops) {
     if (!supportedOps().count(o->name)) bad.insert(o->name);
+    checkRequiredAttrs(*o);
     if (o->name == "custom_call") {
       const std::string& t = o->str("target");
       if (t != "Sharding" && t != "SPMDFullToShardShape" && t != "SPMDShardToFullShape") bad.insert("custom_call @" + t);

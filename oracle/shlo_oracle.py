@@ -122,6 +122,59 @@ class _P:
             else:
                 break
 
+    def skip_loc(self):
+        """`loc(...)` after an op, an argument or a signature is debug information."""
+        save = self.i
+        self.ws()
+        if self.s.startswith("loc(", self.i):
+            self.i += 3
+            self.raw_until_balanced_paren()
+        else:
+            self.i = save
+
+    def raw_until_balanced_paren(self):
+        depth = 0
+        while self.i < self.n:
+            c = self.s[self.i]
+            if c == '"':
+                self.string()
+                continue
+            if c == "(":
+                depth += 1
+            elif c == ")":
+                depth -= 1
+                if depth == 0:
+                    self.i += 1
+                    return
+            self.i += 1
+        self.err("unbalanced parentheses")
+
+    def skip_alias_lines(self):
+        """`#loc3 = loc(...)` definitions outside functions."""
+        while True:
+            self.ws()
+            if self.i >= self.n or self.s[self.i] != "#":
+                return
+            depth = 0
+            while self.i < self.n:
+                c = self.s[self.i]
+                if c == '"':
+                    self.string()
+                    continue
+                if c in "([{<":
+                    depth += 1
+                elif c in ")]}>":
+                    depth -= 1
+                elif c == "\n" and depth <= 0:
+                    break
+                self.i += 1
+
+    def symbol(self) -> str:
+        self.ws()
+        if self.i < self.n and self.s[self.i] == '"':
+            return self.string()
+        return self.ident()
+
     def peek(self, lit: str) -> bool:
         self.ws()
         return self.s.startswith(lit, self.i)
@@ -263,7 +316,7 @@ class _P:
             return self.hash_attr()
         if c == "@":
             self.i += 1
-            return "@" + self.ident()
+            return "@" + self.symbol()
         if s.startswith("dense<", self.i):
             return self.dense()
         if s.startswith("array<", self.i):
@@ -385,7 +438,7 @@ class _P:
     # ---- module structure
     def module(self) -> Dict[str, Func]:
         funcs = {}
-        self.ws()
+        self.skip_alias_lines()
         wrapped = False
         if self.eat("module"):
             wrapped = True
@@ -394,11 +447,16 @@ class _P:
             if self.eat("attributes"):
                 self.attr_dict()
             self.expect("{")
+        self.skip_alias_lines()
         while True:
             self.ws()
             if self.i >= self.n:
                 break
             if wrapped and self.eat("}"):
+                self.skip_loc()
+                break
+            self.skip_alias_lines()
+            if self.i >= self.n:
                 break
             f = self.func()
             funcs[f.name] = f
@@ -410,7 +468,7 @@ class _P:
         if self.peek("public") or self.peek("private"):
             self.ident()
         self.expect("@")
-        f = Func(self.ident())
+        f = Func(self.symbol())
         self.expect("(")
         if not self.eat(")"):
             while True:
@@ -418,6 +476,7 @@ class _P:
                 self.expect(":")
                 f.body.arg_types.append(self.type())
                 self.skip_attr_dict()
+                self.skip_loc()
                 if self.eat(")"):
                     break
                 self.expect(",")
@@ -431,6 +490,7 @@ class _P:
         self.expect("{")
         self.block_ops(f.body)
         self.expect("}")
+        self.skip_loc()
         return f
 
     def block_ops(self, region: Region):
@@ -454,6 +514,7 @@ class _P:
                         r.args.append(self.ssa())
                         self.expect(":")
                         r.arg_types.append(self.type())
+                        self.skip_loc()
                         if self.eat(")"):
                             break
                         self.expect(",")
@@ -466,6 +527,7 @@ class _P:
         op = Op()
         self.ws()
         nres = 1
+        listed = False
         if self.s[self.i] == "%":
             m = re.compile(r"%[A-Za-z0-9_.$]+").match(self.s, self.i)
             base = m.group(0)
@@ -473,9 +535,21 @@ class _P:
             if self.eat(":"):
                 nres = self.integer()
             end_decl = self.i
-            self.expect("=")
             explicit = ":" in self.s[m.end():end_decl]
             op.results = [base] if (nres == 1 and not explicit) else [f"{base}#{k}" for k in range(nres)]
+            # `%a, %b = op`: one name per result (or per run of results with `%a:2`)
+            while self.eat(","):
+                listed = True
+                self.ws()
+                m = re.compile(r"%[A-Za-z0-9_.$]+").match(self.s, self.i)
+                nm = m.group(0)
+                self.i = m.end()
+                if self.eat(":"):
+                    c = self.integer()
+                    op.results += [f"{nm}#{k}" for k in range(c)]
+                else:
+                    op.results.append(nm)
+            self.expect("=")
             has_res = True
         else:
             has_res = False
@@ -496,7 +570,7 @@ class _P:
             elif op.name in ("call", "func.call"):
                 op.name = "call"
                 self.expect("@")
-                op.attrs["callee"] = self.ident()
+                op.attrs["callee"] = self.symbol()
                 self.expect("(")
                 op.operands = [] if self.peek(")") else self.ssa_list()
                 self.expect(")")
@@ -507,8 +581,9 @@ class _P:
                 op.out_types = self.type_list_paren() if self.peek("(") else [self.type()]
             else:
                 self.pretty_op(op)
-        if has_res and nres == 1 and len(op.out_types) > 1:
+        if has_res and not listed and nres == 1 and len(op.out_types) > 1:
             op.results = [f"{op.results[0]}#{k}" for k in range(len(op.out_types))]
+        self.skip_loc()
         return op
 
     def ssa_list(self) -> List[str]:
@@ -540,6 +615,8 @@ class _P:
             t = self.type()
             op.in_types = [t] * len(op.operands)
             op.out_types = [t]
+            if self.eat("->"):      # chlo's pretty form: `type -> type`
+                op.out_types = self.type_list_paren() if self.peek("(") else [self.type()]
 
     def generic_op(self, op: Op):
         self.expect("(")
@@ -635,6 +712,30 @@ class _P:
             ts = self.types_bare()
             op.in_types = ts
             op.out_types = ts
+            return
+        if short == "composite":
+            op.attrs["name"] = self.string()
+            self.ws()
+            op.operands = self.ssa_list() if self.s[self.i] == "%" else []
+            if self.peek("{"):
+                op.attrs.update(self.attr_dict())
+            self.expect(":")
+            self.fn_type(op)
+            return
+        if short == "reduce_precision":
+            op.operands = self.ssa_list()
+            self.expect(",")
+            self.expect("format")
+            self.expect("=")
+            self.ws()
+            m = re.compile(r"e(\d+)m(\d+)").match(self.s, self.i)
+            if not m:
+                self.err("expected a format of the form e<exponent bits>m<mantissa bits>")
+            self.i = m.end()
+            op.attrs["exponent_bits"], op.attrs["mantissa_bits"] = int(m.group(1)), int(m.group(2))
+            self.skip_attr_dict()
+            self.expect(":")
+            self.fn_type(op)
             return
         # generic pretty: operands, then keyword attrs, then type
         self.ws()
@@ -1106,6 +1207,19 @@ class Oracle:
         from scipy import special
         return special.erf(ins[0].astype(np.float64))
     op_chlo_erf = op_erf
+
+    # chlo unary ops, also spelled custom_call @mhlo.<name> (reference: ops/control_flow.cc:53-63)
+    def op_chlo_erf_inv(self, op, ins, env):
+        from scipy import special
+        return special.erfinv(ins[0].astype(np.float64))
+    def op_chlo_asin(self, op, ins, env): return self._f64un(op, ins, np.arcsin)
+    def op_chlo_acos(self, op, ins, env): return self._f64un(op, ins, np.arccos)
+    def op_chlo_atan(self, op, ins, env): return self._f64un(op, ins, np.arctan)
+    def op_chlo_sinh(self, op, ins, env): return self._f64un(op, ins, np.sinh)
+    def op_chlo_cosh(self, op, ins, env): return self._f64un(op, ins, np.cosh)
+    def op_chlo_asinh(self, op, ins, env): return self._f64un(op, ins, np.arcsinh)
+    def op_chlo_acosh(self, op, ins, env): return self._f64un(op, ins, np.arccosh)
+    def op_chlo_atanh(self, op, ins, env): return self._f64un(op, ins, np.arctanh)
 
     def op_clamp(self, op, ins, env):
         lo, x, hi = ins
@@ -1627,6 +1741,11 @@ class Oracle:
         f = self.funcs[op.attrs["callee"]]
         return self._run_region(f.body, ins, {})
 
+    def op_composite(self, op, ins, env):
+        """stablehlo.composite runs its decomposition function (reference: ops/control_flow.cc:2242-2262)."""
+        f = self.funcs[str(op.attrs["decomposition"]).lstrip("@")]
+        return self._run_region(f.body, ins, {})
+
     def op_optimization_barrier(self, op, ins, env): return list(ins)
 
     def op_sort(self, op, ins, env):
@@ -1714,6 +1833,8 @@ class Oracle:
         tgt = op.attrs.get("call_target_name")
         if tgt in ("Sharding", "SPMDFullToShardShape", "SPMDShardToFullShape"):
             return ins[0]
+        if isinstance(tgt, str) and tgt.startswith("mhlo.") and hasattr(self, "op_chlo_" + tgt[5:]) and len(ins) == 1:
+            return getattr(self, "op_chlo_" + tgt[5:])(op, ins, env)
         raise NotImplementedError(f"oracle: custom_call {tgt}")
 
 
