@@ -131,6 +131,8 @@ typedef struct {
 int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* indices, const void* updates,
                        void* workspace, mi355_stream_t s);
 size_t mi355_scatter_workspace_bytes(int64_t num_updates);
+// resolves, for the current device, the library-owned workspace of mi355x_scatter_rows_noalloc (include/mi355x_noalloc.h)
+int mi355_noalloc_setup(void);
 
 int mi355_copy(void* dst, const void* src, size_t bytes, mi355_stream_t s);   // kernel copy (graph-capturable)
 // up to 16 copies between pairwise disjoint buffers in one launch

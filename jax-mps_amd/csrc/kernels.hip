@@ -963,3 +963,90 @@ int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* in
 }
 
 }  // extern "C"
+
+// ---- ordered row scatter for callers that cannot allocate (include/mi355x_noalloc.h) --------------------
+// The sort workspace is a device array of the library instead of a caller / arena buffer.  Host code may not
+// pass the array's name to a kernel (on the host it is a stand-in, not a device address): the address is taken
+// once per device with hipGetSymbolAddress and only that pointer is used afterwards.
+#include <mutex>
+
+#include "../../include/mi355x_noalloc.h"
+
+static_assert(sizeof(mi355x_scatter_desc) == sizeof(mi355_scatter_desc), "public and internal scatter descriptors must agree");
+static_assert(offsetof(mi355x_scatter_desc, index_bytes) == offsetof(mi355_scatter_desc, index_bytes), "descriptor layout");
+
+namespace {
+constexpr size_t kNoAllocScratchBytes = (size_t)4 * MI355X_NOALLOC_MAX_UPDATES * 4 + 256 * kSortBlocks * 4 + 1024;
+constexpr int kMaxDevices = 64;
+std::mutex g_scratchMutex;
+void* g_scratchPtr[kMaxDevices] = {};
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+// Device address of `scratch` on the current device (each GPU holds its own copy at its own address).
+static int noallocScratch(void** out, char* error, size_t error_len) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess && (dev < 0 || dev >= kMaxDevices)) e = hipErrorInvalidDevice;
+  if (e == hipSuccess) {
+    std::lock_guard<std::mutex> lock(g_scratchMutex);
+    if (!g_scratchPtr[dev]) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e == hipSuccess && !p) e = hipErrorInvalidSymbol;
+      if (e == hipSuccess) g_scratchPtr[dev] = p;
+    }
+    if (e == hipSuccess) *out = g_scratchPtr[dev];
+  }
+  if (e != hipSuccess) {
+    if (error && error_len) snprintf(error, error_len, "mi355x_scatter_rows_noalloc: cannot resolve the workspace on device %d: %s", dev, hipGetErrorString(e));
+    return (int)e;
+  }
+  return 0;
+}
+
+extern "C" {
+
+// called when a PJRT client takes a device, so that the first scatter call finds the address resolved
+int mi355_noalloc_setup(void) {
+  void* p = nullptr;
+  return noallocScratch(&p, nullptr, 0);
+}
+
+__attribute__((visibility("default")))
+int mi355x_scatter_rows_noalloc(const mi355x_scatter_desc* desc, void* result, const void* indices, const void* updates,
+                                void* hip_stream, char* error, size_t error_len) {
+  auto fail = [&](int code, const char* msg) {
+    if (error && error_len) snprintf(error, error_len, "mi355x_scatter_rows_noalloc: %s", msg);
+    return code;
+  };
+  if (!desc) return fail(1, "desc is NULL");
+  if (desc->num_updates < 0 || desc->row_elems < 0 || desc->operand_rows < 0) return fail(1, "negative size in desc");
+  if (desc->num_updates > MI355X_NOALLOC_MAX_UPDATES) {
+    if (error && error_len)
+      snprintf(error, error_len, "mi355x_scatter_rows_noalloc: num_updates %lld exceeds the fixed workspace (MI355X_NOALLOC_MAX_UPDATES = %d)",
+               (long long)desc->num_updates, MI355X_NOALLOC_MAX_UPDATES);
+    return 2;
+  }
+  if (desc->kind < 0 || desc->kind > 4) return fail(1, "kind must be 0 (add), 1 (set), 2 (multiply), 3 (minimum) or 4 (maximum)");
+  if (desc->dtype < 0 || desc->dtype > 3) return fail(1, "dtype must be 0 (f32), 1 (bf16), 2 (s32) or 3 (u32)");
+  if (desc->index_bytes != 4 && desc->index_bytes != 8) return fail(1, "index_bytes must be 4 or 8");
+  if (desc->operand_rows > 0xFFFFFFFEll) return fail(1, "operand_rows must fit 32 bits");
+  if (desc->num_updates == 0 || desc->row_elems == 0 || desc->operand_rows == 0) return 0;
+  if (!result || !indices || !updates) return fail(1, "result, indices and updates must be device pointers");
+  void* ws = nullptr;
+  if (int rc = noallocScratch(&ws, error, error_len)) return rc;
+  mi355_scatter_desc d;
+  d.numUpdates = desc->num_updates;
+  d.rowElems = desc->row_elems;
+  d.operandRows = desc->operand_rows;
+  d.kind = desc->kind;
+  d.dtype = desc->dtype;
+  d.index_bytes = desc->index_bytes;
+  int rc = mi355_scatter_rows(&d, result, indices, updates, ws, (mi355_stream_t)hip_stream);
+  if (rc != 0 && error && error_len) snprintf(error, error_len, "mi355x_scatter_rows_noalloc: kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+  return rc;
+}
+
+}  // extern "C"

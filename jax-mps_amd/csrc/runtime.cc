@@ -154,6 +154,8 @@ Device::Device() {
   if (!available(&why)) throw RuntimeError("MI355X plugin: " + why + " (this plugin has no CPU fallback)");
   char name[256], arch[256];
   check(mi355_device_init(0, name, sizeof name, arch, sizeof arch, &cus_, &totalMem_), "device init");
+  // resolve the fixed workspace of mi355x_scatter_rows_noalloc now; a failure is reported by that entry point's first call
+  (void)mi355_noalloc_setup();
   name_ = name;
   arch_ = arch;
   if (baseArch(arch_) != "gfx950")

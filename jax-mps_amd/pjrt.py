@@ -32,6 +32,14 @@ Error_GetCode_Args = _args("Error_GetCode_Args", [("error", _P), ("code", C.c_in
 Plugin_Initialize_Args = _args("Plugin_Initialize_Args", [])
 Event_Args = _args("Event_Args", [("event", _P)])
 Event_IsReady_Args = _args("Event_IsReady_Args", [("event", _P), ("is_ready", C.c_bool)])
+Event_Error_Args = _args("Event_Error_Args", [("event", _P)])
+OnReadyCallback = C.CFUNCTYPE(None, _P, _P)      # void (*)(PJRT_Error* error, void* user_arg); the callback owns the error
+Event_OnReady_Args = _args("Event_OnReady_Args", [("event", _P), ("callback", OnReadyCallback), ("user_arg", _P)])
+Buffer_CopyToDevice_Args = _args("Buffer_CopyToDevice_Args", [("buffer", _P), ("dst_device", _P), ("dst_buffer", _P)])
+LoadedExecutable_GetDeviceAssignment_Args = _args("LoadedExecutable_GetDeviceAssignment_Args", [
+    ("executable", _P), ("serialized_bytes", _P), ("serialized_bytes_size", _SZ), ("serialized_device_assignment", _P),
+    ("serialized_device_assignment_deleter", C.CFUNCTYPE(None, _P))])
+Plugin_Attributes_Args = _args("Plugin_Attributes_Args", [("attributes", _P), ("num_attributes", _SZ)])
 Client_Create_Args = _args("Client_Create_Args", [
     ("create_options", _P), ("num_options", _SZ), ("kv_get_callback", _P), ("kv_get_user_arg", _P),
     ("kv_put_callback", _P), ("kv_put_user_arg", _P), ("client", _P), ("kv_try_get_callback", _P),
@@ -106,6 +114,7 @@ Buffer_ElementType_Args = _args("Buffer_ElementType_Args", [("buffer", _P), ("ty
 Buffer_Dimensions_Args = _args("Buffer_Dimensions_Args", [("buffer", _P), ("dims", C.POINTER(C.c_int64)), ("num_dims", _SZ)])
 Buffer_ToHostBuffer_Args = _args("Buffer_ToHostBuffer_Args", [("src", _P), ("host_layout", _P), ("dst", _P), ("dst_size", _SZ), ("event", _P)])
 Buffer_ReadyEvent_Args = _args("Buffer_ReadyEvent_Args", [("buffer", _P), ("event", _P)])
+Buffer_OpaqueDeviceMemoryDataPointer_Args = _args("Buffer_OpaqueDeviceMemoryDataPointer_Args", [("buffer", _P), ("device_memory_ptr", _P)])
 Buffer_IsDeleted_Args = _args("Buffer_IsDeleted_Args", [("buffer", _P), ("is_deleted", C.c_bool)])
 
 
@@ -246,6 +255,30 @@ class Plugin:
         raise PjrtError(msg, g.code)
 
 
+class ScatterDesc(C.Structure):
+    """mi355x_scatter_desc of include/mi355x_noalloc.h."""
+    _fields_ = [("num_updates", C.c_int64), ("row_elems", C.c_int64), ("operand_rows", C.c_int64), ("kind", C.c_int),
+                ("dtype", C.c_int), ("index_bytes", C.c_int)]
+
+
+SCATTER_KINDS = {"add": 0, "set": 1, "mul": 2, "min": 3, "max": 4}
+SCATTER_DTYPES = {"f32": 0, "bf16": 1, "i32": 2, "ui32": 3}
+
+
+def scatter_rows_noalloc(plugin: Plugin, result_ptr: int, indices_ptr: int, updates_ptr: int, *, num_updates: int, row_elems: int,
+                         operand_rows: int, kind: str = "add", dtype: str = "f32", index_bytes: int = 4, stream: int = 0) -> None:
+    """mi355x_scatter_rows_noalloc (include/mi355x_noalloc.h): ordered row scatter into `result_ptr` in place, enqueued
+    on `stream`, using the library's fixed workspace.  Raises PjrtError with the entry point's message on failure."""
+    fn = plugin.lib.mi355x_scatter_rows_noalloc
+    fn.restype = C.c_int
+    fn.argtypes = [C.POINTER(ScatterDesc), _P, _P, _P, _P, C.c_char_p, _SZ]
+    d = ScatterDesc(num_updates, row_elems, operand_rows, SCATTER_KINDS[kind], SCATTER_DTYPES[dtype], index_bytes)
+    err = C.create_string_buffer(256)
+    rc = fn(C.byref(d), result_ptr or None, indices_ptr or None, updates_ptr or None, stream or None, err, len(err))
+    if rc != 0:
+        raise PjrtError(err.value.decode("utf-8", "replace"), rc)
+
+
 class Buffer:
     def __init__(self, client: "Client", handle):
         self.client = client
@@ -261,6 +294,11 @@ class Buffer:
     def shape(self):
         a = self._p.call("PJRT_Buffer_Dimensions", Buffer_Dimensions_Args(buffer=self.handle))
         return tuple(a.dims[i] for i in range(a.num_dims))
+
+    def device_pointer(self) -> int:
+        """Device address of the buffer's memory (PJRT_Buffer_OpaqueDeviceMemoryDataPointer)."""
+        a = self._p.call("PJRT_Buffer_OpaqueDeviceMemoryDataPointer", Buffer_OpaqueDeviceMemoryDataPointer_Args(buffer=self.handle))
+        return int(a.device_memory_ptr or 0)
 
     def block_until_ready(self):
         a = self._p.call("PJRT_Buffer_ReadyEvent", Buffer_ReadyEvent_Args(buffer=self.handle))
@@ -278,6 +316,17 @@ class Buffer:
             self._p.call("PJRT_Event_Await", Event_Args(event=a.event))
             self._p.call("PJRT_Event_Destroy", Event_Args(event=a.event))
         return out
+
+    def copy_to_device(self) -> "Buffer":
+        a = self._p.call("PJRT_Buffer_CopyToDevice", Buffer_CopyToDevice_Args(buffer=self.handle, dst_device=self.client.devices[0]))
+        return Buffer(self.client, a.dst_buffer)
+
+    def mark_deleted(self):
+        """PJRT_Buffer_Delete: the device memory goes back to the allocator, the handle stays until destroyed."""
+        self._p.call("PJRT_Buffer_Delete", Buffer_Args(buffer=self.handle))
+
+    def is_deleted(self) -> bool:
+        return bool(self._p.call("PJRT_Buffer_IsDeleted", Buffer_IsDeleted_Args(buffer=self.handle)).is_deleted)
 
     def delete(self):
         if self.handle:
@@ -310,7 +359,9 @@ class LoadedExecutable:
             k += n
         return out
 
-    def execute(self, buffers: Sequence[Buffer]) -> List[Buffer]:
+    def execute(self, buffers: Sequence[Buffer], return_event: bool = False):
+        """Outputs of one PJRT_LoadedExecutable_Execute; with `return_event` also the device-complete PJRT_Event
+        handle, which the caller then destroys."""
         p = self.client.plugin
         n = len(buffers)
         arg_arr = (_P * max(n, 1))(*[b.handle for b in buffers])
@@ -323,9 +374,19 @@ class LoadedExecutable:
         a = Execute_Args(executable=self.handle, options=C.pointer(opts), argument_lists=arg_lists, num_devices=1, num_args=n,
                          output_lists=out_lists, device_complete_events=events, execute_device=None)
         p.call("PJRT_LoadedExecutable_Execute", a)
+        outs = [Buffer(self.client, out_arr[i]) for i in range(self.num_outputs)]
+        if return_event:
+            return outs, events[0]
         if events[0]:
             p.call("PJRT_Event_Destroy", Event_Args(event=events[0]))
-        return [Buffer(self.client, out_arr[i]) for i in range(self.num_outputs)]
+        return outs
+
+    def device_assignment_bytes(self) -> bytes:
+        a = self.client.plugin.call("PJRT_LoadedExecutable_GetDeviceAssignment", LoadedExecutable_GetDeviceAssignment_Args(executable=self.handle))
+        data = C.string_at(a.serialized_bytes, a.serialized_bytes_size)
+        if a.serialized_device_assignment_deleter:
+            a.serialized_device_assignment_deleter(a.serialized_device_assignment)
+        return data
 
     def serialize(self) -> bytes:
         """PJRT_Executable_Serialize: bytes that `Client.deserialize_and_load` turns back into a loaded executable."""
@@ -382,6 +443,25 @@ class Client:
         a = self.plugin.call("PJRT_Device_MemoryStats", Device_MemoryStats_Args(device=self.devices[0]))
         return {"bytes_in_use": a.bytes_in_use, "peak_bytes_in_use": a.peak_bytes_in_use, "num_allocs": a.num_allocs,
                 "largest_alloc_size": a.largest_alloc_size, "bytes_limit": a.bytes_limit, "bytes_reserved": a.bytes_reserved}
+
+    def plugin_attributes(self) -> dict:
+        a = self.plugin.call("PJRT_Plugin_Attributes", Plugin_Attributes_Args())
+        out = {}
+        arr = C.cast(a.attributes, C.POINTER(NamedValue))
+        for i in range(a.num_attributes):
+            nv = arr[i]
+            name = C.string_at(nv.name, nv.name_size).decode()
+            if nv.type == 0:
+                out[name] = C.string_at(nv.string_value, nv.value_size).decode()
+            elif nv.type == 1:
+                out[name] = int(nv.int64_value)
+            elif nv.type == 2:
+                out[name] = [C.cast(nv.int64_array_value, C.POINTER(C.c_int64))[k] for k in range(nv.value_size)]
+            elif nv.type == 3:
+                out[name] = float(nv.float_value)
+            else:
+                out[name] = bool(nv.bool_value)
+        return out
 
     def compile_and_load(self, text, devices=None) -> LoadedExecutable:
         code = text.encode() if isinstance(text, str) else bytes(text)

@@ -19,13 +19,25 @@ def plugin():
     return pjrt.Plugin()
 
 
-def test_exports_only_the_declared_symbol():
+def test_exports_only_the_declared_symbols():
+    """Every function include/*.h declares is exported, and nothing else of ours is."""
     declared = re.findall(r"^const PJRT_Api\* (\w+)\(void\);", HEADER, flags=re.M)
     assert declared == ["GetPjrtApi"]
+    noalloc = (ROOT / "include" / "mi355x_noalloc.h").read_text()
+    declared += re.findall(r"^int (mi355x_\w+)\(", noalloc, flags=re.M)
+    assert declared == ["GetPjrtApi", "mi355x_scatter_rows_noalloc"]
     out = subprocess.run(["nm", "-D", "--defined-only", pjrt.default_library_path()], capture_output=True, text=True, check=True).stdout
     syms = {line.split()[-1] for line in out.splitlines() if " T " in line or " W " in line}
     ours = {s for s in syms if "PJRT" in s.upper() or "mi355" in s.lower() or s == "GetPjrtApi"}
-    assert ours == {"GetPjrtApi"}, ours
+    assert ours == set(declared), ours
+
+
+def test_noalloc_descriptor_mirrors_the_header():
+    noalloc = (ROOT / "include" / "mi355x_noalloc.h").read_text()
+    body = noalloc[noalloc.index("typedef struct {"):noalloc.index("} mi355x_scatter_desc;")]
+    fields = re.findall(r"^\s*(?:int64_t|int) (\w+);", body, flags=re.M)
+    assert fields == [f[0] for f in pjrt.ScatterDesc._fields_]
+    assert C.sizeof(pjrt.ScatterDesc) == 40
 
 
 def test_table_header_and_version(plugin):
