@@ -729,10 +729,22 @@ PJRT_Error* Buffer_OnDeviceSizeInBytes(PJRT_Buffer_OnDeviceSizeInBytes_Args* a) 
 }
 PJRT_Error* Buffer_Device(PJRT_Buffer_Device_Args* a) { a->device = &a->buffer->client->device; return nullptr; }
 PJRT_Error* Buffer_Memory(PJRT_Buffer_Memory_Args* a) { a->memory = &a->buffer->client->memory; return nullptr; }
+// Marks the buffer deleted and gives its memory back to the allocator now (work already enqueued that reads it is
+// ordered before any reuse, because everything runs on one stream); the handle lives on until Buffer_Destroy.
+// The reference only sets the flag (mlx_buffer.cc:290-296) and lets MLX's reference counting free the array.
 PJRT_Error* Buffer_Delete(PJRT_Buffer_Delete_Args* a) {
-  std::lock_guard<std::recursive_mutex> lk(apiMutex());
-  a->buffer->buf->deleted = true;
-  return nullptr;
+  return guard([&]() -> PJRT_Error* {
+    std::lock_guard<std::recursive_mutex> lk(apiMutex());
+    DeviceBuffer* b = a->buffer->buf.get();
+    if (!b->deleted) {
+      b->deleted = true;
+      if (b->ptr && a->buffer->buf.use_count() == 1) {
+        Device::get().release(b->ptr);
+        b->ptr = nullptr;
+      }
+    }
+    return nullptr;
+  });
 }
 PJRT_Error* Buffer_IsDeleted(PJRT_Buffer_IsDeleted_Args* a) { a->is_deleted = a->buffer->buf->deleted; return nullptr; }
 

@@ -969,9 +969,13 @@ def _cast_result(a: np.ndarray, t: TType, keep_shape: bool = False) -> np.ndarra
 
 
 class Oracle:
-    def __init__(self, text: str, accum: str = "f64"):
+    def __init__(self, text: str, accum: str = "f64", round_intermediates: bool = True):
+        """`round_intermediates=False` keeps bf16-typed intermediate results unrounded (float32 carriers of the
+        float64 arithmetic): the value the program's formulas define, against which the rounding noise of any
+        bf16 evaluation order can be measured.  Arguments and dense constants keep their bf16 values."""
         self.funcs = parse(text)
         self.accum = np.float64 if accum == "f64" else np.float32
+        self.round_intermediates = round_intermediates
         self.main = self.funcs["main"]
 
     # -- public
@@ -1002,7 +1006,11 @@ class Oracle:
             if not isinstance(outs, (list, tuple)):
                 outs = [outs]
             for name, val, t in zip(op.results, outs, op.out_types):
-                env[name] = _cast_result(val, t, keep_shape=vectorized)
+                if not self.round_intermediates and t.dtype == "bf16":
+                    val = np.asarray(val, dtype=np.float32)
+                    env[name] = val if (vectorized or val.shape == t.shape) else val.reshape(t.shape)
+                else:
+                    env[name] = _cast_result(val, t, keep_shape=vectorized)
                 if name.endswith("#0") and len(op.results) == 1:
                     env[name[:-2]] = env[name]
         return []

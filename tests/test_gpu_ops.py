@@ -1,13 +1,14 @@
 """Per-op parity on the GPU: every case of op_cases.py runs through PJRT_Client_Compile /
 PJRT_LoadedExecutable_Execute / PJRT_Buffer_ToHostBuffer and is compared with the CPU oracle.
 
-Bar: bit-exact for integer, boolean, index and data-movement results; max relative error
-1e-5 for f32 and 2e-2 for bf16 arithmetic."""
+Bar: bit-exact for integer, boolean, index and data-movement results; for float arithmetic the reference's
+elementwise rule |got - want| <= tol + tol |want| (tests/test_ops.py:91-105) with tol = 1e-5 for f32 and
+2e-2 for bf16."""
 import numpy as np
 import pytest
 
 import op_cases
-from conftest import rel_err
+from conftest import closeness
 from shlo_oracle import Oracle, round_bf16
 
 pytestmark = pytest.mark.gpu
@@ -16,6 +17,14 @@ F32_TOL = 1e-5
 BF16_TOL = 2e-2
 # cases the plan compiler rejects (none at present; the error texts are checked in test_frontend.py)
 UNSUPPORTED = set()
+# cases held to a looser elementwise bound than the dtype's, each with its reason
+LOOSER = {
+    # Sums of K products whose magnitudes add up to S ~ 750 (K = 3000 terms of products of uniform(-1, 1) values) or
+    # S ~ 500 (K = 384 terms of uniform(-2, 2) values) while the sum itself can be near 0: float32 accumulation, in
+    # any order, is good to a few 2^-24 S ~ 3e-5 absolute, which an element near 0 cannot meet at 1e-5.
+    "dot-large-k": 4e-5,
+    "dot-sum-two-products-bias": 4e-5,
+}
 
 
 @pytest.mark.parametrize("name", [n for n in op_cases.case_names() if n not in UNSUPPORTED])
@@ -34,8 +43,9 @@ def test_op_case(client, name):
         assert g.shape == tuple(shape)
         if dt in ("f32", "bf16", "f16") and not c.exact:
             tol = BF16_TOL if "bf16" in c.dtypes or dt == "bf16" else F32_TOL
-            e = rel_err(g, w)
-            assert e <= tol, f"{name} output {k}: relative error {e:.3e} > {tol}"
+            tol = LOOSER.get(name, tol)
+            ratio = closeness(g, w, tol, tol)
+            assert ratio <= 1.0, f"{name} output {k}: {ratio:.3f} x the bound |d| <= {tol} + {tol} |want|"
         else:
             gw = g.view(np.uint32) if g.dtype == np.float32 else g
             ww = np.asarray(w).astype(g.dtype)

@@ -3,7 +3,7 @@ finishes in seconds), plus size-independent properties at the full benchmark siz
 import numpy as np
 import pytest
 
-from conftest import rel_err
+from conftest import closeness
 from shlo_oracle import Oracle, round_bf16
 
 pytestmark = pytest.mark.gpu
@@ -18,13 +18,15 @@ def _run_both(client, program):
     return got, want
 
 
-def _worst(program, got, want, kinds=("f",)):
+def _worst(program, got, want, tol=1e-5):
+    """Worst ratio to the reference's elementwise rule |got - want| <= tol + tol |want| (tests/test_ops.py:91-105)
+    over the float outputs (<= 1 passes); integer outputs must be equal."""
     worst, where = 0.0, None
     for n, g, w in zip(program.output_names, got, want):
         if np.asarray(w).dtype.kind in "iub":
             assert np.array_equal(g, w), n
             continue
-        e = rel_err(g, w)
+        e = closeness(g, w, tol, tol)
         if e > worst:
             worst, where = e, n
     return worst, where
@@ -36,7 +38,7 @@ def test_mlp_train_step(client, size):
     p = configs.build_mlp(**getattr(configs, size)["mlp"])
     got, want = _run_both(client, p)
     worst, where = _worst(p, got, want)
-    assert worst <= 1e-5, (where, worst)
+    assert worst <= 1.0, (where, worst)
 
 
 def test_mlp_100_steps_loss_trajectory(client):
@@ -56,7 +58,7 @@ def test_mlp_100_steps_loss_trajectory(client):
             loss = float(runner.download(outs[-1]))
             assert abs(loss - float(ref[-1])) <= 1e-5 * abs(float(ref[-1])) + 1e-6, (step, loss, float(ref[-1]))
     for k in range(4):
-        assert rel_err(runner.download(cp.state[k]), state[k]) <= 2e-5
+        assert closeness(runner.download(cp.state[k]), state[k]) <= 1.0
 
 
 @pytest.mark.parametrize("size", ["SMALL", "MEDIUM"])
@@ -101,14 +103,10 @@ def test_resnet18_train_step(client, size):
     from jax_mps_amd.programs import configs
     p = configs.build_resnet18(**getattr(configs, size)["resnet18"])
     got, want = _run_both(client, p)
-    assert abs(float(got[-1]) - float(want[-1])) <= 1e-5 * abs(float(want[-1]))
-    # Batch statistics over a handful of elements amplify f32 rounding of the accumulation
-    # order; the oracle with float32 accumulation differs from the float64 one by the same amount.
-    ins = list(p.inputs)
-    want32 = Oracle(p.text, accum="f32").run(*ins)
-    noise = max(rel_err(a, b) for a, b in zip(want32, want))
+    assert closeness(got[-1], want[-1]) <= 1.0
     worst, where = _worst(p, got, want)
-    assert worst <= max(1e-5, 4 * noise), (where, worst, noise)
+    print(f"resnet18 {size}: worst closeness {worst:.3f} at {where}", flush=True)
+    assert worst <= 1.0, (where, worst)
 
 
 def test_resnet18_forward_only(client):
@@ -116,7 +114,7 @@ def test_resnet18_forward_only(client):
     p = configs.build_resnet18(batch=8, image=16, width=16, train=False, zero_bn2_scale=False)
     got, want = _run_both(client, p)
     worst, where = _worst(p, got, want)
-    assert worst <= 1e-5, (where, worst)
+    assert worst <= 1.0, (where, worst)
 
 
 @pytest.mark.parametrize("size", ["SMALL", "MEDIUM"])
@@ -125,8 +123,17 @@ def test_distilbert_forward(client, size, dtype, tol):
     from jax_mps_amd.programs import configs
     p = configs.build_distilbert(dtype=dtype, **getattr(configs, size)["distilbert"])
     got, want = _run_both(client, p)
-    worst, where = _worst(p, got, want)
-    assert worst <= tol, (where, worst)
+    if dtype == "bf16":
+        # The plugin keeps fused bf16 chains in float32 and rounds where a tensor is stored; the oracle rounds after
+        # every op.  Both are held to the 2e-2 rule against the unrounded evaluation of the same formulas; against
+        # each other a single element may land a few percent outside it (the roundings fall at different places).
+        ins = [round_bf16(a) if d == "bf16" else a for a, d in zip(p.inputs, p.input_dtypes)]
+        exact = Oracle(p.text, round_intermediates=False).run(*ins)
+        assert _worst(p, got, exact, tol)[0] <= 1.0 and _worst(p, want, exact, tol)[0] <= 1.0
+        assert _worst(p, got, want, tol)[0] <= 1.25
+        return
+    worst, where = _worst(p, got, want, tol)
+    assert worst <= 1.0, (where, worst)
 
 
 @pytest.mark.parametrize("size", ["SMALL", "MEDIUM"])
@@ -134,14 +141,9 @@ def test_lstm_scan_adam(client, size):
     from jax_mps_amd.programs import configs
     p = configs.build_lstm(**getattr(configs, size)["lstm"])
     got, want = _run_both(client, p)
-    for n, g, w in zip(p.output_names, got, want):
-        if n.startswith("nu."):
-            # second moments are squares of gradients: compare at the gradient's scale
-            assert rel_err(np.sqrt(np.abs(g)), np.sqrt(np.abs(w))) <= 2e-5, n
-        elif np.asarray(w).dtype.kind in "iub":
-            assert np.array_equal(g, w), n
-        else:
-            assert rel_err(g, w) <= 2e-5, n
+    worst, where = _worst(p, got, want)
+    print(f"lstm {size}: worst closeness {worst:.3f} at {where}", flush=True)
+    assert worst <= 1.0, (where, worst)
 
 
 def test_lstm_ten_steps(client):
@@ -157,7 +159,7 @@ def test_lstm_ten_steps(client):
         for k, i in p.feedback.items():
             state[i] = ref[k]
     assert int(runner.download(cp.state[15])) == 10
-    assert abs(float(runner.download(outs[-1])) - float(ref[-1])) <= 1e-4 * abs(float(ref[-1]))
+    assert closeness(runner.download(outs[-1]), ref[-1]) <= 1.0
 
 
 def test_error_paths(client):

@@ -1,12 +1,28 @@
 """Pins of the CPU oracle that the golden vectors leave open: library routines (torch CPU conv2d /
 conv_transpose2d, numpy einsum), brute force on tiny inputs, IEEE identities, and torch autograd for
 the five benchmark programs (which also pins the StableHLO emitter's VJP rules)."""
+import importlib
 import math
 
 import numpy as np
 import pytest
-import torch
-import torch.nn.functional as F
+
+
+class _Lazy:
+    """Module imported at first use.  torch ships its own HIP runtime; importing it while pytest collects would put
+    that runtime into the process before the plugin library loads, also in runs that select no test of this file."""
+
+    def __init__(self, name):
+        self._name, self._module = name, None
+
+    def __getattr__(self, attr):
+        if self._module is None:
+            self._module = importlib.import_module(self._name)
+        return getattr(self._module, attr)
+
+
+torch = _Lazy("torch")
+F = _Lazy("torch.nn.functional")
 
 import op_cases
 from jax_mps_amd.programs import configs
