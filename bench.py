@@ -24,6 +24,9 @@ PEAK_HBM_GBS = 8000.0
 PEAK_F32_MFMA_TFLOPS = 157.3
 
 
+_FUSED_SPECS = {}     # name -> ((shape, dtype), ...) of the module's arguments
+
+
 def fused_op_modules():
     """The fused-op bandwidth shapes (elementwise / reduce chains of the reference's benchmark configs,
     tests/configs/benchmark.py:14-45, and of the ResNet18 / DistilBERT programs)."""
@@ -34,6 +37,7 @@ def fused_op_modules():
         args = [b.arg(s, d) for s, d in specs]
         out = fn(b, *args)
         b.ret(*(out if isinstance(out, (list, tuple)) else [out]))
+        _FUSED_SPECS[name] = specs
         return name, b.text()
 
     n = 10_000_000
@@ -60,18 +64,18 @@ _FUSED_BYTES = {   # algorithmic bytes: distinct inputs + outputs, broadcast ope
 }
 
 
-FUSED_REPEAT = 20   # launches of each fused kernel between one pair of HIP events
+FUSED_REPEAT = 64           # launches of each fused kernel between one pair of HIP events ...
+FUSED_ROTATE_BYTES = 640e6  # ... cycling through copies of all its buffers that together hold this much: more than
+                            # twice the 256 MB memory-side cache, so every launch reads its operands from HBM
 
 
 def bench_fused_ops(client, iters=10):
     from jax_mps_amd import pjrt, runner
-    from shlo_oracle import parse
     out = []
     rng = np.random.default_rng(7)
     for name, text in fused_op_modules():
-        main = parse(text)["main"]
-        ins = [rng.standard_normal(t.shape).astype(np.float32) for t in main.body.arg_types]
-        dts = [t.dtype for t in main.body.arg_types]
+        ins = [rng.standard_normal(shape).astype(np.float32) for shape, _ in _FUSED_SPECS[name]]
+        dts = [d for _, d in _FUSED_SPECS[name]]
         exe = client.compile_and_load(text)
         bufs = runner.upload(client, ins, dts)
         for _ in range(3):
@@ -177,6 +181,7 @@ def main():
         os.environ["MI355X_TIMING"] = "all"
         os.environ["MI355X_TIMING_EVERY"] = "1"
         os.environ["MI355X_TIMING_REPEAT"] = str(FUSED_REPEAT)
+        os.environ["MI355X_TIMING_ROTATE_BYTES"] = str(int(FUSED_ROTATE_BYTES))
         print(json.dumps({"fused_ops": bench_fused_ops(client)}))
         return
     if args.config:
@@ -232,6 +237,7 @@ def main():
         os.environ["MI355X_TIMING"] = "all"
         os.environ["MI355X_TIMING_EVERY"] = "1"
         os.environ["MI355X_TIMING_REPEAT"] = str(FUSED_REPEAT)
+        os.environ["MI355X_TIMING_ROTATE_BYTES"] = str(int(FUSED_ROTATE_BYTES))
         line["fused_ops"] = bench_fused_ops(client)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()

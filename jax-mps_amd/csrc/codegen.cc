@@ -1263,7 +1263,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     int64_t vecs = (Rn + V - 1) / V;
     bool wavePerRow = vecs <= 256 && Kn >= 4;
     int64_t P = 1;                 // workgroups per output row
-    static const int perThread = getenv("MI355X_REDUCE_PER_THREAD") ? atoi(getenv("MI355X_REDUCE_PER_THREAD")) : 16;
+    static const int perThread = getenv("MI355X_REDUCE_PER_THREAD") ? atoi(getenv("MI355X_REDUCE_PER_THREAD")) : 8;
     static const int rowUnroll = getenv("MI355X_REDUCE_UNROLL") ? atoi(getenv("MI355X_REDUCE_UNROLL")) : 4;
     if (!wavePerRow && Kn < 512 && vecs > 256 * 16) {
       P = std::min<int64_t>((vecs + 256 * perThread - 1) / (256 * perThread), std::max<int64_t>(1, 8192 / Kn));
@@ -1409,7 +1409,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   int TY = 256 / TX;
   int64_t gridX = (kvecs + TX - 1) / TX;
   int64_t P = 1;
-  static const int colPerThread = getenv("MI355X_REDUCE_COL_PER_THREAD") ? atoi(getenv("MI355X_REDUCE_COL_PER_THREAD")) : 8;
+  static const int colPerThread = getenv("MI355X_REDUCE_COL_PER_THREAD") ? atoi(getenv("MI355X_REDUCE_COL_PER_THREAD")) : 16;
   if (Rn > (int64_t)TY * 16) P = std::min<int64_t>((Rn + TY * colPerThread - 1) / (TY * colPerThread), std::max<int64_t>(1, 2048 / gridX));
   bool partial = P > 1;
   Emitter em(isLeaf, V, i64);

@@ -137,6 +137,20 @@ int mi355_noalloc_setup(void);
 int mi355_copy(void* dst, const void* src, size_t bytes, mi355_stream_t s);   // kernel copy (graph-capturable)
 // up to 16 copies between pairwise disjoint buffers in one launch
 int mi355_copy_multi(int n, void* const* dst, const void* const* src, const size_t* bytes, mi355_stream_t s);
+// The same under a condition the kernel reads from device memory, so that control flow needs no host round trip:
+// mode 1 copies when the int at `flag` is non-zero (commit of a loop iteration while the loop is alive); mode 2 copies
+// when the branch index at `flag` (index_bytes wide, 0 = one-byte predicate; out of range selects branch count-1,
+// reference: ops/control_flow.cc:672-675) equals `want`.  cond == NULL copies unconditionally.
+typedef struct {
+  const void* flag;
+  int mode, index_bytes;
+  long long want, count;
+} mi355_copy_cond;
+int mi355_copy_multi_if(int n, void* const* dst, const void* const* src, const size_t* bytes, const mi355_copy_cond* cond, mi355_stream_t s);
+// loop flag (two ints: alive, iterations run while alive): init sets alive to *parent (the enclosing loop's flag) or 1 and
+// the count to 0; and folds a one-byte predicate into alive and adds the result to the count
+int mi355_flag_init(void* flag, const void* parent, mi355_stream_t s);
+int mi355_flag_and(void* flag, const void* pred, mi355_stream_t s);
 
 #ifdef __cplusplus
 }

@@ -41,8 +41,41 @@ struct MultiCopyArgs {
   const unsigned char* src[16];
   unsigned char* dst[16];
   unsigned long long bytes[16];
+  // optional condition, read on the device: mode 1 copies when *flag != 0 (a loop still running); mode 2 copies when the
+  // branch index at `flag` (indexBytes wide; 0 = one-byte predicate), clamped to the last branch when out of range, is `want`
+  const void* flag;
+  int mode, indexBytes;
+  long long want, count;
 };
+__device__ __forceinline__ bool copyEnabled(const MultiCopyArgs& a) {
+  if (a.mode == 0) return true;
+  if (a.mode == 1) return *(const int*)a.flag != 0;
+  long long idx;
+  switch (a.indexBytes) {
+    case 0: idx = *(const unsigned char*)a.flag ? 1 : 0; break;
+    case 1: idx = *(const signed char*)a.flag; break;
+    case 2: idx = *(const short*)a.flag; break;
+    case 4: idx = *(const int*)a.flag; break;
+    default: idx = *(const long long*)a.flag; break;
+  }
+  if (idx < 0 || idx >= a.count) idx = a.count - 1;
+  return idx == a.want;
+}
+// flag[0] = parent ? *parent : 1, flag[1] = 0  (pred == null), or  flag[0] = flag[0] && *pred, flag[1] += flag[0]
+// (flag[1] counts the iterations that ran while the loop was alive)
+__global__ void flag_update(int* flag, const int* parent, const unsigned char* pred) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  if (pred) {
+    const int alive = (flag[0] != 0 && *pred != 0) ? 1 : 0;
+    flag[0] = alive;
+    flag[1] += alive;
+  } else {
+    flag[0] = parent ? (*parent != 0 ? 1 : 0) : 1;
+    flag[1] = 0;
+  }
+}
 __global__ void __launch_bounds__(256) copy_multi(MultiCopyArgs a) {
+  if (!copyEnabled(a)) return;
   const int j = blockIdx.y;
   const unsigned char* src = a.src[j];
   unsigned char* dst = a.dst[j];
@@ -714,10 +747,29 @@ int mi355_copy(void* dst, const void* src, size_t bytes, mi355_stream_t s) {
   return check("copy");
 }
 
+int mi355_flag_init(void* flag, const void* parent, mi355_stream_t s) {
+  flag_update<<<1, 64, 0, (hipStream_t)s>>>((int*)flag, (const int*)parent, nullptr);
+  return check("flag_init");
+}
+int mi355_flag_and(void* flag, const void* pred, mi355_stream_t s) {
+  flag_update<<<1, 64, 0, (hipStream_t)s>>>((int*)flag, nullptr, (const unsigned char*)pred);
+  return check("flag_and");
+}
+
 int mi355_copy_multi(int n, void* const* dst, const void* const* src, const size_t* bytes, mi355_stream_t s) {
+  return mi355_copy_multi_if(n, dst, src, bytes, nullptr, s);
+}
+
+int mi355_copy_multi_if(int n, void* const* dst, const void* const* src, const size_t* bytes, const mi355_copy_cond* cond, mi355_stream_t s) {
   if (n <= 0) return 0;
   if (n > 16) return 1;
   MultiCopyArgs a;
+  a.flag = cond ? cond->flag : nullptr;
+  a.mode = cond ? cond->mode : 0;
+  a.indexBytes = cond ? cond->index_bytes : 0;
+  a.want = cond ? cond->want : 0;
+  a.count = cond ? cond->count : 0;
+  if (a.mode != 0 && !a.flag) return 1;
   size_t most = 0;
   for (int i = 0; i < n; ++i) {
     a.src[i] = (const unsigned char*)src[i];

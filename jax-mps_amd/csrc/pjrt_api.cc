@@ -551,6 +551,7 @@ PJRT_Error* Executable_GetCostAnalysis(PJRT_Executable_GetCostAnalysis_Args* a) 
     vals.emplace_back("fused_kernels", (double)p.kernels.size());
     vals.emplace_back("arena_bytes", (double)p.arenaBytes);
     vals.emplace_back("compile_seconds", e->exe->compileSeconds);
+    vals.emplace_back("loop.host_syncs", (double)e->exe->loopHostSyncs());
     for (auto& kv : e->exe->timings()) {
       vals.emplace_back(kv.first + ".count", (double)kv.second.count);
       vals.emplace_back(kv.first + ".time_ms", kv.second.ms);

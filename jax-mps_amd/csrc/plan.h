@@ -71,7 +71,7 @@ struct AttentionDesc {   // softmax(scale * Q K^T, masked -> `masked`) V, tensor
 struct Plan;
 
 struct Step {
-  enum Kind { Kernel, Gemm, Conv, ScatterRows, Copy, Fill, While, Case, GemmGroup, Attention } kind = Kernel;
+  enum Kind { Kernel, Gemm, Conv, ScatterRows, Copy, Fill, While, Case, GemmGroup, Attention, FlagInit, FlagAnd } kind = Kernel;
   std::string label;  // op name(s) for profiling ranges and error messages
 
   // Kernel
@@ -100,6 +100,12 @@ struct Step {
   BufRef src, dst;
   int64_t bytes = 0;
   std::vector<int64_t> copyBytes;
+  // Conditional copy, decided on the device (no host read-back): condMode 1 copies while the loop flag at condBuf is
+  // set; condMode 2 copies when the branch index at condBuf (type condType) selects branch condWant of condCount.
+  BufRef condBuf;
+  int condMode = 0;
+  DType condType = DType::S32;
+  int64_t condWant = 0, condCount = 0;
 
   // While / Case
   std::unique_ptr<Plan> cond;                 // While: evaluates the predicate into predBuf
@@ -107,6 +113,13 @@ struct Step {
   BufRef predBuf;                             // i1 (While) or i32 index (Case)
   int64_t tripCount = -1;                     // >= 0 when the loop is counted and the count is static
   DType predType = DType::Pred;
+  // Dynamic While: the loop's alive flag (one int on the device).  Iterations run in chunks without host
+  // round trips: each evaluates the condition, folds it into the flag (FlagAnd), runs the body into temporaries and
+  // commits the carries with copies conditional on the flag; the host reads the flag once per chunk.
+  // FlagInit: flagBuf = parentFlag (kind None: 1).  FlagAnd: flagBuf &= predBuf.
+  // Case with `predicated`: every branch runs and the result copies are conditional on the index (no host read).
+  BufRef flagBuf, parentFlag;
+  bool predicated = false;
 };
 
 struct Plan {

@@ -111,6 +111,13 @@ class Planner {
   std::unordered_set<Op*> emitted_;
   std::unordered_map<Op*, Op*> heldDots_;   // later product of add(dot, dot) -> the earlier one waiting for it
   int time_ = 0;
+  // Regions that may execute speculatively (the body of a dynamic loop past its last iteration, the branches of a
+  // case that runs all of them and keeps one result) must leave every buffer defined outside them untouched: inside,
+  // no value is updated in place in a storage older than the region (ids below the floor).
+  std::vector<int> specFloors_;
+  std::vector<int> aliveFlags_;   // flag storages of the enclosing dynamic loops
+  int loopDepth_ = 0;
+  bool outerStorage(int sid) const { return !specFloors_.empty() && sid < specFloors_.back(); }
 
   // ---------------------------------------------------------------- storages
   int newStorage(size_t bytes, BufRef::Kind kind = BufRef::Temp, int index = 0) {
@@ -1530,7 +1537,8 @@ class Planner {
     int osid = storageOf(operand);
     int sid;
     int t = ++time_;
-    bool inPlace = st_[osid].kind == BufRef::Temp && st_[osid].values == 1 && operand->users.size() == 1 && !boundToOutput_.count(osid);
+    bool inPlace = st_[osid].kind == BufRef::Temp && st_[osid].values == 1 && operand->users.size() == 1 && !boundToOutput_.count(osid) &&
+                   !outerStorage(osid);
     if (inPlace) {
       sid = osid;
     } else {
@@ -1569,7 +1577,7 @@ class Planner {
     if (!hasStorage(operand)) materializeNow(operand, plan);
     int osid = storageOf(operand);
     // in place when every other reader of the operand buffer has already been issued
-    bool inPlace = st_[osid].kind == BufRef::Temp && !boundToOutput_.count(osid);
+    bool inPlace = st_[osid].kind == BufRef::Temp && !boundToOutput_.count(osid) && !outerStorage(osid);
     if (inPlace) {
       for (Op* u : operand->users) {
         if (u == op) continue;
@@ -1648,7 +1656,16 @@ class Planner {
     return n;
   }
 
-  void copyStep(Plan& plan, int src, int dst, int64_t bytes, const char* label) {
+  // `cond` (optional): a step whose condBuf / condMode / condType / condWant / condCount the copy takes over
+  void applyCond(Step& c, const Step* cond, int t) {
+    if (!cond || cond->condMode == 0) return;
+    c.condBuf = ref(cond->condBuf.index, t);
+    c.condMode = cond->condMode;
+    c.condType = cond->condType;
+    c.condWant = cond->condWant;
+    c.condCount = cond->condCount;
+  }
+  void copyStep(Plan& plan, int src, int dst, int64_t bytes, const char* label, const Step* cond = nullptr) {
     if (src == dst) return;
     int t = ++time_;
     Step c;
@@ -1657,16 +1674,18 @@ class Planner {
     c.src = ref(src, t);
     c.dst = ref(dst, t);
     c.bytes = bytes;
+    applyCond(c, cond, t);
     plan.steps.push_back(std::move(c));
   }
 
   // several copies between pairwise disjoint buffers as one launch
-  void multiCopyStep(Plan& plan, const std::vector<std::array<int, 2>>& pairs, const std::vector<int64_t>& bytes, const char* label) {
+  void multiCopyStep(Plan& plan, const std::vector<std::array<int, 2>>& pairs, const std::vector<int64_t>& bytes, const char* label,
+                     const Step* cond = nullptr) {
     std::vector<size_t> live;
     for (size_t i = 0; i < pairs.size(); ++i) if (pairs[i][0] != pairs[i][1]) live.push_back(i);
     for (size_t b = 0; b < live.size(); b += 16) {
       size_t e = std::min(live.size(), b + 16);
-      if (e - b == 1) { copyStep(plan, pairs[live[b]][0], pairs[live[b]][1], bytes[live[b]], label); continue; }
+      if (e - b == 1) { copyStep(plan, pairs[live[b]][0], pairs[live[b]][1], bytes[live[b]], label, cond); continue; }
       int t = ++time_;
       Step c;
       c.kind = Step::Copy;
@@ -1677,6 +1696,7 @@ class Planner {
         c.copyBytes.push_back(bytes[live[k]]);
         c.bytes += bytes[live[k]];
       }
+      applyCond(c, cond, t);
       plan.steps.push_back(std::move(c));
     }
   }
@@ -1730,6 +1750,9 @@ class Planner {
     if (s.dst.kind != BufRef::None) f(s.dst, true);
     if (s.bias.kind != BufRef::None) f(s.bias, false);
     if (s.predBuf.kind != BufRef::None) f(s.predBuf, false);
+    if (s.condBuf.kind != BufRef::None) f(s.condBuf, false);
+    if (s.parentFlag.kind != BufRef::None) f(s.parentFlag, false);
+    if (s.flagBuf.kind != BufRef::None) f(s.flagBuf, s.kind == Step::FlagInit || s.kind == Step::FlagAnd);
     for (auto& part : s.parts) forEachRef(part, f);
   }
 
@@ -1774,7 +1797,8 @@ class Planner {
     for (size_t i = 0; i < n; ++i) {
       Value* v = op->operands[i];
       int osid = storageOf(v);
-      bool reuse = st_[osid].kind == BufRef::Temp && st_[osid].values == 1 && v->users.size() == 1 && !boundToOutput_.count(osid);
+      bool reuse = st_[osid].kind == BufRef::Temp && st_[osid].values == 1 && v->users.size() == 1 && !boundToOutput_.count(osid) &&
+                   !outerStorage(osid);
       if (reuse) slots[i] = osid;
       else {
         slots[i] = newStorage(v->type.bytes());
@@ -1787,6 +1811,25 @@ class Planner {
     w.kind = Step::While;
     w.label = "while";
     w.tripCount = trip;
+    // A loop whose trip count depends on data stays on the device: an alive flag, the condition folded into it every
+    // iteration, the body run into temporaries and committed under the flag, so that the host may queue iterations
+    // ahead and reads the flag once per chunk of them (the reference evaluates the condition on the host every
+    // iteration: ops/control_flow.cc:504-536).
+    static const bool deviceLoops = !getenv("MI355X_DEVICE_LOOPS") || atoi(getenv("MI355X_DEVICE_LOOPS")) != 0;
+    const bool onDevice = trip < 0 && deviceLoops;
+    int aliveSid = -1;
+    if (onDevice) {
+      aliveSid = newStorage(8);   // alive flag + count of iterations run
+      Step f;
+      f.kind = Step::FlagInit;
+      f.label = "loop flag";
+      f.flagBuf = ref(aliveSid, tStart);
+      if (!aliveFlags_.empty()) f.parentFlag = ref(aliveFlags_.back(), tStart);
+      plan.steps.push_back(std::move(f));
+      aliveFlags_.push_back(aliveSid);
+      specFloors_.push_back((int)st_.size());
+    }
+    ++loopDepth_;
     Region& cond = *op->regions[0];
     Region& body = *op->regions[1];
     for (size_t i = 0; i < n; ++i) { bind(cond.args[i].get(), slots[i]); bind(body.args[i].get(), slots[i]); }
@@ -1797,6 +1840,18 @@ class Planner {
     Value* pred = cond.terminator()->operands.at(0);
     if (!hasStorage(pred)) materializeNow(pred, *w.cond);
     w.predBuf = ref(storageOf(pred), ++time_);
+    Step commit;   // carries are written only while the flag is set
+    if (onDevice) {
+      Step a;
+      a.kind = Step::FlagAnd;
+      a.label = "loop flag &= condition";
+      int t = ++time_;
+      a.flagBuf = ref(aliveSid, t);
+      a.predBuf = ref(storageOf(pred), t);
+      w.cond->steps.push_back(std::move(a));
+      commit.condMode = 1;
+      commit.condBuf.index = aliveSid;
+    }
     auto bodyPlan = std::make_unique<Plan>();
     emitRegion(body, *bodyPlan);
     Op* ret = body.terminator();
@@ -1816,6 +1871,7 @@ class Planner {
       bool slotIsSource = false;
       for (size_t j = 0; j < n; ++j) if (j != i && src[j] == slots[i]) slotIsSource = true;
       if (slotIsSource) continue;
+      if (onDevice) continue;   // iterations past the end run too and must not touch the carries
       if (carryInPlace(*bodyPlan, src[i], slots[i], body.args[i].get())) {
         storage_[ret->operands[i]] = slots[i];
         src[i] = slots[i];
@@ -1840,9 +1896,15 @@ class Planner {
       update.push_back({src[i], slots[i]});
       updateBytes.push_back((int64_t)op->operands[i]->type.bytes());
     }
-    multiCopyStep(*bodyPlan, update, updateBytes, "loop carry update");
+    multiCopyStep(*bodyPlan, update, updateBytes, "loop carry update", onDevice ? &commit : nullptr);
     int tEnd = ++time_;
     for (size_t i = 0; i < n; ++i) ref(slots[i], tEnd);
+    --loopDepth_;
+    if (onDevice) {
+      w.flagBuf = ref(aliveSid, tEnd);
+      aliveFlags_.pop_back();
+      specFloors_.pop_back();
+    }
     loops_.push_back({tStart, tEnd});
     w.bodies.push_back(std::move(bodyPlan));
     for (size_t i = 0; i < n; ++i) bind(op->results[i].get(), slots[i]);
@@ -1860,18 +1922,41 @@ class Planner {
     c.predType = index->type.dt;
     std::vector<int> outs;
     for (auto& r : op->results) outs.push_back(newStorage(r->type.bytes()));
-    for (auto& rg : op->regions) {
+    // Inside a loop a case with small branches runs all of them and keeps the selected results (copies conditional on
+    // the index, decided on the device), so that the loop body needs no host round trip and stays one launch sequence.
+    static const bool deviceCases = !getenv("MI355X_DEVICE_CASES") || atoi(getenv("MI355X_DEVICE_CASES")) != 0;
+    int branchOps = 0;
+    for (auto& rg : op->regions) branchOps += countOps(*rg);
+    c.predicated = deviceCases && loopDepth_ > 0 && branchOps <= 96;
+    if (c.predicated) specFloors_.push_back((int)st_.size());
+    Step select;
+    select.condMode = c.predicated ? 2 : 0;
+    select.condBuf.index = storageOf(index);
+    select.condType = index->type.dt;
+    select.condCount = (int64_t)op->regions.size();
+    for (size_t b = 0; b < op->regions.size(); ++b) {
+      auto& rg = op->regions[b];
       analyze(*rg);
       auto bp = std::make_unique<Plan>();
       emitRegion(*rg, *bp);
       Op* ret = rg->terminator();
+      select.condWant = (int64_t)b;
+      std::vector<std::array<int, 2>> pairs;
+      std::vector<int64_t> sizes;
       for (size_t k = 0; k < op->results.size(); ++k) {
         Value* v = ret->operands.at(k);
         if (!hasStorage(v)) materializeNow(v, *bp);
-        copyStep(*bp, storageOf(v), outs[k], (int64_t)v->type.bytes(), "case result");
+        pairs.push_back({storageOf(v), outs[k]});
+        sizes.push_back((int64_t)v->type.bytes());
       }
+      // results of one branch may share a source (the same value returned twice): single copies then
+      bool distinct = true;
+      for (size_t x = 0; x < pairs.size(); ++x) for (size_t y = x + 1; y < pairs.size(); ++y) if (pairs[x][0] == pairs[y][0]) distinct = false;
+      if (distinct) multiCopyStep(*bp, pairs, sizes, "case result", c.predicated ? &select : nullptr);
+      else for (size_t k = 0; k < pairs.size(); ++k) copyStep(*bp, pairs[k][0], pairs[k][1], sizes[k], "case result", c.predicated ? &select : nullptr);
       c.bodies.push_back(std::move(bp));
     }
+    if (c.predicated) specFloors_.pop_back();
     int tEnd = ++time_;
     for (auto o : outs) { ref(o, tStart); ref(o, tEnd); }
     loops_.push_back({tStart, tEnd});
@@ -2070,6 +2155,9 @@ class Planner {
       s.dst = finalRef(s.dst);
       s.bias = finalRef(s.bias);
       s.predBuf = finalRef(s.predBuf);
+      s.condBuf = finalRef(s.condBuf);
+      s.flagBuf = finalRef(s.flagBuf);
+      s.parentFlag = finalRef(s.parentFlag);
       if (s.cond) patch(*s.cond);
       for (auto& b : s.bodies) patch(*b);
     }
@@ -2087,11 +2175,13 @@ class Planner {
 
   void dumpPlan(const Plan& p, int indent) {
     std::ostringstream o;
-    static const char* kinds[] = {"kernel", "gemm", "conv", "scatter", "copy", "fill", "while", "case", "gemm-group", "attention"};
+    static const char* kinds[] = {"kernel", "gemm", "conv", "scatter", "copy", "fill", "while", "case", "gemm-group", "attention", "flag-init", "flag-and"};
     for (auto& s : p.steps) {
       o << std::string(indent, ' ') << kinds[s.kind] << " " << s.label;
       if (s.kind == Step::Kernel) o << " k" << s.kernel << " grid " << s.grid[0] << "x" << s.grid[1] << " bytes " << s.algoBytes;
-      if (s.kind == Step::While) o << " trip " << s.tripCount;
+      if (s.kind == Step::While) o << " trip " << s.tripCount << (s.flagBuf.kind != BufRef::None ? " on-device" : "");
+      if (s.kind == Step::Case && s.predicated) o << " all-branches";
+      if (s.kind == Step::Copy && s.condMode) o << (s.condMode == 1 ? " if-alive" : " if-selected");
       o << "\n";
       P.dump += o.str();
       o.str("");

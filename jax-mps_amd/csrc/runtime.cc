@@ -228,6 +228,8 @@ Executable::Executable(std::unique_ptr<CompiledProgram> prog) : prog_(std::move(
   timingEvery_ = every ? std::max(1, atoi(every)) : 1;
   const char* repeat = getenv("MI355X_TIMING_REPEAT");   // launches of a timed fused kernel per event pair
   timingRepeat_ = repeat ? std::max(1, atoi(repeat)) : 1;
+  const char* rot = getenv("MI355X_TIMING_ROTATE_BYTES");
+  rotateBytes_ = rot ? std::max<long long>(0, atoll(rot)) : 0;
   const char* gr = getenv("MI355X_GRAPHS");   // "0" runs loop bodies launch by launch
   useGraphs_ = !(gr && gr[0] == '0');
   loadKernels();
@@ -245,6 +247,11 @@ Executable::~Executable() {
   try { dev.sync(); } catch (...) {}
   if (arena_) dev.release(arena_);
   if (consts_) dev.release(consts_);
+  for (auto& sh : shadows_) {
+    for (void* p : sh.params) dev.release(p);
+    for (void* p : sh.outs) dev.release(p);
+    if (sh.arena) dev.release(sh.arena);
+  }
   for (auto& g : loopGraphs_) for (auto& e : g.second.entries) if (e.exec) mi355_graph_destroy(e.exec);
   for (auto e : eventPool_) mi355_event_destroy(e);
   for (auto& p : pending_) { mi355_event_destroy(p.a); mi355_event_destroy(p.b); }
@@ -283,6 +290,41 @@ void* Executable::resolve(const BufRef& r, const std::vector<DeviceBuffer*>& in,
     case BufRef::Temp: return (char*)arena_ + r.offset;
     case BufRef::Const: return (char*)consts_ + r.offset;
     default: return nullptr;
+  }
+}
+
+void* Executable::resolveIn(const BufRef& r, int set, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) const {
+  if (set == 0 || shadows_.empty()) return resolve(r, in, out);
+  const ShadowSet& sh = shadows_[(size_t)set - 1];
+  switch (r.kind) {
+    case BufRef::Param: return (char*)sh.params[(size_t)r.index] + r.offset;
+    case BufRef::Output: return (char*)sh.outs[(size_t)r.index] + r.offset;
+    case BufRef::Temp: return (char*)sh.arena + r.offset;
+    default: return resolve(r, in, out);
+  }
+}
+
+// Copies of the call's arguments (same contents), results and arena, until all sets together hold rotateBytes_.
+void Executable::prepareShadows(const std::vector<DeviceBuffer*>& in) {
+  if (rotateBytes_ <= 0 || !shadows_.empty()) return;
+  Device& dev = Device::get();
+  int64_t perSet = prog_->arenaBytes;
+  for (auto& t : prog_->paramTypes) perSet += (int64_t)t.bytes();
+  for (auto& o : prog_->outputs) perSet += (int64_t)o.type.bytes();
+  if (perSet <= 0) return;
+  int64_t sets = std::max<int64_t>(3, (rotateBytes_ + perSet - 1) / perSet);
+  sets = std::min<int64_t>(sets, 256);
+  for (int64_t k = 1; k < sets; ++k) {
+    ShadowSet sh;
+    for (size_t i = 0; i < in.size(); ++i) {
+      size_t bytes = std::max<size_t>(prog_->paramTypes[i].bytes(), 4);
+      void* p = dev.alloc(bytes);
+      check(mi355_memcpy_d2d(p, in[i]->ptr, prog_->paramTypes[i].bytes(), dev.stream()), "shadow copy");
+      sh.params.push_back(p);
+    }
+    for (auto& o : prog_->outputs) sh.outs.push_back(dev.alloc(std::max<size_t>(o.type.bytes(), 4)));
+    if (prog_->arenaBytes > 0) sh.arena = dev.alloc((size_t)prog_->arenaBytes);
+    shadows_.push_back(std::move(sh));
   }
 }
 
@@ -357,6 +399,7 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
   static const bool detail = getenv("MI355X_TIMING_DETAIL") != nullptr;   // one statistics row per step label
   if (doTime && detail) kind += ":" + s.label;
   mi355_event_t ea = nullptr, eb = nullptr;
+  int kernelLaunches = 1;   // launches of a Kernel step between its two events
   if (doTime) {
     ea = getEvent();
     eb = getEvent();
@@ -369,12 +412,25 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       size_t n = s.args.size();
       if (n > 256) throw RuntimeError("fused kernel with more than 256 arguments");
       for (size_t i = 0; i < n; ++i) { ptrs[i] = resolve(s.args[i], in, out); argv[i] = &ptrs[i]; }
-      // A timed fused kernel may be launched several times between its two events: the kernels are pure
-      // functions of their inputs (or rewrite the same window in place), so the result is unchanged, and
-      // the cost of the event pair is spread over the launches.
-      const int launches = doTime ? timingRepeat_ : 1;
-      for (int r = 0; r < launches; ++r)
+      // A timed fused kernel may be launched several times between its two events, which spreads the cost of the
+      // event pair over the launches.  That leaves the result unchanged only for a kernel that is a pure function
+      // of its inputs: one that writes a buffer another of its arguments reads (a loop carry updated in place,
+      // x = f(x)) is launched once.
+      int launches = doTime ? timingRepeat_ : 1;
+      if (launches > 1) {
+        for (size_t i = 0; i < n && launches > 1; ++i) {
+          if (i >= s.argWrites.size() || !s.argWrites[i]) continue;
+          for (size_t j = 0; j < n; ++j)
+            if (j != i && ptrs[j] == ptrs[i]) { launches = 1; break; }
+        }
+      }
+      kernelLaunches = launches;
+      const int sets = launches > 1 ? (int)shadows_.size() + 1 : 1;
+      for (int r = 0; r < launches; ++r) {
+        if (sets > 1)
+          for (size_t i = 0; i < n; ++i) ptrs[i] = resolveIn(s.args[i], r % sets, in, out);
         check(mi355_launch((mi355_function_t)prog_->kernels[s.kernel].function, s.grid, s.block, argv, (int)n, st), s.label.c_str());
+      }
       break;
     }
     case Step::Gemm: {
@@ -443,7 +499,17 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
                                resolve(s.args[3], in, out), st), "scatter");
       break;
     }
-    case Step::Copy:
+    case Step::Copy: {
+      mi355_copy_cond cond;
+      const mi355_copy_cond* pc = nullptr;
+      if (s.condMode != 0) {
+        cond.flag = resolve(s.condBuf, in, out);
+        cond.mode = s.condMode;
+        cond.index_bytes = s.condType == DType::Pred ? 0 : (int)dtypeSize(s.condType);
+        cond.want = s.condWant;
+        cond.count = s.condCount;
+        pc = &cond;
+      }
       if (!s.copyBytes.empty()) {
         const void* srcs[16];
         void* dsts[16];
@@ -454,16 +520,32 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
           dsts[i] = resolve(s.args[2 * i + 1], in, out);
           sizes[i] = (size_t)s.copyBytes[i];
         }
-        check(mi355_copy_multi((int)n, dsts, srcs, sizes, st), "copy");
+        check(mi355_copy_multi_if((int)n, dsts, srcs, sizes, pc, st), "copy");
+        break;
+      }
+      if (pc) {
+        const void* src1 = resolve(s.src, in, out);
+        void* dst1 = resolve(s.dst, in, out);
+        size_t size1 = (size_t)s.bytes;
+        check(mi355_copy_multi_if(1, &dst1, &src1, &size1, pc, st), "conditional copy");
         break;
       }
       check(mi355_copy(resolve(s.dst, in, out), resolve(s.src, in, out), (size_t)s.bytes, st), "copy");
       break;
+    }
     case Step::Fill: break;
+    case Step::FlagInit:
+      check(mi355_flag_init(resolve(s.flagBuf, in, out), s.parentFlag.kind == BufRef::None ? nullptr : resolve(s.parentFlag, in, out), st), "loop flag");
+      break;
+    case Step::FlagAnd:
+      check(mi355_flag_and(resolve(s.flagBuf, in, out), resolve(s.predBuf, in, out), st), "loop flag update");
+      break;
     case Step::While: {
       if (s.tripCount >= 0) {
         // counted loop: the trip count is known, iterations are queued back to back with no host round trip
         runCountedLoop(s, in, out);
+      } else if (s.flagBuf.kind != BufRef::None) {
+        runDeviceLoop(s, in, out);
       } else {
         unsigned char* flag = (unsigned char*)dev.pinnedScratch();
         while (true) {
@@ -477,6 +559,11 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       break;
     }
     case Step::Case: {
+      if (s.predicated) {
+        // every branch runs; only the selected one's result copies take effect (decided on the device)
+        for (auto& b : s.bodies) runPlan(*b, in, out);
+        break;
+      }
       long long idx = 0;
       size_t sz = dtypeSize(s.predType);
       void* host = dev.pinnedScratch();
@@ -496,7 +583,7 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
   }
   if (doTime) {
     mi355_event_record(eb, st);
-    const double launches = s.kind == Step::Kernel ? (double)timingRepeat_ : 1.0;
+    const double launches = (double)kernelLaunches;
     pending_.push_back({ea, eb, kind, flops * launches, bytes * launches, launches});
     if (pending_.size() > 20000) resolvePending();
   }
@@ -508,8 +595,13 @@ bool Executable::capturable(const Plan& p) {
   bool ok = true;
   for (auto& s : p.steps) {
     switch (s.kind) {
-      case Step::Kernel: case Step::Gemm: case Step::GemmGroup: case Step::Attention: case Step::Conv: case Step::ScatterRows: case Step::Copy: case Step::Fill: break;
+      case Step::Kernel: case Step::Gemm: case Step::GemmGroup: case Step::Attention: case Step::Conv: case Step::ScatterRows: case Step::Copy: case Step::Fill:
+      case Step::FlagInit: case Step::FlagAnd: break;
       case Step::While: ok = ok && s.tripCount >= 0 && capturable(*s.bodies[0]); break;   // dynamic loops read a flag back on the host
+      case Step::Case:
+        ok = ok && s.predicated;
+        for (auto& b : s.bodies) ok = ok && capturable(*b);
+        break;
       default: ok = false; break;
     }
   }
@@ -522,15 +614,47 @@ bool Executable::capturable(const Plan& p) {
 // graph holding several iterations and replayed; the host then issues one launch per replay
 // instead of one per kernel.
 void Executable::runCountedLoop(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
+  replayIterations(s, false, s.tripCount, in, out);
+}
+
+// A loop whose trip count depends on data.  Iterations are queued in chunks (4, 4, 8, 16, 32, 64, 64 ...) with no host round trip
+// inside a chunk: each iteration evaluates the condition, folds it into the loop's flag on the device, runs the body
+// into temporaries and commits the carries only while the flag is set, so iterations queued past the end change
+// nothing.  The host reads the flag once per chunk.  At most as many iterations run past the end as ran before it.
+void Executable::runDeviceLoop(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
+  Device& dev = Device::get();
+  int* flag = (int*)dev.pinnedScratch();
+  // The first chunk is as long as the loop ran the last time (plus the evaluation of the condition that ends it):
+  // a loop that repeats its trip count from call to call then costs one round trip and queues nothing past its end.
+  int64_t& last = lastTrips_[&s];
+  int64_t chunk = last > 0 ? std::min<int64_t>(last + 1, 256) : 4;
+  while (true) {
+    replayIterations(s, true, chunk, in, out);
+    check(mi355_memcpy_d2h(flag, resolve(s.flagBuf, in, out), 8, dev.stream()), "loop flag read-back");
+    dev.sync();
+    ++loopSyncs_;
+    if (!flag[0]) break;
+    chunk = std::min<int64_t>(std::max<int64_t>(4, (int64_t)flag[1]), 64);   // as many again as have run, 64 at most
+  }
+  last = flag[1];
+}
+
+// `count` iterations of a loop: the body alone (counted loops) or condition + body (loops kept alive by a device flag).
+void Executable::replayIterations(const Step& s, bool withCond, int64_t trip, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
   Device& dev = Device::get();
   const Plan& body = *s.bodies[0];
-  const int64_t trip = s.tripCount;
-  const bool graphOk = useGraphs_ && !capturing_ && timingKinds_.empty() && trip >= 4 && !body.steps.empty() && capturable(body);
+  auto runOne = [&]() {
+    if (withCond) runPlan(*s.cond, in, out);
+    runPlan(body, in, out);
+  };
+  const size_t unitSteps = body.steps.size() + (withCond ? s.cond->steps.size() : 0);
+  const bool graphOk = useGraphs_ && !capturing_ && timingKinds_.empty() && trip >= (withCond ? 16 : 4) && unitSteps > 0 && capturable(body) &&
+                       (!withCond || capturable(*s.cond));
   if (!graphOk) {
-    for (int64_t i = 0; i < trip; ++i) runPlan(body, in, out);
+    for (int64_t i = 0; i < trip; ++i) runOne();
     return;
   }
-  runPlan(body, in, out);   // first iteration eagerly: finishes lazy one-time set-up outside the capture
+  if (!withCond) runOne();   // first iteration eagerly: finishes lazy one-time set-up outside the capture
   LoopGraphs& lgs = loopGraphs_[&s];
   if (!lgs.scanned) {
     std::function<void(const Plan&)> scan = [&](const Plan& p) {
@@ -544,6 +668,7 @@ void Executable::runCountedLoop(const Step& s, const std::vector<DeviceBuffer*>&
       }
     };
     scan(body);
+    if (withCond) scan(*s.cond);
     lgs.scanned = true;
   }
   uint64_t sig = 1469598103934665603ull;
@@ -562,12 +687,13 @@ void Executable::runCountedLoop(const Step& s, const std::vector<DeviceBuffer*>&
       mi355_graph_destroy(hit->exec);
       hit->exec = nullptr;
     }
-    const int64_t per = std::max<int64_t>(1, std::min<int64_t>(trip - 1, 1024 / (int64_t)body.steps.size()));
+    // a flag-driven loop is replayed in sub-chunks of 16 iterations, so that one graph serves whatever length the next chunk has
+    const int64_t per = std::max<int64_t>(1, std::min<int64_t>(withCond ? 16 : trip - 1, 1024 / (int64_t)unitSteps));
     mi355_stream_t st = dev.stream();
     check(mi355_capture_begin(st), "graph capture");
     capturing_ = true;
     try {
-      for (int64_t i = 0; i < per; ++i) runPlan(body, in, out);
+      for (int64_t i = 0; i < per; ++i) runOne();
     } catch (...) {
       capturing_ = false;
       mi355_graph_t dead = nullptr;
@@ -585,9 +711,9 @@ void Executable::runCountedLoop(const Step& s, const std::vector<DeviceBuffer*>&
   }
   hit->lastUse = ++graphClock_;
   LoopGraph& lg = *hit;
-  int64_t left = trip - 1;
+  int64_t left = withCond ? trip : trip - 1;
   for (; left >= lg.itersPerLaunch; left -= lg.itersPerLaunch) check(mi355_graph_launch(lg.exec, dev.stream()), "graph launch");
-  for (; left > 0; --left) runPlan(body, in, out);
+  for (; left > 0; --left) runOne();
 }
 
 void Executable::runPlan(const Plan& plan, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
@@ -614,6 +740,7 @@ std::vector<std::shared_ptr<DeviceBuffer>> Executable::execute(const std::vector
     outs.push_back(std::move(b));
   }
   timedCall_ = (executeCount_++ % timingEvery_) == 0;
+  if (timedCall_ && timingRepeat_ > 1 && !timingKinds_.empty()) prepareShadows(inputs);
   runPlan(prog_->plan, inputs, outPtrs);
   return outs;
 }

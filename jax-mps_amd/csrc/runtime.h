@@ -87,6 +87,7 @@ class Executable {
   // Aggregated step timings (enabled with MI355X_TIMING=<kinds|all>); resolves pending events.
   std::map<std::string, KindStat> timings();
   double compileSeconds = 0;
+  int64_t loopHostSyncs() const { return loopSyncs_; }   // host round trips spent reading loop flags so far
 
  private:
   std::unique_ptr<CompiledProgram> prog_;
@@ -101,6 +102,14 @@ class Executable {
   std::string timingKinds_;
   int timingEvery_ = 1;
   int timingRepeat_ = 1;
+  // Measurement aid (MI355X_TIMING_ROTATE_BYTES=B): the repeated launches of a timed fused kernel cycle through
+  // private copies of every buffer of the program (arguments, results, arena), enough of them to hold B bytes, so
+  // that no launch finds its operands in a cache left there by the launch before.
+  int64_t rotateBytes_ = 0;
+  struct ShadowSet { std::vector<void*> params, outs; void* arena = nullptr; };
+  std::vector<ShadowSet> shadows_;     // sets 1 .. N-1; set 0 is the call's own buffers
+  void prepareShadows(const std::vector<DeviceBuffer*>& in);
+  void* resolveIn(const BufRef& r, int set, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) const;
   uint64_t executeCount_ = 0;
   bool timedCall_ = true;
 
@@ -119,6 +128,10 @@ class Executable {
   bool capturing_ = false;
   bool capturable(const Plan& p);
   void runCountedLoop(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
+  void runDeviceLoop(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
+  void replayIterations(const Step& s, bool withCond, int64_t count, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
+  std::map<const Step*, int64_t> lastTrips_;   // iterations each dynamic loop ran on the previous call
+  int64_t loopSyncs_ = 0;   // host round trips spent on loop flags (reported by the cost analysis as "loop.host_syncs")
 
   void loadKernels();
   void* resolve(const BufRef& r, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) const;

@@ -598,6 +598,88 @@ for k, v in enumerate([0, 1, 2, 5, -1]):
     case(f"case-index-{v}", _case3, np.int32(v), f32(290 + k, 4), exact=True)
 
 
+# ---- loops whose trip count depends on data (they run in chunks on the device, the host reads one flag per chunk) and
+# cases inside loops (all branches run, the selected result is kept)
+def _collatz(b, n):
+    # steps until n reaches 1 (27 takes 111 steps: several chunks, then iterations past the end that must change nothing)
+    one, two, three = b.constant(1, "i32"), b.constant(2, "i32"), b.constant(3, "i32")
+
+    def body(v, steps):
+        even = b.compare(b.remainder(v, two), b.constant(0, "i32"), "EQ")
+        return [b.select(even, b.div(v, two), b.add(b.mul(v, three), one)), b.add(steps, 1)]
+    r = b.while_loop([n, b.constant(0, "i32")], lambda v, steps: b.compare(v, one, "GT"), body)
+    return [r[0], r[1]]
+
+
+for start in (27, 1, 6, 97, 871):
+    case(f"while-dynamic-collatz-{start}", _collatz, np.int32(start), exact=True)
+
+
+def _dynamic_scan(b, xs, limit):
+    # carries updated by dynamic_update_slice and a running sum; stops when the sum passes a limit given at run time
+    T, n = xs.shape
+    z = b.constant(0, "i32")
+
+    def body(i, acc, out):
+        x_t = b.reshape(b.dynamic_slice(xs, [i, z], [1, n]), (n,))
+        acc2 = b.add(acc, x_t)
+        return [b.add(i, 1), acc2, b.dynamic_update_slice(out, b.reshape(acc2, (1, n)), [i, z])]
+
+    def cond(i, acc, out):
+        return b.and_(b.compare(i, T, "LT"), b.compare(b.reduce_sum(acc, [0]), limit, "LT"))
+    r = b.while_loop([z, b.zeros((n,)), b.zeros((T, n))], cond, body)
+    return [r[0], r[1], r[2]]
+
+
+case("while-dynamic-scan-stops-early", _dynamic_scan, f32(2400, 40, 6, lo=0.0, hi=1.0), np.float32(30.0))
+case("while-dynamic-scan-runs-out", _dynamic_scan, f32(2401, 40, 6, lo=0.0, hi=1.0), np.float32(1e9))
+case("while-dynamic-zero-trip", _dynamic_scan, f32(2402, 40, 6, lo=0.0, hi=1.0), np.float32(-1.0), exact=True)
+
+
+def _dynamic_nested(b, n, x):
+    # outer loop bounded by an argument; inner loop halves a value until it is small (also data dependent); on the
+    # iterations queued past the end of the outer loop the inner one must not run at all
+    z = b.constant(0, "i32")
+
+    def outer(i, acc):
+        start = b.add(b._bcast_np(b.convert(i, "f32"), x.shape), x)
+        inner = b.while_loop([start, b.constant(0, "i32")], lambda v, k: b.compare(b.reduce_max(b.abs(v), [0]), 0.25, "GT"),
+                             lambda v, k: [b.mul(v, 0.5), b.add(k, 1)])
+        return [b.add(i, 1), b.add(acc, b.convert(inner[1], "f32"))]
+    r = b.while_loop([z, b.constant(0.0, "f32")], lambda i, acc: b.compare(i, n, "LT"), outer)
+    return [r[0], r[1]]
+
+
+case("while-dynamic-nested", _dynamic_nested, np.int32(6), f32(2403, 5, lo=0.5, hi=1.0), exact=True)
+
+
+def _case_in_loop(b, sel, x):
+    # a three-way switch on a value read from an argument vector inside a counted loop
+    z = b.constant(0, "i32")
+
+    def body(i, acc):
+        idx = b.reshape(b.dynamic_slice(sel, [i], [1]), ())
+        y = b.case(idx, [lambda: b.mul(acc, 2.0), lambda: b.add(acc, x), lambda: b.neg(acc)], [(x.shape, "f32")])[0]
+        return [b.add(i, 1), y]
+    return b.while_loop([z, x], lambda i, acc: b.compare(i, 8, "LT"), body)[1]
+
+
+case("case-inside-counted-loop", _case_in_loop, np.array([0, 1, 2, 1, 7, -3, 0, 1], np.int32), f32(2404, 6), exact=True)
+
+
+def _case_in_dynamic_loop(b, sel, x, n):
+    z = b.constant(0, "i32")
+
+    def body(i, acc):
+        idx = b.reshape(b.dynamic_slice(sel, [i], [1]), ())
+        y = b.case(idx, [lambda: b.mul(acc, 0.5), lambda: b.add(acc, x)], [(x.shape, "f32")])[0]
+        return [b.add(i, 1), y]
+    return b.while_loop([z, x], lambda i, acc: b.compare(i, n, "LT"), body)[1]
+
+
+case("case-inside-dynamic-loop", _case_in_dynamic_loop, np.array([0, 1, 1, 0, 1, 1, 1, 0, 0, 1], np.int32), f32(2405, 6), np.int32(7), exact=True)
+
+
 def all_cases() -> List[Case]:
     return [mk() for mk in _cases]
 

@@ -58,6 +58,53 @@ def test_counted_loop_detection():
     assert "trip -1" in r.stdout
 
 
+def test_dynamic_loops_and_cases_in_loops_stay_on_the_device():
+    """A data-dependent while runs under a device flag with conditional carry commits; a case inside a loop runs all
+    of its branches with result copies selected on the device; neither needs a host read per iteration."""
+    r = plan(op_cases.get_case("while-dynamic-collatz-27").text, "--dump-plan")
+    assert "flag-init loop flag" in r.stdout and "while while trip -1 on-device" in r.stdout
+    assert "flag-and loop flag &= condition" in r.stdout and "loop carry update if-alive" in r.stdout
+    r = plan(op_cases.get_case("while-dynamic-scan-stops-early").text, "--dump-plan")
+    assert "dynamic_update_slice operand copy" in r.stdout      # no in-place update of a carry that a queued-ahead iteration could spoil
+    r = plan(op_cases.get_case("case-inside-counted-loop").text, "--dump-plan")
+    assert "case case all-branches" in r.stdout and r.stdout.count("case result if-selected") == 3
+    r = plan(op_cases.get_case("case-index-1").text, "--dump-plan")
+    assert "all-branches" not in r.stdout                        # outside loops one branch runs, chosen on the host
+
+
+def test_missing_required_attributes_are_compile_errors():
+    text = 'module { func.func public @main(%a: tensor<4xf32>) -> tensor<4xf32> {\n %0 = "stablehlo.reduce_precision"(%a) : (tensor<4xf32>) -> tensor<4xf32>\n return %0 : tensor<4xf32> } }'
+    r = plan(text)
+    assert r.returncode != 0 and "exponent_bits" in r.stderr
+    text = 'module { func.func public @main(%a: tensor<4xf32>) -> tensor<4x2xf32> {\n %0 = "stablehlo.broadcast_in_dim"(%a) : (tensor<4xf32>) -> tensor<4x2xf32>\n return %0 : tensor<4x2xf32> } }'
+    r = plan(text)
+    assert r.returncode != 0 and "dims" in r.stderr
+
+
+def test_location_aliases_result_lists_and_composites_parse():
+    text = """#loc1 = loc("x")
+module @jit_f attributes {mhlo.num_partitions = 1 : i32} {
+  func.func private @chlo.sinh.impl(%arg0: tensor<4xf32> loc(unknown)) -> tensor<4xf32> {
+    %0 = stablehlo.exponential %arg0 : tensor<4xf32> loc(#loc2)
+    %1 = stablehlo.negate %arg0 : tensor<4xf32> loc(#loc2)
+    %2 = stablehlo.exponential %1 : tensor<4xf32> loc(#loc2)
+    %3 = stablehlo.subtract %0, %2 : tensor<4xf32> loc(#loc2)
+    return %3 : tensor<4xf32> loc(#loc)
+  } loc(#loc)
+  func.func public @main(%arg0: tensor<4xf32> loc("x"), %arg1: tensor<8xf32> loc("y")) -> (tensor<4xf32>, tensor<3xf32>, tensor<3xi32>) {
+    %0 = stablehlo.composite "chlo.sinh" %arg0 {decomposition = @chlo.sinh.impl, version = 1 : i32} : (tensor<4xf32>) -> tensor<4xf32> loc(#loc3)
+    %values, %indices = chlo.top_k(%arg1, k = 3) : tensor<8xf32> -> (tensor<3xf32>, tensor<3xi32>) loc(#loc3)
+    return %0, %values, %indices : tensor<4xf32>, tensor<3xf32>, tensor<3xi32> loc(#loc)
+  } loc(#loc)
+} loc(#loc)
+#loc = loc(unknown)
+#loc2 = loc("/tmp/f.py":3:11 to :58)
+#loc3 = loc("jit(f)/sinh"(#loc2))
+"""
+    r = plan(text, "--dump-plan")
+    assert r.returncode == 0, r.stderr
+
+
 def test_lstm_scan_updates_in_place():
     p = configs.build_lstm(**configs.SMALL["lstm"])
     r = plan(p.text, "--dump-plan")

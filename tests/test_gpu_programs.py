@@ -162,6 +162,29 @@ def test_lstm_ten_steps(client):
     assert closeness(runner.download(outs[-1]), ref[-1]) <= 1.0
 
 
+def test_dynamic_loop_reads_its_flag_once_per_chunk(client):
+    """A loop of 178 data-dependent iterations (Collatz from 871): the host reads the loop's device flag after chunks
+    of 4, 4, 8, 16, 32, 64, 64 queued iterations, seven round trips in all, not one per iteration (the reference
+    evaluates the condition on the host every iteration: ops/control_flow.cc:504-536).  The next call starts with a
+    chunk as long as the loop ran before, so a loop that repeats its trip count costs one round trip."""
+    import op_cases
+    from jax_mps_amd import runner
+    c = op_cases.get_case("while-dynamic-collatz-871")
+    exe = client.compile_and_load(c.text)
+    bufs = runner.upload(client, c.inputs, c.dtypes)
+    outs = exe.execute(bufs)
+    assert [int(runner.download(o)) for o in outs] == [1, 178]
+    assert exe.cost_analysis()["loop.host_syncs"] == 7
+    for _ in range(3):       # replayed from one captured graph of 179 iterations
+        outs = exe.execute(bufs)
+        assert [int(runner.download(o)) for o in outs] == [1, 178]
+    assert exe.cost_analysis()["loop.host_syncs"] == 10
+    outs = exe.execute(runner.upload(client, [np.int32(1)], c.dtypes))      # zero iterations: everything queued runs past the end
+    assert [int(runner.download(o)) for o in outs] == [1, 0]
+    outs = exe.execute(runner.upload(client, [np.int32(27)], c.dtypes))
+    assert [int(runner.download(o)) for o in outs] == [1, 111]
+
+
 def test_error_paths(client):
     """Failures surface as PJRT errors with a code, never as crashes (reference: tests/test_ops.py:284-302)."""
     from jax_mps_amd import pjrt
