@@ -121,6 +121,9 @@ struct Func {
   bool isPublic = false;
   Region body;
   std::vector<TensorType> resultTypes;
+  // per argument: >= 0 the result the argument's buffer may be reused for (`tf.aliasing_output = k`), -2 a donor
+  // without a fixed result (`jax.buffer_donor = true`), -1 neither
+  std::vector<int> argDonation;
 };
 
 struct Module {

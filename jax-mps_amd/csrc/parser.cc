@@ -653,7 +653,15 @@ class Parser {
         v->defIndex = (int)f->body.args.size();
         define(nm, {v.get()});
         f->body.args.push_back(std::move(v));
-        if (peekc() == '{') skipBalanced('{', '}');
+        int donation = -1;
+        if (peekc() == '{') {
+          auto attrs = parseAttrDict();
+          auto al = attrs.find("tf.aliasing_output");
+          if (al != attrs.end() && al->second.kind == Attr::Int) donation = (int)al->second.i;
+          auto dn = attrs.find("jax.buffer_donor");
+          if (donation < 0 && dn != attrs.end() && dn->second.b) donation = -2;
+        }
+        f->argDonation.push_back(donation);
         skipLoc();
         if (eat(")")) break;
         expect(",");

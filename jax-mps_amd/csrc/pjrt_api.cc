@@ -683,7 +683,17 @@ PJRT_Error* LoadedExecutable_Execute(PJRT_LoadedExecutable_Execute_Args* a) {
       if (!b || !b->buf) return makeError("null input buffer at argument " + std::to_string(i), PJRT_Error_Code_INVALID_ARGUMENT);
       ins.push_back(b->buf.get());
     }
-    auto outs = a->executable->executable->exe->execute(ins);
+    // every input may be donated except those the caller lists (they have other holders); which of them the
+    // program actually takes is its own declaration (tf.aliasing_output / jax.buffer_donor on the argument)
+    std::vector<bool> mayDonate(ins.size(), true);
+    if (a->options && a->options->non_donatable_input_indices)
+      for (size_t k = 0; k < a->options->num_non_donatable_input_indices; ++k) {
+        int64_t i = a->options->non_donatable_input_indices[k];
+        if (i >= 0 && (size_t)i < mayDonate.size()) mayDonate[(size_t)i] = false;
+      }
+    for (size_t i = 0; i < ins.size(); ++i)
+      if (a->argument_lists[0][i]->buf.use_count() > 1) mayDonate[i] = false;
+    auto outs = a->executable->executable->exe->execute(ins, &mayDonate);
     for (size_t i = 0; i < outs.size(); ++i) {
       auto* pb = new PJRT_Buffer();
       pb->dims = outs[i]->type.dims;

@@ -135,6 +135,7 @@ struct CompiledProgram {
   Plan plan;
   std::vector<GenKernel> kernels;
   std::vector<TensorType> paramTypes;
+  std::vector<int> paramDonation;   // per parameter: -1 not donated by the program, otherwise donated (>= 0: to that result)
   std::vector<OutputInfo> outputs;
   std::vector<uint8_t> constPool;   // host image of the constant pool
   int64_t arenaBytes = 0;

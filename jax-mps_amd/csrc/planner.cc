@@ -2241,6 +2241,10 @@ mi355_conv_desc toAbi(const ConvDesc& c) {
 
 std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) {
   auto prog = std::make_unique<CompiledProgram>();
+  if (Func* mainFn = module->main()) {
+    prog->paramDonation = mainFn->argDonation;
+    prog->paramDonation.resize(mainFn->body.args.size(), -1);
+  }
   inlineCalls(*module);
   lowerIntegerDots(*module);
   lowerGeneralScatters(*module);

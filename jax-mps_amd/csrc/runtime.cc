@@ -720,7 +720,7 @@ void Executable::runPlan(const Plan& plan, const std::vector<DeviceBuffer*>& in,
   for (auto& s : plan.steps) runStep(s, in, out);
 }
 
-std::vector<std::shared_ptr<DeviceBuffer>> Executable::execute(const std::vector<DeviceBuffer*>& inputs) {
+std::vector<std::shared_ptr<DeviceBuffer>> Executable::execute(const std::vector<DeviceBuffer*>& inputs, const std::vector<bool>* mayDonate) {
   std::lock_guard<std::mutex> lk(mu_);
   Device& dev = Device::get();
   if (inputs.size() != prog_->paramTypes.size())
@@ -742,6 +742,17 @@ std::vector<std::shared_ptr<DeviceBuffer>> Executable::execute(const std::vector
   timedCall_ = (executeCount_++ % timingEvery_) == 0;
   if (timedCall_ && timingRepeat_ > 1 && !timingKinds_.empty()) prepareShadows(inputs);
   runPlan(prog_->plan, inputs, outPtrs);
+  if (mayDonate) {
+    for (size_t i = 0; i < inputs.size() && i < prog_->paramDonation.size(); ++i) {
+      if (prog_->paramDonation[i] == -1 || i >= mayDonate->size() || !(*mayDonate)[i]) continue;
+      bool again = false;   // the same buffer passed for another argument stays alive
+      for (size_t j = 0; j < inputs.size(); ++j) if (j != i && inputs[j] == inputs[i]) again = true;
+      if (again) continue;
+      dev.release(inputs[i]->ptr);
+      inputs[i]->ptr = nullptr;
+      inputs[i]->deleted = true;
+    }
+  }
   return outs;
 }
 

@@ -83,7 +83,11 @@ class Executable {
 
   const CompiledProgram& program() const { return *prog_; }
   // Runs the plan on the device stream; returns freshly allocated outputs (enqueued, not awaited).
-  std::vector<std::shared_ptr<DeviceBuffer>> execute(const std::vector<DeviceBuffer*>& inputs);
+  // `mayDonate` (optional, one entry per input): the caller allows the program to take that input.  An input the
+  // program declares donated (tf.aliasing_output / jax.buffer_donor) and the caller allows is consumed: once the
+  // call's work is queued its memory goes back to the allocator (stream order keeps queued readers safe) and the
+  // buffer is marked deleted (the reference ignores donation: pjrt_executable.cc:198-246).
+  std::vector<std::shared_ptr<DeviceBuffer>> execute(const std::vector<DeviceBuffer*>& inputs, const std::vector<bool>* mayDonate = nullptr);
   // Aggregated step timings (enabled with MI355X_TIMING=<kinds|all>); resolves pending events.
   std::map<std::string, KindStat> timings();
   double compileSeconds = 0;

@@ -359,9 +359,10 @@ class LoadedExecutable:
             k += n
         return out
 
-    def execute(self, buffers: Sequence[Buffer], return_event: bool = False):
+    def execute(self, buffers: Sequence[Buffer], return_event: bool = False, donate: bool = False):
         """Outputs of one PJRT_LoadedExecutable_Execute; with `return_event` also the device-complete PJRT_Event
-        handle, which the caller then destroys."""
+        handle, which the caller then destroys.  Unless `donate` is set every input is listed as non-donatable, so
+        arguments the program marks as donated (tf.aliasing_output / jax.buffer_donor) stay valid."""
         p = self.client.plugin
         n = len(buffers)
         arg_arr = (_P * max(n, 1))(*[b.handle for b in buffers])
@@ -371,6 +372,10 @@ class LoadedExecutable:
         events = (_P * 1)()
         opts = ExecuteOptions()
         opts.struct_size = C.sizeof(opts)
+        keep = (C.c_int64 * max(n, 1))(*range(n))
+        if not donate:
+            opts.non_donatable_input_indices = C.cast(keep, _P)
+            opts.num_non_donatable_input_indices = n
         a = Execute_Args(executable=self.handle, options=C.pointer(opts), argument_lists=arg_lists, num_devices=1, num_args=n,
                          output_lists=out_lists, device_complete_events=events, execute_device=None)
         p.call("PJRT_LoadedExecutable_Execute", a)

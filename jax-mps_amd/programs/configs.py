@@ -35,6 +35,9 @@ class Program:
 
 
 def _finish(name: str, b: Builder, inputs, in_names, out_names, feedback=None, meta=None) -> Program:
+    # train state threaded from step to step is donated, as jax.jit(step, donate_argnums=...) would declare it
+    for k, i in (feedback or {}).items():
+        b.donate(b._main_args[i], k)
     return Program(name, b.text(), list(inputs), list(in_names), list(out_names), [d for _, d in b.arg_types],
                    list(b.result_types), dict(feedback or {}), dict(meta or {}))
 

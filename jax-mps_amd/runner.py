@@ -38,7 +38,7 @@ class CompiledProgram:
 
     def step(self) -> List[pjrt.Buffer]:
         """One execution; outputs named in `feedback` replace the matching inputs (train-state threading)."""
-        outs = self.exe.execute(self.state)
+        outs = self.exe.execute(self.state, donate=True)      # the state inputs are consumed and replaced by the outputs
         for k, i in self.program.feedback.items():
             self.state[i] = outs[k]
         return outs

@@ -16,7 +16,7 @@ from __future__ import annotations
 
 import math
 import struct
-from typing import Callable, List, Optional, Sequence, Tuple, Union
+from typing import Callable, Dict, List, Optional, Sequence, Tuple, Union
 
 import numpy as np
 
@@ -138,6 +138,7 @@ class Builder:
         self._n = 0
         self._blocks: List[_Block] = []
         self._main_args: List[Val] = []
+        self._arg_alias: Dict[str, int] = {}
         self._main_block = _Block(2)
         self._blocks.append(self._main_block)
         self._results: List[Val] = []
@@ -166,10 +167,18 @@ class Builder:
         if vjp is not None:
             self._blk.tape.append(_Node(list(ins), list(outs), vjp))
 
-    def arg(self, shape, dtype="f32") -> Val:
+    def arg(self, shape, dtype="f32", alias_output: Optional[int] = None) -> Val:
+        """Entry-function argument; `alias_output=k` marks it donated to result k (`tf.aliasing_output`, what
+        jax.jit(..., donate_argnums=...) lowers to)."""
         v = Val(self, f"%arg{len(self._main_args)}", shape, dtype, self._main_block)
         self._main_args.append(v)
+        if alias_output is not None:
+            self._arg_alias[v.name] = int(alias_output)
         return v
+
+    def donate(self, arg: Val, output_index: int):
+        """Marks an existing argument as donated to result `output_index`."""
+        self._arg_alias[arg.name] = int(output_index)
 
     def ret(self, *vals: Val):
         self._results = list(vals)
@@ -976,7 +985,8 @@ class Builder:
 
     # -------------------------------------------------------------------- text
     def text(self) -> str:
-        args = ", ".join(f"{a.name}: {a.type}" for a in self._main_args)
+        args = ", ".join(f"{a.name}: {a.type}" + (f" {{tf.aliasing_output = {self._arg_alias[a.name]} : i32}}" if a.name in self._arg_alias else "")
+                         for a in self._main_args)
         if len(self._results) == 1:
             rts = f"({self._results[0].type} {{jax.result_info = \"result\"}})"
         else:

@@ -167,6 +167,33 @@ def test_buffer_delete_releases_the_memory(client):
     assert client.memory_stats()["bytes_in_use"] <= held - 32 * 1024 * 1024
 
 
+def test_donated_inputs_are_consumed_only_when_the_caller_allows_it(client):
+    """An argument the program declares donated (`tf.aliasing_output`, what jax.jit(..., donate_argnums) emits) is
+    consumed by Execute unless the caller lists it in non_donatable_input_indices: the buffer is deleted afterwards and
+    its memory recycled, so a train loop that threads its state does not grow (the reference ignores donation:
+    pjrt_executable.cc:198-246)."""
+    text = ("module { func.func public @main(%w: tensor<1048576xf32> {tf.aliasing_output = 0 : i32}, %g: tensor<1048576xf32>) -> tensor<1048576xf32> {\n"
+            " %0 = stablehlo.subtract %w, %g : tensor<1048576xf32>\n return %0 : tensor<1048576xf32> } }")
+    exe = client.compile_and_load(text)
+    w0 = np.arange(1 << 20, dtype=np.float32)
+    g = client.buffer_from_pyval(np.ones(1 << 20, np.float32))
+    w = client.buffer_from_pyval(w0)
+    kept = exe.execute([w, g])[0]                       # pjrt.py lists every input as non-donatable by default
+    assert not w.is_deleted() and np.array_equal(w.to_numpy(), w0)
+    base = client.memory_stats()["bytes_in_use"]
+    for step in range(5):
+        new = exe.execute([w, g], donate=True)[0]
+        assert w.is_deleted() and not g.is_deleted()    # only the declared argument is taken
+        w = new
+    assert np.array_equal(w.to_numpy(), w0 - 5)
+    assert client.memory_stats()["bytes_in_use"] <= base      # each step's input went back to the allocator
+    assert np.array_equal(kept.to_numpy(), w0 - 1)
+    # the same buffer passed for two arguments is never taken
+    both = client.buffer_from_pyval(w0)
+    out = exe.execute([both, both], donate=True)[0]
+    assert not both.is_deleted() and not out.to_numpy().any()
+
+
 def _read_varint(data, i):
     v, shift = 0, 0
     while True:
