@@ -139,8 +139,11 @@ struct CompileError : std::runtime_error {
   using std::runtime_error::runtime_error;
 };
 
-// Front end: text -> Module.  Throws CompileError with a line number.
+// Front end: program bytes -> Module.  The bytes are StableHLO text or an MLIR bytecode file holding a VHLO portable
+// artifact (rewritten to text first, bytecode.cc).  Throws CompileError with a line number.
 std::unique_ptr<Module> parseStableHLOText(const char* data, size_t size);
+bool isMlirBytecode(const char* data, size_t size);
+std::string vhloBytecodeToStableHLOText(const char* data, size_t size);
 
 // Passes (passes.cc)
 void inlineCalls(Module& m);          // replaces every "call" by the callee body

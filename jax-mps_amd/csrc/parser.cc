@@ -7,6 +7,7 @@
 // (src/pjrt_plugin/stablehlo_parser.cc:263-285, text fallback at :276-282).
 #include <cctype>
 #include <cmath>
+#include <cstdio>
 #include <cstdlib>
 #include <unordered_map>
 
@@ -1317,10 +1318,13 @@ class Parser {
 }  // namespace
 
 std::unique_ptr<Module> parseStableHLOText(const char* data, size_t size) {
-  if (size >= 4 && data[0] == 'M' && data[1] == 'L' && (unsigned char)data[2] == 0xEF && data[3] == 'R')
-    throw CompileError(
-        "the program is an MLIR bytecode (VHLO portable artifact); this build reads StableHLO text only — "
-        "pass the module as text (jax.jit(f).lower(...).as_text())");
+  if (isMlirBytecode(data, size)) {
+    // what jaxlib sends: a VHLO portable artifact in MLIR bytecode (reference: stablehlo_parser.cc:263-285)
+    std::string text = vhloBytecodeToStableHLOText(data, size);
+    if (getenv("MI355X_DUMP_BYTECODE_TEXT")) fprintf(stderr, "%s\n", text.c_str());
+    Parser p(text.data(), text.size());
+    return p.parseModule();
+  }
   Parser p(data, size);
   return p.parseModule();
 }

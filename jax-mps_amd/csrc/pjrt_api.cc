@@ -238,9 +238,29 @@ PJRT_Error* Error_ForEachPayload(PJRT_Error_ForEachPayload_Args*) { return nullp
 
 // ------------------------------------------------------------------ plugin
 PJRT_Error* Plugin_Initialize(PJRT_Plugin_Initialize_Args*) { return nullptr; }
+// The StableHLO versions whose portable artifacts the bytecode reader accepts: jaxlib serialises a module for
+// min(its own version, stablehlo_current_version) and refuses a plugin whose current version is below its minimum.
+// The reader goes by op names with any version suffix and ignores attributes it has no use for, so the range is wide.
+// (The reference advertises nothing, pjrt_client.cc:42-46, and lets MLIR's own reader take whatever jaxlib writes.)
 PJRT_Error* Plugin_Attributes(PJRT_Plugin_Attributes_Args* a) {
-  a->attributes = nullptr;
-  a->num_attributes = 0;
+  static const int64_t current[3] = {1, 9, 0}, minimum[3] = {0, 9, 0};
+  static PJRT_NamedValue attrs[2];
+  static std::once_flag once;
+  std::call_once(once, [] {
+    memset(attrs, 0, sizeof attrs);
+    const char* names[2] = {"stablehlo_current_version", "stablehlo_minimum_version"};
+    const int64_t* values[2] = {current, minimum};
+    for (int k = 0; k < 2; ++k) {
+      attrs[k].struct_size = sizeof(PJRT_NamedValue);
+      attrs[k].name = names[k];
+      attrs[k].name_size = strlen(names[k]);
+      attrs[k].type = PJRT_NamedValue_kInt64List;
+      attrs[k].int64_array_value = values[k];
+      attrs[k].value_size = 3;
+    }
+  });
+  a->attributes = attrs;
+  a->num_attributes = 2;
   return nullptr;
 }
 

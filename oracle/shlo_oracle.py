@@ -395,6 +395,8 @@ class _P:
             c = self.s[j]
             if c in "<[({":
                 depth += 1
+            elif c == ">" and j > 0 and self.s[j - 1] == "-":
+                pass                      # the arrow of a convolution's dimension numbers
             elif c in ">])}":
                 if depth == 0 and c == close:
                     break
@@ -638,6 +640,78 @@ class _P:
         op.in_types = self.type_list_paren()
         self.expect("->")
         op.out_types = self.type_list_paren() if self.peek("(") else [self.type()]
+        self._normalize_generic(op)
+
+    @staticmethod
+    def _normalize_generic(op: Op):
+        """Attribute names and shapes of the generic op form -> the ones the pretty forms produce (what the op_*
+        methods read).  Mirrors the table of the generic StableHLO assembly: each op's attribute dictionary."""
+        a = op.attrs
+        n = op.name[len("stablehlo."):] if op.name.startswith("stablehlo.") else op.name
+
+        def enum(v):
+            return v[1] if isinstance(v, tuple) and isinstance(v[0], str) and v[0].startswith("#") else v
+
+        def ints(v):
+            if isinstance(v, tuple) and len(v) == 2 and isinstance(v[0], np.ndarray):
+                return [int(x) for x in np.asarray(v[0]).reshape(-1)]
+            if isinstance(v, np.ndarray):
+                return [int(x) for x in v.reshape(-1)]
+            return list(v)
+
+        def move(old, new, conv=lambda v: v):
+            if old in a:
+                a[new] = conv(a.pop(old))
+        for k in ("comparison_direction", "compare_type", "rng_algorithm"):
+            if k in a:
+                a[k] = enum(a[k])
+        if n in ("return", "func.return"):
+            op.name = "return"
+        elif n in ("call", "func.call"):
+            op.name = "call"
+            a["callee"] = str(a["callee"]).lstrip("@")
+        elif n == "broadcast_in_dim":
+            move("broadcast_dimensions", "dims", ints)
+        elif n == "transpose":
+            move("permutation", "dims", ints)
+        elif n == "reverse":
+            move("dimensions", "dims", ints)
+        elif n == "concatenate":
+            move("dimension", "dim")
+        elif n == "dynamic_slice":
+            move("slice_sizes", "sizes", ints)
+        elif n == "pad":
+            move("edge_padding_low", "low", ints)
+            move("edge_padding_high", "high", ints)
+            move("interior_padding", "interior", ints)
+        elif n in ("slice", "reduce", "gather", "sort", "reduce_window", "select_and_scatter"):
+            for k in ("start_indices", "limit_indices", "strides", "dimensions", "slice_sizes", "window_dimensions", "window_strides",
+                      "base_dilations", "window_dilations"):
+                if k in a:
+                    a[k] = ints(a[k])
+            if n in ("reduce_window", "select_and_scatter") and "padding" in a and not isinstance(a["padding"], tuple):
+                a["padding"] = (np.asarray(ints(a["padding"]), dtype=np.int64).reshape(-1, 2), None)
+        elif n == "dot_general" and "dot_dimension_numbers" in a:
+            d = a.pop("dot_dimension_numbers")[1] or {}
+            a["batching_dims"] = (ints(d.get("lhs_batching_dimensions", [])), ints(d.get("rhs_batching_dimensions", [])))
+            a["contracting_dims"] = (ints(d.get("lhs_contracting_dimensions", [])), ints(d.get("rhs_contracting_dimensions", [])))
+        elif n == "convolution" and "dimension_numbers" in a:
+            raw = a.pop("dimension_numbers")[1]
+            groups = re.findall(r"\[([^\]]*)\]", raw)
+            a["dim_numbers"] = tuple([t.strip() for t in g.split(",")] for g in groups)
+            nsp = len(a["dim_numbers"][0]) - 2
+            win = {}
+            if "window_strides" in a:
+                win["stride"] = ints(a.pop("window_strides"))
+            if "padding" in a:
+                win["pad"] = np.asarray(ints(a.pop("padding")), dtype=np.int64).reshape(nsp, 2).tolist()
+            if "lhs_dilation" in a:
+                win["lhs_dilate"] = ints(a.pop("lhs_dilation"))
+            if "rhs_dilation" in a:
+                win["rhs_dilate"] = ints(a.pop("rhs_dilation"))
+            if "window_reversal" in a:
+                win["reverse"] = [bool(x) for x in ints(a.pop("window_reversal"))]
+            a["window"] = win
 
     def pretty_op(self, op: Op):
         n = op.name

@@ -72,6 +72,20 @@ def test_static_identity_entries(plugin):
     assert a is not None
 
 
+def test_plugin_attributes_advertise_the_stablehlo_versions(plugin):
+    """jaxlib reads stablehlo_current_version / stablehlo_minimum_version to choose the version it serialises the
+    portable artifact for (the reference advertises none: pjrt_client.cc:42-46)."""
+    a = plugin.call("PJRT_Plugin_Attributes", pjrt.Plugin_Attributes_Args())
+    arr = C.cast(a.attributes, C.POINTER(pjrt.NamedValue))
+    got = {}
+    for i in range(a.num_attributes):
+        nv = arr[i]
+        assert nv.type == 2      # PJRT_NamedValue_kInt64List
+        got[C.string_at(nv.name, nv.name_size).decode()] = [C.cast(nv.int64_array_value, C.POINTER(C.c_int64))[k] for k in range(nv.value_size)]
+    assert set(got) == {"stablehlo_current_version", "stablehlo_minimum_version"}
+    assert len(got["stablehlo_current_version"]) == 3 and got["stablehlo_minimum_version"] <= got["stablehlo_current_version"]
+
+
 def test_client_create_without_gpu_is_a_clean_error(plugin):
     """No CPU fallback: without a device PJRT_Client_Create returns a PJRT_Error (code INTERNAL)."""
     import torch

@@ -42,7 +42,7 @@ def test_unsupported_ops_are_named():
     assert r.returncode == 0   # f64 values may pass through; arithmetic on them is generated as double
 
 
-def test_bytecode_is_rejected_with_a_clear_message():
+def test_malformed_bytecode_is_rejected_with_a_clear_message():
     r = plan(b"ML\xefR" + b"\x00" * 16)
     assert r.returncode != 0 and "bytecode" in r.stderr
 
