@@ -64,6 +64,8 @@ _FUSED_BYTES = {   # algorithmic bytes: distinct inputs + outputs, broadcast ope
 }
 
 
+LOSS_CHECK_STEPS = 3         # losses of the first steps are compared with the CPU baseline's (as many as it ran)
+LOSS_CHECK_RTOL = 1e-4       # float32 losses after float32 accumulation in a different order on each side
 FUSED_REPEAT = 64           # launches of each fused kernel between one pair of HIP events ...
 FUSED_ROTATE_BYTES = 640e6  # ... cycling through copies of all its buffers that together hold this much: more than
                             # twice the 256 MB memory-side cache, so every launch reads its operands from HBM
@@ -108,16 +110,18 @@ def cpu_baseline(budget_s=12.0, batch=128):
     p = configs.build_resnet18(batch=batch)
     o = Oracle(p.text, accum="f32")
     state = list(p.inputs)
+    losses = []
     n, t0 = 0, time.perf_counter()
     while True:
         out = o.run(*state)
         for k, i in p.feedback.items():
             state[i] = out[k]
+        losses.append(float(out[-1]))
         n += 1
         dt = time.perf_counter() - t0
         if dt >= budget_s or n >= 50:
             break
-    return {"value": round(n / dt, 5), "unit": "steps/s", "cores": os.cpu_count(), "kind": "port",
+    return {"value": round(n / dt, 5), "unit": "steps/s", "cores": os.cpu_count(), "kind": "port", "losses": losses,
             "sample": f"{n} ResNet18 train step(s) at batch {batch} in {dt:.1f} s (numpy/BLAS float32 interpreter of the same module)"}
 
 
@@ -190,18 +194,25 @@ def main():
         return
     p = configs.build_resnet18()
     cp = runner.CompiledProgram(p, client)
+    first_losses = []                                  # loss buffers of the first steps, read back after the timed region
     for _ in range(args.warmup):
         outs = cp.step()
-    outs[-1].block_until_ready()
+        if len(first_losses) < LOSS_CHECK_STEPS:
+            first_losses.append(outs[-1])
+    if args.warmup:
+        outs[-1].block_until_ready()
     before = cp.exe.cost_analysis()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         outs = cp.step()
+        if len(first_losses) < LOSS_CHECK_STEPS:
+            first_losses.append(outs[-1])
     outs[-1].block_until_ready()
     dt = time.perf_counter() - t0
     after = cp.exe.cost_analysis()
     loss = float(runner.download(outs[-1]))
     assert np.isfinite(loss), loss
+    first_losses = [float(runner.download(b)) for b in first_losses]
     conv_ms = after.get("conv.time_ms", 0.0) - before.get("conv.time_ms", 0.0)
     conv_n = after.get("conv.count", 0.0) - before.get("conv.count", 0.0)
     conv_flops = p.meta["step_flops"] - 6 * 128 * 512 * 10      # dense head is a GEMM step, not a convolution
@@ -239,10 +250,21 @@ def main():
         os.environ["MI355X_TIMING_REPEAT"] = str(FUSED_REPEAT)
         os.environ["MI355X_TIMING_ROTATE_BYTES"] = str(int(FUSED_ROTATE_BYTES))
         line["fused_ops"] = bench_fused_ops(client)
+    ok = True
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
         line["speedup_vs_cpu_baseline"] = round(line["value"] / line["cpu_baseline"]["value"], 1)
+        # the same steps from the same initial state on both sides: the losses must agree to float32 accumulation noise
+        want = line["cpu_baseline"].pop("losses")[:len(first_losses)]
+        got = first_losses[:len(want)]
+        rel = max(abs(g - w) / max(abs(w), 1e-30) for g, w in zip(got, want))
+        ok = rel <= LOSS_CHECK_RTOL
+        line["loss_check"] = {"steps": len(want), "gpu": [round(g, 6) for g in got], "cpu": [round(w, 6) for w in want],
+                              "max_rel_diff": float("%.3g" % rel), "rtol": LOSS_CHECK_RTOL, "ok": ok}
     print(json.dumps(line))
+    if not ok:
+        print("bench.py: the GPU losses of the first steps differ from the CPU baseline's beyond the stated tolerance", file=sys.stderr)
+        sys.exit(1)
 
 
 if __name__ == "__main__":

@@ -27,6 +27,7 @@
 #include <cstdint>
 #include <vector>
 #include <cstdlib>
+#include <type_traits>
 
 #include "hip_abi.h"
 
@@ -87,8 +88,11 @@ __device__ __forceinline__ int rhsTapOffset(const ConvP& p, int k0, int k1) {
   return a * p.rhsS0 + b * p.rhsS1;
 }
 
+// wavefronts per SIMD the register budget is held to: four workgroups per CU for the vector loaders of the narrower tiles
+constexpr int wavesPerSimd(int bm, int bn, int amode, int bmode) { return bm * bn == 128 * 128 ? 2 : (amode == 0 || bmode == 0 ? 3 : 4); }
+
 template <int BM, int BN, int AMODE, int BMODE, bool KFLAT>
-__global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
+__global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_igemm_f32(ConvP p) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int NA4 = BM / 64, NB4 = BN / 64;            // float4 per thread per tile (vector loaders)
   constexpr int NAS = BM * BK / 256, NBS = BN * BK / 256; // floats per thread per tile (scalar loaders)
@@ -122,9 +126,10 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
     for (int i = 0; i < NAS; ++i) rowsA[i] = makeRow(p, m0 + (tid + 256 * i) / BK);
   }
 
-  float4 ra[NA4 > 0 ? NA4 : 1];
-  float4 rb[NB4 > 0 ? NB4 : 1];
-  float ras[NAS], rbs[NBS];
+  // two register sets: the tile after next is already on its way while the next one is written to LDS
+  float4 ra[2][NA4 > 0 ? NA4 : 1];
+  float4 rb[2][NB4 > 0 ? NB4 : 1];
+  float ras[2][NAS], rbs[2][NBS];
 
   // Position of the next k-tile to fetch, advanced incrementally (no divisions in the loop):
   // window tap (nk0, nk1) and first input feature nc.  Row offsets and validity only change
@@ -153,17 +158,25 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
   const int bKr = tid / (BN / 4);
   const bool bNok = n0 + bNq < p.N;
 
-  auto loadTile = [&](int kt) {
+  // Loads are unconditional: an element outside the input, the filter or K is read from offset 0 of its tensor and
+  // replaced by zero when the tile is written to LDS (a load under a branch would make the compiler drain every
+  // outstanding load before issuing the next ones, which defeats fetching two tiles ahead).
+  unsigned okA[2] = {0, 0}, okB[2] = {0, 0};
+  auto loadTile = [&](int kt, auto setTag) {
+    constexpr int S = decltype(setTag)::value;
+    okA[S] = 0; okB[S] = 0;
     // ---------------- A
     if (AMODE == 1) {
 #pragma unroll
       for (int i = 0; i < NA4; ++i)
-        ra[i] = offA[i] >= 0 ? *(const float4*)(p.lhs + (unsigned)(offA[i] + nc + aKq)) : make_float4(0.f, 0.f, 0.f, 0.f);
+        { const bool ok = offA[i] >= 0; ra[S][i] = *(const float4*)(p.lhs + (unsigned)((ok ? offA[i] : 0) + nc + aKq)); okA[S] |= (unsigned)ok << i; }
     } else if (AMODE == 2) {
 #pragma unroll
       for (int i = 0; i < NA4; ++i) {
         int kr = aKr + (1024 / BM) * i;
-        ra[i] = offA[0] >= 0 ? *(const float4*)(p.lhs + (unsigned)(offA[0] + (nc + kr) * p.lhsF)) : make_float4(0.f, 0.f, 0.f, 0.f);
+        const bool ok = offA[0] >= 0;
+        ra[S][i] = *(const float4*)(p.lhs + (unsigned)((ok ? offA[0] : 0) + (nc + kr) * p.lhsF));
+        okA[S] |= (unsigned)ok << i;
       }
     } else {
 #pragma unroll
@@ -179,7 +192,8 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
         } else {
           off = offA[i];
         }
-        ras[i] = off >= 0 ? p.lhs[off + c * p.lhsF] : 0.f;
+        ras[S][i] = p.lhs[off >= 0 ? off + c * p.lhsF : 0];
+        okA[S] |= (unsigned)(off >= 0) << i;
       }
     }
     // ---------------- B
@@ -187,13 +201,15 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
 #pragma unroll
       for (int i = 0; i < NB4; ++i) {
         int kr = bKr + (1024 / BN) * i;
-        rb[i] = bNok ? *(const float4*)(p.rhs + (unsigned)(toffB + (nc + kr) * p.rhsI + n0 + bNq)) : make_float4(0.f, 0.f, 0.f, 0.f);
+        rb[S][i] = *(const float4*)(p.rhs + (unsigned)(toffB + (nc + kr) * p.rhsI + (bNok ? n0 + bNq : 0)));
+        okB[S] |= (unsigned)bNok << i;
       }
     } else if (BMODE == 2) {
 #pragma unroll
       for (int i = 0; i < NB4; ++i) {
         int n = n0 + (tid >> 2) + 64 * i;
-        rb[i] = n < p.N ? *(const float4*)(p.rhs + (unsigned)(toffB + n * p.rhsO + nc + aKq)) : make_float4(0.f, 0.f, 0.f, 0.f);
+        rb[S][i] = *(const float4*)(p.rhs + (unsigned)(toffB + (n < p.N ? n : 0) * p.rhsO + nc + aKq));
+        okB[S] |= (unsigned)(n < p.N) << i;
       }
     } else {
 #pragma unroll
@@ -210,7 +226,8 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
           int kk0 = t / p.k1n;
           toff = rhsTapOffset(p, kk0, t - kk0 * p.k1n);
         }
-        rbs[i] = ok ? p.rhs[toff + c * p.rhsI + n * p.rhsO] : 0.f;
+        rbs[S][i] = p.rhs[ok ? toff + c * p.rhsI + n * p.rhsO : 0];
+        okB[S] |= (unsigned)ok << i;
       }
     }
     // ---------------- advance to the following tile
@@ -224,40 +241,44 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
     }
   };
 
-  auto storeTile = [&](int st) {
+  auto storeTile = [&](auto stageTag, auto setTag) {
+    constexpr int st = decltype(stageTag)::value;   // compile-time stage: every LDS address is a per-thread base plus an immediate
+    constexpr int S = decltype(setTag)::value;
     if (AMODE == 1) {
       const int kq = (tid & 3) * 4;
 #pragma unroll
       for (int i = 0; i < NA4; ++i) {
         int m = (tid >> 2) + 64 * i;
-        As[st][kq + 0][m] = ra[i].x; As[st][kq + 1][m] = ra[i].y; As[st][kq + 2][m] = ra[i].z; As[st][kq + 3][m] = ra[i].w;
+        if (!((okA[S] >> i) & 1)) ra[S][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        As[st][kq + 0][m] = ra[S][i].x; As[st][kq + 1][m] = ra[S][i].y; As[st][kq + 2][m] = ra[S][i].z; As[st][kq + 3][m] = ra[S][i].w;
       }
     } else if (AMODE == 2) {
 #pragma unroll
       for (int i = 0; i < NA4; ++i) {
         int kr = tid / (BM / 4) + (1024 / BM) * i;
-        *(float4*)&As[st][kr][4 * (tid % (BM / 4))] = ra[i];
+        *(float4*)&As[st][kr][4 * (tid % (BM / 4))] = ((okA[S] >> i) & 1) ? ra[S][i] : make_float4(0.f, 0.f, 0.f, 0.f);
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < NAS; ++i) { int e = tid + 256 * i; As[st][e % BK][e / BK] = ras[i]; }
+      for (int i = 0; i < NAS; ++i) { int e = tid + 256 * i; As[st][e % BK][e / BK] = ((okA[S] >> i) & 1) ? ras[S][i] : 0.f; }
     }
     if (BMODE == 1) {
 #pragma unroll
       for (int i = 0; i < NB4; ++i) {
         int kr = tid / (BN / 4) + (1024 / BN) * i;
-        *(float4*)&Bs[st][kr][4 * (tid % (BN / 4))] = rb[i];
+        *(float4*)&Bs[st][kr][4 * (tid % (BN / 4))] = ((okB[S] >> i) & 1) ? rb[S][i] : make_float4(0.f, 0.f, 0.f, 0.f);
       }
     } else if (BMODE == 2) {
       const int kq = (tid & 3) * 4;
 #pragma unroll
       for (int i = 0; i < NB4; ++i) {
         int n = (tid >> 2) + 64 * i;
-        Bs[st][kq + 0][n] = rb[i].x; Bs[st][kq + 1][n] = rb[i].y; Bs[st][kq + 2][n] = rb[i].z; Bs[st][kq + 3][n] = rb[i].w;
+        if (!((okB[S] >> i) & 1)) rb[S][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        Bs[st][kq + 0][n] = rb[S][i].x; Bs[st][kq + 1][n] = rb[S][i].y; Bs[st][kq + 2][n] = rb[S][i].z; Bs[st][kq + 3][n] = rb[S][i].w;
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < NBS; ++i) { int e = tid + 256 * i; Bs[st][e / BN][e % BN] = rbs[i]; }
+      for (int i = 0; i < NBS; ++i) { int e = tid + 256 * i; Bs[st][e / BN][e % BN] = ((okB[S] >> i) & 1) ? rbs[S][i] : 0.f; }
     }
   };
 
@@ -268,14 +289,11 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
     for (int b = 0; b < TN; ++b) acc[a][b] = (float16v){0};
 
   if (ktBegin < ktEnd) {
-    loadTile(ktBegin);
-    storeTile(0);
-    __syncthreads();
-    int cur = 0;
+    std::integral_constant<int, 0> s0;
+    std::integral_constant<int, 1> s1;
     const int kh = lane >> 5, col = lane & 31;
-    for (int kt = ktBegin; kt < ktEnd; ++kt) {
-      const bool more = kt + 1 < ktEnd;
-      if (more) loadTile(kt + 1);          // global loads in flight while this tile is multiplied
+    auto multiply = [&](auto stageTag) {
+      constexpr int cur = decltype(stageTag)::value;
       __builtin_amdgcn_s_setprio(2);       // a wavefront that has its operands wins the matrix pipe over ones still fetching
 #pragma unroll
       for (int kk = 0; kk < BK; kk += 2) {
@@ -290,9 +308,36 @@ __global__ void __launch_bounds__(256, 2) conv_igemm_f32(ConvP p) {
           for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[b], av[a], acc[a][b], 0, 0, 0);   // operands swapped: the transposed tile
       }
       __builtin_amdgcn_s_setprio(0);
-      if (more) storeTile(cur ^ 1);         // the other stage: nobody reads it during this iteration
+    };
+    // Tile kt is multiplied from LDS while tile kt + 1 waits in one register set and tile kt + 2 is being fetched
+    // into the other: a global load has two multiply phases to arrive before anyone waits for it.
+    loadTile(ktBegin, s0);
+    storeTile(s0, s0);
+    if (ktBegin + 1 < ktEnd) loadTile(ktBegin + 1, s0);
+    __syncthreads();
+    int kt = ktBegin;
+    // Steady state: every fetch is unconditional, so that the wait before an LDS write covers only the older register
+    // set (a fetch under a condition would make the compiler wait for the newer loads as well).  Each half works on
+    // a fixed LDS stage: tile kt in stage 0, tile kt + 1 in stage 1.
+    for (; kt + 3 < ktEnd; kt += 2) {
+      loadTile(kt + 2, s1);
+      multiply(s0);
+      storeTile(s1, s0);                    // the other stage: nobody reads it during this half
       __syncthreads();
-      cur ^= 1;
+      loadTile(kt + 3, s0);
+      multiply(s1);
+      storeTile(s0, s1);
+      __syncthreads();
+    }
+    for (; kt < ktEnd; kt += 2) {           // the last one to three tiles
+      if (kt + 2 < ktEnd) loadTile(kt + 2, s1);
+      multiply(s0);
+      if (kt + 1 < ktEnd) storeTile(s1, s0);
+      __syncthreads();
+      if (kt + 1 >= ktEnd) break;
+      multiply(s1);
+      if (kt + 2 < ktEnd) storeTile(s0, s1);
+      __syncthreads();
     }
   }
 
