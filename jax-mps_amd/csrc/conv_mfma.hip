@@ -53,6 +53,8 @@ struct ConvP {
   int cTiles;           // k-tiles per window tap (tap-chunk tiling)
   int kTiles;           // total k-tiles
   int splitK, tilesPerSplit;
+  unsigned lhsBytes, rhsBytes;   // sizes for the buffer descriptors of the vector-loader kernel (both below 2 GiB)
+  int taps;                      // window taps this launch visits (kc0 * kc1)
 };
 
 struct Row {
@@ -86,6 +88,48 @@ __device__ __forceinline__ int tapOffset(const ConvP& p, const Row& r, int k0, i
 __device__ __forceinline__ int rhsTapOffset(const ConvP& p, int k0, int k1) {
   int a = p.rev0 ? p.k0n - 1 - k0 : k0, b = p.rev1 ? p.k1n - 1 - k1 : k1;
   return a * p.rhsS0 + b * p.rhsS1;
+}
+
+// Writes a workgroup's accumulators.  The products were issued with their operands swapped, so a lane holds the
+// transposed tile: one output row (lane & 31) and, per group of four accumulator registers, four consecutive output
+// columns.  A lane decodes one row per 32-row block instead of sixteen, and stores 16 bytes at a time where the
+// layout allows.
+template <int TM, int TN, int WM, int WN>
+__device__ __forceinline__ void storeAccumulators(const ConvP& p, float16v (&acc)[TM][TN], int m0, int n0, int wm, int wn, int lane) {
+  const bool partial = p.splitK > 1;
+  const bool vec = p.outVec != 0;
+#pragma unroll
+  for (int a = 0; a < TM; ++a) {
+    const int m = m0 + wm * WM + a * 32 + (lane & 31);
+    if (m >= p.M) continue;
+    long long rowOff;
+    if (partial) {
+      rowOff = ((long long)blockIdx.z * p.M + m) * p.N;
+    } else if (p.outRow > 0) {
+      rowOff = (long long)m * p.outRow;
+    } else {
+      int b, o0, o1;
+      if (p.bFast) { b = m % p.Nb; int t = m / p.Nb; o1 = t % p.o1n; o0 = t / p.o1n; }
+      else { o1 = m % p.o1n; int t = m / p.o1n; o0 = t % p.o0n; b = t / p.o0n; }
+      rowOff = (long long)b * p.outB + (long long)o0 * p.outS0 + (long long)o1 * p.outS1;
+    }
+    const long long colStride = partial ? 1 : p.outF;
+#pragma unroll
+    for (int b = 0; b < TN; ++b) {
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int n = n0 + wn * WN + b * 32 + g4 * 8 + (lane >> 5) * 4;
+        if (n >= p.N) continue;
+        if (vec) {
+          *(float4*)(p.out + rowOff + n) = make_float4(acc[a][b][4 * g4], acc[a][b][4 * g4 + 1], acc[a][b][4 * g4 + 2], acc[a][b][4 * g4 + 3]);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < p.N) p.out[rowOff + (n + r) * colStride] = acc[a][b][4 * g4 + r];
+        }
+      }
+    }
+  }
 }
 
 // wavefronts per SIMD the register budget is held to: four workgroups per CU for the vector loaders of the narrower tiles
@@ -341,44 +385,206 @@ __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_
     }
   }
 
-  // ---- epilogue
-  // The products were issued with their operands swapped, so a lane holds the transposed tile: one output row
-  // (lane & 31) and, per group of four accumulator registers, four consecutive output columns.  A lane decodes one
-  // row per 32-row block instead of sixteen, and stores 16 bytes at a time where the layout allows.
-  const bool partial = p.splitK > 1;
-  const bool vec = p.outVec != 0;
+  storeAccumulators<TM, TN, WM, WN>(p, acc, m0, n0, wm, wn, lane);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The kernel for the vector loaders (every large convolution of a training step).  An fp32 MFMA occupies the SIMD
+// for 64 cycles and every other vector instruction costs about four of them, so the k-loop is stripped of vector
+// arithmetic: tiles are fetched with buffer loads whose per-lane offset changes only when the window tap changes
+// (the advance along the features is a scalar offset), an element outside the input, the filter or N is given an
+// offset beyond the buffer and comes back as zero from the hardware range check (no selects, no masks), per-tap row
+// offsets come from a table in LDS filled once per workgroup when the window is small enough, and both LDS stages
+// are compile-time so every LDS address is a per-lane base plus an immediate.
+typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+constexpr unsigned kOutside = 0x80000000u;     // an offset no tensor reaches (tensors stay below 2 GiB here)
+constexpr int kTapTableBytes = 16384;          // largest per-workgroup tap table
+
+template <int BM, int BN, int AMODE, int BMODE, bool TABLE>
+__global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_igemm_lean(ConvP p) {
+  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+  constexpr int NA4 = BM / 64, NB4 = BN / 64;
+  constexpr int PA = AMODE == 1 ? 2 : 4, PB = BMODE == 2 ? 2 : 4;
+  constexpr int LDA = BM + PA, LDB = BN + PB;
+  __shared__ __attribute__((aligned(16))) float As[2 * BK * LDA];
+  __shared__ __attribute__((aligned(16))) float Bs[2 * BK * LDB];
+  extern __shared__ unsigned tapTab[];        // [tap][row of the tile]: byte offset of (row, tap, feature 0) or kOutside
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  int bx = blockIdx.x;
+  if ((gridDim.x & 7) == 0) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);
+  const int m0 = bx * BM, n0 = blockIdx.y * BN;
+  const int ktBegin = blockIdx.z * p.tilesPerSplit;
+  const int ktEnd = min(p.kTiles, ktBegin + p.tilesPerSplit);
+
+  const __amdgpu_buffer_rsrc_t rsA = __builtin_amdgcn_make_buffer_rsrc((void*)p.lhs, 0, (int)p.lhsBytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsB = __builtin_amdgcn_make_buffer_rsrc((void*)p.rhs, 0, (int)p.rhsBytes, 0x00020000);
+
+  // rows of the A tile this lane fetches: NA4 rows 64 apart (K-vector), or one group of four consecutive rows (M-vector)
+  constexpr int NROW = AMODE == 1 ? NA4 : 1;
+  int rowInTile[NROW];
 #pragma unroll
-  for (int a = 0; a < TM; ++a) {
-    const int m = m0 + wm * WM + a * 32 + (lane & 31);
-    if (m >= p.M) continue;
-    long long rowOff;
-    if (partial) {
-      rowOff = ((long long)blockIdx.z * p.M + m) * p.N;
-    } else if (p.outRow > 0) {
-      rowOff = (long long)m * p.outRow;
-    } else {
-      int b, o0, o1;
-      if (p.bFast) { b = m % p.Nb; int t = m / p.Nb; o1 = t % p.o1n; o0 = t / p.o1n; }
-      else { o1 = m % p.o1n; int t = m / p.o1n; o0 = t % p.o0n; b = t / p.o0n; }
-      rowOff = (long long)b * p.outB + (long long)o0 * p.outS0 + (long long)o1 * p.outS1;
+  for (int i = 0; i < NROW; ++i) rowInTile[i] = AMODE == 1 ? (tid >> 2) + 64 * i : 4 * (tid % (BM / 4));
+  Row rowsA[TABLE ? 1 : NROW];
+  if (!TABLE) {
+#pragma unroll
+    for (int i = 0; i < NROW; ++i) rowsA[i] = makeRow(p, m0 + rowInTile[i]);
+  } else {
+    const Row r = makeRow(p, m0 + tid % BM);
+    for (int t = tid / BM; t < p.taps; t += 256 / BM) {
+      const int t0 = t / p.kc1, t1 = t - t0 * p.kc1;
+      const int off = tapOffset(p, r, p.kb0 + p.ks0 * t0, p.kb1 + p.ks1 * t1);
+      tapTab[t * BM + tid % BM] = off >= 0 ? (unsigned)off * 4u : kOutside;
     }
-    const long long colStride = partial ? 1 : p.outF;
+    __syncthreads();
+  }
+
+  // position of the next k-tile to fetch: window tap (nk0, nk1) and first feature nc, all uniform
+  // (integer division runs on the vector unit; the results are the same in every lane and are moved to scalar registers)
+  int tap = __builtin_amdgcn_readfirstlane(ktBegin / p.cTiles);
+  int nc = (ktBegin - tap * p.cTiles) * BK;
+  int nk0 = __builtin_amdgcn_readfirstlane(tap / p.kc1), nk1 = tap - nk0 * p.kc1;
+  const int aKq = (tid & 3) * 4;
+  unsigned aFix[NA4];          // the part of a lane's A offset that never changes
 #pragma unroll
-    for (int b = 0; b < TN; ++b) {
+  for (int i = 0; i < NA4; ++i) aFix[i] = AMODE == 1 ? (unsigned)aKq * 4u : (unsigned)((tid / (BM / 4) + (1024 / BM) * i) * p.lhsF) * 4u;
+  unsigned aV[NA4], bV[NB4];
 #pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const int n = n0 + wn * WN + b * 32 + g4 * 8 + (lane >> 5) * 4;
-        if (n >= p.N) continue;
-        if (vec) {
-          *(float4*)(p.out + rowOff + n) = make_float4(acc[a][b][4 * g4], acc[a][b][4 * g4 + 1], acc[a][b][4 * g4 + 2], acc[a][b][4 * g4 + 3]);
-        } else {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (n + r < p.N) p.out[rowOff + (n + r) * colStride] = acc[a][b][4 * g4 + r];
-        }
-      }
+  for (int i = 0; i < NB4; ++i) {
+    if (BMODE == 1) {
+      const int nq = 4 * (tid % (BN / 4)), kr = tid / (BN / 4) + (1024 / BN) * i;
+      bV[i] = n0 + nq < p.N ? (unsigned)(kr * p.rhsI + n0 + nq) * 4u : kOutside;
+    } else {
+      const int n = n0 + (tid >> 2) + 64 * i;
+      bV[i] = n < p.N ? (unsigned)(n * p.rhsO + aKq) * 4u : kOutside;
     }
   }
+  int toffB = 0;
+  auto newTap = [&]() {
+    const int k0 = p.kb0 + p.ks0 * nk0, k1 = p.kb1 + p.ks1 * nk1;
+#pragma unroll
+    for (int i = 0; i < NROW; ++i) {
+      unsigned o;
+      if (TABLE) {
+        o = tapTab[tap * BM + rowInTile[i]];
+      } else {
+        const int off = tapOffset(p, rowsA[i], k0, k1);
+        o = off >= 0 ? (unsigned)off * 4u : kOutside;
+      }
+      if (AMODE == 1) {
+        aV[i] = o + aFix[i];
+      } else {
+#pragma unroll
+        for (int j = 0; j < NA4; ++j) aV[j] = o + aFix[j];
+      }
+    }
+    toffB = __builtin_amdgcn_readfirstlane(rhsTapOffset(p, k0, k1));
+  };
+  newTap();
+
+  float4 ra[2][NA4], rb[2][NB4];   // two register sets: the tile after next is on its way while the next one goes to LDS
+  auto loadTile = [&](auto setTag) {
+    constexpr int S = decltype(setTag)::value;
+    const unsigned sA = (unsigned)(AMODE == 1 ? nc : nc * p.lhsF) * 4u;
+    const unsigned sB = (unsigned)(BMODE == 1 ? toffB + nc * p.rhsI : toffB + nc) * 4u;
+#pragma unroll
+    for (int i = 0; i < NA4; ++i) ra[S][i] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsA, (int)aV[i], (int)sA, 0));
+#pragma unroll
+    for (int i = 0; i < NB4; ++i) rb[S][i] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rsB, (int)bV[i], (int)sB, 0));
+    nc += BK;
+    if (nc >= p.C) {
+      nc = 0;
+      ++tap;
+      if (++nk1 == p.kc1) { nk1 = 0; ++nk0; }
+      if (tap < p.taps) newTap();
+    }
+  };
+
+  // LDS write positions (per lane, stage 0)
+  float* const aWr = AMODE == 1 ? As + aKq * LDA + (tid >> 2) : As + (tid / (BM / 4)) * LDA + 4 * (tid % (BM / 4));
+  float* const bWr = BMODE == 1 ? Bs + (tid / (BN / 4)) * LDB + 4 * (tid % (BN / 4)) : Bs + aKq * LDB + (tid >> 2);
+  auto storeTile = [&](auto stageTag, auto setTag) {
+    constexpr int ST = decltype(stageTag)::value, S = decltype(setTag)::value;
+#pragma unroll
+    for (int i = 0; i < NA4; ++i) {
+      if (AMODE == 1) {
+        float* d = aWr + ST * BK * LDA + 64 * i;
+        d[0] = ra[S][i].x; d[LDA] = ra[S][i].y; d[2 * LDA] = ra[S][i].z; d[3 * LDA] = ra[S][i].w;
+      } else {
+        *(float4*)(aWr + ST * BK * LDA + (1024 / BM) * i * LDA) = ra[S][i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NB4; ++i) {
+      if (BMODE == 1) {
+        *(float4*)(bWr + ST * BK * LDB + (1024 / BN) * i * LDB) = rb[S][i];
+      } else {
+        float* d = bWr + ST * BK * LDB + 64 * i;
+        d[0] = rb[S][i].x; d[LDB] = rb[S][i].y; d[2 * LDB] = rb[S][i].z; d[3 * LDB] = rb[S][i].w;
+      }
+    }
+  };
+
+  float16v acc[TM][TN];
+#pragma unroll
+  for (int a = 0; a < TM; ++a)
+#pragma unroll
+    for (int b = 0; b < TN; ++b) acc[a][b] = (float16v){0};
+
+  if (ktBegin < ktEnd) {
+    std::integral_constant<int, 0> s0;
+    std::integral_constant<int, 1> s1;
+    const float* const aRd = As + (lane >> 5) * LDA + wm * WM + (lane & 31);
+    const float* const bRd = Bs + (lane >> 5) * LDB + wn * WN + (lane & 31);
+    auto multiply = [&](auto stageTag) {
+      constexpr int ST = decltype(stageTag)::value;
+      __builtin_amdgcn_s_setprio(2);       // a wavefront that has its operands wins the matrix pipe over ones still fetching
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += 2) {
+        float av[TM], bv[TN];
+#pragma unroll
+        for (int a = 0; a < TM; ++a) av[a] = aRd[(ST * BK + kk) * LDA + a * 32];
+#pragma unroll
+        for (int b = 0; b < TN; ++b) bv[b] = bRd[(ST * BK + kk) * LDB + b * 32];
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+          for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[b], av[a], acc[a][b], 0, 0, 0);   // operands swapped: the transposed tile
+      }
+      __builtin_amdgcn_s_setprio(0);
+    };
+    // Tile kt is multiplied from LDS stage 0 while tile kt + 1 waits in one register set and tile kt + 2 is being
+    // fetched into the other: a load has two multiply phases to arrive before anyone waits for it.  Fetches in the
+    // steady state are unconditional, so the wait before an LDS write covers only the older register set.
+    loadTile(s0);
+    storeTile(s0, s0);
+    if (ktBegin + 1 < ktEnd) loadTile(s0);
+    __syncthreads();
+    int kt = ktBegin;
+    for (; kt + 3 < ktEnd; kt += 2) {
+      loadTile(s1);
+      multiply(s0);
+      storeTile(s1, s0);                    // the other stage: nobody reads it during this half
+      __syncthreads();
+      loadTile(s0);
+      multiply(s1);
+      storeTile(s0, s1);
+      __syncthreads();
+    }
+    for (; kt < ktEnd; kt += 2) {           // the last one to three tiles
+      if (kt + 2 < ktEnd) loadTile(s1);
+      multiply(s0);
+      if (kt + 1 < ktEnd) storeTile(s1, s0);
+      __syncthreads();
+      if (kt + 1 >= ktEnd) break;
+      multiply(s1);
+      if (kt + 2 < ktEnd) storeTile(s0, s1);
+      __syncthreads();
+    }
+  }
+
+  storeAccumulators<TM, TN, WM, WN>(p, acc, m0, n0, wm, wn, lane);
 }
 
 // out(m, n) = sum over splits of partial[s][m][n].  32 consecutive outputs per workgroup, the
@@ -458,7 +664,7 @@ struct ConvChoice {
 bool fitsInt(const mi355_conv_desc* d) {
   long long lhs = d->N * d->batchGroups * d->C, rhs = d->C * d->O, out = d->N * d->O;
   for (int k = 0; k < d->nsp; ++k) { lhs *= d->in[k]; rhs *= d->k[k]; out *= d->out[k]; }
-  return lhs < (1ll << 31) && rhs < (1ll << 31) && out < (1ll << 31);
+  return lhs < (1ll << 29) && rhs < (1ll << 29) && out < (1ll << 31);   // inputs below 2 GiB: buffer descriptors and byte offsets are 32-bit
 }
 
 ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
@@ -511,18 +717,22 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
 template <int BM, int BN>
 void launchIgemm(const ConvChoice& c, const ConvP& p, dim3 grid, hipStream_t st) {
 #define CASE(A, B, F) conv_igemm_f32<BM, BN, A, B, F><<<grid, 256, 0, st>>>(p)
+#define LEAN(A, B) do { if (table) conv_igemm_lean<BM, BN, A, B, true><<<grid, 256, table, st>>>(p); else conv_igemm_lean<BM, BN, A, B, false><<<grid, 256, 0, st>>>(p); } while (0)
   if (c.kflat) { CASE(0, 0, true); return; }
+  const size_t tableBytes = (size_t)p.taps * BM * sizeof(unsigned);
+  const unsigned table = tableBytes <= (size_t)kTapTableBytes ? (unsigned)tableBytes : 0u;
   switch (c.amode * 3 + c.bmode) {
     case 0: CASE(0, 0, false); break;
     case 1: CASE(0, 1, false); break;
     case 2: CASE(0, 2, false); break;
     case 3: CASE(1, 0, false); break;
-    case 4: CASE(1, 1, false); break;
-    case 5: CASE(1, 2, false); break;
+    case 4: LEAN(1, 1); break;
+    case 5: LEAN(1, 2); break;
     case 6: CASE(2, 0, false); break;
-    case 7: CASE(2, 1, false); break;
-    case 8: CASE(2, 2, false); break;
+    case 7: LEAN(2, 1); break;
+    case 8: LEAN(2, 2); break;
   }
+#undef LEAN
 #undef CASE
 }
 
@@ -654,6 +864,12 @@ static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, vo
     p.outRow = linear ? unit : 0;
   }
   p.cTiles = c.cTiles; p.kTiles = c.kTiles; p.splitK = c.splitK; p.tilesPerSplit = c.tilesPerSplit;
+  p.taps = part.kc[0] * part.kc[1];
+  {
+    long long lhsN = d->N * d->batchGroups * d->C, rhsN = d->C * d->O;
+    for (int k = 0; k < d->nsp; ++k) { lhsN *= d->in[k]; rhsN *= d->k[k]; }
+    p.lhsBytes = (unsigned)(lhsN * 4); p.rhsBytes = (unsigned)(rhsN * 4);   // below 2 GiB each (fitsInt)
+  }
   float* dst = (float*)out + part.outOffset;
   if (c.splitK > 1) {
     size_t need = (size_t)c.splitK * (size_t)M * (size_t)d->O * sizeof(float);
