@@ -404,9 +404,16 @@ template <int BM, int BN, int AMODE, int BMODE, bool TABLE>
 __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_igemm_lean(ConvP p) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int NA4 = BM / 64, NB4 = BN / 64;
-  constexpr int PA = AMODE == 1 ? 2 : 4, PB = BMODE == 2 ? 2 : 4;
+  // The K-vector loader keeps its A tile row-major ([row][k], rows 20 floats apart): a fetched vector is one 16-byte
+  // LDS write, and a lane reads its operands for four MFMA steps with one 16-byte read.  The order of k inside a tile
+  // is free as long as both operands agree, so lane half h takes k = 8q + 4h + j for step (q, j).  The other tiles
+  // are k-major ([k][row or column]).
+  constexpr bool AROW = AMODE == 1;
+  constexpr int RS = BK + 4;
+  constexpr int PA = 4, PB = BMODE == 2 ? 2 : 4;
   constexpr int LDA = BM + PA, LDB = BN + PB;
-  __shared__ __attribute__((aligned(16))) float As[2 * BK * LDA];
+  constexpr int ASTAGE = AROW ? BM * RS : BK * LDA;
+  __shared__ __attribute__((aligned(16))) float As[2 * ASTAGE];
   __shared__ __attribute__((aligned(16))) float Bs[2 * BK * LDB];
   extern __shared__ unsigned tapTab[];        // [tap][row of the tile]: byte offset of (row, tap, feature 0) or kOutside
 
@@ -502,18 +509,14 @@ __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_
   };
 
   // LDS write positions (per lane, stage 0)
-  float* const aWr = AMODE == 1 ? As + aKq * LDA + (tid >> 2) : As + (tid / (BM / 4)) * LDA + 4 * (tid % (BM / 4));
+  float* const aWr = AROW ? As + (tid >> 2) * RS + aKq : As + (tid / (BM / 4)) * LDA + 4 * (tid % (BM / 4));
   float* const bWr = BMODE == 1 ? Bs + (tid / (BN / 4)) * LDB + 4 * (tid % (BN / 4)) : Bs + aKq * LDB + (tid >> 2);
   auto storeTile = [&](auto stageTag, auto setTag) {
     constexpr int ST = decltype(stageTag)::value, S = decltype(setTag)::value;
 #pragma unroll
     for (int i = 0; i < NA4; ++i) {
-      if (AMODE == 1) {
-        float* d = aWr + ST * BK * LDA + 64 * i;
-        d[0] = ra[S][i].x; d[LDA] = ra[S][i].y; d[2 * LDA] = ra[S][i].z; d[3 * LDA] = ra[S][i].w;
-      } else {
-        *(float4*)(aWr + ST * BK * LDA + (1024 / BM) * i * LDA) = ra[S][i];
-      }
+      if (AROW) *(float4*)(aWr + ST * ASTAGE + 64 * i * RS) = ra[S][i];
+      else *(float4*)(aWr + ST * ASTAGE + (1024 / BM) * i * LDA) = ra[S][i];
     }
 #pragma unroll
     for (int i = 0; i < NB4; ++i) {
@@ -535,22 +538,42 @@ __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_
   if (ktBegin < ktEnd) {
     std::integral_constant<int, 0> s0;
     std::integral_constant<int, 1> s1;
-    const float* const aRd = As + (lane >> 5) * LDA + wm * WM + (lane & 31);
-    const float* const bRd = Bs + (lane >> 5) * LDB + wn * WN + (lane & 31);
+    const int kh = lane >> 5, col = lane & 31;
+    const float* const aRd = AROW ? As + (wm * WM + col) * RS + 4 * kh : As + kh * LDA + wm * WM + col;
+    const float* const bRd = Bs + (AROW ? 4 * kh : kh) * LDB + wn * WN + col;
     auto multiply = [&](auto stageTag) {
       constexpr int ST = decltype(stageTag)::value;
       __builtin_amdgcn_s_setprio(2);       // a wavefront that has its operands wins the matrix pipe over ones still fetching
+      if (AROW) {
 #pragma unroll
-      for (int kk = 0; kk < BK; kk += 2) {
-        float av[TM], bv[TN];
+        for (int q = 0; q < BK / 8; ++q) {
+          float4 av[TM];
 #pragma unroll
-        for (int a = 0; a < TM; ++a) av[a] = aRd[(ST * BK + kk) * LDA + a * 32];
+          for (int a = 0; a < TM; ++a) av[a] = *(const float4*)(aRd + ST * ASTAGE + a * 32 * RS + 8 * q);
 #pragma unroll
-        for (int b = 0; b < TN; ++b) bv[b] = bRd[(ST * BK + kk) * LDB + b * 32];
+          for (int j = 0; j < 4; ++j) {
+            float bv[TN];
 #pragma unroll
-        for (int a = 0; a < TM; ++a)
+            for (int b = 0; b < TN; ++b) bv[b] = bRd[(ST * BK + 8 * q + j) * LDB + b * 32];
 #pragma unroll
-          for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[b], av[a], acc[a][b], 0, 0, 0);   // operands swapped: the transposed tile
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+              for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[b], av[a][j], acc[a][b], 0, 0, 0);   // operands swapped: the transposed tile
+          }
+        }
+      } else {
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+          float av[TM], bv[TN];
+#pragma unroll
+          for (int a = 0; a < TM; ++a) av[a] = aRd[ST * ASTAGE + kk * LDA + a * 32];
+#pragma unroll
+          for (int b = 0; b < TN; ++b) bv[b] = bRd[(ST * BK + kk) * LDB + b * 32];
+#pragma unroll
+          for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[b], av[a], acc[a][b], 0, 0, 0);
+        }
       }
       __builtin_amdgcn_s_setprio(0);
     };
@@ -691,7 +714,10 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
   // largest tile that still leaves minTiles output tiles (split-K then multiplies the workgroups); tuned on the ResNet18 step
   auto tilesOf = [&](int bm, int bn) { return ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   static const int forced = getenv("MI355X_CONV_TILE") ? atoi(getenv("MI355X_CONV_TILE")) : 0;
-  static const int minTiles = getenv("MI355X_CONV_MIN_TILES") ? atoi(getenv("MI355X_CONV_MIN_TILES")) : 128;
+  // (measured on the ResNet18 step: forward and data-gradient shapes prefer 64x64 tiles with little or no split of K over
+  // wider tiles split further, whose partial sums cost a fold pass; the filter gradients, with their long K, prefer wide tiles)
+  static const int minTilesEnv = getenv("MI355X_CONV_MIN_TILES") ? atoi(getenv("MI355X_CONV_MIN_TILES")) : 0;
+  const int minTiles = minTilesEnv ? minTilesEnv : (c.amode == 2 ? 128 : 1024);
   if (forced == 128 || (!forced && N >= 128 && tilesOf(128, 128) >= minTiles)) { c.bm = 128; c.bn = 128; }
   else if (forced == 12864 || (!forced && tilesOf(128, 64) >= minTiles)) { c.bm = 128; c.bn = 64; }
   else { c.bm = 64; c.bn = 64; }
