@@ -404,17 +404,16 @@ template <int BM, int BN, int AMODE, int BMODE, bool TABLE>
 __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_igemm_lean(ConvP p) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int NA4 = BM / 64, NB4 = BN / 64;
-  // The K-vector loader keeps its A tile row-major ([row][k], rows 20 floats apart): a fetched vector is one 16-byte
-  // LDS write, and a lane reads its operands for four MFMA steps with one 16-byte read.  The order of k inside a tile
-  // is free as long as both operands agree, so lane half h takes k = 8q + 4h + j for step (q, j).  The other tiles
-  // are k-major ([k][row or column]).
-  constexpr bool AROW = AMODE == 1;
+  // A tile fetched with K-vectors stays row-major in LDS ([row or column][k], rows 20 floats apart): a fetched vector
+  // is one 16-byte LDS write, and a lane reads its operands for four MFMA steps with one 16-byte read.  The order of k
+  // inside a tile is free as long as both operands agree, so lane half h takes k = 8q + 4h + j for step (q, j).  Tiles
+  // fetched with M- or N-vectors are k-major ([k][row or column]) and follow the same order of k.
+  constexpr bool AROW = AMODE == 1, BROW = BMODE == 2, PERM = AROW || BROW;
   constexpr int RS = BK + 4;
-  constexpr int PA = 4, PB = BMODE == 2 ? 2 : 4;
-  constexpr int LDA = BM + PA, LDB = BN + PB;
-  constexpr int ASTAGE = AROW ? BM * RS : BK * LDA;
+  constexpr int LDA = BM + 4, LDB = BN + 4;
+  constexpr int ASTAGE = AROW ? BM * RS : BK * LDA, BSTAGE = BROW ? BN * RS : BK * LDB;
   __shared__ __attribute__((aligned(16))) float As[2 * ASTAGE];
-  __shared__ __attribute__((aligned(16))) float Bs[2 * BK * LDB];
+  __shared__ __attribute__((aligned(16))) float Bs[2 * BSTAGE];
   extern __shared__ unsigned tapTab[];        // [tap][row of the tile]: byte offset of (row, tap, feature 0) or kOutside
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -510,7 +509,7 @@ __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_
 
   // LDS write positions (per lane, stage 0)
   float* const aWr = AROW ? As + (tid >> 2) * RS + aKq : As + (tid / (BM / 4)) * LDA + 4 * (tid % (BM / 4));
-  float* const bWr = BMODE == 1 ? Bs + (tid / (BN / 4)) * LDB + 4 * (tid % (BN / 4)) : Bs + aKq * LDB + (tid >> 2);
+  float* const bWr = BROW ? Bs + (tid >> 2) * RS + aKq : Bs + (tid / (BN / 4)) * LDB + 4 * (tid % (BN / 4));
   auto storeTile = [&](auto stageTag, auto setTag) {
     constexpr int ST = decltype(stageTag)::value, S = decltype(setTag)::value;
 #pragma unroll
@@ -520,12 +519,8 @@ __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_
     }
 #pragma unroll
     for (int i = 0; i < NB4; ++i) {
-      if (BMODE == 1) {
-        *(float4*)(bWr + ST * BK * LDB + (1024 / BN) * i * LDB) = rb[S][i];
-      } else {
-        float* d = bWr + ST * BK * LDB + 64 * i;
-        d[0] = rb[S][i].x; d[LDB] = rb[S][i].y; d[2 * LDB] = rb[S][i].z; d[3 * LDB] = rb[S][i].w;
-      }
+      if (BROW) *(float4*)(bWr + ST * BSTAGE + 64 * i * RS) = rb[S][i];
+      else *(float4*)(bWr + ST * BSTAGE + (1024 / BN) * i * LDB) = rb[S][i];
     }
   };
 
@@ -539,27 +534,41 @@ __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_
     std::integral_constant<int, 0> s0;
     std::integral_constant<int, 1> s1;
     const int kh = lane >> 5, col = lane & 31;
-    const float* const aRd = AROW ? As + (wm * WM + col) * RS + 4 * kh : As + kh * LDA + wm * WM + col;
-    const float* const bRd = Bs + (AROW ? 4 * kh : kh) * LDB + wn * WN + col;
+    const float* const aRd = AROW ? As + (wm * WM + col) * RS + 4 * kh : As + (PERM ? 4 * kh : kh) * LDA + wm * WM + col;
+    const float* const bRd = BROW ? Bs + (wn * WN + col) * RS + 4 * kh : Bs + (PERM ? 4 * kh : kh) * LDB + wn * WN + col;
     auto multiply = [&](auto stageTag) {
       constexpr int ST = decltype(stageTag)::value;
       __builtin_amdgcn_s_setprio(2);       // a wavefront that has its operands wins the matrix pipe over ones still fetching
-      if (AROW) {
+      if (PERM) {
 #pragma unroll
         for (int q = 0; q < BK / 8; ++q) {
-          float4 av[TM];
+          float av[TM][4], bv[TN][4];
 #pragma unroll
-          for (int a = 0; a < TM; ++a) av[a] = *(const float4*)(aRd + ST * ASTAGE + a * 32 * RS + 8 * q);
+          for (int a = 0; a < TM; ++a) {
+            if (AROW) {
+              const float4 v = *(const float4*)(aRd + ST * ASTAGE + a * 32 * RS + 8 * q);
+              av[a][0] = v.x; av[a][1] = v.y; av[a][2] = v.z; av[a][3] = v.w;
+            } else {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            float bv[TN];
+              for (int j = 0; j < 4; ++j) av[a][j] = aRd[ST * ASTAGE + (8 * q + j) * LDA + a * 32];
+            }
+          }
 #pragma unroll
-            for (int b = 0; b < TN; ++b) bv[b] = bRd[(ST * BK + 8 * q + j) * LDB + b * 32];
+          for (int b = 0; b < TN; ++b) {
+            if (BROW) {
+              const float4 v = *(const float4*)(bRd + ST * BSTAGE + b * 32 * RS + 8 * q);
+              bv[b][0] = v.x; bv[b][1] = v.y; bv[b][2] = v.z; bv[b][3] = v.w;
+            } else {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) bv[b][j] = bRd[ST * BSTAGE + (8 * q + j) * LDB + b * 32];
+            }
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int a = 0; a < TM; ++a)
 #pragma unroll
-              for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[b], av[a][j], acc[a][b], 0, 0, 0);   // operands swapped: the transposed tile
-          }
+              for (int b = 0; b < TN; ++b) acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[b][j], av[a][j], acc[a][b], 0, 0, 0);   // operands swapped: the transposed tile
         }
       } else {
 #pragma unroll
@@ -568,7 +577,7 @@ __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_
 #pragma unroll
           for (int a = 0; a < TM; ++a) av[a] = aRd[ST * ASTAGE + kk * LDA + a * 32];
 #pragma unroll
-          for (int b = 0; b < TN; ++b) bv[b] = bRd[(ST * BK + kk) * LDB + b * 32];
+          for (int b = 0; b < TN; ++b) bv[b] = bRd[ST * BSTAGE + kk * LDB + b * 32];
 #pragma unroll
           for (int a = 0; a < TM; ++a)
 #pragma unroll
@@ -814,6 +823,9 @@ std::vector<ConvPart> partsOf(const mi355_conv_desc* d) {
 // the descriptor that addresses it, or 0.
 size_t repackedFilter(const mi355_conv_desc* d, mi355_conv_desc* out) {
   if (d->dtype != 0 || d->nsp > 2 || d->featureGroups != 1 || d->batchGroups != 1 || !fitsInt(d)) return 0;
+  // (measured: with the row-major B tile of the vector-loader kernel the rewritten copy no longer pays; kept as an option)
+  static const bool on = getenv("MI355X_CONV_REPACK") && getenv("MI355X_CONV_REPACK")[0] == '1';
+  if (!on) return 0;
   if (d->rhsI != 1 || d->rhsO == 1 || d->C % BK != 0 || d->O % 4 != 0) return 0;
   long long M = d->N, taps = 1;
   for (int k = 0; k < d->nsp; ++k) { M *= d->out[k]; taps *= d->k[k]; }
