@@ -792,7 +792,14 @@ class Converter {
       if (d.kind != BAttr::Dict) bad("an operation's attributes are not a dictionary");
       dict = &d;
     }
-    if (mask & 0x40) bad("operations with native properties are not supported (" + dialect + "." + on.name + ")");
+    if (mask & 0x40) {
+      // Native properties (container version 5 and later).  VHLO keeps every attribute in the dictionary, so in a
+      // portable artifact only builtin.module has any (its symbol name and visibility, which nothing here needs):
+      // the index into the properties section is read and dropped.
+      if (!(dialect == "builtin" && on.name == "module"))
+        bad("operations with native properties are not supported (" + dialect + "." + on.name + ")");
+      c.varint();
+    }
     std::vector<int> resultTypes;
     if (mask & 0x02) {
       uint64_t n = c.varint();

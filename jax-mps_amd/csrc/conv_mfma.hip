@@ -742,7 +742,8 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
   int split = 1;
   static const int minSplitTiles = getenv("MI355X_CONV_MIN_SPLIT_KTILES") ? atoi(getenv("MI355X_CONV_MIN_SPLIT_KTILES")) : 1;
   // (measured: splitting pays even for a short K, the shorter dependent chain per workgroup outweighs the fold launch)
-  if (tiles * 2 <= target && c.kTiles >= minSplitTiles) split = (int)std::min<long long>(target / tiles, std::max(1, c.kTiles / (tiles < 64 ? 4 : 8)));
+  static const int splitFactor = getenv("MI355X_CONV_SPLIT_FACTOR") ? atoi(getenv("MI355X_CONV_SPLIT_FACTOR")) : 3;
+  if (tiles * (c.amode == 2 ? 2 : splitFactor) <= target && c.kTiles >= minSplitTiles) split = (int)std::min<long long>(target / tiles, std::max(1, c.kTiles / (tiles < 64 ? 4 : 8)));
   split = std::max(1, std::min(split, 256));
   c.tilesPerSplit = (c.kTiles + split - 1) / split;
   c.splitK = (c.kTiles + c.tilesPerSplit - 1) / c.tilesPerSplit;

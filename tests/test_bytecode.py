@@ -64,7 +64,8 @@ def test_op_cases_survive_the_round_trip(name):
 
 
 @pytest.mark.parametrize("options", [dict(version=1), dict(version=2, isolated_funcs=True), dict(version=3), dict(version=4),
-                                     dict(version=5, isolated_funcs=True), dict(version=6, pack_bools=False), dict(version=6, isolated_funcs=True)],
+                                     dict(version=5, isolated_funcs=True), dict(version=6, pack_bools=False), dict(version=6, isolated_funcs=True),
+                                     dict(version=5, module_properties=True), dict(version=6, isolated_funcs=True, module_properties=True)],
                          ids=lambda o: "-".join(f"{k}={v}" for k, v in o.items()))
 def test_container_variants(options):
     p = configs.build_lstm(**configs.SMALL["lstm"])            # loops, nested regions, constants, dots

@@ -51,10 +51,11 @@ def with_flag(v: int, flag: bool) -> bytes:
 
 
 class Writer:
-    def __init__(self, text: str, version: int = 6, isolated_funcs: bool = False, pack_bools: bool = True):
+    def __init__(self, text: str, version: int = 6, isolated_funcs: bool = False, pack_bools: bool = True, module_properties: bool = False):
         self.funcs = parse(text)
         self.version = version
         self.isolated_funcs = isolated_funcs
+        self.module_properties = module_properties and version >= 5   # builtin.module carries native properties from version 5 on
         self.pack_bools = pack_bools
         self.strings: Dict[str, int] = {}
         self.attrs: Dict[tuple, int] = {}      # key -> provisional id, in first-use order
@@ -470,10 +471,16 @@ class Writer:
             module_region += with_flag(1, self.isolated_funcs)
             body = self.emit_region(f.body, plans, {}, 0, aidx, tidx, loc)
             module_region += self.section(4, body) if (self.isolated_funcs and self.version >= 2) else body
-        ir = with_flag(1, False) + varint(self.op_names[("builtin", "module")]) + bytes([16]) + varint(loc) + with_flag(1, True)
+        ir = with_flag(1, False) + varint(self.op_names[("builtin", "module")]) + bytes([16 | (0x40 if self.module_properties else 0)]) + varint(loc)
+        if self.module_properties:
+            ir += varint(0)                  # index into the properties section
+        ir += with_flag(1, True)
         ir += self.section(4, module_region) if self.version >= 2 else module_region
         out = b"ML\xefR" + varint(self.version) + b"StableHLO_v1.9.0\x00"
         out += self.section(0, string_sec) + self.section(1, dialect_sec) + self.section(2, attr_sec) + self.section(3, offset_sec) + self.section(4, ir)
+        if self.module_properties:
+            # one entry: the module's two optional inherent attributes (symbol name, visibility), both absent
+            out += self.section(8, varint(1) + varint(2) + b"\x00\x00")
         return out
 
 
