@@ -95,7 +95,7 @@ __device__ __forceinline__ int rhsTapOffset(const ConvP& p, int k0, int k1) {
 // columns.  A lane decodes one row per 32-row block instead of sixteen, and stores 16 bytes at a time where the
 // layout allows.
 template <int TM, int TN, int WM, int WN>
-__device__ __forceinline__ void storeAccumulators(const ConvP& p, float16v (&acc)[TM][TN], int m0, int n0, int wm, int wn, int lane) {
+__device__ __forceinline__ void storeAccumulators(const ConvP& p, float16v (&acc)[TM][TN], int m0, int n0, int wm, int wn, int lane, int split) {
   const bool partial = p.splitK > 1;
   const bool vec = p.outVec != 0;
 #pragma unroll
@@ -104,7 +104,7 @@ __device__ __forceinline__ void storeAccumulators(const ConvP& p, float16v (&acc
     if (m >= p.M) continue;
     long long rowOff;
     if (partial) {
-      rowOff = ((long long)blockIdx.z * p.M + m) * p.N;
+      rowOff = ((long long)split * p.M + m) * p.N;
     } else if (p.outRow > 0) {
       rowOff = (long long)m * p.outRow;
     } else {
@@ -385,7 +385,7 @@ __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_
     }
   }
 
-  storeAccumulators<TM, TN, WM, WN>(p, acc, m0, n0, wm, wn, lane);
+  storeAccumulators<TM, TN, WM, WN>(p, acc, m0, n0, wm, wn, lane, (int)blockIdx.z);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -401,7 +401,7 @@ constexpr unsigned kOutside = 0x80000000u;     // an offset no tensor reaches (t
 constexpr int kTapTableBytes = 16384;          // largest per-workgroup tap table
 
 template <int BM, int BN, int AMODE, int BMODE, bool TABLE>
-__global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_igemm_lean(ConvP p) {
+__device__ __forceinline__ void leanBody(const ConvP& p, const int split) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int NA4 = BM / 64, NB4 = BN / 64;
   // A tile fetched with K-vectors stays row-major in LDS ([row or column][k], rows 20 floats apart): a fetched vector
@@ -421,7 +421,8 @@ __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_
   int bx = blockIdx.x;
   if ((gridDim.x & 7) == 0) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);
   const int m0 = bx * BM, n0 = blockIdx.y * BN;
-  const int ktBegin = blockIdx.z * p.tilesPerSplit;
+  if (m0 >= p.M) return;                      // (a launch shared by several problems is as wide as the widest)
+  const int ktBegin = split * p.tilesPerSplit;
   const int ktEnd = min(p.kTiles, ktBegin + p.tilesPerSplit);
 
   const __amdgpu_buffer_rsrc_t rsA = __builtin_amdgcn_make_buffer_rsrc((void*)p.lhs, 0, (int)p.lhsBytes, 0x00020000);
@@ -616,7 +617,22 @@ __global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_
     }
   }
 
-  storeAccumulators<TM, TN, WM, WN>(p, acc, m0, n0, wm, wn, lane);
+  storeAccumulators<TM, TN, WM, WN>(p, acc, m0, n0, wm, wn, lane, split);
+}
+
+template <int BM, int BN, int AMODE, int BMODE, bool TABLE>
+__global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_igemm_lean(ConvP p) {
+  leanBody<BM, BN, AMODE, BMODE, TABLE>(p, (int)blockIdx.z);
+}
+
+// Several unsplit problems of one convolution (the residue classes of an input-dilated one) as one launch:
+// blockIdx.z picks the problem.  Each class alone is a short K loop over few workgroups; together they fill the device.
+constexpr int kMaxPack = 4;
+struct ConvPack { ConvP c[kMaxPack]; };
+
+template <int BM, int BN, int AMODE, int BMODE, bool TABLE>
+__global__ void __launch_bounds__(256, wavesPerSimd(BM, BN, AMODE, BMODE)) conv_igemm_lean_pack(ConvPack ps) {
+  leanBody<BM, BN, AMODE, BMODE, TABLE>(ps.c[blockIdx.z], 0);
 }
 
 // out(m, n) = sum over splits of partial[s][m][n].  32 consecutive outputs per workgroup, the
@@ -699,7 +715,7 @@ bool fitsInt(const mi355_conv_desc* d) {
   return lhs < (1ll << 29) && rhs < (1ll << 29) && out < (1ll << 31);   // inputs below 2 GiB: buffer descriptors and byte offsets are 32-bit
 }
 
-ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
+ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1, int sharedLaunch = 1) {
   ConvChoice c;
   if (d->dtype != 0 || d->nsp > 2 || d->featureGroups != 1 || d->batchGroups != 1 || !fitsInt(d)) return c;
   c.fast = true;
@@ -726,7 +742,8 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
   // (measured on the ResNet18 step: forward and data-gradient shapes prefer 64x64 tiles with little or no split of K over
   // wider tiles split further, whose partial sums cost a fold pass; the filter gradients, with their long K, prefer wide tiles)
   static const int minTilesEnv = getenv("MI355X_CONV_MIN_TILES") ? atoi(getenv("MI355X_CONV_MIN_TILES")) : 0;
-  const int minTiles = minTilesEnv ? minTilesEnv : (c.amode == 2 ? 128 : 1024);
+  static const int minTilesLongK = getenv("MI355X_CONV_MIN_TILES_LONGK") ? atoi(getenv("MI355X_CONV_MIN_TILES_LONGK")) : 128;
+  const int minTiles = minTilesEnv ? minTilesEnv : (c.amode == 2 ? minTilesLongK : 1024);
   if (forced == 128 || (!forced && N >= 128 && tilesOf(128, 128) >= minTiles)) { c.bm = 128; c.bn = 128; }
   else if (forced == 12864 || (!forced && tilesOf(128, 64) >= minTiles)) { c.bm = 128; c.bn = 64; }
   else { c.bm = 64; c.bn = 64; }
@@ -734,7 +751,7 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1) {
   // which halves the partial sums written and folded (measured: 0.7 % of a ResNet step; 64x64 tiles with no split lose).
   // The long-K filter gradients keep the wide tile: their output is small and their K loop is all that matters.
   if (!forced && c.bm == 128 && c.bn == 128 && tilesOf(128, 128) <= 256 && c.kTiles < 2048) c.bn = 64;
-  long long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+  long long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * sharedLaunch;   // problems launched together fill the device together
   // Split K until there are about `target` workgroups: four per CU, which is what stays resident, so that a
   // tile count that is not a multiple of the CU count costs little, without exceeding it (a fifth
   // workgroup per CU waits for a whole workgroup time: 1280 measured a tenth slower than 1024).
@@ -770,6 +787,23 @@ void launchIgemm(const ConvChoice& c, const ConvP& p, dim3 grid, hipStream_t st)
   }
 #undef LEAN
 #undef CASE
+}
+
+template <int BM, int BN>
+void launchPack(const ConvChoice& c, const ConvPack& ps, int count, hipStream_t st) {
+  int maxM = 0, maxTaps = 0;
+  for (int i = 0; i < count; ++i) { maxM = std::max(maxM, ps.c[i].M); maxTaps = std::max(maxTaps, ps.c[i].taps); }
+  dim3 grid((unsigned)((maxM + BM - 1) / BM), (unsigned)((ps.c[0].N + BN - 1) / BN), (unsigned)count);
+  const size_t tableBytes = (size_t)maxTaps * BM * sizeof(unsigned);
+  const unsigned table = tableBytes <= (size_t)kTapTableBytes ? (unsigned)tableBytes : 0u;
+#define PACK(A, B) do { if (table) conv_igemm_lean_pack<BM, BN, A, B, true><<<grid, 256, table, st>>>(ps); else conv_igemm_lean_pack<BM, BN, A, B, false><<<grid, 256, 0, st>>>(ps); } while (0)
+  switch (c.amode * 3 + c.bmode) {
+    case 4: PACK(1, 1); break;
+    case 5: PACK(1, 2); break;
+    case 7: PACK(2, 1); break;
+    case 8: PACK(2, 2); break;
+  }
+#undef PACK
 }
 
 // One launch of the implicit-GEMM kernel: the whole convolution, or one residue class of an
@@ -861,15 +895,17 @@ size_t mi355_conv_workspace_bytes(const mi355_conv_desc* d) {
 
 int mi355_conv_direct(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, mi355_stream_t s);
 
-static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes, hipStream_t st) {
+// Launches one part; with `prepared` set it only fills the kernel parameters of an unsplit part (returns -1 when the part cannot be prepared that way).
+static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes, hipStream_t st,
+                      int sharedLaunch = 1, ConvChoice* preparedChoice = nullptr, ConvP* prepared = nullptr) {
   const mi355_conv_desc* d = &part.d;
-  ConvChoice c = choose(d, part.taps());
+  ConvChoice c = choose(d, part.taps(), sharedLaunch);
   ConvP p;
   p.lhs = (const float*)lhs;
   p.rhs = (const float*)rhs;
   long long M = d->N, K = d->C;
   for (int k = 0; k < d->nsp; ++k) { M *= d->out[k]; K *= d->k[k]; }
-  if (M <= 0 || d->O <= 0) return 0;
+  if (M <= 0 || d->O <= 0) return prepared ? -1 : 0;
   p.M = (int)M; p.N = (int)d->O; p.K = (int)K;
   p.Nb = (int)d->N; p.C = (int)d->C;
   auto dim = [&](const int64_t* a, int k, int64_t dflt) { return k < d->nsp ? (int)a[k] : (int)dflt; };
@@ -920,6 +956,12 @@ static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, vo
     auto mult4 = [](long long x) { return (x & 3) == 0; };
     p.outVec = p.outF == 1 && mult4(p.N) && mult4(p.outB) && mult4(p.outS0) && mult4(p.outS1) && ((uintptr_t)dst & 15) == 0;
   }
+  if (prepared) {
+    if (c.splitK > 1 || c.kflat || c.amode == 0 || c.bmode == 0) return -1;
+    *prepared = p;
+    *preparedChoice = c;
+    return 0;
+  }
   dim3 grid((unsigned)((p.M + c.bm - 1) / c.bm), (unsigned)((p.N + c.bn - 1) / c.bn), (unsigned)c.splitK);
   if (grid.y > 65535) return 4;
   if (c.bm == 128 && c.bn == 128) launchIgemm<128, 128>(c, p, grid, st);
@@ -958,7 +1000,26 @@ int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void*
     d = &d2;
   }
   if (!choose(d).fast) return mi355_conv_direct(d, lhs, rhs, out, s);
-  for (const ConvPart& part : partsOf(d)) {
+  const std::vector<ConvPart> parts = partsOf(d);
+  static const bool packOff = getenv("MI355X_CONV_PACK") && getenv("MI355X_CONV_PACK")[0] == '0';
+  if (parts.size() > 1 && parts.size() <= (size_t)kMaxPack && !packOff) {
+    // residue classes that need no split of K when counted together share one launch
+    ConvPack ps;
+    ConvChoice cs[kMaxPack];
+    bool ok = true;
+    for (size_t i = 0; i < parts.size() && ok; ++i) {
+      ok = launchPart(parts[i], lhs, rhs, out, workspace, workspace_bytes, st, (int)parts.size(), &cs[i], &ps.c[i]) == 0;
+      if (ok && i > 0) ok = cs[i].amode == cs[0].amode && cs[i].bmode == cs[0].bmode && cs[i].bm == cs[0].bm && cs[i].bn == cs[0].bn && ps.c[i].N == ps.c[0].N;
+    }
+    if (ok) {
+      if (cs[0].bm == 128 && cs[0].bn == 128) launchPack<128, 128>(cs[0], ps, (int)parts.size(), st);
+      else if (cs[0].bm == 128) launchPack<128, 64>(cs[0], ps, (int)parts.size(), st);
+      else launchPack<64, 64>(cs[0], ps, (int)parts.size(), st);
+      hipError_t e = hipGetLastError();
+      return e == hipSuccess ? 0 : (int)e;
+    }
+  }
+  for (const ConvPart& part : parts) {
     // parts run back to back on the stream, so they can share the split-K scratch
     if (int r = launchPart(part, lhs, rhs, out, workspace, workspace_bytes, st)) return r;
   }
