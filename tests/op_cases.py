@@ -440,6 +440,16 @@ case("conv-wgrad-vector", lambda b, x, g: b.conv(x, g, strides=(1, 1), padding=(
 case("conv-wgrad-stride1-vector", lambda b, x, g: b.conv(x, g, strides=(1, 1), padding=((1, 1), (1, 1)), dn=("f01b", "i01o", "01bf")),
      u(252, 32, 8, 8, 64), u(253, 32, 8, 8, 64))
 case("conv-1x1-stride2-vector", _conv(strides=(2, 2)), u(254, 8, 8, 8, 64), u(255, 1, 1, 64, 128))
+# branches of the vector-loader kernel: windows too large for the per-tap offset table (offsets recomputed per tap),
+# output features that are no multiple of the tile, rows that are no multiple of the tile, residue classes of
+# different sizes sharing one launch
+case("conv-fwd-11x11-no-tap-table", _conv(padding=((5, 5), (5, 5))), u(1310, 2, 16, 16, 16), u(1311, 11, 11, 16, 32))
+case("conv-wgrad-144-taps-no-tap-table", lambda b, x, g: b.conv(x, g, strides=(1, 1), padding=((1, 1), (1, 1)), dn=("f01b", "i01o", "01bf")),
+     u(1312, 32, 12, 12, 64), u(1313, 32, 12, 12, 64))
+case("conv-fwd-100-features", _conv(padding=((1, 1), (1, 1))), u(1314, 4, 10, 10, 32), u(1315, 3, 3, 32, 100))
+case("conv-fwd-147-rows", _conv(padding=((1, 1), (1, 1))), u(1316, 3, 7, 7, 48), u(1317, 3, 3, 48, 64))
+case("conv-dgrad-classes-share-a-launch-odd", lambda b, g, w: b.conv(g, b.reverse(w, [0, 1]), strides=(1, 1), padding=((1, 1), (1, 1)), lhs_dilation=(2, 2), dn=("b01f", "01oi", "b01f")),
+     u(1318, 4, 7, 5, 32), u(1319, 3, 3, 16, 32))
 case("conv-bf16", _conv(padding=((1, 1), (1, 1))), u(240, 2, 8, 8, 16), u(241, 3, 3, 16, 8), dtypes=["bf16", "bf16"])
 
 # ------------------------------------------------------------------ reduce (tests/configs/reduction.py:8-39)
