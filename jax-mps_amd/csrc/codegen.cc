@@ -1121,7 +1121,7 @@ std::string shflXor(const std::string& accT, const std::string& x, const std::st
 
 }  // namespace
 
-FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeafOuter, const std::vector<Value*>& epilogue) {
+FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeafOuter, const std::vector<Value*>& epilogue, int64_t externalPartials) {
   // values computed from the results right where they are finished (second pass only)
   std::unordered_set<Value*> own;
   for (auto* r : reduces) own.insert(r->result());
@@ -1247,6 +1247,21 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     return l;
   };
 
+  if (externalPartials > 0) {
+    std::vector<int64_t> workOff;
+    int64_t wb = 0;
+    for (size_t j = 0; j < nr; ++j) {
+      workOff.push_back(wb);
+      wb += (externalPartials * Kn * 8 + 255) / 256 * 256;
+    }
+    std::vector<Value*> il;
+    fc.launches.push_back(finalPass(externalPartials, Kn, workOff, il));
+    fc.epilogueFused = !epilogue.empty();
+    fc.leaves = il;
+    fc.workspaceBytes = wb;
+    fc.partialOffsets = workOff;
+    return fc;
+  }
   if (rowStyle) {
     // lanes run along the reduced elements (r, row-major over the reduced dims).  One
     // wavefront per output when rows are short, one workgroup per output when they

@@ -34,6 +34,7 @@ struct FusedCode {
   int64_t workspaceBytes = 0;
   bool epilogueFused = false;
   std::vector<Value*> leaves;   // distinct materialised inputs
+  std::vector<int64_t> partialOffsets;   // generateReduceKernel with external partials: where each reduction's partial sums sit in the workspace
 };
 
 using LeafPredicate = std::function<bool(Value*)>;
@@ -73,7 +74,9 @@ std::string combineKernels(const std::vector<const std::string*>& sources, const
 // Returns false in `ok` when a reducer body is not a single add/mul/max/min/and/or.
 // `epilogue`: values of the result shape computed from the results (and other inputs of that shape); they are
 // produced by the pass that folds partial sums when there is one (FusedCode::epilogueFused), otherwise ignored.
-FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeaf, const std::vector<Value*>& epilogue = {});
+// `externalPartials` > 0: the partial results (that many per output, float accumulators, partial p of output k at
+// [p * outputs + k] from partialOffsets[j] of the workspace) are written by an earlier step; only the folding pass is generated.
+FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeaf, const std::vector<Value*>& epilogue = {}, int64_t externalPartials = 0);
 
 // True if codegen can inline `op` into a consumer (elementwise / indexing ops).
 bool isFusibleOp(const Op& op);

@@ -55,6 +55,11 @@ struct ConvP {
   int splitK, tilesPerSplit;
   unsigned lhsBytes, rhsBytes;   // sizes for the buffer descriptors of the vector-loader kernel (both below 2 GiB)
   int taps;                      // window taps this launch visits (kc0 * kc1)
+  // Column statistics of the output taken from the accumulators (batch-norm's sum and sum of squares over all rows):
+  // workgroup (tile row i, tile column) writes the sums over its rows to statSum[i * N + n] / statSq[i * N + n];
+  // a later pass folds the tile rows in order.  Null when not wanted.
+  float* statSum;
+  float* statSq;
 };
 
 struct Row {
@@ -618,6 +623,50 @@ __device__ __forceinline__ void leanBody(const ConvP& p, const int split) {
   }
 
   storeAccumulators<TM, TN, WM, WN>(p, acc, m0, n0, wm, wn, lane, split);
+
+  if (p.statSum != nullptr) {
+    // Per-column sums over the workgroup's rows (rows past M hold zeros).  Each wavefront lays its 32 x 32 block
+    // (summed over its row blocks) into LDS, lane l < 32 then adds column l and lane 32 + l the squares of column l,
+    // in row order; the two wavefront rows are combined through LDS and one of them writes.  The tiles of the K
+    // loop are dead by now, so their LDS is reused: 32 x 33 floats per wavefront.
+    __syncthreads();
+    constexpr int LDT = 33;
+    static_assert(2 * 32 * LDT <= 2 * ASTAGE && 2 * 32 * LDT <= 2 * BSTAGE, "statistics scratch does not fit the tile buffers");
+    float* const scratch = (wave < 2 ? As : Bs) + (wave & 1) * 32 * LDT;
+    __shared__ float colPart[2][2][2][TN * 32];   // [wave row][wave column][sum / squares][column]
+    const int row = lane & 31, half = lane >> 5;
+#pragma unroll
+    for (int b = 0; b < TN; ++b) {
+      // squares need the rows apart, so each 32-row block goes through the scratch on its own
+      float s = 0.f;
+#pragma unroll
+      for (int a = 0; a < TM; ++a) {
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) scratch[row * LDT + g4 * 8 + half * 4 + r] = acc[a][b][4 * g4 + r];
+        __syncthreads();
+#pragma unroll 8
+        for (int i = 0; i < 32; ++i) {
+          const float v = scratch[i * LDT + row];
+          s += half ? v * v : v;
+        }
+        __syncthreads();
+      }
+      colPart[wm][wn][half][b * 32 + row] = s;
+    }
+    __syncthreads();
+    if (wm == 0) {
+#pragma unroll
+      for (int b = 0; b < TN; ++b) {
+        const int n = n0 + wn * WN + b * 32 + row;
+        if (n < p.N) {
+          const float v = colPart[0][wn][half][b * 32 + row] + colPart[1][wn][half][b * 32 + row];
+          (half ? p.statSq : p.statSum)[(size_t)bx * p.N + n] = v;
+        }
+      }
+    }
+  }
 }
 
 template <int BM, int BN, int AMODE, int BMODE, bool TABLE>
@@ -897,12 +946,14 @@ int mi355_conv_direct(const mi355_conv_desc* d, const void* lhs, const void* rhs
 
 // Launches one part; with `prepared` set it only fills the kernel parameters of an unsplit part (returns -1 when the part cannot be prepared that way).
 static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes, hipStream_t st,
-                      int sharedLaunch = 1, ConvChoice* preparedChoice = nullptr, ConvP* prepared = nullptr) {
+                      int sharedLaunch = 1, ConvChoice* preparedChoice = nullptr, ConvP* prepared = nullptr, float* statSum = nullptr, float* statSq = nullptr) {
   const mi355_conv_desc* d = &part.d;
   ConvChoice c = choose(d, part.taps(), sharedLaunch);
   ConvP p;
   p.lhs = (const float*)lhs;
   p.rhs = (const float*)rhs;
+  p.statSum = statSum;
+  p.statSq = statSq;
   long long M = d->N, K = d->C;
   for (int k = 0; k < d->nsp; ++k) { M *= d->out[k]; K *= d->k[k]; }
   if (M <= 0 || d->O <= 0) return prepared ? -1 : 0;
@@ -978,9 +1029,37 @@ static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, vo
   return e == hipSuccess ? 0 : (int)e;
 }
 
+// Rows of per-tile column sums the convolution can deliver next to its output (one per tile row of the implicit GEMM),
+// or 0 when it cannot: the vector-loader kernel, unsplit, one launch, output rows dense and in GEMM row order.
+int mi355_conv_stats_rows(const mi355_conv_desc* d) {
+  static const bool off = getenv("MI355X_CONV_STATS") && getenv("MI355X_CONV_STATS")[0] == '0';
+  mi355_conv_desc d2;
+  if (off || repackedFilter(d, &d2)) return 0;
+  ConvChoice c = choose(d);
+  if (!c.fast || c.kflat || c.amode == 0 || c.bmode == 0 || c.splitK != 1 || c.bFast) return 0;
+  if (partsOf(d).size() != 1) return 0;
+  long long M = d->N;
+  for (int k = 0; k < d->nsp; ++k) M *= d->out[k];
+  if (M <= 0 || d->outF != 1) return 0;
+  // dense output in GEMM row order: row (b, o0, o1) starts at ((b * out0 + o0) * out1 + o1) * O
+  long long expect = d->O;
+  for (int k = d->nsp - 1; k >= 0; --k) { if (d->outS[k] != expect) return 0; expect *= d->out[k]; }
+  if (d->outB != expect) return 0;
+  return (int)((M + c.bm - 1) / c.bm);
+}
+
+int mi355_conv_stats(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes,
+                     float* stat_sum, float* stat_sq, mi355_stream_t s);
+
 int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes,
                mi355_stream_t s) {
+  return mi355_conv_stats(d, lhs, rhs, out, workspace, workspace_bytes, nullptr, nullptr, s);
+}
+
+int mi355_conv_stats(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes,
+                     float* stat_sum, float* stat_sq, mi355_stream_t s) {
   hipStream_t st = (hipStream_t)s;
+  if (stat_sum && mi355_conv_stats_rows(d) == 0) return 5;   // the planner asked for statistics this convolution cannot deliver
   mi355_conv_desc d2;
   size_t repack = repackedFilter(d, &d2);
   if (repack) {
@@ -1021,7 +1100,7 @@ int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void*
   }
   for (const ConvPart& part : parts) {
     // parts run back to back on the stream, so they can share the split-K scratch
-    if (int r = launchPart(part, lhs, rhs, out, workspace, workspace_bytes, st)) return r;
+    if (int r = launchPart(part, lhs, rhs, out, workspace, workspace_bytes, st, 1, nullptr, nullptr, stat_sum, stat_sq)) return r;
   }
   return 0;
 }

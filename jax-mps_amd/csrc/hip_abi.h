@@ -117,6 +117,12 @@ typedef struct {
 int mi355_conv(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace,
                size_t workspace_bytes, mi355_stream_t s);
 size_t mi355_conv_workspace_bytes(const mi355_conv_desc* d);
+// Column statistics next to the output: mi355_conv_stats_rows(d) > 0 says the convolution can deliver, for each of that
+// many tile rows i and every output feature n, the sum and the sum of squares of its rows' outputs (stat_sum[i * O + n],
+// stat_sq[i * O + n], both rows x O floats); folding the tile rows in order gives the statistics of the whole output.
+int mi355_conv_stats_rows(const mi355_conv_desc* d);
+int mi355_conv_stats(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, void* workspace, size_t workspace_bytes,
+                     float* stat_sum, float* stat_sq, mi355_stream_t s);
 int mi355_conv_direct(const mi355_conv_desc* d, const void* lhs, const void* rhs, void* out, mi355_stream_t s);
 
 typedef struct {

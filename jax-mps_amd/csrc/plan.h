@@ -91,6 +91,7 @@ struct Step {
   ConvDesc conv;
   ScatterDesc scatter;
   BufRef bias;                     // Gemm: per-column values added to the product (kind None: no bias)
+  int statsArg = -1;               // Conv: index in args of the column-sum buffer (the sum-of-squares buffer follows), or -1
   int64_t workspaceOffset = -1;    // arena offset of split-K / sort scratch
   int64_t workspaceBytes = 0;
   int splitK = 1;

@@ -276,7 +276,10 @@ class Planner {
     return id;
   }
 
-  void addFused(Plan& plan, const FusedCode& fc, const std::string& label, const std::vector<Value*>& outs) {
+  // a convolution step that writes the partial sums a folding kernel reads: its statistics land in that kernel's workspace
+  struct ProducerStats { size_t step = 0; int64_t sumOffset = 0, sqOffset = 0; };
+
+  void addFused(Plan& plan, const FusedCode& fc, const std::string& label, const std::vector<Value*>& outs, const ProducerStats* producer = nullptr) {
     int ws = -1;
     int t0 = time_ + 1;
     int t1 = time_ + (int)fc.launches.size();
@@ -284,6 +287,18 @@ class Planner {
       ws = newStorage((size_t)fc.workspaceBytes);
       ref(ws, t0);
       ref(ws, t1);
+      st_[ws].uses.clear();
+    }
+    if (producer) {
+      // (before any step is appended: the reference into plan.steps does not survive a push_back)
+      Step& cs = plan.steps[producer->step];
+      cs.statsArg = (int)cs.args.size();
+      BufRef a = ref(ws, cs.time), b = ref(ws, cs.time);
+      a.offset = producer->sumOffset;
+      b.offset = producer->sqOffset;
+      cs.args.push_back(a);
+      cs.args.push_back(b);
+      cs.label += " + column statistics";
       st_[ws].uses.clear();
     }
     int64_t bytes = 0;
@@ -752,7 +767,38 @@ class Planner {
         epilogueOps.push_back(y);
       }
     }
-    FusedCode fc = generateReduceKernel(group, leafPred(), epilogue);
+    // Batch-norm statistics of a convolution's output: when the step just emitted is the convolution that produced the
+    // reduced tensor, the reductions are its column sum and column sum of squares, and the kernel can take them from
+    // its accumulators (per tile row), the pass over the output is dropped and only the fold of the tile rows remains.
+    int64_t statRows = 0;
+    int sumAt = -1, sqAt = -1;
+    static const bool statsOn = !getenv("MI355X_CONV_STATS") || atoi(getenv("MI355X_CONV_STATS")) != 0;
+    if (statsOn && group.size() == 2 && !plan.steps.empty() && plan.steps.back().kind == Step::Conv && plan.steps.back().statsArg < 0) {
+      Step& cs = plan.steps.back();
+      Value* y = nullptr;
+      Value* ySquared = nullptr;
+      for (int j = 0; j < 2; ++j) {
+        Value* x = group[(size_t)j]->operands[0];
+        const char* kind = simpleReduceKind(*group[(size_t)j]);
+        if (!kind || std::string(kind) != "add") { sumAt = sqAt = -2; break; }
+        if (hasStorage(x)) { sumAt = sumAt == -1 ? j : -2; y = x; }
+        else if (x->def && x->def->name == "multiply" && x->def->operands[0] == x->def->operands[1] && hasStorage(x->def->operands[0])) { sqAt = sqAt == -1 ? j : -2; ySquared = x->def->operands[0]; }
+      }
+      bool ok = sumAt >= 0 && sqAt >= 0 && y == ySquared && y->type.dt == DType::F32 && cs.args.size() >= 3 && cs.args[2].index == storageOf(y) && cs.conv.type == DType::F32;
+      if (ok) {
+        // every dim but the last (the feature axis) is reduced
+        auto dims = op->ints("dimensions");
+        std::sort(dims.begin(), dims.end());
+        ok = (int)dims.size() == y->type.rank() - 1;
+        for (size_t k = 0; ok && k < dims.size(); ++k) ok = dims[k] == (int64_t)k;
+      }
+      if (ok) {
+        mi355_conv_desc abi = toAbi(cs.conv);
+        statRows = mi355_conv_stats_rows(&abi);
+        if (statRows > 0 && (int64_t)abi.O != y->type.dims.back()) statRows = 0;
+      }
+    }
+    FusedCode fc = generateReduceKernel(group, leafPred(), epilogue, statRows);
     std::vector<Value*> outs;
     for (auto* g : group) {
       bind(g->result(), newStorage(g->result()->type.bytes()));
@@ -760,6 +806,7 @@ class Planner {
       emitted_.insert(g);
     }
     std::string label = (group.size() > 1 ? "reduce x" + std::to_string(group.size()) : std::string("reduce"));
+    if (statRows > 0) label = "fold of convolution statistics, " + label;
     if (fc.epilogueFused) {
       for (size_t k = 0; k < epilogue.size(); ++k) {
         bind(epilogue[k], newStorage(epilogue[k]->type.bytes()));
@@ -768,7 +815,15 @@ class Planner {
         label += "+" + epilogueOps[k]->name;
       }
     }
-    addFused(plan, fc, label + " " + group[0]->operands[0]->type.str() + " -> " + outs[0]->type.str(), outs);
+    if (statRows > 0) {
+      ProducerStats ps;
+      ps.step = plan.steps.size() - 1;
+      ps.sumOffset = fc.partialOffsets[(size_t)sumAt];
+      ps.sqOffset = fc.partialOffsets[(size_t)sqAt];
+      addFused(plan, fc, label + " " + group[0]->operands[0]->type.str() + " -> " + outs[0]->type.str(), outs, &ps);
+    } else {
+      addFused(plan, fc, label + " " + group[0]->operands[0]->type.str() + " -> " + outs[0]->type.str(), outs);
+    }
   }
 
   static std::vector<int64_t> stridesOf(const TensorType& t) {
@@ -1479,6 +1534,7 @@ class Planner {
     s.label = "convolution " + lhs->type.str() + " * " + rhs->type.str();
     s.conv = c;
     s.args = {ref(storageOf(lhs), t), ref(storageOf(rhs), t), ref(sid, t)};
+    s.time = t;
     // split-K partial sums for shapes with few output tiles (filter gradients, late stages)
     mi355_conv_desc abi = toAbi(c);
     int64_t ws = ((int64_t)mi355_conv_workspace_bytes(&abi) + kAlign - 1) / kAlign * kAlign;

@@ -482,9 +482,11 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
     }
     case Step::Conv: {
       mi355_conv_desc d = toAbi(s.conv);
-      void* ws = s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
-      check(mi355_conv(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), ws,
-                       (size_t)s.workspaceBytes, st), "convolution");
+      void* ws = s.workspaceBytes > 0 && s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
+      float* statSum = s.statsArg >= 0 ? (float*)resolve(s.args[(size_t)s.statsArg], in, out) : nullptr;
+      float* statSq = s.statsArg >= 0 ? (float*)resolve(s.args[(size_t)s.statsArg + 1], in, out) : nullptr;
+      check(mi355_conv_stats(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out), ws,
+                             (size_t)s.workspaceBytes, statSum, statSq, st), "convolution");
       break;
     }
     case Step::ScatterRows: {

@@ -450,6 +450,26 @@ case("conv-fwd-100-features", _conv(padding=((1, 1), (1, 1))), u(1314, 4, 10, 10
 case("conv-fwd-147-rows", _conv(padding=((1, 1), (1, 1))), u(1316, 3, 7, 7, 48), u(1317, 3, 3, 48, 64))
 case("conv-dgrad-classes-share-a-launch-odd", lambda b, g, w: b.conv(g, b.reverse(w, [0, 1]), strides=(1, 1), padding=((1, 1), (1, 1)), lhs_dilation=(2, 2), dn=("b01f", "01oi", "b01f")),
      u(1318, 4, 7, 5, 32), u(1319, 3, 3, 16, 32))
+# batch-norm statistics taken from the convolution's accumulators: the sum and the sum of squares over every dim but the
+# features, right after the convolution (ragged rows and two feature tiles included), and the same sums when the
+# convolution cannot deliver them (a split of K) or must not (another reduction kind)
+def _conv_stats(padding=((1, 1), (1, 1)), kind="add"):
+    def f(b, x, w):
+        y = b.conv(x, w, padding=padding)
+        axes = list(range(y.ndim - 1))
+        if kind == "add":
+            return [y, b.reduce_sum(y, axes), b.reduce_sum(b.mul(y, y), axes)]
+        return [y, b.reduce_max(y, axes), b.reduce_sum(b.mul(y, y), axes)]
+    return f
+
+
+# (the kernel delivers them only when it runs unsplit, i.e. with a few hundred output tiles; positive inputs, so that the
+# sums do not cancel and the elementwise bound is a relative one)
+case("conv-statistics-from-accumulators", _conv_stats(), f32(1320, 24, 32, 32, 16, lo=0.05, hi=1.0), f32(1321, 3, 3, 16, 64, lo=0.05, hi=1.0))
+case("conv-statistics-ragged-rows-two-feature-tiles", _conv_stats(), f32(1322, 12, 31, 31, 16, lo=0.05, hi=1.0), f32(1323, 3, 3, 16, 128, lo=0.05, hi=1.0))
+case("conv-statistics-100-features", _conv_stats(), f32(1324, 12, 31, 31, 16, lo=0.05, hi=1.0), f32(1325, 3, 3, 16, 100, lo=0.05, hi=1.0))
+case("conv-statistics-split-k-stays-unfused", _conv_stats(), f32(1326, 2, 4, 4, 256, lo=0.05, hi=1.0), f32(1327, 3, 3, 256, 64, lo=0.05, hi=1.0))
+case("conv-statistics-max-stays-unfused", _conv_stats(kind="max"), f32(1328, 24, 32, 32, 16, lo=0.05, hi=1.0), f32(1329, 3, 3, 16, 64, lo=0.05, hi=1.0))
 case("conv-bf16", _conv(padding=((1, 1), (1, 1))), u(240, 2, 8, 8, 16), u(241, 3, 3, 16, 8), dtypes=["bf16", "bf16"])
 
 # ------------------------------------------------------------------ reduce (tests/configs/reduction.py:8-39)

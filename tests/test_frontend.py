@@ -105,6 +105,21 @@ module @jit_f attributes {mhlo.num_partitions = 1 : i32} {
     assert r.returncode == 0, r.stderr
 
 
+def test_convolution_delivers_batch_norm_statistics():
+    """The column sum and sum of squares of an unsplit convolution's output come from its accumulators: the pass over
+    the output is gone and only the fold of the per-tile sums remains; a convolution that splits K, or a reduction
+    of another kind, keeps the two-pass reduction."""
+    r = plan(op_cases.get_case("conv-statistics-from-accumulators").text, "--dump-plan")
+    assert "+ column statistics" in r.stdout and r.stdout.count("kernel ") == 1 and "fold of convolution statistics" in r.stdout
+    r = plan(op_cases.get_case("conv-statistics-split-k-stays-unfused").text, "--dump-plan")
+    assert "column statistics" not in r.stdout and r.stdout.count("kernel ") == 2
+    r = plan(op_cases.get_case("conv-statistics-max-stays-unfused").text, "--dump-plan")
+    assert "column statistics" not in r.stdout
+    p = configs.build_resnet18()
+    r = plan(p.text, "--dump-plan")
+    assert r.stdout.count("+ column statistics") >= 14      # every unsplit forward convolution that feeds a batch norm
+
+
 def test_lstm_scan_updates_in_place():
     p = configs.build_lstm(**configs.SMALL["lstm"])
     r = plan(p.text, "--dump-plan")
