@@ -127,7 +127,7 @@ def cpu_baseline(budget_s=12.0, batch=128):
 
 # HBM bytes per conv_igemm_f32 launch of this workload: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by
 # what the same counter reads for a 256 MiB copy (profiles/conv_igemm_f32_resnet18_b128_hbm_traffic.md).
-CONV_HBM_BYTES_PER_LAUNCH = 105.7e6
+CONV_HBM_BYTES_PER_LAUNCH = 117.5e6
 
 
 # Algorithmic work of the other four benchmark programs (the figures the design notes quote): flops of the MFMA
