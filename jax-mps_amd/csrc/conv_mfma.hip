@@ -55,6 +55,7 @@ struct ConvP {
   int splitK, tilesPerSplit;
   unsigned lhsBytes, rhsBytes;   // sizes for the buffer descriptors of the vector-loader kernel (both below 2 GiB)
   int taps;                      // window taps this launch visits (kc0 * kc1)
+  int tilesM, tilesXY;           // split launches of the vector-loader kernel: tile rows and tiles per K range (tilesXY 0: a 3-d grid)
   // Column statistics of the output taken from the accumulators (batch-norm's sum and sum of squares over all rows):
   // workgroup (tile row i, tile column) writes the sums over its rows to statSum[i * N + n] / statSq[i * N + n];
   // a later pass folds the tile rows in order.  Null when not wanted.
@@ -406,7 +407,7 @@ constexpr unsigned kOutside = 0x80000000u;     // an offset no tensor reaches (t
 constexpr int kTapTableBytes = 16384;          // largest per-workgroup tap table
 
 template <int BM, int BN, int AMODE, int BMODE, bool TABLE>
-__device__ __forceinline__ void leanBody(const ConvP& p, const int split) {
+__device__ __forceinline__ void leanBody(const ConvP& p, int split) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int NA4 = BM / 64, NB4 = BN / 64;
   // A tile fetched with K-vectors stays row-major in LDS ([row or column][k], rows 20 floats apart): a fetched vector
@@ -423,9 +424,21 @@ __device__ __forceinline__ void leanBody(const ConvP& p, const int split) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  int bx = blockIdx.x;
-  if ((gridDim.x & 7) == 0) bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);
-  const int m0 = bx * BM, n0 = blockIdx.y * BN;
+  int bx = blockIdx.x, by = blockIdx.y;
+  if (p.tilesXY > 0) {
+    // A launch that splits K is one-dimensional: workgroups go to the eight XCDs round-robin by their number, and the
+    // numbering here puts all output tiles of one K range on the same XCD, next to each other, so that the tiles of
+    // an operand they share (every tile row reads the same rhs tiles, neighbouring taps the same lhs rows) meet in one L2.
+    const int xcd = bx & 7, slot = bx >> 3;
+    const int group = slot / p.tilesXY, t = slot - group * p.tilesXY;
+    split = xcd + 8 * group;
+    if (split >= p.splitK) return;
+    by = t / p.tilesM;
+    bx = t - by * p.tilesM;
+  } else if ((gridDim.x & 7) == 0) {
+    bx = (bx & 7) * (gridDim.x >> 3) + (bx >> 3);
+  }
+  const int m0 = bx * BM, n0 = by * BN;
   if (m0 >= p.M) return;                      // (a launch shared by several problems is as wide as the widest)
   const int ktBegin = split * p.tilesPerSplit;
   const int ktEnd = min(p.kTiles, ktBegin + p.tilesPerSplit);
@@ -811,6 +824,8 @@ ConvChoice choose(const mi355_conv_desc* d, long long tapsVisited = -1, int shar
   static const int splitFactor = getenv("MI355X_CONV_SPLIT_FACTOR") ? atoi(getenv("MI355X_CONV_SPLIT_FACTOR")) : 3;
   if (tiles * (c.amode == 2 ? 2 : splitFactor) <= target && c.kTiles >= minSplitTiles) split = (int)std::min<long long>(target / tiles, std::max(1, c.kTiles / (tiles < 64 ? 4 : 8)));
   split = std::max(1, std::min(split, 256));
+  static const bool xcdSplit = getenv("MI355X_CONV_XCD_SPLIT") && getenv("MI355X_CONV_XCD_SPLIT")[0] == '1';
+  if (xcdSplit && split >= 16) split = split / 8 * 8;   // whole groups of K ranges per XCD, so that no XCD runs a workgroup more than the others
   c.tilesPerSplit = (c.kTiles + split - 1) / split;
   c.splitK = (c.kTiles + c.tilesPerSplit - 1) / c.tilesPerSplit;
   return c;
@@ -954,6 +969,8 @@ static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, vo
   p.rhs = (const float*)rhs;
   p.statSum = statSum;
   p.statSq = statSq;
+  p.tilesM = 0;
+  p.tilesXY = 0;
   long long M = d->N, K = d->C;
   for (int k = 0; k < d->nsp; ++k) { M *= d->out[k]; K *= d->k[k]; }
   if (M <= 0 || d->O <= 0) return prepared ? -1 : 0;
@@ -1015,6 +1032,12 @@ static int launchPart(const ConvPart& part, const void* lhs, const void* rhs, vo
   }
   dim3 grid((unsigned)((p.M + c.bm - 1) / c.bm), (unsigned)((p.N + c.bn - 1) / c.bn), (unsigned)c.splitK);
   if (grid.y > 65535) return 4;
+  static const bool xcdSplitOn = getenv("MI355X_CONV_XCD_SPLIT") && getenv("MI355X_CONV_XCD_SPLIT")[0] == '1';
+  if (c.splitK >= 16 && !c.kflat && c.amode != 0 && c.bmode != 0 && xcdSplitOn) {   // (with fewer K ranges than a few per XCD the XCDs would not be loaded evenly)
+    p.tilesM = (int)grid.x;
+    p.tilesXY = (int)(grid.x * grid.y);
+    grid = dim3((unsigned)(8 * p.tilesXY * ((c.splitK + 7) / 8)), 1, 1);
+  }
   if (c.bm == 128 && c.bn == 128) launchIgemm<128, 128>(c, p, grid, st);
   else if (c.bm == 128) launchIgemm<128, 64>(c, p, grid, st);
   else launchIgemm<64, 64>(c, p, grid, st);
