@@ -177,7 +177,7 @@ def main():
         print("bench.py: this build drives exactly one GPU (one PJRT device); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     os.environ.setdefault("MI355X_TIMING", "conv")     # HIP-event timing of the convolution launches only,
-    every = int(os.environ.setdefault("MI355X_TIMING_EVERY", "5"))   # on one step in five: the events cost ~5 us per launch
+    every = int(os.environ.setdefault("MI355X_TIMING_EVERY", "10"))  # on one step in ten: the events cost ~5 us per launch, and a timed step runs every launch in order on one stream
     from jax_mps_amd import pjrt, runner
     from jax_mps_amd.programs import configs
     client = pjrt.get_client()

@@ -34,10 +34,12 @@ int mi355_memcpy_d2d(void* dst, const void* src, size_t bytes, mi355_stream_t s)
 
 // streams and events (default priority only)
 int mi355_stream_create(mi355_stream_t* s);
+int mi355_stream_destroy(mi355_stream_t s);
 int mi355_stream_sync(mi355_stream_t s);
 int mi355_event_create(mi355_event_t* e, int timing);
 int mi355_event_destroy(mi355_event_t e);
 int mi355_event_record(mi355_event_t e, mi355_stream_t s);
+int mi355_stream_wait_event(mi355_stream_t s, mi355_event_t e);   // work enqueued on s after this call waits for what e recorded
 int mi355_event_sync(mi355_event_t e);
 int mi355_event_query(mi355_event_t e, int* ready);
 int mi355_event_elapsed_ms(mi355_event_t a, mi355_event_t b, float* ms);

@@ -86,6 +86,10 @@ int mi355_stream_create(mi355_stream_t* s) {
   *s = (mi355_stream_t)st;
   return 0;
 }
+int mi355_stream_destroy(mi355_stream_t s) {
+  HIPCHK(hipStreamDestroy((hipStream_t)s));
+  return 0;
+}
 int mi355_stream_sync(mi355_stream_t s) {
   HIPCHK(hipStreamSynchronize((hipStream_t)s));
   return 0;
@@ -129,6 +133,10 @@ int mi355_event_destroy(mi355_event_t e) {
 }
 int mi355_event_record(mi355_event_t e, mi355_stream_t s) {
   HIPCHK(hipEventRecord((hipEvent_t)e, (hipStream_t)s));
+  return 0;
+}
+int mi355_stream_wait_event(mi355_stream_t s, mi355_event_t e) {
+  HIPCHK(hipStreamWaitEvent((hipStream_t)s, (hipEvent_t)e, 0));
   return 0;
 }
 int mi355_event_sync(mi355_event_t e) {

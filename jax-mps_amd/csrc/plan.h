@@ -92,6 +92,11 @@ struct Step {
   ScatterDesc scatter;
   BufRef bias;                     // Gemm: per-column values added to the product (kind None: no bias)
   int statsArg = -1;               // Conv: index in args of the column-sum buffer (the sum-of-squares buffer follows), or -1
+  // A step whose results nothing needs for a while (a filter gradient, read only by the optimizer update at the end of
+  // the step) may run on a second stream next to the steps that follow it: forkId >= 0 marks it, and the first later
+  // step that touches what it wrote, or writes what it read, lists the id in `joins` and waits for it.
+  int forkId = -1;
+  std::vector<int> joins;
   int64_t workspaceOffset = -1;    // arena offset of split-K / sort scratch
   int64_t workspaceBytes = 0;
   int splitK = 1;
@@ -124,6 +129,7 @@ struct Step {
 };
 
 struct Plan {
+  int numForks = 0;                 // forked steps of this (top-level) plan; those nobody joined are joined at its end
   std::vector<Step> steps;
 };
 

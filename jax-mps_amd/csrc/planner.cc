@@ -93,6 +93,7 @@ class Planner {
     static const bool batching = !getenv("MI355X_BATCH_KERNELS") || atoi(getenv("MI355X_BATCH_KERNELS")) != 0;
     groupSmallGemms(P.plan);
     if (batching) batchKernels(P.plan);
+    forkDistantConvolutions(P.plan);
     assignArena();
     patch(P.plan);
     P.numSteps = countSteps(P.plan);
@@ -2155,6 +2156,35 @@ class Planner {
     steps = std::move(out);
   }
 
+  // Convolutions whose results are not needed for several steps (filter gradients: only the optimizer update at the
+  // end of the step reads them) are marked to run on a second stream.  Every buffer such a step touches then stays
+  // allocated to the end of the plan, because the steps after it no longer wait for it before reusing memory.
+  void forkDistantConvolutions(Plan& plan) {
+    static const int minDistance = getenv("MI355X_FORK_DISTANCE") ? atoi(getenv("MI355X_FORK_DISTANCE")) : 6;
+    if (minDistance <= 0) return;
+    for (auto& s : plan.steps) if (s.kind == Step::While || s.kind == Step::Case) return;   // loops replay from graphs on one stream
+    const size_t n = plan.steps.size();
+    for (size_t i = 0; i < n; ++i) {
+      Step& s = plan.steps[i];
+      if (s.kind != Step::Conv || s.statsArg >= 0) continue;
+      std::unordered_set<int> reads, writes;
+      forEachRef(s, [&](BufRef& r, bool w) { (w ? writes : reads).insert(r.index); });
+      size_t j = i + 1;
+      for (; j < n; ++j) {
+        bool touches = false;
+        forEachRef(plan.steps[j], [&](BufRef& r, bool w) {
+          if (writes.count(r.index) || (w && reads.count(r.index))) touches = true;
+        });
+        if (touches) break;
+      }
+      if (j - i < (size_t)minDistance) continue;
+      s.forkId = plan.numForks++;
+      if (j < n) plan.steps[j].joins.push_back(s.forkId);
+      for (int sid : reads) if (st_[sid].kind == BufRef::Temp) st_[sid].last = std::max(st_[sid].last, time_);
+      for (int sid : writes) if (st_[sid].kind == BufRef::Temp) st_[sid].last = std::max(st_[sid].last, time_);
+    }
+  }
+
   // ---------------------------------------------------------------- arena
   void assignArena() {
     // a buffer that is used inside a loop but defined outside it lives until the loop ends
@@ -2238,6 +2268,8 @@ class Planner {
       if (s.kind == Step::While) o << " trip " << s.tripCount << (s.flagBuf.kind != BufRef::None ? " on-device" : "");
       if (s.kind == Step::Case && s.predicated) o << " all-branches";
       if (s.kind == Step::Copy && s.condMode) o << (s.condMode == 1 ? " if-alive" : " if-selected");
+      if (s.forkId >= 0) o << " [second stream #" << s.forkId << "]";
+      for (int id : s.joins) o << " [waits for #" << id << "]";
       o << "\n";
       P.dump += o.str();
       o.str("");

@@ -255,6 +255,10 @@ Executable::~Executable() {
   for (auto& g : loopGraphs_) for (auto& e : g.second.entries) if (e.exec) mi355_graph_destroy(e.exec);
   for (auto e : eventPool_) mi355_event_destroy(e);
   for (auto& p : pending_) { mi355_event_destroy(p.a); mi355_event_destroy(p.b); }
+  // (work on the second stream was joined into the main stream before each call returned, so it has drained too)
+  for (auto e : forkStart_) mi355_event_destroy(e);
+  for (auto e : forkDone_) mi355_event_destroy(e);
+  if (sideStream_) mi355_stream_destroy(sideStream_);
 }
 
 void Executable::loadKernels() {
@@ -373,7 +377,7 @@ static int dtypeCode(DType d) { return abiDtypeCode(d); }
 
 void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
   Device& dev = Device::get();
-  mi355_stream_t st = dev.stream();
+  mi355_stream_t st = streamOverride_ ? streamOverride_ : dev.stream();
   std::string kind;
   double flops = 0, bytes = 0;
   switch (s.kind) {
@@ -719,7 +723,42 @@ void Executable::replayIterations(const Step& s, bool withCond, int64_t trip, co
 }
 
 void Executable::runPlan(const Plan& plan, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
-  for (auto& s : plan.steps) runStep(s, in, out);
+  // Forked steps run on the second stream: it waits for everything enqueued so far, and the step that first needs the
+  // result (or the end of the plan) makes the main stream wait for it.  A call whose steps are being timed runs
+  // everything in order on the main stream, so that the step times stay those of the kernels alone.
+  static const bool forking = !getenv("MI355X_SECOND_STREAM") || atoi(getenv("MI355X_SECOND_STREAM")) != 0;
+  if (plan.numForks == 0 || !forking || (timedCall_ && !timingKinds_.empty())) {
+    for (auto& s : plan.steps) runStep(s, in, out);
+    return;
+  }
+  Device& dev = Device::get();
+  if (!sideStream_) check(mi355_stream_create(&sideStream_), "second stream");
+  while (forkStart_.size() < (size_t)plan.numForks) {
+    mi355_event_t a = nullptr, b = nullptr;
+    check(mi355_event_create(&a, 0), "event");
+    check(mi355_event_create(&b, 0), "event");
+    forkStart_.push_back(a);
+    forkDone_.push_back(b);
+  }
+  std::vector<char> pending((size_t)plan.numForks, 0);
+  for (auto& s : plan.steps) {
+    for (int id : s.joins) {
+      if (!pending[(size_t)id]) continue;
+      check(mi355_stream_wait_event(dev.stream(), forkDone_[(size_t)id]), "join");
+      pending[(size_t)id] = 0;
+    }
+    if (s.forkId < 0) { runStep(s, in, out); continue; }
+    const size_t id = (size_t)s.forkId;
+    check(mi355_event_record(forkStart_[id], dev.stream()), "fork");
+    check(mi355_stream_wait_event(sideStream_, forkStart_[id]), "fork");
+    streamOverride_ = sideStream_;
+    try { runStep(s, in, out); } catch (...) { streamOverride_ = nullptr; throw; }
+    streamOverride_ = nullptr;
+    check(mi355_event_record(forkDone_[id], sideStream_), "fork");
+    pending[id] = 1;
+  }
+  for (size_t id = 0; id < pending.size(); ++id)
+    if (pending[id]) check(mi355_stream_wait_event(dev.stream(), forkDone_[id]), "join");
 }
 
 std::vector<std::shared_ptr<DeviceBuffer>> Executable::execute(const std::vector<DeviceBuffer*>& inputs, const std::vector<bool>* mayDonate) {

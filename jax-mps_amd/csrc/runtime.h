@@ -140,6 +140,9 @@ class Executable {
   void loadKernels();
   void* resolve(const BufRef& r, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) const;
   void runPlan(const Plan& plan, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
+  mi355_stream_t sideStream_ = nullptr;       // second stream for forked steps, created on first use
+  mi355_stream_t streamOverride_ = nullptr;   // set while a forked step is being enqueued
+  std::vector<mi355_event_t> forkStart_, forkDone_;
   void runStep(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
   bool timed(const std::string& kind) const;
   mi355_event_t getEvent();
