@@ -120,6 +120,20 @@ def test_convolution_delivers_batch_norm_statistics():
     assert r.stdout.count("+ column statistics") >= 14      # every unsplit forward convolution that feeds a batch norm
 
 
+def test_distant_convolutions_take_the_second_stream():
+    """A convolution nothing reads for several steps is marked for the second stream and its first reader waits for it;
+    the filter gradients of the ResNet step are such convolutions, and a program with a loop forks nothing."""
+    import test_gpu_second_stream
+    r = plan(test_gpu_second_stream._program(), "--dump-plan")
+    lines = r.stdout.splitlines()
+    assert "[second stream #0]" in lines[0] and lines[0].startswith("conv ")
+    assert any("[waits for #0]" in l for l in lines[1:]) and sum("[second stream" in l for l in lines) == 1
+    r = plan(configs.build_resnet18().text, "--dump-plan")
+    assert r.stdout.count("[second stream #") >= 13 and r.stdout.count("[waits for #") == r.stdout.count("[second stream #")
+    r = plan(configs.build_lstm(**configs.SMALL["lstm"]).text, "--dump-plan")
+    assert "[second stream" not in r.stdout
+
+
 def test_lstm_scan_updates_in_place():
     p = configs.build_lstm(**configs.SMALL["lstm"])
     r = plan(p.text, "--dump-plan")
