@@ -170,12 +170,16 @@ def main():
     ap.add_argument("--no-other-configs", action="store_true")
     ap.add_argument("--config", default=None, help="time only this benchmark program (mlp, embedding, distilbert, lstm) and print its record")
     ap.add_argument("--fused-only", action="store_true", help="time only the fused-op bandwidth shapes and print their records")
+    ap.add_argument("--one-stream", action="store_true",
+                    help="keep every launch on one stream (no filter gradients on the second stream): kernel traces then show each kernel alone")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device copy (kernel copy_vec16) a few times: the known-size reference for scaling FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives exactly one GPU (one PJRT device); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.one_stream:
+        os.environ["MI355X_SECOND_STREAM"] = "0"
     os.environ.setdefault("MI355X_TIMING", "conv")     # HIP-event timing of the convolution launches only,
     every = int(os.environ.setdefault("MI355X_TIMING_EVERY", "10"))  # on one step in ten: the events cost ~5 us per launch, and a timed step runs every launch in order on one stream
     from jax_mps_amd import pjrt, runner
