@@ -16,11 +16,19 @@
 //             scalar  : anything else
 //
 // A workgroup of four wavefronts owns a BM x BN tile (2 x 2 wavefronts, each WM x WN built
-// from 32x32 accumulators of v_mfma_f32_32x32x2_f32).  Tiles of A and B are staged in LDS
-// k-major, so that every MFMA operand is one conflict-free row read; the next k-tile is
-// fetched into registers while the current one is multiplied.  Problems with few output
-// tiles (filter gradients, late stages) split K across blockIdx.z into partial sums that a
-// second kernel folds in a fixed order, which keeps results reproducible.
+// from 32x32 accumulators of v_mfma_f32_32x32x2_f32).  Tiles of A and B go through two LDS
+// stages and two register sets, so that a tile is being fetched two k-steps ahead of the
+// one being multiplied.  Problems with few output tiles (filter gradients, late stages)
+// split K across workgroups into partial sums that a second kernel folds in a fixed order,
+// which keeps results reproducible.
+//
+// Two kernels share this scheme: conv_igemm_lean for the vector loaders (every large
+// convolution; its k-loop carries next to no vector arithmetic, see the comment above it)
+// and conv_igemm_f32 for the scalar loaders (a 3-channel stem, odd layouts), which computes
+// every element's address and validity as it goes.  The lean kernel can also deliver the
+// column sums and sums of squares of its output (batch-norm statistics), run several
+// unsplit problems in one launch (the residue classes of an input-dilated convolution) and
+// number the workgroups of a split launch by XCD.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
