@@ -171,7 +171,6 @@ class Converter {
     readDialects(sections[kDialect]);
     readOffsets(sections[kAttrTypeOffset], sections[kAttrType]);
     Cursor ir = sections[kIR];
-    out_ << "module {\n";
     // the top-level block holds exactly the module op
     bool hasArgs;
     uint64_t numOps = ir.varintFlag(hasArgs);
@@ -721,7 +720,7 @@ class Converter {
       if (v.kind == BAttr::Tensor && name != "constant") {
         const BType& t = type((uint64_t)v.type);
         const BType& el = type((uint64_t)t.elem);
-        if (t.shape.size() <= 2 && el.code != kBooleanT && el.code != kF32T && el.code != kF64T && el.code != kBF16T && el.code != kF16T) text = i64Array(tensorInts(v));
+        if (k != "replica_groups" && t.shape.size() <= 2 && el.code != kBooleanT && el.code != kF32T && el.code != kF64T && el.code != kBF16T && el.code != kF16T) text = i64Array(tensorInts(v));
         else text = denseText(v);
       } else {
         text = attrText(v);
@@ -840,6 +839,15 @@ class Converter {
     if (dialect == "builtin" && on.name == "module") {
       if (!topLevel) bad("nested modules are not supported");
       if (numRegions != 1) bad("builtin.module must have one region");
+      // the device counts are the only module attributes the compiler reads (partition_id and replica_id need them)
+      out_ << "module";
+      const char* sep = " attributes {";
+      for (const char* key : {"mhlo.num_partitions", "mhlo.num_replicas"})
+        if (const BAttr* v = find(dict, key); v && v->kind == BAttr::Int) {
+          out_ << sep << key << " = " << v->i << " : i32";
+          sep = ", ";
+        }
+      out_ << (sep[0] == ',' ? "} {\n" : " {\n");
       Cursor rc = regionCursor(c);
       Cursor& use = (isolated && version_ >= 2) ? rc : c;
       if (isolated) scopes_.emplace_back();

@@ -128,6 +128,7 @@ struct Func {
 
 struct Module {
   std::vector<std::unique_ptr<Func>> funcs;
+  int64_t numPartitions = 1, numReplicas = 1;   // mhlo.num_partitions / mhlo.num_replicas of the module (1 when absent)
   Func* find(const std::string& name) const {
     for (auto& f : funcs) if (f->name == name) return f.get();
     return nullptr;
@@ -148,6 +149,7 @@ std::string vhloBytecodeToStableHLOText(const char* data, size_t size);
 // Passes (passes.cc)
 void inlineCalls(Module& m);          // replaces every "call" by the callee body
 void lowerIntegerDots(Module& m);    // integer / boolean dot_general -> broadcast, multiply, reduce
+void lowerSingleDeviceOps(Module& m);  // one-device all_reduce -> operands, partition_id / replica_id -> 0, tokens -> f32 scalar placeholders
 void lowerTopK(Module& m);           // chlo.top_k -> stable descending sort of (value, position) + slice
 void lowerRng(Module& m);            // rng_bit_generator -> counter update + threefry2x32 as plain ui32 ops
 void lowerWindowOps(Module& m);      // reduce_window / select_and_scatter with small windows -> pad, strided slices, elementwise ops

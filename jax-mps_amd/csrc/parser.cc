@@ -86,12 +86,12 @@ class Parser {
       wrapped = true;
       ws();
       if (peekc() == '@') { ++i_; ident(); }
-      if (eatWord("attributes")) skipBalanced('{', '}');
+      if (eatWord("attributes")) moduleAttributes(*m);
       expect("{");
     } else if (peek("builtin.module")) {
       i_ += 14;
       wrapped = true;
-      if (eatWord("attributes")) skipBalanced('{', '}');
+      if (eatWord("attributes")) moduleAttributes(*m);
       expect("{");
     }
     skipAliasLines();
@@ -264,6 +264,23 @@ class Parser {
       }
     }
   }
+  // the module's attribute dictionary: only the partition and replica counts matter here
+  void moduleAttributes(Module& m) {
+    ws();
+    const size_t from = i_;
+    skipBalanced('{', '}');
+    const std::string text(s_ + from, s_ + i_);
+    auto count = [&](const char* key, int64_t& out) {
+      size_t at = text.find(key);
+      if (at == std::string::npos) return;
+      at = text.find('=', at);
+      if (at == std::string::npos) return;
+      out = strtoll(text.c_str() + at + 1, nullptr, 10);
+    };
+    count("mhlo.num_partitions", m.numPartitions);
+    count("mhlo.num_replicas", m.numReplicas);
+  }
+
   void skipBalanced(char open, char close) {
     ws();
     if (i_ >= n_ || s_[i_] != open) fail(std::string("expected '") + open + "'");

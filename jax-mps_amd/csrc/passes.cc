@@ -1012,6 +1012,74 @@ void lowerTopKIn(Region& r, int& nextId) {
 
 }  // namespace
 
+// Ops of programs written for several devices that still reach a single-device plugin (reference:
+// ops/collectives.cc:15-84 and ops/control_flow.cc:2266-2288).  With one device an all_reduce returns its operands,
+// the partition and replica ids are zero, and a token, which only orders side effects that run in program order here
+// anyway, is a float32 scalar placeholder (zero), also where it crosses the function boundary.  Anything that names
+// more than one device is a compile error: treating it as the identity would silently give wrong values.
+namespace {
+
+void retypeTokens(Region& r) {
+  for (auto& a : r.args) if (a->type.dt == DType::Token) { a->type.dt = DType::F32; a->type.dims.clear(); }
+  for (auto& o : r.ops) {
+    for (auto& v : o->results) if (v->type.dt == DType::Token) { v->type.dt = DType::F32; v->type.dims.clear(); }
+    for (auto& sub : o->regions) retypeTokens(*sub);
+  }
+}
+
+void lowerSingleDeviceOpsIn(Module& m, Region& r, int& nextId, VMap& repl) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) lowerSingleDeviceOpsIn(m, *sub, nextId, repl);
+    if (op->name == "all_reduce") {
+      if (op->has("replica_groups")) {
+        // members per group: the last dimension of a rank-2 tensor, else the element count (a flat list is one group)
+        const Attr& a = op->attrs.at("replica_groups");
+        int64_t perGroup = 0;
+        if (a.dense) perGroup = a.dense->type.rank() >= 2 ? a.dense->type.dims.back() : a.dense->type.numel();
+        else if (a.kind == Attr::Ints) perGroup = (int64_t)a.ints.size();
+        else throw CompileError("stablehlo.all_reduce: replica_groups is not a tensor of integers");
+        if (perGroup > 1) throw CompileError("stablehlo.all_reduce: multi-device all_reduce is not supported");
+      }
+      if (op->operands.size() != op->results.size()) throw CompileError("stablehlo.all_reduce: operand/result count mismatch");
+      for (size_t i = 0; i < op->results.size(); ++i) repl[op->results[i].get()] = op->operands[i];
+      r.ops.erase(r.ops.begin() + k);
+      --k;
+      continue;
+    }
+    const bool id = op->name == "partition_id" || op->name == "replica_id";
+    const bool token = op->name == "create_token" || op->name == "after_all";
+    if (!id && !token) continue;
+    if (op->name == "partition_id" && m.numPartitions != 1) throw CompileError("stablehlo.partition_id: multi-partition execution is not supported");
+    if (op->name == "replica_id" && m.numReplicas != 1) throw CompileError("stablehlo.replica_id: multi-replica execution is not supported");
+    if (op->results.size() != 1) throw CompileError("stablehlo." + op->name + ": expected one result");
+    TensorType t = op->results[0]->type;
+    if (token) { t.dt = DType::F32; t.dims.clear(); }
+    if (id && (t.rank() != 0 || !isInt(t.dt))) throw CompileError("stablehlo." + op->name + ": result must be a scalar integer tensor");
+    Rewriter rw{r, nextId, op->line, {}};
+    const uint64_t zero = 0;   // all-zero bytes are 0 of every integer type and 0.0f
+    Value* c = rw.splat(t.dt, {}, &zero);
+    repl[op->results[0].get()] = c;
+    size_t nIns = rw.made.size();
+    r.ops.erase(r.ops.begin() + k);
+    r.ops.insert(r.ops.begin() + k, std::make_move_iterator(rw.made.begin()), std::make_move_iterator(rw.made.end()));
+    k += nIns - 1;
+  }
+}
+
+}  // namespace
+
+void lowerSingleDeviceOps(Module& m) {
+  Func* f = m.main();
+  if (!f) return;
+  int nextId = maxValueId(f->body) + 1;
+  VMap repl;
+  lowerSingleDeviceOpsIn(m, f->body, nextId, repl);
+  if (!repl.empty()) applyReplacements(f->body, repl);
+  retypeTokens(f->body);
+  for (auto& t : f->resultTypes) if (t.dt == DType::Token) { t.dt = DType::F32; t.dims.clear(); }
+}
+
 void lowerTopK(Module& m) {
   Func* f = m.main();
   if (!f) return;

@@ -2334,6 +2334,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
     prog->paramDonation.resize(mainFn->body.args.size(), -1);
   }
   inlineCalls(*module);
+  lowerSingleDeviceOps(*module);
   lowerIntegerDots(*module);
   lowerGeneralScatters(*module);
   lowerWindowOps(*module);

@@ -447,7 +447,7 @@ class _P:
             if self.eat("@"):
                 self.ident()
             if self.eat("attributes"):
-                self.attr_dict()
+                self.module_attributes = self.attr_dict()
             self.expect("{")
         self.skip_alias_lines()
         while True:
@@ -1025,13 +1025,20 @@ def parse(text: str) -> Dict[str, Func]:
     return _P(text).module()
 
 
+def parse_with_attributes(text: str):
+    """The functions of a module and the attribute dictionary written after `module @name attributes`."""
+    p = _P(text)
+    funcs = p.module()
+    return funcs, getattr(p, "module_attributes", {})
+
+
 # ----------------------------------------------------------------------------
 # interpreter
 # ----------------------------------------------------------------------------
 def _cast_result(a: np.ndarray, t: TType, keep_shape: bool = False) -> np.ndarray:
     a = np.asarray(a)
     if t.dtype == "token":
-        return a
+        return np.asarray(a, dtype=np.float32).reshape(())
     want = _NP[t.dtype]
     if a.dtype != want:
         a = a.astype(want)
@@ -1042,12 +1049,17 @@ def _cast_result(a: np.ndarray, t: TType, keep_shape: bool = False) -> np.ndarra
     return a
 
 
+def _boundary_type(t: TType):
+    """Type of an argument or result of main as a caller sees it: a token travels as an f32 scalar."""
+    return ((), "f32") if t.dtype == "token" else (t.shape, t.dtype)
+
+
 class Oracle:
     def __init__(self, text: str, accum: str = "f64", round_intermediates: bool = True):
         """`round_intermediates=False` keeps bf16-typed intermediate results unrounded (float32 carriers of the
         float64 arithmetic): the value the program's formulas define, against which the rounding noise of any
         bf16 evaluation order can be measured.  Arguments and dense constants keep their bf16 values."""
-        self.funcs = parse(text)
+        self.funcs, self.module_attributes = parse_with_attributes(text)
         self.accum = np.float64 if accum == "f64" else np.float32
         self.round_intermediates = round_intermediates
         self.main = self.funcs["main"]
@@ -1061,11 +1073,11 @@ class Oracle:
 
     @property
     def arg_types(self):
-        return [(t.shape, t.dtype) for t in self.main.body.arg_types]
+        return [_boundary_type(t) for t in self.main.body.arg_types]
 
     @property
     def result_types(self):
-        return [(t.shape, t.dtype) for t in self.main.result_types]
+        return [_boundary_type(t) for t in self.main.result_types]
 
     # -- engine
     def _run_region(self, region: Region, args, outer_env, vectorized: bool = False) -> List[np.ndarray]:
@@ -1829,6 +1841,54 @@ class Oracle:
         return self._run_region(f.body, ins, {})
 
     def op_optimization_barrier(self, op, ins, env): return list(ins)
+
+    # -- one device only: collectives pass through, ids are zero, tokens are scalar placeholders
+    def _module_count(self, key):
+        v = self.module_attributes.get(key, 1)
+        if isinstance(v, tuple):
+            v = v[0]
+        return int(np.asarray(v).reshape(-1)[0])
+
+    def op_all_reduce(self, op, ins, env):
+        """stablehlo.all_reduce over one device forwards its operands; a replica group with more than one member
+        is an error (reference: src/pjrt_plugin/ops/collectives.cc:20-48: the last dimension of a rank-2
+        `replica_groups`, else its element count, decides)."""
+        groups = op.attrs.get("replica_groups")
+        if groups is not None:
+            g = np.asarray(groups[0] if isinstance(groups, tuple) else groups)
+            if g.size and (g.shape[-1] if g.ndim >= 2 else g.size) > 1:
+                raise ValueError("stablehlo.all_reduce: multi-device all_reduce is not supported")
+        if len(ins) != len(op.results):
+            raise ValueError("stablehlo.all_reduce: operand/result count mismatch")
+        return list(ins)
+
+    def op_partition_id(self, op, ins, env):
+        """Zero, of the result's integer type, when the module declares one partition (reference:
+        src/pjrt_plugin/ops/collectives.cc:56-79)."""
+        if self._module_count("mhlo.num_partitions") != 1:
+            raise ValueError("stablehlo.partition_id: multi-partition execution is not supported")
+        t = op.out_types[0]
+        if t.shape != ():
+            raise ValueError("stablehlo.partition_id: result must be a scalar tensor")
+        return np.zeros((), dtype=_NP[t.dtype])
+
+    def op_replica_id(self, op, ins, env):
+        """The replica counterpart of partition_id (the reference registers no handler for it)."""
+        if self._module_count("mhlo.num_replicas") != 1:
+            raise ValueError("stablehlo.replica_id: multi-replica execution is not supported")
+        t = op.out_types[0]
+        if t.shape != ():
+            raise ValueError("stablehlo.replica_id: result must be a scalar tensor")
+        return np.zeros((), dtype=_NP[t.dtype])
+
+    def op_create_token(self, op, ins, env):
+        """A token carries no data; it is the f32 scalar 0 wherever a value must stand for it, also as an argument
+        or result of main (reference: src/pjrt_plugin/ops/control_flow.cc:2266-2288)."""
+        return np.float32(0.0).reshape(())
+
+    def op_after_all(self, op, ins, env):
+        """A fresh placeholder; the operand tokens are ignored (reference: ops/control_flow.cc:2283-2288)."""
+        return np.float32(0.0).reshape(())
 
     def op_sort(self, op, ins, env):
         """stablehlo.sort: the comparator region decides, ties keep their order (the reference sorts by the first

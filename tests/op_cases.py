@@ -49,6 +49,14 @@ def case(name, fn, *inputs, dtypes=None, exact=False):
     make.case_name = name
     _cases.append(make)
 
+def text_case(name, text, *inputs, dtypes=None, exact=False):
+    """A program given as StableHLO text (for forms the builder does not write)."""
+    def make():
+        dts = list(dtypes) if dtypes else [_MLIR[np.asarray(a).dtype] for a in inputs]
+        return Case(name, text, [np.asarray(a) for a in inputs], dts, exact)
+    make.case_name = name
+    _cases.append(make)
+
 
 def rng(seed):
     return np.random.default_rng(seed)
@@ -708,6 +716,95 @@ def _case_in_dynamic_loop(b, sel, x, n):
 
 
 case("case-inside-dynamic-loop", _case_in_dynamic_loop, np.array([0, 1, 1, 0, 1, 1, 1, 0, 0, 1], np.int32), f32(2405, 6), np.int32(7), exact=True)
+
+# ------------------------------------------------------------------ one device: collectives, ids, tokens
+# (reference tests: tests/configs/collectives.py:35-56 run pmap(pmean) and pmap(axis_index) over one device;
+# tests/test_control_flow_compile.py:95-133 pass tokens into, through and out of jitted functions.  The programs
+# below are the text such functions lower to, written by hand.)
+text_case("all-reduce-one-device-pmean", """module @pmap_f attributes {mhlo.num_partitions = 1 : i32, mhlo.num_replicas = 1 : i32} {
+  func.func public @main(%arg0: tensor<1x4xf32>) -> tensor<1x4xf32> {
+    %0 = stablehlo.reshape %arg0 : (tensor<1x4xf32>) -> tensor<4xf32>
+    %1 = "stablehlo.all_reduce"(%0) <{replica_groups = dense<0> : tensor<1x1xi64>}> ({
+    ^bb0(%arg1: tensor<f32>, %arg2: tensor<f32>):
+      %5 = stablehlo.add %arg1, %arg2 : tensor<f32>
+      stablehlo.return %5 : tensor<f32>
+    }) : (tensor<4xf32>) -> tensor<4xf32>
+    %cst = stablehlo.constant dense<1.000000e+00> : tensor<f32>
+    %2 = stablehlo.broadcast_in_dim %cst, dims = [] : (tensor<f32>) -> tensor<4xf32>
+    %3 = stablehlo.divide %1, %2 : tensor<4xf32>
+    %4 = stablehlo.reshape %3 : (tensor<4xf32>) -> tensor<1x4xf32>
+    return %4 : tensor<1x4xf32>
+  }
+}
+""", f32(2501, 1, 4), exact=True)
+
+text_case("all-reduce-one-device-two-operands", """module @jit_f attributes {mhlo.num_partitions = 1 : i32, mhlo.num_replicas = 1 : i32} {
+  func.func public @main(%arg0: tensor<3x5xf32>, %arg1: tensor<7xi32>) -> (tensor<3x5xf32>, tensor<7xi32>) {
+    %0 = stablehlo.multiply %arg0, %arg0 : tensor<3x5xf32>
+    %1:2 = "stablehlo.all_reduce"(%0, %arg1) <{channel_handle = #stablehlo.channel_handle<handle = 1, type = 1>, replica_groups = dense<0> : tensor<1x1xi64>, use_global_device_ids}> ({
+    ^bb0(%arg2: tensor<f32>, %arg3: tensor<f32>):
+      %3 = stablehlo.maximum %arg2, %arg3 : tensor<f32>
+      stablehlo.return %3 : tensor<f32>
+    }) : (tensor<3x5xf32>, tensor<7xi32>) -> (tensor<3x5xf32>, tensor<7xi32>)
+    %2 = stablehlo.add %1#1, %1#1 : tensor<7xi32>
+    return %1#0, %2 : tensor<3x5xf32>, tensor<7xi32>
+  }
+}
+""", f32(2502, 3, 5), i32(2503, 7), exact=True)
+
+text_case("partition-id-axis-index-zero", """module @pmap_f attributes {mhlo.num_partitions = 1 : i32, mhlo.num_replicas = 1 : i32} {
+  func.func public @main(%arg0: tensor<1x4xi32>) -> (tensor<1x4xi32>, tensor<ui32>) {
+    %0 = stablehlo.reshape %arg0 : (tensor<1x4xi32>) -> tensor<4xi32>
+    %1 = stablehlo.partition_id : tensor<ui32>
+    %2 = stablehlo.convert %1 : (tensor<ui32>) -> tensor<i32>
+    %3 = stablehlo.broadcast_in_dim %2, dims = [] : (tensor<i32>) -> tensor<4xi32>
+    %4 = stablehlo.add %0, %3 : tensor<4xi32>
+    %5 = stablehlo.reshape %4 : (tensor<4xi32>) -> tensor<1x4xi32>
+    %6 = stablehlo.replica_id : tensor<ui32>
+    return %5, %6 : tensor<1x4xi32>, tensor<ui32>
+  }
+}
+""", np.arange(4, dtype=np.int32).reshape(1, 4), exact=True)
+
+text_case("token-created-merged-and-returned", """module @jit_f {
+  func.func public @main(%arg0: tensor<f32>, %arg1: !stablehlo.token) -> (tensor<f32>, !stablehlo.token) {
+    %0 = stablehlo.create_token : !stablehlo.token
+    %1 = stablehlo.after_all %0, %arg1 : !stablehlo.token
+    %cst = stablehlo.constant dense<1.000000e+00> : tensor<f32>
+    %2 = stablehlo.add %arg0, %cst : tensor<f32>
+    return %2, %1 : tensor<f32>, !stablehlo.token
+  }
+}
+""", np.float32(3.0), np.float32(7.0), exact=True)
+
+text_case("token-argument-returned-as-is", """module @jit_f {
+  func.func public @main(%arg0: !stablehlo.token, %arg1: tensor<6xf32>) -> (!stablehlo.token, tensor<6xf32>) {
+    %0 = stablehlo.multiply %arg1, %arg1 : tensor<6xf32>
+    return %arg0, %0 : !stablehlo.token, tensor<6xf32>
+  }
+}
+""", np.float32(5.0), f32(2504, 6), exact=True)
+
+text_case("token-carried-by-a-loop", """module @jit_f {
+  func.func public @main(%arg0: tensor<4xf32>) -> (tensor<4xf32>, !stablehlo.token) {
+    %tok = stablehlo.create_token : !stablehlo.token
+    %c0 = stablehlo.constant dense<0> : tensor<i32>
+    %0:3 = stablehlo.while(%iterArg = %c0, %iterArg_0 = %arg0, %iterArg_1 = %tok) : tensor<i32>, tensor<4xf32>, !stablehlo.token
+     cond {
+      %c3 = stablehlo.constant dense<3> : tensor<i32>
+      %1 = stablehlo.compare  LT, %iterArg, %c3,  SIGNED : (tensor<i32>, tensor<i32>) -> tensor<i1>
+      stablehlo.return %1 : tensor<i1>
+    } do {
+      %c1 = stablehlo.constant dense<1> : tensor<i32>
+      %1 = stablehlo.add %iterArg, %c1 : tensor<i32>
+      %2 = stablehlo.add %iterArg_0, %iterArg_0 : tensor<4xf32>
+      %3 = stablehlo.after_all %iterArg_1 : !stablehlo.token
+      stablehlo.return %1, %2, %3 : tensor<i32>, tensor<4xf32>, !stablehlo.token
+    }
+    return %0#1, %0#2 : tensor<4xf32>, !stablehlo.token
+  }
+}
+""", f32(2505, 4), exact=True)
 
 
 def all_cases() -> List[Case]:

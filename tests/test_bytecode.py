@@ -22,7 +22,9 @@ TOOL = ROOT / "jax-mps_amd" / "mi355x-aot"
 # control-flow and window ops; chlo ops are not part of a vhlo artifact)
 CASES = ["binary-add", "compare-f32-LT", "compare-totalorder", "select", "convert-f32-i32", "while-nested", "while-scan-cumsum",
          "while-dynamic-collatz-27", "case-index-1", "case-inside-counted-loop", "dot-sum-two-products-bias", "int-shifts",
-         "while-swapped-carries", "maxpool-3x3-s2-pad1", "maxpool-grad-ties", "round-half", "unary-specials", "bool-logic"]
+         "while-swapped-carries", "maxpool-3x3-s2-pad1", "maxpool-grad-ties", "round-half", "unary-specials", "bool-logic",
+         "all-reduce-one-device-pmean", "all-reduce-one-device-two-operands", "partition-id-axis-index-zero",
+         "token-created-merged-and-returned", "token-argument-returned-as-is", "token-carried-by-a-loop"]
 
 
 def _to_text(bytecode: bytes, *flags) -> subprocess.CompletedProcess:
@@ -83,6 +85,21 @@ def test_bytecode_plans_like_its_text():
     Path(f.name).unlink()
     assert a.returncode == 0 and b.returncode == 0, a.stderr[-500:]
     assert a.stdout.split(":", 1)[1] == b.stdout.split(":", 1)[1]       # same ops, steps, kernels, arena
+
+
+def test_device_counts_and_replica_groups_travel():
+    """The module's device counts (builtin attributes of builtin.module) and the shape of replica_groups reach the
+    compiler from bytecode too: the multi-device errors fire as they do for text."""
+    c = op_cases.get_case("partition-id-axis-index-zero")
+    r = _to_text(to_vhlo_bytecode(c.text), "--bytecode-to-text")
+    assert "module attributes {mhlo.num_partitions = 1 : i32, mhlo.num_replicas = 1 : i32} {" in r.stdout
+    r = _to_text(to_vhlo_bytecode(c.text.replace("mhlo.num_partitions = 1", "mhlo.num_partitions = 8")))
+    assert r.returncode != 0 and "multi-partition execution is not supported" in r.stderr
+    c = op_cases.get_case("all-reduce-one-device-pmean")
+    r = _to_text(to_vhlo_bytecode(c.text.replace("dense<0> : tensor<1x1xi64>", "dense<[[0, 1]]> : tensor<1x2xi64>")))
+    assert r.returncode != 0 and "multi-device all_reduce is not supported" in r.stderr
+    r = _to_text(to_vhlo_bytecode(c.text.replace("dense<0> : tensor<1x1xi64>", "dense<[[0], [1]]> : tensor<2x1xi64>")))
+    assert r.returncode == 0, r.stderr
 
 
 def test_donation_attributes_travel():

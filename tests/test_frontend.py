@@ -81,6 +81,37 @@ def test_missing_required_attributes_are_compile_errors():
     assert r.returncode != 0 and "dims" in r.stderr
 
 
+def test_collectives_and_ids_of_more_than_one_device_are_compile_errors():
+    """One device only: an all_reduce whose replica groups hold more than one member, a partition_id in a module of
+    several partitions and a replica_id in a module of several replicas fail at compile time with the reference's
+    messages (src/pjrt_plugin/ops/collectives.cc:22-33, 58-66) instead of computing on one device's share."""
+    good = op_cases.get_case("all-reduce-one-device-two-operands").text
+    assert plan(good).returncode == 0
+    r = plan(good.replace("dense<0> : tensor<1x1xi64>", "dense<[[0, 1]]> : tensor<1x2xi64>"))
+    assert r.returncode != 0 and "multi-device all_reduce is not supported" in r.stderr
+    r = plan(good.replace("dense<0> : tensor<1x1xi64>", "dense<[0, 1]> : tensor<2xi64>"))
+    assert r.returncode != 0 and "multi-device all_reduce is not supported" in r.stderr
+    assert plan(good.replace("dense<0> : tensor<1x1xi64>", "dense<[[0], [1]]> : tensor<2x1xi64>")).returncode == 0   # groups of one
+    ids = op_cases.get_case("partition-id-axis-index-zero").text
+    assert plan(ids).returncode == 0
+    r = plan(ids.replace("mhlo.num_partitions = 1", "mhlo.num_partitions = 2"))
+    assert r.returncode != 0 and "multi-partition execution is not supported" in r.stderr
+    r = plan(ids.replace("mhlo.num_replicas = 1", "mhlo.num_replicas = 4"))
+    assert r.returncode != 0 and "replica" in r.stderr
+    r = plan(ids.replace("stablehlo.partition_id : tensor<ui32>", "stablehlo.partition_id : tensor<1xui32>").replace("(tensor<ui32>) -> tensor<i32>", "(tensor<1xui32>) -> tensor<i32>"))
+    assert r.returncode != 0 and "scalar" in r.stderr
+
+
+def test_tokens_travel_as_scalar_placeholders():
+    """Tokens order side effects and carry no data; the plan holds no step for create_token or after_all and the
+    token results of main are f32 scalars (reference: src/pjrt_plugin/ops/control_flow.cc:2266-2288)."""
+    r = plan(op_cases.get_case("token-created-merged-and-returned").text, "--dump-plan")
+    assert r.returncode == 0, r.stderr
+    assert "token" not in r.stdout and "after_all" not in r.stdout
+    r = plan(op_cases.get_case("token-carried-by-a-loop").text, "--dump-plan")
+    assert r.returncode == 0 and "while while trip 3" in r.stdout
+
+
 def test_location_aliases_result_lists_and_composites_parse():
     text = """#loc1 = loc("x")
 module @jit_f attributes {mhlo.num_partitions = 1 : i32} {

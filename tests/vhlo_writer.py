@@ -15,10 +15,11 @@ from typing import Dict, List, Tuple
 
 import numpy as np
 
-from shlo_oracle import parse, f32_to_bf16_bits
+from shlo_oracle import parse_with_attributes, f32_to_bf16_bits
 
 # ---- code tables (mirror bytecode.cc) ------------------------------------------------------------------------------
-B_DICT, B_STRING, B_UNKNOWN_LOC = 1, 2, 15
+B_DICT, B_STRING, B_INTEGER, B_UNKNOWN_LOC = 1, 2, 8, 15
+BT_INTEGER = 0
 (A_ARRAY, A_BOOL, A_CMP_DIR, A_CMP_TYPE, A_API, A_DICT, A_FFT, A_FLOAT, A_INT, A_OOA, A_PRECISION, A_RNG_ALG, A_RNG_DIST, A_STRING, A_TENSOR,
  A_TRANSPOSE, A_TYPE, A_TYPE_EXT) = range(18)
 T_CODES = {"i1": 0, "bf16": 2, "f16": 3, "f32": 4, "f64": 5, "index": 9, "i8": 11, "i16": 12, "i32": 13, "i64": 14, "ui8": 16, "ui16": 17,
@@ -52,7 +53,9 @@ def with_flag(v: int, flag: bool) -> bytes:
 
 class Writer:
     def __init__(self, text: str, version: int = 6, isolated_funcs: bool = False, pack_bools: bool = True, module_properties: bool = False):
-        self.funcs = parse(text)
+        self.funcs, module_attributes = parse_with_attributes(text)
+        # builtin.module keeps its attributes as builtin ones; the device counts are the two the plugin reads
+        self.module_counts = [(k, int(module_attributes[k])) for k in ("mhlo.num_partitions", "mhlo.num_replicas") if k in module_attributes]
         self.version = version
         self.isolated_funcs = isolated_funcs
         self.module_properties = module_properties and version >= 5   # builtin.module carries native properties from version 5 on
@@ -241,6 +244,13 @@ class Writer:
             out["decomposition"] = self.a_str(str(a["decomposition"]).lstrip("@"))
             out["version"] = self.a_int(0, "i32")
             out["composite_attributes"] = self.a_dict([])
+        elif short == "all_reduce":
+            # vhlo.all_reduce_v1: replica_groups (tensor), channel_id (integer; 0 = no channel), use_global_device_ids (bool)
+            groups = a["replica_groups"]
+            out["replica_groups"] = self.a_tensor(np.asarray(groups[0] if isinstance(groups, tuple) else groups), "i64")
+            handle = a.get("channel_handle")
+            out["channel_id"] = self.a_int(handle[1]["handle"] if handle else 0)
+            out["use_global_device_ids"] = self.a_bool(flag(a.get("use_global_device_ids", False)))
         elif short == "call":
             out["callee"] = self.a_str(str(a["callee"]).lstrip("@"))
         elif a and short not in ("while", "case", "return", "optimization_barrier", "select", "clamp"):
@@ -258,6 +268,8 @@ class Writer:
                 for name, value in key[2]:
                     self.collect(("builtin", "string", name))
                     self.collect(value)
+            elif kind == "int":
+                self.type(key[3])
             self.attr(key)
             return
         kind = key[1]
@@ -307,6 +319,8 @@ class Writer:
                 return out
             if key[1] == "unknown_loc":
                 return varint(B_UNKNOWN_LOC)
+            if key[1] == "int":
+                return varint(B_INTEGER) + varint(tidx[key[3]]) + svarint(key[2])
             raise AssertionError(key)
         kind = key[1]
         if kind == "string":
@@ -331,6 +345,9 @@ class Writer:
 
     def encode_type(self, key, tidx) -> bytes:
         kind = key[1]
+        if key[0] == "builtin":
+            assert kind == "integer"
+            return varint(BT_INTEGER) + varint(key[2] << 2)      # width, signless
         if kind == "scalar":
             return varint(T_CODES[key[2]])
         if kind == "token":
@@ -427,9 +444,15 @@ class Writer:
             self.collect(dict_key)
             self.prepare_region(f.body, plans)
             func_plans.append((f, dict_key))
-        # final numbering: attributes grouped by dialect (builtin first, then vhlo), types are all vhlo
+        module_dict = None
+        if self.module_counts:
+            i32 = ("builtin", "integer", 32)
+            module_dict = ("builtin", "dict", tuple((k, ("builtin", "int", v, i32)) for k, v in self.module_counts))
+            self.collect(module_dict)
+        # final numbering: attributes and types grouped by dialect (builtin first, then vhlo)
         order = [k for k in self.attr_keys if k[0] == "builtin"] + [k for k in self.attr_keys if k[0] == "vhlo"]
         aidx = {k: i for i, k in enumerate(order)}
+        self.type_keys = [k for k in self.type_keys if k[0] == "builtin"] + [k for k in self.type_keys if k[0] == "vhlo"]
         tidx = {k: i for i, k in enumerate(self.type_keys)}
         loc = aidx[loc_key]
         attr_blobs = [self.encode_attr(k, aidx, tidx) for k in order]
@@ -461,8 +484,11 @@ class Writer:
         offset_sec += varint(0) + varint(nb) + b"".join(with_flag(len(b), True) for b in attr_blobs[:nb])
         if len(order) > nb:
             offset_sec += varint(1) + varint(len(order) - nb) + b"".join(with_flag(len(b), True) for b in attr_blobs[nb:])
-        if type_blobs:
-            offset_sec += varint(1) + varint(len(type_blobs)) + b"".join(with_flag(len(b), True) for b in type_blobs)
+        nbt = sum(1 for k in self.type_keys if k[0] == "builtin")
+        if nbt:
+            offset_sec += varint(0) + varint(nbt) + b"".join(with_flag(len(b), True) for b in type_blobs[:nbt])
+        if len(type_blobs) > nbt:
+            offset_sec += varint(1) + varint(len(type_blobs) - nbt) + b"".join(with_flag(len(b), True) for b in type_blobs[nbt:])
         attr_sec = b"".join(attr_blobs) + b"".join(type_blobs)
         # IR: top-level block with the module op, whose (isolated) region is a section of its own from version 2 on
         module_region = varint(1) + varint(0) + with_flag(len(func_plans), False)
@@ -471,7 +497,9 @@ class Writer:
             module_region += with_flag(1, self.isolated_funcs)
             body = self.emit_region(f.body, plans, {}, 0, aidx, tidx, loc)
             module_region += self.section(4, body) if (self.isolated_funcs and self.version >= 2) else body
-        ir = with_flag(1, False) + varint(self.op_names[("builtin", "module")]) + bytes([16 | (0x40 if self.module_properties else 0)]) + varint(loc)
+        ir = with_flag(1, False) + varint(self.op_names[("builtin", "module")]) + bytes([16 | (1 if module_dict else 0) | (0x40 if self.module_properties else 0)]) + varint(loc)
+        if module_dict:
+            ir += varint(aidx[module_dict])
         if self.module_properties:
             ir += varint(0)                  # index into the properties section
         ir += with_flag(1, True)
