@@ -167,8 +167,21 @@ void renameUnaryCustomCalls(Region& r) {
   static const std::set<std::string> unary = {"asin", "acos", "atan", "sinh", "cosh", "asinh", "acosh", "atanh", "erf", "erf_inv"};
   for (auto& o : r.ops) {
     for (auto& sub : o->regions) renameUnaryCustomCalls(*sub);
-    if (o->name != "custom_call" || o->operands.size() != 1 || o->results.size() != 1) continue;
+    if (o->name != "custom_call") continue;
     const std::string& t = o->str("target");
+    if (t == "mhlo.topk") {
+      // the older spelling of chlo.top_k: k is the extent of the results' last dim (reference: ops/control_flow.cc:1461-1477)
+      if (o->operands.size() != 1 || o->results.size() != 2) throw CompileError("stablehlo.custom_call mhlo.topk: expected 1 input and 2 outputs");
+      const TensorType& vt = o->results[0]->type;
+      if (vt.rank() < 1) throw CompileError("stablehlo.custom_call mhlo.topk: the results must have at least one dim");
+      Attr k;
+      k.kind = Attr::Int;
+      k.i = vt.dims.back();
+      o->attrs["k"] = k;
+      o->name = "chlo.top_k";
+      continue;
+    }
+    if (o->operands.size() != 1 || o->results.size() != 1) continue;
     if (t.rfind("mhlo.", 0) == 0 && unary.count(t.substr(5))) o->name = "chlo." + t.substr(5);
   }
 }

@@ -1975,6 +1975,9 @@ class Oracle:
         tgt = op.attrs.get("call_target_name")
         if tgt in ("Sharding", "SPMDFullToShardShape", "SPMDShardToFullShape"):
             return ins[0]
+        if tgt == "mhlo.topk":      # the older spelling of chlo.top_k (reference: ops/control_flow.cc:1461-1477)
+            op.attrs["k"] = op.out_types[0].shape[-1]
+            return self.op_chlo_top_k(op, ins, env)
         if isinstance(tgt, str) and tgt.startswith("mhlo.") and hasattr(self, "op_chlo_" + tgt[5:]) and len(ins) == 1:
             return getattr(self, "op_chlo_" + tgt[5:])(op, ins, env)
         raise NotImplementedError(f"oracle: custom_call {tgt}")

@@ -860,6 +860,13 @@ case("top-k-transposed-input", lambda b, x: list(b.top_k(b.transpose(x, [2, 1, 0
 case("top-k-equals-size", lambda b, x: list(b.top_k(x, 8)), f32(2135, 4, 8), exact=True)
 case("top-k-ties-lowest-index-first", lambda b, x: list(b.top_k(x, 6)), _with_ties(2136, 5, 40), exact=True)
 case("top-k-nan-first", lambda b, x: list(b.top_k(x, 4)), _SORT_NAN, exact=True)
+text_case("top-k-custom-call-spelling", """module @jit_f {
+  func.func public @main(%arg0: tensor<3x12xf32>) -> (tensor<3x4xf32>, tensor<3x4xi32>) {
+    %0:2 = stablehlo.custom_call @mhlo.topk(%arg0) {mhlo.attributes = {k = 4 : i64, largest = true}, mhlo.version = 1 : i64} : (tensor<3x12xf32>) -> (tensor<3x4xf32>, tensor<3x4xi32>)
+    return %0#0, %0#1 : tensor<3x4xf32>, tensor<3x4xi32>
+  }
+}
+""", f32(2138, 3, 12), exact=True)
 case("top-k-int32", lambda b, x: list(b.top_k(x, 7)), i32(2137, 3, 100), exact=True)
 case("top-k-vocabulary-row", lambda b, x: list(b.top_k(x, 50)), f32(2138, 2, 8000), exact=True)
 
