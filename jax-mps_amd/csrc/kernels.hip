@@ -544,6 +544,100 @@ __global__ void __launch_bounds__(256) radix_scatter(const u32* __restrict__ key
   }
 }
 
+// Up to 8192 updates (the benchmark's embedding batch) are sorted by one workgroup in LDS: the seven launches of
+// the general path cost more in launch latency than the sort itself.  1024 lanes hold eight (key, update number)
+// pairs each, pair (w, k, lane) at index w * 512 + k * 64 + lane.  One pass per 8-bit digit: a wavefront ranks its
+// 64 pairs of a round among themselves with ballots and keeps a running count per digit in its own column of
+// cnt[digit][wave]; an exclusive scan of cnt in (digit, wave) order gives every (digit, wave) its first output
+// position; pairs are written to LDS at their position and read back in index order.  Equal digits keep their
+// index order in every pass, so the sort is stable.  Slots past n hold key 0xFFFFFFFF: their digits are 255 in
+// every pass and they start behind every real pair, so they end behind every real pair.
+constexpr int kSmallSort = 8192;
+
+__global__ void __launch_bounds__(1024) scatter_sort_small(const void* idx, int idxBytes, int n, long long rows, int bits,
+                                                           u32* __restrict__ keysOut, u32* __restrict__ valsOut) {
+  __shared__ u32 keysL[kSmallSort];
+  __shared__ u16 valsL[kSmallSort];
+  __shared__ u16 cnt[256][16];
+  __shared__ u32 waveTotal[16];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  u32 key[8], val[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int i = w * 512 + k * 64 + lane;
+    val[k] = (u32)i;
+    key[k] = 0xFFFFFFFFu;
+    if (i < n) {
+      long long r = idxBytes == 8 ? ((const long long*)idx)[i] : (long long)((const int*)idx)[i];
+      key[k] = (r < 0 || r >= rows) ? (u32)rows : (u32)r;   // rows = "dropped", sorts behind every row
+    }
+  }
+  for (int shift = 0; shift < bits; shift += 8) {
+    ((u32*)&cnt[0][0])[threadIdx.x] = 0;
+    ((u32*)&cnt[0][0])[threadIdx.x + 1024] = 0;
+    __syncthreads();
+    u32 local[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const u32 digit = (key[k] >> shift) & 255u;
+      unsigned long long peers = ~0ull;
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const unsigned long long m = __ballot((digit >> b) & 1u);
+        peers &= ((digit >> b) & 1u) ? m : ~m;
+      }
+      const unsigned long long lower = peers & ((1ull << lane) - 1ull);
+      const u32 before = cnt[digit][w];                     // pairs of this digit in this wavefront's earlier rounds
+      local[k] = before + (u32)__popcll(lower);
+      __builtin_amdgcn_wave_barrier();                      // every lane has read the count before its leader moves it on
+      if (lower == 0) cnt[digit][w] = (u16)(before + (u32)__popcll(peers));
+      __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    // exclusive scan of the 4096 counts in (digit, wave) order: four per lane, wavefront scan, wavefront totals
+    u16* flat = &cnt[0][0];
+    const u32 c0 = flat[4 * threadIdx.x], c1 = flat[4 * threadIdx.x + 1], c2 = flat[4 * threadIdx.x + 2], c3 = flat[4 * threadIdx.x + 3];
+    const u32 mine = c0 + c1 + c2 + c3;
+    u32 incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const u32 up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    if (lane == 63) waveTotal[w] = incl;
+    __syncthreads();
+    u32 base = incl - mine;
+    for (int q = 0; q < w; ++q) base += waveTotal[q];
+    flat[4 * threadIdx.x] = (u16)base;
+    flat[4 * threadIdx.x + 1] = (u16)(base + c0);
+    flat[4 * threadIdx.x + 2] = (u16)(base + c0 + c1);
+    flat[4 * threadIdx.x + 3] = (u16)(base + c0 + c1 + c2);
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const u32 pos = cnt[(key[k] >> shift) & 255u][w] + local[k];
+      keysL[pos] = key[k];
+      valsL[pos] = (u16)val[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int i = w * 512 + k * 64 + lane;
+      key[k] = keysL[i];
+      val[k] = valsL[i];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int i = w * 512 + k * 64 + lane;
+    if (i < n) {
+      keysOut[i] = key[k];
+      valsOut[i] = val[k];
+    }
+  }
+}
+
 template <typename T>
 struct ScatterOps;
 template <>
@@ -604,7 +698,38 @@ struct Bf16 {
   static __device__ __forceinline__ A apply(int kind, A a, S u) { return bf2f(f2bf(ScatterOps<float>::apply(kind, a, bf2f(u)))); }
 };
 
-constexpr int kLongSegment = 16;   // runs at least this long go to the column-parallel kernel
+// Ends of the run of `key` around a position known to hold it, in sorted keys.  Every lane of a wavefront probes
+// one position per step (64-way search: three dependent loads for 8192 keys where a bisection needs thirteen);
+// all lanes return the same value.
+__device__ __forceinline__ long long runHead(const u32* __restrict__ keys, long long p, u32 key, int lane) {
+  long long lo = 0, hi = p;                 // the first position holding `key` lies in [lo, hi]; keys[hi] == key
+  while (lo < hi) {
+    const long long step = (hi - lo + 62) / 63;                // 63 steps reach hi: the last lane always answers
+    const long long pos = lo + lane * step;
+    const bool here = pos >= hi || keys[pos] == key;           // sorted: positions holding `key` form a suffix of [lo, hi]
+    const int f = __ffsll((long long)__ballot(here)) - 1;      // lane 63 has pos >= hi, so f >= 0
+    const long long top = lo + f * step;
+    lo = f > 0 ? top - step + 1 : lo;
+    hi = top < hi ? top : hi;
+  }
+  return lo;
+}
+__device__ __forceinline__ long long runLast(const u32* __restrict__ keys, long long p, long long n, u32 key, int lane) {
+  long long lo = p, hi = n - 1;             // the last position holding `key` lies in [lo, hi]; keys[lo] == key
+  while (lo < hi) {
+    const long long step = (hi - lo + 62) / 63;
+    const long long pos = hi - lane * step;
+    const bool here = pos <= lo || keys[pos] == key;           // positions holding `key` form a prefix of [lo, hi]
+    const int f = __ffsll((long long)__ballot(here)) - 1;
+    const long long bottom = hi - f * step;
+    hi = f > 0 ? bottom + step - 1 : hi;
+    lo = bottom > lo ? bottom : lo;
+  }
+  return lo;
+}
+
+constexpr int kLongSegment = 16;   // runs at least this long go to the column-parallel kernels
+constexpr int kHugeSegment = 256;  // runs at least this long go to the narrow-column kernel with deep prefetch
 
 template <typename P, int C>
 __device__ __forceinline__ void foldShortRun(typename P::A& acc, const u32* __restrict__ vals, int cnt, const typename P::S* __restrict__ updates,
@@ -620,8 +745,8 @@ __device__ __forceinline__ void foldShortRun(typename P::A& acc, const u32* __re
     if (q < cnt) acc = P::apply(kind, acc, u[q]);
 }
 
-// Short runs (the common case): one workgroup per run head and chunk of 256 columns; every
-// lane fetches all (< 16) updates of its column at once, then applies them in order.
+// Short runs (fewer than kLongSegment updates, the common case): one workgroup per run head and chunk of 256
+// columns; every lane fetches all updates of its column at once, then applies them in order.
 template <typename P>
 __global__ void __launch_bounds__(256) scatter_fold_short(const u32* __restrict__ keys, const u32* __restrict__ vals, long long n, long long rowElems,
                                                           int kind, typename P::S* __restrict__ result, const typename P::S* __restrict__ updates, u32 rows) {
@@ -646,46 +771,138 @@ __global__ void __launch_bounds__(256) scatter_fold_short(const u32* __restrict_
   result[(long long)key * rowElems + col] = P::store(acc);
 }
 
-template <typename P, int KIND>
+// Long runs (hot rows of a skewed index distribution) are bound by the latency of fetching their updates and by
+// the sequential fold (about 5 ns per update and column: one LDS read and one dependent operation), so the row is
+// cut into column chunks, one workgroup each, and many fetches are in flight: four wavefronts stage a round of
+// updates in LDS (32 independent loads per lane), then the first wavefront applies the staged values of its column
+// in order.  Runs of kLongSegment .. kHugeSegment - 1 updates use chunks of 64 columns and rounds of 128 updates
+// (scatter_fold_long); longer ones (the head of a Zipf distribution: a tenth of all updates go to one row) chunks of
+// 8 columns and rounds of 1024, a wavefront load covering eight updates, with the fetches of the next round issued
+// before the staged one is folded and the update numbers of round r + 1 fetched during round r - 1
+// (scatter_fold_huge).  A run of length >= L contains a multiple of L, so only those positions get a workgroup, and
+// the first of them inside the run does the work.
+//
+// Workgroup number = position * chunks + column chunk.  The column chunk is the fast index because workgroups with
+// neighbouring numbers go to different XCDs and shader engines: with the position as the fast index, the few
+// workgroups that find work (one run's chunks) all landed on the eight CUs of one shader engine and ran in turns.
+template <typename P, int KIND, int STRIDE>
 __device__ __forceinline__ void foldStaged(typename P::A& acc, const typename P::S* column, int m) {
   int r = 0;
   for (; r + 16 <= m; r += 16) {
     typename P::S v[16];
 #pragma unroll
-    for (int q = 0; q < 16; ++q) v[q] = column[(r + q) * 64];
+    for (int q = 0; q < 16; ++q) v[q] = column[(r + q) * STRIDE];
 #pragma unroll
     for (int q = 0; q < 16; ++q) acc = P::apply(KIND, acc, v[q]);
   }
-  for (; r < m; ++r) acc = P::apply(KIND, acc, column[r * 64]);
+  for (; r < m; ++r) acc = P::apply(KIND, acc, column[r * STRIDE]);
 }
 
-// Long runs (hot rows of a skewed index distribution): the row is cut into chunks of 64 columns,
-// one workgroup each, so that one hot row keeps many CUs and many loads busy.  Four wavefronts
-// fetch 128 updates x 64 columns per round into LDS (32 independent loads per lane); the first
-// wavefront then applies the 128 staged values of its column in order.  A run of length >= 16
-// contains a multiple of 16, so only those positions get a workgroup, and the first of them
-// inside the run does the work (the run's head is found by bisection in the sorted keys).
+template <typename P, int kCols, int kPerLane>
+__device__ __forceinline__ void foldLongRun(typename P::S* stage, const u32* __restrict__ vals, long long rowElems, int kind,
+                                            typename P::S* __restrict__ result, const typename P::S* __restrict__ updates,
+                                            u32 key, long long head, long long total, u32 chunk, int lane, int w) {
+  typedef typename P::S S;
+  constexpr int kSubs = 64 / kCols;                 // updates per wavefront load
+  constexpr int kStep = 4 * kSubs;                  // updates per load of the whole workgroup
+  constexpr int kRound = kStep * kPerLane;
+  const int sub = lane / kCols, c = lane % kCols;
+  const long long col = (long long)chunk * kCols + c;
+  const bool active = col < rowElems;
+  const long long colc = active ? col : rowElems - 1;
+  const bool folder = w == 0 && sub == 0 && active;
+  typename P::A acc = typename P::A();
+  if (folder) acc = P::load(result[(long long)key * rowElems + col]);
+  // Every load is unconditional (a predicated load is a branch around it): positions past the run repeat its last
+  // update, columns past the row the last column; neither is folded or stored.
+  auto fetchNumbers = [&](long long round, u32* vi) {
+#pragma unroll
+    for (int q = 0; q < kPerLane; ++q) {
+      const long long t = round * kRound + q * kStep + w * kSubs + sub;
+      vi[q] = vals[head + (t < total ? t : total - 1)];
+    }
+  };
+  const long long rounds = (total + kRound - 1) / kRound;
+  u32 vi[kPerLane], vnext[kPerLane];
+  S u[kPerLane];
+  // The scheduling fences keep each group of loads together: interleaved with the loads that depend on them,
+  // every pair waits for its own round trip and the latencies add up.
+  fetchNumbers(0, vi);
+  __builtin_amdgcn_sched_barrier(0);
+  fetchNumbers(rounds > 1 ? 1 : 0, vnext);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int q = 0; q < kPerLane; ++q) u[q] = updates[(long long)vi[q] * rowElems + colc];
+  __builtin_amdgcn_sched_barrier(0);
+  for (long long r = 0; r < rounds; ++r) {
+#pragma unroll
+    for (int q = 0; q < kPerLane; ++q) stage[(q * kStep + w * kSubs + sub) * kCols + c] = u[q];
+    __builtin_amdgcn_sched_barrier(0);
+    if (r + 1 < rounds) {
+#pragma unroll
+      for (int q = 0; q < kPerLane; ++q) u[q] = updates[(long long)vnext[q] * rowElems + colc];
+      __builtin_amdgcn_sched_barrier(0);
+      fetchNumbers(r + 2 < rounds ? r + 2 : r + 1, vnext);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+    if (folder) {
+      const long long left = total - r * kRound;
+      const int m = left < kRound ? (int)left : kRound;
+      // the combiner is fixed outside the loop so that the LDS reads of a column pipeline
+      switch (kind) {
+        case 0: foldStaged<P, 0, kCols>(acc, stage + c, m); break;
+        case 1: foldStaged<P, 1, kCols>(acc, stage + c, m); break;
+        case 2: foldStaged<P, 2, kCols>(acc, stage + c, m); break;
+        case 3: foldStaged<P, 3, kCols>(acc, stage + c, m); break;
+        default: foldStaged<P, 4, kCols>(acc, stage + c, m); break;
+      }
+    }
+    __syncthreads();
+  }
+  if (folder) result[(long long)key * rowElems + col] = P::store(acc);
+}
+
+constexpr int kHugeCols = 8, kHugePerLane = 32;
+
+// Very long runs: chunks of 8 columns and rounds of 1024 updates (see above).
+template <typename P>
+__global__ void __launch_bounds__(256) scatter_fold_huge(const u32* __restrict__ keys, const u32* __restrict__ vals, long long n, long long rowElems,
+                                                          int kind, typename P::S* __restrict__ result, const typename P::S* __restrict__ updates, u32 rows, u32 chunks) {
+  typedef typename P::S S;
+  __shared__ S stage[4 * (64 / kHugeCols) * kHugePerLane * kHugeCols];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const u32 chunk = blockIdx.x % chunks;                       // workgroup number = position * chunks + column chunk
+  const long long p = (long long)(blockIdx.x / chunks) * kHugeSegment;
+  if (p >= n) return;
+  const u32 key = keys[p];
+  if (key >= rows) return;
+  if (p >= kHugeSegment && keys[p - kHugeSegment] == key) return;                    // an earlier workgroup owns this run
+  const long long head = runHead(keys, p, key, lane);
+  if (head + kHugeSegment - 1 >= n || keys[head + kHugeSegment - 1] != key) return;   // shorter run: other kernels
+  const long long total = runLast(keys, head + kHugeSegment - 1, n, key, lane) - head + 1;
+  foldLongRun<P, kHugeCols, kHugePerLane>(stage, vals, rowElems, kind, result, updates, key, head, total, chunk, lane, w);
+}
+
+// Long runs below kHugeSegment: chunks of 64 columns, rounds of 128 updates whose numbers are staged through LDS.
 template <typename P>
 __global__ void __launch_bounds__(256) scatter_fold_long(const u32* __restrict__ keys, const u32* __restrict__ vals, long long n, long long rowElems,
-                                                          int kind, typename P::S* __restrict__ result, const typename P::S* __restrict__ updates, u32 rows) {
+                                                          int kind, typename P::S* __restrict__ result, const typename P::S* __restrict__ updates, u32 rows, u32 chunks) {
   typedef typename P::S S;
   constexpr int kWaves = 4, kPerLane = 32, kRound = kWaves * kPerLane;   // 128 updates x 64 columns staged per round
   __shared__ u32 sval[256];
   __shared__ S stage[kRound][64];
-  const long long p = (long long)blockIdx.x * kLongSegment;
+  const u32 chunk = blockIdx.x % chunks;                       // workgroup number = position * chunks + column chunk
+  const long long p = (long long)(blockIdx.x / chunks) * kLongSegment;
   if (p >= n) return;
   const u32 key = keys[p];
   if (key >= rows) return;
-  long long lo = 0, hi = p;           // first position holding `key`
-  while (lo < hi) {
-    long long mid = (lo + hi) >> 1;
-    if (keys[mid] < key) lo = mid + 1; else hi = mid;
-  }
-  const long long head = lo;
-  if (p - head >= kLongSegment) return;                                             // an earlier workgroup owns this run
-  if (head + kLongSegment - 1 >= n || keys[head + kLongSegment - 1] != key) return;   // short run
+  if (p >= kLongSegment && keys[p - kLongSegment] == key) return;                    // an earlier workgroup owns this run
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const long long col = (long long)blockIdx.y * 64 + lane;
+  const long long head = runHead(keys, p, key, lane);
+  if (head + kLongSegment - 1 >= n || keys[head + kLongSegment - 1] != key) return;   // short run
+  if (head + kHugeSegment - 1 < n && keys[head + kHugeSegment - 1] == key) return;    // very long run: scatter_fold_huge
+  const long long col = (long long)chunk * 64 + lane;
   const bool active = col < rowElems;
   const long long colc = active ? col : rowElems - 1;
   typename P::A acc = typename P::A();
@@ -710,11 +927,11 @@ __global__ void __launch_bounds__(256) scatter_fold_long(const u32* __restrict__
       if (w == 0 && active) {
         // the combiner is fixed outside the loop so that the LDS reads of a column pipeline
         switch (kind) {
-          case 0: foldStaged<P, 0>(acc, &stage[0][lane], m); break;
-          case 1: foldStaged<P, 1>(acc, &stage[0][lane], m); break;
-          case 2: foldStaged<P, 2>(acc, &stage[0][lane], m); break;
-          case 3: foldStaged<P, 3>(acc, &stage[0][lane], m); break;
-          default: foldStaged<P, 4>(acc, &stage[0][lane], m); break;
+          case 0: foldStaged<P, 0, 64>(acc, &stage[0][lane], m); break;
+          case 1: foldStaged<P, 1, 64>(acc, &stage[0][lane], m); break;
+          case 2: foldStaged<P, 2, 64>(acc, &stage[0][lane], m); break;
+          case 3: foldStaged<P, 3, 64>(acc, &stage[0][lane], m); break;
+          default: foldStaged<P, 4, 64>(acc, &stage[0][lane], m); break;
         }
       }
       __syncthreads();
@@ -983,12 +1200,19 @@ int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* in
   u32* vals0 = keys1 + n;
   u32* vals1 = vals0 + n;
   u32* counts = vals1 + n;
-  unsigned gb = (unsigned)((n + 255) / 256);
-  scatter_init_keys<<<gb, 256, 0, st>>>(indices, d->index_bytes, n, d->operandRows, keys0, vals0);
   // keys lie in [0, rows]: sort only the bits that can be set
   int bits = 1;
   while (bits < 32 && (1ll << bits) <= d->operandRows) ++bits;
   u32 *kin = keys0, *kout = keys1, *vin = vals0, *vout = vals1;
+  static const bool smallSort = !(getenv("MI355X_SCATTER_SMALL_SORT") && getenv("MI355X_SCATTER_SMALL_SORT")[0] == '0');
+  const bool small = smallSort && n <= kSmallSort;
+  if (small) {
+    scatter_sort_small<<<1, 1024, 0, st>>>(indices, d->index_bytes, (int)n, d->operandRows, bits, kin, vin);
+    bits = 0;   // sorted
+  } else {
+    unsigned gb = (unsigned)((n + 255) / 256);
+    scatter_init_keys<<<gb, 256, 0, st>>>(indices, d->index_bytes, n, d->operandRows, keys0, vals0);
+  }
   // few keys: few sorting workgroups, so that the single-workgroup scan over their histograms stays short
   int sortBlocks = (int)((n + 2047) / 2048);
   sortBlocks = sortBlocks < 1 ? 1 : (sortBlocks > kSortBlocks ? kSortBlocks : sortBlocks);
@@ -1000,10 +1224,13 @@ int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* in
     t = vin; vin = vout; vout = t;
   }
   dim3 gridShort((unsigned)n, (unsigned)((d->rowElems + 255) / 256));
-  dim3 gridLong((unsigned)((n + kLongSegment - 1) / kLongSegment), (unsigned)((d->rowElems + 63) / 64));
+  const long long chunksHuge = (d->rowElems + kHugeCols - 1) / kHugeCols, chunksLong = (d->rowElems + 63) / 64;
+  const long long blocksHuge = chunksHuge * ((n + kHugeSegment - 1) / kHugeSegment), blocksLong = chunksLong * ((n + kLongSegment - 1) / kLongSegment);
+  if (blocksHuge > 0x7FFFFFFFll || blocksLong > 0x7FFFFFFFll) return 3;   // more workgroups than a grid holds
 #define FOLD(P) do { \
+    if (n >= kHugeSegment) scatter_fold_huge<P><<<(unsigned)blocksHuge, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (typename P::S*)result, (const typename P::S*)updates, (u32)d->operandRows, (u32)chunksHuge); \
+    if (n >= kLongSegment) scatter_fold_long<P><<<(unsigned)blocksLong, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (typename P::S*)result, (const typename P::S*)updates, (u32)d->operandRows, (u32)chunksLong); \
     scatter_fold_short<P><<<gridShort, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (typename P::S*)result, (const typename P::S*)updates, (u32)d->operandRows); \
-    if (n >= kLongSegment) scatter_fold_long<P><<<gridLong, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (typename P::S*)result, (const typename P::S*)updates, (u32)d->operandRows); \
   } while (0)
   if (d->dtype == 0) FOLD(Plain<float>);
   else if (d->dtype == 2) FOLD(Plain<int>);

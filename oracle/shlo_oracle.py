@@ -1789,8 +1789,21 @@ class Oracle:
             kind = body.ops[0].name.replace("stablehlo.", "")
             if kind == "subtract" and body.ops[0].operands != body.args:
                 kind = None
+        stepwise = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply}
         with np.errstate(all="ignore"):
-            if kind == "set":
+            if op.out_types[0].dtype == "bf16" and kind in stepwise and self.round_intermediates:
+                # The body works on bf16 scalars: every application rounds.  Updates are applied in order; round r
+                # applies the r-th update of every element at once (an element occurs at most once per round).
+                order = np.argsort(flat, kind="stable")
+                sf = flat[order]
+                first = np.r_[True, sf[1:] != sf[:-1]] if sf.size else np.zeros(0, bool)
+                start = np.maximum.accumulate(np.where(first, np.arange(sf.size), 0)) if sf.size else sf
+                occurrence = np.empty(sf.size, np.int64)
+                occurrence[order] = np.arange(sf.size) - start
+                for r in range(int(occurrence.max()) + 1 if sf.size else 0):
+                    sel = occurrence == r
+                    out[flat[sel]] = round_bf16(stepwise[kind](out[flat[sel]], u[sel]).astype(np.float32))
+            elif kind == "set":
                 out[flat] = u
             elif kind == "add":
                 if out.dtype == np.bool_:

@@ -227,6 +227,26 @@ case("scatter-add-hot-rows-int", _row_scatter("add"), rng(166).integers(-5, 5, s
 case("scatter-max-hot-rows", _row_scatter("max"), f32(169, 25, 64), _hot(1690, 600, 25), f32(1691, 600, 64), exact=True)
 case("scatter-add-hot-rows-exactly-16", _row_scatter("add"), f32(1692, 8, 33), np.array([5] * 16 + [2] * 15 + [7] * 17, np.int32), f32(1693, 48, 33), exact=True)
 
+# very long runs (at least 256 updates of one row: narrow column chunks, 1024 updates staged per round), run lengths at the
+# tier boundaries, the single-workgroup sort (at most 8192 updates) with one to three digit passes, and the general sort
+def _runs(seed, *lengths_by_row):
+    idx = np.concatenate([np.full(n, row, np.int32) for row, n in lengths_by_row])
+    return rng(seed).permutation(idx).astype(np.int32)
+case("scatter-add-very-long-run-three-rounds", _row_scatter("add"), f32(2600, 20, 13),
+     np.where(rng(2601).random(3000) < 0.8, 3, rng(2602).integers(0, 20, size=3000)).astype(np.int32), f32(2603, 3000, 13), exact=True)
+case("scatter-add-run-lengths-at-the-tier-boundaries", _row_scatter("add"), f32(2604, 12, 20),
+     _runs(2605, (1, 255), (2, 256), (3, 257), (4, 1024), (5, 1025), (6, 15), (7, 16), (8, 17), (9, 1)), f32(2606, 2866, 20), exact=True)
+case("scatter-max-very-long-run", _row_scatter("max"), f32(2607, 6, 9), _runs(2608, (0, 700), (5, 300), (2, 40)), f32(2609, 1040, 9), exact=True)
+case("scatter-add-very-long-run-bf16", _row_scatter("add"), f32(2610, 6, 24, lo=-1, hi=1), _runs(2611, (4, 600), (1, 90), (0, 3)), f32(2612, 693, 24, lo=-1, hi=1),
+     dtypes=["bf16", "i32", "bf16"], exact=True)
+case("scatter-add-row-numbers-of-17-bits", _row_scatter("add"), f32(2613, 70000, 4),
+     np.concatenate([rng(2614).integers(-5, 70010, size=4000), np.full(300, 69999), np.full(20, 65536)]).astype(np.int32)[rng(2615).permutation(4320)],
+     f32(2616, 4320, 4), exact=True)
+case("scatter-add-row-numbers-of-8-bits-int64-indices", _row_scatter("add"), f32(2617, 200, 6), rng(2618).integers(0, 200, size=8192).astype(np.int64),
+     f32(2619, 8192, 6), exact=True)
+case("scatter-add-more-updates-than-one-workgroup-sorts", _row_scatter("add"), f32(2620, 50, 10),
+     np.where(rng(2621).random(9000) < 0.3, 7, rng(2622).integers(0, 50, size=9000)).astype(np.int32), f32(2623, 9000, 10), exact=True)
+
 # ------------------------------------------------------------------ dot_general (tests/configs/matmul.py:19-249)
 case("dot-matmul", lambda b, x, y: b.matmul(x, y), f32(170, 33, 70), f32(171, 70, 45))
 case("dot-vector-matrix", lambda b, x, y: b.dot_general(x, y, ([0], [0])), f32(172, 70), f32(173, 70, 45))

@@ -179,6 +179,19 @@ def test_scatter_is_sequential_in_update_order():
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+def test_bf16_scatter_rounds_after_every_application():
+    # the body adds two bf16 scalars, so each application rounds: a float32 accumulation rounded once at the end differs
+    c = op_cases.get_case("scatter-add-very-long-run-bf16")
+    x, idx, upd = [round_bf16(a) if d == "bf16" else a for a, d in zip(c.inputs, c.dtypes)]
+    got = Oracle(c.text).run(x, idx, upd)[0]
+    want, once = x.copy(), x.copy()
+    for i, u in zip(idx, upd):
+        want[i] = round_bf16((want[i] + u).astype(np.float32))
+        once[i] = once[i] + u
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert not np.array_equal(want, round_bf16(once))      # the case tells the two rules apart
+
+
 # ------------------------------------------------------------------ the five programs vs torch autograd
 def test_mlp_program_vs_torch():
     p = configs.build_mlp(**configs.SMALL["mlp"])
