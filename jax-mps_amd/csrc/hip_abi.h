@@ -138,6 +138,11 @@ typedef struct {
 // holds the operand.  `workspace` needs mi355_scatter_workspace_bytes(numUpdates) bytes.
 int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* indices, const void* updates,
                        void* workspace, mi355_stream_t s);
+// The same with the operand given as a splat: when `fill` is set, `result` need not hold anything on entry and every
+// element starts as `fill_bits` (the element's bit pattern; 16-bit types in the low half).  The fill shares a launch
+// with the sort, which keeps one CU busy while the others write.
+int mi355_scatter_rows_fill(const mi355_scatter_desc* d, void* result, const void* indices, const void* updates,
+                            void* workspace, int fill, uint32_t fill_bits, mi355_stream_t s);
 size_t mi355_scatter_workspace_bytes(int64_t num_updates);
 // resolves, for the current device, the library-owned workspace of mi355x_scatter_rows_noalloc (include/mi355x_noalloc.h)
 int mi355_noalloc_setup(void);

@@ -554,8 +554,26 @@ __global__ void __launch_bounds__(256) radix_scatter(const u32* __restrict__ key
 // every pass and they start behind every real pair, so they end behind every real pair.
 constexpr int kSmallSort = 8192;
 
+// Splat fill of the scatter result for workgroups 1 .. gridDim.x - 1 (workgroup 0 sorts meanwhile, or does nothing
+// in the launch of the general sort path): 16-byte stores, the last bytes of an odd size in 16-bit units.
+__device__ __forceinline__ void fillSplat(unsigned char* dst, unsigned long long bytes, u32 bits32) {
+  const unsigned long long n16 = bytes / 16, lanes = (unsigned long long)(gridDim.x - 1) * blockDim.x;
+  const uint4 v = make_uint4(bits32, bits32, bits32, bits32);
+  for (unsigned long long i = (unsigned long long)(blockIdx.x - 1) * blockDim.x + threadIdx.x; i < n16; i += lanes) ((uint4*)dst)[i] = v;
+  if (blockIdx.x == 1 && threadIdx.x < (bytes % 16) / 2) ((u16*)(dst + n16 * 16))[threadIdx.x] = (u16)(threadIdx.x & 1 ? bits32 >> 16 : bits32);
+}
+
+__global__ void __launch_bounds__(1024) scatter_fill(unsigned char* fillDst, unsigned long long fillBytes, u32 fillBits) {
+  if (blockIdx.x > 0) fillSplat(fillDst, fillBytes, fillBits);
+}
+
 __global__ void __launch_bounds__(1024) scatter_sort_small(const void* idx, int idxBytes, int n, long long rows, int bits,
-                                                           u32* __restrict__ keysOut, u32* __restrict__ valsOut) {
+                                                           u32* __restrict__ keysOut, u32* __restrict__ valsOut,
+                                                           unsigned char* fillDst, unsigned long long fillBytes, u32 fillBits) {
+  if (blockIdx.x > 0) {
+    fillSplat(fillDst, fillBytes, fillBits);
+    return;
+  }
   __shared__ u32 keysL[kSmallSort];
   __shared__ u16 valsL[kSmallSort];
   __shared__ u16 cnt[256][16];
@@ -1192,9 +1210,23 @@ size_t mi355_scatter_workspace_bytes(int64_t n) {
 
 int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* indices, const void* updates, void* workspace,
                        mi355_stream_t s) {
+  return mi355_scatter_rows_fill(d, result, indices, updates, workspace, 0, 0, s);
+}
+
+int mi355_scatter_rows_fill(const mi355_scatter_desc* d, void* result, const void* indices, const void* updates, void* workspace,
+                            int fill, uint32_t fillBits, mi355_stream_t s) {
   long long n = d->numUpdates;
-  if (n <= 0 || d->rowElems <= 0) return 0;
   hipStream_t st = (hipStream_t)s;
+  const int elemBytes = d->dtype == 1 ? 2 : 4;
+  const unsigned long long fillBytes = fill ? (unsigned long long)d->operandRows * d->rowElems * elemBytes : 0;
+  if (elemBytes == 2) fillBits = (fillBits & 0xFFFFu) | (fillBits << 16);
+  // enough workgroups of 1024 lanes to keep every CU writing, each lane storing a few times
+  unsigned fillBlocks = (unsigned)((fillBytes / 16 + 8191) / 8192);
+  fillBlocks = fillBytes == 0 ? 0 : (fillBlocks < 1 ? 1 : (fillBlocks > 2048 ? 2048 : fillBlocks));
+  if (n <= 0 || d->rowElems <= 0) {
+    if (fillBlocks) scatter_fill<<<1 + fillBlocks, 1024, 0, st>>>((unsigned char*)result, fillBytes, fillBits);
+    return check("scatter_rows");
+  }
   u32* keys0 = (u32*)workspace;
   u32* keys1 = keys0 + n;
   u32* vals0 = keys1 + n;
@@ -1207,9 +1239,11 @@ int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* in
   static const bool smallSort = !(getenv("MI355X_SCATTER_SMALL_SORT") && getenv("MI355X_SCATTER_SMALL_SORT")[0] == '0');
   const bool small = smallSort && n <= kSmallSort;
   if (small) {
-    scatter_sort_small<<<1, 1024, 0, st>>>(indices, d->index_bytes, (int)n, d->operandRows, bits, kin, vin);
+    scatter_sort_small<<<1 + fillBlocks, 1024, 0, st>>>(indices, d->index_bytes, (int)n, d->operandRows, bits, kin, vin,
+                                                         (unsigned char*)result, fillBytes, fillBits);
     bits = 0;   // sorted
   } else {
+    if (fillBlocks) scatter_fill<<<1 + fillBlocks, 1024, 0, st>>>((unsigned char*)result, fillBytes, fillBits);
     unsigned gb = (unsigned)((n + 255) / 256);
     scatter_init_keys<<<gb, 256, 0, st>>>(indices, d->index_bytes, n, d->operandRows, keys0, vals0);
   }

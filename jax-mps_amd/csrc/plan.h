@@ -59,6 +59,8 @@ struct ScatterDesc {   // row scatter: operand [rows, rowSize...], one index per
   int64_t numUpdates = 0, rowElems = 0, operandRows = 0;
   int kind = 0;        // 0 add, 1 set, 2 mul, 3 min, 4 max
   DType type = DType::F32, indexType = DType::S32;
+  bool fill = false;   // the operand is a splat that the scatter writes itself (no buffer holds it beforehand)
+  uint32_t fillBits = 0;
 };
 
 struct AttentionDesc {   // softmax(scale * Q K^T, masked -> `masked`) V, tensors addressed as [b, n, t|s, h] through element strides

@@ -163,8 +163,32 @@ class Planner {
     return true;
   }
 
+  // bit pattern of the element every position of `v` holds, when `v` is a broadcast of a constant
+  static bool splatBits(Value* v, uint32_t& bits) {
+    Op* d = v->def;
+    while (d && (d->name == "broadcast_in_dim" || d->name == "reshape") && d->operands[0]->type.dt == v->type.dt) d = d->operands[0]->def;
+    if (!d || d->name != "constant") return false;
+    auto& dd = *d->attrs.at("value").dense;
+    if ((!dd.splat && dd.type.numel() != 1) || dd.type.dt != v->type.dt) return false;
+    const size_t size = dtypeSize(dd.type.dt);
+    if ((size != 2 && size != 4) || dd.bytes.size() < size) return false;
+    bits = 0;
+    memcpy(&bits, dd.bytes.data(), size);
+    return true;
+  }
+
+  // A splat operand of a scatter that nothing else reads (the zeros a gradient is scattered into) is written by
+  // the scatter itself: its fill shares a launch with the sort of the indices.
+  static bool scatterWritesSplat(Value* v, Op* user) {
+    static const bool on = !getenv("MI355X_SCATTER_FILL") || atoi(getenv("MI355X_SCATTER_FILL")) != 0;
+    uint32_t bits;
+    return on && user->name == "scatter" && user->operands.size() == 3 && user->operands[0] == v && user->operands[1] != v && user->operands[2] != v &&
+           v->users.size() == 1 && user->operands[2]->type.numel() > 0 && splatBits(v, bits);
+  }
+
   static bool forcedBy(Value* v, Op* user) {
     if (isWindowReverse(v, user)) return false;
+    if (scatterWritesSplat(v, user)) return false;
     if (dotTakesView(v, user)) return false;
     if (user->name == "gather") return user->operands[0] == v;       // random access needs memory
     if (isFusibleOp(*user)) return false;
@@ -1550,7 +1574,9 @@ class Planner {
     Value* idx = op->operands[1];
     Value* upd = op->operands[2];
     Value* res = op->result();
-    for (Value* v : {operand, idx, upd}) if (!hasStorage(v)) materializeNow(v, plan);
+    uint32_t fillBits = 0;
+    bool fill = !hasStorage(operand) && scatterWritesSplat(operand, op) && splatBits(operand, fillBits);
+    for (Value* v : {operand, idx, upd}) if (!hasStorage(v) && !(fill && v == operand)) materializeNow(v, plan);
     auto& uwd = op->ints("update_window_dims");
     auto& iwd = op->ints("inserted_window_dims");
     auto& sdo = op->ints("scatter_dims_to_operand_dims");
@@ -1591,12 +1617,14 @@ class Planner {
       throw CompileError("stablehlo.scatter: element type not supported");
     if (idx->type.dt != DType::S32 && idx->type.dt != DType::S64 && idx->type.dt != DType::U32) throw CompileError("stablehlo.scatter: index type not supported");
     // result storage: reuse the operand's buffer when nothing else reads it
-    int osid = storageOf(operand);
+    int osid = fill ? -1 : storageOf(operand);
     int sid;
     int t = ++time_;
-    bool inPlace = st_[osid].kind == BufRef::Temp && st_[osid].values == 1 && operand->users.size() == 1 && !boundToOutput_.count(osid) &&
+    bool inPlace = !fill && st_[osid].kind == BufRef::Temp && st_[osid].values == 1 && operand->users.size() == 1 && !boundToOutput_.count(osid) &&
                    !outerStorage(osid);
-    if (inPlace) {
+    if (fill) {
+      sid = newStorage(res->type.bytes());
+    } else if (inPlace) {
       sid = osid;
     } else {
       sid = newStorage(res->type.bytes());
@@ -1613,7 +1641,9 @@ class Planner {
     if (nUpd == 0) return;
     Step s;
     s.kind = Step::ScatterRows;
-    s.label = std::string("scatter-") + kind + " rows";
+    s.label = std::string("scatter-") + kind + " rows" + (fill ? " into a splat" : "");
+    s.scatter.fill = fill;
+    s.scatter.fillBits = fillBits;
     s.scatter.numUpdates = nUpd;
     s.scatter.operandRows = operand->type.dims[0];
     s.scatter.rowElems = operand->type.numel() / std::max<int64_t>(1, operand->type.dims[0]);

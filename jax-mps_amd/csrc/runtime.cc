@@ -501,8 +501,8 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       d.index_bytes = (int)dtypeSize(s.scatter.indexType);
       if ((size_t)s.workspaceBytes < mi355_scatter_workspace_bytes(d.numUpdates))
         throw RuntimeError("internal: scatter workspace is smaller than the kernel needs");
-      check(mi355_scatter_rows(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out),
-                               resolve(s.args[3], in, out), st), "scatter");
+      check(mi355_scatter_rows_fill(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out),
+                                    resolve(s.args[3], in, out), s.scatter.fill ? 1 : 0, s.scatter.fillBits, st), "scatter");
       break;
     }
     case Step::Copy: {

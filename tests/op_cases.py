@@ -247,6 +247,28 @@ case("scatter-add-row-numbers-of-8-bits-int64-indices", _row_scatter("add"), f32
 case("scatter-add-more-updates-than-one-workgroup-sorts", _row_scatter("add"), f32(2620, 50, 10),
      np.where(rng(2621).random(9000) < 0.3, 7, rng(2622).integers(0, 50, size=9000)).astype(np.int32), f32(2623, 9000, 10), exact=True)
 
+# the operand is a splat constant (zeros a gradient is scattered into): the scatter writes it itself, in the launch that sorts
+def _scatter_into(value, rows, cols, dtype="f32", body="add"):
+    def f(b, i, u):
+        x = b.constant(value, dtype, (rows, cols))
+        return b.scatter(x, b.reshape(i, (i.shape[0], 1)), u, update_window_dims=[1], inserted_window_dims=[0], scatter_dims_to_operand_dims=[0],
+                         index_vector_dim=1, body=body)
+    return f
+case("scatter-add-into-zeros", _scatter_into(0.0, 300, 70), rng(2630).integers(0, 300, size=1000).astype(np.int32), f32(2631, 1000, 70), exact=True)
+case("scatter-add-into-zeros-odd-size", _scatter_into(0.0, 31, 3), rng(2632).integers(-2, 33, size=200).astype(np.int32), f32(2633, 200, 3), exact=True)
+case("scatter-max-into-splat", _scatter_into(-0.25, 40, 9, body="max"), _hot(2634, 700, 40), f32(2635, 700, 9), exact=True)
+case("scatter-add-into-ones-bf16", _scatter_into(1.0, 17, 5, dtype="bf16"), rng(2636).integers(0, 17, size=64).astype(np.int32), f32(2637, 64, 5, lo=-1, hi=1),
+     dtypes=["i32", "bf16"], exact=True)
+case("scatter-add-into-int-splat", _scatter_into(7, 20, 6, dtype="i32"), rng(2638).integers(0, 20, size=90).astype(np.int32),
+     rng(2639).integers(-100, 100, size=(90, 6)).astype(np.int32), exact=True)
+case("scatter-add-into-zeros-more-updates-than-one-workgroup-sorts", _scatter_into(0.0, 64, 12), rng(2640).integers(0, 64, size=8200).astype(np.int32),
+     f32(2641, 8200, 12), exact=True)
+def _scatter_splat_read_twice(b, i, u):
+    x = b.constant(0.0, "f32", (50, 8))
+    y = b.scatter(x, b.reshape(i, (i.shape[0], 1)), u, update_window_dims=[1], inserted_window_dims=[0], scatter_dims_to_operand_dims=[0], index_vector_dim=1)
+    return [y, b.add(x, 1.0)]
+case("scatter-add-into-zeros-that-something-else-reads", _scatter_splat_read_twice, rng(2642).integers(0, 50, size=120).astype(np.int32), f32(2643, 120, 8), exact=True)
+
 # ------------------------------------------------------------------ dot_general (tests/configs/matmul.py:19-249)
 case("dot-matmul", lambda b, x, y: b.matmul(x, y), f32(170, 33, 70), f32(171, 70, 45))
 case("dot-vector-matrix", lambda b, x, y: b.dot_general(x, y, ([0], [0])), f32(172, 70), f32(173, 70, 45))
