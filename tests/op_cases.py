@@ -670,6 +670,18 @@ case("while-carry-new-value-read-after-producer", lambda b, x, w: _loop(b, [x, b
 case("while-carry-broadcast-row-of-itself", lambda b, x: _loop(b, [x], lambda i, p: [b.add(p, b.broadcast_in_dim(b.reshape(b.slice(p, [0, 0], [1, 16]), (16,)), (4, 16), [1]))]), f32(2310, 4, 16, lo=-0.1, hi=0.1))
 
 
+# a scatter inside a counted loop (its launches are replayed from a captured graph): splat operand written by the scatter, a very
+# long run, and the result accumulated into a carry
+def _scatter_in_loop(b, i, u):
+    def body(t, acc):
+        x = b.constant(0.0, "f32", (24, 10))
+        scale = b.broadcast_in_dim(b.reshape(b.convert(b.add(t, 1), "f32"), (1, 1)), u.shape, (0, 1))
+        y = b.scatter(x, b.reshape(i, (i.shape[0], 1)), b.mul(u, scale), update_window_dims=[1], inserted_window_dims=[0],
+                      scatter_dims_to_operand_dims=[0], index_vector_dim=1)
+        return [b.add(acc, y)]
+    return _loop(b, [b.constant(0.0, "f32", (24, 10))], body, trips=4)[0]
+case("scatter-add-into-zeros-inside-a-loop", _scatter_in_loop, _runs(2650, (3, 300), (20, 40), (7, 5), (0, 1)), f32(2651, 346, 10), exact=True)
+
 def _case3(b, idx, x):
     return b.case(idx, [lambda: b.mul(x, 2.0), lambda: b.add(x, 10.0), lambda: b.neg(x)], [(x.shape, "f32")])[0]
 
