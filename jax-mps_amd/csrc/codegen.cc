@@ -1192,7 +1192,9 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     const std::string initPre = em.pre_;
     s << initPre;
     for (size_t j = 0; j < nr; ++j) {
-      std::string part = "part" + std::to_string(j) + "[p * " + std::to_string(Kn) + " + kk]";
+      // partial p of output kk lives at [kk * P + p]: the lanes that fold one output read consecutive words (with the
+      // partials of one pass side by side instead, each lane of the fold touched a cache line of its own)
+      std::string part = "part" + std::to_string(j) + "[kk * " + std::to_string(P) + " + p]";
       std::string ST = ops[j].accT == "bool" ? "int" : ops[j].accT;
       std::string a = "a" + std::to_string(j);
       s << "  " << ops[j].accT << " " << a << " = " << ops[j].identity << ";\n";
@@ -1349,7 +1351,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
       s << "  if (lane != 0) return;\n";
     }
     for (size_t j = 0; j < nr; ++j) {
-      if (partial) s << "  out" << j << "[((" << IT << ")blockIdx.x % " << P << ") * " << Kn << " + kk] = acc" << j << ";\n";
+      if (partial) s << "  out" << j << "[kk * " << P << " + ((" << IT << ")blockIdx.x % " << P << ")] = acc" << j << ";\n";
       else {
         s << "  const " << ops[j].accT << " res" << j << " = " << roundTo(ops[j].dt, ops[j].combine(inits[j], "acc" + std::to_string(j))) << ";\n";
         s << "  out" << j << "[kk] = " << storeExpr(ops[j].dt, "res" + std::to_string(j)) << ";\n";
@@ -1487,7 +1489,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   }
   for (size_t j = 0; j < nr; ++j) {
     s << "  #pragma unroll\n  for (int v = 0; v < " << V << "; ++v) ";
-    if (partial) s << "out" << j << "[(" << IT << ")blockIdx.y * " << Kn << " + kb + v] = acc" << j << "[v];\n";
+    if (partial) s << "out" << j << "[(kb + v) * " << P << " + (" << IT << ")blockIdx.y] = acc" << j << "[v];\n";
     else s << "out" << j << "[kb + v] = " << storeExpr(ops[j].dt, roundTo(ops[j].dt, ops[j].combine(inits[j], "acc" + std::to_string(j) + "[v]"))) << ";\n";
   }
   s << "}\n";

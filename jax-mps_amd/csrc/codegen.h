@@ -75,7 +75,7 @@ std::string combineKernels(const std::vector<const std::string*>& sources, const
 // `epilogue`: values of the result shape computed from the results (and other inputs of that shape); they are
 // produced by the pass that folds partial sums when there is one (FusedCode::epilogueFused), otherwise ignored.
 // `externalPartials` > 0: the partial results (that many per output, float accumulators, partial p of output k at
-// [p * outputs + k] from partialOffsets[j] of the workspace) are written by an earlier step; only the folding pass is generated.
+// [k * externalPartials + p] from partialOffsets[j] of the workspace) are written by an earlier step; only the folding pass is generated.
 FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeaf, const std::vector<Value*>& epilogue = {}, int64_t externalPartials = 0);
 
 // True if codegen can inline `op` into a consumer (elementwise / indexing ops).

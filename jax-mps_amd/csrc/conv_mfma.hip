@@ -65,7 +65,7 @@ struct ConvP {
   int taps;                      // window taps this launch visits (kc0 * kc1)
   int tilesM, tilesXY;           // split launches of the vector-loader kernel: tile rows and tiles per K range (tilesXY 0: a 3-d grid)
   // Column statistics of the output taken from the accumulators (batch-norm's sum and sum of squares over all rows):
-  // workgroup (tile row i, tile column) writes the sums over its rows to statSum[i * N + n] / statSq[i * N + n];
+  // workgroup (tile row i, tile column) writes the sums over its rows to statSum[n * tile rows + i] / statSq[n * tile rows + i];
   // a later pass folds the tile rows in order.  Null when not wanted.
   float* statSum;
   float* statSq;
@@ -683,7 +683,7 @@ __device__ __forceinline__ void leanBody(const ConvP& p, int split) {
         const int n = n0 + wn * WN + b * 32 + row;
         if (n < p.N) {
           const float v = colPart[0][wn][half][b * 32 + row] + colPart[1][wn][half][b * 32 + row];
-          (half ? p.statSq : p.statSum)[(size_t)bx * p.N + n] = v;
+          (half ? p.statSq : p.statSum)[(size_t)n * gridDim.x + bx] = v;
         }
       }
     }
