@@ -1428,6 +1428,9 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   int64_t P = 1;
   static const int colPerThread = getenv("MI355X_REDUCE_COL_PER_THREAD") ? atoi(getenv("MI355X_REDUCE_COL_PER_THREAD")) : 16;
   if (Rn > (int64_t)TY * 16) P = std::min<int64_t>((Rn + TY * colPerThread - 1) / (TY * colPerThread), std::max<int64_t>(1, 2048 / gridX));
+  // a small input is cheaper to walk in one launch (a few dozen loads per lane) than to split over a second, dependent one
+  static const int64_t onePassElems = getenv("MI355X_REDUCE_ONE_PASS") ? atoll(getenv("MI355X_REDUCE_ONE_PASS")) : 256 * 1024;
+  if (Rn * Kn <= onePassElems && Rn <= (int64_t)TY * 128) P = 1;
   bool partial = P > 1;
   Emitter em(isLeaf, V, i64);
   IdxDim klin;
