@@ -1462,7 +1462,8 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   s << "  const " << IT << " kb = ((" << IT << ")blockIdx.x * " << TX << " + tx) * " << V << ";\n";
   s << "  const bool active = kb < " << Kn << ";\n";
   s << "  const " << IT << " chunk = (" << Rn << " + " << P << " - 1) / " << P << ";\n";
-  s << "  const " << IT << " r_begin = (" << IT << ")blockIdx.y * chunk;\n";
+  // (a single-pass kernel names no second grid index, so that it can share a launch with its neighbours)
+  s << "  const " << IT << " r_begin = " << (partial ? "(" + IT + ")blockIdx.y * chunk" : std::string("0")) << ";\n";
   s << "  const " << IT << " r_end = r_begin + chunk < " << Rn << " ? r_begin + chunk : " << Rn << ";\n";
   for (size_t j = 0; j < nr; ++j) {
     s << "  " << ops[j].accT << " acc" << j << "[" << V << "];\n";
