@@ -69,7 +69,8 @@ typedef struct {
   int64_t bB0, bB1, bRow, bCol;
   int in_dtype, out_dtype;
   // act 1 (bf16 results only): after the bias, y = act_a * x * (1 + tanh(act_c * (x + act_b * x^3))) on the stored
-  // (rounded) value x, computed in fp32 and rounded again: the tanh form of GELU with the program's own constants
+  // (rounded) value x, computed in fp32 and rounded again: the tanh form of GELU with the program's own constants;
+  // act 2 (small fp32 products only, mi355_gemm_is_small): y = maximum(x, 0)
   int act;
   float act_a, act_b, act_c;
 } mi355_gemm_desc;

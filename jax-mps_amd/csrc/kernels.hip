@@ -193,6 +193,7 @@ struct SmallArgs {
   const float* bias;   // N values or null
   long long M, N;
   int batch1;
+  int relu;            // the stored value is maximum(sum + bias, 0)
 };
 
 // The MFMA contraction does not care which k a lane's operand slot stands for as long as A and B agree, so a
@@ -309,7 +310,8 @@ __device__ __forceinline__ void smallGemmTileBody(const SmallArgs& g, unsigned b
     const long long row = m0 + e / T, col = n0 + e % T;
     if (row < g.M && col < g.N) {
       const float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
-      C[row * g.N + col] = g.bias ? sum + g.bias[col] : sum;
+      const float v = g.bias ? sum + g.bias[col] : sum;
+      C[row * g.N + col] = g.relu ? ((v > 0.f || v != v) ? v : 0.f) : v;   // maximum(v, 0): NaN stays NaN, -0 becomes +0
     }
   }
 }
@@ -1088,6 +1090,7 @@ static bool fillSmall(SmallArgs& g, const mi355_gemm_desc* d1, const void* a1, c
   g.bias = (const float*)bias;
   g.M = d1->M; g.N = d1->N;
   g.batch1 = (int)d1->batch1;
+  g.relu = d1->act == 2;
   return true;
 }
 
@@ -1135,6 +1138,7 @@ int mi355_gemm_small_sum(const mi355_gemm_desc* d1, const void* a1, const void* 
   g.bias = (const float*)bias;
   g.M = d1->M; g.N = d1->N;
   g.batch1 = (int)d1->batch1;
+  g.relu = d1->act == 2;
   dim3 grid((unsigned)((d1->N + t - 1) / t), (unsigned)((d1->M + t - 1) / t), (unsigned)(d1->batch0 * d1->batch1));
   if (t == 16) gemm_f32_small<16><<<grid, 256, 0, (hipStream_t)s>>>(g);
   else gemm_f32_small<32><<<grid, 256, 0, (hipStream_t)s>>>(g);
@@ -1170,7 +1174,7 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
     r = mi355_gemm_bf16_tiled(d, a, b, c, s);
     if (r >= 0) return r ? r : addBias(d, c, bias, s);
   }
-  if (d->act && d->out_dtype != 1) return 2;
+  if (d->act == 2 ? !smallGemmTile(d) : (d->act && d->out_dtype != 1)) return 2;   // epilogues: GELU for bf16 results, maximum(x, 0) for small fp32 products
   if (smallGemmTile(d)) return mi355_gemm_small_sum(d, a, b, nullptr, nullptr, nullptr, c, bias, s);
   mi355_conv_desc cd;
   // strided views may start anywhere; the implicit-GEMM loaders issue 16-byte loads

@@ -1082,6 +1082,52 @@ void lowerSingleDeviceOpsIn(Module& m, Region& r, int& nextId, VMap& repl) {
 
 }  // namespace
 
+// compare(v, 0, GT) next to maximum(v, 0) asks the same of the maximum: maximum(v, 0) > 0 exactly when v > 0 (a NaN
+// stays a NaN and compares false either way).  The backward pass of a ReLU reads its mask this way; with the mask
+// taken from the activation, the value before it has one reader left and the kernel that produces it can apply the
+// maximum while it stores (planner.cc: the ReLU epilogue of small fp32 products).
+namespace {
+bool isZeroSplat(Value* v) {
+  Op* d = v->def;
+  while (d && (d->name == "broadcast_in_dim" || d->name == "reshape") && d->operands.size() == 1) d = d->operands[0]->def;
+  if (!d || d->name != "constant" || !d->has("value") || !d->attrs.at("value").dense) return false;
+  const DenseData& dd = *d->attrs.at("value").dense;
+  if (!dd.splat && dd.type.numel() != 1) return false;
+  if (dd.type.dt != DType::F32 || dd.bytes.size() < 4) return false;
+  uint32_t bits;
+  memcpy(&bits, dd.bytes.data(), 4);
+  return (bits & 0x7FFFFFFFu) == 0;
+}
+// the other operand of maximum(v, 0) / maximum(0, v), or null
+Value* reluInput(Op* op) {
+  if (op->name != "maximum" || op->operands.size() != 2 || op->results.size() != 1) return nullptr;
+  if (isZeroSplat(op->operands[1])) return op->operands[0];
+  if (isZeroSplat(op->operands[0])) return op->operands[1];
+  return nullptr;
+}
+void reluMasksIn(Region& r) {
+  std::unordered_map<Value*, Value*> activationOf;   // v -> maximum(v, 0) seen earlier in this region
+  for (auto& o : r.ops) {
+    for (auto& sub : o->regions) reluMasksIn(*sub);
+    if (Value* v = reluInput(o.get())) {
+      if (v->type.dt == DType::F32) activationOf.emplace(v, o->result());
+      continue;
+    }
+    if (o->name != "compare" || o->operands.size() != 2 || o->str("direction") != "GT") continue;
+    auto it = activationOf.find(o->operands[0]);
+    if (it == activationOf.end() || !isZeroSplat(o->operands[1])) continue;
+    Value* v = o->operands[0];
+    v->users.erase(std::remove(v->users.begin(), v->users.end(), o.get()), v->users.end());
+    o->operands[0] = it->second;
+    it->second->users.push_back(o.get());
+  }
+}
+}  // namespace
+
+void reluMasksFromActivations(Module& m) {
+  for (auto& f : m.funcs) reluMasksIn(f->body);
+}
+
 void lowerSingleDeviceOps(Module& m) {
   Func* f = m.main();
   if (!f) return;

@@ -37,7 +37,7 @@ struct GemmDesc {   // C[b0,b1] = A[b0,b1] x B[b0,b1]; operands addressed throug
   int64_t aB0 = 0, aB1 = 0, aRow = 0, aCol = 0;   // A(m,k) = a[b0*aB0 + b1*aB1 + m*aRow + k*aCol]
   int64_t bB0 = 0, bB1 = 0, bRow = 0, bCol = 0;   // B(k,n) = b[b0*bB0 + b1*bB1 + k*bRow + n*bCol]
   DType inType = DType::F32, outType = DType::F32;
-  int act = 0;                                     // 1: tanh-form GELU epilogue with the constants below
+  int act = 0;                                     // 1: tanh-form GELU epilogue with the constants below; 2: maximum(x, 0)
   float actA = 0.f, actB = 0.f, actC = 0.f;
 };
 

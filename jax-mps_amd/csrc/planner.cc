@@ -1462,6 +1462,22 @@ class Planner {
     ActMatch act;
     const bool fuseAct = !second && c->type.numel() > 0 && g.inType == DType::BF16 && g.outType == DType::BF16 &&
                          matchActivation(biasAdd ? biasAdd->result() : produced, act);
+    // ... -> maximum(x, 0) read by nothing else: a small fp32 product applies it while it stores
+    Op* relu = nullptr;
+    {
+      static const bool reluOn = !getenv("MI355X_GEMM_RELU") || atoi(getenv("MI355X_GEMM_RELU")) != 0;
+      Value* x = biasAdd ? biasAdd->result() : produced;
+      mi355_gemm_desc small = toAbi(g);
+      if (reluOn && !fuseAct && c->type.numel() > 0 && g.inType == DType::F32 && g.outType == DType::F32 && mi355_gemm_is_small(&small) &&
+          x->users.size() == 1 && x->users[0]->parent == x->def->parent) {
+        Op* u = x->users[0];
+        if (u->name == "maximum" && u->operands.size() == 2 && u->operands[0] != u->operands[1]) {
+          float zero = 1.f;
+          Value* other = u->operands[0] == x ? u->operands[1] : u->operands[0];
+          if (splatFloat(other, zero) && zero == 0.f) relu = u;
+        }
+      }
+    }
     int sid = newStorage(c->type.bytes());
     bind(produced, sid);
     if (sumAdd) emitted_.insert(sumAdd);
@@ -1471,8 +1487,13 @@ class Planner {
     s.kind = Step::Gemm;
     s.time = t;
     s.label = "dot_general " + a->type.str() + " x " + b->type.str() + (second ? " + " + second->operands[0]->type.str() + " x " + second->operands[1]->type.str() : "") +
-              (biasV ? " + bias" : "") + (fuseAct ? " + gelu" : "");
+              (biasV ? " + bias" : "") + (fuseAct ? " + gelu" : "") + (relu ? " + relu" : "");
     s.gemm = g;
+    if (relu) {
+      s.gemm.act = 2;
+      bind(relu->result(), sid);   // the step writes the activation; nothing reads the value before it
+      emitted_.insert(relu);
+    }
     if (fuseAct) {
       s.gemm.act = 1;
       s.gemm.actA = act.a; s.gemm.actB = act.b; s.gemm.actC = act.c;
@@ -2370,6 +2391,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   lowerWindowOps(*module);
   lowerRng(*module);
   lowerTopK(*module);
+  reluMasksFromActivations(*module);
   checkSupported(*module);
   eliminateDeadCode(module->main()->body);
   prog->module = std::move(module);

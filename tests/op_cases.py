@@ -316,6 +316,26 @@ case("dot-bias-f32-3d", _linear, f32(1976, 4, 9, 70), f32(1977, 70, 24), f32(197
 case("dot-bias-bf16-async", _linear, f32(1979, 200, 128, lo=-1, hi=1), f32(1980, 128, 328, lo=-1, hi=1), f32(1981, 328), dtypes=["bf16", "bf16", "bf16"])
 case("dot-bias-bf16-tiled", _linear, f32(1982, 200, 136, lo=-1, hi=1), f32(1983, 136, 328, lo=-1, hi=1), f32(1984, 328), dtypes=["bf16", "bf16", "bf16"])
 case("dot-bias-bf16-odd", _linear, f32(1985, 37, 50, lo=-1, hi=1), f32(1986, 50, 29, lo=-1, hi=1), f32(1987, 29), dtypes=["bf16", "bf16", "bf16"])
+# maximum(x, 0) on a small fp32 product is applied while the product is stored; a mask compare(x, 0, GT) next to it reads the
+# activation instead (same truth value), so the value before the activation needs no memory
+def _nan_row(seed, *shape):
+    a = f32(seed, *shape)
+    a[1, 3] = np.nan
+    return a
+case("dot-bias-relu-f32-small", lambda b, x, w, c: b.maximum(_linear(b, x, w, c), 0.0), f32(2660, 33, 70), f32(2661, 70, 45), f32(2662, 45))
+case("dot-relu-f32-small-no-bias-zero-first", lambda b, x, w: b.maximum(b.constant(0.0, "f32", (33, 45)), b.matmul(x, w)), f32(2663, 33, 70), f32(2664, 70, 45))
+case("dot-bias-relu-f32-small-nan-stays", lambda b, x, w, c: b.maximum(_linear(b, x, w, c), 0.0), _nan_row(2665, 33, 70), f32(2666, 70, 45), f32(2667, 45))
+def _relu_and_mask(b, x, w, c, g):
+    z = _linear(b, x, w, c)
+    return [b.maximum(z, 0.0), b.select(b.compare(z, b.constant(0.0, "f32", z.shape), "GT"), g, b.constant(0.0, "f32", z.shape))]
+case("dot-bias-relu-f32-small-mask-from-activation", _relu_and_mask, f32(2668, 33, 70), f32(2669, 70, 45), f32(2670, 45), f32(2671, 33, 45))
+case("dot-bias-relu-f32-small-value-before-also-read", lambda b, x, w, c: (lambda z: [b.maximum(z, 0.0), b.mul(z, 2.0)])(_linear(b, x, w, c)),
+     f32(2672, 33, 70), f32(2673, 70, 45), f32(2674, 45))
+case("dot-relu-f32-igemm-not-small", lambda b, x, w: b.maximum(b.matmul(x, w), 0.0), f32(2675, 520, 384, lo=-1, hi=1), f32(2676, 384, 1030, lo=-1, hi=1))
+def _two_products_relu(b, x, w, h, u, c):
+    y = b.add(b.matmul(x, w), b.matmul(h, u))
+    return b.maximum(b.add(y, b.broadcast_in_dim(c, y.shape, [1])), 0.0)
+case("dot-sum-two-products-bias-relu", _two_products_relu, f32(2677, 20, 30), f32(2678, 30, 40), f32(2679, 20, 50), f32(2680, 50, 40), f32(2681, 40))
 case("dot-bias-computed", lambda b, x, w, c: _linear(b, x, w, b.mul(c, c)), f32(1988, 33, 70), f32(1989, 70, 45), f32(1990, 45))
 case("dot-bias-depends-on-a-later-product", lambda b, x, w, v: (lambda y, z: b.add(y, b.broadcast_in_dim(b.neg(b.reshape(z, (45,))), y.shape, [1])))(b.matmul(x, w), b.matmul(v, w)),
      f32(1994, 33, 70), f32(1995, 70, 45), f32(1996, 1, 70))

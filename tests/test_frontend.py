@@ -112,6 +112,20 @@ def test_tokens_travel_as_scalar_placeholders():
     assert r.returncode == 0 and "while while trip 3" in r.stdout
 
 
+def test_relu_rides_in_a_small_product_and_its_mask_reads_the_activation():
+    """maximum(x, 0) after a small fp32 product is applied while the product is stored; the backward mask compare(x, 0, GT)
+    is taken from the activation, so the value before it is never written.  A second reader of that value, or a product
+    too large for the small-product kernel, keeps the separate kernel."""
+    r = plan(op_cases.get_case("dot-bias-relu-f32-small-mask-from-activation").text, "--dump-plan")
+    assert "+ bias + relu" in r.stdout and "maximum" not in r.stdout
+    r = plan(op_cases.get_case("dot-bias-relu-f32-small-value-before-also-read").text, "--dump-plan")
+    assert "+ relu" not in r.stdout and "maximum" in r.stdout
+    r = plan(op_cases.get_case("dot-relu-f32-igemm-not-small").text, "--dump-plan")
+    assert "+ relu" not in r.stdout
+    r = plan(configs.ALL["mlp"]().text, "--dump-plan")
+    assert r.stdout.count("+ bias + relu") == 1 and " 9 steps" in r.stdout
+
+
 def test_location_aliases_result_lists_and_composites_parse():
     text = """#loc1 = loc("x")
 module @jit_f attributes {mhlo.num_partitions = 1 : i32} {
