@@ -153,11 +153,11 @@ module @jit_f attributes {mhlo.num_partitions = 1 : i32} {
 def test_convolution_delivers_batch_norm_statistics():
     """The column sum and sum of squares of an unsplit convolution's output come from its accumulators: the pass over
     the output is gone and only the fold of the per-tile sums remains; a convolution that splits K, or a reduction
-    of another kind, keeps the two-pass reduction."""
+    of another kind, keeps its own pass over the output."""
     r = plan(op_cases.get_case("conv-statistics-from-accumulators").text, "--dump-plan")
     assert "+ column statistics" in r.stdout and r.stdout.count("kernel ") == 1 and "fold of convolution statistics" in r.stdout
     r = plan(op_cases.get_case("conv-statistics-split-k-stays-unfused").text, "--dump-plan")
-    assert "column statistics" not in r.stdout and r.stdout.count("kernel ") == 2
+    assert "column statistics" not in r.stdout and "reduce" in r.stdout      # (small enough for single-pass reductions, which share a launch)
     r = plan(op_cases.get_case("conv-statistics-max-stays-unfused").text, "--dump-plan")
     assert "column statistics" not in r.stdout
     p = configs.build_resnet18()
