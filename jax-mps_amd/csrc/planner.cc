@@ -106,6 +106,7 @@ class Planner {
   std::vector<Storage> st_;
   std::unordered_map<Value*, int> storage_;
   std::unordered_map<Value*, bool> needMat_;
+  std::unordered_set<Value*> inlineAnyway_;   // stored for a consumer that needs memory, yet cheap enough that kernels recompute it
   std::unordered_map<std::string, int> kernelIds_;
   std::unordered_set<int> boundToOutput_;
   std::vector<std::pair<int, int>> loops_;
@@ -197,6 +198,22 @@ class Planner {
     return true;
   }
 
+  // `v` is at most `budget` cheap elementwise ops away from values that are in memory whatever the analysis decides
+  static bool cheapFromMemory(Value* v, int& budget) {
+    Op* d = v->def;
+    if (!d || !isFusibleOp(*d) || d->results.size() != 1) return alwaysInMemory(v);
+    static const std::set<std::string> cheap = {"add", "subtract", "multiply", "negate", "select", "compare", "and", "or", "not", "convert", "reshape",
+                                                "broadcast_in_dim", "constant", "minimum", "maximum", "clamp", "iota"};
+    if (!cheap.count(d->name)) return false;
+    if (d->name == "constant") {
+      auto& dd = *d->attrs.at("value").dense;
+      return dd.splat || dd.type.numel() == 1;
+    }
+    if (d->name != "reshape" && d->name != "broadcast_in_dim" && d->name != "convert" && --budget < 0) return false;
+    for (auto* o : d->operands) if (!cheapFromMemory(o, budget)) return false;
+    return true;
+  }
+
   void analyze(Region& r) {
     // forward: set of leaves every value depends on (capped)
     std::unordered_map<Value*, std::vector<Value*>> leaves;
@@ -256,8 +273,9 @@ class Planner {
       bool forced = false;
       std::vector<Op*> g;
       auto addGroup = [&](Op* o) { if (g.size() < 4 && std::find(g.begin(), g.end(), o) == g.end()) g.push_back(o); };
+      bool nestedUse = false;
       for (Op* u : v->users) {
-        if (u->parent != &r) { forced = true; continue; }
+        if (u->parent != &r) { forced = true; nestedUse = true; continue; }
         if (forcedBy(v, u)) { forced = true; continue; }
         if (u->name == "reduce" || u->name == "dynamic_update_slice") { addGroup(u); continue; }
         Value* ur = u->result();
@@ -279,6 +297,14 @@ class Planner {
         if ((big >= 2 && ((int)g.size() - 1) * (big - 1) > limit) || expensive) mat = true;
       }
       needMat_[v] = mat;
+      // A small value that a scatter, gather or the like needs in memory, a few integer or select ops away from
+      // buffers that exist anyway (normalised indices, say): the kernels that also read it recompute it, so they do
+      // not depend on the kernel that stores it and can share its launch.
+      static const bool inlineSmall = !getenv("MI355X_INLINE_SMALL") || atoi(getenv("MI355X_INLINE_SMALL")) != 0;
+      if (inlineSmall && mat && forced && !nestedUse && loopDepth_ == 0 && !op->has("force_materialize") && v->type.numel() <= kSmallNumel && v->users.size() >= 2) {
+        int budget = 8;
+        if (cheapFromMemory(v, budget)) inlineAnyway_.insert(v);
+      }
       if (mat) { g.clear(); g.push_back(op); }
       groups[v] = g;
     }
@@ -286,7 +312,7 @@ class Planner {
 
   // ---------------------------------------------------------------- emission
   LeafPredicate leafPred() {
-    return [this](Value* v) { return storage_.count(v) != 0; };
+    return [this](Value* v) { return storage_.count(v) != 0 && !inlineAnyway_.count(v); };
   }
 
   int kernelId(const std::string& source) {
@@ -2080,9 +2106,10 @@ class Planner {
   static constexpr size_t kBatchMaxArgs = 192;
   static constexpr size_t kBatchMaxSegments = 24;
 
+  static constexpr unsigned kBatchMaxBigBlocks = 1u << 20;   // one member of a group may be this big: small neighbours ride in its launch
   bool batchCandidate(const Step& s) const {
     return s.kind == Step::Kernel && s.grid[1] == 1 && s.grid[2] == 1 && s.block[0] == 256 && s.block[1] == 1 && s.block[2] == 1 &&
-           s.grid[0] <= kBatchMaxBlocks && s.argWrites.size() == s.args.size() && batchableKernel(P.kernels[s.kernel].source);
+           s.grid[0] <= kBatchMaxBigBlocks && s.argWrites.size() == s.args.size() && batchableKernel(P.kernels[s.kernel].source);
   }
 
   // the shared prelude never declares LDS, so any __shared__ after the kernel header belongs to the body
@@ -2109,7 +2136,9 @@ class Planner {
       // static LDS of the segments adds up in the combined kernel: at most four segments that use any
       auto usesLds = [&](const Step& st) { return ldsInBody(P.kernels[st.kernel].source); };
       size_t ldsSegments = usesLds(steps[i]) ? 1 : 0;
+      size_t bigSegments = steps[i].grid[0] > kBatchMaxBlocks ? 1 : 0;
       while (j < steps.size() && j - i < kBatchMaxSegments && batchCandidate(steps[j]) && nargs + steps[j].args.size() <= kBatchMaxArgs) {
+        if (steps[j].grid[0] > kBatchMaxBlocks) { if (bigSegments >= 1) break; ++bigSegments; }
         if (usesLds(steps[j])) { if (ldsSegments >= 4) break; ++ldsSegments; }
         bool ok = true;
         for (size_t k = i; k < j && ok; ++k) ok = independent(steps[k], steps[j]);
