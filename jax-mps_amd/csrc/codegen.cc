@@ -1121,7 +1121,21 @@ std::string shflXor(const std::string& accT, const std::string& x, const std::st
 
 }  // namespace
 
-FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeafOuter, const std::vector<Value*>& epilogue, int64_t externalPartials) {
+bool reduceIsColumnStyle(const Op* reduce) {
+  const std::vector<int64_t>& shape = reduce->operands[0]->type.dims;
+  const int rank = (int)shape.size();
+  if (rank == 0) return false;
+  std::vector<bool> isRed(rank, false);
+  for (auto d : reduce->ints("dimensions")) if (d >= 0 && d < rank) isRed[(size_t)d] = true;
+  int64_t Kn = 1;
+  for (int d = 0; d < rank; ++d) if (!isRed[d]) Kn *= shape[d];
+  int inner = rank - 1;
+  while (inner > 0 && shape[inner] == 1) --inner;
+  return !isRed[inner] && Kn != 1;   // the same rule as in generateReduceKernel
+}
+
+FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeafOuter, const std::vector<Value*>& epilogue, int64_t externalPartials,
+                               const std::vector<Value*>& sideStores) {
   // values computed from the results right where they are finished (second pass only)
   std::unordered_set<Value*> own;
   for (auto* r : reduces) own.insert(r->result());
@@ -1447,6 +1461,13 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   Index idx = em.multiIndex(full, shape);
   std::vector<std::string> vals;
   for (auto* r : reduces) vals.push_back(em.gen(r->operands[0], idx));
+  // values the caller wants in memory as well: every (row, column) is visited exactly once, so they are stored on the way
+  for (size_t q = 0; q < sideStores.size(); ++q) {
+    Value* sv = sideStores[q];
+    if (sv->type.dims != shape) throw CompileError("codegen: side store of another shape");
+    const std::string e = em.gen(sv, idx);
+    em.body("side" + std::to_string(q) + "[" + em.dimExpr(em.linearize(full, shape)) + "] = " + storeExpr(sv->type.dt, e) + ";");
+  }
   std::string loopPre = em.pre_;
   em.pre_ = savedPre;
   std::vector<std::string> inits;
@@ -1457,6 +1478,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   std::vector<std::string> outs;
   for (size_t j = 0; j < nr; ++j)
     outs.push_back((partial ? ops[j].accT : storageT(ops[j].dt)) + "* __restrict__ out" + std::to_string(j));
+  for (size_t q = 0; q < sideStores.size(); ++q) outs.push_back(storageT(sideStores[q]->type.dt) + "* __restrict__ side" + std::to_string(q));
   s << kernelHeader(em.leaves_, outs) << " {\n";
   s << "  const int tx = threadIdx.x % " << TX << ", ty = threadIdx.x / " << TX << ";\n";
   s << "  const " << IT << " kb = ((" << IT << ")blockIdx.x * " << TX << " + tx) * " << V << ";\n";
@@ -1518,6 +1540,8 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     }
     l.args.push_back(a);
   }
+  for (auto* sv : sideStores) { KArg a; a.kind = KArg::Out; a.value = sv; l.args.push_back(a); }
+  fc.sideStored = !sideStores.empty();
   fc.leaves = em.leaves_;
   fc.launches.push_back(std::move(l));
   if (partial) {

@@ -34,7 +34,8 @@ struct FusedCode {
   int64_t workspaceBytes = 0;
   bool epilogueFused = false;
   std::vector<Value*> leaves;   // distinct materialised inputs
-  std::vector<int64_t> partialOffsets;   // generateReduceKernel with external partials: where each reduction's partial sums sit in the workspace
+  std::vector<int64_t> partialOffsets;
+  bool sideStored = false;          // the side stores asked for are written by the first launch (extra Out arguments)   // generateReduceKernel with external partials: where each reduction's partial sums sit in the workspace
 };
 
 using LeafPredicate = std::function<bool(Value*)>;
@@ -76,7 +77,13 @@ std::string combineKernels(const std::vector<const std::string*>& sources, const
 // produced by the pass that folds partial sums when there is one (FusedCode::epilogueFused), otherwise ignored.
 // `externalPartials` > 0: the partial results (that many per output, float accumulators, partial p of output k at
 // [k * externalPartials + p] from partialOffsets[j] of the workspace) are written by an earlier step; only the folding pass is generated.
-FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeaf, const std::vector<Value*>& epilogue = {}, int64_t externalPartials = 0);
+// `sideStores`: values of the input's shape that the reductions' inputs are computed from and that are needed in memory too:
+// the pass over the data writes them while it reduces (each element is visited exactly once), so no kernel of their own
+// stores them and the reduction does not read them back.  Only honoured by the column-style kernel (FusedCode::sideStored).
+FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredicate& isLeaf, const std::vector<Value*>& epilogue = {}, int64_t externalPartials = 0,
+                               const std::vector<Value*>& sideStores = {});
+// the kernel generateReduceKernel would choose walks the reduced dims with the kept ones across the lanes (column style)
+bool reduceIsColumnStyle(const Op* reduce);
 
 // True if codegen can inline `op` into a consumer (elementwise / indexing ops).
 bool isFusibleOp(const Op& op);

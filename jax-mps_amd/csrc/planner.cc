@@ -111,6 +111,7 @@ class Planner {
   std::unordered_set<int> boundToOutput_;
   std::vector<std::pair<int, int>> loops_;
   std::unordered_set<Op*> emitted_;
+  std::unordered_set<Value*> deferred_;   // values whose own kernel is held back: the reduction that reads them first stores them on the way
   std::unordered_map<Op*, Op*> heldDots_;   // later product of add(dot, dot) -> the earlier one waiting for it
   int time_ = 0;
   // Regions that may execute speculatively (the body of a dynamic loop past its last iteration, the branches of a
@@ -437,6 +438,7 @@ class Planner {
       if (isFusibleOp(*op) && op->results.size() == 1) {
         Value* v = op->result();
         if (!needMat_[v]) return;
+        if (storedByAReduction(op, r, pos)) { deferred_.insert(v); return; }
         emitLoopGroup(op, r, pos, plan);
         return;
       }
@@ -514,6 +516,44 @@ class Planner {
   // Materialised elementwise values with the same dims whose inputs are already in memory are
   // computed by one kernel with several outputs: later ops of the region are pulled forward
   // (SSA values are pure, so computing them earlier is always valid).
+  // A large elementwise value whose first reader is a column-style reduction over the same index space (the masked
+  // gradient that batch norm's backward pass sums twice before it uses it element by element): the reduction's pass
+  // over the data computes it anyway, visits every element exactly once and can store it, so the value needs no
+  // kernel of its own and the reduction does not read it back.  True when `op`'s result is such a value and nothing
+  // before that reduction needs it in memory.
+  bool storedByAReduction(Op* op, Region& r, size_t pos) {
+    static const bool on = !getenv("MI355X_REDUCE_STORES") || atoi(getenv("MI355X_REDUCE_STORES")) != 0;
+    Value* v = op->result();
+    if (!on || loopDepth_ > 0 || !takesKernel(op) || v->type.numel() < 65536 || op->name == "constant" || op->has("force_materialize")) return false;
+    if (v->type.dt != DType::F32 && v->type.dt != DType::BF16) return false;
+    Op* red = nullptr;
+    size_t posRed = 0;
+    for (size_t q = pos + 1; q < r.ops.size() && q <= pos + 48 && !red; ++q) {
+      Op* y = r.ops[q].get();
+      if (y->name != "reduce" || emitted_.count(y) || !isSimpleReduce(*y)) continue;
+      if (y->operands[0]->type.dims != v->type.dims || !reduceIsColumnStyle(y)) continue;
+      std::vector<Value*> leaves;
+      std::unordered_set<Value*> seen;
+      collectLeavesOf(y->operands[0], leaves, seen);
+      if (std::find(leaves.begin(), leaves.end(), v) != leaves.end()) { red = y; posRed = q; }
+    }
+    if (!red) return false;
+    // every reader of the value that comes before the reduction must be content with recomputing it (none should: it
+    // would not have been marked for memory otherwise), and readers in nested regions need it in memory at once
+    for (Op* u : v->users) {
+      if (u->parent != &r) return false;
+      size_t pu = 0;
+      while (pu < r.ops.size() && r.ops[pu].get() != u) ++pu;
+      if (pu < posRed && (!isFusibleOp(*u) || needMat_[u->result()])) return false;
+    }
+    // what the value is computed from must be in memory by now
+    std::vector<Value*> mine;
+    std::unordered_set<Value*> seen;
+    for (auto* o : op->operands) collectLeavesOf(o, mine, seen);
+    for (auto* l : mine) if (!hasStorage(l)) return false;
+    return true;
+  }
+
   void emitLoopGroup(Op* op, Region& r, size_t pos, Plan& plan) {
     Value* v = op->result();
     static const bool multi = !(getenv("MI355X_MULTI_OUTPUT") && getenv("MI355X_MULTI_OUTPUT")[0] == '0');
@@ -744,6 +784,17 @@ class Planner {
       std::unordered_set<Value*> seen;
       collectLeavesOf(op->operands[0], myLeaves, seen);
     }
+    // values held back for this reduction to store (storedByAReduction); any that it cannot take get their own kernel now
+    std::vector<Value*> side;
+    const bool columnStyle = reduceIsColumnStyle(op);
+    auto takeSide = [&](Value* l) {
+      if (!deferred_.count(l) || hasStorage(l)) return false;
+      if (std::find(side.begin(), side.end(), l) != side.end()) return true;
+      if (columnStyle && side.size() < 2 && l->type.dims == op->operands[0]->type.dims) { side.push_back(l); return true; }
+      materializeNow(l, plan);
+      return false;
+    };
+    for (auto* l : myLeaves) takeSide(l);
     // sibling reductions over the same index space that share an input: one pass over memory
     bool seenSelf = false;
     for (auto& qp : r.ops) {
@@ -762,7 +813,7 @@ class Planner {
       collectLeavesOf(q->operands[1], ql, seen);
       bool ready = true, shares = false;
       for (auto* l : ql) {
-        if (!hasStorage(l)) ready = false;
+        if (!hasStorage(l) && !takeSide(l)) ready = hasStorage(l);
         if (std::find(myLeaves.begin(), myLeaves.end(), l) != myLeaves.end() && l->type.numel() > kSmallNumel) shares = true;
       }
       if (ready && shares) group.push_back(q);
@@ -849,7 +900,16 @@ class Planner {
         if (statRows > 0 && (int64_t)abi.O != y->type.dims.back()) statRows = 0;
       }
     }
-    FusedCode fc = generateReduceKernel(group, leafPred(), epilogue, statRows);
+    if (statRows > 0 && !side.empty()) {   // (the folding pass of convolution statistics walks no data)
+      for (auto* l : side) materializeNow(l, plan);
+      side.clear();
+    }
+    FusedCode fc = generateReduceKernel(group, leafPred(), epilogue, statRows, side);
+    if (!side.empty() && !fc.sideStored) {
+      for (auto* l : side) materializeNow(l, plan);
+      side.clear();
+      fc = generateReduceKernel(group, leafPred(), epilogue, statRows);
+    }
     std::vector<Value*> outs;
     for (auto* g : group) {
       bind(g->result(), newStorage(g->result()->type.bytes()));
@@ -865,6 +925,12 @@ class Planner {
         emitted_.insert(epilogueOps[k]);
         label += "+" + epilogueOps[k]->name;
       }
+    }
+    for (auto* l : side) {
+      bind(l, newStorage(l->type.bytes()));
+      outs.push_back(l);
+      emitted_.insert(l->def);
+      label += " storing " + l->def->name;
     }
     if (statRows > 0) {
       ProducerStats ps;
