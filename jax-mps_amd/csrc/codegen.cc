@@ -1121,6 +1121,11 @@ std::string shflXor(const std::string& accT, const std::string& x, const std::st
 
 }  // namespace
 
+int64_t reduceOnePassLimit() {
+  static const int64_t limit = getenv("MI355X_REDUCE_ONE_PASS") ? atoll(getenv("MI355X_REDUCE_ONE_PASS")) : 256 * 1024;
+  return limit;
+}
+
 bool reduceIsColumnStyle(const Op* reduce) {
   const std::vector<int64_t>& shape = reduce->operands[0]->type.dims;
   const int rank = (int)shape.size();
@@ -1443,8 +1448,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   static const int colPerThread = getenv("MI355X_REDUCE_COL_PER_THREAD") ? atoi(getenv("MI355X_REDUCE_COL_PER_THREAD")) : 16;
   if (Rn > (int64_t)TY * 16) P = std::min<int64_t>((Rn + TY * colPerThread - 1) / (TY * colPerThread), std::max<int64_t>(1, 2048 / gridX));
   // a small input is cheaper to walk in one launch (a few dozen loads per lane) than to split over a second, dependent one
-  static const int64_t onePassElems = getenv("MI355X_REDUCE_ONE_PASS") ? atoll(getenv("MI355X_REDUCE_ONE_PASS")) : 256 * 1024;
-  if (Rn * Kn <= onePassElems && Rn <= (int64_t)TY * 128) P = 1;
+  if (Rn * Kn <= reduceOnePassLimit() && Rn <= (int64_t)TY * 128) P = 1;
   bool partial = P > 1;
   Emitter em(isLeaf, V, i64);
   IdxDim klin;

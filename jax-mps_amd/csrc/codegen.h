@@ -84,6 +84,8 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
                                const std::vector<Value*>& sideStores = {});
 // the kernel generateReduceKernel would choose walks the reduced dims with the kept ones across the lanes (column style)
 bool reduceIsColumnStyle(const Op* reduce);
+// column reductions over at most this many input elements run as one launch of a few workgroups
+int64_t reduceOnePassLimit();
 
 // True if codegen can inline `op` into a consumer (elementwise / indexing ops).
 bool isFusibleOp(const Op& op);

@@ -524,7 +524,8 @@ class Planner {
   bool storedByAReduction(Op* op, Region& r, size_t pos) {
     static const bool on = !getenv("MI355X_REDUCE_STORES") || atoi(getenv("MI355X_REDUCE_STORES")) != 0;
     Value* v = op->result();
-    if (!on || loopDepth_ > 0 || !takesKernel(op) || v->type.numel() < 65536 || op->name == "constant" || op->has("force_materialize")) return false;
+    // (a reduction over a small input is one launch of a few workgroups: too few to also compute and store the value)
+    if (!on || loopDepth_ > 0 || !takesKernel(op) || v->type.numel() <= reduceOnePassLimit() || op->name == "constant" || op->has("force_materialize")) return false;
     if (v->type.dt != DType::F32 && v->type.dt != DType::BF16) return false;
     Op* red = nullptr;
     size_t posRed = 0;

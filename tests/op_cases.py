@@ -593,6 +593,25 @@ def _bn_like(b, x, g):
 case("per-channel-chain-after-reduce", _bn_like, f32(2740, 96, 50, 64), f32(2741, 64, lo=0.5, hi=1.5))
 case("per-channel-chain-no-reduce", lambda b, x, g, v: b.mul(x, b.broadcast_in_dim(b.div(g, b.sqrt(b.add(v, 1e-3))), x.shape, [2])),
      f32(2742, 96, 50, 64), f32(2743, 64, lo=0.5, hi=1.5), f32(2744, 64, lo=0.1, hi=2.0))
+# a large elementwise value (batch norm's masked gradient) that a column reduction reads first and elementwise ops read later: the
+# reduction's pass stores it on the way (unless the input is small enough for a one-launch reduction of a few workgroups), next to
+# sibling reductions, in bf16, and when it is also a result
+def _masked_grad_sums(b, x, dy, kept=(3,), also_return=False):
+    red = [d for d in range(x.ndim) if d not in kept]
+    g = b.select(b.compare(x, b.constant(0.0, x.dtype, x.shape), "GT"), dy, b.constant(0.0, x.dtype, x.shape))
+    s1 = b.reduce_sum(g, red)
+    s2 = b.reduce_sum(b.mul(g, x), red)
+    n = float(np.prod([x.shape[d] for d in red]))
+    dx = b.sub(b.sub(g, b.broadcast_in_dim(b.div(s1, n), x.shape, list(kept))), b.mul(x, b.broadcast_in_dim(b.div(s2, n), x.shape, list(kept))))
+    return [dx, g] if also_return else dx
+case("reduce-column-stores-its-input-two-passes", _masked_grad_sums, f32(2750, 32, 16, 32, 32, lo=-1, hi=1), f32(2751, 32, 16, 32, 32, lo=-1, hi=1))
+case("reduce-column-small-input-keeps-its-own-kernel", lambda b, x, dy: _masked_grad_sums(b, x, dy, kept=(1,)), f32(2752, 128, 512, lo=-1, hi=1), f32(2753, 128, 512, lo=-1, hi=1))
+case("reduce-column-stores-its-input-bf16", _masked_grad_sums, f32(2754, 16, 16, 32, 64, lo=-1, hi=1), f32(2755, 16, 16, 32, 64, lo=-1, hi=1), dtypes=["bf16", "bf16"])
+case("reduce-column-stores-its-input-also-a-result", lambda b, x, dy: _masked_grad_sums(b, x, dy, also_return=True),
+     f32(2756, 32, 16, 16, 64, lo=-1, hi=1), f32(2757, 32, 16, 16, 64, lo=-1, hi=1))
+case("reduce-column-input-read-by-a-product-first", lambda b, x, dy, w: (lambda g: [b.matmul(b.reshape(g, (4096, 32)), w), b.reduce_sum(g, [0, 1, 2])])(
+     b.select(b.compare(x, b.constant(0.0, "f32", x.shape), "GT"), dy, b.constant(0.0, "f32", x.shape))),
+     f32(2758, 16, 16, 16, 32, lo=-1, hi=1), f32(2759, 16, 16, 16, 32, lo=-1, hi=1), f32(2760, 32, 8))
 # a reduction finished in one launch whose per-output values ride in the same launch
 case("reduce-then-scale-one-pass", lambda b, x: b.div(b.reduce_sum(x, [0]), 300.0), f32(2745, 300, lo=-1, hi=1))
 case("reduce-rows-then-scale-one-pass", lambda b, x, w: b.mul(b.reduce_sum(x, [1]), w), f32(2746, 70, 90, lo=-1, hi=1), f32(2747, 70))

@@ -126,6 +126,19 @@ def test_relu_rides_in_a_small_product_and_its_mask_reads_the_activation():
     assert r.stdout.count("+ bias + relu") == 1 and " 9 steps" in r.stdout
 
 
+def test_a_column_reduction_stores_the_value_it_reads_first():
+    """A large elementwise value that has to exist in memory and is first read by a column reduction gets no kernel of its
+    own: the reduction's pass over the data writes it.  A product that reads it earlier keeps the separate kernel."""
+    r = plan(op_cases.get_case("reduce-column-stores-its-input-two-passes").text, "--dump-plan")
+    assert r.stdout.count("storing select") == 2 and "fusion:select" not in r.stdout        # the pass over the data and the fold
+    r = plan(op_cases.get_case("reduce-column-small-input-keeps-its-own-kernel").text, "--dump-plan")
+    assert "storing" not in r.stdout and "fusion:select" in r.stdout        # a one-launch reduction has too few workgroups for the extra work
+    r = plan(op_cases.get_case("reduce-column-input-read-by-a-product-first").text, "--dump-plan")
+    assert "storing" not in r.stdout
+    r = plan(configs.build_resnet18().text, "--dump-plan")
+    assert r.stdout.count("storing select") == 34 and "fusion:select" not in r.stdout        # 17 batch-norm backward passes, two launches each
+
+
 def test_location_aliases_result_lists_and_composites_parse():
     text = """#loc1 = loc("x")
 module @jit_f attributes {mhlo.num_partitions = 1 : i32} {
