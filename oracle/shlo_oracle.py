@@ -1065,11 +1065,23 @@ class Oracle:
         self.main = self.funcs["main"]
 
     # -- public
-    def run(self, *args: np.ndarray) -> List[np.ndarray]:
+    def run(self, *args: np.ndarray, pinned: Optional[Dict[int, np.ndarray]] = None) -> List[np.ndarray]:
+        """Evaluate main.  `pinned` maps an output index of main to an array that replaces that value at the point
+        where the program defines it, so everything computed from it afterwards uses the given array (a checker's
+        aid: two float32 evaluations of a ReLU network take different branches at the few activations that lie
+        within rounding noise of zero, and gradients can only be compared element by element once both sides use
+        the same branch decisions).  The values the oracle itself computed there are kept in `self.replaced`."""
         f = self.main
         assert len(args) == len(f.body.args), (len(args), len(f.body.args))
         vals = [_cast_result(np.asarray(a), t) for a, t in zip(args, f.body.arg_types)]
-        return self._run_region(f.body, vals, {})
+        self._pinned, self.replaced = {}, {}
+        if pinned:
+            ret = [op for op in f.body.ops if op.name == "return"][-1]
+            self._pinned = {ret.operands[k]: (k, np.asarray(v)) for k, v in pinned.items()}
+        try:
+            return self._run_region(f.body, vals, {})
+        finally:
+            self._pinned = {}
 
     @property
     def arg_types(self):
@@ -1099,6 +1111,13 @@ class Oracle:
                     env[name] = _cast_result(val, t, keep_shape=vectorized)
                 if name.endswith("#0") and len(op.results) == 1:
                     env[name[:-2]] = env[name]
+                if getattr(self, "_pinned", None) and region is self.main.body:
+                    for alias in (name, name[:-2] if name.endswith("#0") else name):
+                        if alias in self._pinned and alias in env:
+                            k, given = self._pinned[alias]
+                            assert given.shape == env[alias].shape, (alias, given.shape, env[alias].shape)
+                            self.replaced.setdefault(k, env[alias])
+                            env[alias] = given.astype(env[alias].dtype)
         return []
 
     def _eval(self, op: Op, ins, env):
