@@ -4,7 +4,8 @@ on one MI355X through the plugin's PJRT C API, plus fused-op HBM bandwidth.
 Prints ONE JSON line.  `value` is steps/s with all inputs resident in HBM; `roofline` is the
 convolution kernels' achieved fp32 matrix throughput (algorithmic flops / HIP-event time on the
 compute stream, collected by the plugin and read back through PJRT_Executable_GetCostAnalysis);
-`cpu_baseline` is the numpy oracle on a bounded sample of the same workload on the host cores.
+`cpu_baseline` is the same train step on the host cores for a bounded sample: torch's CPU backend (oneDNN)
+with the numpy oracle's rate next to it.
 """
 import argparse
 import json
@@ -102,9 +103,8 @@ def bench_fused_ops(client, iters=10):
     return out
 
 
-def cpu_baseline(budget_s=12.0, batch=128):
-    """The numpy oracle (float32 BLAS accumulation) on whole train steps of the benchmark workload, on the
-    host cores: as many steps as fit the time budget (at least one)."""
+def _numpy_port_baseline(budget_s, batch):
+    """The numpy oracle (float32 BLAS accumulation) on whole train steps of the benchmark workload."""
     from jax_mps_amd.programs import configs
     from shlo_oracle import Oracle
     p = configs.build_resnet18(batch=batch)
@@ -121,8 +121,48 @@ def cpu_baseline(budget_s=12.0, batch=128):
         dt = time.perf_counter() - t0
         if dt >= budget_s or n >= 50:
             break
-    return {"value": round(n / dt, 5), "unit": "steps/s", "cores": os.cpu_count(), "kind": "port", "losses": losses,
+    return {"value": round(n / dt, 5), "unit": "steps/s", "cores": os.cpu_count(), "kind": "port", "engine": "numpy", "losses": losses,
             "sample": f"{n} ResNet18 train step(s) at batch {batch} in {dt:.1f} s (numpy/BLAS float32 interpreter of the same module)"}
+
+
+def _torch_cpu_baseline(budget_s, batch):
+    """The same train step on torch's CPU backend (oneDNN convolutions, autograd; oracle/torch_resnet.py): the
+    closest thing to a CPU framework backend on the benchmark machine, where no jax is installed.  None when
+    torch is not importable."""
+    try:
+        import torch
+        import torch_resnet
+    except ImportError:
+        return None
+    from jax_mps_amd.programs import configs
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1))
+    torch.set_num_threads(threads)
+    p = configs.build_resnet18(batch=batch)
+    ts = torch_resnet.TrainStep(p, configs.resnet18_param_specs(64, 10), 64)
+    losses = [ts.step()]                      # first step: also warms the oneDNN primitive caches
+    n, t0 = 0, time.perf_counter()
+    while True:
+        losses.append(ts.step())
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s or n >= 200:
+            break
+    return {"value": round(n / dt, 4), "unit": "steps/s", "cores": threads, "kind": "port", "engine": f"torch-cpu {torch.__version__}",
+            "losses": losses,
+            "sample": f"{n} ResNet18 train step(s) at batch {batch} in {dt:.1f} s after one untimed step "
+                      f"(torch CPU backend, float32, {threads} threads)"}
+
+
+def cpu_baseline(budget_s=10.0, batch=128):
+    """Host-CPU baseline on a bounded sample of the benchmark workload: the torch-CPU train step when torch is
+    importable (the record's `numpy_port` then holds the numpy oracle's rate next to it), else the numpy oracle."""
+    port = _numpy_port_baseline(budget_s, batch)
+    tc = _torch_cpu_baseline(budget_s, batch)
+    if tc is None:
+        return port
+    tc["numpy_port"] = {k: port[k] for k in ("value", "unit", "cores", "sample")}
+    tc["numpy_losses"] = port["losses"]
+    return tc
 
 
 # HBM bytes per conv_igemm_f32 launch of this workload: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by
@@ -260,8 +300,9 @@ def main():
         line["speedup_vs_cpu_baseline"] = round(line["value"] / line["cpu_baseline"]["value"], 1)
         # the same steps from the same initial state on both sides: the losses must agree to float32 accumulation noise
         want = line["cpu_baseline"].pop("losses")[:len(first_losses)]
+        others = line["cpu_baseline"].pop("numpy_losses", [])[:len(first_losses)]
         got = first_losses[:len(want)]
-        rel = max(abs(g - w) / max(abs(w), 1e-30) for g, w in zip(got, want))
+        rel = max(abs(g - w) / max(abs(w), 1e-30) for ws in (want, others) for g, w in zip(got, ws))
         ok = rel <= LOSS_CHECK_RTOL
         line["loss_check"] = {"steps": len(want), "gpu": [round(g, 6) for g in got], "cpu": [round(w, 6) for w in want],
                               "max_rel_diff": float("%.3g" % rel), "rtol": LOSS_CHECK_RTOL, "ok": ok}

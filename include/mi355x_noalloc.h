@@ -35,9 +35,11 @@ typedef struct {
  * already holds the operand and is updated in place; all three pointers are device memory of the current HIP
  * device; the work is enqueued on `hip_stream` (a hipStream_t, NULL = the null stream) and not waited for.
  *
- * Returns 0 on success.  Otherwise nothing was enqueued, the return value is non-zero (1 = invalid argument,
- * 2 = num_updates above MI355X_NOALLOC_MAX_UPDATES, other = HIP error code) and, if `error` is non-NULL, a
- * NUL-terminated description is written into error[0 .. error_len).
+ * Returns 0 on success.  1 = invalid argument, 2 = num_updates above MI355X_NOALLOC_MAX_UPDATES, 3 = the sizes need
+ * more workgroups than one launch holds (row_elems above 16 776 960); these three are found before anything is
+ * enqueued.  1000 + e = the HIP runtime reported error e (resolving the workspace, or a launch; launches before the
+ * failing one may have been enqueued and `result` is then undefined).  If `error` is non-NULL a NUL-terminated
+ * description is written into error[0 .. error_len).
  *
  * All calls on one GPU share that GPU's workspace: calls that may run concurrently on one GPU (different
  * streams or threads) race and must be serialised by the caller.  Nothing in the workspace has to start at

@@ -16,10 +16,15 @@ from __future__ import annotations
 
 import os
 import subprocess
+import warnings
+from importlib import metadata
 from pathlib import Path
 
 PLATFORM_NAME = "mi355x"
 LIB_NAME = "libpjrt_plugin_mi355x.so"
+# jaxlib release line whose PJRT C API (0.72) and StableHLO bytecode version the library was written against: the one
+# the reference pins (src/jax_plugins/mps/__init__.py:8-10)
+BUILT_FOR_JAXLIB = (0, 10)
 _PKG_DIR = Path(os.path.dirname(os.path.abspath(__file__)))
 
 
@@ -45,6 +50,22 @@ def find_library() -> str | None:
     return override
 
 
+def check_jaxlib_version() -> None:
+    """Warn when the installed jaxlib is of another major.minor line than the one the library was written against
+    (the PJRT function table and the bytecode version both move with it); never fails initialisation.  Mirrors
+    src/jax_plugins/mps/__init__.py:63-91."""
+    try:
+        installed = metadata.version("jaxlib")
+        major, minor = (int(x) for x in installed.split(".")[:2])
+    except (metadata.PackageNotFoundError, ValueError):
+        return
+    if (major, minor) != BUILT_FOR_JAXLIB:
+        want = "%d.%d" % BUILT_FOR_JAXLIB
+        warnings.warn(f"the {PLATFORM_NAME} plugin was written against jaxlib {want}.x but jaxlib {installed} is installed: "
+                      f"the PJRT function table or the StableHLO bytecode version may differ "
+                      f"(consider jaxlib>={want}.0,<{BUILT_FOR_JAXLIB[0]}.{BUILT_FOR_JAXLIB[1] + 1})", stacklevel=3)
+
+
 def _register(xla_bridge, library_path: str) -> None:
     try:
         xla_bridge.register_plugin(PLATFORM_NAME, priority=500, library_path=library_path, options=None)
@@ -60,6 +81,7 @@ def initialize() -> None:
 
     Needs jax with `xla_bridge.register_plugin`; anything missing raises Mi355xPluginError so that jax's
     plugin discovery reports it instead of silently running elsewhere."""
+    check_jaxlib_version()
     library_path = find_library()
     if library_path is None:
         raise Mi355xPluginError(f"{LIB_NAME} is neither next to {_PKG_DIR} nor named by MI355X_PJRT_LIBRARY_PATH; "
@@ -92,10 +114,12 @@ def build_library(force: bool = True, jobs: int = 8) -> str:
     return str(_PKG_DIR / LIB_NAME)
 
 
-def aot_compile(mlir_paths, quiet: bool = True) -> str:
-    """Cross-compile the fused kernels of StableHLO text files into the kernel cache (no GPU needed)."""
+def aot_compile(mlir_paths, quiet: bool = True, env: dict | None = None) -> str:
+    """Cross-compile the fused kernels of StableHLO text files into the kernel cache (no GPU needed).
+    `env` adds compile switches (the MI355X_* variables the planner reads at every compile)."""
     tool = _PKG_DIR / "mi355x-aot"
-    r = subprocess.run([str(tool)] + [str(p) for p in mlir_paths], capture_output=True, text=True)
+    r = subprocess.run([str(tool)] + [str(p) for p in mlir_paths], capture_output=True, text=True,
+                       env={**os.environ, **(env or {})})
     if r.returncode != 0:
         raise Mi355xPluginError("ahead-of-time kernel compilation failed:\n" + r.stdout[-4000:] + r.stderr[-4000:])
     return r.stdout

@@ -136,6 +136,7 @@ struct BAttr {
   int type = -1;                              // Int / Float / Tensor / Type: type index
   std::vector<uint8_t> blob;                  // Tensor: raw element data
   std::vector<int64_t> ints;                  // TypeExtensions bounds
+  std::string origin;                         // Unknown: which encoding was not understood, for the error that names it
 };
 
 struct Entry {
@@ -401,7 +402,7 @@ class Converter {
           a.i = c.svarint();   // widths up to 64 bits; one-byte form for widths <= 8 is not used by module attributes read here
           break;
         }
-        default: a.kind = BAttr::Unknown; break;   // locations and other attributes nothing here reads
+        default: a.kind = BAttr::Unknown; a.origin = "builtin attribute code " + std::to_string(code); break;   // locations and other attributes nothing here reads
       }
     } else if (dialect == "vhlo") {
       uint64_t code = c.varint();
@@ -466,10 +467,11 @@ class Converter {
           for (uint64_t k = 0; k < n; ++k) a.ints.push_back(c.svarint());
           break;
         }
-        default: a.kind = BAttr::Unknown; break;   // output_operand_alias, result_accuracy: nothing on this path reads them
+        default: a.kind = BAttr::Unknown; a.origin = "vhlo attribute code " + std::to_string(code); break;   // output_operand_alias, result_accuracy: nothing on this path reads them
       }
     } else {
       a.kind = BAttr::Unknown;
+      a.origin = "an attribute of dialect '" + dialect + "'";
     }
     attrs_[idx] = std::move(a);
     return attrs_[idx];
@@ -651,7 +653,15 @@ class Converter {
     if (!dict) return "";
     std::vector<std::string> parts;
     std::vector<std::string> done;
-    auto take = [&](const char* k) { done.push_back(k); return find(dict, k); };
+    // an attribute the op's meaning depends on must have been understood: one whose encoding this reader does not know
+    // is a compile error that names it, never a silent default
+    auto known = [&](const std::string& k, const BAttr* a) {
+      if (a && a->kind == BAttr::Unknown)
+        bad("attribute '" + k + "' of vhlo." + name + " is encoded as " + (a->origin.empty() ? std::string("a textual attribute") : a->origin) +
+            ", which this reader does not know");
+      return a;
+    };
+    auto take = [&](const char* k) { done.push_back(k); return known(k, find(dict, k)); };
     auto dims = [&](const char* k) { return list(intsOf(take(k))); };
     if (name == "dot_general") {
       parts.push_back("dot_dimension_numbers = #stablehlo.dot<lhs_batching_dimensions = " + dims("lhs_batching_dimensions") + ", rhs_batching_dimensions = " +
@@ -713,7 +723,7 @@ class Converter {
       for (auto* s : skip) if (k == s) handled = true;
       if (handled) continue;
       const BAttr& v = attr((uint64_t)kv.second);
-      if (v.kind == BAttr::Unknown) continue;
+      known(k, &v);
       if (name == "compare" && k == "compare_type" && v.s == "NOTYPE") continue;
       if (name == "custom_call" && k == "backend_config" && v.kind != BAttr::String) continue;
       std::string text;

@@ -482,9 +482,10 @@ class Emitter {
   // 16-bit float results are computed in fp32.  Inside a fused chain they are rounded to their
   // own precision only where the program asks for the narrowing (convert and friends) or where
   // they are stored; rounding after every arithmetic op (MI355X_STRICT_BF16=1) costs two
-  // instructions per op and only loses accuracy.
+  // instructions per op and only loses accuracy.  The switch is read at every compile, like the
+  // reference's JAX_MPS_NO_OPTIMIZE (stablehlo_parser.cc:83-85), so one process can hold programs of both kinds.
   std::string def(const TensorType& t, const std::string& expr, bool inBody, bool narrowing = true) {
-    static const bool strict = getenv("MI355X_STRICT_BF16") && getenv("MI355X_STRICT_BF16")[0] == '1';
+    const bool strict = strictBf16();
     std::string name = fresh("t");
     const bool inB = inBody || guard_ > 0 || mentionsBody(expr);
     if (inB) bodyNames_.insert(name);

@@ -12,9 +12,19 @@
 #include <string>
 #include <vector>
 
+#include <cstdlib>
+
 #include "ir.h"
 
 namespace mi355 {
+
+// MI355X_STRICT_BF16=1: every 16-bit float op rounds its result as the program's types say, and the fusions that move
+// a rounding point (activation in the GEMM epilogue, the one-launch attention kernel) are off.  Read at every compile.
+inline bool strictBf16() {
+  const char* e = getenv("MI355X_STRICT_BF16");
+  return e && e[0] == '1';
+}
+
 
 struct KArg {
   enum Kind { In, Out, Work } kind = In;

@@ -137,6 +137,9 @@ typedef struct {
 // Deterministic row scatter: updates are applied to each destination row in the order they
 // appear in `indices` (stable sort by row, then one pass per row segment).  `result` already
 // holds the operand.  `workspace` needs mi355_scatter_workspace_bytes(numUpdates) bytes.
+// returned (before anything is enqueued) when a fold launch would need more workgroups than a grid holds; negative so
+// that it cannot be mistaken for a HIP error code
+#define MI355_SCATTER_GRID_TOO_LARGE (-3)
 int mi355_scatter_rows(const mi355_scatter_desc* d, void* result, const void* indices, const void* updates,
                        void* workspace, mi355_stream_t s);
 // The same with the operand given as a splat: when `fill` is set, `result` need not hold anything on entry and every

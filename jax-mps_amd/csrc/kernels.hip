@@ -1222,6 +1222,12 @@ int mi355_scatter_rows_fill(const mi355_scatter_desc* d, void* result, const voi
   long long n = d->numUpdates;
   hipStream_t st = (hipStream_t)s;
   const int elemBytes = d->dtype == 1 ? 2 : 4;
+  if (d->dtype < 0 || d->dtype > 3) return 2;
+  // grids of the fold launches, checked before anything is enqueued
+  const long long chunksHuge = (d->rowElems + kHugeCols - 1) / kHugeCols, chunksLong = (d->rowElems + 63) / 64;
+  const long long blocksHuge = chunksHuge * ((n + kHugeSegment - 1) / kHugeSegment), blocksLong = chunksLong * ((n + kLongSegment - 1) / kLongSegment);
+  if (blocksHuge > 0x7FFFFFFFll || blocksLong > 0x7FFFFFFFll || n > 0x7FFFFFFFll || (d->rowElems + 255) / 256 > 65535)
+    return MI355_SCATTER_GRID_TOO_LARGE;
   const unsigned long long fillBytes = fill ? (unsigned long long)d->operandRows * d->rowElems * elemBytes : 0;
   if (elemBytes == 2) fillBits = (fillBits & 0xFFFFu) | (fillBits << 16);
   // enough workgroups of 1024 lanes to keep every CU writing, each lane storing a few times
@@ -1262,9 +1268,6 @@ int mi355_scatter_rows_fill(const mi355_scatter_desc* d, void* result, const voi
     t = vin; vin = vout; vout = t;
   }
   dim3 gridShort((unsigned)n, (unsigned)((d->rowElems + 255) / 256));
-  const long long chunksHuge = (d->rowElems + kHugeCols - 1) / kHugeCols, chunksLong = (d->rowElems + 63) / 64;
-  const long long blocksHuge = chunksHuge * ((n + kHugeSegment - 1) / kHugeSegment), blocksLong = chunksLong * ((n + kLongSegment - 1) / kLongSegment);
-  if (blocksHuge > 0x7FFFFFFFll || blocksLong > 0x7FFFFFFFll) return 3;   // more workgroups than a grid holds
 #define FOLD(P) do { \
     if (n >= kHugeSegment) scatter_fold_huge<P><<<(unsigned)blocksHuge, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (typename P::S*)result, (const typename P::S*)updates, (u32)d->operandRows, (u32)chunksHuge); \
     if (n >= kLongSegment) scatter_fold_long<P><<<(unsigned)blocksLong, 256, 0, st>>>(kin, vin, n, d->rowElems, d->kind, (typename P::S*)result, (const typename P::S*)updates, (u32)d->operandRows, (u32)chunksLong); \
@@ -1273,8 +1276,7 @@ int mi355_scatter_rows_fill(const mi355_scatter_desc* d, void* result, const voi
   if (d->dtype == 0) FOLD(Plain<float>);
   else if (d->dtype == 2) FOLD(Plain<int>);
   else if (d->dtype == 3) FOLD(Plain<u32>);
-  else if (d->dtype == 1) FOLD(Bf16);
-  else return 2;
+  else FOLD(Bf16);
 #undef FOLD
   return check("scatter_rows");
 }
@@ -1318,7 +1320,7 @@ static int noallocScratch(void** out, char* error, size_t error_len) {
   }
   if (e != hipSuccess) {
     if (error && error_len) snprintf(error, error_len, "mi355x_scatter_rows_noalloc: cannot resolve the workspace on device %d: %s", dev, hipGetErrorString(e));
-    return (int)e;
+    return 1000 + (int)e;
   }
   return 0;
 }
@@ -1362,8 +1364,10 @@ int mi355x_scatter_rows_noalloc(const mi355x_scatter_desc* desc, void* result, c
   d.dtype = desc->dtype;
   d.index_bytes = desc->index_bytes;
   int rc = mi355_scatter_rows(&d, result, indices, updates, ws, (mi355_stream_t)hip_stream);
+  if (rc == MI355_SCATTER_GRID_TOO_LARGE)      // found before any launch
+    return fail(3, "row_elems x num_updates needs more workgroups than one launch holds (row_elems above 16 776 960, or a fold grid above 2^31 - 1)");
   if (rc != 0 && error && error_len) snprintf(error, error_len, "mi355x_scatter_rows_noalloc: kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
-  return rc;
+  return rc == 0 ? 0 : 1000 + rc;
 }
 
 }  // extern "C"

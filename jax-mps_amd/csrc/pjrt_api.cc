@@ -761,7 +761,7 @@ PJRT_Error* Buffer_OnDeviceSizeInBytes(PJRT_Buffer_OnDeviceSizeInBytes_Args* a) 
 PJRT_Error* Buffer_Device(PJRT_Buffer_Device_Args* a) { a->device = &a->buffer->client->device; return nullptr; }
 PJRT_Error* Buffer_Memory(PJRT_Buffer_Memory_Args* a) { a->memory = &a->buffer->client->memory; return nullptr; }
 // Marks the buffer deleted and gives its memory back to the allocator now (work already enqueued that reads it is
-// ordered before any reuse, because everything runs on one stream); the handle lives on until Buffer_Destroy.
+// ordered before any reuse, because every use is ordered on the main stream: side-stream work is joined before Execute returns or fails); the handle lives on until Buffer_Destroy.
 // The reference only sets the flag (mlx_buffer.cc:290-296) and lets MLX's reference counting free the array.
 PJRT_Error* Buffer_Delete(PJRT_Buffer_Delete_Args* a) {
   return guard([&]() -> PJRT_Error* {

@@ -1134,7 +1134,7 @@ class Planner {
 
   // the chain of same-shape elementwise ops that is the only reader of `x` and has one value read from outside
   bool matchActivation(Value* x, ActMatch& m) {
-    static const bool on = !getenv("MI355X_GEMM_ACT") || atoi(getenv("MI355X_GEMM_ACT")) != 0;
+    const bool on = !strictBf16() && (!getenv("MI355X_GEMM_ACT") || atoi(getenv("MI355X_GEMM_ACT")) != 0);   // read per compile
     if (!on || x->type.dt != DType::BF16 || x->users.empty() || !x->def) return false;
     Region* r = x->def->parent;
     std::unordered_set<Op*> in;
@@ -1240,7 +1240,7 @@ class Planner {
   }
 
   static bool matchAttention(Op* pv, AttnMatch& m) {
-    static const bool on = !getenv("MI355X_ATTENTION") || atoi(getenv("MI355X_ATTENTION")) != 0;
+    const bool on = !strictBf16() && (!getenv("MI355X_ATTENTION") || atoi(getenv("MI355X_ATTENTION")) != 0);   // read per compile
     if (!on || pv->name != "dot_general") return false;
     Value* p = pv->operands[0];
     Value* v = pv->operands[1];

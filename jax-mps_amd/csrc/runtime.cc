@@ -198,8 +198,9 @@ void Device::release(void* ptr) {
   auto it = sizes_.find(ptr);
   if (it == sizes_.end()) return;
   inUse_ -= (int64_t)it->second;
-  // All work is issued on one stream, so a recycled block is only touched by work that is
-  // ordered after everything that used it before.
+  // Every use of a block is ordered on the main stream: work a plan puts on its second stream is joined into the
+  // main stream before execute returns or throws (Executable::runPlan).  So a recycled block is only touched by
+  // work that is ordered after everything that used it before.
   free_.emplace(it->second, ptr);
 }
 
@@ -501,8 +502,10 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       d.index_bytes = (int)dtypeSize(s.scatter.indexType);
       if ((size_t)s.workspaceBytes < mi355_scatter_workspace_bytes(d.numUpdates))
         throw RuntimeError("internal: scatter workspace is smaller than the kernel needs");
-      check(mi355_scatter_rows_fill(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out),
-                                    resolve(s.args[3], in, out), s.scatter.fill ? 1 : 0, s.scatter.fillBits, st), "scatter");
+      const int rc = mi355_scatter_rows_fill(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), resolve(s.args[2], in, out),
+                                             resolve(s.args[3], in, out), s.scatter.fill ? 1 : 0, s.scatter.fillBits, st);
+      if (rc == MI355_SCATTER_GRID_TOO_LARGE) throw RuntimeError("scatter: rows this long or updates this many need more workgroups than one launch holds");
+      check(rc, "scatter");
       break;
     }
     case Step::Copy: {
@@ -741,24 +744,34 @@ void Executable::runPlan(const Plan& plan, const std::vector<DeviceBuffer*>& in,
     forkDone_.push_back(b);
   }
   std::vector<char> pending((size_t)plan.numForks, 0);
-  for (auto& s : plan.steps) {
-    for (int id : s.joins) {
-      if (!pending[(size_t)id]) continue;
-      check(mi355_stream_wait_event(dev.stream(), forkDone_[(size_t)id]), "join");
-      pending[(size_t)id] = 0;
+  bool sideDirty = false;     // something was enqueued on the second stream that the main stream has not joined yet
+  try {
+    for (auto& s : plan.steps) {
+      for (int id : s.joins) {
+        if (!pending[(size_t)id]) continue;
+        check(mi355_stream_wait_event(dev.stream(), forkDone_[(size_t)id]), "join");
+        pending[(size_t)id] = 0;
+      }
+      if (s.forkId < 0) { runStep(s, in, out); continue; }
+      const size_t id = (size_t)s.forkId;
+      check(mi355_event_record(forkStart_[id], dev.stream()), "fork");
+      check(mi355_stream_wait_event(sideStream_, forkStart_[id]), "fork");
+      streamOverride_ = sideStream_;
+      sideDirty = true;
+      try { runStep(s, in, out); } catch (...) { streamOverride_ = nullptr; throw; }
+      streamOverride_ = nullptr;
+      check(mi355_event_record(forkDone_[id], sideStream_), "fork");
+      pending[id] = 1;
     }
-    if (s.forkId < 0) { runStep(s, in, out); continue; }
-    const size_t id = (size_t)s.forkId;
-    check(mi355_event_record(forkStart_[id], dev.stream()), "fork");
-    check(mi355_stream_wait_event(sideStream_, forkStart_[id]), "fork");
-    streamOverride_ = sideStream_;
-    try { runStep(s, in, out); } catch (...) { streamOverride_ = nullptr; throw; }
-    streamOverride_ = nullptr;
-    check(mi355_event_record(forkDone_[id], sideStream_), "fork");
-    pending[id] = 1;
+    for (size_t id = 0; id < pending.size(); ++id)
+      if (pending[id]) check(mi355_stream_wait_event(dev.stream(), forkDone_[id]), "join");
+  } catch (...) {
+    // Invariant the allocator relies on: side-stream work is always joined before execute returns or throws, because
+    // blocks released afterwards are recycled on the assumption that the main stream orders every use of them.  On
+    // the error path the host waits for the second stream (the failing step may have left it without a done event).
+    if (sideDirty) mi355_stream_sync(sideStream_);
+    throw;
   }
-  for (size_t id = 0; id < pending.size(); ++id)
-    if (pending[id]) check(mi355_stream_wait_event(dev.stream(), forkDone_[id]), "join");
 }
 
 std::vector<std::shared_ptr<DeviceBuffer>> Executable::execute(const std::vector<DeviceBuffer*>& inputs, const std::vector<bool>* mayDonate) {

@@ -26,10 +26,13 @@ def test_exports_only_the_declared_symbols():
     noalloc = (ROOT / "include" / "mi355x_noalloc.h").read_text()
     declared += re.findall(r"^int (mi355x_\w+)\(", noalloc, flags=re.M)
     assert declared == ["GetPjrtApi", "mi355x_scatter_rows_noalloc"]
+    # every defined dynamic symbol of whatever kind (functions, kernel handles, weak template instantiations, data):
+    # the reference's build hides all but its entry point (CMakeLists.txt:303-318) and so does the linker script
+    # csrc/exports.map; only the HIP toolchain's own __hip_* bookkeeping symbols would be tolerated
     out = subprocess.run(["nm", "-D", "--defined-only", pjrt.default_library_path()], capture_output=True, text=True, check=True).stdout
-    syms = {line.split()[-1] for line in out.splitlines() if " T " in line or " W " in line}
-    ours = {s for s in syms if "PJRT" in s.upper() or "mi355" in s.lower() or s == "GetPjrtApi"}
-    assert ours == set(declared), ours
+    syms = {line.split()[-1] for line in out.splitlines() if line.strip()}
+    ours = {s for s in syms if not s.startswith("__hip_")}
+    assert ours == set(declared), sorted(ours ^ set(declared))[:20]
 
 
 def test_noalloc_descriptor_mirrors_the_header():

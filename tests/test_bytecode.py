@@ -113,6 +113,21 @@ def test_donation_attributes_travel():
     assert "tf.aliasing_output = 0 : i32" in r.stdout
 
 
+def test_unknown_encoding_of_a_used_attribute_is_a_compile_error():
+    """An attribute an op's meaning depends on, written with an attribute code the reader does not know, must stop the
+    compile with an error that names the attribute and the op: never a silently defaulted comparison."""
+    from vhlo_writer import Writer
+
+    class FutureWriter(Writer):
+        def a_enum(self, code, names, value):
+            key = super().a_enum(code, names, value)
+            return (key[0], key[1], 250, key[3]) if "LT" in names else key     # comparison_direction in an encoding of the future
+    c = op_cases.get_case("compare-f32-LT")
+    r = _to_text(FutureWriter(c.text).write(), "--no-compile")
+    assert r.returncode == 1, r.stdout
+    assert "comparison_direction" in r.stderr and "vhlo.compare" in r.stderr and "attribute code 250" in r.stderr, r.stderr[-400:]
+
+
 @pytest.mark.parametrize("damage", ["truncate", "bad_magic_version", "bad_section"])
 def test_damaged_files_are_compile_errors_not_crashes(damage):
     good = to_vhlo_bytecode(configs.build_mlp(**configs.SMALL["mlp"]).text)

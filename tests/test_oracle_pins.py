@@ -206,41 +206,14 @@ def test_mlp_program_vs_torch():
 
 
 def _torch_resnet(p, width):
+    """Loss and gradients of the program's network from torch autograd in float64 (oracle/torch_resnet.py)."""
+    import torch_resnet
     specs = configs.resnet18_param_specs(width, 10)
     n = len(specs)
     P = {nm: torch.tensor(a, dtype=torch.float64, requires_grad=True) for (nm, _, _), a in zip(specs, p.inputs[:n])}
     x = torch.tensor(p.inputs[-2], dtype=torch.float64).permute(0, 3, 1, 2)
     y = torch.tensor(p.inputs[-1]).long()
-
-    def conv(name, h, stride):
-        w = P[name + ".kernel"].permute(3, 2, 0, 1)
-        k = w.shape[2]
-        n_in = h.shape[2]
-        out = -(-n_in // stride)
-        tot = max((out - 1) * stride + k - n_in, 0)
-        lo, hi = tot // 2, tot - tot // 2
-        return F.conv2d(F.pad(h, (lo, hi, lo, hi)), w, stride=stride)
-
-    def bn(name, h):
-        m = h.mean((0, 2, 3))
-        v = torch.clamp((h * h).mean((0, 2, 3)) - m * m, min=0)
-        return (h - m[None, :, None, None]) * (torch.rsqrt(v + 1e-5) * P[name + ".scale"])[None, :, None, None] + P[name + ".bias"][None, :, None, None]
-
-    h = torch.relu(bn("bn_init", conv("conv_init", x, 1)))
-    cin = width
-    for stage, mult in enumerate((1, 2, 4, 8), 1):
-        cout = width * mult
-        for blk in (1, 2):
-            stride = 2 if (stage > 1 and blk == 1) else 1
-            pn = f"stage{stage}_block{blk}"
-            r = h
-            yv = torch.relu(bn(pn + ".bn1", conv(pn + ".conv1", h, stride)))
-            yv = bn(pn + ".bn2", conv(pn + ".conv2", yv, 1))
-            if cin != cout or stride != 1:
-                r = bn(pn + ".bn_proj", conv(pn + ".conv_proj", r, stride))
-            h = torch.relu(r + yv)
-            cin = cout
-    loss = F.cross_entropy(h.mean((2, 3)) @ P["dense.kernel"] + P["dense.bias"], y)
+    loss = torch_resnet.forward(P, x, y, width)
     loss.backward()
     return specs, P, loss
 
@@ -257,6 +230,33 @@ def test_resnet18_program_vs_torch():
         mom = out[n + nstat + i]          # new momentum = grad (old momentum is zero)
         assert np.abs(mom - g).max() <= 2e-5 * (np.abs(g).max() + 1e-12), nm
         np.testing.assert_allclose(out[i], p.inputs[i] - 0.1 * g, rtol=0, atol=3e-6 * (np.abs(g).max() + 1))
+
+
+def test_torch_train_step_is_the_program(tmp_path):
+    """The torch-CPU train step that bench.py times as its host baseline computes the benchmark program: two chained
+    steps in float64 against the oracle's, every parameter, running statistic, momentum and the loss."""
+    import torch_resnet
+    p = configs.build_resnet18(**configs.SMALL["resnet18"])      # batch 8, 16x16, width 8, every scale one
+    specs = configs.resnet18_param_specs(8, 10)
+    ts = torch_resnet.TrainStep(p, specs, 8, dtype=torch.float64)
+    oracle = Oracle(p.text)
+    state = list(p.inputs)
+    n = len(specs)
+    for step in range(2):
+        out = oracle.run(*state)
+        for k, i in p.feedback.items():
+            state[i] = out[k]
+        loss = ts.step()
+        # the oracle's state is float32 between steps, torch's stays float64
+        assert abs(loss - float(out[-1])) < (2e-5 if step == 0 else 2e-4)
+    for i, nm in enumerate(ts.names):
+        np.testing.assert_allclose(out[i], ts.P[nm].detach().numpy(), rtol=0, atol=2e-5 * (np.abs(out[i]).max() + 1), err_msg=nm)
+    for k, r in enumerate(ts.running):
+        np.testing.assert_allclose(out[n + k], r.numpy(), rtol=1e-4, atol=1e-5)
+    n_stats = len(ts.running)
+    for i, nm in enumerate(ts.names):
+        mom = out[n + n_stats + i]
+        np.testing.assert_allclose(mom, ts.M[nm].numpy(), rtol=0, atol=1e-4 * (np.abs(mom).max() + 1e-12), err_msg=nm)
 
 
 def test_embedding_program_vs_numpy():

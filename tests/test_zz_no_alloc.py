@@ -10,7 +10,10 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 # (rows, cols, updates, combiner, seed) of the calls below, in order; the build step compiles their programs ahead of time
-CASES = [(5000, 768, 8192, "add", 11), (300, 96, 1000, "add", 12), (300, 96, 37, "max", 13)]
+# the first is the largest the fixed workspace holds and the second lies just above the one-workgroup sort's limit: both
+# take the general radix sort, whose second key / position arrays and counters are the upper three quarters of the workspace
+CASES = [(3000, 32, 262144, "add", 9), (700, 64, 9000, "add", 10), (5000, 768, 8192, "add", 11), (300, 96, 1000, "add", 12),
+         (300, 96, 37, "max", 13)]
 
 
 def _scatter_program(rows, cols, n, kind):
@@ -78,6 +81,9 @@ def test_scatter_rows_noalloc_rejects_oversize_and_bad_arguments(client):
     with pytest.raises(pjrt.PjrtError) as e:
         pjrt.scatter_rows_noalloc(client.plugin, 0, 0, 0, num_updates=4, row_elems=4, operand_rows=4)
     assert e.value.code == 1
+    with pytest.raises(pjrt.PjrtError) as e:      # rows too long for one launch's grid: refused before any launch
+        pjrt.scatter_rows_noalloc(client.plugin, 1, 1, 1, num_updates=4, row_elems=16776961, operand_rows=4)
+    assert e.value.code == 3 and "more workgroups" in str(e.value)
     with pytest.raises(pjrt.PjrtError) as e:
         pjrt.scatter_rows_noalloc(client.plugin, 1, 1, 1, num_updates=4, row_elems=4, operand_rows=4, index_bytes=2)
     assert e.value.code == 1
