@@ -572,6 +572,7 @@ PJRT_Error* Executable_GetCostAnalysis(PJRT_Executable_GetCostAnalysis_Args* a) 
     vals.emplace_back("arena_bytes", (double)p.arenaBytes);
     vals.emplace_back("compile_seconds", e->exe->compileSeconds);
     vals.emplace_back("loop.host_syncs", (double)e->exe->loopHostSyncs());
+    vals.emplace_back("plan.graph_launches", (double)e->exe->planGraphLaunches());
     for (auto& kv : e->exe->timings()) {
       vals.emplace_back(kv.first + ".count", (double)kv.second.count);
       vals.emplace_back(kv.first + ".time_ms", kv.second.ms);

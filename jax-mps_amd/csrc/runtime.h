@@ -92,6 +92,7 @@ class Executable {
   std::map<std::string, KindStat> timings();
   double compileSeconds = 0;
   int64_t loopHostSyncs() const { return loopSyncs_; }   // host round trips spent reading loop flags so far
+  int64_t planGraphLaunches() const { return planGraphLaunches_; }   // execute calls served by one graph launch
 
  private:
   std::unique_ptr<CompiledProgram> prog_;
@@ -126,10 +127,22 @@ class Executable {
     std::vector<LoopGraph> entries;    // a few recent address sets (buffers recycle through the allocator)
   };
   std::map<const Step*, LoopGraphs> loopGraphs_;
+  // The whole plan of a program without loops as one graph (one host call per execute instead of one per launch).
+  // Buffers recycle through the allocator, so the address sets of successive calls repeat with a short period: a set is
+  // captured the second time it is seen and a few graphs are kept.  Callers whose addresses never repeat keep running
+  // launch by launch, and after a number of calls without a single repeat the executable stops looking.
+  struct PlanGraph { mi355_graph_t exec = nullptr; uint64_t signature = 0; uint64_t lastUse = 0; };
+  std::vector<PlanGraph> planGraphs_;
+  std::vector<uint64_t> seenSignatures_;
+  bool planGraphsOn_ = false;        // MI355X_PLAN_GRAPHS=1 when the executable was made
+  int planGraphState_ = -1;          // -1 not examined, 0 not eligible / given up, 1 eligible
+  int64_t planGraphMisses_ = 0, planGraphLaunches_ = 0;
+  bool runPlanFromGraph(const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
   uint64_t graphClock_ = 0;
   std::map<const Plan*, bool> capturable_;
   bool useGraphs_ = true;
   bool capturing_ = false;
+  bool forkingAllowed_ = true;        // cleared while a plan is captured with everything on one stream
   bool capturable(const Plan& p);
   void runCountedLoop(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
   void runDeviceLoop(const Step& s, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out);
