@@ -146,7 +146,8 @@ std::unique_ptr<Module> parseStableHLOText(const char* data, size_t size);
 bool isMlirBytecode(const char* data, size_t size);
 std::string vhloBytecodeToStableHLOText(const char* data, size_t size);
 
-// Passes (passes.cc)
+// Passes (passes.cc, fused_calls.cc)
+void lowerFusedOpCalls(Module& m);   // custom_call @mps.sdpa / rms_norm / layer_norm / rope / gelu and their backward forms -> calls of StableHLO functions
 void inlineCalls(Module& m);          // replaces every "call" by the callee body
 void lowerIntegerDots(Module& m);    // integer / boolean dot_general -> broadcast, multiply, reduce
 void lowerSingleDeviceOps(Module& m);  // one-device all_reduce -> operands, partition_id / replica_id -> 0, tokens -> f32 scalar placeholders

@@ -2480,6 +2480,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
     prog->paramDonation = mainFn->argDonation;
     prog->paramDonation.resize(mainFn->body.args.size(), -1);
   }
+  lowerFusedOpCalls(*module);
   inlineCalls(*module);
   lowerSingleDeviceOps(*module);
   lowerIntegerDots(*module);

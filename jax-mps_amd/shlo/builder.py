@@ -861,6 +861,21 @@ class Builder:
         self._emit(f"{name}:2 = chlo.top_k({x.name}, k = {int(k)}) : {x.type} -> ({ttype(shape, x.dtype)}, {ttype(shape, 'i32')})")
         return Val(self, f"{name}#0", shape, x.dtype, self._blk), Val(self, f"{name}#1", shape, "i32", self._blk)
 
+    def custom_call(self, target: str, operands: Sequence[Val], result_types: Sequence[Tuple[Sequence[int], str]], backend_config: str = ""):
+        """`mlir.custom_call(call_target_name=..., backend_config=...)` as jax prints it: the fused-op primitives of the
+        reference's Python layer lower to this (src/jax_plugins/mps/ops.py:81-88 and its siblings).  Returns one Val
+        per result."""
+        name = self._fresh()
+        types = [ttype(tuple(int(d) for d in shape), dt) for shape, dt in result_types]
+        quoted = backend_config.replace("\\", "\\\\").replace('"', '\\22')        # MLIR prints a quote inside a string as \22
+        lhs = name if len(types) == 1 else f"{name}:{len(types)}"
+        res = types[0] if len(types) == 1 else "(" + ", ".join(types) + ")"
+        self._emit(f"{lhs} = stablehlo.custom_call @{target}({', '.join(o.name for o in operands)}) "
+                   f"{{api_version = 2 : i32, backend_config = \"{quoted}\"}} : ({', '.join(o.type for o in operands)}) -> {res}")
+        if len(types) == 1:
+            return [Val(self, name, tuple(result_types[0][0]), result_types[0][1], self._blk)]
+        return [Val(self, f"{name}#{k}", tuple(shape), dt, self._blk) for k, (shape, dt) in enumerate(result_types)]
+
     def rng_bit_generator(self, state: Val, shape, dtype="ui32", algorithm="DEFAULT"):
         """`jax.random.bits` under the rbg / unsafe_rbg PRNG implementations: (new state, bits)."""
         name = self._fresh()

@@ -226,7 +226,12 @@ class _P:
         out = []
         while self.s[j] != '"':
             if self.s[j] == "\\":
-                out.append(self.s[j + 1])
+                pair = self.s[j + 1:j + 3]
+                if len(pair) == 2 and all(ch in "0123456789abcdefABCDEF" for ch in pair):    # MLIR prints a quote as \22
+                    out.append(chr(int(pair, 16)))
+                    j += 3
+                    continue
+                out.append({"n": "\n", "t": "\t"}.get(self.s[j + 1], self.s[j + 1]))
                 j += 2
             else:
                 out.append(self.s[j])
@@ -2012,7 +2017,126 @@ class Oracle:
             return self.op_chlo_top_k(op, ins, env)
         if isinstance(tgt, str) and tgt.startswith("mhlo.") and hasattr(self, "op_chlo_" + tgt[5:]) and len(ins) == 1:
             return getattr(self, "op_chlo_" + tgt[5:])(op, ins, env)
+        if isinstance(tgt, str) and tgt.split(".", 1)[0] in ("mps", "mi355x"):
+            fn = getattr(self, "fused_" + tgt.split(".", 1)[1], None)
+            if fn is not None:
+                import json
+                cfg = op.attrs.get("backend_config") or ""
+                cfg = json.loads(cfg) if isinstance(cfg, str) and cfg.strip() else {}
+                outs = fn([np.asarray(a) for a in ins], cfg)
+                return [np.asarray(o, dtype=np.float64) for o in outs]      # rounded once to the declared type by the caller
         raise NotImplementedError(f"oracle: custom_call {tgt}")
+
+    # ------------------------------------------------------------------
+    # fused-op custom calls of the reference's Python layer (src/jax_plugins/mps/ops.py:52-596; executor side
+    # src/pjrt_plugin/ops/control_flow.cc:1484-2020), evaluated in float64 from the operands as given
+    # ------------------------------------------------------------------
+    @staticmethod
+    def _sdpa_probabilities(q, k, v, mask, causal, scale):
+        """softmax(scale q k^T [masked]) with key / value heads repeated to the query heads (ops.py:63-76, 99-107)."""
+        q, k, v = (a.astype(np.float64) for a in (q, k, v))
+        groups = q.shape[1] // k.shape[1]
+        k, v = np.repeat(k, groups, axis=1), np.repeat(v, groups, axis=1)
+        s = np.einsum("bnth,bnsh->bnts", q, k) * scale
+        lowest = float(np.finfo(np.float32).min)
+        if causal:
+            T, S = q.shape[2], k.shape[2]
+            visible = np.arange(S)[None, :] <= np.arange(T)[:, None] + (S - T)
+            s = np.where(visible[None, None], s, lowest)
+        elif mask is not None:
+            if mask.dtype == np.bool_:
+                s = np.where(np.broadcast_to(mask, s.shape), s, lowest)
+            else:
+                s = s + mask.astype(np.float64)
+        e = np.exp(s - s.max(-1, keepdims=True))
+        return q, k, v, e / e.sum(-1, keepdims=True), groups
+
+    def fused_sdpa(self, ins, cfg, causal=False):
+        q, k, v = ins[:3]
+        _, _, v64, p, _ = self._sdpa_probabilities(q, k, v, None if causal else ins[3], causal, float(cfg.get("scale", 1.0)))
+        return [np.einsum("bnts,bnsh->bnth", p, v64)]
+
+    def fused_sdpa_causal(self, ins, cfg):
+        return self.fused_sdpa(ins, cfg, causal=True)
+
+    def fused_sdpa_bwd(self, ins, cfg, causal=False):
+        q, k, v = ins[:3]
+        g = ins[-1].astype(np.float64)
+        scale = float(cfg.get("scale", 1.0))
+        q64, k64, v64, p, groups = self._sdpa_probabilities(q, k, v, None if causal else ins[3], causal, scale)
+        dv = np.einsum("bnts,bnth->bnsh", p, g)
+        dp = np.einsum("bnth,bnsh->bnts", g, v64)
+        ds = p * (dp - (dp * p).sum(-1, keepdims=True)) * scale
+        dq = np.einsum("bnts,bnsh->bnth", ds, k64)
+        dk = np.einsum("bnts,bnth->bnsh", ds, q64)
+        if groups > 1:
+            B, N, S, H = dk.shape
+            dk = dk.reshape(B, N // groups, groups, S, H).sum(2)
+            dv = dv.reshape(B, N // groups, groups, S, H).sum(2)
+        return [dq, dk, dv]
+
+    def fused_sdpa_causal_bwd(self, ins, cfg):
+        return self.fused_sdpa_bwd(ins, cfg, causal=True)
+
+    def fused_rms_norm(self, ins, cfg):
+        x, w = (a.astype(np.float64) for a in ins)
+        return [x / np.sqrt((x * x).mean(-1, keepdims=True) + float(cfg.get("eps", 1e-6))) * w]
+
+    def fused_rms_norm_bwd(self, ins, cfg):
+        x, w, g = (a.astype(np.float64) for a in ins)
+        r = 1.0 / np.sqrt((x * x).mean(-1, keepdims=True) + float(cfg.get("eps", 1e-6)))
+        xn, gw = x * r, g * w
+        dx = r * (gw - xn * (gw * xn).mean(-1, keepdims=True))
+        return [dx, (g * xn).reshape(-1, x.shape[-1]).sum(0)]
+
+    def fused_layer_norm(self, ins, cfg):
+        x, w, b = (a.astype(np.float64) for a in ins)
+        d = x - x.mean(-1, keepdims=True)
+        return [d / np.sqrt((d * d).mean(-1, keepdims=True) + float(cfg.get("eps", 1e-5))) * w + b]
+
+    def fused_layer_norm_bwd(self, ins, cfg):
+        x, w, b, g = (a.astype(np.float64) for a in ins)
+        d = x - x.mean(-1, keepdims=True)
+        r = 1.0 / np.sqrt((d * d).mean(-1, keepdims=True) + float(cfg.get("eps", 1e-5)))
+        xn, gw = d * r, g * w
+        dx = r * (gw - gw.mean(-1, keepdims=True) - xn * (gw * xn).mean(-1, keepdims=True))
+        return [dx, (g * xn).reshape(-1, x.shape[-1]).sum(0), g.reshape(-1, x.shape[-1]).sum(0)]
+
+    @staticmethod
+    def _rope(x, offset, cfg, inverse):
+        """Rotation of the first `dims` features of (..., T, D) by (position + offset) * rope_scale * base^(-2i/dims):
+        halves (x[i], x[i + dims/2]) as in ops.py:418-438, or neighbouring pairs when "traditional"."""
+        x = x.astype(np.float64)
+        D, T = x.shape[-1], x.shape[-2]
+        dims = int(cfg.get("dims", D))
+        half = dims // 2
+        pos = (np.arange(T, dtype=np.float64) + float(np.asarray(offset).reshape(()))) * float(cfg.get("rope_scale", 1.0))
+        ang = pos[:, None] * float(cfg.get("base", 10000.0)) ** (-2.0 * np.arange(half) / dims)[None, :]
+        c, s = np.cos(ang), np.sin(ang) * (-1.0 if inverse else 1.0)
+        out = x.copy()
+        if cfg.get("traditional", False):
+            a, b = x[..., 0:dims:2], x[..., 1:dims:2]
+            out[..., 0:dims:2], out[..., 1:dims:2] = a * c - b * s, b * c + a * s
+        else:
+            a, b = x[..., :half], x[..., half:dims]
+            out[..., :half], out[..., half:dims] = a * c - b * s, b * c + a * s
+        return out
+
+    def fused_rope(self, ins, cfg):
+        return [self._rope(ins[0], ins[1], cfg, False)]
+
+    def fused_rope_bwd(self, ins, cfg):
+        return [self._rope(ins[2], ins[1], cfg, True)]
+
+    def fused_gelu(self, ins, cfg):
+        x = ins[0].astype(np.float64)
+        return [0.5 * x * (1.0 + np.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x ** 3)))]
+
+    def fused_gelu_bwd(self, ins, cfg):
+        x, g = (a.astype(np.float64) for a in ins)
+        c0, c1 = math.sqrt(2.0 / math.pi), 0.044715
+        th = np.tanh(c0 * (x + c1 * x ** 3))
+        return [g * (0.5 * (1.0 + th) + 0.5 * x * (1.0 - th * th) * c0 * (1.0 + 3.0 * c1 * x * x))]
 
 
 def _total_order_key(x):

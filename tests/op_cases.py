@@ -1023,3 +1023,55 @@ case("cumsum-axis1", lambda b, x: b.reduce_window(x, 0.0, "add", (1, 300), (1, 1
 case("cumsum-axis0-int", lambda b, x: b.reduce_window(x, 0, "add", (200, 1), (1, 1), [(199, 0), (0, 0)]), rng(3021).integers(-50, 50, size=(200, 9)).astype(np.int32), exact=True)
 case("cummax-reverse", lambda b, x: b.reduce_window(x, float("-inf"), "max", (1, 1, 130), (1, 1, 1), [(0, 0), (0, 0), (0, 129)]), f32(3022, 3, 4, 130), exact=True)
 case("cumprod-axis1", lambda b, x: b.reduce_window(x, 1.0, "mul", (1, 100), (1, 1), [(0, 0), (99, 0)]), f32(3023, 5, 100, lo=0.9, hi=1.1))
+
+
+# ------------------------------------------------------------------ fused-op custom calls of the reference's Python layer
+# (src/jax_plugins/mps/ops.py:52-596: the primitives lower to stablehlo.custom_call @mps.<op> with a JSON backend_config;
+# executor side src/pjrt_plugin/ops/control_flow.cc:1484-2020).  Forward and backward forms, float32 and bfloat16.
+def _fused(target, n_out, config=""):
+    def fn(b, *args):
+        shapes = {"sdpa_bwd": [0, 1, 2], "sdpa_causal_bwd": [0, 1, 2], "rms_norm_bwd": [0, 1], "layer_norm_bwd": [0, 1, 2]}.get(target, [0])
+        return b.custom_call("mps." + target, list(args), [(args[k].shape, args[k].dtype) for k in shapes[:n_out]], config)
+    return fn
+
+
+def _sd(seed, *shape, scale=1.0):
+    return (rng(seed).standard_normal(shape) * scale).astype(np.float32)
+
+
+_Q, _K, _V, _G = _sd(4000, 2, 4, 24, 16), _sd(4001, 2, 4, 40, 16), _sd(4002, 2, 4, 40, 16), _sd(4003, 2, 4, 24, 16)
+_KG, _VG = _sd(4004, 2, 2, 40, 16), _sd(4005, 2, 2, 40, 16)                       # two key / value heads for four query heads
+_PAD_MASK = np.broadcast_to(np.arange(40)[None, None, None, :] < np.array([40, 29])[:, None, None, None], (2, 1, 1, 40)).copy()
+_FULL_MASK = rng(4006).random((2, 4, 24, 40)) > 0.25
+_BIAS = _sd(4007, 4, 24, 40, scale=0.5)
+for dt in ("f32", "bf16"):
+    d4, d5 = [dt] * 3 + ["i1"], [dt] * 3 + ["i1", dt]
+    case(f"fused-sdpa-padding-mask-{dt}", _fused("sdpa", 1, '{"scale": 0.25}'), _Q, _K, _V, _PAD_MASK, dtypes=d4)
+    case(f"fused-sdpa-grouped-heads-{dt}", _fused("sdpa", 1, '{"scale": 0.25}'), _Q, _KG, _VG, _PAD_MASK, dtypes=d4)
+    case(f"fused-sdpa-full-mask-{dt}", _fused("sdpa", 1, '{"scale": 0.3}'), _Q, _K, _V, _FULL_MASK, dtypes=d4)
+    case(f"fused-sdpa-additive-bias-{dt}", _fused("sdpa", 1, '{"scale": 0.25}'), _Q, _K, _V, _BIAS, dtypes=[dt] * 4)
+    case(f"fused-sdpa-causal-{dt}", _fused("sdpa_causal", 1, '{"scale": 0.25}'), _Q, _K[:, :, :24], _V[:, :, :24], dtypes=[dt] * 3)
+    case(f"fused-sdpa-causal-longer-keys-{dt}", _fused("sdpa_causal", 1, '{"scale": 0.25}'), _Q, _K, _V, dtypes=[dt] * 3)
+    case(f"fused-sdpa-bwd-{dt}", _fused("sdpa_bwd", 3, '{"scale": 0.25}'), _Q, _K, _V, _PAD_MASK, _G, dtypes=d5)
+    case(f"fused-sdpa-bwd-grouped-heads-{dt}", _fused("sdpa_bwd", 3, '{"scale": 0.25}'), _Q, _KG, _VG, _PAD_MASK, _G, dtypes=d5)
+    case(f"fused-sdpa-causal-bwd-{dt}", _fused("sdpa_causal_bwd", 3, '{"scale": 0.25}'), _Q, _K[:, :, :24], _V[:, :, :24], _G, dtypes=[dt] * 4)
+    case(f"fused-rms-norm-{dt}", _fused("rms_norm", 1, '{"eps": 1e-06}'), _sd(4010, 6, 33, 96), 1.0 + _sd(4011, 96, scale=0.1), dtypes=[dt] * 2)
+    case(f"fused-rms-norm-bwd-{dt}", _fused("rms_norm_bwd", 2, '{"eps": 1e-06}'), _sd(4010, 6, 33, 96), 1.0 + _sd(4011, 96, scale=0.1), _sd(4012, 6, 33, 96),
+         dtypes=[dt] * 3)
+    case(f"fused-layer-norm-{dt}", _fused("layer_norm", 1, '{"eps": 1e-05}'), _sd(4013, 50, 200), 1.0 + _sd(4014, 200, scale=0.1), _sd(4015, 200, scale=0.1),
+         dtypes=[dt] * 3)
+    case(f"fused-layer-norm-bwd-{dt}", _fused("layer_norm_bwd", 3, '{"eps": 1e-05}'), _sd(4013, 50, 200), 1.0 + _sd(4014, 200, scale=0.1),
+         _sd(4015, 200, scale=0.1), _sd(4016, 50, 200), dtypes=[dt] * 4)
+    case(f"fused-rope-{dt}", _fused("rope", 1, '{"dims": 32, "traditional": false, "base": 10000.0, "rope_scale": 1.0}'), _sd(4017, 2, 3, 17, 32),
+         np.int32(5), dtypes=[dt, "i32"])
+    case(f"fused-rope-partial-traditional-{dt}", _fused("rope", 1, '{"dims": 16, "traditional": true, "base": 500.0, "rope_scale": 0.5}'),
+         _sd(4018, 2, 3, 17, 40), np.int32(0), dtypes=[dt, "i32"])
+    case(f"fused-rope-bwd-{dt}", _fused("rope_bwd", 1, '{"dims": 24, "traditional": false, "base": 10000.0, "rope_scale": 1.0}'), _sd(4019, 2, 9, 40),
+         np.int32(3), _sd(4020, 2, 9, 40), dtypes=[dt, "i32", dt])
+    case(f"fused-gelu-{dt}", _fused("gelu", 1), _sd(4021, 37, 130, scale=2.0), dtypes=[dt])
+    case(f"fused-gelu-bwd-{dt}", _fused("gelu_bwd", 1), _sd(4021, 37, 130, scale=2.0), _sd(4022, 37, 130), dtypes=[dt] * 2)
+# the attention of the DistilBERT-shaped benchmark as one custom call: 12 heads of 128 x 128 x 64, padding mask
+case("fused-sdpa-encoder-heads-bf16", _fused("sdpa", 1, '{"scale": 0.125}'), _sd(4030, 2, 12, 128, 64), _sd(4031, 2, 12, 128, 64), _sd(4032, 2, 12, 128, 64),
+     np.broadcast_to(np.arange(128)[None, None, None, :] < np.array([128, 77])[:, None, None, None], (2, 1, 1, 128)).copy(), dtypes=["bf16"] * 3 + ["i1"])
+case("fused-sdpa-causal-encoder-heads-bf16", _fused("sdpa_causal", 1, '{"scale": 0.125}'), _sd(4030, 2, 12, 128, 64), _sd(4031, 2, 12, 128, 64),
+     _sd(4032, 2, 12, 128, 64), dtypes=["bf16"] * 3)

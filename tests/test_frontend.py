@@ -228,3 +228,22 @@ def test_benchmark_programs_plan(name):
     p = configs.ALL[name](**configs.SMALL[name])
     r = plan(p.text)
     assert r.returncode == 0, r.stderr[-500:]
+
+
+def test_fused_op_custom_calls_are_expanded_or_refused_by_name():
+    """custom_call @mps.<op> (the reference's Python primitives, src/jax_plugins/mps/ops.py) is rewritten into plain
+    StableHLO before planning; the bf16 attention call at a shape the attention kernel takes becomes one launch of it;
+    a malformed call, an undeclared result type and an unknown target are compile errors that name the target."""
+    r = plan(op_cases.get_case("fused-sdpa-encoder-heads-bf16").text, "--dump-plan")
+    assert r.returncode == 0 and "attention tensor<2x12x128x64xbf16> masked" in r.stdout and "1 steps" in r.stdout, r.stdout[-400:]
+    # JAX's own spelling of a quote inside a string attribute is \22; the plainer \" is read as well
+    text = op_cases.get_case("fused-rms-norm-f32").text
+    assert "\\22eps\\22" in text
+    assert plan(text.replace("\\22", '\\"')).returncode == 0
+    assert plan(text.replace("@mps.rms_norm", "@mi355x.rms_norm")).returncode == 0
+    r = plan(text.replace("@mps.rms_norm", "@mps.rms_norm_bwd"))
+    assert r.returncode != 0 and "mps.rms_norm_bwd" in r.stderr and "expected 3 inputs and 2 outputs" in r.stderr
+    r = plan(text.replace("-> tensor<6x33x96xf32>", "-> tensor<6x33x95xf32>"))
+    assert r.returncode != 0 and "mps.rms_norm" in r.stderr and "declared" in r.stderr
+    r = plan(text.replace("@mps.rms_norm", "@mps.quantized_matmul"))
+    assert r.returncode != 0 and "mps.quantized_matmul" in r.stderr

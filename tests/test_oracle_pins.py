@@ -456,3 +456,117 @@ def test_pooling_against_torch():
     b.ret(b.select_and_scatter(b.arg(x.shape), b.arg((2, 5, 4, 3)), 0.0, (1, 3, 3, 1), (1, 2, 2, 1), pad))
     got = Oracle(b.text()).run(x, g.permute(0, 2, 3, 1).numpy().copy())[0]
     assert np.allclose(got, xt.grad.permute(0, 2, 3, 1).numpy(), rtol=1e-6, atol=1e-6)
+
+
+# ------------------------------------------------------------------ fused-op custom calls (oracle's `fused_*`) vs torch / closed forms
+def _fused_oracle(name):
+    c = op_cases.get_case(name)
+    ins = [round_bf16(a) if d == "bf16" else a for a, d in zip(c.inputs, c.dtypes)]
+    return ins, Oracle(c.text).run(*ins)
+
+
+def _t64(a, grad=False):
+    return torch.tensor(np.asarray(a, np.float64), requires_grad=grad)
+
+
+def _torch_sdpa(q, k, v, mask, scale):
+    g = q.shape[1] // k.shape[1]
+    return F.scaled_dot_product_attention(q, k.repeat_interleave(g, 1), v.repeat_interleave(g, 1), attn_mask=mask, scale=scale)
+
+
+@pytest.mark.parametrize("name, scale", [("fused-sdpa-padding-mask-f32", 0.25), ("fused-sdpa-grouped-heads-f32", 0.25), ("fused-sdpa-full-mask-f32", 0.3),
+                                         ("fused-sdpa-additive-bias-f32", 0.25)])
+def test_fused_sdpa_vs_torch(name, scale):
+    (q, k, v, m), out = _fused_oracle(name)
+    mask = torch.tensor(m) if m.dtype == np.bool_ else _t64(m)
+    want = _torch_sdpa(_t64(q), _t64(k), _t64(v), mask, scale).numpy()
+    np.testing.assert_allclose(out[0], want, rtol=2e-6, atol=2e-6)
+
+
+@pytest.mark.parametrize("name", ["fused-sdpa-causal-f32", "fused-sdpa-causal-longer-keys-f32"])
+def test_fused_sdpa_causal_vs_torch(name):
+    """Query t sees keys 0 .. t + (S - T): with as many keys as queries this is torch's is_causal; with more keys the
+    window is aligned to the last key (the newest query sees everything), written here as an explicit mask."""
+    (q, k, v), out = _fused_oracle(name)
+    T, S = q.shape[2], k.shape[2]
+    if T == S:
+        want = F.scaled_dot_product_attention(_t64(q), _t64(k), _t64(v), is_causal=True, scale=0.25).numpy()
+    else:
+        mask = torch.tensor(np.tril(np.ones((T, S), bool), k=S - T))
+        want = _torch_sdpa(_t64(q), _t64(k), _t64(v), mask, 0.25).numpy()
+    np.testing.assert_allclose(out[0], want, rtol=2e-6, atol=2e-6)
+
+
+@pytest.mark.parametrize("name, causal", [("fused-sdpa-bwd-f32", False), ("fused-sdpa-bwd-grouped-heads-f32", False), ("fused-sdpa-causal-bwd-f32", True)])
+def test_fused_sdpa_backward_vs_autograd(name, causal):
+    ins, out = _fused_oracle(name)
+    q, k, v = (_t64(a, True) for a in ins[:3])
+    if causal:
+        y = F.scaled_dot_product_attention(q, k, v, is_causal=True, scale=0.25)
+    else:
+        y = _torch_sdpa(q, k, v, torch.tensor(ins[3]), 0.25)
+    y.backward(_t64(ins[-1]))
+    for got, t in zip(out, (q, k, v)):
+        np.testing.assert_allclose(got, t.grad.numpy(), rtol=2e-5, atol=2e-6)
+
+
+def test_fused_norms_vs_torch():
+    (x, w), out = _fused_oracle("fused-rms-norm-f32")
+    np.testing.assert_allclose(out[0], F.rms_norm(_t64(x), (x.shape[-1],), _t64(w), eps=1e-6).numpy(), rtol=2e-6, atol=2e-6)
+    (x, w, g), out = _fused_oracle("fused-rms-norm-bwd-f32")
+    tx, tw = _t64(x, True), _t64(w, True)
+    F.rms_norm(tx, (x.shape[-1],), tw, eps=1e-6).backward(_t64(g))
+    np.testing.assert_allclose(out[0], tx.grad.numpy(), rtol=2e-5, atol=2e-6)
+    np.testing.assert_allclose(out[1], tw.grad.numpy(), rtol=2e-5, atol=2e-5)
+    (x, w, b), out = _fused_oracle("fused-layer-norm-f32")
+    np.testing.assert_allclose(out[0], F.layer_norm(_t64(x), (x.shape[-1],), _t64(w), _t64(b), eps=1e-5).numpy(), rtol=2e-6, atol=2e-6)
+    (x, w, b, g), out = _fused_oracle("fused-layer-norm-bwd-f32")
+    tx, tw, tb = _t64(x, True), _t64(w, True), _t64(b, True)
+    F.layer_norm(tx, (x.shape[-1],), tw, tb, eps=1e-5).backward(_t64(g))
+    for got, t in zip(out, (tx, tw, tb)):
+        np.testing.assert_allclose(got, t.grad.numpy(), rtol=2e-5, atol=2e-5)
+
+
+def test_fused_gelu_vs_torch():
+    (x,), out = _fused_oracle("fused-gelu-f32")
+    np.testing.assert_allclose(out[0], F.gelu(_t64(x), approximate="tanh").numpy(), rtol=2e-6, atol=2e-7)
+    (x, g), out = _fused_oracle("fused-gelu-bwd-f32")
+    tx = _t64(x, True)
+    F.gelu(tx, approximate="tanh").backward(_t64(g))
+    np.testing.assert_allclose(out[0], tx.grad.numpy(), rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("name, dims, base, scale, traditional", [("fused-rope-f32", 32, 10000.0, 1.0, False),
+                                                                  ("fused-rope-partial-traditional-f32", 16, 500.0, 0.5, True)])
+def test_fused_rope_is_a_complex_rotation(name, dims, base, scale, traditional):
+    """Each rotated pair (a, b) is the complex number a + ib multiplied by exp(i * position * frequency): written with
+    numpy's complex arithmetic, which shares nothing with the oracle's cos / sin form."""
+    (x, offset), out = _fused_oracle(name)
+    x = x.astype(np.float64)
+    T, half = x.shape[-2], dims // 2
+    theta = ((np.arange(T) + int(offset)) * scale)[:, None] * base ** (-2.0 * np.arange(half) / dims)[None, :]
+    want = x.copy()
+    if traditional:
+        z = (x[..., 0:dims:2] + 1j * x[..., 1:dims:2]) * np.exp(1j * theta)
+        want[..., 0:dims:2], want[..., 1:dims:2] = z.real, z.imag
+    else:
+        z = (x[..., :half] + 1j * x[..., half:dims]) * np.exp(1j * theta)
+        want[..., :half], want[..., half:dims] = z.real, z.imag
+    np.testing.assert_allclose(out[0], want, rtol=2e-6, atol=2e-6)
+    # position 0 with no offset leaves the row as it is; features past `dims` pass through
+    if int(offset) == 0:
+        np.testing.assert_array_equal(out[0][..., 0, :], x[..., 0, :].astype(np.float32))
+    np.testing.assert_array_equal(out[0][..., dims:], x[..., dims:].astype(np.float32))
+
+
+def test_fused_rope_backward_inverts_the_rotation():
+    """rope is orthogonal per pair, so its vjp is the inverse rotation: rope_bwd(x, offset, rope(g)) == g."""
+    (x, offset, g), out = _fused_oracle("fused-rope-bwd-f32")
+    o = Oracle(op_cases.get_case("fused-rope-bwd-f32").text)
+    cfg = {"dims": 24, "traditional": False, "base": 10000.0, "rope_scale": 1.0}
+    forward = o.fused_rope([g, offset], cfg)[0]
+    back = o.fused_rope_bwd([x, offset, forward], cfg)[0]
+    np.testing.assert_allclose(back, g, rtol=1e-12, atol=1e-12)
+    # and it is the transpose of the forward map: <rope(u), g> == <u, rope_bwd(g)>
+    u = np.random.default_rng(0).standard_normal(g.shape)
+    assert abs((o.fused_rope([u, offset], cfg)[0] * g).sum() - (u * out[0].astype(np.float64)).sum()) < 1e-4

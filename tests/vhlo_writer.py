@@ -238,7 +238,8 @@ class Writer:
         elif short == "custom_call":
             out["call_target_name"] = self.a_str(a["call_target_name"])
             out["has_side_effect"] = self.a_bool(False)
-            out["backend_config"] = self.a_str("")
+            config = a.get("backend_config", "")
+            out["backend_config"] = self.a_str(config if isinstance(config, str) else "")
         elif short == "composite":
             out["name"] = self.a_str(a["name"])
             out["decomposition"] = self.a_str(str(a["decomposition"]).lstrip("@"))
