@@ -21,7 +21,12 @@ struct BufRef {
   enum Kind : uint8_t { None, Param, Output, Temp, Const } kind = None;
   int index = 0;       // parameter / output number
   int64_t offset = 0;  // byte offset inside the arena (Temp) or the constant pool (Const)
-  bool operator==(const BufRef& o) const { return kind == o.kind && index == o.index && offset == o.offset; }
+  // Inside a counted loop whose counter the host follows (Step::hostCounter): the address moves with the iteration,
+  // by CompiledProgram::ivTables[ivTable][k] bytes at iteration k of the loop at nesting depth ivDepth.  That is how a
+  // kernel reads the counter (a table of its values in the constant pool) and how a product reads xs[i] in place.
+  int ivTable = -1;
+  int ivDepth = 0;
+  bool operator==(const BufRef& o) const { return kind == o.kind && index == o.index && offset == o.offset && ivTable == o.ivTable; }
   bool operator!=(const BufRef& o) const { return !(*this == o); }
 };
 
@@ -120,6 +125,10 @@ struct Step {
   std::vector<std::unique_ptr<Plan>> bodies;  // While: [body]; Case: branches
   BufRef predBuf;                             // i1 (While) or i32 index (Case)
   int64_t tripCount = -1;                     // >= 0 when the loop is counted and the count is static
+  // Counted loop whose counter carry is never computed on the device: iteration k reads entry k of a table of the
+  // counter's values, and operands sliced at the counter are addressed by the host (BufRef::ivTable).
+  bool hostCounter = false;
+  int ivDepth = 0;
   DType predType = DType::Pred;
   // Dynamic While: the loop's alive flag (one int on the device).  Iterations run in chunks without host
   // round trips: each evaluates the condition, folds it into the flag (FlagAnd), runs the body into temporaries and
@@ -147,6 +156,7 @@ struct CompiledProgram {
   std::vector<int> paramDonation;   // per parameter: -1 not donated by the program, otherwise donated (>= 0: to that result)
   std::vector<OutputInfo> outputs;
   std::vector<uint8_t> constPool;   // host image of the constant pool
+  std::vector<std::vector<int64_t>> ivTables;   // per-iteration byte offsets of references that follow a host-side loop counter
   int64_t arenaBytes = 0;
   int numOps = 0, numSteps = 0;
   std::string dump;                 // human-readable plan (MI355X_DUMP_PLAN)

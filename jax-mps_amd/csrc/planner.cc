@@ -38,6 +38,8 @@ struct Storage {
   int first = -1, last = -1;
   std::vector<int> uses;
   int values = 0;         // SSA values bound to this storage
+  int ivTable = -1;       // references move with the iteration of a host-counted loop (BufRef::ivTable)
+  int ivDepth = 0;
 };
 
 bool isExpensive(const std::string& n) {
@@ -149,7 +151,19 @@ class Planner {
     BufRef r;
     r.kind = BufRef::Temp;   // patched after arena assignment
     r.index = sid;
+    r.ivTable = s.ivTable;
+    r.ivDepth = s.ivDepth;
     return r;
+  }
+
+  // a reference that follows a view taken at a host-counted loop's counter: byte offsets per iteration
+  void followCounter(BufRef& r, const std::vector<int64_t>& iterElems, int64_t elemBytes) {
+    if (iterElems.empty()) return;
+    std::vector<int64_t> bytes;
+    for (auto e : iterElems) bytes.push_back(e * elemBytes);
+    P.ivTables.push_back(std::move(bytes));
+    r.ivTable = (int)P.ivTables.size() - 1;
+    r.ivDepth = 0;
   }
 
   // ---------------------------------------------------------------- analysis
@@ -981,7 +995,98 @@ class Planner {
     Value* root = nullptr;          // value that owns the memory
     int64_t offset = 0;             // elements from the root's first element
     std::vector<int64_t> strides;   // per dim of the viewed value
+    std::vector<int64_t> iterOffsets;   // inside a host-counted loop: further elements at iteration k (a slice taken at the counter)
   };
+
+  // ---------------------------------------------------------------- loop counters the host follows
+  // The counter carry of a counted loop (init constant, constant step, static trip count) takes known values, so
+  // nothing needs to compute it on the device: kernels read entry k of a table of its values at iteration k, and a
+  // dynamic_slice whose start indices are scalar integer arithmetic on the counter is a view whose offset the host
+  // computes per iteration.  That removes the counter's own kernel from every iteration and lets products read
+  // xs[i] in place (the reference re-evaluates such slices on the device every iteration: ops/control_flow.cc:702-989).
+  struct IvInfo { int64_t init = 0, step = 0, trip = 0; };
+  static std::unordered_map<const Value*, IvInfo>& ivArgs() {
+    static thread_local std::unordered_map<const Value*, IvInfo> m;
+    return m;
+  }
+
+  // value of the scalar integer `v` at iteration k of the host-counted loop it depends on (if any); `trip` receives that
+  // loop's trip count (0 when `v` is a plain constant)
+  static bool evalIndex(Value* v, int64_t k, int64_t& out, int64_t& trip, int depth = 0) {
+    if (depth > 16 || v->type.numel() != 1) return false;
+    auto it = ivArgs().find(v);
+    if (it != ivArgs().end()) {
+      if (trip != 0 && trip != it->second.trip) return false;
+      trip = it->second.trip;
+      out = it->second.init + k * it->second.step;
+      return true;
+    }
+    if (constInt(v, out)) return true;
+    Op* d = v->def;
+    if (!d || d->results.size() != 1 || !(isInt(v->type.dt) || v->type.dt == DType::Pred)) return false;
+    std::vector<int64_t> in;
+    for (auto* o : d->operands) {
+      int64_t x;
+      if (!evalIndex(o, k, x, trip, depth + 1)) return false;
+      in.push_back(x);
+    }
+    const std::string& n = d->name;
+    auto wrap = [&](int64_t x) {   // two's complement of the value's own width
+      const size_t sz = dtypeSize(v->type.dt);
+      if (v->type.dt == DType::Pred) return (int64_t)(x != 0);
+      if (sz >= 8) return x;
+      const int bits = (int)(8 * sz);
+      uint64_t u = (uint64_t)x & ((1ull << bits) - 1);
+      if (isSignedInt(v->type.dt) && (u >> (bits - 1))) return (int64_t)(u | ~((1ull << bits) - 1));
+      return (int64_t)u;
+    };
+    if (n == "reshape" || n == "convert" || n == "broadcast_in_dim") { out = wrap(in[0]); return true; }
+    if (in.size() == 1 && n == "negate") { out = wrap(-in[0]); return true; }
+    if (in.size() == 2) {
+      if (n == "add") { out = wrap(in[0] + in[1]); return true; }
+      if (n == "subtract") { out = wrap(in[0] - in[1]); return true; }
+      if (n == "multiply") { out = wrap(in[0] * in[1]); return true; }
+      if (n == "minimum") { out = std::min(in[0], in[1]); return true; }
+      if (n == "maximum") { out = std::max(in[0], in[1]); return true; }
+      if (n == "compare" && isSignedInt(d->operands[0]->type.dt)) {
+        const std::string& dir = d->str("direction");
+        out = dir == "LT" ? in[0] < in[1] : dir == "LE" ? in[0] <= in[1] : dir == "GT" ? in[0] > in[1] : dir == "GE" ? in[0] >= in[1] : dir == "EQ" ? in[0] == in[1] : in[0] != in[1];
+        return true;
+      }
+    }
+    if (in.size() == 3 && n == "select") { out = in[0] ? in[1] : in[2]; return true; }
+    if (in.size() == 3 && n == "clamp") { out = std::min(std::max(in[1], in[0]), in[2]); return true; }
+    return false;
+  }
+
+  // a dynamic_slice all of whose start indices the host can evaluate; `perIter` receives the element offset at each
+  // iteration relative to `strides` (empty when every index is a constant), `base` the constant part
+  static bool hostSlice(const Op* d, const std::vector<int64_t>& strides, int64_t& base, std::vector<int64_t>& perIter) {
+    if (!d || d->name != "dynamic_slice") return false;
+    const TensorType& xt = d->operands[0]->type;
+    auto& sizes = d->ints("sizes");
+    if ((int)d->operands.size() != 1 + xt.rank() || (int)sizes.size() != xt.rank()) return false;
+    int64_t trip = 0;
+    for (int dim = 0; dim < xt.rank(); ++dim) {
+      int64_t x;
+      if (!evalIndex(d->operands[(size_t)dim + 1], 0, x, trip)) return false;
+    }
+    const int64_t iters = std::max<int64_t>(trip, 1);
+    std::vector<int64_t> offs((size_t)iters, 0);
+    for (int64_t k = 0; k < iters; ++k) {
+      for (int dim = 0; dim < xt.rank(); ++dim) {
+        int64_t x = 0, t2 = 0;
+        if (!evalIndex(d->operands[(size_t)dim + 1], k, x, t2)) return false;
+        x = std::min(std::max<int64_t>(x, 0), xt.dims[(size_t)dim] - sizes[(size_t)dim]);   // start indices are clamped into range
+        offs[(size_t)k] += x * strides[(size_t)dim];
+      }
+    }
+    base = 0;
+    perIter.clear();
+    if (trip == 0) base = offs[0];
+    else perIter = offs;
+    return true;
+  }
 
   // strides of `newDims` over memory laid out as (oldDims, oldStrides), if no copy is needed
   static bool reshapeStrides(const std::vector<int64_t>& oldDims, const std::vector<int64_t>& oldStrides, const std::vector<int64_t>& newDims,
@@ -1016,7 +1121,13 @@ class Planner {
     return oi == od.size();
   }
 
-  static bool isViewOp(const Op* d) { return d && d->results.size() == 1 && (d->name == "reshape" || d->name == "slice" || d->name == "transpose"); }
+  static bool isViewOp(const Op* d) {
+    if (!d || d->results.size() != 1) return false;
+    if (d->name == "reshape" || d->name == "slice" || d->name == "transpose") return true;
+    int64_t base;
+    std::vector<int64_t> perIter;
+    return d->name == "dynamic_slice" && hostSlice(d, stridesOf(d->operands[0]->type), base, perIter);
+  }
 
   // `ownsMemory(v)`: the caller's notion of "v is (or will be) in memory".
   template <typename F>
@@ -1034,6 +1145,20 @@ class Planner {
     const TensorType& xt = d->operands[0]->type;
     out.root = in.root;
     out.offset = in.offset;
+    out.iterOffsets = in.iterOffsets;
+    if (d->name == "dynamic_slice") {
+      int64_t base = 0;
+      std::vector<int64_t> perIter;
+      if (!hostSlice(d, in.strides, base, perIter)) return false;
+      out.offset += base;
+      out.strides = in.strides;
+      if (!perIter.empty()) {
+        if (out.iterOffsets.empty()) out.iterOffsets = perIter;
+        else if (out.iterOffsets.size() == perIter.size()) for (size_t k = 0; k < perIter.size(); ++k) out.iterOffsets[k] += perIter[k];
+        else return false;
+      }
+      return true;
+    }
     if (d->name == "slice") {
       auto& start = d->ints("start");
       auto& stride = d->ints("strides");
@@ -1340,7 +1465,7 @@ class Planner {
     Op* users[3] = {m.qk, m.qk, m.pv};
     for (int i = 0; i < 3; ++i) {
       Value* x = ops3[i];
-      if (!hasStorage(x) && !(dotTakesView(x, users[i]) && resolveView(x, stored, *views[i]))) materializeNow(x, plan);
+      if (!hasStorage(x) && !(dotTakesView(x, users[i]) && resolveView(x, stored, *views[i]) && views[i]->iterOffsets.empty())) materializeNow(x, plan);
       if (hasStorage(x)) { views[i]->root = x; views[i]->offset = 0; views[i]->strides = stridesOf(x->type); }
     }
     AttentionDesc a;
@@ -1431,7 +1556,7 @@ class Planner {
     for (Value* v : {a, b}) {
       View& vw = v == a ? va : vb;
       if (!hasStorage(v) && !(dotTakesView(v, op) && resolveView(v, stored, vw))) materializeNow(v, plan);
-      if (hasStorage(v)) { vw.root = v; vw.offset = 0; vw.strides = stridesOf(v->type); }
+      if (hasStorage(v)) { vw.root = v; vw.offset = 0; vw.strides = stridesOf(v->type); vw.iterOffsets.clear(); }
     }
     if (b == a) vb = va;
     DotPlan dp;
@@ -1596,6 +1721,8 @@ class Planner {
     s.args = {ref(storageOf(va.root), t), ref(storageOf(vb.root), t), ref(sid, t)};
     s.args[0].offset = va.offset * (int64_t)dtypeSize(a->type.dt);
     s.args[1].offset = vb.offset * (int64_t)dtypeSize(b->type.dt);
+    followCounter(s.args[0], va.iterOffsets, (int64_t)dtypeSize(a->type.dt));
+    followCounter(s.args[1], vb.iterOffsets, (int64_t)dtypeSize(b->type.dt));
     if (biasV) {
       s.bias = ref(storageOf(biasV), t);
       bind(biasAdd->result(), sid);   // the step writes the sum; nothing reads the bare product
@@ -1608,6 +1735,8 @@ class Planner {
       s.args.push_back(ref(storageOf(dp2->vb.root), t));
       s.args[3].offset = dp2->va.offset * 4;
       s.args[4].offset = dp2->vb.offset * 4;
+      followCounter(s.args[3], dp2->va.iterOffsets, 4);
+      followCounter(s.args[4], dp2->vb.iterOffsets, 4);
       plan.steps.push_back(std::move(s));
       return;
     }
@@ -1813,7 +1942,9 @@ class Planner {
   }
 
   // counted loop: cond is `carry_i <cmp> const`, body returns carry_i + const, init is a constant
-  int64_t detectTripCount(Op* op) {
+  // `counter` (optional) receives the carry index, start and step of the counter the trip count was read from
+  struct CounterInfo { int carry = -1; int64_t init = 0, step = 0; };
+  int64_t detectTripCount(Op* op, CounterInfo* counter = nullptr) {
     Region& cond = *op->regions[0];
     Region& body = *op->regions[1];
     Op* ret = cond.terminator();
@@ -1854,6 +1985,7 @@ class Planner {
     else if (dir == "GE" && step < 0) n = init >= limit ? (init - limit) / (-step) + 1 : 0;
     else if (dir == "NE" && (limit - init) % step == 0 && (limit - init) / step >= 0) n = (limit - init) / step;
     else return -1;
+    if (counter) { counter->carry = ci; counter->init = init; counter->step = step; }
     return n;
   }
 
@@ -1993,7 +2125,14 @@ class Planner {
   void emitWhile(Op* op, Plan& plan) {
     size_t n = op->operands.size();
     for (auto* v : op->operands) if (!hasStorage(v)) materializeNow(v, plan);
-    int64_t trip = detectTripCount(op);
+    CounterInfo counter;
+    int64_t trip = detectTripCount(op, &counter);
+    // A top-level counted loop of modest length keeps its counter on the host (see ivArgs): only then does one graph
+    // hold every iteration, which is what lets each iteration's launches carry their own addresses.
+    static const bool hostCounters = !getenv("MI355X_HOST_COUNTERS") || atoi(getenv("MI355X_HOST_COUNTERS")) != 0;
+    const bool hostCounter = hostCounters && trip >= 2 && trip <= kHostCounterMaxTrip && loopDepth_ == 0 && specFloors_.empty() && counter.carry >= 0 &&
+                             isInt(op->operands[(size_t)counter.carry]->type.dt) && op->operands[(size_t)counter.carry]->type.numel() == 1;
+    const size_t ivCarry = hostCounter ? (size_t)counter.carry : (size_t)-1;
     std::vector<int> slots(n);
     for (size_t i = 0; i < n; ++i) {
       Value* v = op->operands[i];
@@ -2034,8 +2173,39 @@ class Planner {
     Region& cond = *op->regions[0];
     Region& body = *op->regions[1];
     for (size_t i = 0; i < n; ++i) { bind(cond.args[i].get(), slots[i]); bind(body.args[i].get(), slots[i]); }
+    int counterEnd = -1;   // storage holding the counter's value after the last iteration
+    if (hostCounter) {
+      // table of the counter's values, one per iteration plus the final one
+      const DType dt = op->operands[ivCarry]->type.dt;
+      const size_t esz = dtypeSize(dt);
+      const int64_t off = ((int64_t)P.constPool.size() + kAlign - 1) / kAlign * kAlign;
+      P.constPool.resize((size_t)off + (size_t)(trip + 1) * esz);
+      std::vector<int64_t> steps;
+      for (int64_t k = 0; k <= trip; ++k) {
+        const int64_t x = counter.init + k * counter.step;
+        memcpy(P.constPool.data() + off + (size_t)k * esz, &x, esz);   // little endian: the low bytes are the value
+        if (k < trip) steps.push_back(k * (int64_t)esz);
+      }
+      P.ivTables.push_back(std::move(steps));
+      const int table = newStorage(esz, BufRef::Const);
+      st_[table].offset = off;
+      st_[table].ivTable = (int)P.ivTables.size() - 1;
+      st_[table].ivDepth = 0;
+      storage_[cond.args[ivCarry].get()] = table;
+      storage_[body.args[ivCarry].get()] = table;
+      counterEnd = newStorage(esz, BufRef::Const);
+      st_[counterEnd].offset = off + trip * (int64_t)esz;
+      IvInfo info;
+      info.init = counter.init; info.step = counter.step; info.trip = trip;
+      ivArgs()[body.args[ivCarry].get()] = info;
+    }
     analyze(cond);
     analyze(body);
+    if (hostCounter) {
+      // the counter's next value is never stored: the loop does not read it back, and other readers recompute it from the table
+      Value* next = body.terminator()->operands[ivCarry];
+      if (next->def && next->def->parent == &body) needMat_[next] = false;
+    }
     w.cond = std::make_unique<Plan>();
     emitRegion(cond, *w.cond);
     Value* pred = cond.terminator()->operands.at(0);
@@ -2059,6 +2229,7 @@ class Planner {
     if (ret->operands.size() != n) throw CompileError("while: body returns the wrong number of values");
     std::vector<int> src(n);
     for (size_t i = 0; i < n; ++i) {
+      if (i == ivCarry) { src[i] = slots[i]; continue; }   // never written inside the loop
       Value* v = ret->operands[i];
       if (!hasStorage(v)) materializeNow(v, *bodyPlan);
       src[i] = storageOf(v);
@@ -2108,7 +2279,8 @@ class Planner {
     }
     loops_.push_back({tStart, tEnd});
     w.bodies.push_back(std::move(bodyPlan));
-    for (size_t i = 0; i < n; ++i) bind(op->results[i].get(), slots[i]);
+    w.hostCounter = hostCounter;
+    for (size_t i = 0; i < n; ++i) bind(op->results[i].get(), i == ivCarry ? counterEnd : slots[i]);
     plan.steps.push_back(std::move(w));
   }
 
@@ -2169,6 +2341,7 @@ class Planner {
   // Consecutive kernel steps that touch disjoint buffers (or only read the shared ones) run as
   // the segments of one launch: small kernels cost a launch each whatever their size, and the
   // optimiser updates of a training step or the bookkeeping of a loop body come in such runs.
+  static constexpr int64_t kHostCounterMaxTrip = 512;
   static constexpr unsigned kBatchMaxBlocks = 4096;   // bigger kernels fill the chip on their own
   static constexpr size_t kBatchMaxArgs = 192;
   static constexpr size_t kBatchMaxSegments = 24;
@@ -2374,6 +2547,8 @@ class Planner {
     o.kind = s.kind;
     if (s.kind == BufRef::Param || s.kind == BufRef::Output) { o.index = s.index; o.offset = r.offset; }
     else { o.index = 0; o.offset = s.offset + r.offset; }
+    o.ivTable = r.ivTable;
+    o.ivDepth = r.ivDepth;
     return o;
   }
 

@@ -295,11 +295,13 @@ void Executable::loadKernels() {
 }
 
 void* Executable::resolve(const BufRef& r, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) const {
+  // inside a loop whose counter the host follows, some addresses move with the iteration
+  const int64_t moved = r.ivTable < 0 ? 0 : prog_->ivTables[(size_t)r.ivTable][(size_t)std::min<int64_t>(hostIteration_, (int64_t)prog_->ivTables[(size_t)r.ivTable].size() - 1)];
   switch (r.kind) {
-    case BufRef::Param: return (char*)in[r.index]->ptr + r.offset;
-    case BufRef::Output: return (char*)out[r.index] + r.offset;
-    case BufRef::Temp: return (char*)arena_ + r.offset;
-    case BufRef::Const: return (char*)consts_ + r.offset;
+    case BufRef::Param: return (char*)in[r.index]->ptr + r.offset + moved;
+    case BufRef::Output: return (char*)out[r.index] + r.offset + moved;
+    case BufRef::Temp: return (char*)arena_ + r.offset + moved;
+    case BufRef::Const: return (char*)consts_ + r.offset + moved;
     default: return nullptr;
   }
 }
@@ -658,13 +660,20 @@ void Executable::runDeviceLoop(const Step& s, const std::vector<DeviceBuffer*>& 
 void Executable::replayIterations(const Step& s, bool withCond, int64_t trip, const std::vector<DeviceBuffer*>& in, const std::vector<void*>& out) {
   Device& dev = Device::get();
   const Plan& body = *s.bodies[0];
+  // A loop whose counter the host follows gives every iteration its own addresses (hostIteration_ selects them), so its
+  // graph holds all iterations after the first and is launched once.
+  const bool counted = s.hostCounter;
+  int64_t iteration = 0;
   auto runOne = [&]() {
+    if (counted) hostIteration_ = iteration++;
     if (withCond) runPlan(*s.cond, in, out);
     runPlan(body, in, out);
   };
+  struct ResetIteration { int64_t& v; ~ResetIteration() { v = 0; } } resetIteration{hostIteration_};
   const size_t unitSteps = body.steps.size() + (withCond ? s.cond->steps.size() : 0);
+  const int64_t nodeLimit = counted ? 8192 : 1024;
   const bool graphOk = useGraphs_ && !capturing_ && timingKinds_.empty() && trip >= (withCond ? 16 : 4) && unitSteps > 0 && capturable(body) &&
-                       (!withCond || capturable(*s.cond));
+                       (!withCond || capturable(*s.cond)) && (!counted || (trip - 1) * (int64_t)unitSteps <= nodeLimit);
   if (!graphOk) {
     for (int64_t i = 0; i < trip; ++i) runOne();
     return;
@@ -703,11 +712,12 @@ void Executable::replayIterations(const Step& s, bool withCond, int64_t trip, co
       hit->exec = nullptr;
     }
     // a flag-driven loop is replayed in sub-chunks of 16 iterations, so that one graph serves whatever length the next chunk has
-    const int64_t per = std::max<int64_t>(1, std::min<int64_t>(withCond ? 16 : trip - 1, 1024 / (int64_t)unitSteps));
+    const int64_t per = counted ? trip - 1 : std::max<int64_t>(1, std::min<int64_t>(withCond ? 16 : trip - 1, 1024 / (int64_t)unitSteps));
     mi355_stream_t st = dev.stream();
     check(mi355_capture_begin(st), "graph capture");
     capturing_ = true;
     try {
+      iteration = 1;
       for (int64_t i = 0; i < per; ++i) runOne();
     } catch (...) {
       capturing_ = false;

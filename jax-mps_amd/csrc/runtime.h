@@ -141,6 +141,7 @@ class Executable {
   uint64_t graphClock_ = 0;
   std::map<const Plan*, bool> capturable_;
   bool useGraphs_ = true;
+  int64_t hostIteration_ = 0;         // iteration being enqueued of the loop whose counter the host follows (Step::hostCounter)
   bool capturing_ = false;
   bool forkingAllowed_ = true;        // cleared while a plan is captured with everything on one stream
   bool capturable(const Plan& p);
