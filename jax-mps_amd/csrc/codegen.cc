@@ -1478,13 +1478,11 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   std::vector<std::string> inits;
   for (auto* r : reduces) inits.push_back(em.gen(r->operands[1], em.multiIndex({}, {})));
 
-  std::ostringstream s;
-  s << kPrelude;
+  std::ostringstream s;   // body; the header follows once an epilogue has named its inputs
   std::vector<std::string> outs;
   for (size_t j = 0; j < nr; ++j)
     outs.push_back((partial ? ops[j].accT : storageT(ops[j].dt)) + "* __restrict__ out" + std::to_string(j));
   for (size_t q = 0; q < sideStores.size(); ++q) outs.push_back(storageT(sideStores[q]->type.dt) + "* __restrict__ side" + std::to_string(q));
-  s << kernelHeader(em.leaves_, outs) << " {\n";
   s << "  const int tx = threadIdx.x % " << TX << ", ty = threadIdx.x / " << TX << ";\n";
   s << "  const " << IT << " kb = ((" << IT << ")blockIdx.x * " << TX << " + tx) * " << V << ";\n";
   s << "  const bool active = kb < " << Kn << ";\n";
@@ -1518,14 +1516,42 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   } else {
     s << "  if (!active) return;\n";
   }
-  for (size_t j = 0; j < nr; ++j) {
-    s << "  #pragma unroll\n  for (int v = 0; v < " << V << "; ++v) ";
-    if (partial) s << "out" << j << "[(kb + v) * " << P << " + (" << IT << ")blockIdx.y] = acc" << j << "[v];\n";
-    else s << "out" << j << "[kb + v] = " << storeExpr(ops[j].dt, roundTo(ops[j].dt, ops[j].combine(inits[j], "acc" + std::to_string(j) + "[v]"))) << ";\n";
+  const bool epilogueHere = !partial && !epilogue.empty();
+  if (epilogueHere) {
+    // a single pass holds the finished results: per-output values that only need those are computed by the lane that holds them
+    s << "  #pragma unroll\n  for (int v = 0; v < " << V << "; ++v) {\n    const " << IT << " kk = kb + v;\n";
+    for (size_t j = 0; j < nr; ++j) {
+      s << "    const " << ops[j].accT << " res" << j << " = " << roundTo(ops[j].dt, ops[j].combine(inits[j], "acc" + std::to_string(j) + "[v]")) << ";\n";
+      s << "    out" << j << "[kk] = " << storeExpr(ops[j].dt, "res" + std::to_string(j)) << ";\n";
+      em.rowScalars_[reduces[j]->result()] = "res" + std::to_string(j);
+    }
+    IdxDim klin2;
+    klin2.isConst = false; klin2.base = "kk"; klin2.coef = 0; klin2.mult = 1;
+    const std::string keepPre = em.pre_;
+    em.pre_.clear();
+    auto kd2 = em.delinearize(klin2, keptShape);
+    em.rowKept_ = kd2;
+    Index kidx = em.multiIndex(kd2, keptShape);
+    std::vector<std::string> ev;
+    for (auto* v : epilogue) ev.push_back(em.gen(v, kidx));
+    s << em.pre_;
+    em.pre_ = keepPre;
+    for (size_t q = 0; q < epilogue.size(); ++q) {
+      s << "    outE" << q << "[kk] = " << storeExpr(epilogue[q]->type.dt, ev[q]) << ";\n";
+      outs.push_back(storageT(epilogue[q]->type.dt) + "* __restrict__ outE" + std::to_string(q));
+    }
+    s << "  }\n";
+    fc.epilogueFused = true;
+  } else {
+    for (size_t j = 0; j < nr; ++j) {
+      s << "  #pragma unroll\n  for (int v = 0; v < " << V << "; ++v) ";
+      if (partial) s << "out" << j << "[(kb + v) * " << P << " + (" << IT << ")blockIdx.y] = acc" << j << "[v];\n";
+      else s << "out" << j << "[kb + v] = " << storeExpr(ops[j].dt, roundTo(ops[j].dt, ops[j].combine(inits[j], "acc" + std::to_string(j) + "[v]"))) << ";\n";
+    }
   }
   s << "}\n";
   Launch l;
-  l.source = s.str();
+  l.source = std::string(kPrelude) + kernelHeader(em.leaves_, outs) + " {\n" + s.str();
   l.grid[0] = (unsigned)gridX;
   l.grid[1] = (unsigned)P;
   l.block[0] = 256;
@@ -1546,6 +1572,7 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     l.args.push_back(a);
   }
   for (auto* sv : sideStores) { KArg a; a.kind = KArg::Out; a.value = sv; l.args.push_back(a); }
+  if (epilogueHere) for (auto* v : epilogue) { KArg a; a.kind = KArg::Out; a.value = v; l.args.push_back(a); }
   fc.sideStored = !sideStores.empty();
   fc.leaves = em.leaves_;
   fc.launches.push_back(std::move(l));

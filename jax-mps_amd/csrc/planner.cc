@@ -28,6 +28,9 @@ namespace mi355 {
 namespace {
 
 constexpr int64_t kSmallNumel = 8192;   // values at most this big are never materialised just to avoid recomputation
+// Inside a loop body a launch costs more than any amount of arithmetic on a tensor this small, and a kernel that
+// recomputes what a neighbour also computes does not have to wait for it: the two can share a launch.
+constexpr int64_t kLoopSmallNumel = 131072;
 constexpr int64_t kAlign = 256;
 
 struct Storage {
@@ -40,6 +43,8 @@ struct Storage {
   int values = 0;         // SSA values bound to this storage
   int ivTable = -1;       // references move with the iteration of a host-counted loop (BufRef::ivTable)
   int ivDepth = 0;
+  int aliasOf = -1;       // a window of another storage (the halves of a double-buffered loop carry): no memory of its own
+  int64_t aliasOffset = 0;
 };
 
 bool isExpensive(const std::string& n) {
@@ -94,6 +99,7 @@ class Planner {
     }
     static const bool batching = !getenv("MI355X_BATCH_KERNELS") || atoi(getenv("MI355X_BATCH_KERNELS")) != 0;
     groupSmallGemms(P.plan);
+    if (batching) sinkKernelsInLoops(P.plan, false);
     if (batching) batchKernels(P.plan);
     forkDistantConvolutions(P.plan);
     assignArena();
@@ -143,7 +149,26 @@ class Planner {
     if (it == storage_.end()) throw CompileError("internal: value " + v->name + " has no storage");
     return it->second;
   }
+  // a storage that names `bytes` of `parent` from `offset` on, optionally moving with a host-counted loop's iteration
+  int newAlias(int parent, int64_t offset, int64_t bytes, int ivTable) {
+    int sid = newStorage((size_t)bytes);
+    st_[sid].aliasOf = parent;
+    st_[sid].aliasOffset = offset;
+    st_[sid].ivTable = ivTable;
+    boundToOutput_.insert(sid);     // never turned into an output buffer or taken over as another loop's slot
+    return sid;
+  }
   BufRef ref(int sid, int t) {
+    if (st_[sid].aliasOf >= 0) {    // the memory is the parent's: its lifetime is what the use extends
+      BufRef p = ref(st_[sid].aliasOf, t);
+      (void)p;
+      BufRef r;
+      r.kind = BufRef::Temp;
+      r.index = sid;
+      r.ivTable = st_[sid].ivTable;
+      r.ivDepth = st_[sid].ivDepth;
+      return r;
+    }
     Storage& s = st_[sid];
     s.uses.push_back(t);
     if (s.first < 0 || t < s.first) s.first = t;
@@ -302,7 +327,7 @@ class Planner {
         auto& d = *op->attrs.at("value").dense;
         if (!d.splat && d.type.numel() > 1) mat = true;
       }
-      if (!mat && v->type.numel() > kSmallNumel && g.size() >= 2) {
+      if (!mat && v->type.numel() > (loopDepth_ > 0 ? kLoopSmallNumel : kSmallNumel) && g.size() >= 2) {
         int big = 0;
         for (auto* l : leaves[v]) if (l->type.numel() * 4 >= v->type.numel()) ++big;
         bool expensive = isExpensive(op->name);
@@ -318,6 +343,13 @@ class Planner {
       static const bool inlineSmall = !getenv("MI355X_INLINE_SMALL") || atoi(getenv("MI355X_INLINE_SMALL")) != 0;
       if (inlineSmall && mat && forced && !nestedUse && loopDepth_ == 0 && !op->has("force_materialize") && v->type.numel() <= kSmallNumel && v->users.size() >= 2) {
         int budget = 8;
+        if (cheapFromMemory(v, budget)) inlineAnyway_.insert(v);
+      }
+      // in a loop body the same holds for somewhat larger values (cheap chains only: a column reduction runs few
+      // workgroups, and each lane would walk an expensive chain once per row)
+      if (inlineSmall && mat && forced && !nestedUse && loopDepth_ > 0 && specFloors_.empty() && !op->has("force_materialize") &&
+          v->type.numel() <= kLoopSmallNumel && v->users.size() >= 2 && op->name != "constant" && op->name != "dynamic_update_slice") {
+        int budget = 16;
         if (cheapFromMemory(v, budget)) inlineAnyway_.insert(v);
       }
       if (mat) { g.clear(); g.push_back(op); }
@@ -869,7 +901,7 @@ class Planner {
       };
       size_t pos = 0;
       while (pos < r.ops.size() && r.ops[pos].get() != op) ++pos;
-      for (size_t q = pos + 1; q < r.ops.size() && q <= pos + 64 && epilogue.size() < 6; ++q) {
+      for (size_t q = pos + 1; q < r.ops.size() && q <= pos + 512 && epilogue.size() < 6; ++q) {
         Op* y = r.ops[q].get();
         if (emitted_.count(y) || !isFusibleOp(*y) || y->results.size() != 1) continue;
         Value* w = y->result();
@@ -2133,10 +2165,49 @@ class Planner {
     const bool hostCounter = hostCounters && trip >= 2 && trip <= kHostCounterMaxTrip && loopDepth_ == 0 && specFloors_.empty() && counter.carry >= 0 &&
                              isInt(op->operands[(size_t)counter.carry]->type.dt) && op->operands[(size_t)counter.carry]->type.numel() == 1;
     const size_t ivCarry = hostCounter ? (size_t)counter.carry : (size_t)-1;
+    // With the counter on the host every iteration's launches carry their own addresses, so a carry that the body
+    // overwrites as a whole can alternate between the two halves of one buffer: iteration k reads half k % 2 and
+    // writes the other.  No kernel then updates a carry in place, the carries need no copies, and kernels that read
+    // the old values may share a launch with the ones that write the new.  Carries updated through a window
+    // (dynamic_update_slice) or passed through unchanged keep one slot.
+    static const bool pingPongOn = !getenv("MI355X_CARRY_PING_PONG") || atoi(getenv("MI355X_CARRY_PING_PONG")) != 0;
+    std::vector<char> pingPong(n, 0);
+    std::vector<int> readHalf(n, -1), writeHalf(n, -1), finalHalf(n, -1);
+    if (hostCounter && pingPongOn) {
+      Region& bodyR = *op->regions[1];
+      Op* bret = bodyR.terminator();
+      for (size_t i = 0; i < n && bret && bret->operands.size() == n; ++i) {
+        if (i == ivCarry) continue;
+        Value* y = bret->operands[i];
+        Op* d = y->def;
+        if (!d || d->parent != &bodyR || y->type.bytes() > (size_t)64 << 20 || y->type.numel() == 0) continue;
+        if (std::count(bret->operands.begin(), bret->operands.end(), y) != 1) continue;
+        const bool whole = (isFusibleOp(*d) && d->name != "dynamic_update_slice" && d->name != "reshape" && !isPassThrough(*d) && d->name != "convert" &&
+                            d->name != "broadcast_in_dim" && d->name != "constant") ||
+                           d->name == "dot_general" || d->name == "dot" || d->name == "reduce";
+        if (whole) pingPong[i] = 1;
+      }
+    }
     std::vector<int> slots(n);
+    std::vector<std::array<int, 2>> initPairs;      // the first halves of double-buffered carries are filled by one launch
+    std::vector<int64_t> initBytes;
     for (size_t i = 0; i < n; ++i) {
       Value* v = op->operands[i];
       int osid = storageOf(v);
+      if (pingPong[i]) {
+        const int64_t bytes = (int64_t)((v->type.bytes() + kAlign - 1) / kAlign * kAlign);
+        slots[i] = newStorage((size_t)(2 * bytes));
+        initPairs.push_back({osid, slots[i]});
+        initBytes.push_back((int64_t)v->type.bytes());
+        std::vector<int64_t> rd, wr;
+        for (int64_t k = 0; k < trip; ++k) { rd.push_back((k % 2) * bytes); wr.push_back(((k + 1) % 2) * bytes); }
+        P.ivTables.push_back(std::move(rd));
+        readHalf[i] = newAlias(slots[i], 0, (int64_t)v->type.bytes(), (int)P.ivTables.size() - 1);
+        P.ivTables.push_back(std::move(wr));
+        writeHalf[i] = newAlias(slots[i], 0, (int64_t)v->type.bytes(), (int)P.ivTables.size() - 1);
+        finalHalf[i] = newAlias(slots[i], (trip % 2) * bytes, (int64_t)v->type.bytes(), -1);
+        continue;
+      }
       bool reuse = st_[osid].kind == BufRef::Temp && st_[osid].values == 1 && v->users.size() == 1 && !boundToOutput_.count(osid) &&
                    !outerStorage(osid);
       if (reuse) slots[i] = osid;
@@ -2144,6 +2215,13 @@ class Planner {
         slots[i] = newStorage(v->type.bytes());
         copyStep(plan, osid, slots[i], (int64_t)v->type.bytes(), "loop carry init");
       }
+    }
+    {
+      // (sources may repeat: the same zeros start several carries; then the copies stay separate)
+      bool distinct = true;
+      for (size_t x = 0; x < initPairs.size(); ++x) for (size_t y = x + 1; y < initPairs.size(); ++y) if (initPairs[x][0] == initPairs[y][0]) distinct = false;
+      if (distinct) multiCopyStep(plan, initPairs, initBytes, "loop carry init");
+      else for (size_t k = 0; k < initPairs.size(); ++k) copyStep(plan, initPairs[k][0], initPairs[k][1], initBytes[k], "loop carry init");
     }
     int tStart = ++time_;
     for (size_t i = 0; i < n; ++i) ref(slots[i], tStart);
@@ -2172,7 +2250,12 @@ class Planner {
     ++loopDepth_;
     Region& cond = *op->regions[0];
     Region& body = *op->regions[1];
-    for (size_t i = 0; i < n; ++i) { bind(cond.args[i].get(), slots[i]); bind(body.args[i].get(), slots[i]); }
+    for (size_t i = 0; i < n; ++i) {
+      const int sid = pingPong[i] ? readHalf[i] : slots[i];
+      bind(cond.args[i].get(), sid);
+      bind(body.args[i].get(), sid);
+    }
+    const int bodyFloor = (int)st_.size();   // storages with higher ids are created by the body
     int counterEnd = -1;   // storage holding the counter's value after the last iteration
     if (hostCounter) {
       // table of the counter's values, one per iteration plus the final one
@@ -2233,6 +2316,29 @@ class Planner {
       Value* v = ret->operands[i];
       if (!hasStorage(v)) materializeNow(v, *bodyPlan);
       src[i] = storageOf(v);
+      if (!pingPong[i]) continue;
+      // the producer writes the other half directly when the value has a buffer of its own made in this body;
+      // otherwise one copy moves it there
+      const int from = src[i];
+      const bool own = from >= bodyFloor && st_[from].kind == BufRef::Temp && st_[from].aliasOf < 0 && st_[from].values == 1 &&
+                       st_[from].bytes <= st_[writeHalf[i]].bytes + (int64_t)kAlign;
+      if (own) {
+        std::function<void(Plan&)> redirect = [&](Plan& p) {
+          for (auto& st : p.steps) {
+            forEachRef(st, [&](BufRef& r, bool) { if (r.index == from) { r.index = writeHalf[i]; r.ivTable = st_[writeHalf[i]].ivTable; r.ivDepth = 0; } });
+            if (st.cond) redirect(*st.cond);
+            for (auto& b : st.bodies) redirect(*b);
+          }
+        };
+        redirect(*bodyPlan);
+        for (int t : st_[from].uses) ref(slots[i], t);
+        st_[from].uses.clear();
+        st_[from].first = st_[from].last = -1;
+        storage_[v] = writeHalf[i];
+      } else {
+        copyStep(*bodyPlan, from, writeHalf[i], (int64_t)v->type.bytes(), "loop carry to its other half");
+      }
+      src[i] = slots[i];
     }
     // carries whose producer can write the slot itself need no copy
     for (size_t i = 0; i < n; ++i) {
@@ -2280,7 +2386,7 @@ class Planner {
     loops_.push_back({tStart, tEnd});
     w.bodies.push_back(std::move(bodyPlan));
     w.hostCounter = hostCounter;
-    for (size_t i = 0; i < n; ++i) bind(op->results[i].get(), i == ivCarry ? counterEnd : slots[i]);
+    for (size_t i = 0; i < n; ++i) bind(op->results[i].get(), i == ivCarry ? counterEnd : pingPong[i] ? finalHalf[i] : slots[i]);
     plan.steps.push_back(std::move(w));
   }
 
@@ -2363,6 +2469,36 @@ class Planner {
       for (size_t j = 0; j < b.args.size(); ++j)
         if (a.args[i].index == b.args[j].index && (a.argWrites[i] || b.argWrites[j])) return false;
     return true;
+  }
+
+  static bool stepsIndependent(Step& a, Step& b) {
+    std::vector<std::pair<int, bool>> ra, rb;
+    forEachRef(a, [&](BufRef& r, bool w) { ra.push_back({r.index, w}); });
+    forEachRef(b, [&](BufRef& r, bool w) { rb.push_back({r.index, w}); });
+    for (auto& x : ra) for (auto& y : rb) if (x.first == y.first && (x.second || y.second)) return false;
+    return true;
+  }
+
+  // Inside a loop body, a small kernel followed by a product it has nothing to do with moves behind the product, next
+  // to the kernel that follows: the two kernels can then share a launch (the bookkeeping writes of a scan step beside
+  // the kernel that computes the new state).
+  void sinkKernelsInLoops(Plan& plan, bool inLoop) {
+    for (auto& s : plan.steps) for (auto& b : s.bodies) sinkKernelsInLoops(*b, s.kind == Step::While);
+    if (!inLoop) return;
+    auto& steps = plan.steps;
+    for (int i = (int)steps.size() - 2; i >= 0; --i) {
+      if (!batchCandidate(steps[(size_t)i]) || steps[(size_t)i + 1].kind == Step::Kernel) continue;
+      // (a kernel that can share the launch of the one before it stays where it is)
+      if (i > 0 && batchCandidate(steps[(size_t)i - 1]) && stepsIndependent(steps[(size_t)i - 1], steps[(size_t)i])) continue;
+      size_t j = (size_t)i + 1;
+      while (j < steps.size() && steps[j].kind != Step::Kernel && steps[j].kind != Step::While && steps[j].kind != Step::Case &&
+             stepsIndependent(steps[(size_t)i], steps[j])) ++j;
+      if (j == (size_t)i + 1 || j >= steps.size() || !batchCandidate(steps[j]) || !stepsIndependent(steps[(size_t)i], steps[j])) continue;
+      // the moved kernel's buffers now live until its new neighbour runs
+      for (auto& a : steps[(size_t)i].args) ref(a.index, steps[j].time);
+      steps[(size_t)i].time = steps[j].time;
+      std::rotate(steps.begin() + i, steps.begin() + i + 1, steps.begin() + (long)j);
+    }
   }
 
   void batchKernels(Plan& plan) {
@@ -2545,7 +2681,12 @@ class Planner {
     const Storage& s = st_[r.index];
     BufRef o;
     o.kind = s.kind;
-    if (s.kind == BufRef::Param || s.kind == BufRef::Output) { o.index = s.index; o.offset = r.offset; }
+    if (s.aliasOf >= 0) {
+      const Storage& parent = st_[s.aliasOf];
+      o.kind = parent.kind;
+      o.index = (parent.kind == BufRef::Param || parent.kind == BufRef::Output) ? parent.index : 0;
+      o.offset = ((parent.kind == BufRef::Param || parent.kind == BufRef::Output) ? 0 : parent.offset) + s.aliasOffset + r.offset;
+    } else if (s.kind == BufRef::Param || s.kind == BufRef::Output) { o.index = s.index; o.offset = r.offset; }
     else { o.index = 0; o.offset = s.offset + r.offset; }
     o.ivTable = r.ivTable;
     o.ivDepth = r.ivDepth;

@@ -169,8 +169,11 @@ void* Device::alloc(size_t bytes) {
   std::lock_guard<std::mutex> lk(mu_);
   void* p = nullptr;
   auto it = free_.lower_bound(sz);
-  // reuse a cached block if it is not wastefully large
+  // reuse a cached block if it is not wastefully large; among blocks of that size the one released last (equal keys keep
+  // their insertion order): a train step that releases its old state and allocates its new one then sees the same few
+  // address sets over and over, whatever else sits in the pool, which is what lets captured graphs be replayed
   if (it != free_.end() && it->first <= sz + sz / 4 + 4096) {
+    it = std::prev(free_.upper_bound(it->first));
     p = it->second;
     sz = it->first;
     free_.erase(it);
@@ -669,7 +672,7 @@ void Executable::replayIterations(const Step& s, bool withCond, int64_t trip, co
     if (withCond) runPlan(*s.cond, in, out);
     runPlan(body, in, out);
   };
-  struct ResetIteration { int64_t& v; ~ResetIteration() { v = 0; } } resetIteration{hostIteration_};
+  struct RestoreIteration { int64_t& v; int64_t was; ~RestoreIteration() { v = was; } } restoreIteration{hostIteration_, hostIteration_};   // (an inner loop leaves the outer loop's iteration as it found it)
   const size_t unitSteps = body.steps.size() + (withCond ? s.cond->steps.size() : 0);
   const int64_t nodeLimit = counted ? 8192 : 1024;
   const bool graphOk = useGraphs_ && !capturing_ && timingKinds_.empty() && trip >= (withCond ? 16 : 4) && unitSteps > 0 && capturable(body) &&
@@ -880,7 +883,8 @@ std::vector<std::shared_ptr<DeviceBuffer>> Executable::execute(const std::vector
   if (timedCall_ && timingRepeat_ > 1 && !timingKinds_.empty()) prepareShadows(inputs);
   if (!runPlanFromGraph(inputs, outPtrs)) runPlan(prog_->plan, inputs, outPtrs);
   if (mayDonate) {
-    for (size_t i = 0; i < inputs.size() && i < prog_->paramDonation.size(); ++i) {
+    // (released last to first: the next call's results, allocated first to last, then take these blocks in order)
+    for (size_t i = std::min(inputs.size(), prog_->paramDonation.size()); i-- > 0;) {
       if (prog_->paramDonation[i] == -1 || i >= mayDonate->size() || !(*mayDonate)[i]) continue;
       bool again = false;   // the same buffer passed for another argument stays alive
       for (size_t j = 0; j < inputs.size(); ++j) if (j != i && inputs[j] == inputs[i]) again = true;
