@@ -83,13 +83,23 @@ __device__ __forceinline__ unsigned char* stageBase() {
 template <int N>
 struct Const { static constexpr int value = N; };
 
-template <int BM, int BN, int STAGES, bool BNN>
-__global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
+// WM wavefront rows by 2 wavefront columns per workgroup: 2 x 2 for the tiles up to 256 x 128, 4 x 2 (512 lanes, two
+// wavefronts per SIMD, each 64 x 128 of the result) for the 256 x 256 tile.  The large tile is what the matrix pipes
+// need to stay fed: a stage of it carries 64 KB for 2048 cycles of products per compute unit (32 bytes a cycle through
+// the vector memory path, half of what that path delivers), where a 128 x 64 tile asks for 24 KB per 256 cycles and
+// three resident workgroups together saturate the path at under half of the matrix peak; and with two wavefronts on
+// a SIMD one reads its operands from LDS while the other multiplies.  What it cannot do is keep more than one stage
+// in flight (two stages fill 128 KB of LDS), so it waits for memory about 60 % of the time and pays only for long K.
+template <int BM, int BN, int STAGES, bool BNN, int WM = 2>
+__global__ void __launch_bounds__(WM * 128) gemm_bf16_async(AsyncArgs g) {
   constexpr int BK = 64;
-  constexpr int TM = BM / 64, TN = BN / 64;
+  constexpr int NW = WM * 2;                  // wavefronts per workgroup
+  constexpr int NT = NW * 64;
+  constexpr int TM = BM / (32 * WM), TN = BN / 64;
   constexpr int STAGE_BYTES = (BM + BN) * 128;
-  constexpr int NI = (BM + BN) / 32;          // direct loads per wavefront per stage (8 rows each)
+  constexpr int NI = (BM + BN) / (8 * NW);    // direct loads per wavefront per stage (8 rows each)
   static_assert((STAGES - 2) * NI <= 63, "vmcnt range");
+  static_assert(BM % (32 * WM) == 0 && (BM / 8) % NW == 0 && (BN / 8) % NW == 0, "tile split over the wavefronts");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
 
@@ -112,7 +122,7 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
   const u16* src[NI];
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
-    const int c = j * 4 + wave;                       // 8-row group within the stage
+    const int c = j * NW + wave;                      // 8-row group within the stage
     const int r = c * 8 + (lane >> 3);                // row within [A rows | B rows]
     const int kv = (lane & 7) ^ ((r >> 1) & 7);       // logical k-slot this lane fetches
     if (r < BM) {
@@ -139,9 +149,9 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
     const long long k0 = (long long)(slab < nk ? slab : nk - 1) * BK;   // past the end: harmless re-read keeps the count uniform
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
-      unsigned char* dst = ring + (j * 4 + wave) * 1024;
-      // loads j >= BM/32 fill the B part; an n-contiguous B advances by rows
-      const long long step = (BNN && j >= BM / 32) ? k0 * g.bLd : k0;
+      unsigned char* dst = ring + (j * NW + wave) * 1024;
+      // loads j >= BM / (8 NW) fill the B part; an n-contiguous B advances by rows
+      const long long step = (BNN && j >= BM / (8 * NW)) ? k0 * g.bLd : k0;
       __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[j] + step), LDS_PTR(dst), 16, 0, 0);
     }
   };
@@ -168,7 +178,7 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
   static_assert(STAGES >= 2 && STAGES <= 4, "ring length");
 
   // fragment addresses: row-dependent part of the swizzle is fixed per lane
-  const int arow = wm * (BM / 2) + (lane & 31);
+  const int arow = wm * (BM / WM) + (lane & 31);
   const int brow = BM + wn * (BN / 2) + (lane & 31);
   const int khalf = lane >> 5;
   // n-contiguous B: per-lane byte offset of its transposing reads inside a stage.  Lane d of a 16-lane group
@@ -259,23 +269,27 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
     constexpr int LDW = BN + 8;   // staged row in elements: 16-byte aligned, consecutive rows 4 banks apart
     static_assert(64 * LDW * 2 <= STAGE_BYTES, "a band fits one stage");
     __syncthreads();              // every wavefront has read its last operands; all direct loads have landed
+    // a band is 64 rows: the 32-row block i of two neighbouring wavefront rows (pair p)
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      u16* band = (u16*)((i & 1) ? stageBase<STAGE_BYTES, 1>() : stageBase<STAGE_BYTES, 0>());
+    for (int b = 0; b < TM * (WM / 2); ++b) {
+      const int i = b % TM, p = b / TM;
+      u16* band = (u16*)((b & 1) ? stageBase<STAGE_BYTES, 1>() : stageBase<STAGE_BYTES, 0>());
+      if ((wm >> 1) == p) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int lc = wn * (BN / 2) + j * 32 + (lane & 31);
-        const float bias = biasv[j];
+        for (int j = 0; j < TN; ++j) {
+          const int lc = wn * (BN / 2) + j * 32 + (lane & 31);
+          const float bias = biasv[j];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int lr = wm * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-          band[lr * LDW + lc] = finish16(acc[i][j][e], bias);
+          for (int e = 0; e < 16; ++e) {
+            const int lr = (wm & 1) * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+            band[lr * LDW + lc] = finish16(acc[i][j][e], bias);
+          }
         }
       }
       __syncthreads();   // also orders this band's reads of the other buffer's previous use before its next writes
-      for (int sg = tid; sg < 64 * (BN / 8); sg += 256) {
+      for (int sg = tid; sg < 64 * (BN / 8); sg += NT) {
         const int lr = sg / (BN / 8), cs = sg % (BN / 8);
-        const long long row = m0 + (lr >> 5) * (BM / 2) + i * 32 + (lr & 31);
+        const long long row = m0 + (2 * p + (lr >> 5)) * (BM / WM) + i * 32 + (lr & 31);
         const long long col = n0 + cs * 8;
         if (row < g.M && col < g.N) *(uint4*)((u16*)g.c + cBase + row * g.N + col) = *(const uint4*)(band + lr * LDW + cs * 8);
       }
@@ -291,7 +305,7 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
         const float bias = biasv[j];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const long long row = m0 + wm * (BM / 2) + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          const long long row = m0 + wm * (BM / WM) + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
           if (row >= g.M) continue;
           if (g.outBf16) ((u16*)g.c)[cBase + row * g.N + col] = finish16(acc[i][j][e], bias);
           else ((float*)g.c)[cBase + row * g.N + col] = acc[i][j][e] + bias;
@@ -301,9 +315,9 @@ __global__ void __launch_bounds__(256) gemm_bf16_async(AsyncArgs g) {
   }
 }
 
-template <int BM, int BN, int STAGES, bool BNN>
+template <int BM, int BN, int STAGES, bool BNN, int WM = 2>
 int launch(const AsyncArgs& g, hipStream_t st) {
-  gemm_bf16_async<BM, BN, STAGES, BNN><<<dim3((unsigned)g.total), 256, 0, st>>>(g);   // the ring is static LDS
+  gemm_bf16_async<BM, BN, STAGES, BNN, WM><<<dim3((unsigned)g.total), WM * 128, 0, st>>>(g);   // the ring is static LDS
   return hipGetLastError() == hipSuccess ? 0 : 3;
 }
 
@@ -452,10 +466,22 @@ extern "C" int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, co
   // 42 us on 128x64 tiles against 53 us on 768 tiles of 128x128)
   else if (d->M > 64 && d->N > 64 && tiles(128, 128) >= (pb.rowsOfK ? 1536 : 768)) { bm = 128; bn = 128; }
   else if (d->M > 64 && tiles(128, 64) >= 768) { bm = 128; bn = 64; }
+  // The 256 x 256 tile (eight wavefronts) for large products with a long K.  Measured (k-contiguous / [K][N] rhs):
+  // 8192^3 925 / 895 TFLOP/s against 857 / 818 on 256 x 128 tiles, 4096^3 864 / 821 against 719 / 694; with K = 768
+  // (4096 x 2304 and 4096 x 3072 outputs) it is no faster or slower than the 128 x 64 tiles, and with fewer than 128 tiles
+  // (N = 768) much slower.  One 64 KB stage in flight per compute unit does not cover the load latency (about 5 500
+  // cycles per 64 of K against 2 048 of products), and the 160 KB of LDS hold no third stage of this tile.
+  // MI355X_GEMM_WIDE=0 never, =2 whenever the shape allows.
+  const int wideMode = getenv("MI355X_GEMM_WIDE") ? atoi(getenv("MI355X_GEMM_WIDE")) : 1;   // read at every call: tests switch it
+  bool wide = false;
+  if (!force && wideMode != 0 && d->M >= 256 && d->N >= 256)
+    wide = wideMode == 2 || (tiles(256, 256) >= 192 && d->K >= 2048);
+  if (wide) { bm = 256; bn = 256; }
   g.tilesM = (int)((d->M + bm - 1) / bm);
   g.tilesN = (int)((d->N + bn - 1) / bn);
   g.total = (long long)g.tilesM * g.tilesN * nb;
   if (g.total > 0x7FFFFFFFll) return -1;
+  if (wide) return pb.rowsOfK ? launch<256, 256, 2, true, 4>(g, st) : launch<256, 256, 2, false, 4>(g, st);
   // two ring stages keep three workgroups of 128x64 resident per compute unit; deeper rings (MI355X_GEMM_STAGES=3|4, a tuning aid)
   // leave room for fewer and measured slower on the benchmark shapes: twelve resident wavefronts hide more than a third stage
   static const int stagesEnv = getenv("MI355X_GEMM_STAGES") ? atoi(getenv("MI355X_GEMM_STAGES")) : 0;
