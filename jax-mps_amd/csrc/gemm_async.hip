@@ -110,7 +110,20 @@ __global__ void __launch_bounds__(WM * 128) gemm_bf16_async(AsyncArgs g) {
   const unsigned perBatch = (unsigned)g.tilesM * (unsigned)g.tilesN;
   const unsigned bzu = id / perBatch;
   const unsigned t = id - bzu * perBatch;
-  const int tm = (int)(t / (unsigned)g.tilesN), tn = (int)(t - (unsigned)tm * (unsigned)g.tilesN);
+  int tm, tn;
+  if (WM == 4) {
+    // eight tile rows are walked together, column by column: the 32 workgroups an XCD runs at a time then share 8 + 4
+    // operand slabs per step of K in its L2 instead of 1 + 32
+    const unsigned perGroup = 8u * (unsigned)g.tilesN;
+    const unsigned group = t / perGroup, first = group * 8u;
+    const unsigned rows = (unsigned)g.tilesM - first < 8u ? (unsigned)g.tilesM - first : 8u;
+    const unsigned in = t - group * perGroup;
+    tm = (int)(first + in % rows);
+    tn = (int)(in / rows);
+  } else {
+    tm = (int)(t / (unsigned)g.tilesN);
+    tn = (int)(t - (unsigned)tm * (unsigned)g.tilesN);
+  }
   const long long bz = bzu;
   const long long b0 = bzu / (unsigned)g.batch1, b1 = bzu - (unsigned)b0 * (unsigned)g.batch1;
   const u16* A = g.a + b0 * g.aB0 + b1 * g.aB1;
