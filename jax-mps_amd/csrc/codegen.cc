@@ -943,6 +943,8 @@ bool isSimpleReduce(const Op& reduce) { return reduce.operands.size() == 2 && re
 const char* simpleReduceKind(const Op& reduce) { return reduce.operands.size() == 2 ? reduceKind(reduce) : nullptr; }
 
 // ------------------------------------------------------------------ loop kernels
+static constexpr int64_t kSpreadThreads = 65536;   // lanes a small kernel is spread over before its lanes take vectors (256 compute units x 256)
+
 FusedCode generateLoopKernel(Value* root, const LeafPredicate& isLeaf) { return generateLoopKernel(std::vector<Value*>{root}, isLeaf); }
 
 // One pass over a shared index space that stores several results: all roots have the same
@@ -957,8 +959,11 @@ FusedCode generateLoopKernel(const std::vector<Value*>& roots, const LeafPredica
   int V = 8;
   for (auto* r : roots) V = std::min(V, pickVector(r->type));
   bool i64 = needs64(all);
-  Emitter em(inner, V, i64);
   int64_t N = root->type.numel();
+  // a small index space is spread over more lanes instead of vectors: a lane that walks four elements of a chain of
+  // exponentials in turn takes four times as long, and nothing this size is bound by memory transactions
+  while (V > 1 && N / V < kSpreadThreads) V >>= 1;
+  Emitter em(inner, V, i64);
   IdxDim lin;
   lin.isConst = false;
   lin.base = "base";
@@ -1440,6 +1445,8 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     while (v > 1 && (!innerIsLastKept || lastKept % v != 0)) v >>= 1;
     V = v;
   }
+  const bool onePass = Rn * Kn <= reduceOnePassLimit();
+  if (onePass) while (V > 1 && Rn * Kn / V < kSpreadThreads) V >>= 1;   // small inputs: lanes before vectors, as in the loop kernels
   int64_t kvecs = (Kn + V - 1) / V;
   int TX = 1;
   while (TX < 64 && TX < kvecs) TX <<= 1;
@@ -1450,6 +1457,12 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
   if (Rn > (int64_t)TY * 16) P = std::min<int64_t>((Rn + TY * colPerThread - 1) / (TY * colPerThread), std::max<int64_t>(1, 2048 / gridX));
   // a small input is cheaper to walk in one launch (a few dozen loads per lane) than to split over a second, dependent one
   if (Rn * Kn <= reduceOnePassLimit() && Rn <= (int64_t)TY * 128) P = 1;
+  // one pass over few columns: narrower column tiles put more workgroups on the rows (64 x 1024: 32 workgroups of 32 row
+  // lanes instead of 4 of 4), which matters when every element is a chain of its own
+  if (P == 1) {
+    const int64_t want = std::min<int64_t>(256, std::max<int64_t>(1, Rn * Kn / V / 512));   // about two visits per lane, a workgroup per compute unit at most
+    while (TX > 8 && (kvecs + TX - 1) / TX < want && 256 / (TX / 2) <= Rn) TX >>= 1, TY = 256 / TX, gridX = (kvecs + TX - 1) / TX;
+  }
   bool partial = P > 1;
   Emitter em(isLeaf, V, i64);
   IdxDim klin;

@@ -81,14 +81,15 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
                size_t workspace_bytes, mi355_stream_t s);
 size_t mi355_gemm_workspace_bytes(const mi355_gemm_desc* d);
 // Small fp32 products (mi355_gemm_is_small) run as one launch without workspace; two of them with the same
-// result shape can be summed by the same launch: C = A1 x B1 + A2 x B2 (+ bias).  d2 may be NULL.  -1 = not small.
+// result shape can be summed by the same launch: C = A1 x B1 + A2 x B2 (+ addend) (+ bias).  d2 may be NULL; addend, a
+// tensor laid out like C (it may not be C itself), may be NULL.  -1 = not small.
 int mi355_gemm_is_small(const mi355_gemm_desc* d);   // 0, or the tile edge (16 / 32) the small-product kernel uses
 // n <= 4 independent small products of one tile class in one launch; d2[i] may be NULL.  -1 = the group does not qualify.
 int mi355_gemm_small_group(int n, const mi355_gemm_desc* const* d1, const void* const* a1, const void* const* b1,
                            const mi355_gemm_desc* const* d2, const void* const* a2, const void* const* b2, void* const* c,
-                           const void* const* bias, mi355_stream_t s);
+                           const void* const* bias, const void* const* addend, mi355_stream_t s);
 int mi355_gemm_small_sum(const mi355_gemm_desc* d1, const void* a1, const void* b1, const mi355_gemm_desc* d2, const void* a2,
-                         const void* b2, void* c, const void* bias, mi355_stream_t s);
+                         const void* b2, void* c, const void* bias, const void* addend, mi355_stream_t s);
 // bf16 operands with 16-byte-loadable layouts on 128x128 / 128x64 / 64x64 tiles; -1 = layout does not qualify
 // bf16, both operands k-contiguous, K % 64 == 0: LDS ring filled by direct global->LDS loads
 int mi355_gemm_bf16_async(const mi355_gemm_desc* d, const void* a, const void* b, void* c, const void* bias, void* workspace,

@@ -161,4 +161,14 @@ void rebuildUses(Region& r);          // recompute Value::users for a region tre
 void checkSupported(const Module& m); // throws CompileError naming unsupported ops
 int countOps(const Region& r);
 
+// Loop analysis shared by the passes and the planner (hoist.cc)
+bool constantInt(Value* v, int64_t& out);   // the value of a compile-time constant integer scalar
+struct LoopCounter { int carry = -1; int64_t init = 0, step = 0; };
+// iterations of a `while` whose condition compares one carry with a constant and whose body steps that carry by a
+// constant from a constant start; -1 when the count is not static.  `counter` (optional) receives the carry.
+int64_t staticTripCount(Op* whileOp, LoopCounter* counter = nullptr);
+// inside counted loops, a product of a loop-invariant operand with the counter-selected slice of a loop-invariant tensor
+// becomes one product over the whole tensor ahead of the loop, and the body slices its result
+void hoistLoopProducts(Module& m);
+
 }  // namespace mi355

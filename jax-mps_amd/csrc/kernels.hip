@@ -191,6 +191,7 @@ struct SmallArgs {
   int pairs;
   float* c;
   const float* bias;   // N values or null
+  const float* addend; // a tensor laid out like C that is added to the product (an accumulator carried by a loop), or null
   long long M, N;
   int batch1;
   int relu;            // the stored value is maximum(sum + bias, 0)
@@ -306,10 +307,12 @@ __device__ __forceinline__ void smallGemmTileBody(const SmallArgs& g, unsigned b
   }
   __syncthreads();
   float* C = g.c + (long long)bz * g.M * g.N;
+  const float* D = g.addend ? g.addend + (long long)bz * g.M * g.N : nullptr;
   for (int e = threadIdx.x; e < T * T; e += 256) {
     const long long row = m0 + e / T, col = n0 + e % T;
     if (row < g.M && col < g.N) {
-      const float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
+      float sum = (red[0][e] + red[1][e]) + (red[2][e] + red[3][e]);
+      if (D) sum += D[row * g.N + col];
       const float v = g.bias ? sum + g.bias[col] : sum;
       C[row * g.N + col] = g.relu ? ((v > 0.f || v != v) ? v : 0.f) : v;   // maximum(v, 0): NaN stays NaN, -0 becomes +0
     }
@@ -1079,7 +1082,7 @@ static SmallPair smallPair(const mi355_gemm_desc* d, const void* a, const void* 
 
 int mi355_gemm_is_small(const mi355_gemm_desc* d) { return smallGemmTile(d); }
 
-static bool fillSmall(SmallArgs& g, const mi355_gemm_desc* d1, const void* a1, const void* b1, const mi355_gemm_desc* d2, const void* a2,
+static bool fillSmall(SmallArgs& g, const void* addend, const mi355_gemm_desc* d1, const void* a1, const void* b1, const mi355_gemm_desc* d2, const void* a2,
                       const void* b2, void* c, const void* bias) {
   if (!smallGemmTile(d1)) return false;
   if (d2 && (!smallGemmTile(d2) || d2->M != d1->M || d2->N != d1->N || d2->batch0 != d1->batch0 || d2->batch1 != d1->batch1)) return false;
@@ -1088,17 +1091,18 @@ static bool fillSmall(SmallArgs& g, const mi355_gemm_desc* d1, const void* a1, c
   g.pairs = d2 ? 2 : 1;
   g.c = (float*)c;
   g.bias = (const float*)bias;
+  g.addend = (const float*)addend;
   g.M = d1->M; g.N = d1->N;
   g.batch1 = (int)d1->batch1;
   g.relu = d1->act == 2;
   return true;
 }
 
-// n <= 4 independent problems of one tile class (mi355_gemm_is_small gives it), each C = A1 x B1 (+ A2 x B2) (+ bias);
-// d2[i] may be NULL.
+// n <= 4 independent problems of one tile class (mi355_gemm_is_small gives it), each C = A1 x B1 (+ A2 x B2) (+ addend)
+// (+ bias); d2[i] and addend[i] may be NULL.
 int mi355_gemm_small_group(int n, const mi355_gemm_desc* const* d1, const void* const* a1, const void* const* b1,
                            const mi355_gemm_desc* const* d2, const void* const* a2, const void* const* b2, void* const* c,
-                           const void* const* bias, mi355_stream_t s) {
+                           const void* const* bias, const void* const* addend, mi355_stream_t s) {
   if (n <= 0) return 0;
   if (n > kMaxSmallGroup) return -1;
   SmallGroupArgs g;
@@ -1106,7 +1110,7 @@ int mi355_gemm_small_group(int n, const mi355_gemm_desc* const* d1, const void* 
   unsigned total = 0;
   int k = 0;
   for (int i = 0; i < n; ++i) {
-    if (smallGemmTile(d1[i]) != t || !fillSmall(g.prob[k], d1[i], a1[i], b1[i], d2[i], a2[i], b2[i], c[i], bias[i])) return -1;
+    if (smallGemmTile(d1[i]) != t || !fillSmall(g.prob[k], addend[i], d1[i], a1[i], b1[i], d2[i], a2[i], b2[i], c[i], bias[i])) return -1;
     const long long nb = d1[i]->batch0 * d1[i]->batch1;
     if (d1[i]->M <= 0 || d1[i]->N <= 0 || nb <= 0) continue;
     g.first[k] = total;
@@ -1123,9 +1127,10 @@ int mi355_gemm_small_group(int n, const mi355_gemm_desc* const* d1, const void* 
   return check("gemm group");
 }
 
-// C = A1 x B1 (+ A2 x B2 when d2 is given: same M, N and batch dims) (+ bias), both products small fp32 ones.
+// C = A1 x B1 (+ A2 x B2 when d2 is given: same M, N and batch dims) (+ addend, laid out like C) (+ bias), both products
+// small fp32 ones.
 int mi355_gemm_small_sum(const mi355_gemm_desc* d1, const void* a1, const void* b1, const mi355_gemm_desc* d2, const void* a2,
-                         const void* b2, void* c, const void* bias, mi355_stream_t s) {
+                         const void* b2, void* c, const void* bias, const void* addend, mi355_stream_t s) {
   const int t = smallGemmTile(d1);
   if (!t) return -1;
   if (d2 && (!smallGemmTile(d2) || d2->M != d1->M || d2->N != d1->N || d2->batch0 != d1->batch0 || d2->batch1 != d1->batch1)) return -1;
@@ -1136,6 +1141,7 @@ int mi355_gemm_small_sum(const mi355_gemm_desc* d1, const void* a1, const void* 
   g.pairs = d2 ? 2 : 1;
   g.c = (float*)c;
   g.bias = (const float*)bias;
+  g.addend = (const float*)addend;
   g.M = d1->M; g.N = d1->N;
   g.batch1 = (int)d1->batch1;
   g.relu = d1->act == 2;
@@ -1175,7 +1181,7 @@ int mi355_gemm(const mi355_gemm_desc* d, const void* a, const void* b, void* c, 
     if (r >= 0) return r ? r : addBias(d, c, bias, s);
   }
   if (d->act == 2 ? !smallGemmTile(d) : (d->act && d->out_dtype != 1)) return 2;   // epilogues: GELU for bf16 results, maximum(x, 0) for small fp32 products
-  if (smallGemmTile(d)) return mi355_gemm_small_sum(d, a, b, nullptr, nullptr, nullptr, c, bias, s);
+  if (smallGemmTile(d)) return mi355_gemm_small_sum(d, a, b, nullptr, nullptr, nullptr, c, bias, nullptr, s);
   mi355_conv_desc cd;
   // strided views may start anywhere; the implicit-GEMM loaders issue 16-byte loads
   if (gemmAsPointwiseConv(d, &cd) && (((uintptr_t)a | (uintptr_t)b) & 15) == 0) {

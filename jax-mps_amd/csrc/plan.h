@@ -98,6 +98,7 @@ struct Step {
   ConvDesc conv;
   ScatterDesc scatter;
   BufRef bias;                     // Gemm: per-column values added to the product (kind None: no bias)
+  BufRef addend;                   // Gemm (small fp32 products): a tensor of the result's shape added to the product (kind None: none)
   int statsArg = -1;               // Conv: index in args of the column-sum buffer (the sum-of-squares buffer follows), or -1
   // A step whose results nothing needs for a while (a filter gradient, read only by the optimizer update at the end of
   // the step) may run on a second stream next to the steps that follow it: forkId >= 0 marks it, and the first later

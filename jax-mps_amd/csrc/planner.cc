@@ -427,19 +427,7 @@ class Planner {
   }
 
   // constant scalar value of an i32/i64/etc. value if it is a compile-time constant
-  static bool constInt(Value* v, int64_t& out) {
-    Op* d = v->def;
-    while (d && (d->name == "reshape" || d->name == "convert" || d->name == "broadcast_in_dim") && d->operands[0]->type.numel() == 1) d = d->operands[0]->def;
-    if (!d || d->name != "constant") return false;
-    auto& dd = *d->attrs.at("value").dense;
-    if (!isInt(dd.type.dt) || dd.type.numel() != 1) return false;
-    int64_t x = 0;
-    size_t sz = dtypeSize(dd.type.dt);
-    memcpy(&x, dd.bytes.data(), sz);
-    if (isSignedInt(dd.type.dt) && sz < 8 && ((x >> (8 * sz - 1)) & 1)) x |= ~((int64_t(1) << (8 * sz)) - 1);
-    out = x;
-    return true;
-  }
+  static bool constInt(Value* v, int64_t& out) { return constantInt(v, out); }
 
   void emitRegion(Region& r, Plan& plan) {
     // attention chains: everything between the two products is skipped, the second product emits the fused step
@@ -481,6 +469,7 @@ class Planner {
       if (emitted_.count(op)) return;
       const std::string& n = op->name;
       if (n == "return") return;
+      if (n == "dynamic_slice" && sliceBecomesAlias(op, r)) return;
       if (isFusibleOp(*op) && op->results.size() == 1) {
         Value* v = op->result();
         if (!needMat_[v]) return;
@@ -521,6 +510,41 @@ class Planner {
       if (n == "case") { emitCase(op, plan); return; }
       throw CompileError("no lowering for stablehlo." + n);
     }
+  }
+
+  // Inside a host-counted loop, the counter-selected slice of a tensor that the loop never writes (xs[i], or slice i of a
+  // product taken over the whole sequence ahead of the loop) is a contiguous block whose address the host knows at every
+  // iteration: the value becomes a name for that block, and the kernels that read it take the address as an argument
+  // instead of loading the counter first and the data after it.
+  bool sliceBecomesAlias(Op* op, Region& r) {
+    static const bool on = !getenv("MI355X_SLICE_ALIASES") || atoi(getenv("MI355X_SLICE_ALIASES")) != 0;
+    Value* x = op->operands[0];
+    Value* v = op->result();
+    if (!on || loopDepth_ != 1 || ivArgs().empty() || !hasStorage(x) || v->type.numel() == 0 || !r.parent || r.parent->name != "while") return false;
+    // never written while the loop runs: defined outside it, or a carry handed on unchanged
+    bool invariant = regionOf(x) != &r;
+    if (x->argOf == &r) {
+      Op* ret = r.terminator();
+      invariant = ret && (size_t)x->defIndex < ret->operands.size() && ret->operands[(size_t)x->defIndex] == x;
+    }
+    if (!invariant || st_[storageOf(x)].aliasOf >= 0) return false;
+    const auto& sizes = op->ints("sizes");
+    const auto& dims = x->type.dims;
+    if (sizes.size() != dims.size()) return false;
+    // one contiguous block: unit dims, then at most one partial dim, then whole dims
+    int last = -1;
+    for (int d = 0; d < (int)dims.size(); ++d) if (sizes[(size_t)d] != dims[(size_t)d]) last = d;
+    for (int d = 0; d < last; ++d) if (sizes[(size_t)d] != 1) return false;
+    int64_t base = 0;
+    std::vector<int64_t> perIter;
+    if (!hostSlice(op, stridesOf(x->type), base, perIter) || perIter.empty()) return false;
+    const int64_t esz = (int64_t)dtypeSize(v->type.dt);
+    for (auto& e : perIter) e *= esz;
+    P.ivTables.push_back(std::move(perIter));
+    const int sid = newAlias(storageOf(x), 0, (int64_t)v->type.bytes(), (int)P.ivTables.size() - 1);
+    bind(v, sid);
+    emitted_.insert(op);
+    return true;
   }
 
   // a value that analysis left fused but some consumer needs in memory after all
@@ -571,7 +595,9 @@ class Planner {
     static const bool on = !getenv("MI355X_REDUCE_STORES") || atoi(getenv("MI355X_REDUCE_STORES")) != 0;
     Value* v = op->result();
     // (a reduction over a small input is one launch of a few workgroups: too few to also compute and store the value)
-    if (!on || loopDepth_ > 0 || !takesKernel(op) || v->type.numel() <= reduceOnePassLimit() || op->name == "constant" || op->has("force_materialize")) return false;
+    // (inside a loop body the launch saved is worth more than the workgroups, provided the one pass still has a few dozen)
+    const bool sized = loopDepth_ > 0 ? v->type.numel() >= 16384 && v->type.numel() <= reduceOnePassLimit() : v->type.numel() > reduceOnePassLimit();
+    if (!on || !sized || !takesKernel(op) || op->name == "constant" || op->has("force_materialize")) return false;
     if (v->type.dt != DType::F32 && v->type.dt != DType::BF16) return false;
     Op* red = nullptr;
     size_t posRed = 0;
@@ -1728,6 +1754,21 @@ class Planner {
         }
       }
     }
+    // ... -> add(x, y) with y a tensor in memory and no other reader of the product (a gradient summed into an accumulator
+    // that a loop carries): a small fp32 product adds y while it stores, in the order product + y like the add itself
+    Op* accumulate = nullptr;
+    Value* addendV = nullptr;
+    {
+      static const bool on = !getenv("MI355X_GEMM_ADDEND") || atoi(getenv("MI355X_GEMM_ADDEND")) != 0;
+      mi355_gemm_desc small = toAbi(g);
+      if (on && !biasAdd && !fuseAct && !relu && c->type.numel() > 0 && g.inType == DType::F32 && g.outType == DType::F32 &&
+          mi355_gemm_is_small(&small) && produced->users.size() == 1 && produced->users[0]->name == "add" &&
+          produced->users[0]->parent == op->parent) {
+        Op* u = produced->users[0];
+        Value* y = u->operands[0] == produced ? u->operands[1] : u->operands[0];
+        if (y != produced && y->type == produced->type && hasStorage(y)) accumulate = u, addendV = y;
+      }
+    }
     int sid = newStorage(c->type.bytes());
     bind(produced, sid);
     if (sumAdd) emitted_.insert(sumAdd);
@@ -1737,7 +1778,12 @@ class Planner {
     s.kind = Step::Gemm;
     s.time = t;
     s.label = "dot_general " + a->type.str() + " x " + b->type.str() + (second ? " + " + second->operands[0]->type.str() + " x " + second->operands[1]->type.str() : "") +
-              (biasV ? " + bias" : "") + (fuseAct ? " + gelu" : "") + (relu ? " + relu" : "");
+              (biasV ? " + bias" : "") + (fuseAct ? " + gelu" : "") + (relu ? " + relu" : "") + (accumulate ? " + tensor" : "");
+    if (accumulate) {
+      s.addend = ref(storageOf(addendV), t);
+      storage_[accumulate->result()] = sid;   // the step writes the sum; nothing reads the bare product, so the buffer still holds one value
+      emitted_.insert(accumulate);
+    }
     s.gemm = g;
     if (relu) {
       s.gemm.act = 2;
@@ -1975,51 +2021,8 @@ class Planner {
 
   // counted loop: cond is `carry_i <cmp> const`, body returns carry_i + const, init is a constant
   // `counter` (optional) receives the carry index, start and step of the counter the trip count was read from
-  struct CounterInfo { int carry = -1; int64_t init = 0, step = 0; };
-  int64_t detectTripCount(Op* op, CounterInfo* counter = nullptr) {
-    Region& cond = *op->regions[0];
-    Region& body = *op->regions[1];
-    Op* ret = cond.terminator();
-    if (!ret || ret->operands.size() != 1) return -1;
-    Op* cmp = ret->operands[0]->def;
-    if (!cmp || cmp->name != "compare") return -1;
-    Value* lhs = cmp->operands[0];
-    Value* rhs = cmp->operands[1];
-    std::string dir = cmp->str("direction");
-    int64_t limit;
-    if (!(lhs->argOf == &cond) || !constInt(rhs, limit)) {
-      if (rhs->argOf == &cond && constInt(lhs, limit)) {
-        std::swap(lhs, rhs);
-        dir = dir == "LT" ? "GT" : dir == "GT" ? "LT" : dir == "LE" ? "GE" : dir == "GE" ? "LE" : dir;
-      } else {
-        return -1;
-      }
-    }
-    int ci = lhs->defIndex;
-    int64_t init;
-    if (!constInt(op->operands[ci], init)) return -1;
-    Value* next = body.terminator()->operands[ci];
-    Op* add = next->def;
-    if (!add || (add->name != "add" && add->name != "subtract")) return -1;
-    int64_t step;
-    Value* barg = body.args[ci].get();
-    if (add->operands[0] == barg && constInt(add->operands[1], step)) {
-      if (add->name == "subtract") step = -step;
-    } else if (add->name == "add" && add->operands[1] == barg && constInt(add->operands[0], step)) {
-    } else {
-      return -1;
-    }
-    if (step == 0) return -1;
-    int64_t n = 0;
-    if (dir == "LT" && step > 0) n = limit > init ? (limit - init + step - 1) / step : 0;
-    else if (dir == "LE" && step > 0) n = limit >= init ? (limit - init) / step + 1 : 0;
-    else if (dir == "GT" && step < 0) n = init > limit ? (init - limit + (-step) - 1) / (-step) : 0;
-    else if (dir == "GE" && step < 0) n = init >= limit ? (init - limit) / (-step) + 1 : 0;
-    else if (dir == "NE" && (limit - init) % step == 0 && (limit - init) / step >= 0) n = (limit - init) / step;
-    else return -1;
-    if (counter) { counter->carry = ci; counter->init = init; counter->step = step; }
-    return n;
-  }
+  using CounterInfo = LoopCounter;
+  int64_t detectTripCount(Op* op, CounterInfo* counter = nullptr) { return staticTripCount(op, counter); }
 
   // `cond` (optional): a step whose condBuf / condMode / condType / condWant / condCount the copy takes over
   void applyCond(Step& c, const Step* cond, int t) {
@@ -2114,6 +2117,7 @@ class Planner {
     if (s.src.kind != BufRef::None) f(s.src, false);
     if (s.dst.kind != BufRef::None) f(s.dst, true);
     if (s.bias.kind != BufRef::None) f(s.bias, false);
+    if (s.addend.kind != BufRef::None) f(s.addend, false);
     if (s.predBuf.kind != BufRef::None) f(s.predBuf, false);
     if (s.condBuf.kind != BufRef::None) f(s.condBuf, false);
     if (s.parentFlag.kind != BufRef::None) f(s.parentFlag, false);
@@ -2488,16 +2492,29 @@ class Planner {
     auto& steps = plan.steps;
     for (int i = (int)steps.size() - 2; i >= 0; --i) {
       if (!batchCandidate(steps[(size_t)i]) || steps[(size_t)i + 1].kind == Step::Kernel) continue;
-      // (a kernel that can share the launch of the one before it stays where it is)
-      if (i > 0 && batchCandidate(steps[(size_t)i - 1]) && stepsIndependent(steps[(size_t)i - 1], steps[(size_t)i])) continue;
+      // the kernels just before it that can share its launch move with it, or none moves (splitting them would add a launch)
+      int first = i;
+      while (first > 0 && i - first + 1 < (int)kBatchMaxSegments && batchCandidate(steps[(size_t)first - 1])) {
+        bool apart = true;
+        for (int k = first; k <= i && apart; ++k) apart = stepsIndependent(steps[(size_t)first - 1], steps[(size_t)k]);
+        if (!apart) break;
+        --first;
+      }
+      auto runIndependentOf = [&](Step& other) {
+        for (int k = first; k <= i; ++k) if (!stepsIndependent(steps[(size_t)k], other)) return false;
+        return true;
+      };
       size_t j = (size_t)i + 1;
       while (j < steps.size() && steps[j].kind != Step::Kernel && steps[j].kind != Step::While && steps[j].kind != Step::Case &&
-             stepsIndependent(steps[(size_t)i], steps[j])) ++j;
-      if (j == (size_t)i + 1 || j >= steps.size() || !batchCandidate(steps[j]) || !stepsIndependent(steps[(size_t)i], steps[j])) continue;
-      // the moved kernel's buffers now live until its new neighbour runs
-      for (auto& a : steps[(size_t)i].args) ref(a.index, steps[j].time);
-      steps[(size_t)i].time = steps[j].time;
-      std::rotate(steps.begin() + i, steps.begin() + i + 1, steps.begin() + (long)j);
+             runIndependentOf(steps[j])) ++j;
+      if (j == (size_t)i + 1 || j >= steps.size() || !batchCandidate(steps[j]) || !runIndependentOf(steps[j])) { i = first; continue; }
+      // the moved kernels' buffers now live until their new neighbour runs
+      for (int k = first; k <= i; ++k) {
+        for (auto& a : steps[(size_t)k].args) ref(a.index, steps[j].time);
+        steps[(size_t)k].time = steps[j].time;
+      }
+      std::rotate(steps.begin() + first, steps.begin() + i + 1, steps.begin() + (long)j);
+      i = first;
     }
   }
 
@@ -2568,6 +2585,7 @@ class Planner {
       std::vector<int> r{s.args[0].index, s.args[1].index};
       if (s.dual) { r.push_back(s.args[3].index); r.push_back(s.args[4].index); }
       if (s.bias.kind != BufRef::None) r.push_back(s.bias.index);
+      if (s.addend.kind != BufRef::None) r.push_back(s.addend.index);
       return r;
     };
     const int wa = a.args[2].index, wb = b.args[2].index;
@@ -2698,11 +2716,13 @@ class Planner {
       for (auto& part : s.parts) {
         for (auto& a : part.args) a = finalRef(a);
         part.bias = finalRef(part.bias);
+        part.addend = finalRef(part.addend);
       }
       for (auto& a : s.args) a = finalRef(a);
       s.src = finalRef(s.src);
       s.dst = finalRef(s.dst);
       s.bias = finalRef(s.bias);
+      s.addend = finalRef(s.addend);
       s.predBuf = finalRef(s.predBuf);
       s.condBuf = finalRef(s.condBuf);
       s.flagBuf = finalRef(s.flagBuf);
@@ -2804,6 +2824,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   lowerWindowOps(*module);
   lowerRng(*module);
   lowerTopK(*module);
+  hoistLoopProducts(*module);
   reluMasksFromActivations(*module);
   checkSupported(*module);
   eliminateDeadCode(module->main()->body);

@@ -452,10 +452,13 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
     case Step::Gemm: {
       mi355_gemm_desc d = toAbi(s.gemm);
       const void* bias = s.bias.kind == BufRef::None ? nullptr : resolve(s.bias, in, out);
-      if (s.dual) {
-        mi355_gemm_desc d2 = toAbi(s.gemm2);
-        check(mi355_gemm_small_sum(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), &d2, resolve(s.args[3], in, out),
-                                   resolve(s.args[4], in, out), resolve(s.args[2], in, out), bias, st), "gemm (sum of two products)");
+      const void* addend = s.addend.kind == BufRef::None ? nullptr : resolve(s.addend, in, out);
+      if (s.dual || addend) {
+        mi355_gemm_desc d2;
+        if (s.dual) d2 = toAbi(s.gemm2);
+        check(mi355_gemm_small_sum(&d, resolve(s.args[0], in, out), resolve(s.args[1], in, out), s.dual ? &d2 : nullptr,
+                                   s.dual ? resolve(s.args[3], in, out) : nullptr, s.dual ? resolve(s.args[4], in, out) : nullptr,
+                                   resolve(s.args[2], in, out), bias, addend, st), "gemm (small products summed)");
         break;
       }
       void* ws = s.args.size() > 3 ? resolve(s.args[3], in, out) : nullptr;
@@ -476,7 +479,7 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
       const int n = (int)s.parts.size();
       mi355_gemm_desc d1[4], d2[4];
       const mi355_gemm_desc *p1[4], *p2[4];
-      const void *a1[4], *b1[4], *a2[4], *b2[4], *bias[4];
+      const void *a1[4], *b1[4], *a2[4], *b2[4], *bias[4], *addend[4];
       void* c[4];
       if (n > 4) throw RuntimeError("gemm group of more than 4 products");
       for (int i = 0; i < n; ++i) {
@@ -492,8 +495,9 @@ void Executable::runStep(const Step& s, const std::vector<DeviceBuffer*>& in, co
           p2[i] = nullptr; a2[i] = nullptr; b2[i] = nullptr;
         }
         bias[i] = part.bias.kind == BufRef::None ? nullptr : resolve(part.bias, in, out);
+        addend[i] = part.addend.kind == BufRef::None ? nullptr : resolve(part.addend, in, out);
       }
-      check(mi355_gemm_small_group(n, p1, a1, b1, p2, a2, b2, c, bias, st), "gemm group");
+      check(mi355_gemm_small_group(n, p1, a1, b1, p2, a2, b2, c, bias, addend, st), "gemm group");
       break;
     }
     case Step::Conv: {
@@ -688,8 +692,8 @@ void Executable::replayIterations(const Step& s, bool withCond, int64_t trip, co
       auto add = [&](const BufRef& b) { if (b.kind == BufRef::Param || b.kind == BufRef::Output) lgs.external.push_back(b); };
       for (auto& st : p.steps) {
         for (auto& a : st.args) add(a);
-        for (auto& part : st.parts) { for (auto& a : part.args) add(a); add(part.bias); }
-        add(st.src); add(st.dst); add(st.predBuf); add(st.bias);
+        for (auto& part : st.parts) { for (auto& a : part.args) add(a); add(part.bias); add(part.addend); }
+        add(st.src); add(st.dst); add(st.predBuf); add(st.bias); add(st.addend);
         if (st.cond) scan(*st.cond);
         for (auto& b : st.bodies) scan(*b);
       }

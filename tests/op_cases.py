@@ -709,6 +709,111 @@ case("while-carry-new-value-read-after-producer", lambda b, x, w: _loop(b, [x, b
 case("while-carry-broadcast-row-of-itself", lambda b, x: _loop(b, [x], lambda i, p: [b.add(p, b.broadcast_in_dim(b.reshape(b.slice(p, [0, 0], [1, 16]), (16,)), (4, 16), [1]))]), f32(2310, 4, 16, lo=-0.1, hi=0.1))
 
 
+# products of a loop-invariant operand with the counter-selected slice of a loop-invariant tensor are taken over the whole tensor
+# ahead of the loop (one large product instead of one small one per iteration); the body reads slice i of the result, and slices of
+# tensors the loop never writes are addressed by the host.  Reference: the scan path of ops/control_flow.cc:702-989.
+def _rnn(b, xs, w, u, index=lambda b, i, T: i, trips=None, carry_xs=False, axis=0):
+    T = xs.shape[axis]
+    rest = [d for k, d in enumerate(xs.shape) if k != axis]
+    h0 = b.constant(0.0, xs.dtype, (rest[0], u.shape[0]))
+    zero = b.constant(0, "i32")
+
+    def step(i, h, seq):
+        starts = [zero] * xs.ndim
+        starts[axis] = index(b, i, T)
+        sizes = list(xs.shape)
+        sizes[axis] = 1
+        x_t = b.reshape(b.dynamic_slice(seq, starts, sizes), rest)
+        return b.tanh(b.add(b.matmul(x_t, w), b.matmul(h, u)))
+    n = trips if trips is not None else T
+    if carry_xs:   # the sequence travels as a carry that the body hands on unchanged, as jax.lax.scan passes its constants
+        r = b.while_loop([zero, h0, xs], lambda i, h, q: b.compare(i, n, "LT"), lambda i, h, q: [b.add(i, 1), step(i, h, q), q])
+    else:
+        r = b.while_loop([zero, h0], lambda i, h: b.compare(i, n, "LT"), lambda i, h: [b.add(i, 1), step(i, h, xs)])
+    return r[1]
+
+
+_RNN = (f32(2500, 12, 6, 20, lo=-1, hi=1), f32(2501, 20, 16, lo=-0.4, hi=0.4), f32(2502, 16, 16, lo=-0.4, hi=0.4))
+case("while-hoist-product-of-sequence-slice", lambda b, xs, w, u: _rnn(b, xs, w, u), *_RNN)
+case("while-hoist-reversed-index", lambda b, xs, w, u: _rnn(b, xs, w, u, index=lambda b, i, T: b.sub(b.constant(T - 1, "i32"), i)), *_RNN)
+case("while-hoist-index-clamped-at-the-end", lambda b, xs, w, u: _rnn(b, xs, w, u, index=lambda b, i, T: b.add(i, 3)), *_RNN)
+case("while-hoist-sequence-carried-unchanged", lambda b, xs, w, u: _rnn(b, xs, w, u, carry_xs=True), *_RNN)
+case("while-hoist-slice-of-a-middle-dim", lambda b, xs, w, u: _rnn(b, xs, w, u, axis=1), f32(2503, 6, 12, 20, lo=-1, hi=1), _RNN[1], _RNN[2])
+case("while-short-loop-over-long-sequence-keeps-its-products", lambda b, xs, w, u: _rnn(b, xs, w, u, trips=3), *_RNN)
+case("while-hoist-bf16", lambda b, xs, w, u: _rnn(b, xs, w, u), *_RNN, dtypes=["bf16", "bf16", "bf16"])
+
+
+def _rnn_rhs_slice(b, xs, w, u):
+    # the sliced operand on the right: h' = tanh(W . x_t + U . h) with column-major states
+    T, n_in, batch = xs.shape
+    zero = b.constant(0, "i32")
+
+    def body(i, h):
+        x_t = b.reshape(b.dynamic_slice(xs, [i, zero, zero], [1, n_in, batch]), (n_in, batch))
+        return [b.add(i, 1), b.tanh(b.add(b.matmul(w, x_t), b.matmul(u, h)))]
+    return b.while_loop([zero, b.zeros((u.shape[0], batch))], lambda i, h: b.compare(i, T, "LT"), body)[1]
+
+
+# (here the selected dim and the batch dim are apart in memory, so the products stay in the loop)
+case("while-slice-is-the-right-operand-free-dims-apart", _rnn_rhs_slice, f32(2504, 9, 20, 6, lo=-1, hi=1), f32(2505, 16, 20, lo=-0.4, hi=0.4), f32(2506, 16, 16, lo=-0.4, hi=0.4))
+
+
+def _rnn_rhs_rows(b, xs, w, u):
+    # the sliced operand on the right with its free dims side by side: h' = tanh(W . x_t^T + U . h), x_t one [batch, n_in] block
+    T, batch, n_in = xs.shape
+    zero = b.constant(0, "i32")
+
+    def body(i, h):
+        x_t = b.reshape(b.dynamic_slice(xs, [i, zero, zero], [1, batch, n_in]), (batch, n_in))
+        return [b.add(i, 1), b.tanh(b.add(b.dot_general(w, x_t, ([1], [1])), b.matmul(u, h)))]
+    return b.while_loop([zero, b.zeros((u.shape[0], batch))], lambda i, h: b.compare(i, T, "LT"), body)[1]
+
+
+case("while-hoist-slice-is-the-right-operand", _rnn_rhs_rows, f32(2508, 9, 6, 20, lo=-1, hi=1), f32(2505, 16, 20, lo=-0.4, hi=0.4), f32(2506, 16, 16, lo=-0.4, hi=0.4))
+
+
+def _two_loops_one_product(b, xs, w, u):
+    # a forward loop that stacks its states and a backward loop that recomputes x_t . W: both read one whole product
+    T, batch, n_in = xs.shape
+    n = u.shape[0]
+    zero = b.constant(0, "i32")
+
+    def fwd(i, h, hs):
+        x_t = b.reshape(b.dynamic_slice(xs, [i, zero, zero], [1, batch, n_in]), (batch, n_in))
+        h2 = b.tanh(b.add(b.matmul(x_t, w), b.matmul(h, u)))
+        return [b.add(i, 1), h2, b.dynamic_update_slice(hs, b.reshape(h, (1, batch, n)), [i, zero, zero])]
+    f = b.while_loop([zero, b.zeros((batch, n)), b.zeros((T, batch, n))], lambda i, h, hs: b.compare(i, T, "LT"), fwd)
+    hs = f[2]
+
+    def bwd(i, g, gw, gu):
+        t = b.sub(b.constant(T - 1, "i32"), i)
+        x_t = b.reshape(b.dynamic_slice(xs, [t, zero, zero], [1, batch, n_in]), (batch, n_in))
+        h_t = b.reshape(b.dynamic_slice(hs, [t, zero, zero], [1, batch, n]), (batch, n))
+        y = b.tanh(b.add(b.matmul(x_t, w), b.matmul(h_t, u)))
+        gz = b.mul(g, b.sub(1.0, b.mul(y, y)))
+        return [b.add(i, 1), b.dot_general(gz, u, ([1], [1])), b.add(gw, b.dot_general(x_t, gz, ([0], [0]))), b.add(gu, b.dot_general(h_t, gz, ([0], [0])))]
+    r = b.while_loop([zero, f[1], b.zeros(w.shape), b.zeros(u.shape)], lambda i, g, gw, gu: b.compare(i, T, "LT"), bwd)
+    return [f[1], r[1], r[2], r[3]]
+
+
+case("while-hoist-two-loops-share-the-whole-product", _two_loops_one_product, *_RNN)
+
+
+def _slices_named_by_the_host(b, xs):
+    # xs[i] read elementwise, and a two-row block at 2 * i: contiguous blocks of a tensor the loop never writes
+    T, n = xs.shape
+    zero = b.constant(0, "i32")
+
+    def body(i, acc):
+        row = b.reshape(b.dynamic_slice(xs, [i, zero], [1, n]), (n,))
+        pair = b.dynamic_slice(xs, [b.mul(i, 2), zero], [2, n])
+        return [b.add(i, 1), b.add(b.mul(acc, 0.5), b.add(b.exp(row), b.reduce_sum(pair, [0])))]
+    return b.while_loop([zero, b.zeros((n,))], lambda i, acc: b.compare(i, T // 2, "LT"), body)[1]
+
+
+case("while-slices-of-an-invariant-tensor", _slices_named_by_the_host, f32(2507, 10, 48, lo=-1, hi=1))
+
+
 # a scatter inside a counted loop (its launches are replayed from a captured graph): splat operand written by the scatter, a very
 # long run, and the result accumulated into a carry
 def _scatter_in_loop(b, i, u):

@@ -126,6 +126,36 @@ def test_relu_rides_in_a_small_product_and_its_mask_reads_the_activation():
     assert r.stdout.count("+ bias + relu") == 1 and " 9 steps" in r.stdout
 
 
+def test_products_of_sequence_slices_leave_the_loop():
+    """x[i] . W inside a counted loop, x and W untouched by the loop, is one product over all of x ahead of the loop; two loops
+    that need the same whole product share it.  A loop far shorter than the sequence, or a sequence whose selected dim and
+    other free dims are apart in memory, keeps its products."""
+    r = plan(op_cases.get_case("while-hoist-product-of-sequence-slice").text, "--dump-plan")
+    ahead, body = r.stdout.split("while while trip 12")
+    assert "dot_general tensor<12x6x20xf32> x tensor<20x16xf32>" in ahead
+    assert "dot_general tensor<6x16xf32> x tensor<16x16xf32>" in body and "20x16" not in body
+    for name in ("while-hoist-reversed-index", "while-hoist-index-clamped-at-the-end", "while-hoist-sequence-carried-unchanged"):
+        r = plan(op_cases.get_case(name).text, "--dump-plan")
+        assert "dot_general tensor<12x6x20xf32> x tensor<20x16xf32>" in r.stdout.split("while while trip")[0], name
+    r = plan(op_cases.get_case("while-hoist-slice-of-a-middle-dim").text, "--dump-plan")
+    assert "dot_general tensor<6x12x20xf32> x tensor<20x16xf32>" in r.stdout.split("while while trip")[0]
+    r = plan(op_cases.get_case("while-hoist-slice-is-the-right-operand").text, "--dump-plan")
+    assert "dot_general tensor<16x20xf32> x tensor<9x6x20xf32>" in r.stdout.split("while while trip")[0]
+    r = plan(op_cases.get_case("while-hoist-two-loops-share-the-whole-product").text, "--dump-plan")
+    assert r.stdout.count("dot_general tensor<12x6x20xf32> x tensor<20x16xf32>") == 1 and r.stdout.count("tensor<12x6x16xf32> x tensor<16x16xf32>") == 1
+    assert r.stdout.count("+ tensor") == 2        # the two weight gradients are summed into their carries by the products themselves
+    for name in ("while-short-loop-over-long-sequence-keeps-its-products", "while-slice-is-the-right-operand-free-dims-apart"):
+        r = plan(op_cases.get_case(name).text, "--dump-plan")
+        assert "dot_general" not in r.stdout.split("while while trip")[0], name
+    r = plan(configs.ALL["lstm"]().text, "--dump-plan")
+    loops = r.stdout.split("while while trip 100")
+    assert len(loops) == 3
+    forward = loops[1].split("\ngemm ")[0]
+    assert forward.count("\n  gemm ") == 1 and forward.count("\n  kernel ") == 2        # (one of the two is the unused condition)
+    backward = loops[2].split("\nkernel ")[0]
+    assert backward.count("\n  gemm-group ") == 1 and backward.count("\n  gemm ") == 0 and backward.count("\n  kernel ") == 2
+
+
 def test_a_column_reduction_stores_the_value_it_reads_first():
     """A large elementwise value that has to exist in memory and is first read by a column reduction gets no kernel of its
     own: the reduction's pass over the data writes it.  A product that reads it earlier keeps the separate kernel."""
