@@ -64,6 +64,7 @@ class Planner {
   void run() {
     Func* main = P.module->main();
     Region& body = main->body;
+    ivArgs().clear();
     rebuildUses(body);
     for (auto& a : body.args) {
       P.paramTypes.push_back(a->type);
@@ -2382,6 +2383,7 @@ class Planner {
     int tEnd = ++time_;
     for (size_t i = 0; i < n; ++i) ref(slots[i], tEnd);
     --loopDepth_;
+    if (hostCounter) ivArgs().erase(body.args[ivCarry].get());   // the registry outlives this compile: nothing stale may stay in it
     if (onDevice) {
       w.flagBuf = ref(aliveSid, tEnd);
       aliveFlags_.pop_back();
