@@ -322,6 +322,74 @@ void hoistIn(Region& r, int& nextId, std::vector<WholeProduct>& made) {
 
 }  // namespace
 
+// ---- updates masked by their own index check ---------------------------------------------------------------
+// JAX's x.at[i].add(u) zeroes the update rows whose index is out of range, select(in_range(i), u, 0), before a scatter
+// that ignores exactly those rows anyway (out-of-range scatter indices are dropped by definition).  For a whole-row
+// scatter along dim 0 whose indices are that same i, the select changes nothing the scatter reads: it takes u
+// itself, and the pass over the updates that only rewrote them is gone.
+namespace {
+
+bool isRowMaskOfIndex(Value* mask, Value* index, int64_t rows, int updRank) {
+  Op* bc = mask->def;
+  if (!bc || bc->name != "broadcast_in_dim" || (int)mask->type.rank() != updRank) return false;
+  Value* p = bc->operands[0];
+  const auto& dims = bc->ints("dims");
+  if (p->type.rank() != 1 || dims != std::vector<int64_t>{0} || p->type.dims[0] != index->type.dims[0]) return false;
+  Op* both = p->def;
+  if (!both || both->name != "and") return false;
+  bool lower = false, upper = false;
+  for (Value* side : both->operands) {
+    Op* c = side->def;
+    if (!c || c->name != "compare" || !isSignedInt(c->operands[0]->type.dt)) return false;
+    const std::string& dir = c->str("direction");
+    int64_t k;
+    if (c->operands[0] == index && constantInt(c->operands[1], k)) {
+      if (dir == "GE" && k <= 0) lower = true;                                   // holds for every index >= 0
+      else if (dir == "GT" && k < 0) lower = true;
+      else if ((dir == "LE" && k >= rows - 1) || (dir == "LT" && k >= rows)) upper = true;   // holds for every index < rows
+      else return false;
+    } else if (c->operands[1] == index && constantInt(c->operands[0], k)) {
+      if (dir == "LE" && k <= 0) lower = true;
+      else if (dir == "LT" && k < 0) lower = true;
+      else if ((dir == "GE" && k >= rows - 1) || (dir == "GT" && k >= rows)) upper = true;
+      else return false;
+    } else {
+      return false;
+    }
+  }
+  return lower && upper;
+}
+
+void dropMasksIn(Region& r) {
+  for (auto& op : r.ops) {
+    for (auto& sub : op->regions) dropMasksIn(*sub);
+    if (op->name != "scatter" || op->operands.size() != 3) continue;
+    Value* operand = op->operands[0];
+    Value* idx = op->operands[1];
+    Value* upd = op->operands[2];
+    if (operand->type.rank() < 1 || op->ints("inserted_window_dims") != std::vector<int64_t>{0} ||
+        op->ints("scatter_dims_to_operand_dims") != std::vector<int64_t>{0} || !op->ints("input_batching_dims").empty())
+      continue;
+    // one scatter dim in front: updates [n, row...], indices [n] or [n, 1]
+    if (upd->type.rank() != operand->type.rank() || idx->type.numel() != upd->type.dims[0]) continue;
+    Value* index = idx;
+    if (index->def && index->def->name == "reshape") index = index->def->operands[0];
+    if (index->type.rank() != 1 || !isSignedInt(index->type.dt)) continue;
+    Op* sel = upd->def;
+    if (!sel || sel->name != "select" || sel->operands.size() != 3) continue;
+    if (!isRowMaskOfIndex(sel->operands[0], index, operand->type.dims[0], upd->type.rank())) continue;
+    if (!(sel->operands[1]->type == upd->type)) continue;
+    op->operands[2] = sel->operands[1];
+  }
+}
+
+}  // namespace
+
+void dropScatterIndexMasks(Module& m) {
+  if (getenv("MI355X_SCATTER_MASKS") && atoi(getenv("MI355X_SCATTER_MASKS")) != 0) return;   // 1 keeps the masks
+  if (Func* f = m.main()) dropMasksIn(f->body);
+}
+
 void hoistLoopProducts(Module& m) {
   if (getenv("MI355X_HOIST_PRODUCTS") && atoi(getenv("MI355X_HOIST_PRODUCTS")) == 0) return;
   Func* f = m.main();

@@ -170,5 +170,8 @@ int64_t staticTripCount(Op* whileOp, LoopCounter* counter = nullptr);
 // inside counted loops, a product of a loop-invariant operand with the counter-selected slice of a loop-invariant tensor
 // becomes one product over the whole tensor ahead of the loop, and the body slices its result
 void hoistLoopProducts(Module& m);
+// updates = select(index in range, u, 0) ahead of a whole-row scatter with that index: the scatter reads u (rows out of
+// range are dropped by the scatter itself)
+void dropScatterIndexMasks(Module& m);
 
 }  // namespace mi355

@@ -2827,6 +2827,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   lowerRng(*module);
   lowerTopK(*module);
   hoistLoopProducts(*module);
+  dropScatterIndexMasks(*module);
   reluMasksFromActivations(*module);
   checkSupported(*module);
   eliminateDeadCode(module->main()->body);

@@ -247,6 +247,28 @@ case("scatter-add-row-numbers-of-8-bits-int64-indices", _row_scatter("add"), f32
 case("scatter-add-more-updates-than-one-workgroup-sorts", _row_scatter("add"), f32(2620, 50, 10),
      np.where(rng(2621).random(9000) < 0.3, 7, rng(2622).integers(0, 50, size=9000)).astype(np.int32), f32(2623, 9000, 10), exact=True)
 
+# x.at[i].add(u) as JAX lowers it: negative indices wrapped, updates of out-of-range rows selected to zero, then a scatter that drops those
+# rows anyway.  The select is not computed (the scatter reads u); a mask that is not the scatter's own range check stays.
+def _masked_scatter(lo_bound=0, hi_slack=0, other_index=False, body="add"):
+    def f(b, x, i, u, *more):
+        rows = x.shape[0]
+        wrapped = b.select(b.compare(i, 0, "LT"), b.add(i, rows), i)
+        checked = more[0] if other_index else wrapped
+        ok = b.and_(b.compare(checked, lo_bound, "GE"), b.compare(checked, rows - 1 + hi_slack, "LE"))
+        mask = b.broadcast_in_dim(ok, u.shape, [0])
+        masked = b.select(mask, u, b.zeros(u.shape))
+        return b.scatter(x, b.reshape(wrapped, (i.shape[0], 1)), masked, update_window_dims=[1], inserted_window_dims=[0],
+                         scatter_dims_to_operand_dims=[0], index_vector_dim=1, body=body)
+    return f
+
+
+_MASKED = (f32(2650, 12, 6), np.array([0, 11, -1, 12, 40, -12, -13, 5, 5, -30, 3], np.int32), f32(2651, 11, 6))
+case("scatter-add-updates-masked-by-the-range-check", _masked_scatter(), *_MASKED, exact=True)
+case("scatter-add-updates-masked-by-a-narrower-check", _masked_scatter(lo_bound=2), *_MASKED, exact=True)
+case("scatter-add-updates-masked-by-another-index", _masked_scatter(other_index=True), *_MASKED, np.array([0, 1, 2, 3, 4, 5, 60, 7, -8, 9, 10], np.int32), exact=True)
+case("scatter-max-updates-masked-by-the-range-check", _masked_scatter(body="max"), *_MASKED, exact=True)
+
+
 # the operand is a splat constant (zeros a gradient is scattered into): the scatter writes it itself, in the launch that sorts
 def _scatter_into(value, rows, cols, dtype="f32", body="add"):
     def f(b, i, u):

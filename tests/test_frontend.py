@@ -156,6 +156,19 @@ def test_products_of_sequence_slices_leave_the_loop():
     assert backward.count("\n  gemm-group ") == 1 and backward.count("\n  gemm ") == 0 and backward.count("\n  kernel ") == 2
 
 
+def test_updates_masked_by_the_scatter_s_own_range_check_are_read_unmasked():
+    """select(index in range, u, 0) ahead of a whole-row scatter with that index only rewrites rows the scatter drops anyway:
+    no kernel computes it.  A narrower check, or a check of another index, changes rows the scatter keeps and stays."""
+    for name in ("scatter-add-updates-masked-by-the-range-check", "scatter-max-updates-masked-by-the-range-check"):
+        r = plan(op_cases.get_case(name).text, "--dump-plan")
+        assert r.returncode == 0 and "fusion:select" not in r.stdout, name
+    for name in ("scatter-add-updates-masked-by-a-narrower-check", "scatter-add-updates-masked-by-another-index"):
+        r = plan(op_cases.get_case(name).text, "--dump-plan")
+        assert r.returncode == 0 and "fusion:select" in r.stdout, name
+    r = plan(configs.ALL["embedding"]().text, "--dump-plan")
+    assert " 2 steps" in r.stdout and "arena 0.22 MiB" in r.stdout        # the masked copy of the 25 MB of updates is gone
+
+
 def test_a_column_reduction_stores_the_value_it_reads_first():
     """A large elementwise value that has to exist in memory and is first read by a column reduction gets no kernel of its
     own: the reduction's pass over the data writes it.  A product that reads it earlier keeps the separate kernel."""
