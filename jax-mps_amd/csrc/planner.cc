@@ -596,8 +596,9 @@ class Planner {
     static const bool on = !getenv("MI355X_REDUCE_STORES") || atoi(getenv("MI355X_REDUCE_STORES")) != 0;
     Value* v = op->result();
     // (a reduction over a small input is one launch of a few workgroups: too few to also compute and store the value)
-    // (inside a loop body the launch saved is worth more than the workgroups, provided the one pass still has a few dozen)
-    const bool sized = loopDepth_ > 0 ? v->type.numel() >= 16384 && v->type.numel() <= reduceOnePassLimit() : v->type.numel() > reduceOnePassLimit();
+    // (a one-pass reduction over a small input still has a few dozen workgroups, see the column tiles in codegen.cc, and the
+    // launch saved is worth more than they are; below 16 384 elements the value is cheaper to recompute than to wait for)
+    const bool sized = v->type.numel() >= 16384;
     if (!on || !sized || !takesKernel(op) || op->name == "constant" || op->has("force_materialize")) return false;
     if (v->type.dt != DType::F32 && v->type.dt != DType::BF16) return false;
     Op* red = nullptr;

@@ -627,7 +627,8 @@ def _masked_grad_sums(b, x, dy, kept=(3,), also_return=False):
     dx = b.sub(b.sub(g, b.broadcast_in_dim(b.div(s1, n), x.shape, list(kept))), b.mul(x, b.broadcast_in_dim(b.div(s2, n), x.shape, list(kept))))
     return [dx, g] if also_return else dx
 case("reduce-column-stores-its-input-two-passes", _masked_grad_sums, f32(2750, 32, 16, 32, 32, lo=-1, hi=1), f32(2751, 32, 16, 32, 32, lo=-1, hi=1))
-case("reduce-column-small-input-keeps-its-own-kernel", lambda b, x, dy: _masked_grad_sums(b, x, dy, kept=(1,)), f32(2752, 128, 512, lo=-1, hi=1), f32(2753, 128, 512, lo=-1, hi=1))
+case("reduce-column-small-input-stored-by-one-pass", lambda b, x, dy: _masked_grad_sums(b, x, dy, kept=(1,)), f32(2752, 128, 512, lo=-1, hi=1), f32(2753, 128, 512, lo=-1, hi=1))
+case("reduce-column-tiny-input-keeps-its-own-kernel", lambda b, x, dy: _masked_grad_sums(b, x, dy, kept=(1,)), f32(2761, 24, 96, lo=-1, hi=1), f32(2762, 24, 96, lo=-1, hi=1))
 case("reduce-column-stores-its-input-bf16", _masked_grad_sums, f32(2754, 16, 16, 32, 64, lo=-1, hi=1), f32(2755, 16, 16, 32, 64, lo=-1, hi=1), dtypes=["bf16", "bf16"])
 case("reduce-column-stores-its-input-also-a-result", lambda b, x, dy: _masked_grad_sums(b, x, dy, also_return=True),
      f32(2756, 32, 16, 16, 64, lo=-1, hi=1), f32(2757, 32, 16, 16, 64, lo=-1, hi=1))
