@@ -2491,7 +2491,8 @@ class Planner {
   // the kernel that computes the new state).
   void sinkKernelsInLoops(Plan& plan, bool inLoop) {
     for (auto& s : plan.steps) for (auto& b : s.bodies) sinkKernelsInLoops(*b, s.kind == Step::While);
-    if (!inLoop) return;
+    static const bool everywhere = !getenv("MI355X_SINK_TOP_LEVEL") || atoi(getenv("MI355X_SINK_TOP_LEVEL")) != 0;
+    if (!inLoop && !(everywhere && &plan == &P.plan)) return;
     auto& steps = plan.steps;
     for (int i = (int)steps.size() - 2; i >= 0; --i) {
       if (!batchCandidate(steps[(size_t)i]) || steps[(size_t)i + 1].kind == Step::Kernel) continue;

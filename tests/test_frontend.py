@@ -123,7 +123,7 @@ def test_relu_rides_in_a_small_product_and_its_mask_reads_the_activation():
     r = plan(op_cases.get_case("dot-relu-f32-igemm-not-small").text, "--dump-plan")
     assert "+ relu" not in r.stdout
     r = plan(configs.ALL["mlp"]().text, "--dump-plan")
-    assert r.stdout.count("+ bias + relu") == 1 and " 8 steps" in r.stdout
+    assert r.stdout.count("+ bias + relu") == 1 and " 7 steps" in r.stdout
 
 
 def test_products_of_sequence_slices_leave_the_loop():
