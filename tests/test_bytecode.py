@@ -25,6 +25,7 @@ CASES = ["binary-add", "compare-f32-LT", "compare-totalorder", "select", "conver
          "while-swapped-carries", "maxpool-3x3-s2-pad1", "maxpool-grad-ties", "round-half", "unary-specials", "bool-logic",
          "all-reduce-one-device-pmean", "all-reduce-one-device-two-operands", "partition-id-axis-index-zero",
          "token-created-merged-and-returned", "token-argument-returned-as-is", "token-carried-by-a-loop",
+         "while-hoist-two-loops-share-the-whole-product", "scatter-add-updates-masked-by-the-range-check",
          # custom calls whose JSON backend_config (quotes inside a string attribute) must survive
          "fused-sdpa-padding-mask-f32", "fused-rope-partial-traditional-f32", "fused-layer-norm-bwd-f32"]
 
