@@ -267,6 +267,7 @@ case("scatter-add-updates-masked-by-the-range-check", _masked_scatter(), *_MASKE
 case("scatter-add-updates-masked-by-a-narrower-check", _masked_scatter(lo_bound=2), *_MASKED, exact=True)
 case("scatter-add-updates-masked-by-another-index", _masked_scatter(other_index=True), *_MASKED, np.array([0, 1, 2, 3, 4, 5, 60, 7, -8, 9, 10], np.int32), exact=True)
 case("scatter-max-updates-masked-by-the-range-check", _masked_scatter(body="max"), *_MASKED, exact=True)
+case("scatter-add-updates-masked-int64-indices", _masked_scatter(), _MASKED[0], _MASKED[1].astype(np.int64), _MASKED[2], exact=True)
 
 
 # the operand is a splat constant (zeros a gradient is scattered into): the scatter writes it itself, in the launch that sorts
@@ -820,6 +821,23 @@ def _two_loops_one_product(b, xs, w, u):
 
 
 case("while-hoist-two-loops-share-the-whole-product", _two_loops_one_product, *_RNN)
+
+
+def _slice_of_a_changing_carry(b, buf, w):
+    # the sliced tensor is a carry that the body rewrites (row i + 1 from row i): neither the product nor the slice may leave the loop
+    T, n = buf.shape
+    zero = b.constant(0, "i32")
+
+    def body(i, cur, acc):
+        row = b.reshape(b.dynamic_slice(cur, [i, zero], [1, n]), (1, n))
+        y = b.tanh(b.matmul(row, w))
+        nxt = b.dynamic_update_slice(cur, b.add(y, b.reshape(b.dynamic_slice(cur, [b.add(i, 1), zero], [1, n]), (1, n))), [b.add(i, 1), zero])
+        return [b.add(i, 1), nxt, b.add(acc, y)]
+    r = b.while_loop([zero, buf, b.zeros((1, n))], lambda i, c, a: b.compare(i, T - 1, "LT"), body)
+    return [r[1], r[2]]
+
+
+case("while-slice-of-a-carry-the-body-rewrites", _slice_of_a_changing_carry, f32(2509, 9, 24, lo=-1, hi=1), f32(2510, 24, 24, lo=-0.3, hi=0.3))
 
 
 def _slices_named_by_the_host(b, xs):
