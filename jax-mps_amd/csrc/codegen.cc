@@ -191,7 +191,7 @@ struct Index {
 
 class Emitter {
  public:
-  Emitter(const LeafPredicate& isLeaf, int V, bool idx64) : isLeaf_(isLeaf), V_(V), idx64_(idx64) {
+  Emitter(const LeafPredicate& isLeaf, int V, bool idx64) : V_(V), idx64_(idx64), isLeaf_(isLeaf) {
     body_.emplace_back();
     cache_.emplace_back();
   }
