@@ -306,6 +306,12 @@ class Planner {
       }
     }
     // reverse: materialisation decisions
+    // contexts[v]: at how many different positions one generated kernel would evaluate v.  An elementwise reader evaluates
+    // its operand where it is evaluated itself (and the generator computes a value once per position), a reader that moves
+    // data (reverse, slice, pad, gather ...) at a position of its own.  A chain of such readers doubles the count at
+    // every link (v + reverse(v), forty times over, is 2^40 copies of the first value): beyond a few dozen the value
+    // is stored instead.
+    std::unordered_map<Value*, int64_t> contexts;
     std::unordered_map<Value*, std::vector<Op*>> groups;
     for (int k = (int)r.ops.size() - 1; k >= 0; --k) {
       Op* op = r.ops[k].get();
@@ -328,6 +334,22 @@ class Planner {
         auto& d = *op->attrs.at("value").dense;
         if (!d.splat && d.type.numel() > 1) mat = true;
       }
+      int64_t positions = 1;
+      {
+        int64_t same = 0, moved = 0;
+        for (Op* u : v->users) {
+          if (u->parent != &r || !isFusibleOp(*u) || u->results.size() != 1) continue;
+          auto it = contexts.find(u->result());
+          const int64_t cu = it == contexts.end() ? 1 : it->second;
+          if (sameShapeElementwise(*u)) same = std::max(same, cu);
+          else moved += cu;
+        }
+        positions = std::max<int64_t>(1, same + moved);
+        if (positions > 32 && op->name != "constant" && op->name != "iota" && v->type.numel() > 1) {
+          mat = true;
+          op->attrs["force_materialize"] = Attr();   // and no kernel that stores it may also compute its readers
+        }
+      }
       if (!mat && v->type.numel() > (loopDepth_ > 0 ? kLoopSmallNumel : kSmallNumel) && g.size() >= 2) {
         int big = 0;
         for (auto* l : leaves[v]) if (l->type.numel() * 4 >= v->type.numel()) ++big;
@@ -337,6 +359,7 @@ class Planner {
         static const int limit = getenv("MI355X_RECOMPUTE_LIMIT") ? atoi(getenv("MI355X_RECOMPUTE_LIMIT")) : 1;
         if ((big >= 2 && ((int)g.size() - 1) * (big - 1) > limit) || expensive) mat = true;
       }
+      contexts[v] = mat ? 1 : positions;
       needMat_[v] = mat;
       // A small value that a scatter, gather or the like needs in memory, a few integer or select ops away from
       // buffers that exist anyway (normalised indices, say): the kernels that also read it recompute it, so they do

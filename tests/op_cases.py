@@ -247,6 +247,22 @@ case("scatter-add-row-numbers-of-8-bits-int64-indices", _row_scatter("add"), f32
 case("scatter-add-more-updates-than-one-workgroup-sorts", _row_scatter("add"), f32(2620, 50, 10),
      np.where(rng(2621).random(9000) < 0.3, 7, rng(2622).integers(0, 50, size=9000)).astype(np.int32), f32(2623, 9000, 10), exact=True)
 
+# a chain whose every link reads its input at two positions (v + reverse(v)): fused naively, link n evaluates the first value at 2^n
+# positions; values evaluated at more than a few dozen positions are stored instead
+def _mirrored_chain(links):
+    def f(b, x):
+        v = x
+        for _ in range(links):
+            t = b.tanh(v)
+            v = b.mul(b.add(t, b.reverse(t, [0])), 0.5)
+        return v
+    return f
+
+
+case("elementwise-chain-read-at-mirrored-positions-12-links", _mirrored_chain(12), f32(2800, 6, 40, lo=-1, hi=1))
+case("elementwise-chain-read-at-mirrored-positions-40-links", _mirrored_chain(40), f32(2801, 6, 40, lo=-1, hi=1))
+
+
 # x.at[i].add(u) as JAX lowers it: negative indices wrapped, updates of out-of-range rows selected to zero, then a scatter that drops those
 # rows anyway.  The select is not computed (the scatter reads u); a mask that is not the scatter's own range check stays.
 def _masked_scatter(lo_bound=0, hi_slack=0, other_index=False, body="add"):

@@ -169,6 +169,17 @@ def test_updates_masked_by_the_scatter_s_own_range_check_are_read_unmasked():
     assert " 2 steps" in r.stdout and "arena 0.22 MiB" in r.stdout        # the masked copy of the 25 MB of updates is gone
 
 
+def test_a_value_read_at_ever_more_positions_is_stored():
+    """v + reverse(v), forty times over, would be one kernel evaluating the first value at 2^40 positions; the planner stores a
+    value once a kernel would evaluate it at more than 32 positions, so the program compiles at once into a handful of kernels."""
+    import time
+    t0 = time.time()
+    r = plan(op_cases.get_case("elementwise-chain-read-at-mirrored-positions-40-links").text, "--dump-plan")
+    assert r.returncode == 0 and time.time() - t0 < 20
+    steps = int(r.stdout.rsplit("->", 1)[1].split("steps")[0])
+    assert 5 <= steps <= 12
+
+
 def test_a_column_reduction_stores_the_value_it_reads_first():
     """A large elementwise value that has to exist in memory and is first read by a column reduction gets no kernel of its
     own: the reduction's pass over the data writes it.  A product that reads it earlier keeps the separate kernel."""
