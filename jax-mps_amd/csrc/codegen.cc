@@ -449,6 +449,12 @@ class Emitter {
     return t;
   }
 
+  // What was declared inside a loop body that has been written out is out of scope for the code that follows it.
+  void forgetBodyValues() {
+    for (auto& c : cache_)
+      for (auto it = c.begin(); it != c.end();) it = bodyNames_.count(it->second) ? c.erase(it) : std::next(it);
+  }
+
   // --------------------------------------------------------- value generation
   std::string gen(Value* v, const Index& idx) {
     std::string key = std::to_string(v->id) + "|" + idx.sig;
@@ -1252,13 +1258,16 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
       IdxDim klin;
       klin.isConst = false; klin.base = "kk"; klin.coef = 0; klin.mult = 1;
       em.pre_.clear();
+      const size_t bodyMark = em.body_.front().size();
       auto kd = em.delinearize(klin, keptShape);
       em.rowKept_ = kd;
       Index kidx = em.multiIndex(kd, keptShape);
       std::vector<std::string> ev;
       for (auto* v : epilogue) ev.push_back(em.gen(v, kidx));
-      s << em.pre_;
+      // (guarded reads, of a padded or concatenated operand say, are written as body statements whatever their index)
+      s << em.pre_ << "  { const int v = 0; (void)v;\n" << em.body_.front().substr(bodyMark);
       for (size_t q = 0; q < epilogue.size(); ++q) s << "  outE" << q << "[kk] = " << storeExpr(epilogue[q]->type.dt, ev[q]) << ";\n";
+      s << "  }\n";
     }
     s << "}\n";
     Launch l;
@@ -1400,14 +1409,17 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
       Index kidx = em.multiIndex(kd, keptShape);
       std::string savedPre2 = em.pre_;
       em.pre_.clear();
+      em.forgetBodyValues();
+      const size_t bodyMark = em.body_.front().size();
       std::vector<std::string> ev;
       for (auto* v : epilogue) ev.push_back(em.gen(v, kidx));
-      s << em.pre_;
+      s << em.pre_ << "  { const int v = 0; (void)v;\n" << em.body_.front().substr(bodyMark);
       em.pre_ = savedPre2;
       for (size_t q = 0; q < epilogue.size(); ++q) {
         s << "  outE" << q << "[kk] = " << storeExpr(epilogue[q]->type.dt, ev[q]) << ";\n";
         outs.push_back(storageT(epilogue[q]->type.dt) + "* __restrict__ outE" + std::to_string(q));
       }
+      s << "  }\n";
       header = kernelHeader(em.leaves_, outs);
       fc.epilogueFused = true;
     }
@@ -1552,12 +1564,14 @@ FusedCode generateReduceKernel(const std::vector<Op*>& reduces, const LeafPredic
     klin2.isConst = false; klin2.base = "kk"; klin2.coef = 0; klin2.mult = 1;
     const std::string keepPre = em.pre_;
     em.pre_.clear();
+    em.forgetBodyValues();
+    const size_t bodyMark = em.body_.front().size();
     auto kd2 = em.delinearize(klin2, keptShape);
     em.rowKept_ = kd2;
     Index kidx = em.multiIndex(kd2, keptShape);
     std::vector<std::string> ev;
     for (auto* v : epilogue) ev.push_back(em.gen(v, kidx));
-    s << em.pre_;
+    s << em.pre_ << em.body_.front().substr(bodyMark);
     em.pre_ = keepPre;
     for (size_t q = 0; q < epilogue.size(); ++q) {
       s << "    outE" << q << "[kk] = " << storeExpr(epilogue[q]->type.dt, ev[q]) << ";\n";

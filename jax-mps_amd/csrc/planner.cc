@@ -947,7 +947,14 @@ class Planner {
         if (!d || !isFusibleOp(*d) || d->results.size() != 1 || d->parent != &r || needMat_[v]) return false;
         if (!counted.insert(v).second) return true;   // a shared subexpression is generated once
         if (--budget < 0) return false;
-        for (auto* o : d->operands) if (!can(o, usesResult, budget)) return false;
+        // the lane that holds a finished result knows that one only: whatever stands between the result and the value
+        // must read it where it is evaluated itself (a slice, a reversal or a concatenation reads another output's)
+        for (auto* o : d->operands) {
+          bool below = false;
+          if (!can(o, below, budget)) return false;
+          if (below && (movesData(*d) || o->type.dims != v->type.dims)) return false;
+          usesResult |= below;
+        }
         return true;
       };
       size_t pos = 0;
@@ -961,7 +968,11 @@ class Planner {
         int budget = 64;
         bool ok = true;
         counted.clear();
-        for (auto* o : y->operands) if (!can(o, uses, budget)) ok = false;
+        for (auto* o : y->operands) {
+          bool below = false;
+          if (!can(o, below, budget) || (below && (movesData(*y) || o->type.dims != keptDims))) ok = false;
+          uses |= below;
+        }
         if (!ok || !uses) continue;
         epilogue.push_back(w);
         epilogueOps.push_back(y);
@@ -2099,10 +2110,13 @@ class Planner {
   // iteration.  The kernel that produces it may write the slot directly when nothing still needs the old carry:
   // no step after the producer reads the slot, and the producer itself reads it (if at all) element for element
   // at the position it writes (c' = f * c + i * g).
-  static bool sameShapeElementwise(const Op& op) {
+  static bool movesData(const Op& op) {
     static const std::set<std::string> moves = {"broadcast_in_dim", "reshape", "transpose", "slice", "dynamic_slice", "pad", "concatenate", "gather",
                                                 "reverse", "iota", "dynamic_update_slice", "bitcast_convert", "constant"};
-    if (!isFusibleOp(op) || op.results.size() != 1 || moves.count(op.name)) return false;
+    return moves.count(op.name) != 0;
+  }
+  static bool sameShapeElementwise(const Op& op) {
+    if (!isFusibleOp(op) || op.results.size() != 1 || movesData(op)) return false;
     for (auto* o : op.operands) if (o->type.dims != op.results[0]->type.dims) return false;
     return true;
   }

@@ -655,6 +655,20 @@ case("reduce-column-input-read-by-a-product-first", lambda b, x, dy, w: (lambda 
 # a reduction finished in one launch whose per-output values ride in the same launch
 case("reduce-then-scale-one-pass", lambda b, x: b.div(b.reduce_sum(x, [0]), 300.0), f32(2745, 300, lo=-1, hi=1))
 case("reduce-rows-then-scale-one-pass", lambda b, x, w: b.mul(b.reduce_sum(x, [1]), w), f32(2746, 70, 90, lo=-1, hi=1), f32(2747, 70))
+# readers of a finished reduction that take it from another position get no place in the pass that finishes it
+case("reduce-result-read-transposed", lambda b, x: b.transpose(b.reduce_sum(x, [1]), [1, 0]), f32(2763, 16, 2, 16, lo=-1, hi=1))
+case("reduce-result-read-through-slices-and-a-concatenation",
+     lambda b, x: (lambda s: b.concatenate([b.slice(s, [0, 0], [8, 8]), b.slice(b.exp(s), [0, 8], [8, 16])], 1))(b.reduce_sum(x, [1])),
+     f32(2764, 8, 2, 16, lo=-1, hi=1))
+case("reduce-result-read-reversed-and-in-place", lambda b, x: (lambda s: b.add(b.mul(s, 0.5), b.reverse(s, [0])))(b.reduce_max(x, [0])),
+     f32(2765, 40, 24, lo=-1, hi=1))
+# per-output values that read a padded or concatenated operand (a guarded read) next to the finished result
+case("reduce-column-one-pass-scaled-by-a-padded-vector", lambda b, x, w: b.mul(b.reduce_sum(x, [0]), b.pad(w, 1.5, [2], [2])),
+     f32(2766, 40, 24, lo=-1, hi=1), f32(2767, 20))
+case("reduce-rows-one-pass-scaled-by-a-concatenation", lambda b, x, u, w: b.mul(b.reduce_sum(x, [1]), b.concatenate([u, b.exp(w)], 0)),
+     f32(2768, 70, 90, lo=-1, hi=1), f32(2769, 30), f32(2770, 40))
+case("reduce-column-two-passes-scaled-by-a-padded-vector", lambda b, x, w: b.mul(b.reduce_sum(x, [0]), b.pad(w, -2.0, [4], [0])),
+     f32(2771, 16384, 64, lo=-1, hi=1), f32(2772, 60))
 case("argmax", lambda b, x: b.argmax(x, 1), f32(272, 9, 31), exact=True)
 case("argmax-leading-dim", lambda b, x: b.argmax(x, 0), f32(2720, 150, 7), exact=True)
 case("argmax-middle-dim-long", lambda b, x: b.argmax(x, 1), f32(2721, 3, 1000, 5), exact=True)
