@@ -49,14 +49,31 @@ template <typename I, typename F> __device__ __forceinline__ I f2i(F f) {
   else if (f <= (F)0) return (I)0;
   return (I)f;
 }
+// Integer arithmetic wraps (two's complement), for signed types as well: the 32- and 64-bit ones are computed on their
+// unsigned counterparts, where overflow is defined (narrower types are promoted to int by the language and wrap when
+// they are narrowed again).
+template <typename T> struct Uns { typedef T type; };
+template <> struct Uns<int> { typedef u32 type; };
+template <> struct Uns<i64> { typedef u64 type; };
+template <typename T> __device__ __forceinline__ T wadd(T a, T b) { typedef typename Uns<T>::type U; return (T)((U)a + (U)b); }
+template <typename T> __device__ __forceinline__ T wsub(T a, T b) { typedef typename Uns<T>::type U; return (T)((U)a - (U)b); }
+template <typename T> __device__ __forceinline__ T wmul(T a, T b) { typedef typename Uns<T>::type U; return (T)((U)a * (U)b); }
 template <typename T> __device__ __forceinline__ T ipow(T a, T b) {
   if (b < (T)0) return a == (T)1 ? (T)1 : (a == (T)-1 ? ((b & (T)1) ? (T)-1 : (T)1) : (T)0);
   T r = (T)1;
-  while (b) { if (b & (T)1) r *= a; a *= a; b >>= 1; }
+  while (b) { if (b & (T)1) r = wmul<T>(r, a); a = wmul<T>(a, a); b >>= 1; }
   return r;
 }
-template <typename T> __device__ __forceinline__ T idiv(T a, T b) { return b == (T)0 ? (T)-1 : ((b == (T)-1) ? (T)(0 - a) : (T)(a / b)); }
-template <typename T> __device__ __forceinline__ T irem(T a, T b) { return b == (T)0 ? a : ((b == (T)-1) ? (T)0 : (T)(a % b)); }
+// division by zero gives all ones, the most negative number divided by -1 itself (and remainder 0); an unsigned divisor
+// of all ones is an ordinary number
+template <typename T> __device__ __forceinline__ T idiv(T a, T b) {
+  const bool sg = (T)-1 < (T)0;
+  return b == (T)0 ? (T)-1 : ((sg && b == (T)-1) ? wsub<T>((T)0, a) : (T)(a / b));
+}
+template <typename T> __device__ __forceinline__ T irem(T a, T b) {
+  const bool sg = (T)-1 < (T)0;
+  return b == (T)0 ? a : ((sg && b == (T)-1) ? (T)0 : (T)(a % b));
+}
 // 16-bit results keep 8 (bf16) or 11 (f16) significand bits: the hardware exponential is exact enough there
 __device__ __forceinline__ float tanh_fast(float x) { float t = __expf(-2.f * fabsf(x)); return copysignf((1.f - t) * __builtin_amdgcn_rcpf(1.f + t), x); }
 // f32 tanh to a few ulp: odd polynomial near 0 (where 1 - exp cancels), exponential form elsewhere
@@ -756,9 +773,10 @@ class Emitter {
 
     // ---- binary arithmetic
     std::string T = computeT(rt.dt);
-    if (n == "add") return bin(isP ? "(" + in(0) + " || " + in(1) + ")" : "(" + in(0) + " + " + in(1) + ")");
-    if (n == "subtract") return bin("(" + in(0) + " - " + in(1) + ")");
-    if (n == "multiply") return bin(isP ? "(" + in(0) + " && " + in(1) + ")" : "(" + in(0) + " * " + in(1) + ")");
+    const bool wraps = rt.dt == DType::S32 || rt.dt == DType::S64;   // signed overflow has to wrap, not to be assumed away
+    if (n == "add") return bin(isP ? "(" + in(0) + " || " + in(1) + ")" : wraps ? "wadd<" + T + ">(" + in(0) + ", " + in(1) + ")" : "(" + in(0) + " + " + in(1) + ")");
+    if (n == "subtract") return bin(wraps ? "wsub<" + T + ">(" + in(0) + ", " + in(1) + ")" : "(" + in(0) + " - " + in(1) + ")");
+    if (n == "multiply") return bin(isP ? "(" + in(0) + " && " + in(1) + ")" : wraps ? "wmul<" + T + ">(" + in(0) + ", " + in(1) + ")" : "(" + in(0) + " * " + in(1) + ")");
     if (n == "divide") {
       // a divisor that is one number per row (softmax's sum) is inverted once per row, not once per element
       if (isF && !isD) {
@@ -787,8 +805,8 @@ class Emitter {
     }
 
     // ---- unary
-    if (n == "negate") return bin(isP ? in(0) : "(" + T + ")(-" + in(0) + ")");
-    if (n == "abs") return bin(isF ? "fabs" + sfx + "(" + in(0) + ")" : "(" + T + ")(" + in(0) + " < 0 ? -" + in(0) + " : " + in(0) + ")");
+    if (n == "negate") return bin(isP ? in(0) : wraps ? "wsub<" + T + ">((" + T + ")0, " + in(0) + ")" : "(" + T + ")(-" + in(0) + ")");
+    if (n == "abs") return bin(isF ? "fabs" + sfx + "(" + in(0) + ")" : wraps ? "(" + in(0) + " < 0 ? wsub<" + T + ">((" + T + ")0, " + in(0) + ") : " + in(0) + ")" : "(" + T + ")(" + in(0) + " < 0 ? -" + in(0) + " : " + in(0) + ")");
     if (n == "not") return bin(isP ? "(!" + in(0) + ")" : "(" + T + ")(~" + in(0) + ")");
     if (n == "sign") return bin(isF ? (isD ? "sgnd(" : "sgnf(") + in(0) + ")" : "(" + T + ")((" + in(0) + " > 0) - (" + in(0) + " < 0))");
     if (n == "is_finite") return bin("isfinite(" + in(0) + ")");
@@ -1091,8 +1109,9 @@ struct RedOp {
     std::string k = kind;
     bool p = dt == DType::Pred;
     std::string band = "(bool)((int)" + a + " & (int)" + b + ")", bor = "(bool)((int)" + a + " | (int)" + b + ")";
-    if (k == "add") return p ? bor : "(" + a + " + " + b + ")";
-    if (k == "multiply") return p ? band : "(" + a + " * " + b + ")";
+    const bool wraps = dt == DType::S32 || dt == DType::S64;
+    if (k == "add") return p ? bor : wraps ? "wadd<" + accT + ">(" + a + ", " + b + ")" : "(" + a + " + " + b + ")";
+    if (k == "multiply") return p ? band : wraps ? "wmul<" + accT + ">(" + a + ", " + b + ")" : "(" + a + " * " + b + ")";
     if (k == "maximum") return p ? bor : "mx<" + accT + ">(" + a + ", " + b + ")";
     if (k == "minimum") return p ? band : "mn<" + accT + ">(" + a + ", " + b + ")";
     if (k == "and") return p ? band : "(" + accT + ")(" + a + " & " + b + ")";

@@ -159,7 +159,7 @@ const char* mi355_rtc_fingerprint(void) {
   if (!buf[0]) {
     int major = 0, minor = 0;
     if (hiprtcVersion(&major, &minor) != HIPRTC_SUCCESS) major = minor = -1;
-    snprintf(buf, sizeof buf, "hiprtc-%d.%d -O3 -ffp-contract=off -packed-fp32-ops", major, minor);
+    snprintf(buf, sizeof buf, "hiprtc-%d.%d -O3 -ffp-contract=off -packed-fp32-ops wrapping-ints", major, minor);
   }
   return buf;
 }

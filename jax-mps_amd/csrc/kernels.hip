@@ -689,10 +689,10 @@ struct ScatterOps<float> {
 template <>
 struct ScatterOps<int> {
   static __device__ __forceinline__ int apply(int kind, int a, int u) {
-    switch (kind) {
-      case 0: return a + u;
+    switch (kind) {   // (sums and products wrap: computed on the unsigned type)
+      case 0: return (int)((u32)a + (u32)u);
       case 1: return u;
-      case 2: return a * u;
+      case 2: return (int)((u32)a * (u32)u);
       case 3: return a < u ? a : u;
       default: return a > u ? a : u;
     }

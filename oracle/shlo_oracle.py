@@ -1179,8 +1179,11 @@ class Oracle:
             if a.dtype.kind == "u":
                 q = a // bz
                 return np.where(b == 0, np.iinfo(a.dtype).max, q).astype(a.dtype)
-            q = np.abs(a.astype(np.int64)) // np.abs(bz.astype(np.int64))
-            q = np.where((a < 0) != (b < 0), -q, q)
+            # magnitudes as unsigned 64-bit numbers (the most negative value has no signed magnitude), the sign put
+            # back in wrapping arithmetic: the most negative value divided by -1 is itself
+            mag = lambda v: np.where(v < 0, ~v.astype(np.int64).astype(np.uint64) + np.uint64(1), v.astype(np.int64).astype(np.uint64))
+            q = mag(a) // mag(bz)
+            q = np.where((a < 0) != (b < 0), ~q + np.uint64(1), q).astype(np.int64)
             return np.where(b == 0, -1, q).astype(a.dtype)
 
     def op_remainder(self, op, ins, env):

@@ -112,6 +112,22 @@ for d in ["EQ", "NE", "LT", "LE", "GT", "GE"]:
     case("compare-f32-" + d, (lambda dd: lambda b, x, y: b.compare(x, y, dd))(d),
          np.array([1.0, 2.0, 2.0, np.nan, -0.0, np.inf], np.float32), np.array([2.0, 2.0, 1.0, 1.0, 0.0, np.inf], np.float32), exact=True)
 case("compare-i32", lambda b, x, y: [b.compare(x, y, "LT"), b.compare(x, y, "GE")], i32(90, 40, lo=-3, hi=3), i32(91, 40, lo=-3, hi=3), exact=True)
+# integer arithmetic wraps, for signed types too, and nothing downstream may be simplified as if it could not: the square of
+# a 32-bit number can be negative, x - y can exceed x, x + 1 can be below x
+_I32_WIDE = np.array([1790545064, -1206374848, 46341, -46341, 2**31 - 1, -2**31, 65536, 3, 0, -1], np.int32)
+_I64_WIDE = np.array([-6927189342267442211, 2**63 - 1, -2**63, 5, -5, 2**62, -2**62 - 1, 0], np.int64)
+case("signed-overflow-square-then-remainder", lambda b, x: b.remainder(b.mul(x, x), b.or_(x, 1)), _I32_WIDE, exact=True)
+case("signed-overflow-difference-then-compare", lambda b, x, y: b.compare(x, b.sub(x, y), "GE"), _I64_WIDE, _I64_WIDE[::-1].copy(), exact=True)
+case("signed-overflow-increment-then-compare", lambda b, x: [b.compare(b.add(x, 1), x, "GT"), b.compare(b.sub(x, 1), x, "LT")], _I32_WIDE, exact=True)
+case("signed-overflow-negate-abs-most-negative", lambda b, x: [b.neg(x), b.abs(x), b.div(b.abs(x), 3)], _I32_WIDE, exact=True)
+case("signed-overflow-sum-reduction", lambda b, x: [b.compare(b.reduce_sum(x, [0]), 0, "LT"), b.reduce_sum(x, [0])],
+     np.array([[2**31 - 1, 2**30, 5], [1, 2**30, -5], [0, 1, 0]], np.int32), exact=True)
+case("divide-i64-most-negative", lambda b, x, y: [b.div(x, y), b.remainder(x, y)], np.array([-2**63, -2**63, -2**63, -2**63 + 1, 2**63 - 1, -2**63], np.int64),
+     np.array([-2**63 + 1, -1, 2**62 - 1, -1, -2**63, 0], np.int64), exact=True)
+# an unsigned divisor of all ones is an ordinary number (the same bits mean -1 for a signed type, the one divisor that overflows)
+case("divide-unsigned-by-all-ones-u8", lambda b, x, y: [b.div(x, y), b.remainder(x, y)], np.array([251, 1, 255, 0, 254, 7], np.uint8), np.array([255, 255, 255, 255, 255, 0], np.uint8), exact=True)
+case("divide-unsigned-by-all-ones-u32", lambda b, x, y: [b.div(x, y), b.remainder(x, y)], np.array([4197786975, 2**32 - 1, 0, 2**32 - 2], np.uint32), np.array([2**32 - 1] * 4, np.uint32), exact=True)
+case("divide-unsigned-by-all-ones-u64", lambda b, x, y: [b.div(x, y), b.remainder(x, y)], np.array([2**64 - 1, 2**64 - 5, 12, 2**63], np.uint64), np.array([2**64 - 1, 2**64 - 1, 2**64 - 1, 3], np.uint64), exact=True)
 case("compare-u32", lambda b, x, y: b.compare(x, y, "LT"), np.array([1, 0xFFFFFFFF, 5], np.uint32), np.array([0xFFFFFFFF, 1, 5], np.uint32), exact=True)
 case("compare-totalorder", lambda b, x, y: b.compare(x, y, "LT", "TOTALORDER"),
      np.array([-0.0, 0.0, 1.0, -np.inf, -1.0], np.float32), np.array([0.0, -0.0, 2.0, np.inf, -2.0], np.float32), exact=True)

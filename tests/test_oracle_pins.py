@@ -158,6 +158,41 @@ def test_convert_float_to_int_saturates():
     assert np.array_equal(run(lambda b, a: b.convert(a, "i32"), x)[0], np.array([2**31 - 1, -2**31, 0, 1, -1], np.int32))
 
 
+def test_integer_division_against_exact_integers():
+    """Quotient truncated toward zero and remainder with the dividend's sign, both wrapped to the type (the most negative
+    value divided by -1 is itself), a zero divisor giving all ones and the dividend: every pair of int8 and uint8 values
+    and the corners of the 64-bit types against Python's unbounded integers (reference: arithmetic.cc:46-83, 496-513)."""
+    def exact(x, y, bits, signed):
+        if y == 0:
+            return (-1 if signed else 2 ** bits - 1), x
+        q = abs(x) // abs(y)
+        q = -q if (x < 0) != (y < 0) else q
+        r = x - q * y
+        if signed:
+            q = (q + 2 ** (bits - 1)) % 2 ** bits - 2 ** (bits - 1)
+        return q, r
+    for dt, name, signed in ((np.int8, "i8", True), (np.uint8, "ui8", False)):
+        v = np.arange(np.iinfo(dt).min, np.iinfo(dt).max + 1).astype(dt)
+        a, b_ = [m.ravel() for m in np.meshgrid(v, v, indexing="ij")]
+        q = run(lambda b, x, y: b.div(x, y), a, b_, dtypes=[name, name])[0]
+        r = run(lambda b, x, y: b.remainder(x, y), a, b_, dtypes=[name, name])[0]
+        want = [exact(int(x), int(y), 8, signed) for x, y in zip(a, b_)]
+        assert np.array_equal(q.astype(np.int64), np.array([w[0] for w in want])) and np.array_equal(r.astype(np.int64), np.array([w[1] for w in want]))
+    lo, hi = np.iinfo(np.int64).min, np.iinfo(np.int64).max
+    a = np.array([lo, lo, lo, lo, lo + 1, hi, hi, 7, -7, lo], np.int64)
+    b_ = np.array([lo + 1, -1, 2 ** 62 - 1, lo, -1, -1, lo, -2, 2, 0], np.int64)
+    q = run(lambda b, x, y: b.div(x, y), a, b_, dtypes=["i64", "i64"])[0]
+    r = run(lambda b, x, y: b.remainder(x, y), a, b_, dtypes=["i64", "i64"])[0]
+    want = [exact(int(x), int(y), 64, True) for x, y in zip(a, b_)]
+    assert [int(t) for t in q] == [w[0] for w in want] and [int(t) for t in r] == [w[1] for w in want]
+    a = np.array([2 ** 64 - 1, 2 ** 64 - 5, 12, 2 ** 63, 9], np.uint64)
+    b_ = np.array([2 ** 64 - 1, 2 ** 64 - 1, 2 ** 64 - 1, 3, 0], np.uint64)
+    q = run(lambda b, x, y: b.div(x, y), a, b_, dtypes=["ui64", "ui64"])[0]
+    r = run(lambda b, x, y: b.remainder(x, y), a, b_, dtypes=["ui64", "ui64"])[0]
+    want = [exact(int(x), int(y), 64, False) for x, y in zip(a, b_)]
+    assert [int(t) for t in q] == [w[0] for w in want] and [int(t) for t in r] == [w[1] for w in want]
+
+
 def test_total_order_compare():
     a = np.array([-0.0, 0.0], np.float32)
     b_ = np.array([0.0, -0.0], np.float32)
