@@ -36,7 +36,10 @@ __device__ __forceinline__ float bf2f(u16 b) { return __uint_as_float(((u32)b) <
 // gfx950 rounds f32 -> bf16 (nearest even, NaN stays NaN) in one instruction
 __device__ __forceinline__ u16 f2bf(float f) { return __builtin_bit_cast(u16, (__bf16)f); }
 __device__ __forceinline__ float bfr(float f) { return bf2f(f2bf(f)); }
-__device__ __forceinline__ float hfr(float f) { return (float)(_Float16)f; }
+// f32 -> f16 of a value that exists as an f32 first: without the empty statement the compiler folds a product and its
+// narrowing into one mixed-precision multiply-add with a +0 addend, which rounds once and turns a product of -0 into +0
+__device__ __forceinline__ _Float16 f2h(float f) { asm volatile("" : "+v"(f)); return (_Float16)f; }
+__device__ __forceinline__ float hfr(float f) { return (float)f2h(f); }
 template <typename T> __device__ __forceinline__ T mx(T a, T b) { return (a > b || a != a) ? a : b; }
 template <typename T> __device__ __forceinline__ T mn(T a, T b) { return (a < b || a != a) ? a : b; }
 template <typename I, typename F> __device__ __forceinline__ I f2i(F f) {
@@ -136,7 +139,7 @@ std::string loadExpr(DType d, const std::string& e) {
 }
 std::string storeExpr(DType d, const std::string& e) {
   if (d == DType::BF16) return "f2bf(" + e + ")";
-  if (d == DType::F16) return "(_Float16)(" + e + ")";
+  if (d == DType::F16) return "f2h(" + e + ")";
   if (d == DType::Pred) return "(u8)((" + e + ") ? 1 : 0)";
   return e;
 }
@@ -823,6 +826,15 @@ class Emitter {
       if (bits == 64) return bin("(" + T + ")__clzll((i64)" + in(0) + ")");
       std::string U = bits == 8 ? "u8" : bits == 16 ? "u16" : "u32";
       return bin("(" + T + ")(__clz((int)(u32)(" + U + ")" + in(0) + ") - " + std::to_string(32 - bits) + ")");
+    }
+    if (n == "round_nearest_afz" && isF) {
+      // the reference's formula, sign(x) * floor(|x| + 0.5) in the operand type (ops/arithmetic.cc:316-327): where the sum
+      // is not representable it rounds first, so the predecessor of 0.5 gives 1 and an odd integer from 2^23 on (2^7 for
+      // bf16, 2^10 for f16) its even neighbour; an exact rounding would differ from the reference there
+      const std::string x = in(0);
+      const std::string sum = roundTo(rt.dt, "(fabs" + sfx + "(" + x + ") + " + (isD ? "0.5" : "0.5f") + ")");
+      const std::string FT = isD ? "double" : "float";   // (the sign as the difference of two comparisons: zero for either zero)
+      return bin("((" + FT + ")((" + x + " > 0) - (" + x + " < 0)) * floor" + sfx + "(" + sum + "))");
     }
     static const std::unordered_map<std::string, const char*> unary = {
         {"exponential", "exp"}, {"exponential_minus_one", "expm1"}, {"log", "log"}, {"log_plus_one", "log1p"},

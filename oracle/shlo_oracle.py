@@ -1311,8 +1311,20 @@ class Oracle:
     def op_round_nearest_even(self, op, ins, env): return self._un(op, ins, np.rint)
 
     def op_round_nearest_afz(self, op, ins, env):
-        """Half away from zero (arithmetic.cc:316-327)."""
-        return self._un(op, ins, lambda x: np.where(np.isfinite(x), np.sign(x) * np.floor(np.abs(x) + 0.5), x))
+        """Half away from zero as the reference computes it, sign(x) * floor(|x| + 0.5) in the operand type
+        (arithmetic.cc:316-327).  The sum is rounded to the type before the floor, so the formula differs from an exact
+        rounding at the predecessor of 0.5 (the sum rounds to 1) and at odd integers from 2^(significand bits - 1) on
+        (the sum rounds to the even neighbour)."""
+        dt = op.out_types[0].dtype
+
+        def f(x):
+            s = np.abs(x) + x.dtype.type(0.5)
+            if dt == "bf16":
+                s = round_bf16(s)
+            elif dt == "f16":
+                s = s.astype(np.float16).astype(np.float32)
+            return np.where(np.isfinite(x), np.sign(x) * np.floor(s), x)
+        return self._un(op, ins, f)
 
     def op_is_finite(self, op, ins, env): return np.isfinite(ins[0])
 

@@ -82,6 +82,16 @@ case("unary-specials", lambda b, x: [b.exp(x), b.sign(x), b.abs(x), b._unary("is
      np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-40, -3.5, 88.0], np.float32))
 case("round-half", lambda b, x: [b._unary("round_nearest_even", x), b._unary("round_nearest_afz", x)],
      np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.49, -3.51], np.float32), exact=True)
+# where |x| + 0.5 is not a number of the type the reference's formula rounds the sum first (ops/arithmetic.cc:316-327)
+_AFZ = [0.49999997, -0.49999997, 0.5, 8388609.0, -8404769.0, 12606725.0, 16777215.0, 8388608.0, 4194303.5, -4194304.5, 1e-45, np.inf, -np.inf, np.nan, -0.0, 3e38]
+case("round-half-away-where-the-sum-rounds", lambda b, x: b._unary("round_nearest_afz", x), np.array(_AFZ, np.float32), exact=True)
+case("round-half-away-where-the-sum-rounds-bf16", lambda b, x: b._unary("round_nearest_afz", x),
+     np.array([0.498046875, -0.498046875, 0.5, 129.0, -131.0, 255.0, 127.5, 64.5, -2.5, 1.0, 256.0, 3e38], np.float32), dtypes=["bf16"], exact=True)
+case("round-half-away-where-the-sum-rounds-f16", lambda b, x: b._unary("round_nearest_afz", x),
+     np.array([0.49975586, -0.49975586, 0.5, 1025.0, -1027.0, 2047.0, 1023.5, 512.5, -2.5, 65504.0], np.float16), exact=True)
+# a product narrowed to f16 is rounded to f32 first and keeps the sign of a zero
+case("convert-f16-of-a-product", lambda b, x, y: [b.convert(b.convert(b.mul(x, y), "f16"), "f32"), b.div(1.0, b.convert(b.convert(b.mul(b.abs(x), x), "f16"), "f32"))],
+     np.array([-0.0, 0.0, 1.0009766, 3.0, -1e-5, 1e-30, 255.9, -0.0], np.float32), np.array([0.0, -0.0, 1.0009766, 0.33333334, 1e-4, -1e-30, 255.9, -5.0], np.float32), exact=True)
 
 # ------------------------------------------------------------------ binary (tests/configs/binary.py)
 for k, op in enumerate(["add", "sub", "mul", "div", "maximum", "minimum"]):

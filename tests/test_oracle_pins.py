@@ -193,6 +193,21 @@ def test_integer_division_against_exact_integers():
     assert [int(t) for t in q] == [w[0] for w in want] and [int(t) for t in r] == [w[1] for w in want]
 
 
+def test_round_half_away_is_the_reference_s_formula():
+    """sign(x) * floor(|x| + 0.5) evaluated in float32 (arithmetic.cc:316-327): exact halves go away from zero, and where the
+    sum is not a float32 it rounds before the floor (the predecessor of 0.5 gives 1, an odd integer above 2^23 its even
+    neighbour), checked against the same formula in exact rational arithmetic with one rounding of the sum."""
+    from fractions import Fraction
+    xs = np.array([0.5, 1.5, 2.5, -0.5, -2.5, 0.49999997, -0.49999997, 8388609.0, -8404769.0, 16777215.0, 4194303.5, 0.25, -7.75, 1e-45], np.float32)
+    got = run(lambda b, x: b._unary("round_nearest_afz", x), xs)[0]
+    want = []
+    for x in xs:
+        s = float(np.float32(float(abs(Fraction(float(x))) + Fraction(1, 2))))   # the one rounding: the sum to float32
+        want.append(math.copysign(math.floor(s), float(x)))
+    assert np.array_equal(got, np.array(want, np.float32))
+    assert got[5] == 1.0 and got[7] == 8388610.0
+
+
 def test_total_order_compare():
     a = np.array([-0.0, 0.0], np.float32)
     b_ = np.array([0.0, -0.0], np.float32)
