@@ -78,7 +78,12 @@ template <typename T> __device__ __forceinline__ T irem(T a, T b) {
   return b == (T)0 ? a : ((sg && b == (T)-1) ? (T)0 : (T)(a % b));
 }
 // 16-bit results keep 8 (bf16) or 11 (f16) significand bits: the hardware exponential is exact enough there
-__device__ __forceinline__ float tanh_fast(float x) { float t = __expf(-2.f * fabsf(x)); return copysignf((1.f - t) * __builtin_amdgcn_rcpf(1.f + t), x); }
+// (near zero 1 - exp cancels: three terms of the series there, exact to 1e-7 relative below 0.1)
+__device__ __forceinline__ float tanh_fast(float x) {
+  float t = __expf(-2.f * fabsf(x)), x2 = x * x;
+  float r = copysignf((1.f - t) * __builtin_amdgcn_rcpf(1.f + t), x);
+  return fabsf(x) < 0.1f ? x * (1.f + x2 * (-0.33333334f + x2 * 0.13333334f)) : r;
+}
 // f32 tanh to a few ulp: odd polynomial near 0 (where 1 - exp cancels), exponential form elsewhere
 __device__ __forceinline__ float tanh_f32(float x) {
   float ax = fabsf(x), x2 = x * x;

@@ -18,7 +18,9 @@ reference's own tests, torch-CPU conv2d / conv_transpose2d and brute-force loops
 for convolution, numpy einsum for dot_general, closed forms for while/case,
 IEEE special cases for shifts/remainder/sign/round.  bf16 results are pinned only
 by the rounding rule (round-to-nearest-even of the f32 result) — the reference
-holds no bf16 expectation ("parity unpinned" by the reference for bf16).
+holds no bf16 expectation ("parity unpinned" by the reference for bf16).  Also
+parity unpinned: which zero maximum / minimum return for two zeros of different
+sign (MLX's published element rule restated; no test of the reference holds the case).
 """
 from __future__ import annotations
 
@@ -1200,13 +1202,22 @@ class Oracle:
         a, b = ins
         if a.dtype == np.bool_:
             return a | b
-        return np.maximum(a, b)  # NaN-propagating, as in StableHLO
+        if a.dtype.kind != "f":
+            return np.maximum(a, b)
+        # NaN-propagating, as in StableHLO.  The reference hands the op to mlx::core::maximum (arithmetic.cc:573), whose
+        # published element rule is "x if x is NaN, else x > y ? x : y": of two equal operands (the two zeros) the second
+        # is returned, which is what tells +0 from -0 in the result.
+        with np.errstate(all="ignore"):
+            return np.where(np.isnan(a), a, np.where(a > b, a, b)).astype(a.dtype)
 
     def op_minimum(self, op, ins, env):
         a, b = ins
         if a.dtype == np.bool_:
             return a & b
-        return np.minimum(a, b)
+        if a.dtype.kind != "f":
+            return np.minimum(a, b)
+        with np.errstate(all="ignore"):   # mlx::core::minimum: x if x is NaN, else x < y ? x : y (arithmetic.cc:575)
+            return np.where(np.isnan(a), a, np.where(a < b, a, b)).astype(a.dtype)
 
     def op_power(self, op, ins, env):
         a, b = ins

@@ -92,6 +92,12 @@ case("round-half-away-where-the-sum-rounds-f16", lambda b, x: b._unary("round_ne
 # a product narrowed to f16 is rounded to f32 first and keeps the sign of a zero
 case("convert-f16-of-a-product", lambda b, x, y: [b.convert(b.convert(b.mul(x, y), "f16"), "f32"), b.div(1.0, b.convert(b.convert(b.mul(b.abs(x), x), "f16"), "f32"))],
      np.array([-0.0, 0.0, 1.0009766, 3.0, -1e-5, 1e-30, 255.9, -0.0], np.float32), np.array([0.0, -0.0, 1.0009766, 0.33333334, 1e-4, -1e-30, 255.9, -5.0], np.float32), exact=True)
+# tanh of a 16-bit float near zero is the argument itself, not the cancelled difference of two exponentials
+case("tanh-bf16-near-zero", lambda b, x: b.tanh(x), np.array([1e-8, -1e-8, 3e-5, -2e-4, 1e-3, 0.05, 0.0996, 0.1004, -0.3, 1e-19, 0.0, 2.5], np.float32), dtypes=["bf16"])
+case("tanh-f16-near-zero", lambda b, x: b.tanh(x), np.array([6e-8, -6e-8, 3e-5, -2e-4, 1e-3, 0.05, 0.0996, 0.1004, -0.3, 0.0, 2.5], np.float16))
+# of two zeros of different sign maximum and minimum return the second operand (x > y ? x : y after the NaN test)
+case("maximum-minimum-of-signed-zeros", lambda b, x, y: [b.div(1.0, b.maximum(x, y)), b.div(1.0, b.minimum(x, y))],
+     np.array([0.0, -0.0, 0.0, -0.0, np.nan, 1.0, -0.0], np.float32), np.array([-0.0, 0.0, 0.0, -0.0, -0.0, np.nan, 1e-45], np.float32), exact=True)
 
 # ------------------------------------------------------------------ binary (tests/configs/binary.py)
 for k, op in enumerate(["add", "sub", "mul", "div", "maximum", "minimum"]):
