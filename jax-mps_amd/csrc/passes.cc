@@ -1139,6 +1139,37 @@ void lowerSingleDeviceOps(Module& m) {
   for (auto& t : f->resultTypes) if (t.dt == DType::Token) { t.dt = DType::F32; t.dims.clear(); }
 }
 
+// A reduction over no elements returns its init values: each result becomes a broadcast of the matching init operand.
+namespace {
+void lowerEmptyReductionsIn(Region& r) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) lowerEmptyReductionsIn(*sub);
+    if (op->name != "reduce" || op->operands.size() < 2 || op->operands.size() != 2 * op->results.size()) continue;
+    if (op->operands[0]->type.numel() != 0 || op->results[0]->type.numel() == 0) continue;
+    const size_t n = op->results.size();
+    std::vector<std::unique_ptr<Op>> made;
+    for (size_t j = 0; j < n; ++j) {
+      auto bc = makeOp("broadcast_in_dim", {op->operands[n + j]}, &r, op->line);
+      bc->attrs["dims"] = intsAttr({});
+      bc->results.push_back(std::move(op->results[j]));
+      bc->results[0]->def = bc.get();
+      bc->results[0]->defIndex = 0;
+      made.push_back(std::move(bc));
+    }
+    for (auto* o : op->operands) o->users.erase(std::remove(o->users.begin(), o->users.end(), op), o->users.end());
+    for (auto& b : made) b->operands[0]->users.push_back(b.get());
+    r.ops.erase(r.ops.begin() + (long)k);
+    r.ops.insert(r.ops.begin() + (long)k, std::make_move_iterator(made.begin()), std::make_move_iterator(made.end()));
+    k += n - 1;
+  }
+}
+}  // namespace
+
+void lowerEmptyReductions(Module& m) {
+  if (Func* f = m.main()) lowerEmptyReductionsIn(f->body);
+}
+
 void lowerTopK(Module& m) {
   Func* f = m.main();
   if (!f) return;

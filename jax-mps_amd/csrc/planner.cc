@@ -2865,6 +2865,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   lowerWindowOps(*module);
   lowerRng(*module);
   lowerTopK(*module);
+  lowerEmptyReductions(*module);
   hoistLoopProducts(*module);
   dropScatterIndexMasks(*module);
   reluMasksFromActivations(*module);

@@ -701,6 +701,10 @@ case("reduce-rows-one-pass-scaled-by-a-concatenation", lambda b, x, u, w: b.mul(
      f32(2768, 70, 90, lo=-1, hi=1), f32(2769, 30), f32(2770, 40))
 case("reduce-column-two-passes-scaled-by-a-padded-vector", lambda b, x, w: b.mul(b.reduce_sum(x, [0]), b.pad(w, -2.0, [4], [0])),
      f32(2771, 16384, 64, lo=-1, hi=1), f32(2772, 60))
+# a reduction over no elements returns its init value
+case("reduce-over-an-empty-tensor", lambda b, x, y: [b.reduce_sum(x, [0]), b.reduce_max(x, [0]), b.add(b.reduce_sum(x, [0]), y)],
+     np.zeros((0, 4), np.float32), f32(2773, 4), exact=True)
+case("argmax-over-an-empty-dim", lambda b, x: b.argmax(x, 1), np.zeros((3, 0), np.float32), exact=True)
 case("argmax", lambda b, x: b.argmax(x, 1), f32(272, 9, 31), exact=True)
 case("argmax-leading-dim", lambda b, x: b.argmax(x, 0), f32(2720, 150, 7), exact=True)
 case("argmax-middle-dim-long", lambda b, x: b.argmax(x, 1), f32(2721, 3, 1000, 5), exact=True)
