@@ -21,7 +21,7 @@ int main(int argc, char** argv) {
   int rc = 0;
   for (int i = 1; i < argc; ++i) {
     std::string a = argv[i];
-    if (a == "--dump-plan") { dumpPlan = true; setenv("MI355X_DUMP_PLAN", "1", 1); continue; }
+    if (a == "--dump-plan") { dumpPlan = true; setenv("MI355X_DUMP_PLAN", "1", 0); continue; }
     if (a == "--dump-kernels") { dumpKernels = true; continue; }
     if (a == "--no-compile") { compile = false; continue; }
     if (a == "--bytecode-to-text") { toText = true; continue; }

@@ -365,14 +365,16 @@ class Planner {
       // buffers that exist anyway (normalised indices, say): the kernels that also read it recompute it, so they do
       // not depend on the kernel that stores it and can share its launch.
       static const bool inlineSmall = !getenv("MI355X_INLINE_SMALL") || atoi(getenv("MI355X_INLINE_SMALL")) != 0;
-      if (inlineSmall && mat && forced && !nestedUse && loopDepth_ == 0 && !op->has("force_materialize") && v->type.numel() <= kSmallNumel && v->users.size() >= 2) {
+      // (not the sum a product writes together with its bias: the bare product it would be recomputed from is never stored)
+      if (inlineSmall && mat && forced && !nestedUse && loopDepth_ == 0 && !op->has("force_materialize") && v->type.numel() <= kSmallNumel && v->users.size() >= 2 &&
+          !alwaysInMemory(v)) {
         int budget = 8;
         if (cheapFromMemory(v, budget)) inlineAnyway_.insert(v);
       }
       // in a loop body the same holds for somewhat larger values (cheap chains only: a column reduction runs few
       // workgroups, and each lane would walk an expensive chain once per row)
       if (inlineSmall && mat && forced && !nestedUse && loopDepth_ > 0 && specFloors_.empty() && !op->has("force_materialize") &&
-          v->type.numel() <= kLoopSmallNumel && v->users.size() >= 2 && op->name != "constant" && op->name != "dynamic_update_slice") {
+          v->type.numel() <= kLoopSmallNumel && v->users.size() >= 2 && op->name != "constant" && op->name != "dynamic_update_slice" && !alwaysInMemory(v)) {
         int budget = 16;
         if (cheapFromMemory(v, budget)) inlineAnyway_.insert(v);
       }
@@ -1272,25 +1274,16 @@ class Planner {
     return reshapeStrides(xt.dims, in.strides, v->type.dims, out.strides);
   }
 
-  // the add that emitDot folds into the product of `dot` as a bias epilogue, or null
-  static Op* foldedBiasAdd(Op* dot) {
-    if (dot->name != "dot_general" && dot->name != "dot") return nullptr;
-    // exactly one free rhs dim, so that the last result dim is the GEMM's column index
-    Value* b = dot->operands[1];
-    int64_t used = (int64_t)dot->ints("rhs_batch").size() + (int64_t)dot->ints("rhs_contract").size();
-    if (dot->name == "dot") used = 1;
-    if (b->type.rank() - used != 1) return nullptr;
-    return biasAddOf(dot->result());
-  }
-
   // values that are in memory whatever the fusion analysis decides: arguments, results of ops that
   // are steps of their own, and bias sums folded into their product
   static bool alwaysInMemory(Value* v) {
     if (!v->def) return true;
     if (!isFusibleOp(*v->def)) return v->def->name != "return";
+    // the sum a product step may write itself (with its bias, with an addend, with a second product): the bare product
+    // is then never stored, so the sum cannot be recomputed from it
     if (v->def->name == "add")
       for (auto* o : v->def->operands)
-        if (o->def && (o->def->name == "dot_general" || o->def->name == "dot") && foldedBiasAdd(o->def) == v->def) return true;
+        if (o->def && (o->def->name == "dot_general" || o->def->name == "dot") && o->users.size() == 1) return true;
     return false;
   }
 
@@ -2794,6 +2787,10 @@ class Planner {
       if (s.kind == Step::Copy && s.condMode) o << (s.condMode == 1 ? " if-alive" : " if-selected");
       if (s.forkId >= 0) o << " [second stream #" << s.forkId << "]";
       for (int id : s.joins) o << " [waits for #" << id << "]";
+      if (getenv("MI355X_DUMP_PLAN") && atoi(getenv("MI355X_DUMP_PLAN")) >= 2) {   // what the step reads and writes
+        static const char* where[] = {"none", "param", "out", "temp", "const"};
+        forEachRef(const_cast<Step&>(s), [&](BufRef& r, bool wr) { o << (wr ? " W:" : " R:") << where[r.kind] << r.index << "+" << r.offset; });
+      }
       o << "\n";
       P.dump += o.str();
       o.str("");

@@ -705,6 +705,21 @@ case("reduce-column-two-passes-scaled-by-a-padded-vector", lambda b, x, w: b.mul
 case("reduce-over-an-empty-tensor", lambda b, x, y: [b.reduce_sum(x, [0]), b.reduce_max(x, [0]), b.add(b.reduce_sum(x, [0]), y)],
      np.zeros((0, 4), np.float32), f32(2773, 4), exact=True)
 case("argmax-over-an-empty-dim", lambda b, x: b.argmax(x, 1), np.zeros((3, 0), np.float32), exact=True)
+# a small sum that a product step writes itself (bias, addend, second product) and that two readers share, one of them a
+# product: the readers load the sum, the bare product is not in memory to recompute it from
+case("dot-bias-sum-read-by-a-product-and-a-kernel", lambda b, x, w, c, u: (lambda y: b.mul(y, b.logistic(b.matmul(y, u))))(b.add(b.matmul(x, w), b.broadcast_in_dim(c, (4, 8), [1]))),
+     f32(2780, 4, 64, lo=-1, hi=1), f32(2781, 64, 8, lo=-0.3, hi=0.3), f32(2782, 8), f32(2783, 8, 8, lo=-0.5, hi=0.5))
+case("dot-addend-sum-read-by-a-product-and-a-kernel", lambda b, x, w, y0, u: (lambda y: b.mul(y, b.tanh(b.matmul(y, u))))(b.add(b.tanh(y0), b.matmul(x, w))),
+     f32(2784, 16, 24, lo=-1, hi=1), f32(2785, 24, 8, lo=-0.3, hi=0.3), f32(2786, 16, 8), f32(2787, 8, 8, lo=-0.5, hi=0.5))
+case("dot-two-products-sum-read-by-a-product-and-a-kernel", lambda b, x, w, h, v, u: (lambda y: b.add(y, b.matmul(y, u)))(b.add(b.matmul(x, w), b.matmul(h, v))),
+     f32(2788, 16, 24, lo=-1, hi=1), f32(2789, 24, 8, lo=-0.3, hi=0.3), f32(2790, 16, 12, lo=-1, hi=1), f32(2791, 12, 8, lo=-0.3, hi=0.3), f32(2792, 8, 8, lo=-0.5, hi=0.5))
+def _gated_loop(b, x, w, c, u):
+    zero = b.constant(0, "i32")
+    def body(i, h):
+        y = b.add(b.matmul(h, w), b.broadcast_in_dim(c, (4, 8), [1]))
+        return [b.add(i, 1), b.mul(y, b.logistic(b.matmul(y, u)))]
+    return b.while_loop([zero, x], lambda i, h: b.compare(i, 3, "LT"), body)[1]
+case("while-dot-bias-sum-read-by-a-product-and-a-kernel", _gated_loop, f32(2793, 4, 8, lo=-1, hi=1), f32(2794, 8, 8, lo=-0.6, hi=0.6), f32(2795, 8), f32(2796, 8, 8, lo=-0.5, hi=0.5))
 case("argmax", lambda b, x: b.argmax(x, 1), f32(272, 9, 31), exact=True)
 case("argmax-leading-dim", lambda b, x: b.argmax(x, 0), f32(2720, 150, 7), exact=True)
 case("argmax-middle-dim-long", lambda b, x: b.argmax(x, 1), f32(2721, 3, 1000, 5), exact=True)
