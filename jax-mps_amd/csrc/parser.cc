@@ -101,6 +101,12 @@ class Parser {
       if (wrapped && eat("}")) break;
       skipAliasLines();
       if (i_ >= n_) break;
+      // Shardy's module-level declarations (sdy.mesh @mesh = <["x"=1]>) say nothing a single device needs: skipped, as
+      // the reference lets unregistered dialects pass (stablehlo_parser.cc:74-75)
+      if (peek("sdy.")) {
+        while (i_ < n_ && s_[i_] != '\n') ++i_;
+        continue;
+      }
       m->funcs.push_back(parseFunc());
     }
     if (wrapped) skipLoc();
@@ -581,6 +587,24 @@ class Parser {
           --depth;
         }
         ++i_;
+      }
+      a.s = std::string(s_ + b, i_ - b);
+      expect(">");
+      return a;
+    }
+    if (name.compare(0, 4, "sdy.") == 0) {
+      // Shardy attributes (#sdy.sharding<@mesh, [{}, {"x"}]>): kept as their text, read by nothing
+      a.kind = Attr::Str;
+      size_t b = i_;
+      int depth = 0;
+      bool quoted = false;
+      for (; i_ < n_; ++i_) {
+        char c = s_[i_];
+        if (c == '"') quoted = !quoted;
+        if (quoted) continue;
+        if (c == '<' || c == '[' || c == '{') ++depth;
+        else if (c == ']' || c == '}') --depth;
+        else if (c == '>') { if (depth == 0) break; --depth; }
       }
       a.s = std::string(s_ + b, i_ - b);
       expect(">");

@@ -1131,6 +1131,35 @@ def all_cases() -> List[Case]:
     return [mk() for mk in _cases]
 
 
+def raw_case(name, text, *inputs, dtypes, exact=False):
+    """A case given as module text (forms the builder does not print)."""
+    def make():
+        return Case(name, text, [np.asarray(a) for a in inputs], list(dtypes), exact)
+    make.case_name = name
+    _cases.append(make)
+
+
+raw_case("text-hex-constant-bool-list-barrier-sharding-call", """module @jit_f attributes {mhlo.num_partitions = 1 : i32, mhlo.num_replicas = 1 : i32} {
+  func.func public @main(%arg0: tensor<3xf32> {mhlo.layout_mode = "default"}, %arg1: tensor<2x4xf32> {jax.buffer_donor = true}) -> (tensor<3xf32> {jax.result_info = "[0]"}, tensor<2xi1>, tensor<1x2xf32>) {
+    %cst = stablehlo.constant dense<"0x0000803F0000004000004040"> : tensor<3xf32>
+    %c = stablehlo.constant dense<[true, false]> : tensor<2xi1>
+    %c_0 = stablehlo.constant dense<true> : tensor<i1>
+    %cst_2 = stablehlo.constant dense<1.500000e+00> : tensor<3xf32>
+    %0 = stablehlo.add %arg0, %cst : tensor<3xf32>
+    %1 = stablehlo.multiply %0, %cst_2 : tensor<3xf32>
+    %2 = stablehlo.broadcast_in_dim %c_0, dims = [] : (tensor<i1>) -> tensor<2xi1>
+    %3 = stablehlo.and %c, %2 : tensor<2xi1>
+    %c_3 = stablehlo.constant dense<1> : tensor<i32>
+    %c_4 = stablehlo.constant dense<0> : tensor<i32>
+    %4 = stablehlo.dynamic_slice %arg1, %c_4, %c_3, sizes = [1, 2] : (tensor<2x4xf32>, tensor<i32>, tensor<i32>) -> tensor<1x2xf32>
+    %5 = stablehlo.custom_call @Sharding(%4) {backend_config = "", mhlo.sharding = "{replicated}"} : (tensor<1x2xf32>) -> tensor<1x2xf32>
+    %6 = stablehlo.optimization_barrier %5 : tensor<1x2xf32>
+    return %1, %3, %6 : tensor<3xf32>, tensor<2xi1>, tensor<1x2xf32>
+  }
+}
+""", np.array([10, 20, 30], np.float32), np.arange(8, dtype=np.float32).reshape(2, 4), dtypes=["f32", "f32"], exact=True)
+
+
 def case_names() -> List[str]:
     return [mk.case_name for mk in _cases]
 

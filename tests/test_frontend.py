@@ -219,6 +219,41 @@ module @jit_f attributes {mhlo.num_partitions = 1 : i32} {
     assert r.returncode == 0, r.stderr
 
 
+def test_shardy_declarations_hex_constants_and_argument_attributes_parse():
+    """What jax prints around a single-device program when the Shardy partitioner is on (module-level sdy.mesh, #sdy.sharding
+    argument attributes), large constants as hex strings, boolean lists, layout / donor attributes, @Sharding custom calls
+    and optimization barriers: all accepted, as the reference lets unregistered dialects pass (stablehlo_parser.cc:74-75)."""
+    text = """#loc = loc(unknown)
+module @jit_f attributes {jax.uses_shape_polymorphism = false, mhlo.num_partitions = 1 : i32, mhlo.num_replicas = 1 : i32} {
+  sdy.mesh @mesh = <["x"=1]>
+  func.func public @main(%arg0: tensor<3xf32> {mhlo.layout_mode = "default", sdy.sharding = #sdy.sharding<@mesh, [{"x"}]>} loc(unknown), %arg1: tensor<2x4xf32> {jax.buffer_donor = true}) -> (tensor<3xf32> {jax.result_info = "[0]", mhlo.layout_mode = "default"}, tensor<2xi1>, tensor<1x2xf32>) {
+    %cst = stablehlo.constant dense<"0x0000803F0000004000004040"> : tensor<3xf32> loc(#loc)
+    %c = stablehlo.constant dense<[true, false]> : tensor<2xi1> loc(#loc)
+    %c_0 = stablehlo.constant dense<true> : tensor<i1>
+    %cst_2 = stablehlo.constant dense<1.500000e+00> : tensor<3xf32>
+    %0 = stablehlo.add %arg0, %cst : tensor<3xf32> loc(#loc)
+    %1 = stablehlo.multiply %0, %cst_2 : tensor<3xf32>
+    %2 = stablehlo.broadcast_in_dim %c_0, dims = [] : (tensor<i1>) -> tensor<2xi1>
+    %3 = stablehlo.and %c, %2 : tensor<2xi1>
+    %c_3 = stablehlo.constant dense<1> : tensor<i32>
+    %c_4 = stablehlo.constant dense<0> : tensor<i32>
+    %4 = stablehlo.dynamic_slice %arg1, %c_4, %c_3, sizes = [1, 2] : (tensor<2x4xf32>, tensor<i32>, tensor<i32>) -> tensor<1x2xf32>
+    %5 = stablehlo.custom_call @Sharding(%4) {backend_config = "", mhlo.sharding = "{replicated}"} : (tensor<1x2xf32>) -> tensor<1x2xf32>
+    %6 = stablehlo.optimization_barrier %5 : tensor<1x2xf32>
+    return %1, %3, %6 : tensor<3xf32>, tensor<2xi1>, tensor<1x2xf32> loc(#loc)
+  } loc(#loc)
+} loc(#loc)
+"""
+    r = plan(text)
+    assert r.returncode == 0, r.stderr
+    # the hex string holds 1, 2, 3: the oracle reads the same text and adds it to the argument
+    import numpy as np
+    from shlo_oracle import Oracle
+    plain = text.replace('  sdy.mesh @mesh = <["x"=1]>\n', "").replace(', sdy.sharding = #sdy.sharding<@mesh, [{"x"}]>', "")   # (the oracle reads no Shardy)
+    got = Oracle(plain).run(np.array([10, 20, 30], np.float32), np.arange(8, dtype=np.float32).reshape(2, 4))
+    assert np.array_equal(got[0], np.array([16.5, 33.0, 49.5], np.float32)) and np.array_equal(got[1], [True, False]) and np.array_equal(got[2], [[1.0, 2.0]])
+
+
 def test_convolution_delivers_batch_norm_statistics():
     """The column sum and sum of squares of an unsplit convolution's output come from its accumulators: the pass over
     the output is gone and only the fold of the per-tile sums remains; a convolution that splits K, or a reduction
