@@ -2015,14 +2015,16 @@ FusedCode generateRowProgram(const RowProgram& rp, const LeafPredicate& isLeaf) 
     std::string idxPre;
     Index full, keptIdx;
     rowIndex(*em, idxPre, full, keptIdx);
+    // the per-row results first, ahead of the walk: a full-shape result that reads one of them (through a broadcast)
+    // then finds it declared where the store after the walk can see it too
+    std::vector<std::string> kvals;
+    for (auto* v : rp.keptRoots) kvals.push_back(em->gen(v, keptIdx));
     std::string savedPre = em->pre_;
     em->pre_.clear();
     std::vector<std::string> vals;
     for (auto* v : rp.fullRoots) vals.push_back(em->gen(v, full));
     std::string loopPre = idxPre + em->pre_;
     em->pre_ = savedPre;
-    std::vector<std::string> kvals;
-    for (auto* v : rp.keptRoots) kvals.push_back(em->gen(v, keptIdx));
     std::ostringstream h, t;
     h << "  {\n" << em->pre_;
     if (!rp.fullRoots.empty()) {

@@ -720,6 +720,11 @@ def _gated_loop(b, x, w, c, u):
         return [b.add(i, 1), b.mul(y, b.logistic(b.matmul(y, u)))]
     return b.while_loop([zero, x], lambda i, h: b.compare(i, 3, "LT"), body)[1]
 case("while-dot-bias-sum-read-by-a-product-and-a-kernel", _gated_loop, f32(2793, 4, 8, lo=-1, hi=1), f32(2794, 8, 8, lo=-0.6, hi=0.6), f32(2795, 8), f32(2796, 8, 8, lo=-0.5, hi=0.5))
+# a row program whose per-row result is an output of its own and is also read back, broadcast, by the full-shape result
+case("row-program-per-row-result-returned-and-read-back", lambda b, x, y: (lambda v: (lambda r: [r, b.sub(v, b.broadcast_in_dim(r, (378, 2), [0]))])(
+     b.rsqrt(b.add(b.abs(b.mul(b.reduce_sum(v, [1]), 0.5)), 1e-3))))(b.mul(x, y)), f32(2797, 378, 2, lo=-1, hi=1), f32(2798, 378, 2, lo=-1, hi=1))
+case("row-program-per-row-result-returned-and-read-back-wide", lambda b, x: (lambda m: [m, b.exp(b.sub(x, b.broadcast_in_dim(m, (50, 700), [0])))])(b.reduce_max(x, [1])),
+     f32(2799, 50, 700, lo=-2, hi=2))
 case("argmax", lambda b, x: b.argmax(x, 1), f32(272, 9, 31), exact=True)
 case("argmax-leading-dim", lambda b, x: b.argmax(x, 0), f32(2720, 150, 7), exact=True)
 case("argmax-middle-dim-long", lambda b, x: b.argmax(x, 1), f32(2721, 3, 1000, 5), exact=True)
