@@ -693,6 +693,45 @@ std::vector<Value*> tapSlices(Rewriter& rw, Value* padded, const WindowSpec& w, 
   return taps;
 }
 
+// whether `init` is a constant holding the identity of the reducer `comb` for its element type
+bool isReducerIdentity(Value* init, const std::string& comb) {
+  Op* d = init->def;
+  while (d && (d->name == "broadcast_in_dim" || d->name == "reshape") && d->operands.size() == 1) d = d->operands[0]->def;
+  if (!d || d->name != "constant" || !d->has("value") || !d->attrs.at("value").dense) return false;
+  const DenseData& dd = *d->attrs.at("value").dense;
+  if (!dd.splat && dd.type.numel() != 1) return false;
+  const DType dt = dd.type.dt;
+  const size_t sz = dtypeSize(dt);
+  if (dd.bytes.size() < sz) return false;
+  if (isFloat(dt)) {
+    double v;
+    if (dt == DType::F32) { float f; memcpy(&f, dd.bytes.data(), 4); v = f; }
+    else if (dt == DType::F64) memcpy(&v, dd.bytes.data(), 8);
+    else if (dt == DType::BF16) { uint16_t h; memcpy(&h, dd.bytes.data(), 2); uint32_t u = (uint32_t)h << 16; float f; memcpy(&f, &u, 4); v = f; }
+    else if (dt == DType::F16) { _Float16 h; memcpy(&h, dd.bytes.data(), 2); v = (double)(float)h; }
+    else return false;
+    if (comb == "add") return v == 0.0;
+    if (comb == "multiply") return v == 1.0;
+    if (comb == "maximum") return v == -__builtin_inf();
+    if (comb == "minimum") return v == __builtin_inf();
+    return false;
+  }
+  uint64_t bits = 0;
+  memcpy(&bits, dd.bytes.data(), sz);
+  const uint64_t ones = sz == 8 ? ~0ull : ((1ull << (8 * sz)) - 1);
+  const bool sg = dt == DType::S8 || dt == DType::S16 || dt == DType::S32 || dt == DType::S64;
+  if (dt == DType::Pred) {
+    const bool b = dd.bytes[0] != 0;
+    return (comb == "add" || comb == "or" || comb == "xor" || comb == "maximum") ? !b : b;   // multiply, and, minimum: true
+  }
+  if (comb == "add" || comb == "or" || comb == "xor") return bits == 0;
+  if (comb == "multiply") return bits == 1;
+  if (comb == "and") return bits == ones;
+  if (comb == "maximum") return bits == (sg ? (1ull << (8 * sz - 1)) : 0ull);
+  if (comb == "minimum") return bits == (sg ? (ones >> 1) : ones);
+  return false;
+}
+
 void lowerWindowOpsIn(Region& r, int& nextId) {
   for (size_t k = 0; k < r.ops.size(); ++k) {
     Op* op = r.ops[k].get();
@@ -722,8 +761,49 @@ void lowerWindowOpsIn(Region& r, int& nextId) {
         const int64_t n = axis >= 0 ? x->type.dims[axis] : 0;
         const bool forward = cumulative && axis >= 0 && w.padLo[axis] == n - 1 && w.padHi[axis] == 0;
         const bool backward = cumulative && axis >= 0 && w.padLo[axis] == 0 && w.padHi[axis] == n - 1;
-        if (!forward && !backward)
-          throw CompileError("stablehlo.reduce_window: windows of more than 64 elements are supported only in the cumulative form (one whole dim, padded by n-1 on one side)");
+        if (!forward && !backward) {
+          // A rectangular window is the product of one window per dim, and the reducers taken here are associative
+          // and commutative: reduce dim after dim (14 + 14 taps for a 14 x 14 pooling window instead of 196).  Padding
+          // cells hold the init value, which has to be the reducer's identity for the stages to compose.
+          bool perDim = isReducerIdentity(init, comb);
+          for (int d = 0; d < w.rank; ++d) if (w.size[d] > kMaxWindowTaps) perDim = false;
+          if (!perDim)
+            throw CompileError("stablehlo.reduce_window: windows of more than 64 elements need the reducer's identity as init value and at most 64 elements per dim "
+                               "(or the cumulative form: one whole dim, padded by n-1 on one side)");
+          Value* cur = x;
+          std::vector<int> stages;
+          for (int d = 0; d < w.rank; ++d)
+            if (w.size[d] != 1 || w.stride[d] != 1 || w.padLo[d] || w.padHi[d] || w.baseDil[d] != 1) stages.push_back(d);
+          for (size_t q = 0; q < stages.size(); ++q) {
+            const int d = stages[q];
+            WindowSpec one;
+            one.rank = w.rank;
+            one.size.assign(w.rank, 1); one.stride.assign(w.rank, 1); one.baseDil.assign(w.rank, 1); one.winDil.assign(w.rank, 1);
+            one.padLo.assign(w.rank, 0); one.padHi.assign(w.rank, 0);
+            one.size[d] = w.size[d]; one.stride[d] = w.stride[d]; one.winDil[d] = w.winDil[d];
+            one.taps = w.size[d];
+            std::vector<int64_t> lo(w.rank, 0), hi(w.rank, 0), interior(w.rank, 0);
+            lo[d] = w.padLo[d]; hi[d] = w.padHi[d]; interior[d] = w.baseDil[d] - 1;
+            Value* padded = rw.pad(cur, init, lo, hi, interior);
+            TensorType st = cur->type;
+            st.dims[d] = rt.dims[d];
+            auto taps = tapSlices(rw, padded, one, st.dims);
+            const bool lastStage = q + 1 == stages.size();
+            Value* acc = taps[0];
+            for (size_t t = 1; t < taps.size(); ++t) {
+              if (lastStage && t + 1 == taps.size()) break;
+              acc = rw.binary(comb, acc, taps[t], st);
+            }
+            if (lastStage) {
+              // (a last stage of one tap still needs an op to carry the results: the identity combined with it)
+              auto last = taps.size() == 1 ? makeOp(comb, {rw.broadcastScalar(init, st), acc}, &r, op->line) : makeOp(comb, {acc, taps.back()}, &r, op->line);
+              rw.finish(k, op, std::move(last));
+            } else {
+              cur = acc;
+            }
+          }
+          continue;
+        }
         Value* cur = x;
         std::vector<int64_t> zeros(w.rank, 0);
         for (int64_t sft = 1; sft < n; sft *= 2) {

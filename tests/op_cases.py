@@ -1279,6 +1279,12 @@ case("maxpool-grad-ties", lambda b, x, g: b.select_and_scatter(x, g, 0.0, (1, 2,
      np.round(f32(3007, 1, 6, 6, 2) * 2).astype(np.float32), f32(3008, 1, 5, 5, 2))
 case("minpool-grad", lambda b, x, g: b.select_and_scatter(x, g, 0.0, (1, 2, 2, 1), (1, 2, 2, 1), direction="LE"), f32(3009, 2, 6, 6, 4), f32(3010, 2, 3, 3, 4))
 
+# windows of more than 64 elements that are not cumulative sums: reduced dim after dim
+case("avgpool-whole-16x16-extent", lambda b, x: b.mul(b.reduce_window(x, 0.0, "add", (1, 16, 16, 1), (1, 1, 1, 1)), 1.0 / 256), f32(3030, 2, 16, 16, 8))
+case("maxpool-9x9-s2-pad4", lambda b, x: b.reduce_window(x, float("-inf"), "max", (1, 9, 9, 1), (1, 2, 2, 1), [(0, 0), (4, 4), (4, 4), (0, 0)]), f32(3031, 2, 20, 17, 4), exact=True)
+case("sumpool-5x5x5-dilated-int", lambda b, x: b.reduce_window(x, 0, "add", (5, 5, 5), (2, 1, 1), [(2, 2), (0, 3), (1, 0)], (1, 2, 1), (1, 1, 2)),
+     rng(3032).integers(-9, 9, size=(11, 9, 12)).astype(np.int32), exact=True)
+
 # cumulative reductions as JAX lowers them: a reduce_window over one whole dim padded by n-1 (tests/configs/reduction.py:41-77)
 case("cumsum-axis1", lambda b, x: b.reduce_window(x, 0.0, "add", (1, 300), (1, 1), [(0, 0), (299, 0)]), f32(3020, 7, 300))
 case("cumsum-axis0-int", lambda b, x: b.reduce_window(x, 0, "add", (200, 1), (1, 1), [(199, 0), (0, 0)]), rng(3021).integers(-50, 50, size=(200, 9)).astype(np.int32), exact=True)
