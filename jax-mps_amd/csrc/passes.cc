@@ -1250,6 +1250,112 @@ void lowerEmptyReductions(Module& m) {
   if (Func* f = m.main()) lowerEmptyReductionsIn(f->body);
 }
 
+// A product step reads each operand as one strided matrix per batch: its free dims, its contracted dims and its batch
+// dims each have to collapse to one stride (two for the batch).  jax leaves the operand dims of an einsum or tensordot
+// where they are (free dims on both sides of a contracted one, say); such an operand gets a transpose in front, to
+// [batch..., free..., contracted...] on the left and [batch..., contracted..., free...] on the right, which the result
+// dims (batch, left free, right free) do not notice.  Reference: ops/linalg.cc:89-250 takes any dimension numbers.
+namespace {
+bool runCollapses(const TensorType& t, const std::vector<int64_t>& dims) {
+  std::vector<int64_t> st((size_t)t.rank(), 1);
+  for (int d = t.rank() - 2; d >= 0; --d) st[(size_t)d] = st[(size_t)d + 1] * t.dims[(size_t)d + 1];
+  bool have = false;
+  int64_t expect = 0;
+  for (int64_t d : dims) {
+    if (t.dims[(size_t)d] == 1) continue;
+    if (have && st[(size_t)d] * t.dims[(size_t)d] != expect) return false;
+    have = true;
+    expect = st[(size_t)d];
+  }
+  return true;
+}
+void canonicalizeDotLayoutsIn(Region& r, int& nextId) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) canonicalizeDotLayoutsIn(*sub, nextId);
+    if (op->name != "dot_general" || op->operands.size() != 2) continue;
+    Value* a = op->operands[0];
+    Value* b = op->operands[1];
+    if (!isFloat(a->type.dt)) continue;
+    std::vector<int64_t> ab = op->ints("lhs_batch"), bb = op->ints("rhs_batch"), ac = op->ints("lhs_contract"), bc = op->ints("rhs_contract");
+    auto has = [](const std::vector<int64_t>& v, int64_t x) { return std::find(v.begin(), v.end(), x) != v.end(); };
+    std::vector<int64_t> af, bf;
+    for (int d = 0; d < a->type.rank(); ++d) if (!has(ab, d) && !has(ac, d)) af.push_back(d);
+    for (int d = 0; d < b->type.rank(); ++d) if (!has(bb, d) && !has(bc, d)) bf.push_back(d);
+    // the contracted dims in the order of the left operand's memory, as the planner takes them
+    std::vector<size_t> order(ac.size());
+    for (size_t q = 0; q < order.size(); ++q) order[q] = q;
+    std::sort(order.begin(), order.end(), [&](size_t x, size_t y) { return ac[x] < ac[y]; });
+    std::vector<int64_t> acs, bcs;
+    for (auto q : order) { acs.push_back(ac[q]); bcs.push_back(bc[q]); }
+    // batch dims: at most two runs that collapse on both sides together
+    size_t runs = 0;
+    {
+      std::vector<int64_t> sa((size_t)a->type.rank(), 1), sb((size_t)b->type.rank(), 1);
+      for (int d = a->type.rank() - 2; d >= 0; --d) sa[(size_t)d] = sa[(size_t)d + 1] * a->type.dims[(size_t)d + 1];
+      for (int d = b->type.rank() - 2; d >= 0; --d) sb[(size_t)d] = sb[(size_t)d + 1] * b->type.dims[(size_t)d + 1];
+      int64_t ea = 0, eb = 0;
+      for (size_t q = 0; q < ab.size(); ++q) {
+        const int64_t n = a->type.dims[(size_t)ab[q]];
+        if (n == 1) continue;
+        if (runs == 0 || sa[(size_t)ab[q]] * n != ea || sb[(size_t)bb[q]] * n != eb) ++runs;
+        ea = sa[(size_t)ab[q]];
+        eb = sb[(size_t)bb[q]];
+      }
+    }
+    const bool fine = runCollapses(a->type, acs) && runCollapses(b->type, bcs) && runCollapses(a->type, af) && runCollapses(b->type, bf) && runs <= 2;
+    if (fine) continue;
+    std::vector<std::unique_ptr<Op>> made;
+    auto transposed = [&](Value* v, const std::vector<int64_t>& perm) -> Value* {
+      bool identity = true;
+      for (size_t q = 0; q < perm.size(); ++q) if (perm[q] != (int64_t)q) identity = false;
+      if (identity) return v;
+      auto t = makeOp("transpose", {v}, &r, op->line);
+      t->attrs["dims"] = intsAttr(perm);
+      TensorType tt = v->type;
+      for (size_t q = 0; q < perm.size(); ++q) tt.dims[q] = v->type.dims[(size_t)perm[q]];
+      Value* out = addResult(t.get(), tt, nextId);
+      v->users.push_back(t.get());
+      made.push_back(std::move(t));
+      return out;
+    };
+    std::vector<int64_t> pa = ab, pb = bb;
+    pa.insert(pa.end(), af.begin(), af.end());
+    pa.insert(pa.end(), ac.begin(), ac.end());
+    pb.insert(pb.end(), bc.begin(), bc.end());
+    pb.insert(pb.end(), bf.begin(), bf.end());
+    Value* na = transposed(a, pa);
+    Value* nb = transposed(b, pb);
+    auto swapOperand = [&](size_t at, Value* from, Value* to) {
+      if (from == to) return;
+      from->users.erase(std::remove(from->users.begin(), from->users.end(), op), from->users.end());
+      op->operands[at] = to;
+      to->users.push_back(op);
+    };
+    swapOperand(0, a, na);
+    swapOperand(1, b, nb);
+    const int64_t nbat = (int64_t)ab.size(), nfa = (int64_t)af.size(), nc = (int64_t)ac.size();
+    std::vector<int64_t> batch, lc, rc;
+    for (int64_t q = 0; q < nbat; ++q) batch.push_back(q);
+    for (int64_t q = 0; q < nc; ++q) { lc.push_back(nbat + nfa + q); rc.push_back(nbat + q); }
+    op->attrs["lhs_batch"] = intsAttr(batch);
+    op->attrs["rhs_batch"] = intsAttr(batch);
+    op->attrs["lhs_contract"] = intsAttr(lc);
+    op->attrs["rhs_contract"] = intsAttr(rc);
+    const size_t n = made.size();
+    r.ops.insert(r.ops.begin() + (long)k, std::make_move_iterator(made.begin()), std::make_move_iterator(made.end()));
+    k += n;
+  }
+}
+}  // namespace
+
+void canonicalizeDotLayouts(Module& m) {
+  Func* f = m.main();
+  if (!f) return;
+  int nextId = maxValueId(f->body) + 1;
+  canonicalizeDotLayoutsIn(f->body, nextId);
+}
+
 void lowerTopK(Module& m) {
   Func* f = m.main();
   if (!f) return;

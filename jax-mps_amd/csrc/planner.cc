@@ -1640,45 +1640,57 @@ class Planner {
       throw CompileError("dot_general: only f32 and bf16 operands are supported");
     View va, vb;
     auto stored = [this](Value* v) { return hasStorage(v); };
-    for (Value* v : {a, b}) {
-      View& vw = v == a ? va : vb;
-      if (!hasStorage(v) && !(dotTakesView(v, op) && resolveView(v, stored, vw))) materializeNow(v, plan);
-      if (hasStorage(v)) { vw.root = v; vw.offset = 0; vw.strides = stridesOf(v->type); vw.iterOffsets.clear(); }
-    }
-    if (b == a) vb = va;
     DotPlan dp;
     GemmDesc& g = dp.g;
     g.inType = a->type.dt;
     g.outType = c->type.dt;
-    // contraction dims: order both sides by the lhs stride so each side collapses when it can
-    std::vector<size_t> order(ac.size());
-    for (size_t k = 0; k < order.size(); ++k) order[k] = k;
-    const std::vector<int64_t>& ast = va.strides;
-    std::sort(order.begin(), order.end(), [&](size_t x, size_t y) { return ast[ac[x]] > ast[ac[y]]; });
-    std::vector<int64_t> acs, bcs;
-    for (auto k : order) { acs.push_back(ac[k]); bcs.push_back(bc[k]); }
-    int64_t Ka = 0, Kb = 0, M = 0, N = 0;
-    bool ok = mergeDims(a->type, va.strides, acs, Ka, g.aCol) && mergeDims(b->type, vb.strides, bcs, Kb, g.bRow) &&
-              mergeDims(a->type, va.strides, af, M, g.aRow) && mergeDims(b->type, vb.strides, bf, N, g.bCol);
-    g.M = M; g.N = N; g.K = Ka;
-    // batch dims: up to two independent strides per operand
     std::vector<int64_t> bsz;
     std::vector<int64_t> abst, bbst;
-    const std::vector<int64_t>& bstr = vb.strides;
-    for (size_t k = 0; k < ab.size(); ++k) {
-      if (a->type.dims[ab[k]] == 1) continue;
-      if (!bsz.empty() && ast[ab[k]] * a->type.dims[ab[k]] == abst.back() && bstr[bb[k]] * b->type.dims[bb[k]] == bbst.back()) {
-        bsz.back() *= a->type.dims[ab[k]];
-        abst.back() = ast[ab[k]];
-        bbst.back() = bstr[bb[k]];
-      } else {
-        bsz.push_back(a->type.dims[ab[k]]);
-        abst.push_back(ast[ab[k]]);
-        bbst.push_back(bstr[bb[k]]);
+    // An operand that is a chain of views over a buffer is read in place when its dims then still collapse to one
+    // strided 2-D matrix per batch; otherwise the chain is written out first and read as the plain tensor it makes
+    // (canonicalizeDotLayouts has put a transpose in front of every product whose plain operands would not collapse).
+    for (int attempt = 0; attempt < 2; ++attempt) {
+      const bool viewsAllowed = attempt == 0;
+      bool usedView = false;
+      for (Value* v : {a, b}) {
+        View& vw = v == a ? va : vb;
+        if (!hasStorage(v)) {
+          if (viewsAllowed && dotTakesView(v, op) && resolveView(v, stored, vw)) usedView = true;
+          else materializeNow(v, plan);
+        }
+        if (hasStorage(v)) { vw.root = v; vw.offset = 0; vw.strides = stridesOf(v->type); vw.iterOffsets.clear(); }
       }
+      if (b == a) vb = va;
+      // contraction dims: order both sides by the lhs stride so each side collapses when it can
+      std::vector<size_t> order(ac.size());
+      for (size_t k = 0; k < order.size(); ++k) order[k] = k;
+      const std::vector<int64_t>& ast = va.strides;
+      std::sort(order.begin(), order.end(), [&](size_t x, size_t y) { return ast[ac[x]] > ast[ac[y]]; });
+      std::vector<int64_t> acs, bcs;
+      for (auto k : order) { acs.push_back(ac[k]); bcs.push_back(bc[k]); }
+      int64_t Ka = 0, Kb = 0, M = 0, N = 0;
+      bool ok = mergeDims(a->type, va.strides, acs, Ka, g.aCol) && mergeDims(b->type, vb.strides, bcs, Kb, g.bRow) &&
+                mergeDims(a->type, va.strides, af, M, g.aRow) && mergeDims(b->type, vb.strides, bf, N, g.bCol);
+      g.M = M; g.N = N; g.K = Ka;
+      // batch dims: up to two independent strides per operand
+      bsz.clear(); abst.clear(); bbst.clear();
+      const std::vector<int64_t>& bstr = vb.strides;
+      for (size_t k = 0; k < ab.size(); ++k) {
+        if (a->type.dims[ab[k]] == 1) continue;
+        if (!bsz.empty() && ast[ab[k]] * a->type.dims[ab[k]] == abst.back() && bstr[bb[k]] * b->type.dims[bb[k]] == bbst.back()) {
+          bsz.back() *= a->type.dims[ab[k]];
+          abst.back() = ast[ab[k]];
+          bbst.back() = bstr[bb[k]];
+        } else {
+          bsz.push_back(a->type.dims[ab[k]]);
+          abst.push_back(ast[ab[k]]);
+          bbst.push_back(bstr[bb[k]]);
+        }
+      }
+      if (ok && bsz.size() <= 2 && Ka == Kb) break;
+      if (!usedView)
+        throw CompileError("dot_general: operand layout needs a transposed copy (dims do not collapse to strided 2-D); not supported yet: " + a->type.str() + " x " + b->type.str());
     }
-    if (!ok || bsz.size() > 2 || Ka != Kb)
-      throw CompileError("dot_general: operand layout needs a transposed copy (dims do not collapse to strided 2-D); not supported yet: " + a->type.str() + " x " + b->type.str());
     if (bsz.size() >= 1) { g.batch0 = bsz[0]; g.aB0 = abst[0]; g.bB0 = bbst[0]; }
     if (bsz.size() == 2) { g.batch1 = bsz[1]; g.aB1 = abst[1]; g.bB1 = bbst[1]; }
     dp.va = va;
@@ -2863,6 +2875,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   lowerRng(*module);
   lowerTopK(*module);
   lowerEmptyReductions(*module);
+  canonicalizeDotLayouts(*module);
   hoistLoopProducts(*module);
   dropScatterIndexMasks(*module);
   reluMasksFromActivations(*module);

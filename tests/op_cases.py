@@ -493,6 +493,15 @@ case("attention-bf16-probabilities-read-twice", lambda b, q, k, v: (lambda lg: [
      f32(2222, 2, 64, 2, 64, lo=-1, hi=1), f32(2223, 2, 64, 2, 64, lo=-1, hi=1), f32(2224, 2, 64, 2, 64, lo=-1, hi=1), dtypes=_B16)
 
 
+# dimension numbers whose operand dims do not collapse to one strided matrix per batch (free dims on both sides of a contracted
+# one, contracted dims in another order on the other side, batch dims apart): a transposed copy is made first
+case("dot-general-vector-times-the-middle-dim", lambda b, v, t: b.dot_general(v, t, ([0], [1])), f32(2300, 5), f32(2301, 4, 5, 6))
+case("dot-general-three-contracted-dims-in-another-order", lambda b, x, y: b.dot_general(x, y, ([3, 1, 2], [3, 1, 0])), f32(2302, 3, 4, 3, 2), f32(2303, 3, 4, 4, 2))
+case("dot-general-batch-dim-between-contracted-dims", lambda b, x, y: b.dot_general(x, y, ([1, 2], [3, 1]), ([0], [2])), f32(2304, 3, 3, 2), f32(2305, 4, 2, 3, 3))
+case("dot-general-free-dims-around-a-contracted-one-bf16", lambda b, x, y: b.dot_general(x, y, ([3], [2])), f32(2306, 4, 5, 2, 5, lo=-1, hi=1), f32(2307, 3, 2, 5, 2, lo=-1, hi=1),
+     dtypes=["bf16", "bf16"])
+case("dot-general-tensordot-two-axes-swapped", lambda b, x, y: b.tanh(b.dot_general(x, y, ([0, 2], [1, 0]))), f32(2308, 16, 7, 33, lo=-1, hi=1), f32(2309, 33, 16, 9, lo=-1, hi=1))
+
 # independent small products next to each other share one launch (the gradients of one recurrent step)
 case("dot-group-three-independent", lambda b, dz, wh, h, x: [b.dot_general(dz, wh, ([1], [1])), b.dot_general(h, dz, ([0], [0])), b.dot_general(x, dz, ([0], [0]))],
      f32(2050, 20, 96), f32(2051, 40, 96), f32(2052, 20, 40), f32(2053, 20, 24))
