@@ -1349,6 +1349,60 @@ void canonicalizeDotLayoutsIn(Region& r, int& nextId) {
 }
 }  // namespace
 
+// float16 products and convolutions run on the float32 path: operands widened, the float32 result narrowed once
+// (every f16 value is an f32 value, and the sums are accumulated in float32 as the fused kernels do for bf16).
+namespace {
+void widenHalfProductsIn(Region& r, int& nextId) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) widenHalfProductsIn(*sub, nextId);
+    if (op->name != "dot_general" && op->name != "dot" && op->name != "convolution") continue;
+    if (op->operands.size() != 2 || op->results.size() != 1) continue;
+    if (op->operands[0]->type.dt != DType::F16 && op->operands[1]->type.dt != DType::F16) continue;
+    std::vector<std::unique_ptr<Op>> before;
+    for (size_t q = 0; q < 2; ++q) {
+      Value* v = op->operands[q];
+      if (v->type.dt != DType::F16) continue;
+      auto cv = makeOp("convert", {v}, &r, op->line);
+      TensorType t = v->type;
+      t.dt = DType::F32;
+      Value* wide = addResult(cv.get(), t, nextId);
+      v->users.erase(std::remove(v->users.begin(), v->users.end(), op), v->users.end());
+      v->users.push_back(cv.get());
+      op->operands[q] = wide;
+      wide->users.push_back(op);
+      before.push_back(std::move(cv));
+    }
+    Value* out = op->result();
+    std::unique_ptr<Op> after;
+    if (out->type.dt == DType::F16) {
+      // the product keeps a new float32 result; the old result value (and its readers) moves to the narrowing convert
+      after = makeOp("convert", {}, &r, op->line);
+      after->results.push_back(std::move(op->results[0]));
+      after->results[0]->def = after.get();
+      after->results[0]->defIndex = 0;
+      op->results.clear();
+      TensorType t = after->results[0]->type;
+      t.dt = DType::F32;
+      Value* wide = addResult(op, t, nextId);
+      after->operands.push_back(wide);
+      wide->users.push_back(after.get());
+    }
+    const size_t nb = before.size();
+    r.ops.insert(r.ops.begin() + (long)k, std::make_move_iterator(before.begin()), std::make_move_iterator(before.end()));
+    k += nb;
+    if (after) { r.ops.insert(r.ops.begin() + (long)k + 1, std::move(after)); ++k; }
+  }
+}
+}  // namespace
+
+void widenHalfProducts(Module& m) {
+  Func* f = m.main();
+  if (!f) return;
+  int nextId = maxValueId(f->body) + 1;
+  widenHalfProductsIn(f->body, nextId);
+}
+
 void canonicalizeDotLayouts(Module& m) {
   Func* f = m.main();
   if (!f) return;

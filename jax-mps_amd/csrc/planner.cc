@@ -2870,6 +2870,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   inlineCalls(*module);
   lowerSingleDeviceOps(*module);
   lowerIntegerDots(*module);
+  widenHalfProducts(*module);
   lowerGeneralScatters(*module);
   lowerWindowOps(*module);
   lowerRng(*module);

@@ -502,6 +502,14 @@ case("dot-general-free-dims-around-a-contracted-one-bf16", lambda b, x, y: b.dot
      dtypes=["bf16", "bf16"])
 case("dot-general-tensordot-two-axes-swapped", lambda b, x, y: b.tanh(b.dot_general(x, y, ([0, 2], [1, 0]))), f32(2308, 16, 7, 33, lo=-1, hi=1), f32(2309, 33, 16, 9, lo=-1, hi=1))
 
+# float16 products and convolutions: widened to the float32 path, the result narrowed once
+case("dot-f16-bias-tanh", lambda b, x, w, c: b.tanh(b.add(b.matmul(x, w), b.broadcast_in_dim(c, (16, 8), [1]))),
+     f32(2310, 16, 32, lo=-1, hi=1).astype(np.float16), f32(2311, 32, 8, lo=-0.3, hi=0.3).astype(np.float16), f32(2312, 8).astype(np.float16))
+case("dot-f16-batched-f32-result", lambda b, x, w: b.dot_general(x, w, ([2], [1]), ([0], [0]), out_dtype="f32"),
+     f32(2313, 3, 20, 64, lo=-1, hi=1).astype(np.float16), f32(2314, 3, 64, 24, lo=-1, hi=1).astype(np.float16))
+case("conv-f16-3x3-pad1", lambda b, x, f: b.conv(x, f, padding=((1, 1), (1, 1))), f32(2315, 2, 8, 8, 16, lo=-1, hi=1).astype(np.float16),
+     f32(2316, 3, 3, 16, 8, lo=-0.2, hi=0.2).astype(np.float16))
+
 # independent small products next to each other share one launch (the gradients of one recurrent step)
 case("dot-group-three-independent", lambda b, dz, wh, h, x: [b.dot_general(dz, wh, ([1], [1])), b.dot_general(h, dz, ([0], [0])), b.dot_general(x, dz, ([0], [0]))],
      f32(2050, 20, 96), f32(2051, 40, 96), f32(2052, 20, 40), f32(2053, 20, 24))

@@ -15,6 +15,7 @@ pytestmark = pytest.mark.gpu
 
 F32_TOL = 1e-5
 BF16_TOL = 2e-2
+F16_TOL = 2e-3    # two units in the last place of an 11-bit significand
 # cases the plan compiler rejects (none at present; the error texts are checked in test_frontend.py)
 UNSUPPORTED = set()
 # cases held to a looser elementwise bound than the dtype's, each with its reason
@@ -42,7 +43,7 @@ def test_op_case(client, name):
     for k, (g, w, (shape, dt)) in enumerate(zip(got, want, oracle.result_types)):
         assert g.shape == tuple(shape)
         if dt in ("f32", "bf16", "f16") and not c.exact:
-            tol = BF16_TOL if "bf16" in c.dtypes or dt == "bf16" else F32_TOL
+            tol = BF16_TOL if "bf16" in c.dtypes or dt == "bf16" else F16_TOL if "f16" in c.dtypes or dt == "f16" else F32_TOL
             tol = LOOSER.get(name, tol)
             ratio = closeness(g, w, tol, tol)
             assert ratio <= 1.0, f"{name} output {k}: {ratio:.3f} x the bound |d| <= {tol} + {tol} |want|"
