@@ -153,6 +153,7 @@ void lowerIntegerDots(Module& m);    // integer / boolean dot_general -> broadca
 void lowerSingleDeviceOps(Module& m);  // one-device all_reduce -> operands, partition_id / replica_id -> 0, tokens -> f32 scalar placeholders
 void reluMasksFromActivations(Module& m);  // compare(v, 0, GT) beside maximum(v, 0) reads the maximum instead
 void lowerTopK(Module& m);           // chlo.top_k -> stable descending sort of (value, position) + slice
+void lowerBitcastWidths(Module& m);      // bitcast_convert between types of different width -> shifts and same-width bitcasts
 void widenHalfProducts(Module& m);       // f16 dot_general / convolution -> f32 product between converts
 void canonicalizeDotLayouts(Module& m);  // dot_general whose operand dims do not collapse to strided matrices: transposes in front
 void lowerEmptyReductions(Module& m);   // reduce over zero elements -> broadcast of the init values

@@ -1396,6 +1396,98 @@ void widenHalfProductsIn(Region& r, int& nextId) {
 }
 }  // namespace
 
+// bitcast_convert between element types of different width (jnp's x.view(dtype), lax.bitcast_convert_type): to a narrower
+// type the result gains a last dim of (wide / narrow) elements, least significant first; from a narrower type the last
+// dim is folded into one element.  Written with same-width bitcasts, shifts by multiples of the narrow width and, for
+// the widening form, an OR of the shifted parts.
+namespace {
+DType unsignedOfSize(size_t n) { return n == 1 ? DType::U8 : n == 2 ? DType::U16 : n == 4 ? DType::U32 : DType::U64; }
+void lowerBitcastWidthsIn(Region& r, int& nextId) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) lowerBitcastWidthsIn(*sub, nextId);
+    if (op->name != "bitcast_convert" || op->operands.size() != 1 || op->results.size() != 1) continue;
+    Value* x = op->operands[0];
+    const TensorType rt = op->result()->type;
+    if (x->type.dt == DType::Pred || rt.dt == DType::Pred) continue;
+    const size_t a = dtypeSize(x->type.dt), b = dtypeSize(rt.dt);
+    if (a == b) continue;
+    Rewriter rw{r, nextId, op->line, {}};
+    auto same = [&](Value* v, DType dt) -> Value* {   // same-width bitcast (a no-op when the type is already that)
+      if (v->type.dt == dt) return v;
+      TensorType t = v->type;
+      t.dt = dt;
+      return rw.unary("bitcast_convert", v, t);
+    };
+    auto shiftAmounts = [&](const TensorType& like, int64_t bitsPerStep) {   // iota along the last dim times the step, in `like`'s type
+      auto io = makeOp("iota", {}, &r, op->line);
+      Attr dimA;
+      dimA.kind = Attr::Int;
+      dimA.i = like.rank() - 1;
+      io->attrs["dim"] = dimA;
+      Value* pos = rw.emit(std::move(io), like);
+      uint64_t step = (uint64_t)bitsPerStep;
+      return rw.binary("multiply", pos, rw.splat(like.dt, like.dims, &step), like);
+    };
+    if (a > b) {
+      const int64_t q = (int64_t)(a / b);
+      if (rt.rank() != x->type.rank() + 1 || rt.dims.back() != q) throw CompileError("stablehlo.bitcast_convert: the result of a narrowing bitcast must add a last dim of " + std::to_string(q));
+      const DType U = unsignedOfSize(a), Ub = unsignedOfSize(b);
+      Value* bits = same(x, U);
+      TensorType wide = rt;
+      wide.dt = U;
+      auto bc = makeOp("broadcast_in_dim", {bits}, &r, op->line);
+      std::vector<int64_t> dims;
+      for (int d = 0; d < x->type.rank(); ++d) dims.push_back(d);
+      bc->attrs["dims"] = intsAttr(dims);
+      Value* spread = rw.emit(std::move(bc), wide);
+      Value* parts = rw.binary("shift_right_logical", spread, shiftAmounts(wide, (int64_t)b * 8), wide);
+      TensorType narrow = rt;
+      narrow.dt = Ub;
+      if (rt.dt == Ub) {
+        rw.finish(k, op, makeOp("convert", {parts}, &r, op->line));
+      } else {
+        Value* low = rw.unary("convert", parts, narrow);
+        rw.finish(k, op, makeOp("bitcast_convert", {low}, &r, op->line));
+      }
+    } else {
+      const int64_t q = (int64_t)(b / a);
+      if (x->type.rank() != rt.rank() + 1 || x->type.dims.back() != q) throw CompileError("stablehlo.bitcast_convert: the operand of a widening bitcast must have a last dim of " + std::to_string(q));
+      const DType Ua = unsignedOfSize(a), U = unsignedOfSize(b);
+      Value* bits = same(x, Ua);
+      TensorType wide = x->type;
+      wide.dt = U;
+      Value* ext = rw.unary("convert", bits, wide);
+      Value* placed = rw.binary("shift_left", ext, shiftAmounts(wide, (int64_t)a * 8), wide);
+      TensorType ut = rt;
+      ut.dt = U;
+      Value* acc = nullptr;
+      for (int64_t j = 0; j < q; ++j) {
+        std::vector<int64_t> start((size_t)wide.rank(), 0), count = wide.dims, stride((size_t)wide.rank(), 1);
+        start.back() = j;
+        count.back() = 1;
+        Value* part = rw.unary("reshape", rw.slice(placed, start, count, stride), ut);
+        acc = acc ? rw.binary("or", acc, part, ut) : part;
+      }
+      if (rt.dt == U) {
+        // (the results move to an op of their own: OR with zero keeps the value)
+        uint64_t zero = 0;
+        rw.finish(k, op, makeOp("or", {acc, rw.splat(U, ut.dims, &zero)}, &r, op->line));
+      } else {
+        rw.finish(k, op, makeOp("bitcast_convert", {acc}, &r, op->line));
+      }
+    }
+  }
+}
+}  // namespace
+
+void lowerBitcastWidths(Module& m) {
+  Func* f = m.main();
+  if (!f) return;
+  int nextId = maxValueId(f->body) + 1;
+  lowerBitcastWidthsIn(f->body, nextId);
+}
+
 void widenHalfProducts(Module& m) {
   Func* f = m.main();
   if (!f) return;

@@ -2871,6 +2871,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   lowerSingleDeviceOps(*module);
   lowerIntegerDots(*module);
   widenHalfProducts(*module);
+  lowerBitcastWidths(*module);
   lowerGeneralScatters(*module);
   lowerWindowOps(*module);
   lowerRng(*module);

@@ -510,6 +510,19 @@ case("dot-f16-batched-f32-result", lambda b, x, w: b.dot_general(x, w, ([2], [1]
 case("conv-f16-3x3-pad1", lambda b, x, f: b.conv(x, f, padding=((1, 1), (1, 1))), f32(2315, 2, 8, 8, 16, lo=-1, hi=1).astype(np.float16),
      f32(2316, 3, 3, 16, 8, lo=-0.2, hi=0.2).astype(np.float16))
 
+# bitcast_convert between element types of different width (x.view(dtype)): a last dim of wide / narrow elements, least
+# significant first, appears or is folded away
+def _bitcast_to(b, x, dtype, shape):
+    v = b._new(shape, dtype)
+    b._emit(f"{v.name} = stablehlo.bitcast_convert {x.name} : ({x.type}) -> {v.type}")
+    return v
+case("bitcast-f32-to-four-u8", lambda b, x: _bitcast_to(b, x, "ui8", (3, 5, 4)), f32(2320, 3, 5), exact=True)
+case("bitcast-i64-to-two-i32-and-back", lambda b, x: (lambda h: [h, _bitcast_to(b, h, "i64", (7,))])(_bitcast_to(b, x, "i32", (7, 2))),
+     np.array([0, 1, -1, 2**40 + 5, -2**63, 2**63 - 1, 123456789012345], np.int64), exact=True)
+case("bitcast-four-u8-to-f32", lambda b, x: _bitcast_to(b, x, "f32", (6,)), rng(2321).integers(0, 256, size=(6, 4)).astype(np.uint8), exact=True)
+case("bitcast-two-bf16-to-u32-and-f32-to-two-f16", lambda b, x, y: [_bitcast_to(b, x, "ui32", (5,)), _bitcast_to(b, y, "f16", (5, 2))],
+     f32(2322, 5, 2), f32(2323, 5), dtypes=["bf16", "f32"], exact=True)
+
 # independent small products next to each other share one launch (the gradients of one recurrent step)
 case("dot-group-three-independent", lambda b, dz, wh, h, x: [b.dot_general(dz, wh, ([1], [1])), b.dot_general(h, dz, ([0], [0])), b.dot_general(x, dz, ([0], [0]))],
      f32(2050, 20, 96), f32(2051, 40, 96), f32(2052, 20, 40), f32(2053, 20, 24))
