@@ -154,6 +154,7 @@ void lowerSingleDeviceOps(Module& m);  // one-device all_reduce -> operands, par
 void reluMasksFromActivations(Module& m);  // compare(v, 0, GT) beside maximum(v, 0) reads the maximum instead
 void lowerTopK(Module& m);           // chlo.top_k -> stable descending sort of (value, position) + slice
 void lowerBitcastWidths(Module& m);      // bitcast_convert between types of different width -> shifts and same-width bitcasts
+void widenScatterTypes(Module& m);       // scatter on bool / 8- and 16-bit integers / f16 -> on the 32-bit type that holds them
 void widenHalfProducts(Module& m);       // f16 dot_general / convolution -> f32 product between converts
 void canonicalizeDotLayouts(Module& m);  // dot_general whose operand dims do not collapse to strided matrices: transposes in front
 void lowerEmptyReductions(Module& m);   // reduce over zero elements -> broadcast of the init values

@@ -1488,6 +1488,76 @@ void lowerBitcastWidths(Module& m) {
   lowerBitcastWidthsIn(f->body, nextId);
 }
 
+// Scatters on element types the scatter kernels do not take (bool, 8- and 16-bit integers, float16) run on the 32-bit
+// type that holds them: operand and updates widened, the combiner retyped, the result narrowed.  Sums and products of
+// narrow integers wrap the same way after one narrowing as after every step, a boolean sum is an OR (any count above
+// zero is true), minima, maxima and plain writes are order-preserving under sign or zero extension.  Index tensors of
+// 8 or 16 bits are widened to int32.
+namespace {
+void retypeRegion(Region& rg, DType from, DType to) {
+  for (auto& a : rg.args) if (a->type.dt == from) a->type.dt = to;
+  for (auto& o : rg.ops) {
+    for (auto& v : o->results) if (v->type.dt == from) v->type.dt = to;
+    for (auto& sub : o->regions) retypeRegion(*sub, from, to);
+  }
+}
+void widenScatterTypesIn(Region& r, int& nextId) {
+  for (size_t k = 0; k < r.ops.size(); ++k) {
+    Op* op = r.ops[k].get();
+    for (auto& sub : op->regions) widenScatterTypesIn(*sub, nextId);
+    if (op->name != "scatter" || op->operands.size() != 3 || op->results.size() != 1 || op->regions.size() != 1) continue;
+    std::vector<std::unique_ptr<Op>> before;
+    auto converted = [&](size_t at, DType to) {
+      Value* v = op->operands[at];
+      auto cv = makeOp("convert", {v}, &r, op->line);
+      TensorType t = v->type;
+      t.dt = to;
+      Value* w = addResult(cv.get(), t, nextId);
+      v->users.erase(std::remove(v->users.begin(), v->users.end(), op), v->users.end());
+      v->users.push_back(cv.get());
+      op->operands[at] = w;
+      w->users.push_back(op);
+      before.push_back(std::move(cv));
+    };
+    const DType it = op->operands[1]->type.dt;
+    if (it == DType::S8 || it == DType::U8 || it == DType::S16 || it == DType::U16) converted(1, DType::S32);
+    const DType et = op->operands[0]->type.dt;
+    DType wide = et;
+    if (et == DType::F16) wide = DType::F32;
+    else if (et == DType::S8 || et == DType::S16) wide = DType::S32;
+    else if (et == DType::U8 || et == DType::U16 || et == DType::Pred) wide = DType::U32;
+    std::unique_ptr<Op> after;
+    if (wide != et && op->operands[2]->type.dt == et) {
+      converted(0, wide);
+      converted(2, wide);
+      retypeRegion(*op->regions[0], et, wide);
+      after = makeOp("convert", {}, &r, op->line);
+      after->results.push_back(std::move(op->results[0]));
+      after->results[0]->def = after.get();
+      after->results[0]->defIndex = 0;
+      op->results.clear();
+      TensorType t = after->results[0]->type;
+      t.dt = wide;
+      Value* w = addResult(op, t, nextId);
+      after->operands.push_back(w);
+      w->users.push_back(after.get());
+    }
+    const size_t nb = before.size();
+    if (nb == 0 && !after) continue;
+    r.ops.insert(r.ops.begin() + (long)k, std::make_move_iterator(before.begin()), std::make_move_iterator(before.end()));
+    k += nb;
+    if (after) { r.ops.insert(r.ops.begin() + (long)k + 1, std::move(after)); ++k; }
+  }
+}
+}  // namespace
+
+void widenScatterTypes(Module& m) {
+  Func* f = m.main();
+  if (!f) return;
+  int nextId = maxValueId(f->body) + 1;
+  widenScatterTypesIn(f->body, nextId);
+}
+
 void widenHalfProducts(Module& m) {
   Func* f = m.main();
   if (!f) return;

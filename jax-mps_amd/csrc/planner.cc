@@ -2872,6 +2872,7 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   lowerIntegerDots(*module);
   widenHalfProducts(*module);
   lowerBitcastWidths(*module);
+  widenScatterTypes(*module);
   lowerGeneralScatters(*module);
   lowerWindowOps(*module);
   lowerRng(*module);

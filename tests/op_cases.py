@@ -226,6 +226,16 @@ case("scatter-add", _row_scatter("add"), np.zeros((10, 4), np.float32), np.array
 case("scatter-add-duplicates", _row_scatter("add"), f32(150, 10, 4), np.array([3, 3, 0, 3, 9, 0, 3], np.int32), f32(151, 7, 4), exact=True)
 case("scatter-add-oob-dropped", _row_scatter("add"), f32(152, 6, 5), np.array([0, 6, -1, 5, 100], np.int32), f32(153, 5, 5), exact=True)
 case("scatter-set", _row_scatter("set"), f32(154, 5, 3), np.array([0, 2], np.int32), f32(155, 2, 3), exact=True)
+# element types the scatter kernels do not take run on the 32-bit type that holds them (and narrow index types on int32)
+case("scatter-set-bool-mask", _row_scatter("set"), np.zeros((10, 4), np.bool_), np.array([3, 7, 3, 12, -1], np.int32), rng(160).random((5, 4)) > 0.4, dtypes=["i1", "i32", "i1"], exact=True)
+case("scatter-add-bool-is-or", _row_scatter("add"), rng(161).random((6, 3)) > 0.7, np.array([0, 0, 5, 2], np.int64), rng(162).random((4, 3)) > 0.5, dtypes=["i1", "i64", "i1"], exact=True)
+case("scatter-add-u8-wraps", _row_scatter("add"), rng(163).integers(0, 256, size=(5, 6)).astype(np.uint8), np.array([1, 1, 1, 4, 0, 1], np.int32),
+     rng(164).integers(100, 256, size=(6, 6)).astype(np.uint8), exact=True)
+case("scatter-min-i8-u8-indices", _row_scatter("min"), rng(165).integers(-128, 128, size=(7, 5)).astype(np.int8), np.array([6, 0, 6, 3, 200], np.uint8),
+     rng(166).integers(-128, 128, size=(5, 5)).astype(np.int8), exact=True)
+case("scatter-mul-i16-wraps-i16-indices", _row_scatter("mul"), rng(167).integers(-300, 300, size=(4, 3)).astype(np.int16), np.array([2, 2, 2, 0, -1], np.int16),
+     rng(168).integers(-300, 300, size=(5, 3)).astype(np.int16), exact=True)
+case("scatter-add-f16", _row_scatter("add"), f32(169, 9, 8, lo=-1, hi=1).astype(np.float16), np.array([4, 4, 0, 8, 4], np.int32), f32(170, 5, 8, lo=-1, hi=1).astype(np.float16))
 case("scatter-mul", _row_scatter("mul", unique_indices=True), np.ones((10, 4), np.float32), np.array([0, 2, 5], np.int32), np.full((3, 4), 2.0, np.float32), exact=True)
 case("scatter-min", _row_scatter("min"), f32(156, 10, 4), np.array([0, 2, 5], np.int32), f32(157, 3, 4), exact=True)
 case("scatter-max", _row_scatter("max"), f32(158, 10, 4), np.array([0, 2, 2], np.int32), f32(159, 3, 4), exact=True)
