@@ -1542,6 +1542,46 @@ void widenScatterTypesIn(Region& r, int& nextId) {
       after->operands.push_back(w);
       w->users.push_back(after.get());
     }
+    // A plain write of 64-bit elements moves two 32-bit halves: the same update wins both (updates are applied in
+    // order), so operand and updates are read as [..., 2] uint32 tensors with the pair as one more window dim.
+    // (lowerBitcastWidths, which runs later, spells the bitcasts out.)  Sums, minima and maxima of 64-bit elements
+    // do not split this way and stay refused.
+    Region& body = *op->regions[0];
+    const bool plainWrite = body.args.size() == 2 && body.ops.size() == 1 && body.ops[0]->name == "return" && body.ops[0]->operands.size() == 1 &&
+                            body.ops[0]->operands[0] == body.args[1].get();
+    if ((et == DType::S64 || et == DType::U64) && op->operands[2]->type.dt == et && plainWrite) {
+      auto halves = [&](size_t at) {
+        Value* v = op->operands[at];
+        auto bc = makeOp("bitcast_convert", {v}, &r, op->line);
+        TensorType t = v->type;
+        t.dt = DType::U32;
+        t.dims.push_back(2);
+        Value* w = addResult(bc.get(), t, nextId);
+        v->users.erase(std::remove(v->users.begin(), v->users.end(), op), v->users.end());
+        v->users.push_back(bc.get());
+        op->operands[at] = w;
+        w->users.push_back(op);
+        before.push_back(std::move(bc));
+      };
+      const int64_t updatesRank = op->operands[2]->type.rank();
+      halves(0);
+      halves(2);
+      auto uwd = op->ints("update_window_dims");
+      uwd.push_back(updatesRank);
+      op->attrs["update_window_dims"] = intsAttr(uwd);
+      retypeRegion(body, et, DType::U32);
+      after = makeOp("bitcast_convert", {}, &r, op->line);
+      after->results.push_back(std::move(op->results[0]));
+      after->results[0]->def = after.get();
+      after->results[0]->defIndex = 0;
+      op->results.clear();
+      TensorType t = after->results[0]->type;
+      t.dt = DType::U32;
+      t.dims.push_back(2);
+      Value* w = addResult(op, t, nextId);
+      after->operands.push_back(w);
+      w->users.push_back(after.get());
+    }
     const size_t nb = before.size();
     if (nb == 0 && !after) continue;
     r.ops.insert(r.ops.begin() + (long)k, std::make_move_iterator(before.begin()), std::make_move_iterator(before.end()));

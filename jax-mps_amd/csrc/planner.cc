@@ -2871,8 +2871,8 @@ std::unique_ptr<CompiledProgram> compileProgram(std::unique_ptr<Module> module) 
   lowerSingleDeviceOps(*module);
   lowerIntegerDots(*module);
   widenHalfProducts(*module);
-  lowerBitcastWidths(*module);
   widenScatterTypes(*module);
+  lowerBitcastWidths(*module);
   lowerGeneralScatters(*module);
   lowerWindowOps(*module);
   lowerRng(*module);

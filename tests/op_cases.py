@@ -235,6 +235,10 @@ case("scatter-min-i8-u8-indices", _row_scatter("min"), rng(165).integers(-128, 1
      rng(166).integers(-128, 128, size=(5, 5)).astype(np.int8), exact=True)
 case("scatter-mul-i16-wraps-i16-indices", _row_scatter("mul"), rng(167).integers(-300, 300, size=(4, 3)).astype(np.int16), np.array([2, 2, 2, 0, -1], np.int16),
      rng(168).integers(-300, 300, size=(5, 3)).astype(np.int16), exact=True)
+case("scatter-set-i64-as-two-halves", _row_scatter("set"), np.array([[2**40 + 5, -1], [7, -2**63], [2**63 - 1, 0], [3, 4]], np.int64), np.array([2, 0, 2, 9], np.int32),
+     np.array([[-2**50, 11], [2**33, -2**33], [12345678901234, -98765432109876], [1, 1]], np.int64), exact=True)
+case("scatter-set-u64-rank-3-i64-indices", _row_scatter("set"), rng(171).integers(0, 2**63, size=(5, 2, 3)).astype(np.uint64) * np.uint64(2), np.array([4, 1, 4], np.int64),
+     rng(172).integers(0, 2**63, size=(3, 2, 3)).astype(np.uint64) * np.uint64(2) + np.uint64(1), exact=True)
 case("scatter-add-f16", _row_scatter("add"), f32(169, 9, 8, lo=-1, hi=1).astype(np.float16), np.array([4, 4, 0, 8, 4], np.int32), f32(170, 5, 8, lo=-1, hi=1).astype(np.float16))
 case("scatter-mul", _row_scatter("mul", unique_indices=True), np.ones((10, 4), np.float32), np.array([0, 2, 5], np.int32), np.full((3, 4), 2.0, np.float32), exact=True)
 case("scatter-min", _row_scatter("min"), f32(156, 10, 4), np.array([0, 2, 5], np.int32), f32(157, 3, 4), exact=True)
